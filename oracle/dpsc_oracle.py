@@ -1,0 +1,425 @@
+"""ctypes bindings of the CPU checker (test infrastructure only).
+
+Only tests/, the smoke check and the benchmark's cpu_baseline leg import this
+module.  Extension elements cross as numpy uint64 arrays of shape (..., 2)
+holding (c0, c1).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libdpsc_oracle.so")
+
+P = 0xFFFFFFFF00000001
+MAX_FACTORS = 8
+AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
+
+
+def build(force=False):
+    """Compile the checker with the Makefile beside this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
+    return _LIB_PATH
+
+
+class Term(C.Structure):
+    _fields_ = [("coeff", C.c_uint64 * 2), ("n_factors", C.c_uint32), ("factors", C.c_uint32 * MAX_FACTORS)]
+
+
+class Transcript(C.Structure):
+    _fields_ = [("state", C.c_uint8 * 32), ("n_rounds", C.c_uint32)]
+
+
+class LogupInstance(C.Structure):
+    _fields_ = [
+        ("n_cols", C.c_uint32),
+        ("len", C.c_uint64),
+        ("cols", C.POINTER(C.c_void_p)),
+        ("numer", C.c_void_p),
+        ("c", C.c_uint64 * 2),
+        ("beta", C.c_uint64 * 2),
+    ]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        u64, i64, vp = C.c_uint64, C.c_int64, C.c_void_p
+        for name in ("add", "sub", "mul", "pow"):
+            f = getattr(_lib, "orc_gl_" + name)
+            f.restype, f.argtypes = u64, [u64, u64]
+        for name in ("neg", "inv"):
+            f = getattr(_lib, "orc_gl_" + name)
+            f.restype, f.argtypes = u64, [u64]
+        _lib.orc_gl_from_i64.restype, _lib.orc_gl_from_i64.argtypes = u64, [i64]
+        _lib.orc_gl_to_i64.restype, _lib.orc_gl_to_i64.argtypes = i64, [u64]
+        _lib.orc_logup_arena_len.restype, _lib.orc_logup_arena_len.argtypes = u64, [u64]
+        _lib.orc_logup_layer_offset.restype, _lib.orc_logup_layer_offset.argtypes = u64, [u64, C.c_uint32]
+        _lib.orc_partial_eval.restype = i64
+        _lib.orc_stacking_coeffs.restype = i64
+        _lib.orc_logup_batch_prove.restype = i64
+        _lib.orc_sc_prove.restype = C.c_int
+        _lib.orc_sc_verify.restype = C.c_int
+        _lib.orc_logup_batch_verify.restype = C.c_int
+        _lib.orc_num_threads.restype = C.c_int
+    return _lib
+
+
+def _e2arr(x):
+    a = np.ascontiguousarray(x, dtype=np.uint64)
+    assert a.shape[-1] == 2, a.shape
+    return a
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def e2(c0, c1=0):
+    return np.array([c0 % P, c1 % P], dtype=np.uint64)
+
+
+# ---- field ----
+def gl_mul(a, b):
+    return lib().orc_gl_mul(int(a), int(b))
+
+
+def gl_add(a, b):
+    return lib().orc_gl_add(int(a), int(b))
+
+
+def gl_sub(a, b):
+    return lib().orc_gl_sub(int(a), int(b))
+
+
+def gl_inv(a):
+    return lib().orc_gl_inv(int(a))
+
+
+def gl_from_i64(x):
+    return lib().orc_gl_from_i64(int(x))
+
+
+def gl_to_i64(x):
+    return lib().orc_gl_to_i64(int(x))
+
+
+def _bin(name, a, b):
+    a, b = _e2arr(a), _e2arr(b)
+    out = np.zeros(2, dtype=np.uint64)
+    getattr(lib(), name)(_p(a), _p(b), _p(out))
+    return out
+
+
+def e2_add(a, b):
+    return _bin("orc_e2_add", a, b)
+
+
+def e2_sub(a, b):
+    return _bin("orc_e2_sub", a, b)
+
+
+def e2_mul(a, b):
+    return _bin("orc_e2_mul", a, b)
+
+
+def e2_inv(a):
+    a = _e2arr(a)
+    out = np.zeros(2, dtype=np.uint64)
+    lib().orc_e2_inv(_p(a), _p(out))
+    return out
+
+
+# ---- tables ----
+def eq_evals(point):
+    point = _e2arr(point).reshape(-1, 2)
+    m = point.shape[0]
+    out = np.zeros((1 << m, 2), dtype=np.uint64)
+    lib().orc_eq_evals(_p(point), C.c_uint32(m), _p(out))
+    return out
+
+
+def identity_eval(r1, r2):
+    r1, r2 = _e2arr(r1).reshape(-1, 2), _e2arr(r2).reshape(-1, 2)
+    n = min(len(r1), len(r2))
+    out = np.zeros(2, dtype=np.uint64)
+    lib().orc_identity_eval(_p(r1), _p(r2), C.c_uint32(n), _p(out))
+    return out
+
+
+def embed_base(v):
+    v = np.ascontiguousarray(v, dtype=np.uint64)
+    out = np.zeros((v.size, 2), dtype=np.uint64)
+    lib().orc_embed_base(_p(v), C.c_uint64(v.size), _p(out))
+    return out
+
+
+def embed_i64(v):
+    v = np.ascontiguousarray(v, dtype=np.int64)
+    out = np.zeros((v.size, 2), dtype=np.uint64)
+    lib().orc_embed_i64(_p(v), C.c_uint64(v.size), _p(out))
+    return out
+
+
+def _nvars(tbl):
+    n = int(tbl.shape[0]).bit_length() - 1
+    assert 1 << n == tbl.shape[0]
+    return n
+
+
+def mle_evaluate(tbl, point):
+    tbl, point = _e2arr(tbl), _e2arr(point).reshape(-1, 2)
+    n = _nvars(tbl)
+    assert point.shape[0] == n
+    out = np.zeros(2, dtype=np.uint64)
+    lib().orc_mle_evaluate(_p(tbl), C.c_uint32(n), _p(point), _p(out))
+    return out
+
+
+def mle_fix_low(tbl, point):
+    tbl, point = _e2arr(tbl), _e2arr(point).reshape(-1, 2)
+    n, k = _nvars(tbl), point.shape[0]
+    out = np.zeros((1 << (n - k), 2), dtype=np.uint64)
+    lib().orc_mle_fix_low(_p(tbl), C.c_uint32(n), _p(point), C.c_uint32(k), _p(out))
+    return out
+
+
+def mle_fix_high(tbl, point):
+    tbl, point = _e2arr(tbl), _e2arr(point).reshape(-1, 2)
+    n, k = _nvars(tbl), point.shape[0]
+    out = np.zeros((1 << (n - k), 2), dtype=np.uint64)
+    lib().orc_mle_fix_high(_p(tbl), C.c_uint32(n), _p(point), C.c_uint32(k), _p(out))
+    return out
+
+
+# ---- hash / transcript ----
+def blake3(data: bytes) -> bytes:
+    out = (C.c_uint8 * 32)()
+    buf = (C.c_uint8 * max(1, len(data))).from_buffer_copy(data or b"\0")
+    lib().orc_blake3(buf, C.c_size_t(len(data)), out)
+    return bytes(out)
+
+
+class OracleTranscript:
+    def __init__(self, label: bytes = b"m2vec"):
+        self.t = Transcript()
+        lib().orc_tr_new(C.byref(self.t), label, C.c_size_t(len(label)))
+
+    def state(self):
+        return bytes(self.t.state), int(self.t.n_rounds)
+
+    def append_message(self, label: bytes):
+        lib().orc_tr_append_message(C.byref(self.t), label, C.c_size_t(len(label)))
+
+    def append_bytes(self, data: bytes):
+        lib().orc_tr_append_bytes(C.byref(self.t), data, C.c_size_t(len(data)))
+
+    def append_u64(self, x):
+        lib().orc_tr_append_u64(C.byref(self.t), C.c_uint64(x))
+
+    def append_scalars(self, xs):
+        xs = _e2arr(xs).reshape(-1, 2)
+        lib().orc_tr_append_scalars(C.byref(self.t), _p(xs), C.c_size_t(xs.shape[0]))
+
+    def challenge_scalar(self):
+        out = np.zeros(2, dtype=np.uint64)
+        lib().orc_tr_challenge_scalar(C.byref(self.t), _p(out))
+        return out
+
+    def append_and_sample(self, label: bytes):
+        out = np.zeros(2, dtype=np.uint64)
+        lib().orc_tr_append_and_sample(C.byref(self.t), label, C.c_size_t(len(label)), _p(out))
+        return out
+
+    def read_challenges(self, n):
+        return np.stack([self.challenge_scalar() for _ in range(n)]) if n else np.zeros((0, 2), np.uint64)
+
+
+# ---- sumcheck ----
+def make_terms(terms):
+    """terms: list of (coeff e2, [mle indices])"""
+    arr = (Term * max(1, len(terms)))()
+    for i, (coeff, factors) in enumerate(terms):
+        c = _e2arr(coeff)
+        arr[i].coeff[0], arr[i].coeff[1] = int(c[0]), int(c[1])
+        arr[i].n_factors = len(factors)
+        for k, f in enumerate(factors):
+            arr[i].factors[k] = f
+    return arr
+
+
+def _table_ptrs(tables):
+    tabs = [_e2arr(t) for t in tables]
+    ptrs = (C.c_void_p * max(1, len(tabs)))(*[t.ctypes.data for t in tabs])
+    nvs = (C.c_uint32 * max(1, len(tabs)))(*[_nvars(t) for t in tabs])
+    return tabs, ptrs, nvs
+
+
+def sc_round_poly(live, tables, cur_nvars, terms):
+    tabs, ptrs, _ = _table_ptrs(tables)
+    nvs = (C.c_uint32 * len(tabs))(*cur_nvars)
+    tarr = make_terms(terms)
+    degree = max((len(f) for _, f in terms), default=0)
+    out = np.zeros((degree + 1, 2), dtype=np.uint64)
+    lib().orc_sc_round_poly(C.c_uint32(live), C.c_uint32(len(tabs)), ptrs, nvs, tarr, C.c_uint32(len(terms)),
+                            C.c_uint32(degree), _p(out))
+    return out
+
+
+def sc_prove(n_vars, tables, terms, transcript):
+    """Returns (proof[n_vars, d+1, 2], point[n_vars, 2], final_evals[n_mles, 2])."""
+    tabs, ptrs, nvs = _table_ptrs(tables)
+    tarr = make_terms(terms)
+    degree = max((len(f) for _, f in terms), default=0)
+    proof = np.zeros((n_vars, degree + 1, 2), dtype=np.uint64)
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    final = np.zeros((len(tabs), 2), dtype=np.uint64)
+    rc = lib().orc_sc_prove(C.c_uint32(n_vars), C.c_uint32(len(tabs)), ptrs, nvs, tarr, C.c_uint32(len(terms)),
+                            C.byref(transcript.t), _p(proof), _p(point), _p(final))
+    if rc != 0:
+        raise ValueError(f"orc_sc_prove failed: {rc}")
+    return proof, point, final
+
+
+def sc_verify(claimed_sum, proof, transcript):
+    """Returns (bad_round (0 = ok), point, expected_evaluation)."""
+    proof = _e2arr(proof)
+    n_vars, npts = proof.shape[0], proof.shape[1]
+    claimed = _e2arr(claimed_sum)
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    expected = np.zeros(2, dtype=np.uint64)
+    rc = lib().orc_sc_verify(_p(claimed), _p(proof), C.c_uint32(n_vars), C.c_uint32(npts - 1),
+                             C.byref(transcript.t), _p(point), _p(expected))
+    return rc, point, expected
+
+
+def interpolate(evals, r):
+    evals, r = _e2arr(evals).reshape(-1, 2), _e2arr(r)
+    out = np.zeros(2, dtype=np.uint64)
+    lib().orc_interpolate(_p(evals), C.c_uint32(evals.shape[0] - 1), _p(r), _p(out))
+    return out
+
+
+# ---- einsum partial evaluation ----
+def _points_ptrs(points):
+    keep = [None if p is None else _e2arr(p).reshape(-1, 2) for p in points]
+    ptrs = (C.c_void_p * len(keep))(*[None if p is None else p.ctypes.data for p in keep])
+    return keep, ptrs
+
+
+def partial_eval(tensor, padded_dims, unpadded_dims, kinds, points):
+    tensor = np.ascontiguousarray(tensor, dtype=np.int64)
+    nd = len(padded_dims)
+    pd = (C.c_uint64 * nd)(*padded_dims)
+    ud = (C.c_uint64 * nd)(*unpadded_dims)
+    kd = (C.c_int32 * nd)(*kinds)
+    keep, ptrs = _points_ptrs(points)
+    cap = 1
+    for d in unpadded_dims:
+        cap *= d
+    cap = 2 * cap + 2
+    out = np.zeros((cap, 2), dtype=np.uint64)
+    tl = C.c_uint64(0)
+    n = lib().orc_partial_eval(_p(tensor), pd, ud, C.c_uint32(nd), kd, ptrs, _p(out), C.c_uint64(cap), C.byref(tl))
+    if n < 0:
+        raise ValueError(f"orc_partial_eval failed: {n}")
+    return out[: n * tl.value].reshape(n, tl.value, 2).copy()
+
+
+def stacking_coeffs(padded_dims, unpadded_dims, kinds, points):
+    nd = len(padded_dims)
+    pd = (C.c_uint64 * nd)(*padded_dims)
+    ud = (C.c_uint64 * nd)(*unpadded_dims)
+    kd = (C.c_int32 * nd)(*kinds)
+    keep, ptrs = _points_ptrs(points)
+    cap = 1
+    for d, k in zip(unpadded_dims, kinds):
+        if k == AXIS_STACKED:
+            cap *= d
+    out = np.zeros((cap, 2), dtype=np.uint64)
+    n = lib().orc_stacking_coeffs(pd, ud, C.c_uint32(nd), kd, ptrs, _p(out), C.c_uint64(cap))
+    if n < 0:
+        raise ValueError(f"orc_stacking_coeffs failed: {n}")
+    return out[:n].copy()
+
+
+# ---- LogUp ----
+def logup_build(cols, numer, c, beta):
+    cols = [np.ascontiguousarray(x, dtype=np.uint64) for x in cols]
+    ln = cols[0].size
+    ptrs = (C.c_void_p * len(cols))(*[x.ctypes.data for x in cols])
+    nm = None if numer is None else np.ascontiguousarray(numer, dtype=np.uint64)
+    alen = lib().orc_logup_arena_len(C.c_uint64(ln))
+    arena = np.zeros((alen + 1, 2), dtype=np.uint64)
+    cc, bb = _e2arr(c), _e2arr(beta)
+    lib().orc_logup_build(ptrs, C.c_uint32(len(cols)), None if nm is None else _p(nm), C.c_uint64(ln), _p(cc), _p(bb),
+                          _p(arena))
+    layers = []
+    top = ln.bit_length() - 1
+    for k in range(1, top):
+        off = lib().orc_logup_layer_offset(C.c_uint64(ln), C.c_uint32(k))
+        sz = ln >> k
+        layers.append((arena[off:off + sz].copy(), arena[off + sz:off + 2 * sz].copy()))
+    return layers
+
+
+def _instances(instances):
+    """instances: list of dicts {cols: [u64 arrays], numer: array|None, c: e2, beta: e2}"""
+    arr = (LogupInstance * len(instances))()
+    keep = []
+    for i, ins in enumerate(instances):
+        cols = [np.ascontiguousarray(x, dtype=np.uint64) for x in ins["cols"]]
+        ptrs = (C.c_void_p * len(cols))(*[x.ctypes.data for x in cols])
+        nm = None if ins.get("numer") is None else np.ascontiguousarray(ins["numer"], dtype=np.uint64)
+        keep.append((cols, ptrs, nm))
+        arr[i].n_cols = len(cols)
+        arr[i].len = cols[0].size
+        arr[i].cols = C.cast(ptrs, C.POINTER(C.c_void_p))
+        arr[i].numer = None if nm is None else nm.ctypes.data
+        c, b = _e2arr(ins["c"]), _e2arr(ins["beta"])
+        arr[i].c[0], arr[i].c[1] = int(c[0]), int(c[1])
+        arr[i].beta[0], arr[i].beta[1] = int(b[0]), int(b[1])
+    return arr, keep
+
+
+def logup_batch_prove(instances, transcript):
+    """Returns the flat proof stream (see orc_logup_batch_prove)."""
+    arr, keep = _instances(instances)
+    total = max(int(i["cols"][0].size).bit_length() - 2 for i in instances)
+    cap = sum(v * 4 for v in range(1, total + 1))
+    cap += (total + 2) * sum(2 * len(i["cols"]) + 6 for i in instances) + total + 8
+    out = np.zeros((cap, 2), dtype=np.uint64)
+    n = lib().orc_logup_batch_prove(arr, C.c_uint32(len(instances)), C.byref(transcript.t), _p(out), C.c_uint64(cap))
+    if n < 0:
+        raise ValueError(f"orc_logup_batch_prove failed: {n}")
+    return out[:n].copy()
+
+
+def logup_batch_verify(instances_meta, is_table, stream, transcript):
+    """instances_meta: list of (n_cols, num_vars, c, beta).  Returns (rc, claims, point)."""
+    n = len(instances_meta)
+    ncols = (C.c_uint32 * n)(*[m[0] for m in instances_meta])
+    nvars = (C.c_uint32 * n)(*[m[1] for m in instances_meta])
+    cs = np.stack([_e2arr(m[2]) for m in instances_meta])
+    bs = np.stack([_e2arr(m[3]) for m in instances_meta])
+    stream = _e2arr(stream)
+    total = max(m[1] for m in instances_meta)
+    n_claims = sum(m[0] + (1 if is_table else 0) for m in instances_meta)
+    claims = np.zeros((n_claims, 2), dtype=np.uint64)
+    point = np.zeros((total + 1, 2), dtype=np.uint64)
+    rc = lib().orc_logup_batch_verify(ncols, nvars, _p(cs), _p(bs), C.c_int(1 if is_table else 0), C.c_uint32(n),
+                                      _p(stream), C.c_uint64(stream.shape[0]), C.byref(transcript.t), _p(claims),
+                                      _p(point))
+    return rc, claims, point
+
+
+def num_threads():
+    return lib().orc_num_threads()
