@@ -1,0 +1,460 @@
+"""MI355X sumcheck prover: Python bindings of the C ABI (libdpsumcheck.so, the
+HIP library) and of the C++ host mirror (libdpsc_host.so: transcript,
+prove/verify loops, einsum and LogUp drivers).
+
+The directory name carries a hyphen, so load it with
+``importlib.import_module("deep-prove_amd")``.
+
+There is no CPU implementation behind these calls: if the HIP library has not
+been built, importing this package fails; on a machine without a GPU
+``Context()`` fails.  Extension-field values cross as numpy uint64 arrays whose
+last axis is (c0, c1).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+P = 0xFFFFFFFF00000001
+MAX_FACTORS = 8
+AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
+KIND_BASE, KIND_EXT2, KIND_I64 = 0, 1, 2
+KERNELS = ["eval_first", "fold_eval", "eval_terms", "fold", "eq", "axis_dot", "logup", "finalize"]
+
+
+class DpsError(RuntimeError):
+    def __init__(self, status, msg):
+        super().__init__(f"[status {status}] {msg}")
+        self.status = status
+
+
+def _load(name):
+    path = os.path.join(LIB_DIR, name)
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')")
+    return C.CDLL(path, mode=C.RTLD_GLOBAL)
+
+
+dev = _load("libdpsumcheck.so")
+host = _load("libdpsc_host.so")
+
+
+class Term(C.Structure):
+    _fields_ = [("coeff", C.c_uint64 * 2), ("n_factors", C.c_uint32), ("factors", C.c_uint32 * MAX_FACTORS)]
+
+
+_vp, _u32, _u64, _i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32
+dev.dps_last_error.restype = C.c_char_p
+dev.dps_last_error.argtypes = [_vp]
+dev.dps_status_str.restype = C.c_char_p
+dev.dps_kernel_name.restype = C.c_char_p
+host.dph_last_error.restype = C.c_char_p
+host.dph_tr_new.restype = _vp
+host.dph_tr_new.argtypes = [C.c_char_p]
+host.dph_tr_clone.restype = _vp
+host.dph_tr_clone.argtypes = [_vp]
+for _f, _a in [("dph_tr_free", [_vp]), ("dph_tr_append_message", [_vp, C.c_char_p]),
+               ("dph_tr_append_bytes", [_vp, C.c_char_p, C.c_size_t]), ("dph_tr_append_u64", [_vp, _u64]),
+               ("dph_tr_append_scalars", [_vp, _vp, C.c_size_t]), ("dph_tr_challenge_scalar", [_vp, _vp]),
+               ("dph_tr_append_and_sample", [_vp, C.c_char_p, _vp]), ("dph_tr_state", [_vp, _vp, _vp]),
+               ("dph_blake3", [C.c_char_p, C.c_size_t, _vp])]:
+    getattr(host, _f).restype = None
+    getattr(host, _f).argtypes = _a
+
+# every dps_* entry point takes pointers and integers; declare the ones whose
+# integer arguments are 64-bit so that ctypes does not truncate them
+dev.dps_mle_from_i64.argtypes = [_vp, _vp, _u64, _u32, _vp]
+dev.dps_tensor_from_i64.argtypes = [_vp, _vp, _u64, _vp]
+dev.dps_mle_wrap_device.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
+dev.dps_mle_view.argtypes = [_vp, _u64, _u32, _vp]
+dev.dps_debug_field_op.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
+for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
+           "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
+           "dps_partial_eval", "dps_sc_begin", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_free",
+           "dps_sc_prove", "dps_logup_build", "dps_logup_num_layers", "dps_logup_layer", "dps_logup_outputs",
+           "dps_logup_free", "dps_profile_enable", "dps_profile_reset", "dps_profile_read"]:
+    getattr(dev, _f).restype = _i32
+dev.dps_ctx_create.argtypes = [_i32, _vp]
+dev.dps_ctx_destroy.argtypes = [_vp]
+dev.dps_ctx_sync.argtypes = [_vp]
+dev.dps_mle_from_base.argtypes = [_vp, _vp, _u32, _vp]
+dev.dps_mle_from_ext2.argtypes = [_vp, _vp, _vp, _u32, _vp]
+dev.dps_mle_info.argtypes = [_vp, _vp, _vp]
+dev.dps_mle_download.argtypes = [_vp, _vp, _vp]
+dev.dps_mle_free.argtypes = [_vp]
+dev.dps_eq_build.argtypes = [_vp, _vp, _u32, _vp]
+dev.dps_mle_evaluate.argtypes = [_vp, _vp, _vp, _u32, _vp]
+dev.dps_mle_fix_low.argtypes = [_vp, _vp, _vp, _u32, _vp]
+dev.dps_mle_fix_high.argtypes = [_vp, _vp, _vp, _u32, _vp]
+dev.dps_partial_eval.argtypes = [_vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _u32, _vp]
+dev.dps_sc_begin.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp]
+dev.dps_sc_degree.argtypes = [_vp, _vp]
+dev.dps_sc_round.argtypes = [_vp, _vp, _vp]
+dev.dps_sc_finish.argtypes = [_vp, _vp, _vp]
+dev.dps_sc_free.argtypes = [_vp]
+dev.dps_sc_prove.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
+dev.dps_logup_build.argtypes = [_vp, _vp, _u32, _vp, _vp, _vp, _vp]
+dev.dps_logup_num_layers.argtypes = [_vp, _vp]
+dev.dps_logup_layer.argtypes = [_vp, _u32, _vp, _vp]
+dev.dps_logup_outputs.argtypes = [_vp, _vp]
+dev.dps_logup_free.argtypes = [_vp]
+dev.dps_profile_enable.argtypes = [_vp, _i32]
+dev.dps_profile_reset.argtypes = [_vp]
+dev.dps_profile_read.argtypes = [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]
+host.dph_sumcheck_prove.restype = _i32
+host.dph_sumcheck_prove.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]
+host.dph_sumcheck_verify.restype = _i32
+host.dph_sumcheck_verify.argtypes = [_vp, _vp, _u32, _u32, _vp, _vp, _vp]
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_vp)
+
+
+def _e2(x):
+    a = np.ascontiguousarray(x, dtype=np.uint64)
+    assert a.shape[-1] == 2, a.shape
+    return a
+
+
+def make_terms(terms):
+    """terms: iterable of (coeff (c0, c1), [table indices])."""
+    terms = list(terms)
+    arr = (Term * max(1, len(terms)))()
+    for i, (coeff, factors) in enumerate(terms):
+        c = _e2(coeff)
+        arr[i].coeff[0], arr[i].coeff[1] = int(c[0]), int(c[1])
+        arr[i].n_factors = len(factors)
+        for k, f in enumerate(factors):
+            arr[i].factors[k] = f
+    return arr, len(terms)
+
+
+class Transcript:
+    """Blake3Transcript of the host mirror."""
+
+    def __init__(self, label=b"m2vec", _raw=None):
+        self._t = _raw if _raw is not None else host.dph_tr_new(label)
+
+    def __del__(self):
+        if getattr(self, "_t", None):
+            host.dph_tr_free(self._t)
+            self._t = None
+
+    def clone(self):
+        return Transcript(_raw=host.dph_tr_clone(self._t))
+
+    def append_message(self, label: bytes):
+        host.dph_tr_append_message(self._t, label)
+
+    def append_bytes(self, data: bytes):
+        host.dph_tr_append_bytes(self._t, data, len(data))
+
+    def append_u64(self, x):
+        host.dph_tr_append_u64(self._t, x)
+
+    def append_scalars(self, xs):
+        xs = _e2(xs).reshape(-1, 2)
+        host.dph_tr_append_scalars(self._t, _ptr(xs), xs.shape[0])
+
+    def challenge_scalar(self):
+        out = np.zeros(2, dtype=np.uint64)
+        host.dph_tr_challenge_scalar(self._t, _ptr(out))
+        return out
+
+    def append_and_sample(self, label: bytes):
+        out = np.zeros(2, dtype=np.uint64)
+        host.dph_tr_append_and_sample(self._t, label, _ptr(out))
+        return out
+
+    def read_challenges(self, n):
+        return np.stack([self.challenge_scalar() for _ in range(n)]) if n else np.zeros((0, 2), np.uint64)
+
+    def state(self):
+        st = (C.c_uint8 * 32)()
+        n = C.c_uint32(0)
+        host.dph_tr_state(self._t, st, C.byref(n))
+        return bytes(st), int(n.value)
+
+
+def blake3(data: bytes) -> bytes:
+    out = (C.c_uint8 * 32)()
+    host.dph_blake3(data, len(data), out)
+    return bytes(out)
+
+
+class Mle:
+    """A table in HBM (owned, borrowed or a view)."""
+
+    def __init__(self, ctx, handle):
+        self.ctx, self._h = ctx, handle
+
+    def __del__(self):
+        self.free()
+
+    def free(self):
+        if getattr(self, "_h", None) and self.ctx._c:
+            dev.dps_mle_free(self._h)
+        self._h = None
+
+    @property
+    def handle(self):
+        return self._h
+
+    def info(self):
+        k, n = _i32(0), _u64(0)
+        self.ctx._chk(dev.dps_mle_info(self._h, C.byref(k), C.byref(n)), "dps_mle_info")
+        return int(k.value), int(n.value)
+
+    def __len__(self):
+        return self.info()[1]
+
+    @property
+    def kind(self):
+        return self.info()[0]
+
+    def download(self):
+        """(len, 2) uint64 for field tables; int64 vector for raw tensors."""
+        kind, n = self.info()
+        c0 = np.zeros(n, dtype=np.uint64)
+        c1 = np.zeros(n, dtype=np.uint64)
+        self.ctx._chk(dev.dps_mle_download(self._h, _ptr(c0), _ptr(c1)), "dps_mle_download")
+        if kind == KIND_I64:
+            return c0.view(np.int64)
+        return np.stack([c0, c1], axis=-1)
+
+    def view(self, offset, n_vars):
+        h = _vp()
+        self.ctx._chk(dev.dps_mle_view(self._h, offset, n_vars, C.byref(h)), "dps_mle_view")
+        return Mle(self.ctx, h)
+
+    def evaluate(self, point):
+        point = _e2(point).reshape(-1, 2)
+        out = np.zeros(2, dtype=np.uint64)
+        self.ctx._chk(dev.dps_mle_evaluate(self.ctx._c, self._h, _ptr(point), point.shape[0], _ptr(out)), "dps_mle_evaluate")
+        return out
+
+    def fix_low(self, point):
+        point = _e2(point).reshape(-1, 2)
+        h = _vp()
+        self.ctx._chk(dev.dps_mle_fix_low(self.ctx._c, self._h, _ptr(point), point.shape[0], C.byref(h)), "dps_mle_fix_low")
+        return Mle(self.ctx, h)
+
+    def fix_high(self, point):
+        point = _e2(point).reshape(-1, 2)
+        h = _vp()
+        self.ctx._chk(dev.dps_mle_fix_high(self.ctx._c, self._h, _ptr(point), point.shape[0], C.byref(h)), "dps_mle_fix_high")
+        return Mle(self.ctx, h)
+
+
+class Logup:
+    def __init__(self, ctx, handle):
+        self.ctx, self._h = ctx, handle
+
+    def __del__(self):
+        if getattr(self, "_h", None) and self.ctx._c:
+            dev.dps_logup_free(self._h)
+        self._h = None
+
+    def num_layers(self):
+        n = _u32(0)
+        self.ctx._chk(dev.dps_logup_num_layers(self._h, C.byref(n)), "dps_logup_num_layers")
+        return int(n.value)
+
+    def layer(self, k):
+        a, b = _vp(), _vp()
+        self.ctx._chk(dev.dps_logup_layer(self._h, k, C.byref(a), C.byref(b)), "dps_logup_layer")
+        return Mle(self.ctx, a), Mle(self.ctx, b)
+
+    def outputs(self):
+        out = np.zeros((4, 2), dtype=np.uint64)
+        self.ctx._chk(dev.dps_logup_outputs(self._h, _ptr(out)), "dps_logup_outputs")
+        return out
+
+
+class Session:
+    """Round-by-round access to a sumcheck (dps_sc_begin / round / finish)."""
+
+    def __init__(self, ctx, n_vars, mles, terms):
+        self.ctx, self.n_vars, self.n_mles = ctx, n_vars, len(mles)
+        self._keep = list(mles)
+        hs = (_vp * max(1, len(mles)))(*[m.handle for m in mles])
+        tarr, nt = make_terms(terms)
+        h = _vp()
+        ctx._chk(dev.dps_sc_begin(ctx._c, n_vars, hs, len(mles), tarr, nt, C.byref(h)), "dps_sc_begin")
+        self._h = h
+        d = _u32(0)
+        dev.dps_sc_degree(h, C.byref(d))
+        self.degree = int(d.value)
+
+    def __del__(self):
+        if getattr(self, "_h", None) and self.ctx._c:
+            dev.dps_sc_free(self._h)
+        self._h = None
+
+    def round(self, challenge=None):
+        out = np.zeros((self.degree + 1, 2), dtype=np.uint64)
+        ch = None if challenge is None else _e2(challenge)
+        self.ctx._chk(dev.dps_sc_round(self._h, None if ch is None else _ptr(ch), _ptr(out)), "dps_sc_round")
+        return out
+
+    def finish(self, challenge=None):
+        out = np.zeros((max(1, self.n_mles), 2), dtype=np.uint64)
+        ch = None if challenge is None else _e2(challenge)
+        self.ctx._chk(dev.dps_sc_finish(self._h, None if ch is None else _ptr(ch), _ptr(out)), "dps_sc_finish")
+        return out[: self.n_mles]
+
+
+class Context:
+    """One GPU context: a HIP stream plus a device memory pool."""
+
+    def __init__(self, device=0):
+        self._c = None
+        c = _vp()
+        rc = dev.dps_ctx_create(device, C.byref(c))
+        if rc != 0:
+            raise DpsError(rc, "dps_ctx_create failed (no usable GPU?): " + dev.dps_status_str(rc).decode())
+        self._c = c
+
+    def __del__(self):
+        self.close()
+
+    def close(self):
+        if getattr(self, "_c", None):
+            dev.dps_ctx_destroy(self._c)
+        self._c = None
+
+    def _chk(self, rc, what):
+        if rc != 0:
+            raise DpsError(rc, f"{what}: {dev.dps_status_str(rc).decode()}: {dev.dps_last_error(self._c).decode()}")
+
+    def _chk_host(self, rc, what):
+        if rc != 0:
+            raise DpsError(rc, f"{what}: {host.dph_last_error().decode()}")
+
+    def sync(self):
+        self._chk(dev.dps_ctx_sync(self._c), "dps_ctx_sync")
+
+    # ---- tables ----
+    def mle_from_base(self, v):
+        v = np.ascontiguousarray(v, dtype=np.uint64)
+        nv = int(v.size).bit_length() - 1
+        assert 1 << nv == v.size, "length must be a power of two"
+        h = _vp()
+        self._chk(dev.dps_mle_from_base(self._c, _ptr(v), nv, C.byref(h)), "dps_mle_from_base")
+        return Mle(self, h)
+
+    def mle_from_ext2(self, v):
+        v = _e2(v).reshape(-1, 2)
+        nv = int(v.shape[0]).bit_length() - 1
+        assert 1 << nv == v.shape[0], "length must be a power of two"
+        c0, c1 = np.ascontiguousarray(v[:, 0]), np.ascontiguousarray(v[:, 1])
+        h = _vp()
+        self._chk(dev.dps_mle_from_ext2(self._c, _ptr(c0), _ptr(c1), nv, C.byref(h)), "dps_mle_from_ext2")
+        return Mle(self, h)
+
+    def mle_from_i64(self, v, n_vars=None):
+        v = np.ascontiguousarray(v, dtype=np.int64).reshape(-1)
+        if n_vars is None:
+            n_vars = max(0, int(v.size - 1).bit_length())
+        h = _vp()
+        self._chk(dev.dps_mle_from_i64(self._c, _ptr(v), v.size, n_vars, C.byref(h)), "dps_mle_from_i64")
+        return Mle(self, h)
+
+    def tensor_from_i64(self, v):
+        v = np.ascontiguousarray(v, dtype=np.int64).reshape(-1)
+        h = _vp()
+        self._chk(dev.dps_tensor_from_i64(self._c, _ptr(v), v.size, C.byref(h)), "dps_tensor_from_i64")
+        return Mle(self, h)
+
+    def wrap_device(self, kind, ptr_c0, ptr_c1, length):
+        h = _vp()
+        self._chk(dev.dps_mle_wrap_device(self._c, kind, ptr_c0, ptr_c1, length, C.byref(h)), "dps_mle_wrap_device")
+        return Mle(self, h)
+
+    def eq_build(self, point):
+        point = _e2(point).reshape(-1, 2)
+        h = _vp()
+        self._chk(dev.dps_eq_build(self._c, _ptr(point), point.shape[0], C.byref(h)), "dps_eq_build")
+        return Mle(self, h)
+
+    def partial_eval(self, tensor, padded_dims, unpadded_dims, kinds, points):
+        nd = len(padded_dims)
+        pd = (_u64 * nd)(*padded_dims)
+        ud = (_u64 * nd)(*unpadded_dims)
+        kd = (_i32 * nd)(*kinds)
+        keep = [None if p is None else _e2(p).reshape(-1, 2) for p in points]
+        pts = (_vp * nd)(*[None if p is None else p.ctypes.data for p in keep])
+        cap = 1
+        for d, k in zip(unpadded_dims, kinds):
+            if k == AXIS_STACKED:
+                cap *= d
+        out = (_vp * cap)()
+        n = _u32(0)
+        self._chk(dev.dps_partial_eval(self._c, tensor.handle, pd, ud, nd, kd, pts, out, cap, C.byref(n)), "dps_partial_eval")
+        return [Mle(self, _vp(out[i])) for i in range(n.value)]
+
+    # ---- sumcheck ----
+    def session(self, n_vars, mles, terms):
+        return Session(self, n_vars, mles, terms)
+
+    def sumcheck_prove(self, n_vars, mles, terms, transcript):
+        """IOPProverState::prove with the native transcript.
+        Returns (proof[n_vars, d+1, 2], point[n_vars, 2], final_evals[n_mles, 2])."""
+        hs = (_vp * max(1, len(mles)))(*[m.handle for m in mles])
+        tarr, nt = make_terms(terms)
+        degree = max((len(f) for _, f in terms), default=0)
+        proof = np.zeros((n_vars, degree + 1, 2), dtype=np.uint64)
+        point = np.zeros((n_vars, 2), dtype=np.uint64)
+        finals = np.zeros((max(1, len(mles)), 2), dtype=np.uint64)
+        d = _u32(0)
+        self._chk_host(host.dph_sumcheck_prove(self._c, n_vars, hs, len(mles), tarr, nt, transcript._t, _ptr(proof), _ptr(point),
+                                               _ptr(finals), C.byref(d)), "dph_sumcheck_prove")
+        return proof, point, finals[: len(mles)]
+
+    def sumcheck_verify(self, claimed_sum, proof, transcript):
+        proof = _e2(proof)
+        n_vars, npts = proof.shape[0], proof.shape[1]
+        cs = _e2(claimed_sum)
+        point = np.zeros((n_vars, 2), dtype=np.uint64)
+        expected = np.zeros(2, dtype=np.uint64)
+        rc = host.dph_sumcheck_verify(_ptr(cs), _ptr(proof), n_vars, npts - 1, transcript._t, _ptr(point), _ptr(expected))
+        return rc, point, expected
+
+    # ---- LogUp ----
+    def logup_build(self, cols, numer, c, beta):
+        hs = (_vp * len(cols))(*[m.handle for m in cols])
+        cc, bb = _e2(c), _e2(beta)
+        h = _vp()
+        self._chk(dev.dps_logup_build(self._c, hs, len(cols), None if numer is None else numer.handle, _ptr(cc), _ptr(bb), C.byref(h)),
+                  "dps_logup_build")
+        return Logup(self, h)
+
+    # ---- measurement ----
+    def profile(self, on=True):
+        self._chk(dev.dps_profile_enable(self._c, 1 if on else 0), "dps_profile_enable")
+
+    def profile_reset(self):
+        self._chk(dev.dps_profile_reset(self._c), "dps_profile_reset")
+
+    def profile_read(self):
+        out = {}
+        for k, name in enumerate(KERNELS):
+            n, mn = _u64(0), _u64(0)
+            ms, by, mms, mby = C.c_double(0), C.c_double(0), C.c_double(0), C.c_double(0)
+            self._chk(dev.dps_profile_read(self._c, k, C.byref(n), C.byref(ms), C.byref(by), C.byref(mn), C.byref(mms), C.byref(mby)),
+                      "dps_profile_read")
+            out[name] = dict(launches=n.value, ms=ms.value, bytes=by.value, max_launches=mn.value, max_ms=mms.value, max_bytes=mby.value,
+                             symbol=dev.dps_kernel_name(k).decode())
+        return out
+
+    def field_op(self, op, a, b):
+        a, b = _e2(a).reshape(-1, 2), _e2(b).reshape(-1, 2)
+        n = a.shape[0]
+        aa = np.ascontiguousarray(np.concatenate([a[:, 0], a[:, 1]]))
+        bb = np.ascontiguousarray(np.concatenate([b[:, 0], b[:, 1]]))
+        out = np.zeros(2 * n, dtype=np.uint64)
+        self._chk(dev.dps_debug_field_op(self._c, op, _ptr(aa), _ptr(bb), n, _ptr(out)), "dps_debug_field_op")
+        return np.stack([out[:n], out[n:]], axis=-1)

@@ -1,0 +1,1565 @@
+// C ABI of the sumcheck prover library: contexts, table storage, sessions.
+// Device code is in kernels.hpp; this file owns memory, launch geometry and the
+// round protocol.  There is no CPU path: every entry point that computes
+// launches kernels on the context's stream.
+#include "../../include/dpsumcheck.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "kernels.hpp"
+
+using gl::E2;
+using gl::u32;
+using gl::u64;
+
+namespace {
+
+constexpr u32 MAX_BLOCKS = 2048;  // 8 workgroups per CU on 256 CUs
+
+// ---------------------------------------------------------------------------
+// context
+// ---------------------------------------------------------------------------
+struct ProfRec {
+    int kernel;
+    hipEvent_t a, b;
+    double bytes;
+};
+
+struct ProfStat {
+    u64 launches = 0;
+    double ms = 0, bytes = 0;
+    u64 max_launches = 0;
+    double max_ms = 0, max_bytes = 0;
+};
+
+}  // namespace
+
+struct dps_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string err;
+    // cached device blocks, keyed by size
+    std::multimap<size_t, void *> free_blocks;
+    std::map<void *, size_t> live_blocks;
+    u64 *d_lagrange = nullptr;  // [9][9][9]
+    u64 *h_pinned = nullptr;    // host-visible result buffer
+    u64 *d_pinned = nullptr;    // device address of the same buffer
+    size_t pinned_words = 0;
+    bool profiling = false;
+    std::vector<ProfRec> recs;
+    std::vector<hipEvent_t> ev_pool;
+    ProfStat stats[DPS_K_COUNT];
+};
+
+namespace {
+
+int32_t fail(dps_ctx *ctx, int32_t code, const char *fmt, ...)
+{
+    if (ctx) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof buf, fmt, ap);
+        va_end(ap);
+        ctx->err = buf;
+    }
+    return code;
+}
+
+#define HIPCHK(ctx, call)                                                                                       \
+    do {                                                                                                        \
+        hipError_t e_ = (call);                                                                                 \
+        if (e_ != hipSuccess)                                                                                   \
+            return fail(ctx, e_ == hipErrorOutOfMemory ? DPS_ERR_OOM : DPS_ERR_HIP, "%s: %s (%s:%d)", #call,   \
+                        hipGetErrorString(e_), __FILE__, __LINE__);                                             \
+    } while (0)
+
+#define CHK(expr)                       \
+    do {                                \
+        int32_t rc_ = (expr);           \
+        if (rc_ != DPS_OK) return rc_;  \
+    } while (0)
+
+struct DeviceGuard {
+    int prev = -1;
+    explicit DeviceGuard(int dev)
+    {
+        if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+        if (prev != dev) (void)hipSetDevice(dev);
+    }
+    ~DeviceGuard()
+    {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+int32_t pool_alloc(dps_ctx *ctx, size_t bytes, void **out)
+{
+    bytes = round_up(std::max<size_t>(bytes, 256), 256);
+    auto it = ctx->free_blocks.lower_bound(bytes);
+    if (it != ctx->free_blocks.end() && it->first <= bytes + bytes / 2 + 4096) {
+        *out = it->second;
+        ctx->live_blocks[it->second] = it->first;
+        ctx->free_blocks.erase(it);
+        return DPS_OK;
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+        // give cached blocks back to the driver and retry once
+        for (auto &kv : ctx->free_blocks) (void)hipFree(kv.second);
+        ctx->free_blocks.clear();
+        e = hipMalloc(&p, bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(ctx, DPS_ERR_OOM, "hipMalloc(%zu bytes): %s", bytes, hipGetErrorString(e));
+        }
+    }
+    ctx->live_blocks[p] = bytes;
+    *out = p;
+    return DPS_OK;
+}
+
+void pool_free(dps_ctx *ctx, void *p)
+{
+    if (!p) return;
+    auto it = ctx->live_blocks.find(p);
+    if (it == ctx->live_blocks.end()) return;
+    ctx->free_blocks.emplace(it->second, p);
+    ctx->live_blocks.erase(it);
+}
+
+// profiling -----------------------------------------------------------------
+hipEvent_t prof_event(dps_ctx *ctx)
+{
+    if (!ctx->ev_pool.empty()) {
+        hipEvent_t e = ctx->ev_pool.back();
+        ctx->ev_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
+struct ProfScope {
+    dps_ctx *ctx;
+    ProfRec rec;
+    bool on;
+    ProfScope(dps_ctx *c, int kernel, double bytes) : ctx(c), on(c->profiling)
+    {
+        if (!on) return;
+        rec.kernel = kernel;
+        rec.bytes = bytes;
+        rec.a = prof_event(ctx);
+        rec.b = prof_event(ctx);
+        (void)hipEventRecord(rec.a, ctx->stream);
+    }
+    ~ProfScope()
+    {
+        if (!on) return;
+        (void)hipEventRecord(rec.b, ctx->stream);
+        ctx->recs.push_back(rec);
+    }
+};
+
+void prof_collect(dps_ctx *ctx)
+{
+    for (auto &r : ctx->recs) {
+        float ms = 0;
+        (void)hipEventSynchronize(r.b);
+        (void)hipEventElapsedTime(&ms, r.a, r.b);
+        ProfStat &s = ctx->stats[r.kernel];
+        s.launches++;
+        s.ms += ms;
+        s.bytes += r.bytes;
+        if (r.bytes > s.max_bytes * 1.0000001) {
+            s.max_bytes = r.bytes;
+            s.max_ms = ms;
+            s.max_launches = 1;
+        } else if (r.bytes >= s.max_bytes * 0.9999999 && s.max_launches > 0) {
+            s.max_ms += ms;
+            s.max_launches++;
+        }
+        ctx->ev_pool.push_back(r.a);
+        ctx->ev_pool.push_back(r.b);
+    }
+    ctx->recs.clear();
+}
+
+u32 grid_for(u64 items, u32 per_block = dpk::BLOCK)
+{
+    u64 b = (items + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    return (u32)std::min<u64>(b, MAX_BLOCKS);
+}
+
+// host-side field helpers for constants (Lagrange weights, powers of two)
+u64 h_pow(u64 a, u64 e)
+{
+    u64 r = 1;
+    while (e) {
+        if (e & 1) r = gl::mul(r, a);
+        a = gl::mul(a, a);
+        e >>= 1;
+    }
+    return r;
+}
+u64 h_inv(u64 a) { return h_pow(a, gl::P - 2); }
+
+// ---------------------------------------------------------------------------
+// storage
+// ---------------------------------------------------------------------------
+struct Storage {
+    dps_ctx *ctx = nullptr;
+    u64 *c0 = nullptr;
+    u64 *c1 = nullptr;
+    bool owned = true;
+    ~Storage()
+    {
+        if (owned && ctx) {
+            pool_free(ctx, c0);
+            pool_free(ctx, c1);
+        }
+    }
+};
+
+}  // namespace
+
+struct dps_mle {
+    dps_ctx *ctx;
+    std::shared_ptr<Storage> st;
+    int32_t kind;
+    u64 offset;
+    u64 len;
+    const u64 *p0() const { return st->c0 + offset; }
+    const u64 *p1() const { return st->c1 ? st->c1 + offset : nullptr; }
+};
+
+namespace {
+
+bool is_pow2(u64 x) { return x && !(x & (x - 1)); }
+u32 log2u(u64 x)
+{
+    u32 l = 0;
+    while ((1ull << l) < x) l++;
+    return l;
+}
+
+int32_t new_table(dps_ctx *ctx, int32_t kind, u64 len, dps_mle **out)
+{
+    auto st = std::make_shared<Storage>();
+    st->ctx = ctx;
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, len * 8, &p));
+    st->c0 = (u64 *)p;
+    if (kind == DPS_EXT2) {
+        CHK(pool_alloc(ctx, len * 8, &p));
+        st->c1 = (u64 *)p;
+    }
+    dps_mle *m = new (std::nothrow) dps_mle{ctx, st, kind, 0, len};
+    if (!m) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
+    *out = m;
+    return DPS_OK;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// context entry points
+// ---------------------------------------------------------------------------
+extern "C" const char *dps_status_str(int32_t s)
+{
+    switch (s) {
+    case DPS_OK: return "ok";
+    case DPS_ERR_INVALID: return "invalid argument";
+    case DPS_ERR_HIP: return "HIP runtime error";
+    case DPS_ERR_OOM: return "out of memory";
+    case DPS_ERR_STATE: return "call out of order";
+    case DPS_ERR_UNSUPPORTED: return "unsupported degree or arity";
+    case DPS_ERR_CALLBACK: return "transcript callback failed";
+    default: return "unknown status";
+    }
+}
+
+extern "C" const char *dps_kernel_name(int32_t k)
+{
+    static const char *names[DPS_K_COUNT] = {"prod_kernel<first round>", "prod_kernel<fold+eval>", "eval_terms_kernel",
+                                             "fold_kernel",              "eq_expand_kernel",       "axis_dot_kernel",
+                                             "logup_layer_kernel",       "finalize_kernel"};
+    return (k >= 0 && k < DPS_K_COUNT) ? names[k] : "?";
+}
+
+extern "C" const char *dps_last_error(const dps_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+
+extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
+{
+    if (!out) return DPS_ERR_INVALID;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) {
+        (void)hipGetLastError();
+        return DPS_ERR_HIP;
+    }
+    dps_ctx *ctx = new (std::nothrow) dps_ctx();
+    if (!ctx) return DPS_ERR_OOM;
+    ctx->device = device;
+    DeviceGuard g(device);
+    auto bail = [&](int32_t rc) {
+        delete ctx;
+        return rc;
+    };
+    if (hipStreamCreate(&ctx->stream) != hipSuccess) return bail(DPS_ERR_HIP);
+    // Lagrange weights: a polynomial of degree k known at 0..k, evaluated at t <= 8
+    std::vector<u64> lag(9 * 9 * 9, 0);
+    for (u32 k = 0; k <= 8; k++)
+        for (u32 t = 0; t <= 8; t++)
+            for (u32 i = 0; i <= k; i++) {
+                u64 num = 1, den = 1;
+                for (u32 m = 0; m <= k; m++) {
+                    if (m == i) continue;
+                    num = gl::mul(num, gl::sub((u64)t, (u64)m));
+                    den = gl::mul(den, gl::sub((u64)i, (u64)m));
+                }
+                lag[(k * 9 + t) * 9 + i] = gl::mul(num, h_inv(den));
+            }
+    if (hipMalloc((void **)&ctx->d_lagrange, lag.size() * 8) != hipSuccess) return bail(DPS_ERR_OOM);
+    if (hipMemcpy(ctx->d_lagrange, lag.data(), lag.size() * 8, hipMemcpyHostToDevice) != hipSuccess) return bail(DPS_ERR_HIP);
+    ctx->pinned_words = 4096;
+    if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped) != hipSuccess) return bail(DPS_ERR_OOM);
+    if (hipHostGetDevicePointer((void **)&ctx->d_pinned, ctx->h_pinned, 0) != hipSuccess) return bail(DPS_ERR_HIP);
+    *out = ctx;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
+{
+    if (!ctx) return DPS_OK;
+    DeviceGuard g(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    prof_collect(ctx);
+    for (auto e : ctx->ev_pool) (void)hipEventDestroy(e);
+    for (auto &kv : ctx->free_blocks) (void)hipFree(kv.second);
+    for (auto &kv : ctx->live_blocks) (void)hipFree(kv.first);
+    if (ctx->d_lagrange) (void)hipFree(ctx->d_lagrange);
+    if (ctx->h_pinned) (void)hipHostFree(ctx->h_pinned);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_ctx_sync(dps_ctx *ctx)
+{
+    if (!ctx) return DPS_ERR_INVALID;
+    DeviceGuard g(ctx->device);
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_profile_enable(dps_ctx *ctx, int32_t on)
+{
+    if (!ctx) return DPS_ERR_INVALID;
+    ctx->profiling = on != 0;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_profile_reset(dps_ctx *ctx)
+{
+    if (!ctx) return DPS_ERR_INVALID;
+    DeviceGuard g(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    prof_collect(ctx);
+    for (auto &s : ctx->stats) s = ProfStat();
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_profile_read(dps_ctx *ctx, int32_t kernel, uint64_t *launches, double *total_ms, double *total_bytes,
+                                    uint64_t *max_launches, double *max_ms, double *max_bytes)
+{
+    if (!ctx || kernel < 0 || kernel >= DPS_K_COUNT) return DPS_ERR_INVALID;
+    DeviceGuard g(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    prof_collect(ctx);
+    const ProfStat &s = ctx->stats[kernel];
+    if (launches) *launches = s.launches;
+    if (total_ms) *total_ms = s.ms;
+    if (total_bytes) *total_bytes = s.bytes;
+    if (max_launches) *max_launches = s.max_launches;
+    if (max_ms) *max_ms = s.max_ms;
+    if (max_bytes) *max_bytes = s.max_bytes;
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// table storage
+// ---------------------------------------------------------------------------
+extern "C" int32_t dps_mle_from_base(dps_ctx *ctx, const uint64_t *host, uint32_t n_vars, dps_mle **out)
+{
+    if (!ctx || !host || !out || n_vars > 40) return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_base: bad argument");
+    DeviceGuard g(ctx->device);
+    u64 len = 1ull << n_vars;
+    dps_mle *m = nullptr;
+    CHK(new_table(ctx, DPS_BASE, len, &m));
+    hipError_t e = hipMemcpyAsync(m->st->c0, host, len * 8, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        delete m;
+        return fail(ctx, DPS_ERR_HIP, "upload: %s", hipGetErrorString(e));
+    }
+    *out = m;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_from_ext2(dps_ctx *ctx, const uint64_t *c0, const uint64_t *c1, uint32_t n_vars, dps_mle **out)
+{
+    if (!ctx || !c0 || !c1 || !out || n_vars > 40) return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_ext2: bad argument");
+    DeviceGuard g(ctx->device);
+    u64 len = 1ull << n_vars;
+    dps_mle *m = nullptr;
+    CHK(new_table(ctx, DPS_EXT2, len, &m));
+    hipError_t e = hipMemcpyAsync(m->st->c0, c0, len * 8, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(m->st->c1, c1, len * 8, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        delete m;
+        return fail(ctx, DPS_ERR_HIP, "upload: %s", hipGetErrorString(e));
+    }
+    *out = m;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_tensor_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, dps_mle **out)
+{
+    if (!ctx || !out || (len && !host)) return fail(ctx, DPS_ERR_INVALID, "dps_tensor_from_i64: bad argument");
+    DeviceGuard g(ctx->device);
+    dps_mle *m = nullptr;
+    CHK(new_table(ctx, DPS_I64, std::max<u64>(len, 1), &m));
+    m->len = len;
+    if (len) {
+        hipError_t e = hipMemcpyAsync(m->st->c0, host, len * 8, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            delete m;
+            return fail(ctx, DPS_ERR_HIP, "upload: %s", hipGetErrorString(e));
+        }
+    }
+    *out = m;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, uint32_t n_vars, dps_mle **out)
+{
+    if (!ctx || !out || n_vars > 40 || len > (1ull << n_vars) || (len && !host))
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_i64: bad argument");
+    DeviceGuard g(ctx->device);
+    dps_mle *raw = nullptr;
+    CHK(dps_tensor_from_i64(ctx, host, len, &raw));
+    u64 padded = 1ull << n_vars;
+    dps_mle *m = nullptr;
+    int32_t rc = new_table(ctx, DPS_BASE, padded, &m);
+    if (rc != DPS_OK) {
+        delete raw;
+        return rc;
+    }
+    dpk::embed_i64_kernel<<<grid_for(padded), dpk::BLOCK, 0, ctx->stream>>>((const int64_t *)raw->st->c0, len, padded, m->st->c0);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    delete raw;
+    if (e != hipSuccess) {
+        delete m;
+        return fail(ctx, DPS_ERR_HIP, "embed: %s", hipGetErrorString(e));
+    }
+    *out = m;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, void *d_c1, uint64_t len, dps_mle **out)
+{
+    if (!ctx || !out || !d_c0 || kind < DPS_BASE || kind > DPS_I64 || (kind == DPS_EXT2) != (d_c1 != nullptr))
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_wrap_device: bad argument");
+    if (((uintptr_t)d_c0 & 15) || ((uintptr_t)d_c1 & 15)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_wrap_device: pointers must be 16-byte aligned");
+    auto st = std::make_shared<Storage>();
+    st->ctx = ctx;
+    st->c0 = (u64 *)d_c0;
+    st->c1 = (u64 *)d_c1;
+    st->owned = false;
+    *out = new (std::nothrow) dps_mle{ctx, st, kind, 0, len};
+    return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
+}
+
+extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_vars, dps_mle **out)
+{
+    if (!src || !out) return DPS_ERR_INVALID;
+    dps_ctx *ctx = src->ctx;
+    u64 len = 1ull << n_vars;
+    if (n_vars > 40 || offset > src->len || len > src->len - offset) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: window outside the table");
+    // pair loads are 16 bytes wide
+    if (n_vars >= 1 && ((src->offset + offset) & 1)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: offset must be even");
+    *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len};
+    return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
+}
+
+extern "C" int32_t dps_mle_info(const dps_mle *mle, int32_t *kind, uint64_t *len)
+{
+    if (!mle) return DPS_ERR_INVALID;
+    if (kind) *kind = mle->kind;
+    if (len) *len = mle->len;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *c1)
+{
+    if (!mle || !c0) return DPS_ERR_INVALID;
+    dps_ctx *ctx = mle->ctx;
+    DeviceGuard g(ctx->device);
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (mle->len) HIPCHK(ctx, hipMemcpy(c0, mle->p0(), mle->len * 8, hipMemcpyDeviceToHost));
+    if (c1) {
+        if (mle->kind == DPS_EXT2) {
+            if (mle->len) HIPCHK(ctx, hipMemcpy(c1, mle->p1(), mle->len * 8, hipMemcpyDeviceToHost));
+        } else {
+            memset(c1, 0, mle->len * 8);
+        }
+    }
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_free(dps_mle *mle)
+{
+    if (!mle) return DPS_OK;
+    DeviceGuard g(mle->ctx->device);
+    // work that still reads the storage may be queued
+    (void)hipStreamSynchronize(mle->ctx->stream);
+    delete mle;
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// eq table
+// ---------------------------------------------------------------------------
+namespace {
+
+// uploads `words` 64-bit words through the pinned buffer region [slot, slot+words)
+int32_t stage_words(dps_ctx *ctx, const u64 *src, size_t words, size_t slot, const u64 **dev)
+{
+    if (slot + words > ctx->pinned_words) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
+    // the buffer may still be read by queued kernels
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    memcpy(ctx->h_pinned + slot, src, words * 8);
+    *dev = ctx->d_pinned + slot;
+    return DPS_OK;
+}
+
+bool canonical(const u64 *v, size_t n)
+{
+    for (size_t i = 0; i < n; i++)
+        if (v[i] >= gl::P) return false;
+    return true;
+}
+
+// eq table of point[0..m) (device pointer to 2*m limbs) into out (2^m entries)
+int32_t eq_build_dev(dps_ctx *ctx, const u64 *d_point, u32 m, u64 *o0, u64 *o1)
+{
+    if (m <= 8) {
+        dpk::eq_seed_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(d_point, m, o0, o1);
+        HIPCHK(ctx, hipGetLastError());
+        return DPS_OK;
+    }
+    // low 8 variables as the in-register factor, the rest recursively
+    const u32 b = 8;
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, (256 + (1ull << (m - b))) * 16, &p));
+    u64 *lo0 = (u64 *)p, *lo1 = lo0 + 256, *hi0 = lo1 + 256, *hi1 = hi0 + (1ull << (m - b));
+    int32_t rc = eq_build_dev(ctx, d_point, b, lo0, lo1);
+    if (rc == DPS_OK) rc = eq_build_dev(ctx, d_point + 2 * b, m - b, hi0, hi1);
+    if (rc == DPS_OK) {
+        u64 n_hi = 1ull << (m - b);
+        u32 blocks = (u32)std::min<u64>(n_hi, MAX_BLOCKS * 4);
+        u32 per_block = (u32)((n_hi + blocks - 1) / blocks);
+        blocks = (u32)((n_hi + per_block - 1) / per_block);
+        ProfScope ps(ctx, DPS_K_EQ, (double)(1ull << m) * 16 + (double)n_hi * 16);
+        dpk::eq_expand_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(hi0, hi1, n_hi, lo0, lo1, b, o0, o1, per_block);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq_expand launch: %s", hipGetErrorString(e));
+    }
+    // stream order makes the block reusable by later launches on this stream
+    pool_free(ctx, p);
+    return rc;
+}
+
+}  // namespace
+
+extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m, dps_mle **out)
+{
+    if (!ctx || !out || (m && !point) || m > 34) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: bad argument");
+    if (!canonical(point, 2 * (size_t)m)) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: point not canonical");
+    DeviceGuard g(ctx->device);
+    const u64 *d_point = nullptr;
+    u64 dummy[2] = {0, 0};
+    CHK(stage_words(ctx, m ? point : dummy, m ? 2 * (size_t)m : 2, 0, &d_point));
+    dps_mle *t = nullptr;
+    CHK(new_table(ctx, DPS_EXT2, 1ull << m, &t));
+    int32_t rc = eq_build_dev(ctx, d_point, m, t->st->c0, t->st->c1);
+    if (rc != DPS_OK) {
+        delete t;
+        return rc;
+    }
+    *out = t;
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// contraction of one axis (partial evaluation, evaluate, fix_high)
+// ---------------------------------------------------------------------------
+namespace {
+
+struct AxisJob {
+    const u64 *in0 = nullptr, *in1 = nullptr;
+    bool in_is_i64 = false;
+    const u64 *b0 = nullptr, *b1 = nullptr;
+    u64 K = 1, stride_k = 1;
+    std::vector<u64> pre_dims, pre_strides, post_dims, post_strides;
+    u64 *o0 = nullptr, *o1 = nullptr;
+};
+
+int32_t axis_dot(dps_ctx *ctx, const AxisJob &j)
+{
+    dpk::AxisArgs a;
+    memset(&a, 0, sizeof a);
+    if (j.pre_dims.size() > dpk::AX_MAX_DIMS || j.post_dims.size() > dpk::AX_MAX_DIMS)
+        return fail(ctx, DPS_ERR_UNSUPPORTED, "tensor rank above %d", dpk::AX_MAX_DIMS);
+    a.in0 = j.in0;
+    a.in1 = j.in1;
+    a.in_is_i64 = j.in_is_i64;
+    a.b0 = j.b0;
+    a.b1 = j.b1;
+    a.K = j.K;
+    a.stride_k = j.stride_k;
+    a.n_pre = (u32)j.pre_dims.size();
+    a.n_post = (u32)j.post_dims.size();
+    a.P = a.C = 1;
+    for (u32 d = 0; d < a.n_pre; d++) {
+        a.pre_dims[d] = j.pre_dims[d];
+        a.pre_strides[d] = j.pre_strides[d];
+        a.P *= j.pre_dims[d];
+    }
+    for (u32 d = 0; d < a.n_post; d++) {
+        a.post_dims[d] = j.post_dims[d];
+        a.post_strides[d] = j.post_strides[d];
+        a.C *= j.post_dims[d];
+    }
+    const u64 outputs = a.P * a.C;
+    if (outputs == 0 || a.K == 0) return fail(ctx, DPS_ERR_INVALID, "empty axis contraction");
+    const bool col = a.C >= 32;
+    // split k over workgroups when there are too few outputs to fill the chip
+    const u64 out_blocks = col ? a.P * ((a.C + dpk::WAVE - 1) / dpk::WAVE) : outputs;
+    const u64 k_unit = col ? 64 : 1024;  // k values one workgroup should at least own
+    u32 n_slices = 1;
+    if (out_blocks < 1024 && a.K > k_unit) n_slices = (u32)std::min<u64>((a.K + k_unit - 1) / k_unit, std::max<u64>(1, 2048 / out_blocks));
+    if (n_slices > 65535) n_slices = 65535;
+    a.k_per_slice = (a.K + n_slices - 1) / n_slices;
+    n_slices = (u32)((a.K + a.k_per_slice - 1) / a.k_per_slice);
+    a.n_slices = n_slices;
+    if (out_blocks > 0x7fffffffull) return fail(ctx, DPS_ERR_UNSUPPORTED, "axis contraction too large");
+    void *tmp = nullptr;
+    if (n_slices > 1) {
+        CHK(pool_alloc(ctx, (size_t)n_slices * outputs * 16, &tmp));
+        a.o0 = (u64 *)tmp;
+        a.o1 = a.o0 + (size_t)n_slices * outputs;
+    } else {
+        a.o0 = j.o0;
+        a.o1 = j.o1;
+    }
+    const double elem = j.in1 ? 16.0 : 8.0;
+    hipError_t e;
+    {
+        ProfScope ps(ctx, DPS_K_AXIS_DOT, (double)outputs * (double)a.K * elem + (double)outputs * 16.0);
+        if (col)
+            dpk::axis_dot_col_kernel<<<dim3((u32)out_blocks, n_slices), dpk::BLOCK, 0, ctx->stream>>>(a);
+        else
+            dpk::axis_dot_row_kernel<<<dim3((u32)out_blocks, n_slices), dpk::BLOCK, 0, ctx->stream>>>(a);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess && n_slices > 1) {
+        dpk::slice_sum_kernel<<<(u32)((outputs + dpk::BLOCK - 1) / dpk::BLOCK), dpk::BLOCK, 0, ctx->stream>>>(
+            a.o0, a.o1, outputs, n_slices, j.o0, j.o1);
+        e = hipGetLastError();
+    }
+    pool_free(ctx, tmp);
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "axis_dot launch: %s", hipGetErrorString(e));
+    return DPS_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t n, uint64_t out[2])
+{
+    if (!ctx || !mle || !out || (n && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: bad argument");
+    if (!is_pow2(mle->len) || (1ull << n) != mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: point length does not match the table");
+    DeviceGuard g(ctx->device);
+    dps_mle *eq = nullptr;
+    CHK(dps_eq_build(ctx, point, n, &eq));
+    AxisJob j;
+    j.in0 = mle->p0();
+    j.in1 = mle->p1();
+    j.in_is_i64 = mle->kind == DPS_I64;
+    j.b0 = eq->p0();
+    j.b1 = eq->p1();
+    j.K = mle->len;
+    j.stride_k = 1;
+    // the result lands in the second half of the pinned buffer (the first half staged the point)
+    j.o0 = ctx->d_pinned + ctx->pinned_words / 2;
+    j.o1 = j.o0 + 1;
+    int32_t rc = axis_dot(ctx, j);
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    delete eq;
+    if (rc != DPS_OK) return rc;
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "evaluate: %s", hipGetErrorString(e));
+    out[0] = ctx->h_pinned[ctx->pinned_words / 2];
+    out[1] = ctx->h_pinned[ctx->pinned_words / 2 + 1];
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t k, dps_mle **out)
+{
+    if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: bad argument");
+    if (!is_pow2(mle->len) || (1ull << k) > mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: too many variables");
+    DeviceGuard g(ctx->device);
+    dps_mle *eq = nullptr;
+    CHK(dps_eq_build(ctx, point, k, &eq));
+    u64 rest = mle->len >> k;
+    dps_mle *res = nullptr;
+    int32_t rc = new_table(ctx, DPS_EXT2, rest, &res);
+    if (rc == DPS_OK) {
+        AxisJob j;
+        j.in0 = mle->p0();
+        j.in1 = mle->p1();
+        j.in_is_i64 = mle->kind == DPS_I64;
+        j.b0 = eq->p0();
+        j.b1 = eq->p1();
+        j.K = 1ull << k;
+        j.stride_k = rest;
+        j.post_dims = {rest};
+        j.post_strides = {1};
+        j.o0 = res->st->c0;
+        j.o1 = res->st->c1;
+        rc = axis_dot(ctx, j);
+    }
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    delete eq;
+    if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "fix_high: %s", hipGetErrorString(e));
+    if (rc != DPS_OK) {
+        delete res;
+        return rc;
+    }
+    *out = res;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t k, dps_mle **out)
+{
+    if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: bad argument");
+    if (!is_pow2(mle->len) || (1ull << k) > mle->len || mle->kind == DPS_I64)
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: needs a power-of-two field table and k <= log2(len)");
+    if (!canonical(point, 2 * (size_t)k)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: point not canonical");
+    DeviceGuard g(ctx->device);
+    if (k == 0) return dps_mle_view(mle, 0, log2u(mle->len), out);
+    // ping-pong between two buffers; the last one written becomes the result
+    u64 len = mle->len;
+    dps_mle *bufs[2] = {nullptr, nullptr};
+    CHK(new_table(ctx, DPS_EXT2, len >> 1, &bufs[0]));
+    if (k > 1) {
+        int32_t rc = new_table(ctx, DPS_EXT2, len >> 2, &bufs[1]);
+        if (rc != DPS_OK) {
+            delete bufs[0];
+            return rc;
+        }
+    }
+    const u64 *s0 = mle->p0(), *s1 = mle->p1();
+    int32_t rc = DPS_OK;
+    int w = 0;
+    for (u32 j = 0; j < k && rc == DPS_OK; j++) {
+        len >>= 1;
+        dpk::FoldDesc d{s0, s1, bufs[w]->st->c0, bufs[w]->st->c1, len};
+        const u64 *dd = nullptr;
+        rc = stage_words(ctx, (const u64 *)&d, sizeof d / 8, 0, &dd);
+        if (rc != DPS_OK) break;
+        ProfScope ps(ctx, DPS_K_FOLD, (double)len * (s1 ? 32.0 : 16.0) + (double)len * 16.0);
+        dpk::fold_kernel<<<dim3(grid_for(len), 1), dpk::BLOCK, 0, ctx->stream>>>((const dpk::FoldDesc *)dd, point[2 * j], point[2 * j + 1]);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "fold launch: %s", hipGetErrorString(e));
+        s0 = bufs[w]->st->c0;
+        s1 = bufs[w]->st->c1;
+        w ^= 1;
+    }
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "fix_low: %s", hipGetErrorString(e));
+    dps_mle *res = bufs[w ^ 1], *other = bufs[w];
+    delete other;
+    if (rc != DPS_OK) {
+        delete res;
+        return rc;
+    }
+    res->len = len;
+    *out = res;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const uint64_t *padded_dims,
+                                    const uint64_t *unpadded_dims, uint32_t n_dims, const int32_t *kinds,
+                                    const uint64_t *const *points, dps_mle **out, uint32_t out_cap, uint32_t *n_out)
+{
+    if (!ctx || !tensor || !padded_dims || !unpadded_dims || !kinds || !out || !n_out || n_dims == 0 || n_dims > dpk::AX_MAX_DIMS)
+        return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: bad argument");
+    DeviceGuard g(ctx->device);
+    u64 padded_total = 1, contraction = 1, stacked = 1;
+    for (u32 a = 0; a < n_dims; a++) {
+        if (unpadded_dims[a] == 0 || unpadded_dims[a] > padded_dims[a]) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: dimension %u", a);
+        if (kinds[a] < 0 || kinds[a] > 2) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: axis kind %u", a);
+        if (kinds[a] == DPS_AXIS_OUTER && (!points || !points[a] || !is_pow2(padded_dims[a])))
+            return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: outer axis %u needs a point and a power-of-two padded size", a);
+        padded_total *= padded_dims[a];
+        if (kinds[a] == DPS_AXIS_CONTRACTED) contraction *= unpadded_dims[a];
+        if (kinds[a] == DPS_AXIS_STACKED) stacked *= unpadded_dims[a];
+    }
+    if (padded_total > tensor->len) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: tensor shorter than its padded shape");
+    if (stacked > out_cap) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: %llu tables do not fit out_cap", (unsigned long long)stacked);
+
+    // current tensor: dims (unpadded sizes of the axes still present) and element strides
+    std::vector<u64> dims(unpadded_dims, unpadded_dims + n_dims), strides(n_dims);
+    std::vector<int32_t> kd(kinds, kinds + n_dims);
+    std::vector<u32> orig(n_dims);
+    {
+        u64 s = 1;
+        for (int a = (int)n_dims - 1; a >= 0; a--) {
+            strides[a] = s;
+            s *= padded_dims[a];
+            orig[a] = a;
+        }
+    }
+    const u64 *in0 = tensor->p0(), *in1 = tensor->p1();
+    bool in_is_i64 = tensor->kind == DPS_I64;
+    dps_mle *cur = nullptr;  // owns the intermediate
+    int32_t rc = DPS_OK;
+    // the reference walks the axes from the last to the first (axis.rs:1152)
+    for (int a = (int)dims.size() - 1; a >= 0 && rc == DPS_OK; a--) {
+        if (kd[a] != DPS_AXIS_OUTER) continue;
+        u32 oa = orig[a];
+        u32 m = log2u(padded_dims[oa]);
+        dps_mle *beta = nullptr;
+        rc = dps_eq_build(ctx, points[oa], m, &beta);
+        if (rc != DPS_OK) break;
+        AxisJob j;
+        j.in0 = in0;
+        j.in1 = in1;
+        j.in_is_i64 = in_is_i64;
+        j.b0 = beta->p0();
+        j.b1 = beta->p1();
+        j.K = dims[a];  // evals(point)[..size]
+        j.stride_k = strides[a];
+        u64 outputs = 1;
+        for (int d = 0; d < (int)dims.size(); d++) {
+            if (d == a) continue;
+            (d < a ? j.pre_dims : j.post_dims).push_back(dims[d]);
+            (d < a ? j.pre_strides : j.post_strides).push_back(strides[d]);
+            outputs *= dims[d];
+        }
+        dps_mle *next = nullptr;
+        rc = new_table(ctx, DPS_EXT2, outputs, &next);
+        if (rc == DPS_OK) {
+            j.o0 = next->st->c0;
+            j.o1 = next->st->c1;
+            rc = axis_dot(ctx, j);
+        }
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "partial eval: %s", hipGetErrorString(e));
+        delete beta;
+        delete cur;
+        cur = next;
+        if (rc != DPS_OK) break;
+        // the result is compact over the remaining axes
+        dims.erase(dims.begin() + a);
+        kd.erase(kd.begin() + a);
+        orig.erase(orig.begin() + a);
+        strides.assign(dims.size(), 1);
+        for (int d = (int)dims.size() - 2; d >= 0; d--) strides[d] = strides[d + 1] * dims[d + 1];
+        in0 = cur->st->c0;
+        in1 = cur->st->c1;
+        in_is_i64 = false;
+    }
+    if (rc != DPS_OK) {
+        delete cur;
+        return rc;
+    }
+    // What is left is indexed by the stacked and contracted axes in their original
+    // order; like the reference (axis.rs:1222-1233) the flat result is cut into
+    // chunks of `contraction` entries, one table per chunk.
+    // gather (strided source when no outer axis was fixed) into padded rows
+    u32 nv = log2u(contraction);
+    u64 tl = 1ull << nv;
+    dps_mle *all = nullptr;
+    rc = new_table(ctx, DPS_EXT2, stacked * tl, &all);
+    if (rc == DPS_OK) {
+        if (cur) {
+            dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(cur->st->c0, cur->st->c1, stacked, contraction, tl,
+                                                                                    all->st->c0, all->st->c1);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
+        } else {
+            // no outer axis: contract a unit axis with the table {1} to copy the unpadded region
+            u64 one[2] = {0, 0};
+            dps_mle *unit = nullptr;
+            rc = dps_eq_build(ctx, one, 0, &unit);
+            dps_mle *flat = nullptr;
+            if (rc == DPS_OK) rc = new_table(ctx, DPS_EXT2, stacked * contraction, &flat);
+            if (rc == DPS_OK) {
+                AxisJob j;
+                j.in0 = in0;
+                j.in1 = in1;
+                j.in_is_i64 = in_is_i64;
+                j.b0 = unit->p0();
+                j.b1 = unit->p1();
+                j.K = 1;
+                j.stride_k = 0;
+                j.post_dims = dims;
+                j.post_strides = strides;
+                j.o0 = flat->st->c0;
+                j.o1 = flat->st->c1;
+                rc = axis_dot(ctx, j);
+            }
+            if (rc == DPS_OK) {
+                dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(flat->st->c0, flat->st->c1, stacked, contraction,
+                                                                                        tl, all->st->c0, all->st->c1);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
+            }
+            (void)hipStreamSynchronize(ctx->stream);
+            delete unit;
+            delete flat;
+        }
+    }
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "partial eval: %s", hipGetErrorString(e));
+    delete cur;
+    if (rc != DPS_OK) {
+        delete all;
+        return rc;
+    }
+    for (u64 s = 0; s < stacked; s++) {
+        rc = dps_mle_view(all, s * tl, nv, &out[s]);
+        if (rc != DPS_OK) {
+            for (u64 q = 0; q < s; q++) delete out[q];
+            delete all;
+            return rc;
+        }
+    }
+    delete all;  // the views keep the storage alive
+    *n_out = (u32)stacked;
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// sumcheck session
+// ---------------------------------------------------------------------------
+namespace {
+
+struct SessMle {
+    const u64 *c0, *c1;  // current table
+    u32 nv;              // current number of variables
+    u64 *buf0[2], *buf1[2];  // ping-pong scratch, extension limbs
+    int next;
+};
+
+}  // namespace
+
+struct dps_sc {
+    dps_ctx *ctx;
+    u32 n_vars, n_mles, n_terms, degree;
+    u32 round;  // rounds completed
+    bool finished;
+    std::vector<SessMle> m;
+    std::vector<std::shared_ptr<Storage>> keep;  // borrowed tables stay alive
+    std::vector<dps_term> terms;                 // non-constant terms
+    E2 const_sum;                                // sum of the constant terms
+    // fast path: one term, 2 or 3 distinct full-size tables
+    bool fast;
+    u32 fast_nf;
+    u32 fast_order[3];  // term factors sorted base-first
+    void *scratch;      // one pool block holding every ping-pong buffer
+    void *dev_block;    // descriptors, partials, per-round result
+    // precomputed descriptors (device)
+    std::vector<u32> fold_off, fold_cnt;            // per step j = 2..n_vars+1: all tables that fold
+    std::vector<u32> fold_extra_off, fold_extra_cnt;  // same, without the fast term's tables
+    std::vector<u32> term_off;                      // per round j = 1..n_vars
+    dpk::FoldDesc *d_fold;
+    dpk::FoldDesc *d_fold_extra;
+    dpk::TermDesc *d_terms;
+    dpk::FinTerm *d_fin;
+    dpk::GatherDesc *d_gather;
+    u64 *d_partial;
+    u64 *d_result;
+    std::vector<dpk::ProdArgs> fast_args;  // per round
+    std::vector<u32> fast_nb;              // base-field sources per round
+    u32 max_blocks;
+};
+
+namespace {
+
+template <int NF, int NB, bool FOLD>
+void launch_prod(dps_ctx *ctx, const dpk::ProdArgs &a, u32 blocks, u64 *partial)
+{
+    dpk::prod_kernel<NF, NB, FOLD><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial);
+}
+
+int32_t launch_prod_dispatch(dps_ctx *ctx, u32 nf, u32 nb, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial)
+{
+#define PK(NF_, NB_)                                               \
+    if (nf == NF_ && nb == NB_) {                                  \
+        if (fold)                                                  \
+            launch_prod<NF_, NB_, true>(ctx, a, blocks, partial);  \
+        else                                                       \
+            launch_prod<NF_, NB_, false>(ctx, a, blocks, partial); \
+        return DPS_OK;                                             \
+    }
+    PK(2, 0) PK(2, 1) PK(2, 2) PK(3, 0) PK(3, 1) PK(3, 2) PK(3, 3)
+#undef PK
+    return fail(ctx, DPS_ERR_UNSUPPORTED, "no product kernel for %u factors, %u base", nf, nb);
+}
+
+u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
+
+}  // namespace
+
+extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
+                                const dps_term *terms, uint32_t n_terms, dps_sc **out)
+{
+    if (!ctx || !out || (n_mles && !mles) || (n_terms && !terms) || n_vars > 40)
+        return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: bad argument");
+    DeviceGuard g(ctx->device);
+    std::unique_ptr<dps_sc> sc(new (std::nothrow) dps_sc());
+    if (!sc) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
+    sc->ctx = ctx;
+    sc->n_vars = n_vars;
+    sc->n_mles = n_mles;
+    sc->round = 0;
+    sc->finished = false;
+    sc->scratch = sc->dev_block = nullptr;
+    sc->const_sum = gl::e2_zero();
+    sc->degree = 0;
+    std::vector<u32> nv0(n_mles);
+    for (u32 k = 0; k < n_mles; k++) {
+        const dps_mle *t = mles[k];
+        if (!t || t->ctx != ctx) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u belongs to another context", k);
+        if (t->kind == DPS_I64 || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
+        nv0[k] = log2u(t->len);
+        if (nv0[k] > n_vars) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u has %u variables, the sum has %u", k, nv0[k], n_vars);
+        sc->keep.push_back(t->st);
+    }
+    for (u32 i = 0; i < n_terms; i++) {
+        const dps_term &t = terms[i];
+        if (!canonical(t.coeff, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: coefficient of term %u not canonical", i);
+        if (t.n_factors > DPS_MAX_FACTORS) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u has %u factors", i, t.n_factors);
+        if (t.n_factors > DPS_MAX_DEGREE) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_sc_begin: degree %u above %d", t.n_factors, DPS_MAX_DEGREE);
+        for (u32 f = 0; f < t.n_factors; f++)
+            if (t.factors[f] >= n_mles) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u names table %u", i, t.factors[f]);
+        if (t.n_factors == 0) {
+            sc->const_sum = gl::add(sc->const_sum, gl::e2(t.coeff[0], t.coeff[1]));
+        } else {
+            sc->terms.push_back(t);
+            sc->degree = std::max(sc->degree, t.n_factors);
+        }
+    }
+    sc->n_terms = (u32)sc->terms.size();
+
+    // fast path test
+    sc->fast = false;
+    if (sc->n_terms == 1 && (sc->terms[0].n_factors == 2 || sc->terms[0].n_factors == 3) && n_vars >= 1) {
+        const dps_term &t = sc->terms[0];
+        bool ok = true;
+        for (u32 f = 0; f < t.n_factors && ok; f++) {
+            if (nv0[t.factors[f]] != n_vars) ok = false;
+            for (u32 q = 0; q < f; q++)
+                if (t.factors[q] == t.factors[f]) ok = false;
+        }
+        if (ok) {
+            sc->fast = true;
+            sc->fast_nf = t.n_factors;
+            u32 w = 0;
+            for (u32 f = 0; f < t.n_factors; f++)
+                if (mles[t.factors[f]]->kind == DPS_BASE) sc->fast_order[w++] = t.factors[f];
+            for (u32 f = 0; f < t.n_factors; f++)
+                if (mles[t.factors[f]]->kind != DPS_BASE) sc->fast_order[w++] = t.factors[f];
+        }
+    }
+
+    // scratch: two ping-pong buffers per table, extension limbs
+    size_t scratch_words = 0;
+    std::vector<size_t> off_a(n_mles), off_b(n_mles);
+    for (u32 k = 0; k < n_mles; k++) {
+        u64 la = nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : 0, lb = nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : 0;
+        off_a[k] = scratch_words;
+        scratch_words += round_up(2 * la, 32);
+        off_b[k] = scratch_words;
+        scratch_words += round_up(2 * lb, 32);
+    }
+    if (scratch_words) CHK(pool_alloc(ctx, scratch_words * 8, &sc->scratch));
+    auto cleanup = [&](int32_t rc) {
+        pool_free(ctx, sc->scratch);
+        pool_free(ctx, sc->dev_block);
+        return rc;
+    };
+    u64 *sbase = (u64 *)sc->scratch;
+    sc->m.resize(n_mles);
+    for (u32 k = 0; k < n_mles; k++) {
+        SessMle &s = sc->m[k];
+        s.c0 = mles[k]->p0();
+        s.c1 = mles[k]->p1();
+        s.nv = nv0[k];
+        u64 la = nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : 0, lb = nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : 0;
+        s.buf0[0] = sbase ? sbase + off_a[k] : nullptr;
+        s.buf1[0] = s.buf0[0] ? s.buf0[0] + la : nullptr;
+        s.buf0[1] = sbase ? sbase + off_b[k] : nullptr;
+        s.buf1[1] = s.buf0[1] ? s.buf0[1] + lb : nullptr;
+        s.next = 0;
+    }
+
+    // simulate the rounds to precompute every descriptor
+    std::vector<dpk::FoldDesc> folds, folds_extra;
+    std::vector<dpk::TermDesc> tdescs;
+    std::vector<SessMle> sim = sc->m;
+    auto in_fast = [&](u32 k) {
+        if (!sc->fast) return false;
+        for (u32 f = 0; f < sc->fast_nf; f++)
+            if (sc->fast_order[f] == k) return true;
+        return false;
+    };
+    sc->fold_off.assign(n_vars + 2, 0);
+    sc->fold_cnt.assign(n_vars + 2, 0);
+    sc->fold_extra_off.assign(n_vars + 2, 0);
+    sc->fold_extra_cnt.assign(n_vars + 2, 0);
+    sc->term_off.assign(n_vars + 2, 0);
+    sc->fast_args.resize(n_vars + 2);
+    sc->fast_nb.assign(n_vars + 2, 0);
+    for (u32 j = 1; j <= n_vars + 1; j++) {
+        // step j starts by folding, with the challenge of round j-1, the tables that were live-sized then
+        if (j >= 2) {
+            u32 prev_live = n_vars - (j - 1) + 1;
+            sc->fold_off[j] = (u32)folds.size();
+            sc->fold_extra_off[j] = (u32)folds_extra.size();
+            if (sc->fast && j <= n_vars) {
+                dpk::ProdArgs &pa = sc->fast_args[j];
+                memset(&pa, 0, sizeof pa);
+                u32 nb = 0;
+                for (u32 f = 0; f < sc->fast_nf; f++) {
+                    const SessMle &s = sim[sc->fast_order[f]];
+                    pa.s0[f] = s.c0;
+                    pa.s1[f] = s.c1;
+                    if (!s.c1) nb++;
+                    pa.d0[f] = s.buf0[s.next];
+                    pa.d1[f] = s.buf1[s.next];
+                }
+                pa.n_pairs = 1ull << (n_vars - j);
+                sc->fast_nb[j] = nb;
+            }
+            for (u32 k = 0; k < n_mles; k++) {
+                SessMle &s = sim[k];
+                if (s.nv != prev_live) continue;
+                dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1)};
+                folds.push_back(d);
+                if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
+                s.c0 = d.d0;
+                s.c1 = d.d1;
+                s.nv -= 1;
+                s.next ^= 1;
+            }
+            sc->fold_cnt[j] = (u32)folds.size() - sc->fold_off[j];
+            sc->fold_extra_cnt[j] = (u32)folds_extra.size() - sc->fold_extra_off[j];
+        } else if (sc->fast) {
+            dpk::ProdArgs &pa = sc->fast_args[1];
+            memset(&pa, 0, sizeof pa);
+            u32 nb = 0;
+            for (u32 f = 0; f < sc->fast_nf; f++) {
+                const SessMle &s = sim[sc->fast_order[f]];
+                pa.s0[f] = s.c0;
+                pa.s1[f] = s.c1;
+                if (!s.c1) nb++;
+            }
+            pa.n_pairs = 1ull << (n_vars - 1);
+            sc->fast_nb[1] = nb;
+        }
+        if (j <= n_vars && !sc->fast) {
+            u32 live = n_vars - j + 1;
+            sc->term_off[j] = (u32)tdescs.size();
+            for (const dps_term &t : sc->terms) {
+                dpk::TermDesc td;
+                memset(&td, 0, sizeof td);
+                td.n_factors = t.n_factors;
+                for (u32 f = 0; f < t.n_factors; f++) {
+                    const SessMle &s = sim[t.factors[f]];
+                    td.f[f].c0 = s.c0;
+                    td.f[f].c1 = s.c1;
+                    if (s.nv >= live) {
+                        td.f[f].pair = 1;
+                        td.f[f].shift = 0;
+                    } else {
+                        td.f[f].pair = 0;
+                        td.f[f].shift = live - 1 - s.nv;
+                    }
+                }
+                tdescs.push_back(td);
+            }
+        }
+    }
+    std::vector<dpk::FinTerm> fins;
+    for (const dps_term &t : sc->terms) fins.push_back(dpk::FinTerm{t.coeff[0], t.coeff[1], t.n_factors, 0});
+    std::vector<dpk::GatherDesc> gath;
+    for (u32 k = 0; k < n_mles; k++) gath.push_back(dpk::GatherDesc{sim[k].c0, sim[k].c1});
+
+    sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
+    size_t bytes_fold = round_up(folds.size() * sizeof(dpk::FoldDesc), 256);
+    size_t bytes_fold_x = round_up(folds_extra.size() * sizeof(dpk::FoldDesc), 256);
+    size_t bytes_terms = round_up(tdescs.size() * sizeof(dpk::TermDesc), 256);
+    size_t bytes_fin = round_up(fins.size() * sizeof(dpk::FinTerm), 256);
+    size_t bytes_gath = round_up(gath.size() * sizeof(dpk::GatherDesc), 256);
+    size_t bytes_partial = round_up((size_t)std::max<u32>(sc->n_terms, 1) * sc->max_blocks * 2 * dpk::MAX_PTS * 8, 256);
+    size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256);
+    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_partial + bytes_result;
+    int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
+    if (rc != DPS_OK) return cleanup(rc);
+    char *p = (char *)sc->dev_block;
+    sc->d_fold = (dpk::FoldDesc *)p;
+    p += bytes_fold;
+    sc->d_fold_extra = (dpk::FoldDesc *)p;
+    p += bytes_fold_x;
+    sc->d_terms = (dpk::TermDesc *)p;
+    p += bytes_terms;
+    sc->d_fin = (dpk::FinTerm *)p;
+    p += bytes_fin;
+    sc->d_gather = (dpk::GatherDesc *)p;
+    p += bytes_gath;
+    sc->d_partial = (u64 *)p;
+    p += bytes_partial;
+    sc->d_result = (u64 *)p;
+    // one staged upload of all descriptors
+    std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath, 0);
+    char *q = stage.data();
+    if (!folds.empty()) memcpy(q, folds.data(), folds.size() * sizeof(dpk::FoldDesc));
+    q += bytes_fold;
+    if (!folds_extra.empty()) memcpy(q, folds_extra.data(), folds_extra.size() * sizeof(dpk::FoldDesc));
+    q += bytes_fold_x;
+    if (!tdescs.empty()) memcpy(q, tdescs.data(), tdescs.size() * sizeof(dpk::TermDesc));
+    q += bytes_terms;
+    if (!fins.empty()) memcpy(q, fins.data(), fins.size() * sizeof(dpk::FinTerm));
+    q += bytes_fin;
+    if (!gath.empty()) memcpy(q, gath.data(), gath.size() * sizeof(dpk::GatherDesc));
+    if (!stage.empty()) {
+        hipError_t e = hipMemcpyAsync(sc->dev_block, stage.data(), stage.size(), hipMemcpyHostToDevice, ctx->stream);
+        // the staging vector dies with this call
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) return cleanup(fail(ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e)));
+    }
+    *out = sc.release();
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_sc_degree(const dps_sc *sc, uint32_t *degree)
+{
+    if (!sc || !degree) return DPS_ERR_INVALID;
+    *degree = sc->degree;
+    return DPS_OK;
+}
+
+namespace {
+
+int32_t launch_folds(dps_sc *sc, u32 step, bool extra_only, const u64 *chal)
+{
+    dps_ctx *ctx = sc->ctx;
+    u32 cnt = extra_only ? sc->fold_extra_cnt[step] : sc->fold_cnt[step];
+    if (!cnt) return DPS_OK;
+    const dpk::FoldDesc *d = extra_only ? sc->d_fold_extra + sc->fold_extra_off[step] : sc->d_fold + sc->fold_off[step];
+    // every table folding in one step has the same size
+    u32 prev_live = sc->n_vars - (step - 1) + 1;
+    u64 half = 1ull << (prev_live - 1);
+    for (u32 base = 0; base < cnt; base += 65535) {
+        u32 n = std::min<u32>(cnt - base, 65535);
+        ProfScope ps(ctx, DPS_K_FOLD, (double)n * (double)half * 48.0);
+        dpk::fold_kernel<<<dim3(grid_for(half), n), dpk::BLOCK, 0, ctx->stream>>>(d + base, chal[0], chal[1]);
+        HIPCHK(ctx, hipGetLastError());
+    }
+    return DPS_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
+{
+    if (!sc || !evals_out) return DPS_ERR_INVALID;
+    dps_ctx *ctx = sc->ctx;
+    if (sc->finished || sc->round >= sc->n_vars) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: all %u rounds are done", sc->n_vars);
+    const u32 j = sc->round + 1;
+    if ((j == 1) != (challenge == nullptr)) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: round %u %s a challenge", j, j == 1 ? "takes no" : "needs");
+    if (challenge && !canonical(challenge, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_round: challenge not canonical");
+    DeviceGuard g(ctx->device);
+    const u32 live = sc->n_vars - j + 1;
+    const u64 n_pairs = 1ull << (live - 1);
+    u32 blocks = blocks_for_pairs(n_pairs);
+    if (sc->n_terms == 0) {
+        blocks = 0;
+        if (j >= 2) CHK(launch_folds(sc, j, false, challenge));
+    } else if (sc->fast) {
+        dpk::ProdArgs a = sc->fast_args[j];
+        if (j >= 2) {
+            a.r0 = challenge[0];
+            a.r1 = challenge[1];
+            CHK(launch_folds(sc, j, true, challenge));
+        }
+        double bytes = 0;
+        for (u32 f = 0; f < sc->fast_nf; f++) {
+            double eb = a.s1[f] ? 16.0 : 8.0;
+            bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
+        }
+        {
+            ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
+            CHK(launch_prod_dispatch(ctx, sc->fast_nf, sc->fast_nb[j], j >= 2, a, blocks, sc->d_partial));
+            HIPCHK(ctx, hipGetLastError());
+        }
+    } else {
+        if (j >= 2) CHK(launch_folds(sc, j, false, challenge));
+        for (u32 base = 0; base < sc->n_terms; base += 65535) {
+            u32 n = std::min<u32>(sc->n_terms - base, 65535);
+            ProfScope ps(ctx, DPS_K_EVAL_TERMS, 0.0);
+            dpk::eval_terms_kernel<<<dim3(blocks, n), dpk::BLOCK, 0, ctx->stream>>>(
+                sc->d_terms + sc->term_off[j] + base, n_pairs, sc->d_partial + (size_t)base * blocks * 2 * dpk::MAX_PTS);
+            HIPCHK(ctx, hipGetLastError());
+        }
+    }
+    // constant terms: c summed over 2^(live-1) suffixes at every evaluation point
+    E2 cst = gl::mul_base(sc->const_sum, h_pow(2, live - 1));
+    {
+        ProfScope ps(ctx, DPS_K_FINALIZE, 0.0);
+        dpk::finalize_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(sc->d_partial, blocks, sc->d_fin, sc->n_terms, sc->degree, ctx->d_lagrange,
+                                                                  cst.c0, cst.c1, sc->d_result, ctx->d_pinned);
+        HIPCHK(ctx, hipGetLastError());
+    }
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    memcpy(evals_out, ctx->h_pinned, 2 * (sc->degree + 1) * 8);
+    sc->round = j;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t *final_evals_out)
+{
+    if (!sc || (sc->n_mles && !final_evals_out)) return DPS_ERR_INVALID;
+    dps_ctx *ctx = sc->ctx;
+    if (sc->finished || sc->round != sc->n_vars) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: %u of %u rounds done", sc->round, sc->n_vars);
+    if (sc->n_vars >= 1 && !challenge) return fail(ctx, DPS_ERR_INVALID, "dps_sc_finish: the last challenge is missing");
+    if (challenge && !canonical(challenge, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_finish: challenge not canonical");
+    DeviceGuard g(ctx->device);
+    if (sc->n_vars >= 1) CHK(launch_folds(sc, sc->n_vars + 1, sc->fast, challenge));
+    if (sc->n_mles) {
+        if (2 * (size_t)sc->n_mles > ctx->pinned_words) return fail(ctx, DPS_ERR_UNSUPPORTED, "too many tables in one session");
+        dpk::gather_kernel<<<(sc->n_mles + 63) / 64, 64, 0, ctx->stream>>>(sc->d_gather, sc->n_mles, ctx->d_pinned);
+        HIPCHK(ctx, hipGetLastError());
+    }
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (sc->n_mles) memcpy(final_evals_out, ctx->h_pinned, 2 * (size_t)sc->n_mles * 8);
+    sc->finished = true;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_sc_free(dps_sc *sc)
+{
+    if (!sc) return DPS_OK;
+    dps_ctx *ctx = sc->ctx;
+    DeviceGuard g(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    pool_free(ctx, sc->scratch);
+    pool_free(ctx, sc->dev_block);
+    delete sc;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_sc_prove(dps_sc *sc, dps_round_fn fn, void *user, uint64_t *proof_out, uint64_t *point_out,
+                                uint64_t *final_evals_out)
+{
+    if (!sc || !fn) return DPS_ERR_INVALID;
+    dps_ctx *ctx = sc->ctx;
+    if (sc->round != 0 || sc->finished) return fail(ctx, DPS_ERR_STATE, "dps_sc_prove: session already started");
+    if (sc->n_vars && (!proof_out || !point_out)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_prove: output buffers missing");
+    const u32 npts = sc->degree + 1;
+    uint64_t chal[2] = {0, 0};
+    for (u32 j = 1; j <= sc->n_vars; j++) {
+        uint64_t *msg = proof_out + (size_t)(j - 1) * npts * 2;
+        CHK(dps_sc_round(sc, j == 1 ? nullptr : chal, msg));
+        if (fn(user, j, msg, npts, chal) != 0) return fail(ctx, DPS_ERR_CALLBACK, "transcript callback failed in round %u", j);
+        if (!canonical(chal, 2)) return fail(ctx, DPS_ERR_CALLBACK, "transcript callback returned a non-canonical challenge in round %u", j);
+        point_out[2 * (j - 1)] = chal[0];
+        point_out[2 * (j - 1) + 1] = chal[1];
+    }
+    return dps_sc_finish(sc, sc->n_vars ? chal : nullptr, final_evals_out);
+}
+
+// ---------------------------------------------------------------------------
+// LogUp fraction-sum circuit
+// ---------------------------------------------------------------------------
+struct dps_logup {
+    dps_ctx *ctx;
+    u64 len;
+    u32 n_layers;  // including the input layer
+    std::shared_ptr<Storage> arena;
+    std::vector<u64> layer_off;  // per layer k >= 1: offset of the numerator array; the denominator follows
+};
+
+extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uint32_t n_cols, const dps_mle *numer,
+                                   const uint64_t c[2], const uint64_t beta[2], dps_logup **out)
+{
+    if (!ctx || !cols || !out || !c || !beta || n_cols == 0) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: bad argument");
+    if (n_cols > dpk::LOGUP_MAX_COLS) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_logup_build: more than %d columns", dpk::LOGUP_MAX_COLS);
+    if (!canonical(c, 2) || !canonical(beta, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: challenge not canonical");
+    DeviceGuard g(ctx->device);
+    u64 len = cols[0] ? cols[0]->len : 0;
+    if (!is_pow2(len) || len < 2) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: column length must be a power of two >= 2");
+    for (u32 k = 0; k < n_cols; k++)
+        if (!cols[k] || cols[k]->kind != DPS_BASE || cols[k]->len != len || cols[k]->ctx != ctx)
+            return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: column %u is not a base table of %llu entries", k, (unsigned long long)len);
+    if (numer && (numer->kind != DPS_BASE || numer->len != len)) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: multiplicity table mismatch");
+    std::unique_ptr<dps_logup> lg(new (std::nothrow) dps_logup());
+    if (!lg) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
+    lg->ctx = ctx;
+    lg->len = len;
+    u32 top = log2u(len);
+    lg->n_layers = top;  // layers 0 .. top-1; the last has 2 entries per array
+    lg->layer_off.assign(top, 0);
+    u64 words = 0;
+    for (u32 k = 1; k < top; k++) {
+        lg->layer_off[k] = words;
+        words += round_up(2 * (len >> k), 2);
+    }
+    auto st = std::make_shared<Storage>();
+    st->ctx = ctx;
+    void *p0 = nullptr, *p1 = nullptr;
+    CHK(pool_alloc(ctx, std::max<u64>(words, 4) * 8, &p0));
+    st->c0 = (u64 *)p0;
+    CHK(pool_alloc(ctx, std::max<u64>(words, 4) * 8, &p1));
+    st->c1 = (u64 *)p1;
+    lg->arena = st;
+    if (top >= 2) {
+        dpk::LogupFirstArgs a;
+        memset(&a, 0, sizeof a);
+        for (u32 k = 0; k < n_cols; k++) a.cols[k] = cols[k]->p0();
+        a.n_cols = n_cols;
+        a.numer = numer ? numer->p0() : nullptr;
+        a.c0 = c[0];
+        a.c1 = c[1];
+        E2 pw = gl::e2_one(), b = gl::e2(beta[0], beta[1]);
+        for (u32 k = 0; k < n_cols; k++) {
+            a.pw[2 * k] = pw.c0;
+            a.pw[2 * k + 1] = pw.c1;
+            pw = gl::mul(pw, b);
+        }
+        u64 half = len >> 1;
+        a.half = half;
+        a.n0 = st->c0 + lg->layer_off[1];
+        a.n1 = st->c1 + lg->layer_off[1];
+        a.d0 = a.n0 + half;
+        a.d1 = a.n1 + half;
+        {
+            ProfScope ps(ctx, DPS_K_LOGUP, (double)len * 8.0 * (n_cols + (numer ? 1 : 0)) + (double)half * 32.0);
+            dpk::logup_first_kernel<<<grid_for(half), dpk::BLOCK, 0, ctx->stream>>>(a);
+            HIPCHK(ctx, hipGetLastError());
+        }
+        for (u32 k = 2; k < top; k++) {
+            u64 prev = len >> (k - 1), cur = len >> k;
+            const u64 *pn0 = st->c0 + lg->layer_off[k - 1], *pn1 = st->c1 + lg->layer_off[k - 1];
+            u64 *n0 = st->c0 + lg->layer_off[k], *n1 = st->c1 + lg->layer_off[k];
+            ProfScope ps(ctx, DPS_K_LOGUP, (double)prev * 32.0 + (double)cur * 32.0);
+            dpk::logup_next_kernel<<<grid_for(cur), dpk::BLOCK, 0, ctx->stream>>>(pn0, pn1, pn0 + prev, pn1 + prev, cur, n0, n1, n0 + cur, n1 + cur);
+            HIPCHK(ctx, hipGetLastError());
+        }
+    }
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    *out = lg.release();
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_logup_num_layers(const dps_logup *lg, uint32_t *n_layers)
+{
+    if (!lg || !n_layers) return DPS_ERR_INVALID;
+    *n_layers = lg->n_layers;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_logup_layer(const dps_logup *lg, uint32_t k, dps_mle **num, dps_mle **den)
+{
+    if (!lg || !num || !den) return DPS_ERR_INVALID;
+    if (k < 1 || k >= lg->n_layers) return fail(lg->ctx, DPS_ERR_INVALID, "dps_logup_layer: layer %u of %u", k, lg->n_layers);
+    u64 sz = lg->len >> k;
+    *num = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k], sz};
+    *den = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k] + sz, sz};
+    if (!*num || !*den) return fail(lg->ctx, DPS_ERR_OOM, "host allocation failed");
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8])
+{
+    if (!lg || !out) return DPS_ERR_INVALID;
+    dps_ctx *ctx = lg->ctx;
+    if (lg->n_layers < 2) return fail(ctx, DPS_ERR_STATE, "dps_logup_outputs: the instance has no layer above its input");
+    DeviceGuard g(ctx->device);
+    u64 off = lg->layer_off[lg->n_layers - 1];
+    u64 a[4], b[4];
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(a, lg->arena->c0 + off, 32, hipMemcpyDeviceToHost));
+    HIPCHK(ctx, hipMemcpy(b, lg->arena->c1 + off, 32, hipMemcpyDeviceToHost));
+    for (int i = 0; i < 4; i++) {
+        out[2 * i] = a[i];
+        out[2 * i + 1] = b[i];
+    }
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_logup_free(dps_logup *lg)
+{
+    if (!lg) return DPS_OK;
+    DeviceGuard g(lg->ctx->device);
+    (void)hipStreamSynchronize(lg->ctx->stream);
+    delete lg;
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// arithmetic self-check: element-wise field operations on the device
+// ---------------------------------------------------------------------------
+extern "C" int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *a /* 2*n: c0.., c1.. */, const uint64_t *b,
+                                      uint64_t n, uint64_t *out)
+{
+    if (!ctx || !a || !b || !out || n == 0) return fail(ctx, DPS_ERR_INVALID, "dps_debug_field_op: bad argument");
+    DeviceGuard g(ctx->device);
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, 6 * n * 8, &p));
+    u64 *d = (u64 *)p;
+    hipError_t e = hipMemcpy(d, a, 2 * n * 8, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(d + 2 * n, b, 2 * n * 8, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        dpk::field_op_kernel<<<(u32)((n + dpk::BLOCK - 1) / dpk::BLOCK), dpk::BLOCK, 0, ctx->stream>>>(op, d, d + n, d + 2 * n, d + 3 * n, n,
+                                                                                                 d + 4 * n, d + 5 * n);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = hipMemcpy(out, d + 4 * n, 2 * n * 8, hipMemcpyDeviceToHost);
+    pool_free(ctx, p);
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "field op: %s", hipGetErrorString(e));
+    return DPS_OK;
+}

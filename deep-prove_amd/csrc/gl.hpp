@@ -1,0 +1,112 @@
+// Goldilocks (p = 2^64 - 2^32 + 1) and its quadratic extension X^2 = 7 for gfx950.
+//
+// Every value handed between functions is canonical (< p).  The 64x64 product is
+// formed from 32-bit multiplies (v_mad_u64_u32 / v_mul_hi_u32) and reduced with
+// 2^64 = 2^32 - 1 and 2^96 = -1 (mod p); nothing here maps onto the matrix cores.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gl {
+
+typedef uint64_t u64;
+typedef uint32_t u32;
+
+constexpr u64 P = 0xFFFFFFFF00000001ULL;
+constexpr u64 EPS = 0xFFFFFFFFULL;  // 2^64 mod p
+constexpr u64 W = 7;                // X^2 = W
+
+#define GL_FN __host__ __device__ __forceinline__
+
+GL_FN u64 add(u64 a, u64 b)
+{
+    u64 s = a + b;
+    // a + b < 2p: one conditional subtraction; on carry the true sum is s + 2^64
+    return (s < a || s >= P) ? s + EPS : s;
+}
+
+GL_FN u64 sub(u64 a, u64 b)
+{
+    u64 d = a - b;
+    return a < b ? d - EPS : d;  // wrapped by 2^64 = p + EPS
+}
+
+GL_FN u64 neg(u64 a) { return a ? P - a : 0; }
+
+GL_FN u64 dbl(u64 a) { return add(a, a); }
+
+// (hi * 2^64 + lo) mod p, canonical
+GL_FN u64 reduce128(u64 lo, u64 hi)
+{
+    u32 hh = (u32)(hi >> 32), hl = (u32)hi;
+    u64 t0 = lo - hh;  // 2^96 = -1
+    if (lo < hh) t0 -= EPS;
+    u64 t1 = ((u64)hl << 32) - hl;  // hl * (2^32 - 1)
+    u64 r = t0 + t1;
+    if (r < t1) r += EPS;
+    return r >= P ? r - P : r;
+}
+
+GL_FN u64 mulhi64(u64 a, u64 b)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __umul64hi(a, b);
+#else
+    return (u64)(((unsigned __int128)a * b) >> 64);
+#endif
+}
+
+GL_FN u64 mul(u64 a, u64 b) { return reduce128(a * b, mulhi64(a, b)); }
+
+// a * small constant (c < 2^32)
+GL_FN u64 mul_small(u64 a, u32 c)
+{
+    u64 lo = a * (u64)c;
+    u64 hi = mulhi64(a, (u64)c);  // < 2^32
+    u64 t1 = (hi << 32) - hi;
+    u64 r = lo + t1;
+    if (r < t1) r += EPS;
+    return r >= P ? r - P : r;
+}
+
+GL_FN u64 from_i64(int64_t x)
+{
+    // negatives map to p - |x|; |x| < 2^63 < p
+    if (x >= 0) return (u64)x;
+    u64 mag = (u64)0 - (u64)x;
+    return P - mag;
+}
+
+GL_FN u64 canon(u64 x) { return x >= P ? x - P : x; }
+
+struct E2 {
+    u64 c0, c1;
+};
+
+GL_FN E2 e2(u64 c0, u64 c1)
+{
+    E2 r;
+    r.c0 = c0;
+    r.c1 = c1;
+    return r;
+}
+GL_FN E2 e2_zero() { return e2(0, 0); }
+GL_FN E2 e2_one() { return e2(1, 0); }
+GL_FN E2 add(E2 a, E2 b) { return e2(add(a.c0, b.c0), add(a.c1, b.c1)); }
+GL_FN E2 sub(E2 a, E2 b) { return e2(sub(a.c0, b.c0), sub(a.c1, b.c1)); }
+GL_FN E2 neg(E2 a) { return e2(neg(a.c0), neg(a.c1)); }
+
+// Karatsuba: three base products
+GL_FN E2 mul(E2 a, E2 b)
+{
+    u64 v0 = mul(a.c0, b.c0);
+    u64 v1 = mul(a.c1, b.c1);
+    u64 v2 = mul(add(a.c0, a.c1), add(b.c0, b.c1));
+    return e2(add(v0, mul_small(v1, (u32)W)), sub(sub(v2, v0), v1));
+}
+
+GL_FN E2 mul_base(E2 a, u64 b) { return e2(mul(a.c0, b), mul(a.c1, b)); }
+
+GL_FN bool eq(E2 a, E2 b) { return a.c0 == b.c0 && a.c1 == b.c1; }
+
+}  // namespace gl

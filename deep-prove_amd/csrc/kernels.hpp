@@ -1,0 +1,655 @@
+// HIP kernels of the sumcheck prover for gfx950 (wave64, 256 CUs in 8 XCDs).
+//
+// All of them are streaming kernels over structure-of-arrays limb tables; the
+// bound is HBM bandwidth, so the rules are: 16-byte per-lane loads of adjacent
+// table entries, every live table read once and every folded table written
+// once per round, reductions finished in registers/LDS with one partial per
+// workgroup, and grids sized to a few workgroups per CU.
+#pragma once
+#include "gl.hpp"
+
+namespace dpk {
+
+using gl::E2;
+using gl::u32;
+using gl::u64;
+
+constexpr int BLOCK = 256;  // 4 wavefronts
+constexpr int WAVE = 64;
+constexpr int MAX_PTS = 8;  // evaluation points per term (degree + 1 <= 7)
+
+// ---------------------------------------------------------------------------
+// loads
+// ---------------------------------------------------------------------------
+struct __attribute__((aligned(16))) U64x2 {
+    u64 x, y;
+};
+
+__device__ __forceinline__ U64x2 ld2(const u64 *p) { return *reinterpret_cast<const U64x2 *>(p); }
+__device__ __forceinline__ void st2(u64 *p, u64 x, u64 y)
+{
+    U64x2 v;
+    v.x = x;
+    v.y = y;
+    *reinterpret_cast<U64x2 *>(p) = v;
+}
+
+// A table as the kernels see it.  c1 == nullptr: base-field entries in c0.
+// is_i64: c0 holds raw int64 values that are embedded on load.
+struct Tab {
+    const u64 *c0;
+    const u64 *c1;
+};
+
+__device__ __forceinline__ E2 tab_get(const u64 *c0, const u64 *c1, u64 i)
+{
+    return gl::e2(c0[i], c1 ? c1[i] : 0);
+}
+
+// ---------------------------------------------------------------------------
+// block reduction of NP extension elements; result valid in thread 0
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ u64 shfl_down64(u64 v, int delta)
+{
+    u32 lo = (u32)v, hi = (u32)(v >> 32);
+    lo = __shfl_down(lo, delta, WAVE);
+    hi = __shfl_down(hi, delta, WAVE);
+    return ((u64)hi << 32) | lo;
+}
+
+template <int NP>
+__device__ __forceinline__ void block_reduce(E2 (&acc)[NP], u64 *lds /* [BLOCK/WAVE][2*NP] */)
+{
+#pragma unroll
+    for (int t = 0; t < NP; t++) {
+#pragma unroll
+        for (int d = WAVE / 2; d >= 1; d >>= 1) {
+            acc[t].c0 = gl::add(acc[t].c0, shfl_down64(acc[t].c0, d));
+            acc[t].c1 = gl::add(acc[t].c1, shfl_down64(acc[t].c1, d));
+        }
+    }
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    if (lane == 0) {
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            lds[wave * 2 * NP + 2 * t] = acc[t].c0;
+            lds[wave * 2 * NP + 2 * t + 1] = acc[t].c1;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < BLOCK / WAVE; w++) {
+#pragma unroll
+            for (int t = 0; t < NP; t++) {
+                acc[t].c0 = gl::add(acc[t].c0, lds[w * 2 * NP + 2 * t]);
+                acc[t].c1 = gl::add(acc[t].c1, lds[w * 2 * NP + 2 * t + 1]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// eq(r, x) table
+// ---------------------------------------------------------------------------
+// Seed: up to 2^8 entries, one per thread, straight from the definition.
+__global__ void __launch_bounds__(BLOCK) eq_seed_kernel(const u64 *__restrict__ point /* 2*m limbs */, u32 m,
+                                                         u64 *__restrict__ o0, u64 *__restrict__ o1)
+{
+    u32 i = threadIdx.x;
+    if (i >= (1u << m)) return;
+    E2 acc = gl::e2_one();
+    for (u32 j = 0; j < m; j++) {
+        E2 r = gl::e2(point[2 * j], point[2 * j + 1]);
+        acc = gl::mul(acc, ((i >> j) & 1) ? r : gl::sub(gl::e2_one(), r));
+    }
+    o0[i] = acc.c0;
+    o1[i] = acc.c1;
+}
+
+// Expansion: out[h * 2^b + l] = hi[h] * lo[l], lo has 2^b <= 256 entries.  Each
+// thread keeps one lo entry in registers and walks hi entries; stores of one
+// wavefront cover 512 contiguous bytes per limb array.
+__global__ void __launch_bounds__(BLOCK)
+eq_expand_kernel(const u64 *__restrict__ hi0, const u64 *__restrict__ hi1, u64 n_hi, const u64 *__restrict__ lo0,
+                 const u64 *__restrict__ lo1, u32 b, u64 *__restrict__ o0, u64 *__restrict__ o1, u32 hi_per_block)
+{
+    const u32 n_lo = 1u << b;
+    const u32 l = threadIdx.x & (n_lo - 1);
+    const u32 sub = threadIdx.x >> b;  // several hi rows per pass when n_lo < BLOCK
+    const u32 rows_per_pass = BLOCK >> b;
+    E2 lo = gl::e2(lo0[l], lo1[l]);
+    u64 h_begin = (u64)blockIdx.x * hi_per_block;
+    u64 h_end = h_begin + hi_per_block;
+    if (h_end > n_hi) h_end = n_hi;
+    for (u64 h = h_begin + sub; h < h_end; h += rows_per_pass) {
+        E2 v = gl::mul(gl::e2(hi0[h], hi1[h]), lo);
+        u64 o = (h << b) | l;
+        o0[o] = v.c0;
+        o1[o] = v.c1;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// stand-alone fold: dst[i] = src[2i] + r * (src[2i+1] - src[2i])
+// ---------------------------------------------------------------------------
+struct FoldDesc {
+    const u64 *s0;
+    const u64 *s1;  // nullptr: base-field source
+    u64 *d0;
+    u64 *d1;
+    u64 half;  // entries written
+};
+
+__device__ __forceinline__ E2 fold1(E2 lo, E2 hi, E2 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
+__device__ __forceinline__ E2 fold1_base(u64 lo, u64 hi, E2 r)
+{
+    E2 d = gl::mul_base(r, gl::sub(hi, lo));
+    d.c0 = gl::add(d.c0, lo);
+    return d;
+}
+
+__global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict__ descs, u64 r0, u64 r1)
+{
+    const FoldDesc d = descs[blockIdx.y];
+    const E2 r = gl::e2(r0, r1);
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < d.half; i += (u64)gridDim.x * BLOCK) {
+        U64x2 a = ld2(d.s0 + 2 * i);
+        E2 v;
+        if (d.s1) {
+            U64x2 b = ld2(d.s1 + 2 * i);
+            v = fold1(gl::e2(a.x, b.x), gl::e2(a.y, b.y), r);
+        } else {
+            v = fold1_base(a.x, a.y, r);
+        }
+        d.d0[i] = v.c0;
+        d.d1[i] = v.c1;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// general term evaluation: one grid row (blockIdx.y) per term
+// ---------------------------------------------------------------------------
+struct FactorDesc {
+    const u64 *c0;
+    const u64 *c1;  // nullptr: base field
+    u32 shift;      // broadcast tables: entry index = pair index >> shift
+    u32 pair;       // 1: read entries 2i, 2i+1; 0: broadcast
+};
+
+struct TermDesc {
+    u32 n_factors;
+    u32 pad;
+    FactorDesc f[DPS_MAX_FACTORS];
+};
+
+// partial sums: out[(term * gridDim.x + block) * 2 * MAX_PTS + 2 * t + limb]
+template <int NF>
+__device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, u64 *__restrict__ partial, u64 *lds)
+{
+    constexpr int NP = NF + 1;
+    E2 acc[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < n_pairs; i += (u64)gridDim.x * BLOCK) {
+        E2 cur[NF], dl[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            const FactorDesc &fd = td.f[f];
+            if (fd.pair) {
+                U64x2 a = ld2(fd.c0 + 2 * i);
+                if (fd.c1) {
+                    U64x2 b = ld2(fd.c1 + 2 * i);
+                    cur[f] = gl::e2(a.x, b.x);
+                    dl[f] = gl::e2(gl::sub(a.y, a.x), gl::sub(b.y, b.x));
+                } else {
+                    cur[f] = gl::e2(a.x, 0);
+                    dl[f] = gl::e2(gl::sub(a.y, a.x), 0);
+                }
+            } else {
+                cur[f] = tab_get(fd.c0, fd.c1, i >> fd.shift);
+                dl[f] = gl::e2_zero();
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            E2 prod = cur[0];
+#pragma unroll
+            for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
+            acc[t] = gl::add(acc[t], prod);
+            if (t + 1 < NP) {
+#pragma unroll
+                for (int f = 0; f < NF; f++) cur[f] = gl::add(cur[f], dl[f]);
+            }
+        }
+    }
+    block_reduce<NP>(acc, lds);
+    if (threadIdx.x == 0) {
+        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            o[2 * t] = acc[t].c0;
+            o[2 * t + 1] = acc[t].c1;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(BLOCK)
+eval_terms_kernel(const TermDesc *__restrict__ terms, u64 n_pairs, u64 *__restrict__ partial)
+{
+    __shared__ u64 lds[(BLOCK / WAVE) * 2 * MAX_PTS];
+    const TermDesc &td = terms[blockIdx.y];
+    switch (td.n_factors) {
+    case 1: eval_term_body<1>(td, n_pairs, partial, lds); break;
+    case 2: eval_term_body<2>(td, n_pairs, partial, lds); break;
+    case 3: eval_term_body<3>(td, n_pairs, partial, lds); break;
+    case 4: eval_term_body<4>(td, n_pairs, partial, lds); break;
+    case 5: eval_term_body<5>(td, n_pairs, partial, lds); break;
+    case 6: eval_term_body<6>(td, n_pairs, partial, lds); break;
+    default: break;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fused product kernels: one term, NF full-size tables, the first NB of them
+// base-field in the source.  FOLD = false: first round, evaluate the source
+// pairs.  FOLD = true: read source quads, fold with r, write the folded pair,
+// evaluate it.
+// ---------------------------------------------------------------------------
+struct ProdArgs {
+    const u64 *s0[3];
+    const u64 *s1[3];
+    u64 *d0[3];
+    u64 *d1[3];
+    u64 n_pairs;  // pairs evaluated this round
+    u64 r0, r1;   // fold challenge
+};
+
+template <int NF, int NB, bool FOLD>
+__global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial)
+{
+    constexpr int NP = NF + 1;
+    __shared__ u64 lds[(BLOCK / WAVE) * 2 * NP];
+    const E2 r = gl::e2(a.r0, a.r1);
+    E2 acc[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.n_pairs; i += (u64)gridDim.x * BLOCK) {
+        E2 lo[NF], hi[NF];
+        bool is_base[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            is_base[f] = (f < NB) && !FOLD;
+            if (FOLD) {
+                if (f < NB) {
+                    U64x2 p = ld2(a.s0[f] + 4 * i), q = ld2(a.s0[f] + 4 * i + 2);
+                    lo[f] = fold1_base(p.x, p.y, r);
+                    hi[f] = fold1_base(q.x, q.y, r);
+                } else {
+                    U64x2 p0 = ld2(a.s0[f] + 4 * i), q0 = ld2(a.s0[f] + 4 * i + 2);
+                    U64x2 p1 = ld2(a.s1[f] + 4 * i), q1 = ld2(a.s1[f] + 4 * i + 2);
+                    lo[f] = fold1(gl::e2(p0.x, p1.x), gl::e2(p0.y, p1.y), r);
+                    hi[f] = fold1(gl::e2(q0.x, q1.x), gl::e2(q0.y, q1.y), r);
+                }
+                st2(a.d0[f] + 2 * i, lo[f].c0, hi[f].c0);
+                st2(a.d1[f] + 2 * i, lo[f].c1, hi[f].c1);
+            } else {
+                U64x2 p = ld2(a.s0[f] + 2 * i);
+                if (f < NB) {
+                    lo[f] = gl::e2(p.x, 0);
+                    hi[f] = gl::e2(p.y, 0);
+                } else {
+                    U64x2 q = ld2(a.s1[f] + 2 * i);
+                    lo[f] = gl::e2(p.x, q.x);
+                    hi[f] = gl::e2(p.y, q.y);
+                }
+            }
+        }
+        E2 dl[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++) dl[f] = gl::sub(hi[f], lo[f]);
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            // base-field factors first (plain products), then the extension ones
+            E2 prod;
+            if (!FOLD && NB > 0) {
+                u64 b = lo[0].c0;
+#pragma unroll
+                for (int f = 1; f < NB; f++) b = gl::mul(b, lo[f].c0);
+                if (NB == NF) {
+                    prod = gl::e2(b, 0);
+                } else {
+                    prod = gl::mul_base(lo[NB], b);
+#pragma unroll
+                    for (int f = NB + 1; f < NF; f++) prod = gl::mul(prod, lo[f]);
+                }
+            } else {
+                prod = lo[0];
+#pragma unroll
+                for (int f = 1; f < NF; f++) prod = gl::mul(prod, lo[f]);
+            }
+            acc[t] = gl::add(acc[t], prod);
+            if (t + 1 < NP) {
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    lo[f].c0 = gl::add(lo[f].c0, dl[f].c0);
+                    if (!is_base[f]) lo[f].c1 = gl::add(lo[f].c1, dl[f].c1);
+                }
+            }
+        }
+    }
+    block_reduce<NP>(acc, lds);
+    if (threadIdx.x == 0) {
+        u64 *o = partial + (u64)blockIdx.x * 2 * MAX_PTS;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            o[2 * t] = acc[t].c0;
+            o[2 * t + 1] = acc[t].c1;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// finalize: sum the block partials of every term, scale by the term's
+// coefficient, extend a degree-k term to the d+1 points of the round message
+// (Lagrange weights over the nodes 0..k), add the constant terms.  One block.
+// ---------------------------------------------------------------------------
+struct FinTerm {
+    u64 coeff0, coeff1;
+    u32 n_factors;
+    u32 pad;
+};
+
+__global__ void __launch_bounds__(BLOCK)
+finalize_kernel(const u64 *__restrict__ partial, u32 blocks_per_term, const FinTerm *__restrict__ terms, u32 n_terms,
+                u32 degree, const u64 *__restrict__ lagrange /* [k][t][i], 9*9*9 */, u64 const0, u64 const1,
+                u64 *__restrict__ out_dev, u64 *__restrict__ out_host)
+{
+    __shared__ u64 lds[(BLOCK / WAVE) * 2 * MAX_PTS];
+    __shared__ u64 res[2 * MAX_PTS];
+    if (threadIdx.x < 2 * MAX_PTS) res[threadIdx.x] = 0;
+    __syncthreads();
+    for (u32 ti = 0; ti < n_terms; ti++) {
+        const u32 k = terms[ti].n_factors;
+        E2 acc[MAX_PTS];
+#pragma unroll
+        for (int t = 0; t < MAX_PTS; t++) acc[t] = gl::e2_zero();
+        for (u32 b = threadIdx.x; b < blocks_per_term; b += BLOCK) {
+            const u64 *p = partial + ((u64)ti * blocks_per_term + b) * 2 * MAX_PTS;
+#pragma unroll
+            for (int t = 0; t < MAX_PTS; t++) {
+                if ((u32)t <= k) {
+                    acc[t].c0 = gl::add(acc[t].c0, p[2 * t]);
+                    acc[t].c1 = gl::add(acc[t].c1, p[2 * t + 1]);
+                }
+            }
+        }
+        block_reduce<MAX_PTS>(acc, lds);
+        if (threadIdx.x == 0) {
+            const E2 coeff = gl::e2(terms[ti].coeff0, terms[ti].coeff1);
+            for (u32 t = 0; t <= degree; t++) {
+                E2 v;
+                if (t <= k) {
+                    v = acc[0];
+#pragma unroll
+                    for (int i = 1; i < MAX_PTS; i++)
+                        if ((u32)i == t) v = acc[i];
+                } else {
+                    v = gl::e2_zero();
+#pragma unroll
+                    for (int i = 0; i < MAX_PTS; i++) {
+                        if ((u32)i <= k) v = gl::add(v, gl::mul_base(acc[i], lagrange[(k * 9 + t) * 9 + i]));
+                    }
+                }
+                v = gl::mul(v, coeff);
+                res[2 * t] = gl::add(res[2 * t], v.c0);
+                res[2 * t + 1] = gl::add(res[2 * t + 1], v.c1);
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x <= degree) {
+        u32 t = threadIdx.x;
+        u64 c0 = gl::add(res[2 * t], const0), c1 = gl::add(res[2 * t + 1], const1);
+        out_dev[2 * t] = c0;
+        out_dev[2 * t + 1] = c1;
+        if (out_host) {
+            out_host[2 * t] = c0;
+            out_host[2 * t + 1] = c1;
+        }
+    }
+}
+
+// final evaluations: entry 0 of every table after the last fold
+struct GatherDesc {
+    const u64 *c0;
+    const u64 *c1;
+};
+__global__ void gather_kernel(const GatherDesc *__restrict__ d, u32 n, u64 *__restrict__ out)
+{
+    u32 i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    out[2 * i] = d[i].c0[0];
+    out[2 * i + 1] = d[i].c1 ? d[i].c1[0] : 0;
+}
+
+// ---------------------------------------------------------------------------
+// embedding / padding of quantised integers
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(BLOCK)
+embed_i64_kernel(const int64_t *__restrict__ in, u64 len, u64 padded_len, u64 *__restrict__ out)
+{
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < padded_len; i += (u64)gridDim.x * BLOCK)
+        out[i] = i < len ? gl::from_i64(in[i]) : 0;
+}
+
+// ---------------------------------------------------------------------------
+// contraction of one tensor axis with a table beta (partial evaluation):
+//   out[pre][i] = sum_k in[off_pre(pre) + k * stride_k + off_post(i)] * beta[k]
+// The input is addressed through per-dimension strides so that the unpadded
+// region of a padded tensor is read in place.
+// ---------------------------------------------------------------------------
+constexpr int AX_MAX_DIMS = 6;
+struct AxisArgs {
+    const u64 *in0;
+    const u64 *in1;  // nullptr: base field or raw int64
+    int in_is_i64;
+    const u64 *b0;
+    const u64 *b1;
+    u64 K, stride_k;
+    u32 n_pre, n_post;
+    u64 pre_dims[AX_MAX_DIMS], pre_strides[AX_MAX_DIMS];
+    u64 post_dims[AX_MAX_DIMS], post_strides[AX_MAX_DIMS];
+    u64 P, C;  // products of pre_dims / post_dims
+    u64 k_per_slice;
+    u32 n_slices;
+    u64 *o0;
+    u64 *o1;  // [slice][pre][i] when n_slices > 1, else [pre][i]
+};
+
+__device__ __forceinline__ u64 ax_offset(u64 flat, u32 n, const u64 *dims, const u64 *strides)
+{
+    u64 off = 0;
+    for (int d = (int)n - 1; d >= 0; d--) {
+        u64 q = flat / dims[d];
+        off += (flat - q * dims[d]) * strides[d];
+        flat = q;
+    }
+    return off;
+}
+
+__device__ __forceinline__ E2 ax_load(const AxisArgs &a, u64 off)
+{
+    if (a.in_is_i64) return gl::e2(gl::from_i64(((const int64_t *)a.in0)[off]), 0);
+    return gl::e2(a.in0[off], a.in1 ? a.in1[off] : 0);
+}
+
+// lanes over the kept trailing index i (coalesced when the last kept dimension is contiguous)
+__global__ void __launch_bounds__(BLOCK) axis_dot_col_kernel(AxisArgs a)
+{
+    __shared__ u64 lds[BLOCK * 2];
+    const u32 lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const u64 tiles = (a.C + WAVE - 1) / WAVE;
+    const u64 pre = blockIdx.x / tiles;
+    const u64 i = (blockIdx.x - pre * tiles) * WAVE + lane;
+    const u32 slice = blockIdx.y;
+    E2 acc = gl::e2_zero();
+    if (i < a.C) {
+        const u64 base = ax_offset(pre, a.n_pre, a.pre_dims, a.pre_strides) + ax_offset(i, a.n_post, a.post_dims, a.post_strides);
+        u64 k0 = (u64)slice * a.k_per_slice, k1 = k0 + a.k_per_slice;
+        if (k1 > a.K) k1 = a.K;
+        for (u64 k = k0 + wave; k < k1; k += BLOCK / WAVE) {
+            E2 v = ax_load(a, base + k * a.stride_k);
+            E2 b = gl::e2(a.b0[k], a.b1[k]);
+            acc = gl::add(acc, (a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0)));
+        }
+    }
+    lds[threadIdx.x * 2] = acc.c0;
+    lds[threadIdx.x * 2 + 1] = acc.c1;
+    __syncthreads();
+    if (wave == 0 && i < a.C) {
+#pragma unroll
+        for (int w = 1; w < BLOCK / WAVE; w++) {
+            acc.c0 = gl::add(acc.c0, lds[(w * WAVE + lane) * 2]);
+            acc.c1 = gl::add(acc.c1, lds[(w * WAVE + lane) * 2 + 1]);
+        }
+        u64 o = ((u64)slice * a.P + pre) * a.C + i;
+        a.o0[o] = acc.c0;
+        a.o1[o] = acc.c1;
+    }
+}
+
+// one workgroup per output, lanes over k (for C < 64, e.g. a row dot product)
+__global__ void __launch_bounds__(BLOCK) axis_dot_row_kernel(AxisArgs a)
+{
+    __shared__ u64 lds[(BLOCK / WAVE) * 2];
+    const u64 pre = blockIdx.x / a.C;
+    const u64 i = blockIdx.x - pre * a.C;
+    const u32 slice = blockIdx.y;
+    const u64 base = ax_offset(pre, a.n_pre, a.pre_dims, a.pre_strides) + ax_offset(i, a.n_post, a.post_dims, a.post_strides);
+    u64 k0 = (u64)slice * a.k_per_slice, k1 = k0 + a.k_per_slice;
+    if (k1 > a.K) k1 = a.K;
+    E2 acc[1] = {gl::e2_zero()};
+    for (u64 k = k0 + threadIdx.x; k < k1; k += BLOCK) {
+        E2 v = ax_load(a, base + k * a.stride_k);
+        E2 b = gl::e2(a.b0[k], a.b1[k]);
+        acc[0] = gl::add(acc[0], (a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0)));
+    }
+    block_reduce<1>(acc, lds);
+    if (threadIdx.x == 0) {
+        u64 o = ((u64)slice * a.P + pre) * a.C + i;
+        a.o0[o] = acc[0].c0;
+        a.o1[o] = acc[0].c1;
+    }
+}
+
+// sum the k-slices: out[j] = sum_s in[s * n + j]
+__global__ void __launch_bounds__(BLOCK)
+slice_sum_kernel(const u64 *__restrict__ i0, const u64 *__restrict__ i1, u64 n, u32 n_slices, u64 *__restrict__ o0,
+                 u64 *__restrict__ o1)
+{
+    u64 j = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (j >= n) return;
+    u64 a0 = 0, a1 = 0;
+    for (u32 s = 0; s < n_slices; s++) {
+        a0 = gl::add(a0, i0[(u64)s * n + j]);
+        a1 = gl::add(a1, i1[(u64)s * n + j]);
+    }
+    o0[j] = a0;
+    o1[j] = a1;
+}
+
+// copy `rows` rows of `row_len` entries into rows of `padded_len`, zero filling
+__global__ void __launch_bounds__(BLOCK)
+pad_rows_kernel(const u64 *__restrict__ i0, const u64 *__restrict__ i1, u64 rows, u64 row_len, u64 padded_len,
+                u64 *__restrict__ o0, u64 *__restrict__ o1)
+{
+    u64 total = rows * padded_len;
+    for (u64 j = (u64)blockIdx.x * BLOCK + threadIdx.x; j < total; j += (u64)gridDim.x * BLOCK) {
+        u64 r = j / padded_len, c = j - r * padded_len;
+        bool in = c < row_len;
+        o0[j] = in ? i0[r * row_len + c] : 0;
+        o1[j] = in ? (i1 ? i1[r * row_len + c] : 0) : 0;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// LogUp fraction-sum layers: (n1, d1) + (n2, d2) = (n1 d2 + n2 d1, d1 d2) over the
+// low/high halves of the previous layer
+// ---------------------------------------------------------------------------
+constexpr int LOGUP_MAX_COLS = 8;
+struct LogupFirstArgs {
+    const u64 *cols[LOGUP_MAX_COLS];  // base-field columns
+    u32 n_cols;
+    const u64 *numer;  // base-field multiplicities or nullptr (numerators -1)
+    u64 c0, c1;        // constant challenge
+    u64 pw[2 * LOGUP_MAX_COLS];  // powers of the column challenge
+    u64 half;
+    u64 *n0, *n1, *d0, *d1;
+};
+
+__global__ void __launch_bounds__(BLOCK) logup_first_kernel(LogupFirstArgs a)
+{
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.half; i += (u64)gridDim.x * BLOCK) {
+        E2 dlo = gl::e2(a.c0, a.c1), dhi = dlo;
+        for (u32 k = 0; k < a.n_cols; k++) {
+            E2 pw = gl::e2(a.pw[2 * k], a.pw[2 * k + 1]);
+            dlo = gl::add(dlo, gl::mul_base(pw, a.cols[k][i]));
+            dhi = gl::add(dhi, gl::mul_base(pw, a.cols[k][i + a.half]));
+        }
+        E2 num;
+        if (a.numer) {
+            num = gl::add(gl::mul_base(dhi, a.numer[i]), gl::mul_base(dlo, a.numer[i + a.half]));
+        } else {
+            num = gl::neg(gl::add(dlo, dhi));
+        }
+        E2 den = gl::mul(dlo, dhi);
+        a.n0[i] = num.c0;
+        a.n1[i] = num.c1;
+        a.d0[i] = den.c0;
+        a.d1[i] = den.c1;
+    }
+}
+
+__global__ void __launch_bounds__(BLOCK)
+logup_next_kernel(const u64 *__restrict__ pn0, const u64 *__restrict__ pn1, const u64 *__restrict__ pd0,
+                  const u64 *__restrict__ pd1, u64 half, u64 *__restrict__ n0, u64 *__restrict__ n1,
+                  u64 *__restrict__ d0, u64 *__restrict__ d1)
+{
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += (u64)gridDim.x * BLOCK) {
+        E2 nl = gl::e2(pn0[i], pn1[i]), nh = gl::e2(pn0[i + half], pn1[i + half]);
+        E2 dl = gl::e2(pd0[i], pd1[i]), dh = gl::e2(pd0[i + half], pd1[i + half]);
+        E2 num = gl::add(gl::mul(nl, dh), gl::mul(nh, dl));
+        E2 den = gl::mul(dl, dh);
+        n0[i] = num.c0;
+        n1[i] = num.c1;
+        d0[i] = den.c0;
+        d1[i] = den.c1;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// element-wise field operations on device vectors (arithmetic self-check)
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(BLOCK)
+field_op_kernel(int op, const u64 *__restrict__ a0, const u64 *__restrict__ a1, const u64 *__restrict__ b0,
+                const u64 *__restrict__ b1, u64 n, u64 *__restrict__ o0, u64 *__restrict__ o1)
+{
+    u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= n) return;
+    E2 a = gl::e2(a0[i], a1[i]), b = gl::e2(b0[i], b1[i]), r;
+    switch (op) {
+    case 0: r = gl::add(a, b); break;
+    case 1: r = gl::sub(a, b); break;
+    case 2: r = gl::mul(a, b); break;
+    case 3: r = gl::e2(gl::mul(a.c0, b.c0), gl::mul(a.c1, b.c1)); break;  // two independent base products
+    case 4: r = gl::mul_base(a, b.c0); break;
+    case 5: r = gl::e2(gl::from_i64((int64_t)a.c0), gl::mul_small(a.c1, (u32)b.c1)); break;
+    default: r = gl::e2_zero();
+    }
+    o0[i] = r.c0;
+    o1[i] = r.c1;
+}
+
+}  // namespace dpk

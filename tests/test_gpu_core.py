@@ -1,0 +1,261 @@
+"""GPU parity: field arithmetic, table routines and the sumcheck engine through
+the C ABI, bit for bit against the CPU checker on the same seeded inputs."""
+import importlib
+
+import numpy as np
+import pytest
+
+import pyfield as pf
+from pyfield import E2, P
+from util import from_E2, py_rng, rand_base, rand_e2, rand_i64, to_E2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dp():
+    return importlib.import_module("deep-prove_amd")
+
+
+@pytest.fixture(scope="module")
+def ctx(dp):
+    c = dp.Context(0)
+    yield c
+    c.close()
+
+
+ONE = np.array([1, 0], dtype=np.uint64)
+EDGE = [0, 1, 2, 7, P - 1, P - 2, 2**32, 2**32 - 1, 2**32 + 1, 2**63, 2**63 - 1, (P - 1) // 2, (P + 1) // 2, 0xFFFFFFFF,
+        0xFFFFFFFF00000000, 0xFFFFFFFE00000001, 0xFFFFFFFEFFFFFFFF]
+
+
+def test_device_field_arithmetic(ctx):
+    rng = py_rng(11)
+    vals = EDGE + [rng.randrange(P) for _ in range(2000)]
+    # all edge pairs, then random pairs
+    a0 = [x for x in EDGE for _ in EDGE] + vals
+    b0 = [y for _ in EDGE for y in EDGE] + list(reversed(vals))
+    a1 = list(reversed(a0))
+    b1 = [b0[(i * 7 + 3) % len(b0)] for i in range(len(b0))]
+    A = np.array(list(zip(a0, a1)), dtype=np.uint64)
+    B = np.array(list(zip(b0, b1)), dtype=np.uint64)
+    got = {op: ctx.field_op(op, A, B) for op in range(5)}
+    for i in range(len(a0)):
+        x, y = E2(a0[i], a1[i]), E2(b0[i], b1[i])
+        assert tuple(int(v) for v in got[0][i]) == (x + y).pair()
+        assert tuple(int(v) for v in got[1][i]) == (x - y).pair()
+        assert tuple(int(v) for v in got[2][i]) == (x * y).pair()
+        assert tuple(int(v) for v in got[3][i]) == (a0[i] * b0[i] % P, a1[i] * b1[i] % P)
+        assert tuple(int(v) for v in got[4][i]) == (x * E2(b0[i])).pair()
+    # int64 embedding and multiplication by a 32-bit constant
+    ints = [0, 1, -1, 2047, -2048, 2**40, -(2**40), 2**62, -(2**62), -(2**63), 2**63 - 1]
+    A = np.array([[x % 2**64, vals[i]] for i, x in enumerate(ints)], dtype=np.uint64)
+    B = np.array([[0, c] for c in [7, 1, 0, 2**32 - 1, 12345, 7, 7, 7, 7, 7, 7]], dtype=np.uint64)
+    got = ctx.field_op(5, A, B)
+    for i, x in enumerate(ints):
+        assert int(got[i][0]) == x % P
+        assert int(got[i][1]) == vals[i] * int(B[i][1]) % P
+
+
+@pytest.mark.parametrize("m", [0, 1, 2, 5, 8, 9, 11, 16, 17])
+def test_eq_table(ctx, orc, m):
+    point = rand_e2(m, 20 + m)
+    got = ctx.eq_build(point).download()
+    assert (got == orc.eq_evals(point)).all()
+
+
+def test_i64_embedding_and_padding(ctx, orc):
+    v = rand_i64(300, 31, lo=-2**40, hi=2**40)
+    v[:4] = [0, -1, 2**62, -(2**62)]
+    got = ctx.mle_from_i64(v).download()
+    assert got.shape[0] == 512
+    assert (got[:300] == orc.embed_i64(v)).all() and (got[300:] == 0).all()
+
+
+@pytest.mark.parametrize("n", [1, 4, 9, 14])
+def test_evaluate_fix_low_fix_high(ctx, orc, n):
+    tab = rand_e2(1 << n, 40 + n)
+    base = rand_base(1 << n, 50 + n)
+    point = rand_e2(n, 60 + n)
+    m, mb = ctx.mle_from_ext2(tab), ctx.mle_from_base(base)
+    assert (m.evaluate(point) == orc.mle_evaluate(tab, point)).all()
+    assert (mb.evaluate(point) == orc.mle_evaluate(orc.embed_base(base), point)).all()
+    for k in sorted({0, 1, n // 2, n}):
+        assert (m.fix_low(point[:k]).download() == orc.mle_fix_low(tab, point[:k])).all()
+        assert (mb.fix_low(point[:k]).download() == orc.mle_fix_low(orc.embed_base(base), point[:k])).all()
+        assert (m.fix_high(point[n - k:]).download() == orc.mle_fix_high(tab, point[n - k:])).all()
+
+
+def test_vector_and_tensor_mle_layout(ctx):
+    # zkml/src/lib.rs:357-369 and zkml/src/tensor/mod.rs:1874-1897 restated on the GPU tables
+    n = 6
+    v = rand_e2(1 << n, 70)
+    m = ctx.mle_from_ext2(v)
+    for i in [0, 5, 37, 63]:
+        assert (m.evaluate(from_E2([E2((i >> j) & 1) for j in range(n)])) == v[i]).all()
+    rows, cols = 8, 8
+    for r in [0, 3, 7]:
+        row = m.fix_high(from_E2([E2((r >> j) & 1) for j in range(3)]))
+        assert (row.download() == v[r * cols:(r + 1) * cols]).all()
+
+
+def _check_prove(dp, ctx, orc, n, gpu_tabs, orc_tabs, terms, label=b"m2vec"):
+    tr, otr = dp.Transcript(label), orc.OracleTranscript(label)
+    proof, point, finals = ctx.sumcheck_prove(n, gpu_tabs, terms, tr)
+    oproof, opoint, ofinals = orc.sc_prove(n, orc_tabs, terms, otr)
+    assert (proof == oproof).all()
+    assert (point == opoint).all()
+    assert (finals == ofinals).all()
+    assert tr.state() == otr.state()
+    return proof, point, finals
+
+
+SHAPES = [
+    (4, [4, 4], [((1, 0), [0, 1])]),
+    (4, [4, 4, 4], [((1, 0), [0, 1, 2])]),
+    (3, [3, 3, 3, 3], [((5, 9), [0, 2]), ((11, 3), [1, 3])]),
+    (4, [4, 2, 4, 2], [((3, 1), [0, 2]), ((2, 2), [1, 3]), ((7, 0), [0, 1, 2])]),
+    (3, [3], [((1, 0), [0])]),
+    (3, [3, 3, 3, 3, 3], [((1, 0), [0, 1, 2, 3, 4])]),
+    (6, [6, 6, 6, 6, 6, 6], [((1, 0), [0, 1, 2, 3, 4, 5])]),
+    (9, [9, 9, 0, 4], [((2, 3), [0, 1]), ((4, 5), [2, 3, 0]), ((9, 9), [])]),
+    (1, [1, 1], [((1, 0), [0, 1])]),
+    (5, [5, 5], [((1, 0), [0, 0, 1])]),
+    (10, [10, 10, 10, 7, 7, 7], [((1, 1), [0, 1, 2]), ((2, 5), [3, 4, 5]), ((3, 0), [0, 5])]),
+]
+
+
+@pytest.mark.parametrize("case", range(len(SHAPES)))
+def test_sumcheck_matches_checker_small_shapes(dp, ctx, orc, case):
+    n, nvars, terms = SHAPES[case]
+    terms = [(np.array(c, dtype=np.uint64), f) for c, f in terms]
+    tabs = [rand_e2(1 << m, 1000 + 17 * case + k) for k, m in enumerate(nvars)]
+    gpu = [ctx.mle_from_ext2(t) for t in tabs]
+    _check_prove(dp, ctx, orc, n, gpu, tabs, terms)
+
+
+@pytest.mark.parametrize("n", [2, 7, 16])
+def test_config1_plain_product_base_field(dp, ctx, orc, n):
+    # two base-field tables, degree 2 (configuration 1 at n = 16)
+    f, g = rand_base(1 << n, 2000 + n), rand_base(1 << n, 2100 + n)
+    gpu = [ctx.mle_from_base(f), ctx.mle_from_base(g)]
+    proof, _, _ = _check_prove(dp, ctx, orc, n, gpu, [orc.embed_base(f), orc.embed_base(g)], [(ONE, [0, 1])])
+    s = sum(int(a) * int(b) for a, b in zip(f, g)) % P
+    p1 = to_E2(proof[0])
+    assert p1[0] + p1[1] == E2(s)
+
+
+@pytest.mark.parametrize("n,mix", [(3, "bbe"), (8, "bbe"), (15, "bbe"), (9, "bee"), (9, "eee"), (9, "bbb"), (9, "ebe"), (8, "be"), (8, "ee")])
+def test_hadamard_shape_mixed_fields(dp, ctx, orc, n, mix):
+    # eq(r, x) * f(x) * g(x) (zkml/src/layers/hadamard.rs:93-131) with base and extension inputs in every order
+    gpu, ref = [], []
+    for k, kind in enumerate(mix):
+        if kind == "b":
+            v = rand_base(1 << n, 3000 + 31 * n + k)
+            gpu.append(ctx.mle_from_base(v))
+            ref.append(orc.embed_base(v))
+        else:
+            v = rand_e2(1 << n, 3500 + 31 * n + k)
+            gpu.append(ctx.mle_from_ext2(v))
+            ref.append(v)
+    _check_prove(dp, ctx, orc, n, gpu, ref, [(ONE, list(range(len(mix))))])
+
+
+def test_hadamard_proving_roundtrip(dp, ctx, orc):
+    # test_hadamard_proving (zkml/src/layers/hadamard.rs:173-209): prove, verify, check the input claim
+    n = 10
+    v1, v2 = rand_i64(1 << n, 4000), rand_i64(1 << n, 4001)
+    r = rand_e2(n, 4002)
+    out = ctx.mle_from_i64(v1 * v2)
+    claim = out.evaluate(r)
+    m1, m2, beta = ctx.mle_from_i64(v1), ctx.mle_from_i64(v2), ctx.eq_build(r)
+    tr = dp.Transcript()
+    proof, point, finals = ctx.sumcheck_prove(n, [m1, m2, beta], [(ONE, [0, 1, 2])], tr)
+    p1 = to_E2(proof[0])
+    assert p1[0] + p1[1] == to_E2(claim)[0]  # extract_sum == claim
+    rc, vpoint, expected = ctx.sumcheck_verify(claim, proof, dp.Transcript())
+    assert rc == 0 and (vpoint == point).all()
+    beta_eval = orc.identity_eval(r, point)
+    e = to_E2(finals)
+    assert to_E2(beta_eval)[0] == e[2]
+    assert e[0] * e[1] * e[2] == to_E2(expected)[0]
+    assert (m1.evaluate(point) == finals[0]).all() and (m2.evaluate(point) == finals[1]).all()
+    # a tampered proof is rejected
+    bad = proof.copy()
+    bad[3, 0, 0] ^= np.uint64(1)
+    rc, _, _ = ctx.sumcheck_verify(claim, bad, dp.Transcript())
+    assert rc != 0
+
+
+def test_same_poly_shape(dp, ctx, orc):
+    # zkml/src/iop/same_poly.rs:84-114: poly * sum_i a_i * eq_i, challenges as coefficients
+    n, k = 10, 14
+    poly = rand_e2(1 << n, 5000)
+    points = [rand_e2(n, 5001 + i) for i in range(k)]
+    tr, otr = dp.Transcript(), orc.OracleTranscript()
+    a = tr.read_challenges(k)
+    assert (a == otr.read_challenges(k)).all()
+    gpu = [ctx.mle_from_ext2(poly)] + [ctx.eq_build(p) for p in points]
+    ref = [poly] + [orc.eq_evals(p) for p in points]
+    terms = [(a[i], [0, 1 + i]) for i in range(k)]
+    proof, point, finals = ctx.sumcheck_prove(n, gpu, terms, tr)
+    oproof, opoint, ofinals = orc.sc_prove(n, ref, terms, otr)
+    assert (proof == oproof).all() and (point == opoint).all() and (finals == ofinals).all()
+    assert tr.state() == otr.state()
+
+
+def test_round_by_round_session_and_errors(dp, ctx, orc):
+    n = 5
+    tabs = [rand_e2(1 << n, 6000 + k) for k in range(2)]
+    gpu = [ctx.mle_from_ext2(t) for t in tabs]
+    terms = [(ONE, [0, 1])]
+    s = ctx.session(n, gpu, terms)
+    with pytest.raises(dp.DpsError):
+        s.round(ONE)  # round 1 takes no challenge
+    msgs, chal = [], None
+    otr = orc.OracleTranscript()
+    oproof, opoint, ofinals = orc.sc_prove(n, tabs, terms, otr)
+    for j in range(n):
+        msgs.append(s.round(chal))
+        chal = opoint[j]
+    with pytest.raises(dp.DpsError):
+        s.round(chal)  # no round n+1
+    finals = s.finish(chal)
+    with pytest.raises(dp.DpsError):
+        s.finish(chal)
+    assert (np.stack(msgs) == oproof).all() and (finals == ofinals).all()
+    # the borrowed tables are untouched
+    assert (gpu[0].download() == tabs[0]).all()
+    # misuse is reported, not executed
+    with pytest.raises(dp.DpsError):
+        ctx.session(3, gpu, terms)  # tables larger than the sum
+    with pytest.raises(dp.DpsError):
+        ctx.session(n, gpu, [(ONE, [0, 2])])  # unknown table
+    with pytest.raises(dp.DpsError):
+        ctx.session(n, gpu, [(np.array([P, 0], dtype=np.uint64), [0, 1])])  # non-canonical coefficient
+    with pytest.raises(dp.DpsError):
+        ctx.session(n, gpu, [(ONE, [0] * 7)])  # degree above the compiled kernels
+
+
+def test_views_are_borrowed_halves(dp, ctx, orc):
+    # SmartSlice::Borrowed halves as used by the LogUp layers (circuit.rs:260-271)
+    n = 8
+    tab = rand_e2(1 << n, 7000)
+    m = ctx.mle_from_ext2(tab)
+    lo, hi = m.view(0, n - 1), m.view(1 << (n - 1), n - 1)
+    assert (lo.download() == tab[:1 << (n - 1)]).all() and (hi.download() == tab[1 << (n - 1):]).all()
+    _check_prove(dp, ctx, orc, n - 1, [lo, hi], [tab[:1 << (n - 1)], tab[1 << (n - 1):]], [(ONE, [0, 1])])
+    with pytest.raises(dp.DpsError):
+        m.view(1, 3)  # pair loads need an even offset
+    with pytest.raises(dp.DpsError):
+        m.view(1 << n, 1)
+
+
+def test_config3_shape_mid_size(dp, ctx, orc):
+    # eq * f * g with base f, g and extension eq at a size that spans many workgroups
+    n = 20
+    f, g = rand_base(1 << n, 8000), rand_base(1 << n, 8001)
+    r = rand_e2(n, 8002)
+    gpu = [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(r)]
+    ref = [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(r)]
+    _check_prove(dp, ctx, orc, n, gpu, ref, [(ONE, [2, 0, 1])])
