@@ -29,7 +29,25 @@ uint64_t orc_gl_sub(uint64_t a, uint64_t b) { return a >= b ? a - b : (uint64_t)
 
 uint64_t orc_gl_neg(uint64_t a) { return a ? P - a : 0; }
 
+#ifdef ORC_FAST_REDUCE
+/* Build variant used only as the timed CPU baseline: the same product reduced
+ * with 2^64 = 2^32 - 1 and 2^96 = -1 instead of a 128-bit division.  The test
+ * suite checks it against the plain variant. */
+uint64_t orc_gl_mul(uint64_t a, uint64_t b)
+{
+    u128 x = (u128)a * b;
+    uint64_t lo = (uint64_t)x, hi = (uint64_t)(x >> 64);
+    uint64_t hh = hi >> 32, hl = hi & 0xFFFFFFFFu;
+    u128 t = (u128)lo + (u128)hl * 0xFFFFFFFFu + P - hh; /* < 2^64 + 2^64 + 2^64 */
+    uint64_t tl = (uint64_t)t, th = (uint64_t)(t >> 64); /* th <= 2 */
+    u128 u = (u128)tl + th * 0xFFFFFFFFull;
+    uint64_t r = (uint64_t)u;
+    if (u >> 64) r += 0xFFFFFFFFull;
+    return r >= P ? r - P : r;
+}
+#else
 uint64_t orc_gl_mul(uint64_t a, uint64_t b) { return (uint64_t)(((u128)a * b) % P); }
+#endif
 
 uint64_t orc_gl_pow(uint64_t a, uint64_t e)
 {

@@ -20,7 +20,7 @@ AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
 
 def build(force=False):
     """Compile the checker with the Makefile beside this file."""
-    if force or not os.path.exists(_LIB_PATH):
+    if force or not os.path.exists(_LIB_PATH) or not os.path.exists(os.path.join(_HERE, "libdpsc_oracle_fast.so")):
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"])
     return _LIB_PATH
 
@@ -45,13 +45,23 @@ class LogupInstance(C.Structure):
 
 
 _lib = None
+_FAST_PATH = os.path.join(_HERE, "libdpsc_oracle_fast.so")
+_use_fast = False
+
+
+def select(fast: bool):
+    """Switch between the plain checker and its division-free build (the timed
+    CPU baseline).  Both come from the same source; tests compare them."""
+    global _lib, _use_fast
+    if fast != _use_fast:
+        _use_fast, _lib = fast, None
 
 
 def lib():
     global _lib
     if _lib is None:
         build()
-        _lib = C.CDLL(_LIB_PATH)
+        _lib = C.CDLL(_FAST_PATH if _use_fast else _LIB_PATH)
         u64, i64, vp = C.c_uint64, C.c_int64, C.c_void_p
         for name in ("add", "sub", "mul", "pow"):
             f = getattr(_lib, "orc_gl_" + name)

@@ -128,3 +128,23 @@ def test_transcript_layout(orc):
     tr.append_bytes(b"x" * 300); py.append_bytes(b"x" * 300)
     assert tuple(int(v) for v in tr.challenge_scalar()) == py.challenge_scalar()
     assert tr.state() == (py.state, py.k)
+
+
+def test_fast_build_matches_plain_build(orc):
+    # the division-free build (timed as the CPU baseline) against the plain one
+    n = 10
+    tabs = [rand_e2(1 << n, 600 + k) for k in range(3)]
+    terms = [(np.array([3, 4], np.uint64), [0, 1, 2]), (np.array([1, 0], np.uint64), [0, 2])]
+    vals = [0, 1, pf.P - 1, 2**32, 2**32 - 1, 2**63, 0xFFFFFFFF00000000] + [int(x) for x in rand_base(200, 601)]
+    try:
+        orc.select(False)
+        ref = orc.sc_prove(n, tabs, terms, orc.OracleTranscript())
+        orc.select(True)
+        for a in vals:
+            for b in vals[:12]:
+                assert orc.gl_mul(a, b) == a * b % pf.P
+        fast = orc.sc_prove(n, tabs, terms, orc.OracleTranscript())
+    finally:
+        orc.select(False)
+    for x, y in zip(ref, fast):
+        assert (x == y).all()
