@@ -458,3 +458,109 @@ class Context:
         out = np.zeros(2 * n, dtype=np.uint64)
         self._chk(dev.dps_debug_field_op(self._c, op, _ptr(aa), _ptr(bb), n, _ptr(out)), "dps_debug_field_op")
         return np.stack([out[:n], out[n:]], axis=-1)
+
+
+# ---- einsum and LogUp drivers of the host mirror ----
+host.dph_einsum_prove.restype = _i32
+host.dph_einsum_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
+host.dph_logup_batch_prove.restype = _i32
+host.dph_logup_batch_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
+host.dph_logup_batch_verify.restype = _i32
+host.dph_logup_batch_verify.argtypes = [_u32, _vp, _vp, _vp, _vp, _i32, _vp, _u64, _vp, _vp, _vp]
+
+
+def _parse_proof(words, pos):
+    rounds, npts = int(words[pos]), int(words[pos + 1])
+    pos += 2
+    proof = words[pos:pos + 2 * rounds * npts].reshape(rounds, npts, 2).copy()
+    return proof, pos + 2 * rounds * npts
+
+
+def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
+    """EinSum::prove_internal.  ops: list of (lhs_labels, rhs_labels, out_labels);
+    lhs: int64 ndarray (unpadded); rhs: list of int64 ndarrays; claims: list of
+    (point[k, 2], eval[2]) on the outputs.  Returns a dict with the sumcheck proof,
+    the final evaluations, the optional aggregation proof and the input claims."""
+    R = len(ops)
+    lab = []
+    for o in ops:
+        lab += [s.encode() for s in o]
+    labels = (C.c_char_p * (3 * R))(*lab)
+    lhs = np.ascontiguousarray(lhs, dtype=np.int64)
+    lshape = (_u64 * lhs.ndim)(*lhs.shape)
+    rk = [np.ascontiguousarray(x, dtype=np.int64) for x in rhs]
+    rptr = (_vp * R)(*[x.ctypes.data for x in rk])
+    rshapes_keep = [(_u64 * x.ndim)(*x.shape) for x in rk]
+    rshapes = (_vp * R)(*[C.cast(s, _vp).value for s in rshapes_keep])
+    rranks = (_u32 * R)(*[x.ndim for x in rk])
+    pts_keep = [_e2(p).reshape(-1, 2) for p, _ in claims]
+    pts = (_vp * R)(*[p.ctypes.data for p in pts_keep])
+    plens = (_u32 * R)(*[p.shape[0] for p in pts_keep])
+    evals = np.ascontiguousarray(np.stack([_e2(e) for _, e in claims]))
+    cap = 1 << 16
+    out = np.zeros(cap, dtype=np.uint64)
+    n = _u64(0)
+    ctx._chk_host(host.dph_einsum_prove(ctx._c, R, labels, _ptr(lhs), lshape, lhs.ndim, rptr, rshapes, rranks, pts, plens, _ptr(evals),
+                                        transcript._t, _ptr(out), cap, C.byref(n)), "dph_einsum_prove")
+    w = out[: n.value]
+    res = {}
+    res["proof"], pos = _parse_proof(w, 0)
+    ne = int(w[pos])
+    pos += 1
+    res["evaluations"] = w[pos:pos + 2 * ne].reshape(ne, 2).copy()
+    pos += 2 * ne
+    if int(w[pos]) == 0:
+        res["aggregation_proof"] = None
+        pos += 1
+    else:
+        res["aggregation_proof"], pos = _parse_proof(w, pos)
+    nc = int(w[pos])
+    pos += 1
+    res["claims"] = []
+    for _ in range(nc):
+        pl = int(w[pos])
+        pos += 1
+        point = w[pos:pos + 2 * pl].reshape(pl, 2).copy()
+        pos += 2 * pl
+        res["claims"].append((point, w[pos:pos + 2].copy()))
+        pos += 2
+    return res
+
+
+def logup_batch_prove(ctx, instances, transcript):
+    """new_batch_multiple_sizes_prove.  instances: list of dicts with keys cols
+    (list of Mle), numer (Mle or None), c, beta.  Returns the flat proof stream
+    (elements, shape (k, 2)); see dph_logup_batch_prove for the layout."""
+    n = len(instances)
+    ncols = (_u32 * n)(*[len(i["cols"]) for i in instances])
+    flat = [m.handle for i in instances for m in i["cols"]]
+    cols = (_vp * len(flat))(*flat)
+    is_table = instances[0].get("numer") is not None
+    numer = (_vp * n)(*[i["numer"].handle for i in instances]) if is_table else None
+    cs = np.ascontiguousarray(np.stack([_e2(i["c"]) for i in instances]))
+    bs = np.ascontiguousarray(np.stack([_e2(i["beta"]) for i in instances]))
+    total = max(len(i["cols"][0]).bit_length() - 2 for i in instances)
+    cap = sum(v * 4 for v in range(1, total + 1)) + (total + 2) * sum(2 * len(i["cols"]) + 6 for i in instances) + total + 8
+    out = np.zeros((cap, 2), dtype=np.uint64)
+    ne = _u64(0)
+    ctx._chk_host(host.dph_logup_batch_prove(ctx._c, n, ncols, cols, numer, _ptr(cs), _ptr(bs), transcript._t, _ptr(out), cap, C.byref(ne)),
+                  "dph_logup_batch_prove")
+    return out[: ne.value].copy()
+
+
+def logup_batch_verify(instances_meta, is_table, stream, transcript):
+    """new_verify_logup_proof_multiple_sizes.  instances_meta: list of (n_cols,
+    num_vars, c, beta).  Returns (status, claims, point); status 0 = accepted."""
+    n = len(instances_meta)
+    ncols = (_u32 * n)(*[m[0] for m in instances_meta])
+    nvars = (_u32 * n)(*[m[1] for m in instances_meta])
+    cs = np.ascontiguousarray(np.stack([_e2(m[2]) for m in instances_meta]))
+    bs = np.ascontiguousarray(np.stack([_e2(m[3]) for m in instances_meta]))
+    stream = _e2(stream)
+    total = max(m[1] for m in instances_meta)
+    n_claims = sum(m[0] + (1 if is_table else 0) for m in instances_meta)
+    claims = np.zeros((n_claims, 2), dtype=np.uint64)
+    point = np.zeros((total + 1, 2), dtype=np.uint64)
+    rc = host.dph_logup_batch_verify(n, ncols, nvars, _ptr(cs), _ptr(bs), 1 if is_table else 0, _ptr(stream), stream.shape[0], transcript._t,
+                                     _ptr(claims), _ptr(point))
+    return rc, claims, point

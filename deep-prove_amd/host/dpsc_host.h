@@ -45,6 +45,39 @@ int32_t dph_sumcheck_prove(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *
 int32_t dph_sumcheck_verify(const uint64_t claimed_sum[2], const uint64_t *proof, uint32_t n_vars, uint32_t degree,
                             dph_transcript *t, uint64_t *point_out, uint64_t expected_out[2]);
 
+/* ---- EinSum::prove_internal (zkml/src/layers/einsum/prove.rs:46-333) ----
+ * n_ops batched operations share one LHS.  labels: 3*n_ops C strings (lhs, rhs,
+ * out per operation, e.g. "ik","kj","ij").  Tensors arrive unpadded, row-major.
+ * claim_points[r]: 2*len limbs of the claim point on output r, claim_evals 2 per op.
+ * The result is written as 64-bit words:
+ *   rounds, points_per_round, proof limbs..., n_evals, eval limbs...,
+ *   agg_rounds (0 = none), agg proof limbs (3 points per round)...,
+ *   n_claims, then per claim: point_len, point limbs..., eval limbs
+ * Returns DPS_OK and the word count through *n_words. */
+int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const int64_t *lhs,
+                         const uint64_t *lhs_shape, uint32_t lhs_rank, const int64_t *const *rhs,
+                         const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                         const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
+                         const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
+                         uint64_t *n_words);
+
+/* ---- new_batch_multiple_sizes_prove (zkml/src/lookup/logup_gkr/prover.rs:91-344) ----
+ * Instance i has n_cols[i] base-field column tables (handles, flattened in
+ * cols) and, for table instances, a multiplicity table numer[i] (numer is NULL
+ * for lookups).  cs / betas: 2 limbs per instance.  The proof is written as
+ * extension elements (2 words each) in this order: for every layer round v =
+ * 1..total: the v*4 round-message elements, then that round's evaluations;
+ * then the output claim evaluations; the 4 circuit outputs per instance; the
+ * final point (total + 1 elements). */
+int32_t dph_logup_batch_prove(dps_ctx *ctx, uint32_t n_inst, const uint32_t *n_cols, const dps_mle *const *cols,
+                              const dps_mle *const *numer, const uint64_t *cs, const uint64_t *betas,
+                              dph_transcript *t, uint64_t *out, uint64_t out_cap, uint64_t *n_elems);
+/* new_verify_logup_proof_multiple_sizes (verifier.rs:77-256) over the same stream.
+ * claims_out: one element per (multiplicity and) column per instance; point_out: total + 1. */
+int32_t dph_logup_batch_verify(uint32_t n_inst, const uint32_t *n_cols, const uint32_t *inst_nvars, const uint64_t *cs,
+                               const uint64_t *betas, int32_t is_table, const uint64_t *stream, uint64_t n_elems,
+                               dph_transcript *t, uint64_t *claims_out, uint64_t *point_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -3,6 +3,8 @@
 
 #include <string>
 
+#include "dpsc/einsum.hpp"
+#include "dpsc/logup.hpp"
 #include "dpsc/sumcheck.hpp"
 
 using namespace dpsc;
@@ -114,6 +116,163 @@ int32_t dph_sumcheck_verify(const uint64_t claimed_sum[2], const uint64_t *proof
         }
         expected_out[0] = sc.expected_evaluation.c0;
         expected_out[1] = sc.expected_evaluation.c1;
+    });
+}
+
+int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const int64_t *lhs,
+                         const uint64_t *lhs_shape, uint32_t lhs_rank, const int64_t *const *rhs,
+                         const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                         const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
+                         const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
+                         uint64_t *n_words)
+{
+    return guarded([&] {
+        Context c(ctx);
+        auto count = [](const uint64_t *shape, uint32_t rank) {
+            uint64_t n = 1;
+            for (uint32_t i = 0; i < rank; i++) n *= shape[i];
+            return n;
+        };
+        std::vector<einsum::Op> ops;
+        std::vector<einsum::Tensor> rts;
+        std::vector<einsum::Claim> claims;
+        einsum::Tensor lt = einsum::Tensor::from_unpadded(c, std::vector<int64_t>(lhs, lhs + count(lhs_shape, lhs_rank)),
+                                                          std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
+        for (uint32_t r = 0; r < n_ops; r++) {
+            ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
+            rts.push_back(einsum::Tensor::from_unpadded(c, std::vector<int64_t>(rhs[r], rhs[r] + count(rhs_shapes[r], rhs_ranks[r])),
+                                                        std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
+            claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
+        }
+        auto info = einsum::prove_internal(c, ops, lt, rts, claims, t->t);
+        std::vector<uint64_t> w;
+        auto put = [&](const F &x) {
+            w.push_back(x.c0);
+            w.push_back(x.c1);
+        };
+        auto put_proof = [&](const IOPProof &p) {
+            w.push_back(p.proofs.size());
+            w.push_back(p.proofs.empty() ? 0 : p.proofs[0].evaluations.size());
+            for (auto &m : p.proofs)
+                for (auto &e : m.evaluations) put(e);
+        };
+        put_proof(info.proof.einsum_sumcheck);
+        w.push_back(info.proof.einsum_evaluations.size());
+        for (auto &e : info.proof.einsum_evaluations) put(e);
+        if (info.proof.has_aggregation)
+            put_proof(info.proof.input_aggregation_sumcheck);
+        else
+            w.push_back(0);
+        w.push_back(info.claims.size());
+        for (auto &cl : info.claims) {
+            w.push_back(cl.point.size());
+            for (auto &x : cl.point) put(x);
+            put(cl.eval);
+        }
+        if (w.size() > out_cap) throw Error(DPS_ERR_INVALID, "dph_einsum_prove: output buffer too small");
+        memcpy(out, w.data(), w.size() * 8);
+        *n_words = w.size();
+    });
+}
+
+int32_t dph_logup_batch_prove(dps_ctx *ctx, uint32_t n_inst, const uint32_t *n_cols, const dps_mle *const *cols,
+                              const dps_mle *const *numer, const uint64_t *cs, const uint64_t *betas,
+                              dph_transcript *t, uint64_t *out, uint64_t out_cap, uint64_t *n_elems)
+{
+    return guarded([&] {
+        Context c(ctx);
+        // borrowed wrappers around the caller's handles: views share the storage and free only themselves
+        std::vector<std::unique_ptr<DensePolynomial>> keep;
+        auto borrow = [&](const dps_mle *h) {
+            uint64_t len = 0;
+            dps_mle_info(h, nullptr, &len);
+            dps_mle *v = nullptr;
+            c.check(dps_mle_view(h, 0, DensePolynomial::log2_strict(len), &v), "dps_mle_view");
+            keep.emplace_back(new DensePolynomial(c, v));
+            return keep.back().get();
+        };
+        std::vector<logup::LogUpInput> inputs;
+        size_t k = 0;
+        for (uint32_t i = 0; i < n_inst; i++) {
+            std::vector<const DensePolynomial *> cl;
+            for (uint32_t j = 0; j < n_cols[i]; j++) cl.push_back(borrow(cols[k++]));
+            F cc(cs[2 * i], cs[2 * i + 1]), bb(betas[2 * i], betas[2 * i + 1]);
+            if (numer)
+                inputs.push_back(logup::LogUpInput::new_table(cl, borrow(numer[i]), cc, bb));
+            else
+                inputs.push_back(logup::LogUpInput::new_lookup(cl, cc, bb, n_cols[i]));
+        }
+        auto proof = logup::new_batch_multiple_sizes_prove(c, inputs, t->t);
+        std::vector<uint64_t> w;
+        auto put = [&](const F &x) {
+            w.push_back(x.c0);
+            w.push_back(x.c1);
+        };
+        for (size_t v = 0; v < proof.sumcheck_proofs.size(); v++) {
+            for (auto &m : proof.sumcheck_proofs[v].proofs) {
+                if (m.evaluations.size() != 4) throw Error(DPS_ERR_INVALID, "LogUp round message is not degree 3");
+                for (auto &e : m.evaluations) put(e);
+            }
+            for (auto &e : proof.round_evaluations[v]) put(e);
+        }
+        for (auto &cl : proof.output_claims) put(cl.eval);
+        for (auto &o : proof.circuit_outputs)
+            for (auto &e : o) put(e);
+        for (auto &x : proof.output_claims[0].point) put(x);
+        if (w.size() > 2 * out_cap) throw Error(DPS_ERR_INVALID, "dph_logup_batch_prove: output buffer too small");
+        memcpy(out, w.data(), w.size() * 8);
+        *n_elems = w.size() / 2;
+    });
+}
+
+int32_t dph_logup_batch_verify(uint32_t n_inst, const uint32_t *n_cols, const uint32_t *inst_nvars, const uint64_t *cs,
+                               const uint64_t *betas, int32_t is_table, const uint64_t *stream, uint64_t n_elems,
+                               dph_transcript *t, uint64_t *claims_out, uint64_t *point_out)
+{
+    return guarded([&] {
+        std::vector<logup::LogUpVerifierInstance> inst(n_inst);
+        size_t total = 0;
+        for (uint32_t i = 0; i < n_inst; i++) {
+            inst[i].constant_challenge = F(cs[2 * i], cs[2 * i + 1]);
+            inst[i].column_separation_challenge = F(betas[2 * i], betas[2 * i + 1]);
+            inst[i].num_columns = n_cols[i];
+            inst[i].instance_type = is_table ? logup::ProofType::Table : logup::ProofType::Lookup;
+            inst[i].num_vars = inst_nvars[i];
+            total = std::max<size_t>(total, inst_nvars[i]);
+        }
+        auto all = from_limbs(stream, n_elems);
+        size_t pos = 0;
+        auto take = [&](size_t n) {
+            if (pos + n > all.size()) throw Error(DPS_ERR_INVALID, "LogUp proof stream too short");
+            std::vector<F> v(all.begin() + pos, all.begin() + pos + n);
+            pos += n;
+            return v;
+        };
+        logup::LogUpBatchProof proof;
+        proof.proof_type = is_table ? logup::ProofType::Table : logup::ProofType::Lookup;
+        for (size_t v = 1; v <= total; v++) {
+            IOPProof p;
+            for (size_t j = 0; j < v; j++) p.proofs.push_back(IOPProverMessage{take(4)});
+            proof.sumcheck_proofs.push_back(std::move(p));
+            const size_t remaining = total - (v - 1);
+            size_t ne = 0;
+            for (auto &in : inst)
+                if (in.num_vars >= remaining) ne += (v == total) ? in.num_final_round_evals() : 4;
+            proof.round_evaluations.push_back(take(ne));
+        }
+        size_t n_claims = 0;
+        for (auto &in : inst) n_claims += in.num_columns + (is_table ? 1 : 0);
+        take(n_claims);  // the prover's own claim evaluations are recomputed below
+        for (uint32_t i = 0; i < n_inst; i++) proof.circuit_outputs.push_back(take(4));
+        auto res = logup::new_verify_logup_proof_multiple_sizes(proof, inst, t->t);
+        for (size_t i = 0; i < res.output_claims.size(); i++) {
+            claims_out[2 * i] = res.output_claims[i].eval.c0;
+            claims_out[2 * i + 1] = res.output_claims[i].eval.c1;
+        }
+        for (size_t i = 0; i < res.point.size(); i++) {
+            point_out[2 * i] = res.point[i].c0;
+            point_out[2 * i + 1] = res.point[i].c1;
+        }
     });
 }
 

@@ -1,0 +1,318 @@
+"""GPU parity for the callers of the engine: einsum partial evaluation and
+proof (configurations 2 and 4), LogUp-GKR layer build and batched proof
+(configuration 5), each against the CPU checker on the same seeded inputs."""
+import importlib
+
+import numpy as np
+import pytest
+
+from pyfield import E2, P
+from util import from_E2, rand_base, rand_e2, rand_i64, to_E2
+
+pytestmark = pytest.mark.gpu
+C_, O_, S_ = 0, 1, 2
+
+
+@pytest.fixture(scope="module")
+def dp():
+    return importlib.import_module("deep-prove_amd")
+
+
+@pytest.fixture(scope="module")
+def ctx(dp):
+    c = dp.Context(0)
+    yield c
+    c.close()
+
+
+def _pad(shape):
+    return [1 << max(0, (d - 1).bit_length()) for d in shape]
+
+
+def _padded(t):
+    out = np.zeros(_pad(t.shape), dtype=np.int64)
+    out[tuple(slice(0, d) for d in t.shape)] = t
+    return out
+
+
+PE_CASES = [
+    # shape, kinds
+    ((5, 6), [O_, C_]),            # strided column contraction
+    ((6, 7), [C_, O_]),            # contiguous row contraction
+    ((300, 350), [O_, C_]),        # the reference's matmul test sizes (einsum/mod.rs:700-722)
+    ((350, 256), [C_, O_]),
+    ((3, 4, 5), [S_, O_, C_]),     # heads stacked
+    ((4, 8, 2), [O_, C_, O_]),     # two outer axes around the contraction
+    ((2, 3, 4, 5), [S_, O_, C_, C_]),
+    ((8, 16), [C_, C_]),           # nothing to fix: copy and pad
+    ((1, 9), [O_, C_]),
+    ((512, 768), [O_, C_]),        # configuration 2, X
+    ((768, 3072), [C_, O_]),       # configuration 2, W
+    ((8, 512, 256), [S_, O_, C_]), # configuration 4, Q / K
+]
+
+
+@pytest.mark.parametrize("case", range(len(PE_CASES)))
+def test_partial_eval_matches_checker(ctx, orc, case):
+    shape, kinds = PE_CASES[case]
+    t = rand_i64(shape, 100 + case)
+    pd = _pad(shape)
+    points = [rand_e2(max(0, (p - 1).bit_length()), 200 + 10 * case + a) if k != C_ else None for a, (p, k) in enumerate(zip(pd, kinds))]
+    ref = orc.partial_eval(_padded(t), pd, list(shape), kinds, points)
+    dev_t = ctx.tensor_from_i64(_padded(t))
+    got = ctx.partial_eval(dev_t, pd, list(shape), kinds, points)
+    assert len(got) == ref.shape[0]
+    for g, r in zip(got, ref):
+        assert (g.download() == r).all()
+
+
+def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec"):
+    """prove_internal restated with the checker's pieces (einsum/prove.rs:138-316), one or more RHS."""
+    R = len(ops)
+    tr = orc.OracleTranscript(label)
+    lp, lpad = _padded(lhs), _pad(lhs.shape)
+
+    def classify(op, ch):
+        l, r, o = ch in op[0], ch in op[1], ch in op[2]
+        return S_ if (l and r and o) else C_ if (l and r) else O_
+
+    def split(shape, point):
+        out, start = [None] * len(shape), 0
+        for a in reversed(range(len(shape))):
+            ln = max(0, (shape[a] - 1).bit_length())
+            out[a] = point[start:start + ln]
+            start += ln
+        return out
+
+    def reconstruct(fixes, pts, sc_point, shape):
+        out, skip = [], 0
+        for a in reversed(range(len(fixes))):
+            if fixes[a] == C_:
+                ln = max(0, (shape[a] - 1).bit_length())
+                out.append(sc_point[skip:skip + ln])
+                skip += ln
+            else:
+                out.append(pts[a])
+        return np.concatenate(out) if out else np.zeros((0, 2), np.uint64)
+
+    lfix, rfix, lpts, rpts, ltabs, rtabs, coeffs = [], [], [], [], [], [], []
+    for r, op in enumerate(ops):
+        rpad = _pad(rhs[r].shape)
+        out_shape = [lpad[op[0].index(c)] if c in op[0] else rpad[op[1].index(c)] for c in op[2]]
+        sl = split(out_shape, claims[r][0])
+        lk = [classify(op, c) for c in op[0]]
+        rk = [classify(op, c) for c in op[1]]
+        lpt = [None if k == C_ else sl[op[2].index(c)] for c, k in zip(op[0], lk)]
+        rpt = [None if k == C_ else sl[op[2].index(c)] for c, k in zip(op[1], rk)]
+        lfix.append(lk); rfix.append(rk); lpts.append(lpt); rpts.append(rpt)
+        ltabs.append(orc.partial_eval(lp, lpad, list(lhs.shape), lk, lpt))
+        rtabs.append(orc.partial_eval(_padded(rhs[r]), rpad, list(rhs[r].shape), rk, rpt))
+        coeffs.append(orc.stacking_coeffs(lpad, list(lhs.shape), lk, lpt))
+    S = ltabs[0].shape[0]
+    gamma = tr.append_and_sample(b"batching_challenge")
+    tabs = [t for v in ltabs for t in v] + [t for v in rtabs for t in v]
+    nv = int(tabs[0].shape[0]).bit_length() - 1
+    terms, gpow = [], np.array([1, 0], np.uint64)
+    for r in range(R):
+        for j in range(S):
+            terms.append((orc.e2_mul(gpow, coeffs[r][j]), [r * S + j, R * S + r * S + j]))
+        gpow = orc.e2_mul(gpow, gamma)
+    proof, point, finals = orc.sc_prove(nv, tabs, terms, tr)
+    half = len(finals) // 2
+    out_claims = []
+    for r in range(R):
+        ev = np.zeros(2, np.uint64)
+        for j in range(S):
+            ev = orc.e2_add(ev, orc.e2_mul(coeffs[r][j], finals[half + r * S + j]))
+        out_claims.append((reconstruct(rfix[r], rpts[r], point, _pad(rhs[r].shape)), ev))
+    agg = None
+    if R > 1:
+        eqs = [orc.eq_evals(reconstruct(lfix[r], lpts[r], point, lpad)) for r in range(R)]
+        g2 = tr.append_and_sample(b"input_batching_challenge")
+        aterms, gp = [], np.array([1, 0], np.uint64)
+        for r in range(R):
+            aterms.append((gp, [0, 1 + r]))
+            gp = orc.e2_mul(gp, g2)
+        full = orc.embed_i64(lp.reshape(-1))
+        agg, apoint, afinals = orc.sc_prove(int(full.shape[0]).bit_length() - 1, [full] + eqs, aterms, tr)
+        lhs_claim = (apoint, afinals[0])
+    else:
+        ev = np.zeros(2, np.uint64)
+        for j in range(S):
+            ev = orc.e2_add(ev, orc.e2_mul(coeffs[0][j], finals[j]))
+        lhs_claim = (reconstruct(lfix[0], lpts[0], point, lpad), ev)
+    return dict(proof=proof, evaluations=finals, aggregation_proof=agg, claims=[lhs_claim] + out_claims), tr
+
+
+def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed):
+    # output claims: the true MLE evaluations of the integer results
+    claims = []
+    for r, op in enumerate(ops):
+        out = np.einsum(f"{op[0]},{op[1]}->{op[2]}", lhs, rhs[r])
+        nvars = sum(max(0, (d - 1).bit_length()) for d in _pad(out.shape))
+        pt = rand_e2(nvars, seed + r)
+        ev = orc.mle_evaluate(orc.embed_i64(_padded(out).reshape(-1)), pt)
+        claims.append((pt, ev))
+    tr = dp.Transcript()
+    got = dp.einsum_prove(ctx, ops, lhs, rhs, claims, tr)
+    ref, otr = _oracle_einsum(orc, ops, lhs, rhs, claims)
+    assert (got["proof"] == ref["proof"]).all()
+    assert (got["evaluations"] == ref["evaluations"]).all()
+    if ref["aggregation_proof"] is None:
+        assert got["aggregation_proof"] is None
+    else:
+        assert (got["aggregation_proof"] == ref["aggregation_proof"]).all()
+    assert len(got["claims"]) == len(ref["claims"])
+    for (gp, ge), (rp, re) in zip(got["claims"], ref["claims"]):
+        assert (gp == rp).all() and (ge == re).all()
+    assert tr.state() == otr.state()
+    # the proof proves the output claim: p_1(0) + p_1(1) = sum_r gamma^r claim_r
+    vt = orc.OracleTranscript()
+    gamma = vt.append_and_sample(b"batching_challenge")
+    acc, gp = E2(0), E2(1)
+    for _, ev in claims:
+        acc = acc + gp * to_E2(ev)[0]
+        gp = gp * to_E2(gamma)[0]
+    p1 = to_E2(got["proof"][0])
+    assert p1[0] + p1[1] == acc
+    # every input claim is the input tensor's MLE at the claim point
+    tensors = [lhs] + list(rhs)
+    for (pt, ev), t in zip(got["claims"], tensors):
+        assert (orc.mle_evaluate(orc.embed_i64(_padded(t).reshape(-1)), pt) == ev).all()
+    return got
+
+
+def test_einsum_matmul_small(dp, ctx, orc):
+    _check_einsum(dp, ctx, orc, [("ik", "kj", "ij")], rand_i64((5, 6), 1), [rand_i64((6, 7), 2)], 300)
+
+
+def test_einsum_matmul_reference_test_sizes(dp, ctx, orc):
+    # zkml/src/layers/einsum/mod.rs:700-722: 300 x 350 x 256
+    _check_einsum(dp, ctx, orc, [("ik", "kj", "ij")], rand_i64((300, 350), 3), [rand_i64((350, 256), 4)], 310)
+
+
+def test_einsum_stacked(dp, ctx, orc):
+    # A(ijk) @ B(ikl): i stacked
+    _check_einsum(dp, ctx, orc, [("ijk", "ikl", "ijl")], rand_i64((3, 5, 6), 5), [rand_i64((3, 6, 4), 6)], 320)
+
+
+def test_einsum_three_rhs_with_aggregation(dp, ctx, orc):
+    # QKV-like: one LHS against three weights, then the input aggregation sumcheck (prove.rs:260-302)
+    x = rand_i64((6, 8), 7)
+    ws = [rand_i64((8, 5), 8 + k) for k in range(3)]
+    got = _check_einsum(dp, ctx, orc, [("ik", "kj", "ij")] * 3, x, ws, 330)
+    assert got["aggregation_proof"] is not None
+
+
+def test_config2_gpt2_mlp_up_projection(dp, ctx, orc):
+    # X [512 x 768] @ W [768 x 3072], 12-bit entries; 10-variable degree-2 sumcheck over the contraction
+    X, W = rand_i64((512, 768), 11), rand_i64((768, 3072), 12)
+    got = _check_einsum(dp, ctx, orc, [("ik", "kj", "ij")], X, [W], 340)
+    assert got["proof"].shape == (10, 3, 2)
+
+
+def test_config4_attention_scores(dp, ctx, orc):
+    # 'hsd,htd->hst': Q, K [8 x 512 x 256]; 8-variable sumcheck over head_dim with the heads stacked
+    Q, K = rand_i64((8, 512, 256), 13), rand_i64((8, 512, 256), 14)
+    got = _check_einsum(dp, ctx, orc, [("hsd", "htd", "hst")], Q, [K], 350)
+    assert got["proof"].shape == (8, 3, 2) and got["evaluations"].shape[0] == 16
+
+
+def _download_layers(lg):
+    out = []
+    for k in range(1, lg.num_layers()):
+        n, d = lg.layer(k)
+        out.append((n.download(), d.download()))
+    return out
+
+
+@pytest.mark.parametrize("n,ncols,table", [(2, 1, False), (5, 1, False), (10, 2, False), (10, 2, True), (14, 1, True), (16, 3, False)])
+def test_logup_layers_match_checker(ctx, orc, n, ncols, table):
+    cols = [rand_base(1 << n, 400 + 10 * n + k) for k in range(ncols)]
+    numer = rand_base(1 << n, 450 + n) if table else None
+    c, beta = rand_e2(1, 460 + n)[0], rand_e2(1, 470 + n)[0]
+    ref = orc.logup_build(cols, numer, c, beta)
+    lg = ctx.logup_build([ctx.mle_from_base(x) for x in cols], None if numer is None else ctx.mle_from_base(numer), c, beta)
+    got = _download_layers(lg)
+    assert len(got) == len(ref) == n - 1
+    for (gn, gd), (rn, rd) in zip(got, ref):
+        assert (gn == rn).all() and (gd == rd).all()
+    assert (lg.outputs() == np.concatenate(ref[-1])).all()
+
+
+def test_logup_circuit_construction_identity(ctx):
+    # test_circuit_construction (circuit.rs:603-624) on the GPU circuit
+    col = rand_base(1 << 10, 480)
+    lg = ctx.logup_build([ctx.mle_from_base(col)], None, (0, 0), (1, 0))
+    o = to_E2(lg.outputs())
+    expect = 0
+    for v in col:
+        expect = (expect - pow(int(v), P - 2, P)) % P
+    assert (o[0] * o[3] + o[1] * o[2]) * (o[2] * o[3]).inv() == E2(expect)
+
+
+def _logup_case(ctx, sizes, reps, ncols, table, seed):
+    host, dev, meta = [], [], []
+    for n in sizes:
+        for rep in range(reps):
+            cols = [rand_base(1 << n, seed + 100 * n + 10 * rep + k) for k in range(ncols)]
+            numer = rand_base(1 << n, seed + 7 * n + rep) if table else None
+            c, beta = rand_e2(1, seed + 30 + n + rep)[0], rand_e2(1, seed + 40 + n + rep)[0]
+            host.append(dict(cols=cols, numer=numer, c=c, beta=beta))
+            dev.append(dict(cols=[ctx.mle_from_base(x) for x in cols], numer=None if numer is None else ctx.mle_from_base(numer), c=c, beta=beta))
+            meta.append((ncols, n - 1, c, beta))
+    return host, dev, meta
+
+
+@pytest.mark.parametrize("sizes,reps,ncols,table", [((4,), 1, 1, False), ((7, 6, 5), 2, 1, False), ((8, 6), 1, 2, True), ((11, 10, 9, 8, 7), 2, 1, False)])
+def test_logup_batch_prove_matches_checker_and_verifies(dp, ctx, orc, sizes, reps, ncols, table):
+    # the last case is test_logup_batch_prove (logup_gkr/mod.rs:24-79): sizes 2^7..2^11, two instances each
+    host, dev, meta = _logup_case(ctx, sizes, reps, ncols, table, 500)
+    tr, otr = dp.Transcript(), orc.OracleTranscript()
+    got = dp.logup_batch_prove(ctx, dev, tr)
+    ref = orc.logup_batch_prove(host, otr)
+    assert got.shape == ref.shape and (got == ref).all()
+    assert tr.state() == otr.state()
+    # the host mirror's verifier accepts, the checker's verifier accepts, both return the same claims
+    rc, claims, point = dp.logup_batch_verify(meta, table, got, dp.Transcript())
+    orc_rc, oclaims, opoint = orc.logup_batch_verify(meta, table, got, orc.OracleTranscript())
+    assert rc == 0 and orc_rc == 0
+    assert (claims == oclaims).all() and (point == opoint).all()
+    # output claims are the column MLEs at the final point (logup_gkr/mod.rs:70-78)
+    k = 0
+    for (nc, nv, _, _), ins in zip(meta, dev):
+        sub = point[len(point) - (nv + 1):]
+        for col in ([ins["numer"]] if table else []) + ins["cols"]:
+            assert (col.evaluate(sub) == claims[k]).all()
+            k += 1
+    bad = got.copy()
+    bad[3, 1] ^= np.uint64(1)
+    rc, _, _ = dp.logup_batch_verify(meta, table, bad, dp.Transcript())
+    assert rc != 0
+
+
+def test_config5_lookup_argument_reduced(dp, ctx, orc):
+    # configuration 5 at 2^16 lookups into a 2^10-entry table of 16-bit values (full size runs in the benchmark):
+    # multiplicities are exact counts, so the two fraction sums cancel
+    rng = np.random.Generator(np.random.PCG64(600))
+    t_in = np.arange(1 << 10, dtype=np.uint64)
+    t_out = (t_in * np.uint64(40503) + np.uint64(17)) & np.uint64(0xFFFF)
+    idx = rng.integers(0, 1 << 10, size=1 << 16)
+    mult = np.bincount(idx, minlength=1 << 10).astype(np.uint64)
+    tr, otr = dp.Transcript(), orc.OracleTranscript()
+    c, beta = tr.append_and_sample(b"c"), tr.append_and_sample(b"beta")
+    otr.append_and_sample(b"c"), otr.append_and_sample(b"beta")
+    look_h = [dict(cols=[t_in[idx], t_out[idx]], numer=None, c=c, beta=beta)]
+    tab_h = [dict(cols=[t_in, t_out], numer=mult, c=c, beta=beta)]
+    look_d = [dict(cols=[ctx.mle_from_base(x) for x in look_h[0]["cols"]], numer=None, c=c, beta=beta)]
+    tab_d = [dict(cols=[ctx.mle_from_base(x) for x in tab_h[0]["cols"]], numer=ctx.mle_from_base(mult), c=c, beta=beta)]
+    gl, gt = dp.logup_batch_prove(ctx, look_d, tr), dp.logup_batch_prove(ctx, tab_d, tr)
+    rl, rt = orc.logup_batch_prove(look_h, otr), orc.logup_batch_prove(tab_h, otr)
+    assert (gl == rl).all() and (gt == rt).all() and tr.state() == otr.state()
+
+    def frac(stream, total):
+        o = to_E2(stream[-(total + 1) - 4:-(total + 1)])
+        return o[0] * o[3] + o[1] * o[2], o[2] * o[3]
+
+    (nl, dl), (nt, dt) = frac(gl, 15), frac(gt, 9)
+    assert nl * dt + nt * dl == E2(0)
