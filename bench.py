@@ -77,15 +77,18 @@ def main():
     for _ in range(args.warmup):
         prove()
     ctx.sync()
-    per_step = []
+    per_step, proofs = [], []
     t_begin = time.perf_counter()
     for _ in range(args.steps):
         t0 = time.perf_counter()
         (proof, point, finals), tr = prove()
         per_step.append(time.perf_counter() - t0)
+        proofs.append(proof)
     ctx.sync()
     total_s = time.perf_counter() - t_begin
     ms_per_step = 1e3 * total_s / args.steps
+    # every step proves the same statement: all proofs must be identical
+    repeatable = all((q == proofs[0]).all() for q in proofs)
 
     # same steps again with the library's HIP events on, for per-kernel durations
     ctx.profile(True)
@@ -143,6 +146,7 @@ def main():
         "field_elements_per_s": round(element_visits / (ms_per_step * 1e-3), 1),
         "min_step_ms": round(1e3 * min(per_step), 4),
         "eq_build_ms": round(eq_ms, 4),
+        "all_steps_identical": bool(repeatable),
         "upload_s": round(upload_s, 4),
         "roofline": roofline,
     }

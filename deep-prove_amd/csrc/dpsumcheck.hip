@@ -52,9 +52,12 @@ struct dps_ctx {
     std::multimap<size_t, void *> free_blocks;
     std::map<void *, size_t> live_blocks;
     u64 *d_lagrange = nullptr;  // [9][9][9]
+    std::vector<u64> h_lagrange;
     u64 *h_pinned = nullptr;    // host-visible result buffer
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
+    size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
+    u64 seq = 0;                // last sequence number handed to a launch
     bool profiling = false;
     std::vector<ProfRec> recs;
     std::vector<hipEvent_t> ev_pool;
@@ -218,6 +221,17 @@ u64 h_pow(u64 a, u64 e)
     return r;
 }
 u64 h_inv(u64 a) { return h_pow(a, gl::P - 2); }
+E2 h_e2_inv(E2 a)
+{
+    u64 n = h_inv(gl::sub(gl::mul(a.c0, a.c0), gl::mul_small(gl::mul(a.c1, a.c1), (u32)gl::W)));
+    return gl::e2(gl::mul(a.c0, n), gl::mul(gl::neg(a.c1), n));
+}
+// eq1(a, b) = a b + (1 - a)(1 - b)
+E2 h_eq1(E2 a, E2 b)
+{
+    E2 one = gl::e2_one();
+    return gl::add(gl::mul(a, b), gl::mul(gl::sub(one, a), gl::sub(one, b)));
+}
 
 // ---------------------------------------------------------------------------
 // storage
@@ -238,12 +252,22 @@ struct Storage {
 
 }  // namespace
 
+// A table built by dps_eq_build remembers its point.  Behind the 2^m entries of
+// eq(rho, .) the storage holds the tables eq(rho_{l..m-1}, .) for l = 1..m (2^(m-l)
+// entries each, level l at entry offset 2^(m+1) - 2^(m-l+1)): the sumcheck reads
+// level j in round j instead of folding the full table.
+struct EqInfo {
+    u32 m;
+    std::vector<E2> point;
+};
+
 struct dps_mle {
     dps_ctx *ctx;
     std::shared_ptr<Storage> st;
     int32_t kind;
     u64 offset;
     u64 len;
+    std::shared_ptr<EqInfo> eq;  // set on eq tables (and on views covering the whole table)
     const u64 *p0() const { return st->c0 + offset; }
     const u64 *p1() const { return st->c1 ? st->c1 + offset : nullptr; }
 };
@@ -269,7 +293,7 @@ int32_t new_table(dps_ctx *ctx, int32_t kind, u64 len, dps_mle **out)
         CHK(pool_alloc(ctx, len * 8, &p));
         st->c1 = (u64 *)p;
     }
-    dps_mle *m = new (std::nothrow) dps_mle{ctx, st, kind, 0, len};
+    dps_mle *m = new (std::nothrow) dps_mle{ctx, st, kind, 0, len, nullptr};
     if (!m) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
     *out = m;
     return DPS_OK;
@@ -335,11 +359,18 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
                 }
                 lag[(k * 9 + t) * 9 + i] = gl::mul(num, h_inv(den));
             }
+    ctx->h_lagrange = lag;
     if (hipMalloc((void **)&ctx->d_lagrange, lag.size() * 8) != hipSuccess) return bail(DPS_ERR_OOM);
     if (hipMemcpy(ctx->d_lagrange, lag.data(), lag.size() * 8, hipMemcpyHostToDevice) != hipSuccess) return bail(DPS_ERR_HIP);
     ctx->pinned_words = 4096;
-    if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped) != hipSuccess) return bail(DPS_ERR_OOM);
+    // fine-grained host memory: a kernel's system-scope stores become visible to the polling host while the kernel runs
+    if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess) {
+        (void)hipGetLastError();
+        if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped) != hipSuccess) return bail(DPS_ERR_OOM);
+    }
     if (hipHostGetDevicePointer((void **)&ctx->d_pinned, ctx->h_pinned, 0) != hipSuccess) return bail(DPS_ERR_HIP);
+    memset(ctx->h_pinned, 0, ctx->pinned_words * 8);
+    ctx->res_off = ctx->pinned_words - 64;
     *out = ctx;
     return DPS_OK;
 }
@@ -495,7 +526,7 @@ extern "C" int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, v
     st->c0 = (u64 *)d_c0;
     st->c1 = (u64 *)d_c1;
     st->owned = false;
-    *out = new (std::nothrow) dps_mle{ctx, st, kind, 0, len};
+    *out = new (std::nothrow) dps_mle{ctx, st, kind, 0, len, nullptr};
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
 }
 
@@ -507,7 +538,8 @@ extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_
     if (n_vars > 40 || offset > src->len || len > src->len - offset) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: window outside the table");
     // pair loads are 16 bytes wide
     if (n_vars >= 1 && ((src->offset + offset) & 1)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: offset must be even");
-    *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len};
+    *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len, nullptr};
+    if (*out && offset == 0 && len == src->len) (*out)->eq = src->eq;
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
 }
 
@@ -554,7 +586,7 @@ namespace {
 // uploads `words` 64-bit words through the pinned buffer region [slot, slot+words)
 int32_t stage_words(dps_ctx *ctx, const u64 *src, size_t words, size_t slot, const u64 **dev)
 {
-    if (slot + words > ctx->pinned_words) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
+    if (slot + words > ctx->res_off) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
     // the buffer may still be read by queued kernels
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     memcpy(ctx->h_pinned + slot, src, words * 8);
@@ -569,33 +601,72 @@ bool canonical(const u64 *v, size_t n)
     return true;
 }
 
-// eq table of point[0..m) (device pointer to 2*m limbs) into out (2^m entries)
+u64 eq_level_off(u32 m, u32 l) { return (2ull << m) - (2ull << (m - l)); }
+
+// Builds eq(rho, .) and every level eq(rho_{l..m-1}, .), l = 1..m, into o0/o1
+// (2^(m+1) entries).  Levels of at most 2^16 entries come straight from the
+// definition in one launch, together with the 2^8-entry seeds eq(rho_{l..l+7}, .)
+// the larger levels need; level l > 2^16 entries is level l+8 expanded by seed l.
 int32_t eq_build_dev(dps_ctx *ctx, const u64 *d_point, u32 m, u64 *o0, u64 *o1)
 {
-    if (m <= 8) {
-        dpk::eq_seed_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(d_point, m, o0, o1);
-        HIPCHK(ctx, hipGetLastError());
-        return DPS_OK;
+    dpk::EqJobs js;
+    memset(&js, 0, sizeof js);
+    js.point = d_point;
+    js.o0 = o0;
+    js.o1 = o1;
+    u32 n_jobs = 0, max_bits = 0;
+    const u32 first_small = m > 16 ? m - 16 : 0;  // levels first_small..m have at most 16 variables
+    for (u32 l = first_small; l <= m; l++) {
+        js.job[n_jobs++] = dpk::EqJob{l, m - l, eq_level_off(m, l)};
+        max_bits = std::max(max_bits, m - l);
     }
-    // low 8 variables as the in-register factor, the rest recursively
-    const u32 b = 8;
-    void *p = nullptr;
-    CHK(pool_alloc(ctx, (256 + (1ull << (m - b))) * 16, &p));
-    u64 *lo0 = (u64 *)p, *lo1 = lo0 + 256, *hi0 = lo1 + 256, *hi1 = hi0 + (1ull << (m - b));
-    int32_t rc = eq_build_dev(ctx, d_point, b, lo0, lo1);
-    if (rc == DPS_OK) rc = eq_build_dev(ctx, d_point + 2 * b, m - b, hi0, hi1);
-    if (rc == DPS_OK) {
-        u64 n_hi = 1ull << (m - b);
-        u32 blocks = (u32)std::min<u64>(n_hi, MAX_BLOCKS * 4);
-        u32 per_block = (u32)((n_hi + blocks - 1) / blocks);
-        blocks = (u32)((n_hi + per_block - 1) / per_block);
-        ProfScope ps(ctx, DPS_K_EQ, (double)(1ull << m) * 16 + (double)n_hi * 16);
-        dpk::eq_expand_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(hi0, hi1, n_hi, lo0, lo1, b, o0, o1, per_block);
+    // seeds live in a scratch block behind nothing: a separate allocation
+    void *seed_block = nullptr;
+    u64 *seed0 = nullptr, *seed1 = nullptr;
+    if (first_small > 0) {
+        CHK(pool_alloc(ctx, (size_t)first_small * 256 * 16, &seed_block));
+        seed0 = (u64 *)seed_block;
+        seed1 = seed0 + (size_t)first_small * 256;
+    }
+    {
+        ProfScope ps(ctx, DPS_K_EQ, (double)(1ull << std::min<u32>(m, 16)) * 32.0);
+        dpk::eq_define_kernel<<<dim3((u32)(((1ull << max_bits) + dpk::BLOCK - 1) / dpk::BLOCK), n_jobs), dpk::BLOCK, 0, ctx->stream>>>(js);
         hipError_t e = hipGetLastError();
-        if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq_expand launch: %s", hipGetErrorString(e));
+        if (e != hipSuccess) {
+            pool_free(ctx, seed_block);
+            return fail(ctx, DPS_ERR_HIP, "eq_define launch: %s", hipGetErrorString(e));
+        }
+    }
+    int32_t rc = DPS_OK;
+    if (first_small > 0) {
+        // seeds, up to EQ_MAX_JOBS per launch
+        for (u32 base = 0; base < first_small && rc == DPS_OK; base += dpk::EQ_MAX_JOBS) {
+            dpk::EqJobs ss;
+            memset(&ss, 0, sizeof ss);
+            ss.point = d_point;
+            ss.o0 = seed0;
+            ss.o1 = seed1;
+            u32 n = std::min<u32>(first_small - base, dpk::EQ_MAX_JOBS);
+            for (u32 k = 0; k < n; k++) ss.job[k] = dpk::EqJob{base + k, 8, (u64)(base + k) * 256};
+            dpk::eq_define_kernel<<<dim3(1, n), dpk::BLOCK, 0, ctx->stream>>>(ss);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq seed launch: %s", hipGetErrorString(e));
+        }
+        for (u32 l = first_small; l-- > 0 && rc == DPS_OK;) {
+            const u64 n_hi = 1ull << (m - l - 8);
+            const u64 hi_off = eq_level_off(m, l + 8), out_off = eq_level_off(m, l);
+            u32 blocks = (u32)std::min<u64>(n_hi, MAX_BLOCKS * 4);
+            u32 per_block = (u32)((n_hi + blocks - 1) / blocks);
+            blocks = (u32)((n_hi + per_block - 1) / per_block);
+            ProfScope ps(ctx, DPS_K_EQ, (double)(n_hi << 8) * 16 + (double)n_hi * 16);
+            dpk::eq_expand_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(o0 + hi_off, o1 + hi_off, n_hi, seed0 + (size_t)l * 256, seed1 + (size_t)l * 256, 8,
+                                                                         o0 + out_off, o1 + out_off, per_block);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq_expand launch: %s", hipGetErrorString(e));
+        }
     }
     // stream order makes the block reusable by later launches on this stream
-    pool_free(ctx, p);
+    pool_free(ctx, seed_block);
     return rc;
 }
 
@@ -610,12 +681,16 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     u64 dummy[2] = {0, 0};
     CHK(stage_words(ctx, m ? point : dummy, m ? 2 * (size_t)m : 2, 0, &d_point));
     dps_mle *t = nullptr;
-    CHK(new_table(ctx, DPS_EXT2, 1ull << m, &t));
+    CHK(new_table(ctx, DPS_EXT2, 2ull << m, &t));
+    t->len = 1ull << m;
     int32_t rc = eq_build_dev(ctx, d_point, m, t->st->c0, t->st->c1);
     if (rc != DPS_OK) {
         delete t;
         return rc;
     }
+    t->eq = std::make_shared<EqInfo>();
+    t->eq->m = m;
+    for (u32 i = 0; i < m; i++) t->eq->point.push_back(gl::e2(point[2 * i], point[2 * i + 1]));
     *out = t;
     return DPS_OK;
 }
@@ -993,10 +1068,17 @@ struct dps_sc {
     std::vector<std::shared_ptr<Storage>> keep;  // borrowed tables stay alive
     std::vector<dps_term> terms;                 // non-constant terms
     E2 const_sum;                                // sum of the constant terms
-    // fast path: one term, 2 or 3 distinct full-size tables
+    // fast path: one term of distinct full-size tables, at most one of them an eq table
     bool fast;
-    u32 fast_nf;
-    u32 fast_order[3];  // term factors sorted base-first
+    u32 fast_nf;        // streamed tables (the eq factor not counted)
+    u32 fast_order[3];  // streamed factors sorted base-first
+    int fast_eq;        // index of the eq table handled in closed form, or -1
+    std::shared_ptr<EqInfo> eq_info;
+    const u64 *eq_c0, *eq_c1;  // its storage (level 0 at entry 0)
+    E2 fast_coeff;
+    E2 eq_scalar;       // product of eq1(rho_i, r_{i+1}) over the bound variables
+    E2 claim;           // p(0) + p(1) expected from the next message (valid from round 2)
+    std::vector<E2> last_msg;
     void *scratch;      // one pool block holding every ping-pong buffer
     void *dev_block;    // descriptors, partials, per-round result
     // precomputed descriptors (device)
@@ -1010,6 +1092,7 @@ struct dps_sc {
     dpk::GatherDesc *d_gather;
     u64 *d_partial;
     u64 *d_result;
+    u32 *d_counter;  // ticket counter of the evaluation launches, zero between rounds
     std::vector<dpk::ProdArgs> fast_args;  // per round
     std::vector<u32> fast_nb;              // base-field sources per round
     u32 max_blocks;
@@ -1017,25 +1100,27 @@ struct dps_sc {
 
 namespace {
 
-template <int NF, int NB, bool FOLD>
-void launch_prod(dps_ctx *ctx, const dpk::ProdArgs &a, u32 blocks, u64 *partial)
+template <int NF, int NB, bool EQ>
+void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial, const dpk::FastFin &ff)
 {
-    dpk::prod_kernel<NF, NB, FOLD><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial);
+    if (fold)
+        dpk::prod_kernel<NF, NB, true, EQ><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+    else
+        dpk::prod_kernel<NF, NB, false, EQ><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
 }
 
-int32_t launch_prod_dispatch(dps_ctx *ctx, u32 nf, u32 nb, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial)
+int32_t launch_prod_dispatch(dps_ctx *ctx, u32 nf, u32 nb, bool eq, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial,
+                             const dpk::FastFin &ff)
 {
-#define PK(NF_, NB_)                                               \
-    if (nf == NF_ && nb == NB_) {                                  \
-        if (fold)                                                  \
-            launch_prod<NF_, NB_, true>(ctx, a, blocks, partial);  \
-        else                                                       \
-            launch_prod<NF_, NB_, false>(ctx, a, blocks, partial); \
-        return DPS_OK;                                             \
+#define PK(NF_, NB_, EQ_)                                             \
+    if (nf == NF_ && nb == NB_ && eq == EQ_) {                        \
+        launch_prod<NF_, NB_, EQ_>(ctx, fold, a, blocks, partial, ff); \
+        return DPS_OK;                                                \
     }
-    PK(2, 0) PK(2, 1) PK(2, 2) PK(3, 0) PK(3, 1) PK(3, 2) PK(3, 3)
+    PK(2, 0, false) PK(2, 1, false) PK(2, 2, false) PK(3, 0, false) PK(3, 1, false) PK(3, 2, false) PK(3, 3, false)
+    PK(1, 0, true) PK(1, 1, true) PK(2, 0, true) PK(2, 1, true) PK(2, 2, true)
 #undef PK
-    return fail(ctx, DPS_ERR_UNSUPPORTED, "no product kernel for %u factors, %u base", nf, nb);
+    return fail(ctx, DPS_ERR_UNSUPPORTED, "no product kernel for %u tables, %u base, eq %d", nf, nb, (int)eq);
 }
 
 u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
@@ -1085,7 +1170,10 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
 
     // fast path test
     sc->fast = false;
-    if (sc->n_terms == 1 && (sc->terms[0].n_factors == 2 || sc->terms[0].n_factors == 3) && n_vars >= 1) {
+    sc->fast_eq = -1;
+    sc->eq_scalar = gl::e2_one();
+    sc->claim = gl::e2_zero();
+    if (sc->n_terms == 1 && sc->terms[0].n_factors >= 2 && sc->terms[0].n_factors <= 3 && n_vars >= 1) {
         const dps_term &t = sc->terms[0];
         bool ok = true;
         for (u32 f = 0; f < t.n_factors && ok; f++) {
@@ -1094,13 +1182,25 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                 if (t.factors[q] == t.factors[f]) ok = false;
         }
         if (ok) {
-            sc->fast = true;
-            sc->fast_nf = t.n_factors;
+            for (u32 f = 0; f < t.n_factors && sc->fast_eq < 0; f++) {
+                const dps_mle *h = mles[t.factors[f]];
+                if (h->eq && h->eq->m == n_vars && h->kind == DPS_EXT2) {
+                    sc->fast_eq = (int)t.factors[f];
+                    sc->eq_info = h->eq;
+                    sc->eq_c0 = h->p0();
+                    sc->eq_c1 = h->p1();
+                }
+            }
             u32 w = 0;
             for (u32 f = 0; f < t.n_factors; f++)
-                if (mles[t.factors[f]]->kind == DPS_BASE) sc->fast_order[w++] = t.factors[f];
+                if ((int)t.factors[f] != sc->fast_eq && mles[t.factors[f]]->kind == DPS_BASE) sc->fast_order[w++] = t.factors[f];
             for (u32 f = 0; f < t.n_factors; f++)
-                if (mles[t.factors[f]]->kind != DPS_BASE) sc->fast_order[w++] = t.factors[f];
+                if ((int)t.factors[f] != sc->fast_eq && mles[t.factors[f]]->kind != DPS_BASE) sc->fast_order[w++] = t.factors[f];
+            sc->fast_nf = w;
+            // compiled variants: 2 or 3 streamed tables without an eq factor, 1 or 2 with one
+            sc->fast = sc->fast_eq >= 0 ? (w >= 1 && w <= 2) : (w >= 2 && w <= 3);
+            if (!sc->fast) sc->fast_eq = -1;
+            sc->fast_coeff = gl::e2(t.coeff[0], t.coeff[1]);
         }
     }
 
@@ -1175,7 +1275,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             }
             for (u32 k = 0; k < n_mles; k++) {
                 SessMle &s = sim[k];
-                if (s.nv != prev_live) continue;
+                if (s.nv != prev_live || (int)k == sc->fast_eq) continue;
                 dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1)};
                 folds.push_back(d);
                 if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
@@ -1234,7 +1334,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     size_t bytes_fin = round_up(fins.size() * sizeof(dpk::FinTerm), 256);
     size_t bytes_gath = round_up(gath.size() * sizeof(dpk::GatherDesc), 256);
     size_t bytes_partial = round_up((size_t)std::max<u32>(sc->n_terms, 1) * sc->max_blocks * 2 * dpk::MAX_PTS * 8, 256);
-    size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256);
+    size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256) + 256;
     size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_partial + bytes_result;
     int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
     if (rc != DPS_OK) return cleanup(rc);
@@ -1252,6 +1352,11 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->d_partial = (u64 *)p;
     p += bytes_partial;
     sc->d_result = (u64 *)p;
+    sc->d_counter = (u32 *)(p + bytes_result - 256);
+    {
+        hipError_t e = hipMemsetAsync(sc->d_counter, 0, 256, ctx->stream);
+        if (e != hipSuccess) return cleanup(fail(ctx, DPS_ERR_HIP, "counter reset: %s", hipGetErrorString(e)));
+    }
     // one staged upload of all descriptors
     std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath, 0);
     char *q = stage.data();
@@ -1303,6 +1408,30 @@ int32_t launch_folds(dps_sc *sc, u32 step, bool extra_only, const u64 *chal)
 
 }  // namespace
 
+namespace {
+
+// Wait until the launch that carries `seq` has published its result.  The host
+// polls the sequence word the last workgroup stores after the message; if it
+// does not arrive the stream is synchronised to surface the error.
+int32_t wait_result(dps_ctx *ctx, u64 seq)
+{
+    volatile u64 *flag = ctx->h_pinned + ctx->res_off + dpk::HOST_SEQ_SLOT;
+    for (u64 spins = 0;; spins++) {
+        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return DPS_OK;
+        if ((spins & 0xFFFFF) == 0xFFFFF) {
+            // about once per several milliseconds: has the stream died or finished without publishing?
+            hipError_t q = hipStreamQuery(ctx->stream);
+            if (q == hipSuccess) {
+                if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return DPS_OK;
+                return fail(ctx, DPS_ERR_HIP, "round result was not published");
+            }
+            if (q != hipErrorNotReady) return fail(ctx, DPS_ERR_HIP, "stream error while waiting for a round: %s", hipGetErrorString(q));
+        }
+    }
+}
+
+}  // namespace
+
 extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
 {
     if (!sc || !evals_out) return DPS_ERR_INVALID;
@@ -1315,24 +1444,100 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
     const u32 live = sc->n_vars - j + 1;
     const u64 n_pairs = 1ull << (live - 1);
     u32 blocks = blocks_for_pairs(n_pairs);
+    // constant terms: c summed over 2^(live-1) suffixes at every evaluation point
+    E2 cst = gl::mul_base(sc->const_sum, h_pow(2, live - 1));
+    dpk::FinArgs fa;
+    memset(&fa, 0, sizeof fa);
+    fa.partial = sc->d_partial;
+    fa.blocks_per_term = sc->n_terms ? blocks : 0;
+    fa.n_terms = sc->n_terms;
+    fa.terms = sc->d_fin;
+    fa.degree = sc->degree;
+    fa.total_blocks = blocks * sc->n_terms;
+    fa.lagrange = ctx->d_lagrange;
+    fa.const0 = cst.c0;
+    fa.const1 = cst.c1;
+    fa.out_dev = sc->d_result;
+    fa.out_host = ctx->d_pinned + ctx->res_off;
+    fa.seq = ++ctx->seq;
+    fa.counter = sc->d_counter;
     if (sc->n_terms == 0) {
-        blocks = 0;
         if (j >= 2) CHK(launch_folds(sc, j, false, challenge));
+        ProfScope ps(ctx, DPS_K_FINALIZE, 0.0);
+        dpk::finalize_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(fa);
+        HIPCHK(ctx, hipGetLastError());
     } else if (sc->fast) {
         dpk::ProdArgs a = sc->fast_args[j];
+        const bool has_eq = sc->fast_eq >= 0;
+        const u32 nf = sc->fast_nf;
+        dpk::FastFin ff;
+        memset(&ff, 0, sizeof ff);
         if (j >= 2) {
-            a.r0 = challenge[0];
-            a.r1 = challenge[1];
+            const E2 r = gl::e2(challenge[0], challenge[1]);
+            a.r0 = r.c0;
+            a.r1 = r.c1;
             CHK(launch_folds(sc, j, true, challenge));
+            // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
+            const u32 d = sc->degree;
+            E2 acc = gl::e2_zero();
+            for (u32 k = 0; k <= d; k++) {
+                E2 num = gl::e2_one();
+                u64 den = 1;
+                for (u32 m = 0; m <= d; m++) {
+                    if (m == k) continue;
+                    num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+                    den = gl::mul(den, gl::sub((u64)k, (u64)m));
+                }
+                acc = gl::add(acc, gl::mul(gl::mul_base(num, h_inv(den)), sc->last_msg[k]));
+            }
+            sc->claim = acc;
+            if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
         }
-        double bytes = 0;
-        for (u32 f = 0; f < sc->fast_nf; f++) {
+        // scale(t) = coeff * S * eq1(rho_{j-1}, t)
+        E2 base_scale = sc->fast_coeff;
+        if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
+        for (u32 t = 0; t <= sc->degree; t++) {
+            E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
+            ff.scale[2 * t] = sc_t.c0;
+            ff.scale[2 * t + 1] = sc_t.c1;
+        }
+        E2 s1 = gl::e2(ff.scale[2], ff.scale[3]);
+        const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
+        if (skip1) {
+            E2 inv = h_e2_inv(s1);
+            ff.inv_s1_0 = inv.c0;
+            ff.inv_s1_1 = inv.c1;
+            // the constant terms add c to p(0) and to p(1)
+            E2 cl = gl::sub(sc->claim, gl::add(cst, cst));
+            ff.claim0 = cl.c0;
+            ff.claim1 = cl.c1;
+        }
+        a.skip1 = skip1 ? 1 : 0;
+        if (has_eq) {
+            const u64 off = eq_level_off(sc->n_vars, j);
+            a.q0 = sc->eq_c0 + off;
+            a.q1 = sc->eq_c1 + off;
+            for (u32 i = 0; i <= nf; i++) ff.ext[i] = ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i];
+        }
+        ff.partial = sc->d_partial;
+        ff.n_blocks = blocks;
+        ff.degree = sc->degree;
+        ff.has_eq = has_eq ? 1 : 0;
+        ff.skip1 = a.skip1;
+        ff.const0 = cst.c0;
+        ff.const1 = cst.c1;
+        ff.out_dev = sc->d_result;
+        ff.out_host = fa.out_host;
+        ff.seq = fa.seq;
+        ff.counter = sc->d_counter;
+        double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
+        for (u32 f = 0; f < nf; f++) {
             double eb = a.s1[f] ? 16.0 : 8.0;
             bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
         }
         {
             ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
-            CHK(launch_prod_dispatch(ctx, sc->fast_nf, sc->fast_nb[j], j >= 2, a, blocks, sc->d_partial));
+            CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j], has_eq, j >= 2, a, blocks, sc->d_partial, ff));
             HIPCHK(ctx, hipGetLastError());
         }
     } else {
@@ -1341,20 +1546,16 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             u32 n = std::min<u32>(sc->n_terms - base, 65535);
             ProfScope ps(ctx, DPS_K_EVAL_TERMS, 0.0);
             dpk::eval_terms_kernel<<<dim3(blocks, n), dpk::BLOCK, 0, ctx->stream>>>(
-                sc->d_terms + sc->term_off[j] + base, n_pairs, sc->d_partial + (size_t)base * blocks * 2 * dpk::MAX_PTS);
+                sc->d_terms + sc->term_off[j] + base, n_pairs, sc->d_partial + (size_t)base * blocks * 2 * dpk::MAX_PTS, fa);
             HIPCHK(ctx, hipGetLastError());
         }
     }
-    // constant terms: c summed over 2^(live-1) suffixes at every evaluation point
-    E2 cst = gl::mul_base(sc->const_sum, h_pow(2, live - 1));
-    {
-        ProfScope ps(ctx, DPS_K_FINALIZE, 0.0);
-        dpk::finalize_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(sc->d_partial, blocks, sc->d_fin, sc->n_terms, sc->degree, ctx->d_lagrange,
-                                                                  cst.c0, cst.c1, sc->d_result, ctx->d_pinned);
-        HIPCHK(ctx, hipGetLastError());
+    CHK(wait_result(ctx, fa.seq));
+    memcpy(evals_out, ctx->h_pinned + ctx->res_off, 2 * (sc->degree + 1) * 8);
+    if (sc->fast) {
+        sc->last_msg.resize(sc->degree + 1);
+        for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
     }
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    memcpy(evals_out, ctx->h_pinned, 2 * (sc->degree + 1) * 8);
     sc->round = j;
     return DPS_OK;
 }
@@ -1375,6 +1576,12 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
     }
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     if (sc->n_mles) memcpy(final_evals_out, ctx->h_pinned, 2 * (size_t)sc->n_mles * 8);
+    if (sc->fast_eq >= 0) {
+        // the eq table was never folded: its value at the challenge point is the product of the one-variable factors
+        E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], gl::e2(challenge[0], challenge[1])));
+        final_evals_out[2 * sc->fast_eq] = v.c0;
+        final_evals_out[2 * sc->fast_eq + 1] = v.c1;
+    }
     sc->finished = true;
     return DPS_OK;
 }
@@ -1506,8 +1713,8 @@ extern "C" int32_t dps_logup_layer(const dps_logup *lg, uint32_t k, dps_mle **nu
     if (!lg || !num || !den) return DPS_ERR_INVALID;
     if (k < 1 || k >= lg->n_layers) return fail(lg->ctx, DPS_ERR_INVALID, "dps_logup_layer: layer %u of %u", k, lg->n_layers);
     u64 sz = lg->len >> k;
-    *num = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k], sz};
-    *den = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k] + sz, sz};
+    *num = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k], sz, nullptr};
+    *den = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k] + sz, sz, nullptr};
     if (!*num || !*den) return fail(lg->ctx, DPS_ERR_OOM, "host allocation failed");
     return DPS_OK;
 }

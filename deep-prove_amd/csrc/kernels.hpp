@@ -49,62 +49,107 @@ __device__ __forceinline__ E2 tab_get(const u64 *c0, const u64 *c1, u64 i)
 // ---------------------------------------------------------------------------
 // block reduction of NP extension elements; result valid in thread 0
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ u64 shfl_down64(u64 v, int delta)
+// Sum over the workgroup of canonical field values.  Modular additions across
+// lanes would cost a shuffle pair plus a conditional subtraction per step; instead
+// every value is cut into three chunks of at most 22 bits, the chunks are summed
+// as plain 32-bit integers (256 threads x 2^22 < 2^31) with DPP row operations,
+// and the three integer sums are recombined and reduced once.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ u32 dpp_add(u32 x)
 {
-    u32 lo = (u32)v, hi = (u32)(v >> 32);
-    lo = __shfl_down(lo, delta, WAVE);
-    hi = __shfl_down(hi, delta, WAVE);
-    return ((u64)hi << 32) | lo;
+    // lanes outside ROW_MASK receive 0
+    return x + (u32)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, ROW_MASK, 0xF, true);
 }
 
-template <int NP>
-__device__ __forceinline__ void block_reduce(E2 (&acc)[NP], u64 *lds /* [BLOCK/WAVE][2*NP] */)
+// after this call lane 63 holds the sum over the wavefront
+__device__ __forceinline__ u32 wave_sum_u32(u32 x)
 {
-#pragma unroll
-    for (int t = 0; t < NP; t++) {
-#pragma unroll
-        for (int d = WAVE / 2; d >= 1; d >>= 1) {
-            acc[t].c0 = gl::add(acc[t].c0, shfl_down64(acc[t].c0, d));
-            acc[t].c1 = gl::add(acc[t].c1, shfl_down64(acc[t].c1, d));
-        }
-    }
+    x = dpp_add<0xB1, 0xF>(x);   // quad_perm [1,0,3,2]
+    x = dpp_add<0x4E, 0xF>(x);   // quad_perm [2,3,0,1]
+    x = dpp_add<0x141, 0xF>(x);  // row_half_mirror: the other quad of each 8 lanes
+    x = dpp_add<0x140, 0xF>(x);  // row_mirror: the other half of each row of 16
+    x = dpp_add<0x142, 0xA>(x);  // row_bcast:15 into rows 1 and 3
+    x = dpp_add<0x143, 0xC>(x);  // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
+// values in, sums out (valid in thread 0 only).  lds: (BLOCK / WAVE) * 3 * NV words.
+template <int NV>
+__device__ __forceinline__ void block_sum(u64 (&v)[NV], u32 *lds)
+{
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    if (lane == 0) {
 #pragma unroll
-        for (int t = 0; t < NP; t++) {
-            lds[wave * 2 * NP + 2 * t] = acc[t].c0;
-            lds[wave * 2 * NP + 2 * t + 1] = acc[t].c1;
+    for (int i = 0; i < NV; i++) {
+        u32 lo = (u32)v[i], hi = (u32)(v[i] >> 32);
+        u32 c0 = wave_sum_u32(lo & 0x3FFFFFu);
+        u32 c1 = wave_sum_u32((lo >> 22) | ((hi & 0xFFFu) << 10));
+        u32 c2 = wave_sum_u32(hi >> 12);
+        if (lane == WAVE - 1) {
+            lds[(wave * NV + i) * 3 + 0] = c0;
+            lds[(wave * NV + i) * 3 + 1] = c1;
+            lds[(wave * NV + i) * 3 + 2] = c2;
         }
     }
     __syncthreads();
     if (threadIdx.x == 0) {
 #pragma unroll
-        for (int w = 1; w < BLOCK / WAVE; w++) {
+        for (int i = 0; i < NV; i++) {
+            u64 c0 = 0, c1 = 0, c2 = 0;
 #pragma unroll
-            for (int t = 0; t < NP; t++) {
-                acc[t].c0 = gl::add(acc[t].c0, lds[w * 2 * NP + 2 * t]);
-                acc[t].c1 = gl::add(acc[t].c1, lds[w * 2 * NP + 2 * t + 1]);
+            for (int w = 0; w < BLOCK / WAVE; w++) {
+                c0 += lds[(w * NV + i) * 3 + 0];
+                c1 += lds[(w * NV + i) * 3 + 1];
+                c2 += lds[(w * NV + i) * 3 + 2];
             }
+            // c0 + c1 * 2^22 + c2 * 2^44 < 2^75
+            unsigned __int128 t = (unsigned __int128)c0 + ((unsigned __int128)c1 << 22) + ((unsigned __int128)c2 << 44);
+            v[i] = gl::reduce128((u64)t, (u64)(t >> 64));
         }
     }
+}
+
+template <int NP>
+__device__ __forceinline__ void block_reduce(E2 (&acc)[NP], u32 *lds /* (BLOCK / WAVE) * 6 * NP words */)
+{
+    u64 v[2 * NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) {
+        v[2 * t] = acc[t].c0;
+        v[2 * t + 1] = acc[t].c1;
+    }
+    block_sum<2 * NP>(v, lds);
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::e2(v[2 * t], v[2 * t + 1]);
 }
 
 // ---------------------------------------------------------------------------
 // eq(r, x) table
 // ---------------------------------------------------------------------------
-// Seed: up to 2^8 entries, one per thread, straight from the definition.
-__global__ void __launch_bounds__(BLOCK) eq_seed_kernel(const u64 *__restrict__ point /* 2*m limbs */, u32 m,
-                                                         u64 *__restrict__ o0, u64 *__restrict__ o1)
+// Small tables straight from the definition, many per launch.  Job k (blockIdx.y)
+// writes 2^n_bits entries: out[i] = prod_b (bit_b(i) ? r[first + b] : 1 - r[first + b]).
+constexpr int EQ_MAX_JOBS = 48;
+struct EqJob {
+    u32 first, n_bits;
+    u64 out_off;  // entries from the start of the output arrays
+};
+struct EqJobs {
+    const u64 *point;  // 2 limbs per coordinate
+    u64 *o0, *o1;
+    EqJob job[EQ_MAX_JOBS];
+};
+
+__global__ void __launch_bounds__(BLOCK) eq_define_kernel(EqJobs js)
 {
-    u32 i = threadIdx.x;
-    if (i >= (1u << m)) return;
+    const EqJob j = js.job[blockIdx.y];
+    const u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= ((u64)1 << j.n_bits)) return;
     E2 acc = gl::e2_one();
-    for (u32 j = 0; j < m; j++) {
-        E2 r = gl::e2(point[2 * j], point[2 * j + 1]);
-        acc = gl::mul(acc, ((i >> j) & 1) ? r : gl::sub(gl::e2_one(), r));
+    for (u32 b = 0; b < j.n_bits; b++) {
+        E2 r = gl::e2(js.point[2 * (j.first + b)], js.point[2 * (j.first + b) + 1]);
+        acc = gl::mul(acc, ((i >> b) & 1) ? r : gl::sub(gl::e2_one(), r));
     }
-    o0[i] = acc.c0;
-    o1[i] = acc.c1;
+    js.o0[j.out_off + i] = acc.c0;
+    js.o1[j.out_off + i] = acc.c1;
 }
 
 // Expansion: out[h * 2^b + l] = hi[h] * lo[l], lo has 2^b <= 256 entries.  Each
@@ -168,6 +213,138 @@ __global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict_
 }
 
 // ---------------------------------------------------------------------------
+// round result: the last workgroup of an evaluation launch sums the block
+// partials of every term, scales by the term's coefficient, extends a degree-k
+// term to the d+1 points of the round message (Lagrange weights over the nodes
+// 0..k), adds the constant terms, and publishes the message to host-visible
+// memory followed by a sequence number the host polls.
+// ---------------------------------------------------------------------------
+struct FinTerm {
+    u64 coeff0, coeff1;
+    u32 n_factors;
+    u32 pad;
+};
+
+struct FinArgs {
+    const u64 *partial;    // [term][block][2 * MAX_PTS]
+    u32 blocks_per_term;
+    u32 n_terms;
+    const FinTerm *terms;
+    u32 degree;
+    u32 total_blocks;      // workgroups that take a ticket before the result is complete
+    const u64 *lagrange;   // [k][t][i], 9*9*9
+    u64 const0, const1;    // constant terms summed over the remaining hypercube
+    u64 *out_dev;          // 2 * (degree + 1) limbs
+    u64 *out_host;         // same, host-visible; out_host[HOST_SEQ_SLOT] receives seq
+    u64 seq;
+    u32 *counter;          // ticket counter, zero between launches
+};
+constexpr int HOST_SEQ_SLOT = 2 * MAX_PTS;
+
+// Block partials cross XCDs (each XCD has its own L2).  They are written and read
+// with agent-scope accesses, which go through to the coherence point, so that no
+// workgroup has to write back or invalidate a whole L2: a cache-wide release or
+// acquire per workgroup stalls the streaming loads of every other workgroup on
+// that XCD.
+__device__ __forceinline__ u64 ld_agent(const u64 *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(u64 *p, u64 v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Called by every thread of one workgroup once all partials are visible.
+template <int NPMAX>
+__device__ __forceinline__ void finalize_block(const FinArgs &fa, u32 *lds /* (BLOCK / WAVE) * 6 * MAX_PTS words */, u64 *res /* 2 * MAX_PTS */)
+{
+    if (threadIdx.x < 2 * MAX_PTS) res[threadIdx.x] = 0;
+    __syncthreads();
+    for (u32 ti = 0; ti < fa.n_terms; ti++) {
+        const u32 k = fa.terms[ti].n_factors;
+        E2 acc[NPMAX];
+#pragma unroll
+        for (int t = 0; t < NPMAX; t++) acc[t] = gl::e2_zero();
+        for (u32 b = threadIdx.x; b < fa.blocks_per_term; b += BLOCK) {
+            const u64 *p = fa.partial + ((u64)ti * fa.blocks_per_term + b) * 2 * MAX_PTS;
+#pragma unroll
+            for (int t = 0; t < NPMAX; t++) {
+                if ((u32)t <= k) {
+                    acc[t].c0 = gl::add(acc[t].c0, ld_agent(p + 2 * t));
+                    acc[t].c1 = gl::add(acc[t].c1, ld_agent(p + 2 * t + 1));
+                }
+            }
+        }
+        block_reduce<NPMAX>(acc, lds);
+        if (threadIdx.x == 0) {
+            const E2 coeff = gl::e2(fa.terms[ti].coeff0, fa.terms[ti].coeff1);
+            for (u32 t = 0; t <= fa.degree; t++) {
+                E2 v;
+                if (t <= k) {
+                    v = acc[0];
+#pragma unroll
+                    for (int i = 1; i < NPMAX; i++)
+                        if ((u32)i == t) v = acc[i];
+                } else {
+                    v = gl::e2_zero();
+#pragma unroll
+                    for (int i = 0; i < NPMAX; i++) {
+                        if ((u32)i <= k) v = gl::add(v, gl::mul_base(acc[i], fa.lagrange[(k * 9 + t) * 9 + i]));
+                    }
+                }
+                v = gl::mul(v, coeff);
+                res[2 * t] = gl::add(res[2 * t], v.c0);
+                res[2 * t + 1] = gl::add(res[2 * t + 1], v.c1);
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x <= fa.degree) {
+        u32 t = threadIdx.x;
+        u64 c0 = gl::add(res[2 * t], fa.const0), c1 = gl::add(res[2 * t + 1], fa.const1);
+        fa.out_dev[2 * t] = c0;
+        fa.out_dev[2 * t + 1] = c1;
+        // system-scope stores go through to host memory; no cache-wide write-back is needed for them
+        __hip_atomic_store(fa.out_host + 2 * t, c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(fa.out_host + 2 * t + 1, c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __builtin_amdgcn_s_waitcnt(0);  // the message has been acknowledged ...
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        *fa.counter = 0;
+        // ... before the sequence number the host polls is stored
+        __hip_atomic_store(fa.out_host + HOST_SEQ_SLOT, fa.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+// Every workgroup calls this after writing its partial (thread 0 wrote it).
+// Returns true in the workgroup that took the last ticket.
+__device__ __forceinline__ bool take_ticket(u32 *counter, u32 total_blocks, int *flag_lds)
+{
+    if (threadIdx.x == 0) {
+        // thread 0 wrote the partial with agent-scope stores: wait for them to be acknowledged, then take the ticket
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        u32 t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag_lds = (t == total_blocks - 1);
+    }
+    __syncthreads();
+    bool last = *flag_lds != 0;
+    // one cache invalidation, in the last workgroup only; its loads of the partials are agent-scope as well
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return last;
+}
+
+// used when a round has no evaluation launch (a sum with constant terms only)
+__global__ void __launch_bounds__(BLOCK) finalize_kernel(FinArgs fa)
+{
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * MAX_PTS];
+    __shared__ u64 res[2 * MAX_PTS];
+    finalize_block<MAX_PTS>(fa, lds, res);
+}
+
+// ---------------------------------------------------------------------------
 // general term evaluation: one grid row (blockIdx.y) per term
 // ---------------------------------------------------------------------------
 struct FactorDesc {
@@ -185,7 +362,7 @@ struct TermDesc {
 
 // partial sums: out[(term * gridDim.x + block) * 2 * MAX_PTS + 2 * t + limb]
 template <int NF>
-__device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, u64 *__restrict__ partial, u64 *lds)
+__device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, u64 *__restrict__ partial, u32 *lds)
 {
     constexpr int NP = NF + 1;
     E2 acc[NP];
@@ -228,16 +405,18 @@ __device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, 
         u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            o[2 * t] = acc[t].c0;
-            o[2 * t + 1] = acc[t].c1;
+            st_agent(o + 2 * t, acc[t].c0);
+            st_agent(o + 2 * t + 1, acc[t].c1);
         }
     }
 }
 
 __global__ void __launch_bounds__(BLOCK)
-eval_terms_kernel(const TermDesc *__restrict__ terms, u64 n_pairs, u64 *__restrict__ partial)
+eval_terms_kernel(const TermDesc *__restrict__ terms, u64 n_pairs, u64 *__restrict__ partial, FinArgs fa)
 {
-    __shared__ u64 lds[(BLOCK / WAVE) * 2 * MAX_PTS];
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * MAX_PTS];
+    __shared__ u64 res[2 * MAX_PTS];
+    __shared__ int last_flag;
     const TermDesc &td = terms[blockIdx.y];
     switch (td.n_factors) {
     case 1: eval_term_body<1>(td, n_pairs, partial, lds); break;
@@ -248,39 +427,140 @@ eval_terms_kernel(const TermDesc *__restrict__ terms, u64 n_pairs, u64 *__restri
     case 6: eval_term_body<6>(td, n_pairs, partial, lds); break;
     default: break;
     }
+    if (take_ticket(fa.counter, fa.total_blocks, &last_flag)) finalize_block<MAX_PTS>(fa, lds, res);
 }
 
 // ---------------------------------------------------------------------------
-// fused product kernels: one term, NF full-size tables, the first NB of them
-// base-field in the source.  FOLD = false: first round, evaluate the source
-// pairs.  FOLD = true: read source quads, fold with r, write the folded pair,
-// evaluate it.
+// fused product kernels: one term, NF full-size tables (the first NB of them
+// base-field in the source), optionally times an eq(rho, x) factor.
+//
+// FOLD = false: first round, the source pairs are evaluated as they are.
+// FOLD = true : source quads are folded with r, the folded pair is written and
+//               evaluated: every table is read once and written once per round.
+//
+// The eq factor is never folded or streamed as a table of this round's size.
+// After the variables below v are bound, eq(rho, .) restricted to the remaining
+// cube is  S * eq1(rho_v, x_v) * R(x')  with a scalar S, the one-variable factor
+// eq1(a, b) = a b + (1 - a)(1 - b), and R = eq(rho_{v+1..}, .) a table of half this
+// round's size, prepared when the eq table was built.  The kernel sums
+// q(t) = sum_{x'} R(x') prod_f table_f(t, x') at t = 0..NF; the round message
+// p(t) = coeff * S * eq1(rho_v, t) * q(t) at t = 0..NF+1 is finished by the last
+// workgroup (q has degree NF, so q(NF+1) follows from the NF+1 sums).
+//
+// From round 2 on the caller knows the claim p(0) + p(1); then t = 1 is skipped
+// in the loop and q(1) is solved from the claim.
 // ---------------------------------------------------------------------------
 struct ProdArgs {
     const u64 *s0[3];
     const u64 *s1[3];
     u64 *d0[3];
     u64 *d1[3];
+    const u64 *q0;  // R of this round, n_pairs entries (eq factor only)
+    const u64 *q1;
     u64 n_pairs;  // pairs evaluated this round
     u64 r0, r1;   // fold challenge
+    u32 skip1;    // 1: do not evaluate t = 1
 };
 
-template <int NF, int NB, bool FOLD>
-__global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial)
+// What the last workgroup needs to turn the sums q(t) into the round message.
+struct FastFin {
+    const u64 *partial;
+    u32 n_blocks;
+    u32 degree;       // of the message: NF, or NF + 1 with an eq factor
+    u32 has_eq;
+    u32 skip1;
+    u64 scale[2 * MAX_PTS];  // scale(t) for t = 0..degree, extension elements
+    u64 claim0, claim1;      // p(0) + p(1), used when skip1
+    u64 inv_s1_0, inv_s1_1;  // 1 / scale(1), used when skip1
+    u64 ext[MAX_PTS];        // Lagrange weights of q(NF + 1) over the nodes 0..NF (eq factor only)
+    u64 const0, const1;      // constant terms summed over the remaining hypercube
+    u64 *out_dev;
+    u64 *out_host;
+    u64 seq;
+    u32 *counter;
+};
+
+template <int NF>
+__device__ __forceinline__ void fast_finalize(const FastFin &ff, u32 *lds, u64 *res)
 {
     constexpr int NP = NF + 1;
-    __shared__ u64 lds[(BLOCK / WAVE) * 2 * NP];
+    E2 q[NP + 1];
+#pragma unroll
+    for (int t = 0; t <= NP; t++) q[t] = gl::e2_zero();
+    for (u32 b = threadIdx.x; b < ff.n_blocks; b += BLOCK) {
+        const u64 *p = ff.partial + (u64)b * 2 * MAX_PTS;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            q[t].c0 = gl::add(q[t].c0, ld_agent(p + 2 * t));
+            q[t].c1 = gl::add(q[t].c1, ld_agent(p + 2 * t + 1));
+        }
+    }
+    {
+        E2 qq[NP];
+#pragma unroll
+        for (int t = 0; t < NP; t++) qq[t] = q[t];
+        block_reduce<NP>(qq, lds);
+#pragma unroll
+        for (int t = 0; t < NP; t++) q[t] = qq[t];
+    }
+    if (threadIdx.x == 0) {
+        if (ff.skip1) {
+            // scale(0) q(0) + scale(1) q(1) = claim
+            E2 s0 = gl::e2(ff.scale[0], ff.scale[1]);
+            E2 rest = gl::sub(gl::e2(ff.claim0, ff.claim1), gl::mul(s0, q[0]));
+            q[1] = gl::mul(rest, gl::e2(ff.inv_s1_0, ff.inv_s1_1));
+        }
+        if (ff.has_eq) {
+            E2 e = gl::e2_zero();
+#pragma unroll
+            for (int i = 0; i < NP; i++) e = gl::add(e, gl::mul_base(q[i], ff.ext[i]));
+            q[NP] = e;
+        }
+#pragma unroll
+        for (int t = 0; t <= NP; t++) {
+            if ((u32)t <= ff.degree) {
+                E2 v = gl::mul(q[t], gl::e2(ff.scale[2 * t], ff.scale[2 * t + 1]));
+                res[2 * t] = gl::add(v.c0, ff.const0);
+                res[2 * t + 1] = gl::add(v.c1, ff.const1);
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x <= ff.degree) {
+        u32 t = threadIdx.x;
+        u64 c0 = res[2 * t], c1 = res[2 * t + 1];
+        ff.out_dev[2 * t] = c0;
+        ff.out_dev[2 * t + 1] = c1;
+        __hip_atomic_store(ff.out_host + 2 * t, c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(ff.out_host + 2 * t + 1, c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __builtin_amdgcn_s_waitcnt(0);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        *ff.counter = 0;
+        __hip_atomic_store(ff.out_host + HOST_SEQ_SLOT, ff.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+template <int NF, int NB, bool FOLD, bool EQ>
+__global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial, FastFin ff)
+{
+    constexpr int NP = NF + 1;
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
+    __shared__ u64 res[2 * MAX_PTS];
+    __shared__ int last_flag;
     const E2 r = gl::e2(a.r0, a.r1);
+    const bool skip1 = a.skip1 != 0;
     E2 acc[NP];
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
 
     for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.n_pairs; i += (u64)gridDim.x * BLOCK) {
         E2 lo[NF], hi[NF];
-        bool is_base[NF];
+        // base-field arithmetic applies only while the sources are read unfolded
+        constexpr int NBE = FOLD ? 0 : NB;
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            is_base[f] = (f < NB) && !FOLD;
             if (FOLD) {
                 if (f < NB) {
                     U64x2 p = ld2(a.s0[f] + 4 * i), q = ld2(a.s0[f] + 4 * i + 2);
@@ -306,35 +586,48 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 }
             }
         }
+        E2 rest = gl::e2_one();
+        if (EQ) rest = gl::e2(a.q0[i], a.q1[i]);
         E2 dl[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) dl[f] = gl::sub(hi[f], lo[f]);
+        // cur holds the factors at t: lo at 0, hi at 1, then hi + (t - 1) dl
+        E2 cur[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++) cur[f] = lo[f];
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            // base-field factors first (plain products), then the extension ones
-            E2 prod;
-            if (!FOLD && NB > 0) {
-                u64 b = lo[0].c0;
+            if (!(t == 1 && skip1)) {
+                E2 prod;
+                if (NBE > 0) {
+                    u64 b = cur[0].c0;
 #pragma unroll
-                for (int f = 1; f < NB; f++) b = gl::mul(b, lo[f].c0);
-                if (NB == NF) {
-                    prod = gl::e2(b, 0);
+                    for (int f = 1; f < NBE; f++) b = gl::mul(b, cur[f].c0);
+                    if (NBE == NF) {
+                        prod = EQ ? gl::mul_base(rest, b) : gl::e2(b, 0);
+                    } else {
+                        prod = gl::mul_base(cur[NBE], b);
+#pragma unroll
+                        for (int f = NBE + 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
+                        if (EQ) prod = gl::mul(prod, rest);
+                    }
                 } else {
-                    prod = gl::mul_base(lo[NB], b);
+                    prod = cur[0];
 #pragma unroll
-                    for (int f = NB + 1; f < NF; f++) prod = gl::mul(prod, lo[f]);
+                    for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
+                    if (EQ) prod = gl::mul(prod, rest);
                 }
-            } else {
-                prod = lo[0];
-#pragma unroll
-                for (int f = 1; f < NF; f++) prod = gl::mul(prod, lo[f]);
+                acc[t] = gl::add(acc[t], prod);
             }
-            acc[t] = gl::add(acc[t], prod);
             if (t + 1 < NP) {
 #pragma unroll
                 for (int f = 0; f < NF; f++) {
-                    lo[f].c0 = gl::add(lo[f].c0, dl[f].c0);
-                    if (!is_base[f]) lo[f].c1 = gl::add(lo[f].c1, dl[f].c1);
+                    if (t == 0) {
+                        cur[f] = hi[f];
+                    } else {
+                        cur[f].c0 = gl::add(cur[f].c0, dl[f].c0);
+                        if (f >= NBE) cur[f].c1 = gl::add(cur[f].c1, dl[f].c1);
+                    }
                 }
             }
         }
@@ -344,81 +637,11 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         u64 *o = partial + (u64)blockIdx.x * 2 * MAX_PTS;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            o[2 * t] = acc[t].c0;
-            o[2 * t + 1] = acc[t].c1;
+            st_agent(o + 2 * t, acc[t].c0);
+            st_agent(o + 2 * t + 1, acc[t].c1);
         }
     }
-}
-
-// ---------------------------------------------------------------------------
-// finalize: sum the block partials of every term, scale by the term's
-// coefficient, extend a degree-k term to the d+1 points of the round message
-// (Lagrange weights over the nodes 0..k), add the constant terms.  One block.
-// ---------------------------------------------------------------------------
-struct FinTerm {
-    u64 coeff0, coeff1;
-    u32 n_factors;
-    u32 pad;
-};
-
-__global__ void __launch_bounds__(BLOCK)
-finalize_kernel(const u64 *__restrict__ partial, u32 blocks_per_term, const FinTerm *__restrict__ terms, u32 n_terms,
-                u32 degree, const u64 *__restrict__ lagrange /* [k][t][i], 9*9*9 */, u64 const0, u64 const1,
-                u64 *__restrict__ out_dev, u64 *__restrict__ out_host)
-{
-    __shared__ u64 lds[(BLOCK / WAVE) * 2 * MAX_PTS];
-    __shared__ u64 res[2 * MAX_PTS];
-    if (threadIdx.x < 2 * MAX_PTS) res[threadIdx.x] = 0;
-    __syncthreads();
-    for (u32 ti = 0; ti < n_terms; ti++) {
-        const u32 k = terms[ti].n_factors;
-        E2 acc[MAX_PTS];
-#pragma unroll
-        for (int t = 0; t < MAX_PTS; t++) acc[t] = gl::e2_zero();
-        for (u32 b = threadIdx.x; b < blocks_per_term; b += BLOCK) {
-            const u64 *p = partial + ((u64)ti * blocks_per_term + b) * 2 * MAX_PTS;
-#pragma unroll
-            for (int t = 0; t < MAX_PTS; t++) {
-                if ((u32)t <= k) {
-                    acc[t].c0 = gl::add(acc[t].c0, p[2 * t]);
-                    acc[t].c1 = gl::add(acc[t].c1, p[2 * t + 1]);
-                }
-            }
-        }
-        block_reduce<MAX_PTS>(acc, lds);
-        if (threadIdx.x == 0) {
-            const E2 coeff = gl::e2(terms[ti].coeff0, terms[ti].coeff1);
-            for (u32 t = 0; t <= degree; t++) {
-                E2 v;
-                if (t <= k) {
-                    v = acc[0];
-#pragma unroll
-                    for (int i = 1; i < MAX_PTS; i++)
-                        if ((u32)i == t) v = acc[i];
-                } else {
-                    v = gl::e2_zero();
-#pragma unroll
-                    for (int i = 0; i < MAX_PTS; i++) {
-                        if ((u32)i <= k) v = gl::add(v, gl::mul_base(acc[i], lagrange[(k * 9 + t) * 9 + i]));
-                    }
-                }
-                v = gl::mul(v, coeff);
-                res[2 * t] = gl::add(res[2 * t], v.c0);
-                res[2 * t + 1] = gl::add(res[2 * t + 1], v.c1);
-            }
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x <= degree) {
-        u32 t = threadIdx.x;
-        u64 c0 = gl::add(res[2 * t], const0), c1 = gl::add(res[2 * t + 1], const1);
-        out_dev[2 * t] = c0;
-        out_dev[2 * t + 1] = c1;
-        if (out_host) {
-            out_host[2 * t] = c0;
-            out_host[2 * t + 1] = c1;
-        }
-    }
+    if (take_ticket(ff.counter, gridDim.x, &last_flag)) fast_finalize<NF>(ff, lds, res);
 }
 
 // final evaluations: entry 0 of every table after the last fold
@@ -523,7 +746,7 @@ __global__ void __launch_bounds__(BLOCK) axis_dot_col_kernel(AxisArgs a)
 // one workgroup per output, lanes over k (for C < 64, e.g. a row dot product)
 __global__ void __launch_bounds__(BLOCK) axis_dot_row_kernel(AxisArgs a)
 {
-    __shared__ u64 lds[(BLOCK / WAVE) * 2];
+    __shared__ u32 lds[(BLOCK / WAVE) * 6];
     const u64 pre = blockIdx.x / a.C;
     const u64 i = blockIdx.x - pre * a.C;
     const u32 slice = blockIdx.y;
