@@ -107,6 +107,56 @@ GL_FN E2 mul(E2 a, E2 b)
 
 GL_FN E2 mul_base(E2 a, u64 b) { return e2(mul(a.c0, b), mul(a.c1, b)); }
 
+// ---------------------------------------------------------------------------
+// Products with one reduction per output limb.  The second operand carries
+// w = 7 * c1 (mod p), computed once and reused, so that
+//   (a0 + a1 X)(b0 + b1 X) + (c0 + c1 X) = (a0 b0 + a1 w + c0) + (a0 b1 + a1 b0 + c1) X
+// is two sums of two 128-bit products plus a 64-bit term, each reduced once.
+// ---------------------------------------------------------------------------
+typedef unsigned __int128 u128;
+
+struct E2P {
+    u64 c0, c1, w;
+};
+
+GL_FN E2P prep(E2 b)
+{
+    E2P r;
+    r.c0 = b.c0;
+    r.c1 = b.c1;
+    r.w = mul_small(b.c1, (u32)W);
+    return r;
+}
+
+// (x + y + z) mod p for 128-bit x, y and 64-bit z: a 130-bit sum, reduced once
+GL_FN u64 reduce_sum(u128 x, u128 y, u64 z)
+{
+    u128 s = x + y;
+    u64 carry = s < x;  // bit 128
+    u128 t = s + z;
+    carry += t < s;
+    u64 lo = (u64)t, hi = (u64)(t >> 64);
+    // value = lo + hl 2^64 + hh 2^96 + carry 2^128, with 2^64 = 2^32 - 1, 2^96 = -1, 2^128 = -2^32
+    u64 hl = (u32)hi;
+    u64 sub = (hi >> 32) + (carry << 32) + hl;  // subtracted: hh + carry 2^32 + hl (from hl (2^32 - 1))
+    u64 a = lo + (hl << 32);
+    u64 c1 = a < lo;  // wrapped past 2^64: add 2^32 - 1
+    u64 r = a - sub;
+    u64 b1 = a < sub;  // wrapped below 0: subtract 2^32 - 1
+    r += c1 * EPS;     // cannot wrap: a wrapped sum is below 2^64 - 2^32
+    r -= b1 * EPS;     // cannot wrap: a wrapped difference is above 2^64 - 2^36
+    return r >= P ? r - P : r;
+}
+
+GL_FN E2 fma(E2 a, E2P b, E2 c)
+{
+    u64 r0 = reduce_sum((u128)a.c0 * b.c0, (u128)a.c1 * b.w, c.c0);
+    u64 r1 = reduce_sum((u128)a.c0 * b.c1, (u128)a.c1 * b.c0, c.c1);
+    return e2(r0, r1);
+}
+
+GL_FN E2 mulp(E2 a, E2P b) { return fma(a, b, e2_zero()); }
+
 GL_FN bool eq(E2 a, E2 b) { return a.c0 == b.c0 && a.c1 == b.c1; }
 
 }  // namespace gl

@@ -187,6 +187,8 @@ struct FoldDesc {
 };
 
 __device__ __forceinline__ E2 fold1(E2 lo, E2 hi, E2 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
+// lo + (hi - lo) * r with r prepared: one reduction per output limb
+__device__ __forceinline__ E2 fold1p(E2 lo, E2 hi, gl::E2P r) { return gl::fma(gl::sub(hi, lo), r, lo); }
 __device__ __forceinline__ E2 fold1_base(u64 lo, u64 hi, E2 r)
 {
     E2 d = gl::mul_base(r, gl::sub(hi, lo));
@@ -480,13 +482,12 @@ struct FastFin {
     u32 *counter;
 };
 
-template <int NF>
-__device__ __forceinline__ void fast_finalize(const FastFin &ff, u32 *lds, u64 *res)
+// sums of the workgroups' partials, valid in thread 0
+template <int NP>
+__device__ __forceinline__ void gather_partials(const FastFin &ff, u32 *lds, E2 (&q)[NP])
 {
-    constexpr int NP = NF + 1;
-    E2 q[NP + 1];
 #pragma unroll
-    for (int t = 0; t <= NP; t++) q[t] = gl::e2_zero();
+    for (int t = 0; t < NP; t++) q[t] = gl::e2_zero();
     for (u32 b = threadIdx.x; b < ff.n_blocks; b += BLOCK) {
         const u64 *p = ff.partial + (u64)b * 2 * MAX_PTS;
 #pragma unroll
@@ -495,14 +496,18 @@ __device__ __forceinline__ void fast_finalize(const FastFin &ff, u32 *lds, u64 *
             q[t].c1 = gl::add(q[t].c1, ld_agent(p + 2 * t + 1));
         }
     }
-    {
-        E2 qq[NP];
+    block_reduce<NP>(q, lds);
+}
+
+// sums[t] = q(t) for t = 0..NF, valid in thread 0
+template <int NF>
+__device__ __forceinline__ void fast_finalize(const FastFin &ff, const E2 (&sums)[NF + 1], u64 *res)
+{
+    constexpr int NP = NF + 1;
+    E2 q[NP + 1];
 #pragma unroll
-        for (int t = 0; t < NP; t++) qq[t] = q[t];
-        block_reduce<NP>(qq, lds);
-#pragma unroll
-        for (int t = 0; t < NP; t++) q[t] = qq[t];
-    }
+    for (int t = 0; t < NP; t++) q[t] = sums[t];
+    q[NP] = gl::e2_zero();
     if (threadIdx.x == 0) {
         if (ff.skip1) {
             // scale(0) q(0) + scale(1) q(1) = claim
@@ -550,6 +555,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     __shared__ u64 res[2 * MAX_PTS];
     __shared__ int last_flag;
     const E2 r = gl::e2(a.r0, a.r1);
+    const gl::E2P rp = gl::prep(r);
     const bool skip1 = a.skip1 != 0;
     E2 acc[NP];
 #pragma unroll
@@ -569,8 +575,8 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 } else {
                     U64x2 p0 = ld2(a.s0[f] + 4 * i), q0 = ld2(a.s0[f] + 4 * i + 2);
                     U64x2 p1 = ld2(a.s1[f] + 4 * i), q1 = ld2(a.s1[f] + 4 * i + 2);
-                    lo[f] = fold1(gl::e2(p0.x, p1.x), gl::e2(p0.y, p1.y), r);
-                    hi[f] = fold1(gl::e2(q0.x, q1.x), gl::e2(q0.y, q1.y), r);
+                    lo[f] = fold1p(gl::e2(p0.x, p1.x), gl::e2(p0.y, p1.y), rp);
+                    hi[f] = fold1p(gl::e2(q0.x, q1.x), gl::e2(q0.y, q1.y), rp);
                 }
                 st2(a.d0[f] + 2 * i, lo[f].c0, hi[f].c0);
                 st2(a.d1[f] + 2 * i, lo[f].c1, hi[f].c1);
@@ -587,7 +593,11 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             }
         }
         E2 rest = gl::e2_one();
-        if (EQ) rest = gl::e2(a.q0[i], a.q1[i]);
+        gl::E2P restp = gl::prep(rest);
+        if (EQ) {
+            rest = gl::e2(a.q0[i], a.q1[i]);
+            restp = gl::prep(rest);
+        }
         E2 dl[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) dl[f] = gl::sub(hi[f], lo[f]);
@@ -599,6 +609,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         for (int t = 0; t < NP; t++) {
             if (!(t == 1 && skip1)) {
                 E2 prod;
+                bool continue_step = false;
                 if (NBE > 0) {
                     u64 b = cur[0].c0;
 #pragma unroll
@@ -615,9 +626,13 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                     prod = cur[0];
 #pragma unroll
                     for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
-                    if (EQ) prod = gl::mul(prod, rest);
+                    // the last product and the running sum share one reduction
+                    if (EQ) {
+                        acc[t] = gl::fma(prod, restp, acc[t]);
+                        continue_step = true;
+                    }
                 }
-                acc[t] = gl::add(acc[t], prod);
+                if (!continue_step) acc[t] = gl::add(acc[t], prod);
             }
             if (t + 1 < NP) {
 #pragma unroll
@@ -633,6 +648,11 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         }
     }
     block_reduce<NP>(acc, lds);
+    if (gridDim.x == 1) {
+        // a single workgroup: its sums are the round's sums, no partials and no ticket
+        fast_finalize<NF>(ff, acc, res);
+        return;
+    }
     if (threadIdx.x == 0) {
         u64 *o = partial + (u64)blockIdx.x * 2 * MAX_PTS;
 #pragma unroll
@@ -641,7 +661,11 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             st_agent(o + 2 * t + 1, acc[t].c1);
         }
     }
-    if (take_ticket(ff.counter, gridDim.x, &last_flag)) fast_finalize<NF>(ff, lds, res);
+    if (take_ticket(ff.counter, gridDim.x, &last_flag)) {
+        E2 q[NP];
+        gather_partials<NP>(ff, lds, q);
+        fast_finalize<NF>(ff, q, res);
+    }
 }
 
 // final evaluations: entry 0 of every table after the last fold
