@@ -21,7 +21,7 @@ P = 0xFFFFFFFF00000001
 MAX_FACTORS = 8
 AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
 KIND_BASE, KIND_EXT2, KIND_I64 = 0, 1, 2
-KERNELS = ["eval_first", "fold_eval", "eval_terms", "fold", "eq", "axis_dot", "logup", "finalize"]
+KERNELS = ["eval_first", "fold_eval", "eval_terms", "fold", "eq", "axis_dot", "logup", "finalize", "tail"]
 
 
 class DpsError(RuntimeError):

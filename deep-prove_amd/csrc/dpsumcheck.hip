@@ -24,7 +24,9 @@ using gl::u64;
 
 namespace {
 
-constexpr u32 MAX_BLOCKS = 2048;  // 8 workgroups per CU on 256 CUs
+// 3 workgroups per CU on 256 CUs: measured best for the streaming kernels (each workgroup pays a fixed
+// reduction + ticket epilogue, so more, thinner workgroups lose more than they gain in latency hiding)
+constexpr u32 MAX_BLOCKS = 768;
 
 // ---------------------------------------------------------------------------
 // context
@@ -58,6 +60,7 @@ struct dps_ctx {
     size_t pinned_words = 0;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
     u64 seq = 0;                // last sequence number handed to a launch
+    struct dps_sc *tail_owner = nullptr;  // session whose tail kernel is resident on the stream
     bool profiling = false;
     std::vector<ProfRec> recs;
     std::vector<hipEvent_t> ev_pool;
@@ -107,6 +110,10 @@ struct DeviceGuard {
 };
 
 size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// A resident tail kernel blocks the stream until its session finishes.  Any other
+// use of the context first makes that kernel exit (its session is then failed).
+void tail_abort(dps_ctx *ctx);
 
 int32_t pool_alloc(dps_ctx *ctx, size_t bytes, void **out)
 {
@@ -322,7 +329,7 @@ extern "C" const char *dps_kernel_name(int32_t k)
 {
     static const char *names[DPS_K_COUNT] = {"prod_kernel<first round>", "prod_kernel<fold+eval>", "eval_terms_kernel",
                                              "fold_kernel",              "eq_expand_kernel",       "axis_dot_kernel",
-                                             "logup_layer_kernel",       "finalize_kernel"};
+                                             "logup_layer_kernel",       "finalize_kernel",        "tail_kernel"};
     return (k >= 0 && k < DPS_K_COUNT) ? names[k] : "?";
 }
 
@@ -379,6 +386,7 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
 {
     if (!ctx) return DPS_OK;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     prof_collect(ctx);
     for (auto e : ctx->ev_pool) (void)hipEventDestroy(e);
@@ -395,6 +403,7 @@ extern "C" int32_t dps_ctx_sync(dps_ctx *ctx)
 {
     if (!ctx) return DPS_ERR_INVALID;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return DPS_OK;
 }
@@ -410,6 +419,7 @@ extern "C" int32_t dps_profile_reset(dps_ctx *ctx)
 {
     if (!ctx) return DPS_ERR_INVALID;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     prof_collect(ctx);
     for (auto &s : ctx->stats) s = ProfStat();
@@ -421,6 +431,7 @@ extern "C" int32_t dps_profile_read(dps_ctx *ctx, int32_t kernel, uint64_t *laun
 {
     if (!ctx || kernel < 0 || kernel >= DPS_K_COUNT) return DPS_ERR_INVALID;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     prof_collect(ctx);
     const ProfStat &s = ctx->stats[kernel];
@@ -440,6 +451,7 @@ extern "C" int32_t dps_mle_from_base(dps_ctx *ctx, const uint64_t *host, uint32_
 {
     if (!ctx || !host || !out || n_vars > 40) return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_base: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     u64 len = 1ull << n_vars;
     dps_mle *m = nullptr;
     CHK(new_table(ctx, DPS_BASE, len, &m));
@@ -457,6 +469,7 @@ extern "C" int32_t dps_mle_from_ext2(dps_ctx *ctx, const uint64_t *c0, const uin
 {
     if (!ctx || !c0 || !c1 || !out || n_vars > 40) return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_ext2: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     u64 len = 1ull << n_vars;
     dps_mle *m = nullptr;
     CHK(new_table(ctx, DPS_EXT2, len, &m));
@@ -475,6 +488,7 @@ extern "C" int32_t dps_tensor_from_i64(dps_ctx *ctx, const int64_t *host, uint64
 {
     if (!ctx || !out || (len && !host)) return fail(ctx, DPS_ERR_INVALID, "dps_tensor_from_i64: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     dps_mle *m = nullptr;
     CHK(new_table(ctx, DPS_I64, std::max<u64>(len, 1), &m));
     m->len = len;
@@ -495,6 +509,7 @@ extern "C" int32_t dps_mle_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t 
     if (!ctx || !out || n_vars > 40 || len > (1ull << n_vars) || (len && !host))
         return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_i64: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     dps_mle *raw = nullptr;
     CHK(dps_tensor_from_i64(ctx, host, len, &raw));
     u64 padded = 1ull << n_vars;
@@ -556,6 +571,7 @@ extern "C" int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *
     if (!mle || !c0) return DPS_ERR_INVALID;
     dps_ctx *ctx = mle->ctx;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     if (mle->len) HIPCHK(ctx, hipMemcpy(c0, mle->p0(), mle->len * 8, hipMemcpyDeviceToHost));
     if (c1) {
@@ -572,6 +588,7 @@ extern "C" int32_t dps_mle_free(dps_mle *mle)
 {
     if (!mle) return DPS_OK;
     DeviceGuard g(mle->ctx->device);
+    tail_abort(mle->ctx);
     // work that still reads the storage may be queued
     (void)hipStreamSynchronize(mle->ctx->stream);
     delete mle;
@@ -586,7 +603,7 @@ namespace {
 // uploads `words` 64-bit words through the pinned buffer region [slot, slot+words)
 int32_t stage_words(dps_ctx *ctx, const u64 *src, size_t words, size_t slot, const u64 **dev)
 {
-    if (slot + words > ctx->res_off) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
+    if (slot + words > ctx->res_off - 64) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
     // the buffer may still be read by queued kernels
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     memcpy(ctx->h_pinned + slot, src, words * 8);
@@ -677,6 +694,7 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     if (!ctx || !out || (m && !point) || m > 34) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: bad argument");
     if (!canonical(point, 2 * (size_t)m)) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: point not canonical");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     const u64 *d_point = nullptr;
     u64 dummy[2] = {0, 0};
     CHK(stage_words(ctx, m ? point : dummy, m ? 2 * (size_t)m : 2, 0, &d_point));
@@ -784,6 +802,7 @@ extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint
     if (!ctx || !mle || !out || (n && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: bad argument");
     if (!is_pow2(mle->len) || (1ull << n) != mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: point length does not match the table");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     dps_mle *eq = nullptr;
     CHK(dps_eq_build(ctx, point, n, &eq));
     AxisJob j;
@@ -812,6 +831,7 @@ extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint
     if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: bad argument");
     if (!is_pow2(mle->len) || (1ull << k) > mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: too many variables");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     dps_mle *eq = nullptr;
     CHK(dps_eq_build(ctx, point, k, &eq));
     u64 rest = mle->len >> k;
@@ -850,6 +870,7 @@ extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint6
         return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: needs a power-of-two field table and k <= log2(len)");
     if (!canonical(point, 2 * (size_t)k)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: point not canonical");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     if (k == 0) return dps_mle_view(mle, 0, log2u(mle->len), out);
     // ping-pong between two buffers; the last one written becomes the result
     u64 len = mle->len;
@@ -899,6 +920,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
     if (!ctx || !tensor || !padded_dims || !unpadded_dims || !kinds || !out || !n_out || n_dims == 0 || n_dims > dpk::AX_MAX_DIMS)
         return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     u64 padded_total = 1, contraction = 1, stacked = 1;
     for (u32 a = 0; a < n_dims; a++) {
         if (unpadded_dims[a] == 0 || unpadded_dims[a] > padded_dims[a]) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: dimension %u", a);
@@ -1079,6 +1101,10 @@ struct dps_sc {
     E2 eq_scalar;       // product of eq1(rho_i, r_{i+1}) over the bound variables
     E2 claim;           // p(0) + p(1) expected from the next message (valid from round 2)
     std::vector<E2> last_msg;
+    bool broken;        // its tail kernel was interrupted by another call on the context
+    u32 tail_j0;        // first round run by the resident tail kernel, 0 = none
+    bool tail_running;
+    u64 tail_seq0;
     void *scratch;      // one pool block holding every ping-pong buffer
     void *dev_block;    // descriptors, partials, per-round result
     // precomputed descriptors (device)
@@ -1099,6 +1125,26 @@ struct dps_sc {
 };
 
 namespace {
+
+u64 *mailbox(dps_ctx *ctx) { return ctx->h_pinned + ctx->res_off - 64; }
+
+void tail_abort(dps_ctx *ctx)
+{
+    dps_sc *owner = ctx->tail_owner;
+    if (!owner) return;
+    __atomic_store_n(mailbox(ctx) + dpk::MAIL_ABORT, (u64)1, __ATOMIC_RELEASE);
+    (void)hipStreamSynchronize(ctx->stream);
+    __atomic_store_n(mailbox(ctx) + dpk::MAIL_ABORT, (u64)0, __ATOMIC_RELEASE);
+    owner->tail_running = false;
+    owner->broken = true;
+    ctx->tail_owner = nullptr;
+}
+
+template <int NF, bool EQ>
+void launch_tail(dps_ctx *ctx, const dpk::TailArgs &a)
+{
+    dpk::tail_kernel<NF, EQ><<<1, dpk::BLOCK, 0, ctx->stream>>>(a);
+}
 
 template <int NF, int NB, bool EQ>
 void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial, const dpk::FastFin &ff)
@@ -1133,6 +1179,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     if (!ctx || !out || (n_mles && !mles) || (n_terms && !terms) || n_vars > 40)
         return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     std::unique_ptr<dps_sc> sc(new (std::nothrow) dps_sc());
     if (!sc) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
     sc->ctx = ctx;
@@ -1170,6 +1217,10 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
 
     // fast path test
     sc->fast = false;
+    sc->broken = false;
+    sc->tail_j0 = 0;
+    sc->tail_running = false;
+    sc->tail_seq0 = 0;
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
@@ -1203,6 +1254,9 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             sc->fast_coeff = gl::e2(t.coeff[0], t.coeff[1]);
         }
     }
+
+    // the last rounds run in one resident workgroup when every registered table belongs to the term
+    if (sc->fast && n_vars >= 11 && n_mles == sc->terms[0].n_factors) sc->tail_j0 = n_vars - 8;  // 2^8 = TAIL_PAIRS pairs
 
     // scratch: two ping-pong buffers per table, extension limbs
     size_t scratch_words = 0;
@@ -1440,7 +1494,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
     const u32 j = sc->round + 1;
     if ((j == 1) != (challenge == nullptr)) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: round %u %s a challenge", j, j == 1 ? "takes no" : "needs");
     if (challenge && !canonical(challenge, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_round: challenge not canonical");
+    if (sc->broken) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the session was interrupted by another call on its context");
     DeviceGuard g(ctx->device);
+    if (ctx->tail_owner != sc) tail_abort(ctx);
     const u32 live = sc->n_vars - j + 1;
     const u64 n_pairs = 1ull << (live - 1);
     u32 blocks = blocks_for_pairs(n_pairs);
@@ -1530,6 +1586,58 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         ff.out_host = fa.out_host;
         ff.seq = fa.seq;
         ff.counter = sc->d_counter;
+        if (sc->tail_j0 && j >= sc->tail_j0) {
+            // mail for the resident kernel: challenge, scales, claim; then the sequence number it waits for
+            u64 *mb = mailbox(ctx);
+            mb[dpk::MAIL_R] = a.r0;
+            mb[dpk::MAIL_R + 1] = a.r1;
+            for (u32 k = 0; k < 2 * dpk::MAX_PTS; k++) mb[dpk::MAIL_SCALE + k] = ff.scale[k];
+            mb[dpk::MAIL_CLAIM] = ff.claim0;
+            mb[dpk::MAIL_CLAIM + 1] = ff.claim1;
+            mb[dpk::MAIL_INV] = ff.inv_s1_0;
+            mb[dpk::MAIL_INV + 1] = ff.inv_s1_1;
+            mb[dpk::MAIL_CONST] = cst.c0;
+            mb[dpk::MAIL_CONST + 1] = cst.c1;
+            mb[dpk::MAIL_SKIP1] = a.skip1;
+            mb[dpk::MAIL_ABORT] = 0;
+            __atomic_store_n(mb + dpk::MAIL_SEQ, fa.seq, __ATOMIC_RELEASE);
+            if (j == sc->tail_j0) {
+                dpk::TailArgs ta;
+                memset(&ta, 0, sizeof ta);
+                for (u32 f = 0; f < nf; f++) {
+                    ta.s0[f] = a.s0[f];
+                    ta.s1[f] = a.s1[f];
+                }
+                ta.eq0 = sc->eq_c0;
+                ta.eq1 = sc->eq_c1;
+                ta.n_vars = sc->n_vars;
+                ta.j0 = j;
+                ta.degree = sc->degree;
+                ta.has_eq = has_eq ? 1 : 0;
+                for (u32 k = 0; k < dpk::MAX_PTS; k++) ta.ext[k] = ff.ext[k];
+                ta.mail = ctx->d_pinned + (ctx->res_off - 64);
+                ta.out_host = fa.out_host;
+                ta.out_dev = sc->d_result;
+                ta.seq0 = fa.seq;
+                sc->tail_seq0 = fa.seq;
+                ta.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
+                ProfScope ps(ctx, DPS_K_TAIL, 0.0);
+                if (has_eq && nf == 1) launch_tail<1, true>(ctx, ta);
+                else if (has_eq && nf == 2) launch_tail<2, true>(ctx, ta);
+                else if (!has_eq && nf == 2) launch_tail<2, false>(ctx, ta);
+                else if (!has_eq && nf == 3) launch_tail<3, false>(ctx, ta);
+                else return fail(ctx, DPS_ERR_UNSUPPORTED, "no tail kernel for %u tables, eq %d", nf, (int)has_eq);
+                HIPCHK(ctx, hipGetLastError());
+                sc->tail_running = true;
+                ctx->tail_owner = sc;
+            }
+            CHK(wait_result(ctx, fa.seq));
+            memcpy(evals_out, ctx->h_pinned + ctx->res_off, 2 * (sc->degree + 1) * 8);
+            sc->last_msg.resize(sc->degree + 1);
+            for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
+            sc->round = j;
+            return DPS_OK;
+        }
         double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
         for (u32 f = 0; f < nf; f++) {
             double eb = a.s1[f] ? 16.0 : 8.0;
@@ -1567,10 +1675,39 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
     if (sc->finished || sc->round != sc->n_vars) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: %u of %u rounds done", sc->round, sc->n_vars);
     if (sc->n_vars >= 1 && !challenge) return fail(ctx, DPS_ERR_INVALID, "dps_sc_finish: the last challenge is missing");
     if (challenge && !canonical(challenge, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_finish: challenge not canonical");
+    if (sc->broken) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: the session was interrupted by another call on its context");
     DeviceGuard g(ctx->device);
+    if (ctx->tail_owner != sc) tail_abort(ctx);
+    if (sc->tail_running) {
+        // the resident kernel folds with the last challenge and publishes the final evaluations
+        u64 *mb = mailbox(ctx);
+        const u64 seq = ++ctx->seq;
+        mb[dpk::MAIL_R] = challenge[0];
+        mb[dpk::MAIL_R + 1] = challenge[1];
+        __atomic_store_n(mb + dpk::MAIL_SEQ, seq, __ATOMIC_RELEASE);
+        int32_t rc = wait_result(ctx, seq);
+        // the kernel exits right after publishing
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        sc->tail_running = false;
+        ctx->tail_owner = nullptr;
+        if (rc != DPS_OK) return rc;
+        if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "tail kernel: %s", hipGetErrorString(e));
+        const u64 *fin = ctx->h_pinned + ctx->res_off + dpk::HOST_FINALS_SLOT;
+        for (u32 f = 0; f < sc->fast_nf; f++) {
+            final_evals_out[2 * sc->fast_order[f]] = fin[2 * f];
+            final_evals_out[2 * sc->fast_order[f] + 1] = fin[2 * f + 1];
+        }
+        if (sc->fast_eq >= 0) {
+            E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], gl::e2(challenge[0], challenge[1])));
+            final_evals_out[2 * sc->fast_eq] = v.c0;
+            final_evals_out[2 * sc->fast_eq + 1] = v.c1;
+        }
+        sc->finished = true;
+        return DPS_OK;
+    }
     if (sc->n_vars >= 1) CHK(launch_folds(sc, sc->n_vars + 1, sc->fast, challenge));
     if (sc->n_mles) {
-        if (2 * (size_t)sc->n_mles > ctx->pinned_words) return fail(ctx, DPS_ERR_UNSUPPORTED, "too many tables in one session");
+        if (2 * (size_t)sc->n_mles > ctx->res_off - 64) return fail(ctx, DPS_ERR_UNSUPPORTED, "too many tables in one session");
         dpk::gather_kernel<<<(sc->n_mles + 63) / 64, 64, 0, ctx->stream>>>(sc->d_gather, sc->n_mles, ctx->d_pinned);
         HIPCHK(ctx, hipGetLastError());
     }
@@ -1591,6 +1728,7 @@ extern "C" int32_t dps_sc_free(dps_sc *sc)
     if (!sc) return DPS_OK;
     dps_ctx *ctx = sc->ctx;
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     pool_free(ctx, sc->scratch);
     pool_free(ctx, sc->dev_block);
@@ -1636,6 +1774,7 @@ extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uin
     if (n_cols > dpk::LOGUP_MAX_COLS) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_logup_build: more than %d columns", dpk::LOGUP_MAX_COLS);
     if (!canonical(c, 2) || !canonical(beta, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: challenge not canonical");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     u64 len = cols[0] ? cols[0]->len : 0;
     if (!is_pow2(len) || len < 2) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: column length must be a power of two >= 2");
     for (u32 k = 0; k < n_cols; k++)
@@ -1725,6 +1864,7 @@ extern "C" int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8])
     dps_ctx *ctx = lg->ctx;
     if (lg->n_layers < 2) return fail(ctx, DPS_ERR_STATE, "dps_logup_outputs: the instance has no layer above its input");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     u64 off = lg->layer_off[lg->n_layers - 1];
     u64 a[4], b[4];
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
@@ -1741,6 +1881,7 @@ extern "C" int32_t dps_logup_free(dps_logup *lg)
 {
     if (!lg) return DPS_OK;
     DeviceGuard g(lg->ctx->device);
+    tail_abort(lg->ctx);
     (void)hipStreamSynchronize(lg->ctx->stream);
     delete lg;
     return DPS_OK;
@@ -1754,6 +1895,7 @@ extern "C" int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *
 {
     if (!ctx || !a || !b || !out || n == 0) return fail(ctx, DPS_ERR_INVALID, "dps_debug_field_op: bad argument");
     DeviceGuard g(ctx->device);
+    tail_abort(ctx);
     void *p = nullptr;
     CHK(pool_alloc(ctx, 6 * n * 8, &p));
     u64 *d = (u64 *)p;

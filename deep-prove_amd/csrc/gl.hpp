@@ -47,16 +47,14 @@ GL_FN u64 reduce128(u64 lo, u64 hi)
     return r >= P ? r - P : r;
 }
 
-GL_FN u64 mulhi64(u64 a, u64 b)
-{
-#if defined(__HIP_DEVICE_COMPILE__)
-    return __umul64hi(a, b);
-#else
-    return (u64)(((unsigned __int128)a * b) >> 64);
-#endif
-}
+GL_FN u64 mulhi64(u64 a, u64 b) { return (u64)(((unsigned __int128)a * b) >> 64); }
 
-GL_FN u64 mul(u64 a, u64 b) { return reduce128(a * b, mulhi64(a, b)); }
+// the 128-bit product compiles to four v_mad_u64_u32 on the device
+GL_FN u64 mul(u64 a, u64 b)
+{
+    unsigned __int128 p = (unsigned __int128)a * b;
+    return reduce128((u64)p, (u64)(p >> 64));
+}
 
 // a * small constant (c < 2^32)
 GL_FN u64 mul_small(u64 a, u32 c)

@@ -542,7 +542,7 @@ __device__ __forceinline__ void fast_finalize(const FastFin &ff, const E2 (&sums
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        *ff.counter = 0;
+        if (ff.counter) *ff.counter = 0;
         __hip_atomic_store(ff.out_host + HOST_SEQ_SLOT, ff.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
@@ -561,7 +561,41 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
 
-    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.n_pairs; i += (u64)gridDim.x * BLOCK) {
+    // Raw operands of one loop step.  The first-round kernel has little arithmetic
+    // per byte, so it loads the next step's operands before working on the
+    // current ones; the fold kernels are arithmetic-bound and keep one set.
+    struct Raw {
+        U64x2 a0[NF], b0[NF], a1[NF], b1[NF];
+        u64 q0, q1;
+    };
+    auto load_raw = [&](u64 i, Raw &w) {
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            if (FOLD) {
+                w.a0[f] = ld2(a.s0[f] + 4 * i);
+                w.b0[f] = ld2(a.s0[f] + 4 * i + 2);
+                if (f >= NB) {
+                    w.a1[f] = ld2(a.s1[f] + 4 * i);
+                    w.b1[f] = ld2(a.s1[f] + 4 * i + 2);
+                }
+            } else {
+                w.a0[f] = ld2(a.s0[f] + 2 * i);
+                if (f >= NB) w.a1[f] = ld2(a.s1[f] + 2 * i);
+            }
+        }
+        if (EQ) {
+            w.q0 = a.q0[i];
+            w.q1 = a.q1[i];
+        }
+    };
+    const u64 stride = (u64)gridDim.x * BLOCK;
+    u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    Raw w;
+    if (i < a.n_pairs) load_raw(i, w);
+    for (; i < a.n_pairs; i += stride) {
+        Raw nxt;
+        const bool more = i + stride < a.n_pairs;
+        if (!FOLD && more) load_raw(i + stride, nxt);
         E2 lo[NF], hi[NF];
         // base-field arithmetic applies only while the sources are read unfolded
         constexpr int NBE = FOLD ? 0 : NB;
@@ -569,33 +603,28 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         for (int f = 0; f < NF; f++) {
             if (FOLD) {
                 if (f < NB) {
-                    U64x2 p = ld2(a.s0[f] + 4 * i), q = ld2(a.s0[f] + 4 * i + 2);
-                    lo[f] = fold1_base(p.x, p.y, r);
-                    hi[f] = fold1_base(q.x, q.y, r);
+                    lo[f] = fold1_base(w.a0[f].x, w.a0[f].y, r);
+                    hi[f] = fold1_base(w.b0[f].x, w.b0[f].y, r);
                 } else {
-                    U64x2 p0 = ld2(a.s0[f] + 4 * i), q0 = ld2(a.s0[f] + 4 * i + 2);
-                    U64x2 p1 = ld2(a.s1[f] + 4 * i), q1 = ld2(a.s1[f] + 4 * i + 2);
-                    lo[f] = fold1p(gl::e2(p0.x, p1.x), gl::e2(p0.y, p1.y), rp);
-                    hi[f] = fold1p(gl::e2(q0.x, q1.x), gl::e2(q0.y, q1.y), rp);
+                    lo[f] = fold1p(gl::e2(w.a0[f].x, w.a1[f].x), gl::e2(w.a0[f].y, w.a1[f].y), rp);
+                    hi[f] = fold1p(gl::e2(w.b0[f].x, w.b1[f].x), gl::e2(w.b0[f].y, w.b1[f].y), rp);
                 }
                 st2(a.d0[f] + 2 * i, lo[f].c0, hi[f].c0);
                 st2(a.d1[f] + 2 * i, lo[f].c1, hi[f].c1);
             } else {
-                U64x2 p = ld2(a.s0[f] + 2 * i);
                 if (f < NB) {
-                    lo[f] = gl::e2(p.x, 0);
-                    hi[f] = gl::e2(p.y, 0);
+                    lo[f] = gl::e2(w.a0[f].x, 0);
+                    hi[f] = gl::e2(w.a0[f].y, 0);
                 } else {
-                    U64x2 q = ld2(a.s1[f] + 2 * i);
-                    lo[f] = gl::e2(p.x, q.x);
-                    hi[f] = gl::e2(p.y, q.y);
+                    lo[f] = gl::e2(w.a0[f].x, w.a1[f].x);
+                    hi[f] = gl::e2(w.a0[f].y, w.a1[f].y);
                 }
             }
         }
         E2 rest = gl::e2_one();
         gl::E2P restp = gl::prep(rest);
         if (EQ) {
-            rest = gl::e2(a.q0[i], a.q1[i]);
+            rest = gl::e2(w.q0, w.q1);
             restp = gl::prep(rest);
         }
         E2 dl[NF];
@@ -646,6 +675,12 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 }
             }
         }
+        if (more) {
+            if (FOLD)
+                load_raw(i + stride, w);
+            else
+                w = nxt;
+        }
     }
     block_reduce<NP>(acc, lds);
     if (gridDim.x == 1) {
@@ -666,6 +701,184 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         gather_partials<NP>(ff, lds, q);
         fast_finalize<NF>(ff, q, res);
     }
+}
+
+// ---------------------------------------------------------------------------
+// tail kernel: the last rounds of a product sumcheck in one launch
+//
+// Once a round has at most TAIL_PAIRS pairs a launch per round is pure latency
+// (dispatch, a single wavefront's instruction stream, the result hand-off).  One
+// workgroup then stays resident for all remaining rounds: the tables live in LDS,
+// each round's message goes to host-visible memory as before, and the workgroup
+// waits for the next challenge in a mailbox the host writes (fine-grained pinned
+// memory, system-scope loads).  The wait is bounded: without mail the kernel
+// gives up after `spin_limit` polls and exits.
+// ---------------------------------------------------------------------------
+constexpr int TAIL_PAIRS = 256;
+constexpr int MAIL_SEQ = 0, MAIL_R = 1, MAIL_SCALE = 3, MAIL_CLAIM = 3 + 2 * MAX_PTS, MAIL_INV = MAIL_CLAIM + 2,
+              MAIL_CONST = MAIL_INV + 2, MAIL_SKIP1 = MAIL_CONST + 2, MAIL_ABORT = MAIL_SKIP1 + 1, MAIL_WORDS = MAIL_ABORT + 1;
+constexpr int HOST_FINALS_SLOT = HOST_SEQ_SLOT + 8;
+
+struct TailArgs {
+    const u64 *s0[3];
+    const u64 *s1[3];  // extension tables of the first tail round, 4 * n_pairs0 entries each
+    const u64 *eq0;    // eq storage (level 0 at entry 0), eq factor only
+    const u64 *eq1;
+    u32 n_vars, j0;    // the sum's variables, first round handled here (1-based)
+    u32 degree, has_eq;
+    u64 ext[MAX_PTS];  // Lagrange weights of q(NF + 1) (eq factor only)
+    const u64 *mail;   // host mailbox, MAIL_WORDS words
+    u64 *out_host;     // message limbs, HOST_SEQ_SLOT, HOST_FINALS_SLOT
+    u64 *out_dev;
+    u64 seq0;          // sequence number of round j0; round j uses seq0 + (j - j0), the final evaluations seq0 + (n_vars - j0 + 1)
+    u32 spin_limit;
+};
+
+__device__ __forceinline__ u64 ld_sys(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
+__device__ __forceinline__ void st_sys(u64 *p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
+
+// Waits for mail number `want`; copies it to `box` (LDS).  Returns false on abort or timeout.
+__device__ __forceinline__ bool tail_wait_mail(const TailArgs &a, u64 want, u64 *box, int *ok_lds)
+{
+    if (threadIdx.x == 0) {
+        int ok = 0;
+        for (u32 spins = 0; spins < a.spin_limit; spins++) {
+            u64 s = __hip_atomic_load(a.mail + MAIL_SEQ, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (s == want) {
+                ok = 1;
+                break;
+            }
+            if (ld_sys(a.mail + MAIL_ABORT) != 0) break;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        *ok_lds = ok;
+    }
+    __syncthreads();
+    if (!*ok_lds) return false;
+    if (threadIdx.x < MAIL_WORDS) box[threadIdx.x] = ld_sys(a.mail + threadIdx.x);
+    __syncthreads();
+    return true;
+}
+
+template <int NF, bool EQ>
+__global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
+{
+    constexpr int NP = NF + 1;
+    // ping: tables after the first tail round (2 * TAIL_PAIRS entries), pong: half of that
+    __shared__ u64 ping[NF][2][2 * TAIL_PAIRS];
+    __shared__ u64 pong[NF][2][TAIL_PAIRS];
+    __shared__ u64 box[MAIL_WORDS];
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
+    __shared__ u64 res[2 * MAX_PTS];
+    __shared__ int ok_flag;
+
+    u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
+    bool to_ping = true;  // destination of this round's folded tables
+    for (u32 j = a.j0; j <= a.n_vars; j++) {
+        if (!tail_wait_mail(a, a.seq0 + (j - a.j0), box, &ok_flag)) return;
+        const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+        const gl::E2P rp = gl::prep(r);
+        const bool skip1 = box[MAIL_SKIP1] != 0;
+        E2 acc[NP];
+#pragma unroll
+        for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+        const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) : 0;
+        for (u64 i = threadIdx.x; i < n_pairs; i += BLOCK) {
+            E2 lo[NF], hi[NF];
+#pragma unroll
+            for (int f = 0; f < NF; f++) {
+                E2 x0, x1, x2, x3;
+                if (j == a.j0) {
+                    U64x2 p0 = ld2(a.s0[f] + 4 * i), q0 = ld2(a.s0[f] + 4 * i + 2);
+                    U64x2 p1 = ld2(a.s1[f] + 4 * i), q1 = ld2(a.s1[f] + 4 * i + 2);
+                    x0 = gl::e2(p0.x, p1.x);
+                    x1 = gl::e2(p0.y, p1.y);
+                    x2 = gl::e2(q0.x, q1.x);
+                    x3 = gl::e2(q0.y, q1.y);
+                } else {
+                    // the source is the other LDS buffer
+                    const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
+                    const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
+                    x0 = gl::e2(c0[4 * i], c1[4 * i]);
+                    x1 = gl::e2(c0[4 * i + 1], c1[4 * i + 1]);
+                    x2 = gl::e2(c0[4 * i + 2], c1[4 * i + 2]);
+                    x3 = gl::e2(c0[4 * i + 3], c1[4 * i + 3]);
+                }
+                lo[f] = fold1p(x0, x1, rp);
+                hi[f] = fold1p(x2, x3, rp);
+                u64 *d0 = to_ping ? ping[f][0] : pong[f][0];
+                u64 *d1 = to_ping ? ping[f][1] : pong[f][1];
+                d0[2 * i] = lo[f].c0;
+                d0[2 * i + 1] = hi[f].c0;
+                d1[2 * i] = lo[f].c1;
+                d1[2 * i + 1] = hi[f].c1;
+            }
+            gl::E2P restp = gl::prep(gl::e2_one());
+            if (EQ) restp = gl::prep(gl::e2(a.eq0[eq_off + i], a.eq1[eq_off + i]));
+            E2 dl[NF], cur[NF];
+#pragma unroll
+            for (int f = 0; f < NF; f++) {
+                dl[f] = gl::sub(hi[f], lo[f]);
+                cur[f] = lo[f];
+            }
+#pragma unroll
+            for (int t = 0; t < NP; t++) {
+                if (!(t == 1 && skip1)) {
+                    E2 prod = cur[0];
+#pragma unroll
+                    for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
+                    if (EQ)
+                        acc[t] = gl::fma(prod, restp, acc[t]);
+                    else
+                        acc[t] = gl::add(acc[t], prod);
+                }
+                if (t + 1 < NP) {
+#pragma unroll
+                    for (int f = 0; f < NF; f++) cur[f] = (t == 0) ? hi[f] : gl::add(cur[f], dl[f]);
+                }
+            }
+        }
+        block_reduce<NP>(acc, lds);
+        // the round message, as in the per-round kernels
+        FastFin ff;
+        ff.degree = a.degree;
+        ff.has_eq = a.has_eq;
+        ff.skip1 = skip1 ? 1 : 0;
+#pragma unroll
+        for (int k = 0; k < 2 * MAX_PTS; k++) ff.scale[k] = box[MAIL_SCALE + k];
+        ff.claim0 = box[MAIL_CLAIM];
+        ff.claim1 = box[MAIL_CLAIM + 1];
+        ff.inv_s1_0 = box[MAIL_INV];
+        ff.inv_s1_1 = box[MAIL_INV + 1];
+#pragma unroll
+        for (int k = 0; k < MAX_PTS; k++) ff.ext[k] = a.ext[k];
+        ff.const0 = box[MAIL_CONST];
+        ff.const1 = box[MAIL_CONST + 1];
+        ff.out_dev = a.out_dev;
+        ff.out_host = a.out_host;
+        ff.seq = a.seq0 + (j - a.j0);
+        ff.counter = nullptr;
+        fast_finalize<NF>(ff, acc, res);
+        __syncthreads();
+        to_ping = !to_ping;
+        n_pairs >>= 1;
+    }
+    // final evaluations: the last challenge folds the two remaining entries of every table
+    const u64 fin_seq = a.seq0 + (a.n_vars - a.j0 + 1);
+    if (!tail_wait_mail(a, fin_seq, box, &ok_flag)) return;
+    if (threadIdx.x < NF) {
+        const int f = threadIdx.x;
+        const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+        // the last round wrote its pair to the buffer `to_ping` now points away from
+        const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
+        const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
+        E2 v = fold1(gl::e2(c0[0], c1[0]), gl::e2(c0[1], c1[1]), r);
+        st_sys(a.out_host + HOST_FINALS_SLOT + 2 * f, v.c0);
+        st_sys(a.out_host + HOST_FINALS_SLOT + 2 * f + 1, v.c1);
+        __builtin_amdgcn_s_waitcnt(0);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) st_sys(a.out_host + HOST_SEQ_SLOT, fin_seq);
 }
 
 // final evaluations: entry 0 of every table after the last fold

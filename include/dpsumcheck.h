@@ -167,8 +167,9 @@ enum {
     DPS_K_EQ = 4,         /* eq table expansion */
     DPS_K_AXIS_DOT = 5,   /* partial evaluation of one axis */
     DPS_K_LOGUP = 6,      /* fraction-sum layer */
-    DPS_K_FINALIZE = 7,   /* block-partial reduction */
-    DPS_K_COUNT = 8
+    DPS_K_FINALIZE = 7,   /* round result without an evaluation launch */
+    DPS_K_TAIL = 8,       /* resident kernel running the last rounds (duration includes the host's turns) */
+    DPS_K_COUNT = 9
 };
 /* when enabled every launch of the kernels above is bracketed by events on the
  * context's stream (adds a few microseconds per launch) */
