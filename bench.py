@@ -101,6 +101,10 @@ def main():
     def gbs(by, ms):
         return by / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
+    # plain device copy moving as many bytes as the dominant launch does (half read, half written)
+    copy_bytes = 9 * (1 << n) * 2
+    copy_ms = ctx.copy_ms(copy_bytes, 10)
+
     fe, ef = stats["fold_eval"], stats["eval_first"]
     # dominant kernel: the fused fold+evaluate launch of round 2.  It reads f and g
     # (base field) and the half-size eq suffix table, writes the folded f and g.
@@ -125,6 +129,8 @@ def main():
         "avg_launch_ms": round(dom_ms, 5),
         "survey_bytes_per_launch": survey_round2,
         "survey_equivalent_gbs": round(gbs(survey_round2, dom_ms), 1),
+        "copy_kernel_gbs": round(gbs(2 * copy_bytes, copy_ms), 1),
+        "frac_of_copy_kernel": round(achieved / gbs(2 * copy_bytes, copy_ms), 4),
         "first_round_kernel_gbs": round(gbs(ef["bytes"], ef["ms"]), 1),
         "all_rounds_algorithmic_bytes": stream_bytes,
         "all_rounds_survey_bytes": survey_total,

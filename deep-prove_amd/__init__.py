@@ -70,6 +70,8 @@ dev.dps_tensor_from_i64.argtypes = [_vp, _vp, _u64, _vp]
 dev.dps_mle_wrap_device.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_mle_view.argtypes = [_vp, _u64, _u32, _vp]
 dev.dps_debug_field_op.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
+dev.dps_debug_copy.restype = _i32
+dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
            "dps_partial_eval", "dps_sc_begin", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_free",
@@ -458,6 +460,12 @@ class Context:
         out = np.zeros(2 * n, dtype=np.uint64)
         self._chk(dev.dps_debug_field_op(self._c, op, _ptr(aa), _ptr(bb), n, _ptr(out)), "dps_debug_field_op")
         return np.stack([out[:n], out[n:]], axis=-1)
+
+    def copy_ms(self, n_bytes, reps=10):
+        """average duration of a plain device copy of n_bytes (the bandwidth yardstick)"""
+        ms = C.c_double(0)
+        self._chk(dev.dps_debug_copy(self._c, n_bytes, reps, C.byref(ms)), "dps_debug_copy")
+        return ms.value
 
 
 # ---- einsum and LogUp drivers of the host mirror ----

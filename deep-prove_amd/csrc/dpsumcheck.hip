@@ -55,6 +55,8 @@ struct dps_ctx {
     std::map<void *, size_t> live_blocks;
     u64 *d_lagrange = nullptr;  // [9][9][9]
     std::vector<u64> h_lagrange;
+    u64 h_inv_den[9][9] = {};   // [d][k]: 1 / prod_{m != k, m <= d} (k - m), the Lagrange denominators over the nodes 0..d
+    u32 *d_counter = nullptr;   // ticket counter of the evaluation launches; every launch leaves it at zero
     u64 *h_pinned = nullptr;    // host-visible result buffer
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
@@ -367,8 +369,18 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
                 lag[(k * 9 + t) * 9 + i] = gl::mul(num, h_inv(den));
             }
     ctx->h_lagrange = lag;
-    if (hipMalloc((void **)&ctx->d_lagrange, lag.size() * 8) != hipSuccess) return bail(DPS_ERR_OOM);
+    for (u32 d = 0; d <= 8; d++)
+        for (u32 k = 0; k <= d; k++) {
+            u64 den = 1;
+            for (u32 m = 0; m <= d; m++)
+                if (m != k) den = gl::mul(den, gl::sub((u64)k, (u64)m));
+            ctx->h_inv_den[d][k] = h_inv(den);
+        }
+    const size_t lag_bytes = round_up(lag.size() * 8, 256);
+    if (hipMalloc((void **)&ctx->d_lagrange, lag_bytes + 256) != hipSuccess) return bail(DPS_ERR_OOM);
     if (hipMemcpy(ctx->d_lagrange, lag.data(), lag.size() * 8, hipMemcpyHostToDevice) != hipSuccess) return bail(DPS_ERR_HIP);
+    ctx->d_counter = (u32 *)((char *)ctx->d_lagrange + lag_bytes);
+    if (hipMemset(ctx->d_counter, 0, 256) != hipSuccess) return bail(DPS_ERR_HIP);
     ctx->pinned_words = 4096;
     // fine-grained host memory: a kernel's system-scope stores become visible to the polling host while the kernel runs
     if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess) {
@@ -1128,13 +1140,23 @@ namespace {
 
 u64 *mailbox(dps_ctx *ctx) { return ctx->h_pinned + ctx->res_off - 64; }
 
+// completes a mail: check word over the payload as it stands, then the sequence number the kernel waits for
+void send_mail(dps_ctx *ctx, u64 seq)
+{
+    u64 *mb = mailbox(ctx);
+    u64 chk = seq;
+    for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mb[i], i);
+    mb[dpk::MAIL_CHK] = chk;
+    __atomic_store_n(mb + dpk::MAIL_SEQ, seq, __ATOMIC_RELEASE);
+}
+
 void tail_abort(dps_ctx *ctx)
 {
     dps_sc *owner = ctx->tail_owner;
     if (!owner) return;
-    __atomic_store_n(mailbox(ctx) + dpk::MAIL_ABORT, (u64)1, __ATOMIC_RELEASE);
+    __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
     (void)hipStreamSynchronize(ctx->stream);
-    __atomic_store_n(mailbox(ctx) + dpk::MAIL_ABORT, (u64)0, __ATOMIC_RELEASE);
+    __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
     owner->tail_running = false;
     owner->broken = true;
     ctx->tail_owner = nullptr;
@@ -1406,11 +1428,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->d_partial = (u64 *)p;
     p += bytes_partial;
     sc->d_result = (u64 *)p;
-    sc->d_counter = (u32 *)(p + bytes_result - 256);
-    {
-        hipError_t e = hipMemsetAsync(sc->d_counter, 0, 256, ctx->stream);
-        if (e != hipSuccess) return cleanup(fail(ctx, DPS_ERR_HIP, "counter reset: %s", hipGetErrorString(e)));
-    }
+    sc->d_counter = ctx->d_counter;
     // one staged upload of all descriptors
     std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath, 0);
     char *q = stage.data();
@@ -1423,7 +1441,9 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     if (!fins.empty()) memcpy(q, fins.data(), fins.size() * sizeof(dpk::FinTerm));
     q += bytes_fin;
     if (!gath.empty()) memcpy(q, gath.data(), gath.size() * sizeof(dpk::GatherDesc));
-    if (!stage.empty()) {
+    // a product session that ends in the resident kernel reads none of the descriptors
+    const bool needs_descs = !(sc->fast && sc->tail_j0);
+    if (!stage.empty() && needs_descs) {
         hipError_t e = hipMemcpyAsync(sc->dev_block, stage.data(), stage.size(), hipMemcpyHostToDevice, ctx->stream);
         // the staging vector dies with this call
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -1464,19 +1484,31 @@ int32_t launch_folds(dps_sc *sc, u32 step, bool extra_only, const u64 *chal)
 
 namespace {
 
-// Wait until the launch that carries `seq` has published its result.  The host
-// polls the sequence word the last workgroup stores after the message; if it
-// does not arrive the stream is synchronised to surface the error.
-int32_t wait_result(dps_ctx *ctx, u64 seq)
+// Wait until the launch that carries `seq` has published its `n` result words
+// (at slot0 of the result area) and copy them out.  The host polls the sequence
+// word; the words are accepted once the check word agrees with them, since the
+// kernel's stores may land in any order.  If the result does not arrive the
+// stream is queried to surface the error.
+int32_t wait_result(dps_ctx *ctx, u64 seq, u32 slot0, u32 n, u64 *out)
 {
-    volatile u64 *flag = ctx->h_pinned + ctx->res_off + dpk::HOST_SEQ_SLOT;
+    volatile u64 *base = ctx->h_pinned + ctx->res_off;
+    volatile u64 *flag = base + dpk::HOST_SEQ_SLOT;
+    auto take = [&]() {
+        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) return false;
+        u64 chk = seq;
+        for (u32 i = 0; i < n; i++) {
+            out[i] = base[slot0 + i];
+            chk ^= dpk::rotl64(out[i], i + 1);
+        }
+        return chk == base[dpk::HOST_CHK_SLOT];
+    };
     for (u64 spins = 0;; spins++) {
-        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return DPS_OK;
+        if (take()) return DPS_OK;
         if ((spins & 0xFFFFF) == 0xFFFFF) {
             // about once per several milliseconds: has the stream died or finished without publishing?
             hipError_t q = hipStreamQuery(ctx->stream);
             if (q == hipSuccess) {
-                if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return DPS_OK;
+                if (take()) return DPS_OK;
                 return fail(ctx, DPS_ERR_HIP, "round result was not published");
             }
             if (q != hipErrorNotReady) return fail(ctx, DPS_ERR_HIP, "stream error while waiting for a round: %s", hipGetErrorString(q));
@@ -1538,13 +1570,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             E2 acc = gl::e2_zero();
             for (u32 k = 0; k <= d; k++) {
                 E2 num = gl::e2_one();
-                u64 den = 1;
-                for (u32 m = 0; m <= d; m++) {
-                    if (m == k) continue;
-                    num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
-                    den = gl::mul(den, gl::sub((u64)k, (u64)m));
-                }
-                acc = gl::add(acc, gl::mul(gl::mul_base(num, h_inv(den)), sc->last_msg[k]));
+                for (u32 m = 0; m <= d; m++)
+                    if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+                acc = gl::add(acc, gl::mul(gl::mul_base(num, ctx->h_inv_den[d][k]), sc->last_msg[k]));
             }
             sc->claim = acc;
             if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
@@ -1559,21 +1587,30 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         }
         E2 s1 = gl::e2(ff.scale[2], ff.scale[3]);
         const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
-        if (skip1) {
-            E2 inv = h_e2_inv(s1);
-            ff.inv_s1_0 = inv.c0;
-            ff.inv_s1_1 = inv.c1;
-            // the constant terms add c to p(0) and to p(1)
-            E2 cl = gl::sub(sc->claim, gl::add(cst, cst));
-            ff.claim0 = cl.c0;
-            ff.claim1 = cl.c1;
-        }
         a.skip1 = skip1 ? 1 : 0;
+        ff.claim0 = sc->claim.c0;
+        ff.claim1 = sc->claim.c1;
         if (has_eq) {
             const u64 off = eq_level_off(sc->n_vars, j);
             a.q0 = sc->eq_c0 + off;
             a.q1 = sc->eq_c1 + off;
-            for (u32 i = 0; i <= nf; i++) ff.ext[i] = ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i];
+            // p(nf + 1) = sum_i cext_i q(i) + k + const
+            const E2 s_top = gl::e2(ff.scale[2 * (nf + 1)], ff.scale[2 * (nf + 1) + 1]);
+            E2 cext[dpk::MAX_PTS];
+            for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
+            if (skip1) {
+                // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
+                const E2 A = gl::mul(cext[1], h_e2_inv(s1));
+                cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(ff.scale[0], ff.scale[1])));
+                const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
+                ff.k0 = kk.c0;
+                ff.k1 = kk.c1;
+                cext[1] = gl::e2_zero();
+            }
+            for (u32 i = 0; i <= nf; i++) {
+                ff.cext[2 * i] = cext[i].c0;
+                ff.cext[2 * i + 1] = cext[i].c1;
+            }
         }
         ff.partial = sc->d_partial;
         ff.n_blocks = blocks;
@@ -1591,16 +1628,18 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             u64 *mb = mailbox(ctx);
             mb[dpk::MAIL_R] = a.r0;
             mb[dpk::MAIL_R + 1] = a.r1;
-            for (u32 k = 0; k < 2 * dpk::MAX_PTS; k++) mb[dpk::MAIL_SCALE + k] = ff.scale[k];
+            for (u32 k = 0; k < 2 * dpk::MAX_PTS; k++) {
+                mb[dpk::MAIL_SCALE + k] = ff.scale[k];
+                mb[dpk::MAIL_CEXT + k] = ff.cext[k];
+            }
+            mb[dpk::MAIL_K] = ff.k0;
+            mb[dpk::MAIL_K + 1] = ff.k1;
             mb[dpk::MAIL_CLAIM] = ff.claim0;
             mb[dpk::MAIL_CLAIM + 1] = ff.claim1;
-            mb[dpk::MAIL_INV] = ff.inv_s1_0;
-            mb[dpk::MAIL_INV + 1] = ff.inv_s1_1;
             mb[dpk::MAIL_CONST] = cst.c0;
             mb[dpk::MAIL_CONST + 1] = cst.c1;
             mb[dpk::MAIL_SKIP1] = a.skip1;
-            mb[dpk::MAIL_ABORT] = 0;
-            __atomic_store_n(mb + dpk::MAIL_SEQ, fa.seq, __ATOMIC_RELEASE);
+            send_mail(ctx, fa.seq);
             if (j == sc->tail_j0) {
                 dpk::TailArgs ta;
                 memset(&ta, 0, sizeof ta);
@@ -1614,7 +1653,6 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 ta.j0 = j;
                 ta.degree = sc->degree;
                 ta.has_eq = has_eq ? 1 : 0;
-                for (u32 k = 0; k < dpk::MAX_PTS; k++) ta.ext[k] = ff.ext[k];
                 ta.mail = ctx->d_pinned + (ctx->res_off - 64);
                 ta.out_host = fa.out_host;
                 ta.out_dev = sc->d_result;
@@ -1631,8 +1669,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 sc->tail_running = true;
                 ctx->tail_owner = sc;
             }
-            CHK(wait_result(ctx, fa.seq));
-            memcpy(evals_out, ctx->h_pinned + ctx->res_off, 2 * (sc->degree + 1) * 8);
+            CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
             sc->last_msg.resize(sc->degree + 1);
             for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
             sc->round = j;
@@ -1658,8 +1695,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             HIPCHK(ctx, hipGetLastError());
         }
     }
-    CHK(wait_result(ctx, fa.seq));
-    memcpy(evals_out, ctx->h_pinned + ctx->res_off, 2 * (sc->degree + 1) * 8);
+    CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
     if (sc->fast) {
         sc->last_msg.resize(sc->degree + 1);
         for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
@@ -1684,15 +1720,15 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         const u64 seq = ++ctx->seq;
         mb[dpk::MAIL_R] = challenge[0];
         mb[dpk::MAIL_R + 1] = challenge[1];
-        __atomic_store_n(mb + dpk::MAIL_SEQ, seq, __ATOMIC_RELEASE);
-        int32_t rc = wait_result(ctx, seq);
+        send_mail(ctx, seq);
+        u64 fin[2 * 3];
+        int32_t rc = wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * sc->fast_nf, fin);
         // the kernel exits right after publishing
         hipError_t e = hipStreamSynchronize(ctx->stream);
         sc->tail_running = false;
         ctx->tail_owner = nullptr;
         if (rc != DPS_OK) return rc;
         if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "tail kernel: %s", hipGetErrorString(e));
-        const u64 *fin = ctx->h_pinned + ctx->res_off + dpk::HOST_FINALS_SLOT;
         for (u32 f = 0; f < sc->fast_nf; f++) {
             final_evals_out[2 * sc->fast_order[f]] = fin[2 * f];
             final_evals_out[2 * sc->fast_order[f] + 1] = fin[2 * f + 1];
@@ -1910,5 +1946,44 @@ extern "C" int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *
     if (e == hipSuccess) e = hipMemcpy(out, d + 4 * n, 2 * n * 8, hipMemcpyDeviceToHost);
     pool_free(ctx, p);
     if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "field op: %s", hipGetErrorString(e));
+    return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// streaming copy: the yardstick the memory counters and the evaluation kernels'
+// bandwidth are read against
+// ---------------------------------------------------------------------------
+extern "C" int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out)
+{
+    if (!ctx || n_bytes == 0 || (n_bytes & 15) || reps == 0) return fail(ctx, DPS_ERR_INVALID, "dps_debug_copy: bad argument");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, 2 * n_bytes, &p));
+    const uint4 *src = (const uint4 *)p;
+    uint4 *dst = (uint4 *)((char *)p + n_bytes);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipMemsetAsync(p, 0x5a, n_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const u64 n16 = n_bytes / 16;
+    const u32 blocks = (u32)std::min<u64>((n16 + dpk::BLOCK - 1) / dpk::BLOCK, 8 * MAX_BLOCKS);
+    if (e == hipSuccess) {
+        dpk::copy_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(src, dst, n16);  // untimed first touch
+        e = hipEventRecord(e0, ctx->stream);
+    }
+    for (u32 r = 0; r < reps && e == hipSuccess; r++) {
+        dpk::copy_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(src, dst, n16);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    pool_free(ctx, p);
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "copy: %s", hipGetErrorString(e));
+    if (avg_ms_out) *avg_ms_out = (double)ms / reps;
     return DPS_OK;
 }

@@ -242,6 +242,8 @@ struct FinArgs {
     u32 *counter;          // ticket counter, zero between launches
 };
 constexpr int HOST_SEQ_SLOT = 2 * MAX_PTS;
+constexpr int HOST_CHK_SLOT = HOST_SEQ_SLOT + 1;
+constexpr int HOST_FINALS_SLOT = HOST_SEQ_SLOT + 8;
 
 // Block partials cross XCDs (each XCD has its own L2).  They are written and read
 // with agent-scope accesses, which go through to the coherence point, so that no
@@ -255,6 +257,31 @@ __device__ __forceinline__ u64 ld_agent(const u64 *p)
 __device__ __forceinline__ void st_agent(u64 *p, u64 v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// host-visible (fine-grained pinned) memory
+__device__ __forceinline__ u64 ld_sys(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
+__device__ __forceinline__ void st_sys(u64 *p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
+
+__host__ __device__ __forceinline__ u64 rotl64(u64 x, u32 k)
+{
+    k &= 63;
+    return k ? (x << k) | (x >> (64 - k)) : x;
+}
+
+// Hand `n` result words to the host (one thread calls this): the words, a check
+// word and the sequence number the host polls.  Nothing waits for a store to be
+// acknowledged, and the order in which the stores land does not matter: the
+// host accepts the words only when  check == seq ^ xor_i rotl(word_i, i + 1).
+__device__ __forceinline__ void publish_words(u64 *out_host, u32 slot0, const u64 *words, u32 n, u64 seq)
+{
+    u64 chk = seq;
+    for (u32 i = 0; i < n; i++) {
+        const u64 w = words[i];
+        chk ^= rotl64(w, i + 1);
+        st_sys(out_host + slot0 + i, w);
+    }
+    st_sys(out_host + HOST_CHK_SLOT, chk);
+    st_sys(out_host + HOST_SEQ_SLOT, seq);
 }
 
 // Called by every thread of one workgroup once all partials are visible.
@@ -307,16 +334,13 @@ __device__ __forceinline__ void finalize_block(const FinArgs &fa, u32 *lds /* (B
         u64 c0 = gl::add(res[2 * t], fa.const0), c1 = gl::add(res[2 * t + 1], fa.const1);
         fa.out_dev[2 * t] = c0;
         fa.out_dev[2 * t + 1] = c1;
-        // system-scope stores go through to host memory; no cache-wide write-back is needed for them
-        __hip_atomic_store(fa.out_host + 2 * t, c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        __hip_atomic_store(fa.out_host + 2 * t + 1, c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        __builtin_amdgcn_s_waitcnt(0);  // the message has been acknowledged ...
+        res[2 * t] = c0;
+        res[2 * t + 1] = c1;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         *fa.counter = 0;
-        // ... before the sequence number the host polls is stored
-        __hip_atomic_store(fa.out_host + HOST_SEQ_SLOT, fa.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        publish_words(fa.out_host, 0, res, 2 * (fa.degree + 1), fa.seq);
     }
 }
 
@@ -464,7 +488,18 @@ struct ProdArgs {
     u32 skip1;    // 1: do not evaluate t = 1
 };
 
-// What the last workgroup needs to turn the sums q(t) into the round message.
+// What the last workgroup needs to turn the sums q(t), t = 0..NF, into the round
+// message p(t) = scale(t) q(t) + const, t = 0..degree.
+//
+// With an eq factor the message has one point more than the kernel sums:
+// q(NF + 1) = sum_i ext_i q(i) (Lagrange over the nodes 0..NF), so
+// p(NF + 1) = sum_i cext_i q(i) + const with cext_i = scale(NF + 1) ext_i.
+//
+// skip1: the caller knows claim = p(0) + p(1); the kernel did not sum q(1).
+// Then p(1) = claim - p(0), and q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
+// is folded into the coefficients by the host: with A = cext_1 / scale(1),
+// cext_0 becomes cext_0 - A scale(0), and k = A (claim - 2 const) is added.
+// Every product is then independent of the others: one lane each.
 struct FastFin {
     const u64 *partial;
     u32 n_blocks;
@@ -472,9 +507,9 @@ struct FastFin {
     u32 has_eq;
     u32 skip1;
     u64 scale[2 * MAX_PTS];  // scale(t) for t = 0..degree, extension elements
+    u64 cext[2 * MAX_PTS];   // coefficient of q(i) in p(NF + 1), i = 0..NF (eq factor only; entry 1 unused when skip1)
+    u64 k0, k1;              // constant part of p(NF + 1) (eq factor and skip1 only, else 0)
     u64 claim0, claim1;      // p(0) + p(1), used when skip1
-    u64 inv_s1_0, inv_s1_1;  // 1 / scale(1), used when skip1
-    u64 ext[MAX_PTS];        // Lagrange weights of q(NF + 1) over the nodes 0..NF (eq factor only)
     u64 const0, const1;      // constant terms summed over the remaining hypercube
     u64 *out_dev;
     u64 *out_host;
@@ -499,51 +534,62 @@ __device__ __forceinline__ void gather_partials(const FastFin &ff, u32 *lds, E2 
     block_reduce<NP>(q, lds);
 }
 
-// sums[t] = q(t) for t = 0..NF, valid in thread 0
+// sums[t] = q(t) for t = 0..NF, valid in thread 0.  res: 6 * MAX_PTS words of LDS.
 template <int NF>
 __device__ __forceinline__ void fast_finalize(const FastFin &ff, const E2 (&sums)[NF + 1], u64 *res)
 {
     constexpr int NP = NF + 1;
-    E2 q[NP + 1];
-#pragma unroll
-    for (int t = 0; t < NP; t++) q[t] = sums[t];
-    q[NP] = gl::e2_zero();
+    u64 *q = res;                  // 2 * NP words
+    u64 *prod = res + 2 * MAX_PTS; // 2 * (2 * NP) words
+    u64 *out = res + 2 * MAX_PTS;  // reused for the message after the products are consumed
     if (threadIdx.x == 0) {
-        if (ff.skip1) {
-            // scale(0) q(0) + scale(1) q(1) = claim
-            E2 s0 = gl::e2(ff.scale[0], ff.scale[1]);
-            E2 rest = gl::sub(gl::e2(ff.claim0, ff.claim1), gl::mul(s0, q[0]));
-            q[1] = gl::mul(rest, gl::e2(ff.inv_s1_0, ff.inv_s1_1));
-        }
-        if (ff.has_eq) {
-            E2 e = gl::e2_zero();
 #pragma unroll
-            for (int i = 0; i < NP; i++) e = gl::add(e, gl::mul_base(q[i], ff.ext[i]));
-            q[NP] = e;
+        for (int t = 0; t < NP; t++) {
+            q[2 * t] = sums[t].c0;
+            q[2 * t + 1] = sums[t].c1;
         }
+    }
+    __syncthreads();
+    // lane t < NP: scale(t) q(t); lane NP + i: cext_i q(i)
+    if (threadIdx.x < 2 * NP) {
+        const u32 l = threadIdx.x, i = l < NP ? l : l - NP;
+        const bool needed = !(ff.skip1 && i == 1) && (l < NP || ff.has_eq);
+        E2 v = gl::e2_zero();
+        if (needed) {
+            // the coefficient is picked with constant indices so that it stays in registers
+            E2 c = gl::e2_zero();
+#pragma unroll
+            for (int k = 0; k < NP; k++) {
+                if (l == (u32)k) c = gl::e2(ff.scale[2 * k], ff.scale[2 * k + 1]);
+                if (l == (u32)(NP + k)) c = gl::e2(ff.cext[2 * k], ff.cext[2 * k + 1]);
+            }
+            v = gl::mul(gl::e2(q[2 * i], q[2 * i + 1]), c);
+        }
+        prod[2 * l] = v.c0;
+        prod[2 * l + 1] = v.c1;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        E2 msg[NP + 1];
+        const E2 cst = gl::e2(ff.const0, ff.const1);
+#pragma unroll
+        for (int t = 0; t < NP; t++) msg[t] = gl::add(gl::e2(prod[2 * t], prod[2 * t + 1]), cst);
+        if (ff.skip1) msg[1] = gl::sub(gl::e2(ff.claim0, ff.claim1), msg[0]);
+        E2 e = gl::add(gl::e2(ff.k0, ff.k1), cst);
+#pragma unroll
+        for (int i = 0; i < NP; i++) e = gl::add(e, gl::e2(prod[2 * (NP + i)], prod[2 * (NP + i) + 1]));
+        msg[NP] = e;
 #pragma unroll
         for (int t = 0; t <= NP; t++) {
             if ((u32)t <= ff.degree) {
-                E2 v = gl::mul(q[t], gl::e2(ff.scale[2 * t], ff.scale[2 * t + 1]));
-                res[2 * t] = gl::add(v.c0, ff.const0);
-                res[2 * t + 1] = gl::add(v.c1, ff.const1);
+                out[2 * t] = msg[t].c0;
+                out[2 * t + 1] = msg[t].c1;
+                ff.out_dev[2 * t] = msg[t].c0;
+                ff.out_dev[2 * t + 1] = msg[t].c1;
             }
         }
-    }
-    __syncthreads();
-    if (threadIdx.x <= ff.degree) {
-        u32 t = threadIdx.x;
-        u64 c0 = res[2 * t], c1 = res[2 * t + 1];
-        ff.out_dev[2 * t] = c0;
-        ff.out_dev[2 * t + 1] = c1;
-        __hip_atomic_store(ff.out_host + 2 * t, c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        __hip_atomic_store(ff.out_host + 2 * t + 1, c1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        __builtin_amdgcn_s_waitcnt(0);
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
         if (ff.counter) *ff.counter = 0;
-        __hip_atomic_store(ff.out_host + HOST_SEQ_SLOT, ff.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        publish_words(ff.out_host, 0, out, 2 * (ff.degree + 1), ff.seq);
     }
 }
 
@@ -552,7 +598,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 {
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
-    __shared__ u64 res[2 * MAX_PTS];
+    __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
     const E2 r = gl::e2(a.r0, a.r1);
     const gl::E2P rp = gl::prep(r);
@@ -715,9 +761,14 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 // gives up after `spin_limit` polls and exits.
 // ---------------------------------------------------------------------------
 constexpr int TAIL_PAIRS = 256;
-constexpr int MAIL_SEQ = 0, MAIL_R = 1, MAIL_SCALE = 3, MAIL_CLAIM = 3 + 2 * MAX_PTS, MAIL_INV = MAIL_CLAIM + 2,
-              MAIL_CONST = MAIL_INV + 2, MAIL_SKIP1 = MAIL_CONST + 2, MAIL_ABORT = MAIL_SKIP1 + 1, MAIL_WORDS = MAIL_ABORT + 1;
-constexpr int HOST_FINALS_SLOT = HOST_SEQ_SLOT + 8;
+// mailbox words; MAIL_SEQ == MAIL_ABORT_SEQ tells the kernel to exit
+constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SCALE = 4, MAIL_CEXT = MAIL_SCALE + 2 * MAX_PTS, MAIL_K = MAIL_CEXT + 2 * MAX_PTS,
+              MAIL_CLAIM = MAIL_K + 2, MAIL_CONST = MAIL_CLAIM + 2, MAIL_SKIP1 = MAIL_CONST + 2, MAIL_WORDS = MAIL_SKIP1 + 1;
+static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
+constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
+
+// check word of a mailbox: seq ^ xor over the payload words of rotl(word_i, i)
+__host__ __device__ __forceinline__ u64 mail_mix(u64 w, u32 i) { return (i >= (u32)MAIL_R && i < (u32)MAIL_WORDS) ? rotl64(w, i) : 0; }
 
 struct TailArgs {
     const u64 *s0[3];
@@ -726,7 +777,6 @@ struct TailArgs {
     const u64 *eq1;
     u32 n_vars, j0;    // the sum's variables, first round handled here (1-based)
     u32 degree, has_eq;
-    u64 ext[MAX_PTS];  // Lagrange weights of q(NF + 1) (eq factor only)
     const u64 *mail;   // host mailbox, MAIL_WORDS words
     u64 *out_host;     // message limbs, HOST_SEQ_SLOT, HOST_FINALS_SLOT
     u64 *out_dev;
@@ -734,30 +784,34 @@ struct TailArgs {
     u32 spin_limit;
 };
 
-__device__ __forceinline__ u64 ld_sys(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
-__device__ __forceinline__ void st_sys(u64 *p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
-
-// Waits for mail number `want`; copies it to `box` (LDS).  Returns false on abort or timeout.
+// Waits for mail number `want` and copies it to `box` (LDS).  The first wavefront
+// polls: every lane loads one mailbox word, so one load instruction (one trip over
+// the host link) fetches the whole mail; it is accepted when the sequence number
+// matches and the check word agrees with the payload, which makes a torn read
+// (the host still writing) look like no mail yet.  Returns false on abort or timeout.
 __device__ __forceinline__ bool tail_wait_mail(const TailArgs &a, u64 want, u64 *box, int *ok_lds)
 {
-    if (threadIdx.x == 0) {
+    if (threadIdx.x < WAVE) {
+        const u32 l = threadIdx.x;
         int ok = 0;
         for (u32 spins = 0; spins < a.spin_limit; spins++) {
-            u64 s = __hip_atomic_load(a.mail + MAIL_SEQ, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
-            if (s == want) {
+            const u64 w = l < (u32)MAIL_WORDS ? ld_sys(a.mail + l) : 0;
+            u64 x = mail_mix(w, l);
+#pragma unroll
+            for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
+            const u64 seq = __shfl(w, MAIL_SEQ, WAVE), chk = __shfl(w, MAIL_CHK, WAVE);
+            if (seq == MAIL_ABORT_SEQ) break;
+            if (seq == want && chk == (x ^ seq)) {
+                if (l < (u32)MAIL_WORDS) box[l] = w;
                 ok = 1;
                 break;
             }
-            if (ld_sys(a.mail + MAIL_ABORT) != 0) break;
-            __builtin_amdgcn_s_sleep(4);
+            __builtin_amdgcn_s_sleep(2);
         }
-        *ok_lds = ok;
+        if (l == 0) *ok_lds = ok;
     }
     __syncthreads();
-    if (!*ok_lds) return false;
-    if (threadIdx.x < MAIL_WORDS) box[threadIdx.x] = ld_sys(a.mail + threadIdx.x);
-    __syncthreads();
-    return true;
+    return *ok_lds != 0;
 }
 
 template <int NF, bool EQ>
@@ -769,7 +823,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
     __shared__ u64 pong[NF][2][TAIL_PAIRS];
     __shared__ u64 box[MAIL_WORDS];
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
-    __shared__ u64 res[2 * MAX_PTS];
+    __shared__ u64 res[6 * MAX_PTS];
     __shared__ int ok_flag;
 
     u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
@@ -848,10 +902,10 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
         for (int k = 0; k < 2 * MAX_PTS; k++) ff.scale[k] = box[MAIL_SCALE + k];
         ff.claim0 = box[MAIL_CLAIM];
         ff.claim1 = box[MAIL_CLAIM + 1];
-        ff.inv_s1_0 = box[MAIL_INV];
-        ff.inv_s1_1 = box[MAIL_INV + 1];
+        ff.k0 = box[MAIL_K];
+        ff.k1 = box[MAIL_K + 1];
 #pragma unroll
-        for (int k = 0; k < MAX_PTS; k++) ff.ext[k] = a.ext[k];
+        for (int k = 0; k < 2 * MAX_PTS; k++) ff.cext[k] = box[MAIL_CEXT + k];
         ff.const0 = box[MAIL_CONST];
         ff.const1 = box[MAIL_CONST + 1];
         ff.out_dev = a.out_dev;
@@ -873,12 +927,11 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
         const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
         const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
         E2 v = fold1(gl::e2(c0[0], c1[0]), gl::e2(c0[1], c1[1]), r);
-        st_sys(a.out_host + HOST_FINALS_SLOT + 2 * f, v.c0);
-        st_sys(a.out_host + HOST_FINALS_SLOT + 2 * f + 1, v.c1);
-        __builtin_amdgcn_s_waitcnt(0);
+        res[2 * f] = v.c0;
+        res[2 * f + 1] = v.c1;
     }
     __syncthreads();
-    if (threadIdx.x == 0) st_sys(a.out_host + HOST_SEQ_SLOT, fin_seq);
+    if (threadIdx.x == 0) publish_words(a.out_host, HOST_FINALS_SLOT, res, 2 * NF, fin_seq);
 }
 
 // final evaluations: entry 0 of every table after the last fold
@@ -1110,6 +1163,12 @@ field_op_kernel(int op, const u64 *__restrict__ a0, const u64 *__restrict__ a1, 
     }
     o0[i] = r.c0;
     o1[i] = r.c1;
+}
+
+// plain streaming copy, 16 bytes per lane
+__global__ __launch_bounds__(BLOCK) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, u64 n16)
+{
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < n16; i += (u64)gridDim.x * BLOCK) dst[i] = src[i];
 }
 
 }  // namespace dpk

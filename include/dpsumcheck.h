@@ -187,6 +187,12 @@ const char *dps_kernel_name(int32_t kernel);
  * base (b.c0), 5 (embed int64 a.c0, a.c1 times the 32-bit constant b.c1). */
 int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *a, const uint64_t *b, uint64_t n, uint64_t *out);
 
+/* ---- bandwidth yardstick: `reps` launches of a plain device-to-device copy of
+ * n_bytes (a multiple of 16); returns the average launch duration.  No
+ * counterpart in the reference; it is what the evaluation kernels' bandwidth
+ * and the profiler's memory counters are read against. */
+int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
+
 #ifdef __cplusplus
 }
 #endif
