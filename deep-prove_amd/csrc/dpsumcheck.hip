@@ -1171,10 +1171,14 @@ void launch_tail(dps_ctx *ctx, const dpk::TailArgs &a)
 template <int NF, int NB, bool EQ>
 void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial, const dpk::FastFin &ff)
 {
-    if (fold)
-        dpk::prod_kernel<NF, NB, true, EQ><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+    if (fold && a.skip1)
+        dpk::prod_kernel<NF, NB, true, EQ, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+    else if (fold)
+        dpk::prod_kernel<NF, NB, true, EQ, false><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+    else if (a.skip1)
+        dpk::prod_kernel<NF, NB, false, EQ, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
     else
-        dpk::prod_kernel<NF, NB, false, EQ><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+        dpk::prod_kernel<NF, NB, false, EQ, false><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
 }
 
 int32_t launch_prod_dispatch(dps_ctx *ctx, u32 nf, u32 nb, bool eq, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial,

@@ -485,7 +485,7 @@ struct ProdArgs {
     const u64 *q1;
     u64 n_pairs;  // pairs evaluated this round
     u64 r0, r1;   // fold challenge
-    u32 skip1;    // 1: do not evaluate t = 1
+    u32 skip1;    // 1: t = 1 is not evaluated (the launch picks the kernel variant accordingly)
 };
 
 // What the last workgroup needs to turn the sums q(t), t = 0..NF, into the round
@@ -593,7 +593,7 @@ __device__ __forceinline__ void fast_finalize(const FastFin &ff, const E2 (&sums
     }
 }
 
-template <int NF, int NB, bool FOLD, bool EQ>
+template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1>
 __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial, FastFin ff)
 {
     constexpr int NP = NF + 1;
@@ -602,7 +602,8 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     __shared__ int last_flag;
     const E2 r = gl::e2(a.r0, a.r1);
     const gl::E2P rp = gl::prep(r);
-    const bool skip1 = a.skip1 != 0;
+    // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
+    constexpr bool skip1 = SKIP1;
     E2 acc[NP];
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
@@ -634,14 +635,8 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             w.q1 = a.q1[i];
         }
     };
-    const u64 stride = (u64)gridDim.x * BLOCK;
-    u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
-    Raw w;
-    if (i < a.n_pairs) load_raw(i, w);
-    for (; i < a.n_pairs; i += stride) {
-        Raw nxt;
-        const bool more = i + stride < a.n_pairs;
-        if (!FOLD && more) load_raw(i + stride, nxt);
+    // one loop step on loaded operands
+    auto step = [&](u64 i, const Raw &w) {
         E2 lo[NF], hi[NF];
         // base-field arithmetic applies only while the sources are read unfolded
         constexpr int NBE = FOLD ? 0 : NB;
@@ -700,7 +695,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 } else {
                     prod = cur[0];
 #pragma unroll
-                    for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
+                    for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
                     // the last product and the running sum share one reduction
                     if (EQ) {
                         acc[t] = gl::fma(prod, restp, acc[t]);
@@ -721,11 +716,28 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 }
             }
         }
-        if (more) {
-            if (FOLD)
-                load_raw(i + stride, w);
-            else
-                w = nxt;
+    };
+    const u64 stride = (u64)gridDim.x * BLOCK;
+    u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (FOLD) {
+        Raw w;
+        if (i < a.n_pairs) load_raw(i, w);
+        for (; i < a.n_pairs; i += stride) {
+            step(i, w);
+            if (i + stride < a.n_pairs) load_raw(i + stride, w);
+        }
+    } else {
+        // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
+        Raw wa, wb;
+        if (i < a.n_pairs) load_raw(i, wa);
+        while (i < a.n_pairs) {
+            if (i + stride < a.n_pairs) load_raw(i + stride, wb);
+            step(i, wa);
+            i += stride;
+            if (i >= a.n_pairs) break;
+            if (i + stride < a.n_pairs) load_raw(i + stride, wa);
+            step(i, wb);
+            i += stride;
         }
     }
     block_reduce<NP>(acc, lds);
