@@ -157,4 +157,80 @@ GL_FN E2 mulp(E2 a, E2P b) { return fma(a, b, e2_zero()); }
 
 GL_FN bool eq(E2 a, E2 b) { return a.c0 == b.c0 && a.c1 == b.c1; }
 
+// ---------------------------------------------------------------------------
+// Unreduced accumulation.  A long sum of products needs no reduction per term:
+// the low and the high 64 bits of every 128-bit product are added into two
+// 64-bit words whose carries are counted, and the whole is reduced once,
+//   value = lo + cl 2^64 + (hi + ch 2^64) 2^64,   2^64 = 2^32 - 1,  2^128 = -2^32.
+// Good for up to 2^32 - 1 terms.
+// ---------------------------------------------------------------------------
+struct Acc {
+    u64 lo, hi;
+    u32 cl, ch;
+};
+
+GL_FN Acc acc_zero()
+{
+    Acc a;
+    a.lo = a.hi = 0;
+    a.cl = a.ch = 0;
+    return a;
+}
+
+GL_FN void acc_add64(Acc &a, u64 x)
+{
+    u64 s;
+    a.cl += __builtin_add_overflow(a.lo, x, &s) ? 1u : 0u;
+    a.lo = s;
+}
+
+GL_FN void acc_add(Acc &a, u128 p)
+{
+    u64 s;
+    a.cl += __builtin_add_overflow(a.lo, (u64)p, &s) ? 1u : 0u;
+    a.lo = s;
+    a.ch += __builtin_add_overflow(a.hi, (u64)(p >> 64), &s) ? 1u : 0u;
+    a.hi = s;
+}
+
+GL_FN u64 acc_reduce(const Acc &a)
+{
+    u64 r = reduce128(a.lo, a.hi);
+    r = add(r, (u64)a.cl * EPS);      // cl (2^32 - 1) < p
+    return sub(r, (u64)a.ch << 32);  // ch 2^32 < p
+}
+
+struct E2Acc {
+    Acc c0, c1;
+};
+
+GL_FN E2Acc e2acc_zero()
+{
+    E2Acc a;
+    a.c0 = acc_zero();
+    a.c1 = acc_zero();
+    return a;
+}
+// += v
+GL_FN void acc_e2(E2Acc &a, E2 v)
+{
+    acc_add64(a.c0, v.c0);
+    acc_add64(a.c1, v.c1);
+}
+// += x * b, b in the base field
+GL_FN void acc_mul_base(E2Acc &a, E2 x, u64 b)
+{
+    acc_add(a.c0, (u128)x.c0 * b);
+    acc_add(a.c1, (u128)x.c1 * b);
+}
+// += x * y, y prepared
+GL_FN void acc_mul(E2Acc &a, E2 x, E2P y)
+{
+    acc_add(a.c0, (u128)x.c0 * y.c0);
+    acc_add(a.c0, (u128)x.c1 * y.w);
+    acc_add(a.c1, (u128)x.c0 * y.c1);
+    acc_add(a.c1, (u128)x.c1 * y.c0);
+}
+GL_FN E2 acc_reduce(const E2Acc &a) { return e2(acc_reduce(a.c0), acc_reduce(a.c1)); }
+
 }  // namespace gl

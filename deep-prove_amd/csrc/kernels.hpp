@@ -604,9 +604,10 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     const gl::E2P rp = gl::prep(r);
     // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
     constexpr bool skip1 = SKIP1;
-    E2 acc[NP];
+    // running sums, reduced once after the loop
+    gl::E2Acc lz[NP];
 #pragma unroll
-    for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+    for (int t = 0; t < NP; t++) lz[t] = gl::e2acc_zero();
 
     // Raw operands of one loop step.  The first-round kernel has little arithmetic
     // per byte, so it loads the next step's operands before working on the
@@ -678,31 +679,33 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 #pragma unroll
         for (int t = 0; t < NP; t++) {
             if (!(t == 1 && skip1)) {
-                E2 prod;
-                bool continue_step = false;
                 if (NBE > 0) {
                     u64 b = cur[0].c0;
 #pragma unroll
                     for (int f = 1; f < NBE; f++) b = gl::mul(b, cur[f].c0);
                     if (NBE == NF) {
-                        prod = EQ ? gl::mul_base(rest, b) : gl::e2(b, 0);
+                        if (EQ)
+                            gl::acc_mul_base(lz[t], rest, b);
+                        else
+                            gl::acc_add64(lz[t].c0, b);
                     } else {
-                        prod = gl::mul_base(cur[NBE], b);
+                        E2 prod = gl::mul_base(cur[NBE], b);
 #pragma unroll
                         for (int f = NBE + 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
-                        if (EQ) prod = gl::mul(prod, rest);
+                        if (EQ)
+                            gl::acc_mul(lz[t], prod, restp);
+                        else
+                            gl::acc_e2(lz[t], prod);
                     }
                 } else {
-                    prod = cur[0];
+                    E2 prod = cur[0];
 #pragma unroll
                     for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
-                    // the last product and the running sum share one reduction
-                    if (EQ) {
-                        acc[t] = gl::fma(prod, restp, acc[t]);
-                        continue_step = true;
-                    }
+                    if (EQ)
+                        gl::acc_mul(lz[t], prod, restp);
+                    else
+                        gl::acc_e2(lz[t], prod);
                 }
-                if (!continue_step) acc[t] = gl::add(acc[t], prod);
             }
             if (t + 1 < NP) {
 #pragma unroll
@@ -740,6 +743,9 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             i += stride;
         }
     }
+    E2 acc[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
     block_reduce<NP>(acc, lds);
     if (gridDim.x == 1) {
         // a single workgroup: its sums are the round's sums, no partials and no ticket
