@@ -69,6 +69,8 @@ dev.dps_mle_from_i64.argtypes = [_vp, _vp, _u64, _u32, _vp]
 dev.dps_tensor_from_i64.argtypes = [_vp, _vp, _u64, _vp]
 dev.dps_mle_wrap_device.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_mle_view.argtypes = [_vp, _u64, _u32, _vp]
+dev.dps_mle_zero_pad.restype = _i32
+dev.dps_mle_zero_pad.argtypes = [_vp, _u32, _vp]
 dev.dps_debug_field_op.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
@@ -230,6 +232,12 @@ class Mle:
     def view(self, offset, n_vars):
         h = _vp()
         self.ctx._chk(dev.dps_mle_view(self._h, offset, n_vars, C.byref(h)), "dps_mle_view")
+        return Mle(self.ctx, h)
+
+    def zero_pad(self, n_vars):
+        """the table as a sumcheck over n_vars variables reads it: 0 wherever an added variable is 1"""
+        h = _vp()
+        self.ctx._chk(dev.dps_mle_zero_pad(self._h, n_vars, C.byref(h)), "dps_mle_zero_pad")
         return Mle(self.ctx, h)
 
     def evaluate(self, point):

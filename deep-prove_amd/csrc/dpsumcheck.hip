@@ -277,6 +277,7 @@ struct dps_mle {
     u64 offset;
     u64 len;
     std::shared_ptr<EqInfo> eq;  // set on eq tables (and on views covering the whole table)
+    u32 pad_vars = 0;            // > 0: read by a sumcheck as zero-padded to this many variables
     const u64 *p0() const { return st->c0 + offset; }
     const u64 *p1() const { return st->c1 ? st->c1 + offset : nullptr; }
 };
@@ -562,11 +563,22 @@ extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_
     if (!src || !out) return DPS_ERR_INVALID;
     dps_ctx *ctx = src->ctx;
     u64 len = 1ull << n_vars;
+    if (src->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_view: the table is a zero-padded view");
     if (n_vars > 40 || offset > src->len || len > src->len - offset) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: window outside the table");
     // pair loads are 16 bytes wide
     if (n_vars >= 1 && ((src->offset + offset) & 1)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: offset must be even");
     *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len, nullptr};
     if (*out && offset == 0 && len == src->len) (*out)->eq = src->eq;
+    return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
+}
+
+extern "C" int32_t dps_mle_zero_pad(const dps_mle *src, uint32_t n_vars, dps_mle **out)
+{
+    if (!src || !out) return DPS_ERR_INVALID;
+    dps_ctx *ctx = src->ctx;
+    if (src->kind == DPS_I64 || !is_pow2(src->len)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: not a power-of-two field table");
+    if (n_vars > 40 || (1ull << n_vars) < src->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: %u variables are fewer than the table has", n_vars);
+    *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset, src->len, nullptr, n_vars};
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
 }
 
@@ -812,6 +824,7 @@ int32_t axis_dot(dps_ctx *ctx, const AxisJob &j)
 extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t n, uint64_t out[2])
 {
     if (!ctx || !mle || !out || (n && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: bad argument");
+    if (mle->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_evaluate: the table is a zero-padded view");
     if (!is_pow2(mle->len) || (1ull << n) != mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: point length does not match the table");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
@@ -841,6 +854,7 @@ extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint
 extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t k, dps_mle **out)
 {
     if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: bad argument");
+    if (mle->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_fix_high: the table is a zero-padded view");
     if (!is_pow2(mle->len) || (1ull << k) > mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: too many variables");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
@@ -878,6 +892,7 @@ extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint
 extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t k, dps_mle **out)
 {
     if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: bad argument");
+    if (mle->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_fix_low: the table is a zero-padded view");
     if (!is_pow2(mle->len) || (1ull << k) > mle->len || mle->kind == DPS_I64)
         return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: needs a power-of-two field table and k <= log2(len)");
     if (!canonical(point, 2 * (size_t)k)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: point not canonical");
@@ -931,6 +946,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
 {
     if (!ctx || !tensor || !padded_dims || !unpadded_dims || !kinds || !out || !n_out || n_dims == 0 || n_dims > dpk::AX_MAX_DIMS)
         return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: bad argument");
+    if (tensor->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_partial_eval: the tensor is a zero-padded view");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
     u64 padded_total = 1, contraction = 1, stacked = 1;
@@ -1089,6 +1105,7 @@ struct SessMle {
     u32 nv;              // current number of variables
     u64 *buf0[2], *buf1[2];  // ping-pong scratch, extension limbs
     int next;
+    bool zpad;  // fewer variables than the sum and zero-padded: depends on the low variables, 0 where a higher one is 1
 };
 
 }  // namespace
@@ -1223,6 +1240,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         if (t->kind == DPS_I64 || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
         nv0[k] = log2u(t->len);
         if (nv0[k] > n_vars) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u has %u variables, the sum has %u", k, nv0[k], n_vars);
+        if (t->pad_vars && t->pad_vars != n_vars)
+            return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is zero-padded to %u variables, the sum has %u", k, t->pad_vars, n_vars);
         sc->keep.push_back(t->st);
     }
     for (u32 i = 0; i < n_terms; i++) {
@@ -1287,8 +1306,12 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     // scratch: two ping-pong buffers per table, extension limbs
     size_t scratch_words = 0;
     std::vector<size_t> off_a(n_mles), off_b(n_mles);
+    // a zero-padded table keeps folding after it is down to one entry: both buffers hold at least that entry
+    auto zpad_of = [&](u32 k) { return mles[k]->pad_vars != 0 && nv0[k] < n_vars; };
+    auto len_a = [&](u32 k) { return nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : (zpad_of(k) ? 1ull : 0ull); };
+    auto len_b = [&](u32 k) { return nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : (zpad_of(k) ? 1ull : 0ull); };
     for (u32 k = 0; k < n_mles; k++) {
-        u64 la = nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : 0, lb = nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : 0;
+        u64 la = len_a(k), lb = len_b(k);
         off_a[k] = scratch_words;
         scratch_words += round_up(2 * la, 32);
         off_b[k] = scratch_words;
@@ -1307,7 +1330,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         s.c0 = mles[k]->p0();
         s.c1 = mles[k]->p1();
         s.nv = nv0[k];
-        u64 la = nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : 0, lb = nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : 0;
+        s.zpad = zpad_of(k);
+        u64 la = len_a(k), lb = len_b(k);
         s.buf0[0] = sbase ? sbase + off_a[k] : nullptr;
         s.buf1[0] = s.buf0[0] ? s.buf0[0] + la : nullptr;
         s.buf0[1] = sbase ? sbase + off_b[k] : nullptr;
@@ -1355,8 +1379,21 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             }
             for (u32 k = 0; k < n_mles; k++) {
                 SessMle &s = sim[k];
-                if (s.nv != prev_live || (int)k == sc->fast_eq) continue;
-                dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1)};
+                if ((int)k == sc->fast_eq) continue;
+                if (s.zpad) {
+                    // depends on the low variables: folds in every step, and keeps folding against 0 once it is one entry
+                    const bool single = s.nv == 0;
+                    dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], single ? 1ull : 1ull << (s.nv - 1), single ? 1ull : 0ull};
+                    folds.push_back(d);
+                    folds_extra.push_back(d);
+                    s.c0 = d.d0;
+                    s.c1 = d.d1;
+                    if (!single) s.nv -= 1;
+                    s.next ^= 1;
+                    continue;
+                }
+                if (s.nv != prev_live) continue;
+                dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1), 0};
                 folds.push_back(d);
                 if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
                 s.c0 = d.d0;
@@ -1386,11 +1423,17 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                 dpk::TermDesc td;
                 memset(&td, 0, sizeof td);
                 td.n_factors = t.n_factors;
+                td.n_pairs = 1ull << (live - 1);
                 for (u32 f = 0; f < t.n_factors; f++) {
                     const SessMle &s = sim[t.factors[f]];
                     td.f[f].c0 = s.c0;
                     td.f[f].c1 = s.c1;
-                    if (s.nv >= live) {
+                    if (s.zpad) {
+                        // non-zero only where the higher variables are 0: the first 2^(nv-1) pairs, or entry 0 against 0
+                        td.f[f].pair = s.nv >= 1 ? 1 : 2;
+                        td.f[f].shift = 0;
+                        td.n_pairs = std::min<u64>(td.n_pairs, s.nv >= 1 ? 1ull << (s.nv - 1) : 1ull);
+                    } else if (s.nv >= live) {
                         td.f[f].pair = 1;
                         td.f[f].shift = 0;
                     } else {
@@ -1472,7 +1515,7 @@ int32_t launch_folds(dps_sc *sc, u32 step, bool extra_only, const u64 *chal)
     u32 cnt = extra_only ? sc->fold_extra_cnt[step] : sc->fold_cnt[step];
     if (!cnt) return DPS_OK;
     const dpk::FoldDesc *d = extra_only ? sc->d_fold_extra + sc->fold_extra_off[step] : sc->d_fold + sc->fold_off[step];
-    // every table folding in one step has the same size
+    // the grid is sized for the largest table that can fold in this step; smaller (zero-padded) ones leave blocks idle
     u32 prev_live = sc->n_vars - (step - 1) + 1;
     u64 half = 1ull << (prev_live - 1);
     for (u32 base = 0; base < cnt; base += 65535) {
@@ -1695,7 +1738,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             u32 n = std::min<u32>(sc->n_terms - base, 65535);
             ProfScope ps(ctx, DPS_K_EVAL_TERMS, 0.0);
             dpk::eval_terms_kernel<<<dim3(blocks, n), dpk::BLOCK, 0, ctx->stream>>>(
-                sc->d_terms + sc->term_off[j] + base, n_pairs, sc->d_partial + (size_t)base * blocks * 2 * dpk::MAX_PTS, fa);
+                sc->d_terms + sc->term_off[j] + base, sc->d_partial + (size_t)base * blocks * 2 * dpk::MAX_PTS, fa);
             HIPCHK(ctx, hipGetLastError());
         }
     }
@@ -1818,7 +1861,7 @@ extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uin
     u64 len = cols[0] ? cols[0]->len : 0;
     if (!is_pow2(len) || len < 2) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: column length must be a power of two >= 2");
     for (u32 k = 0; k < n_cols; k++)
-        if (!cols[k] || cols[k]->kind != DPS_BASE || cols[k]->len != len || cols[k]->ctx != ctx)
+        if (!cols[k] || cols[k]->kind != DPS_BASE || cols[k]->len != len || cols[k]->ctx != ctx || cols[k]->pad_vars)
             return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: column %u is not a base table of %llu entries", k, (unsigned long long)len);
     if (numer && (numer->kind != DPS_BASE || numer->len != len)) return fail(ctx, DPS_ERR_INVALID, "dps_logup_build: multiplicity table mismatch");
     std::unique_ptr<dps_logup> lg(new (std::nothrow) dps_logup());

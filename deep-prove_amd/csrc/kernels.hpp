@@ -198,6 +198,7 @@ struct FoldDesc {
     u64 *d0;
     u64 *d1;
     u64 half;  // entries written
+    u64 single;  // 1: the source is one entry s of a zero-padded table (its partner is 0): dst[0] = s (1 - r)
 };
 
 __device__ __forceinline__ E2 fold1(E2 lo, E2 hi, E2 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
@@ -214,6 +215,14 @@ __global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict_
 {
     const FoldDesc d = descs[blockIdx.y];
     const E2 r = gl::e2(r0, r1);
+    if (d.single) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            E2 v = fold1(gl::e2(d.s0[0], d.s1 ? d.s1[0] : 0), gl::e2_zero(), r);
+            d.d0[0] = v.c0;
+            d.d1[0] = v.c1;
+        }
+        return;
+    }
     for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < d.half; i += (u64)gridDim.x * BLOCK) {
         U64x2 a = ld2(d.s0 + 2 * i);
         E2 v;
@@ -391,19 +400,21 @@ struct FactorDesc {
     const u64 *c0;
     const u64 *c1;  // nullptr: base field
     u32 shift;      // broadcast tables: entry index = pair index >> shift
-    u32 pair;       // 1: read entries 2i, 2i+1; 0: broadcast
+    u32 pair;       // 1: read entries 2i, 2i+1; 0: broadcast; 2: entry 0 paired with 0 (a zero-padded table down to one entry)
 };
 
 struct TermDesc {
     u32 n_factors;
     u32 pad;
+    u64 n_pairs;  // pairs on which the product can be non-zero: zero-padded factors cut the range short
     FactorDesc f[DPS_MAX_FACTORS];
 };
 
 // partial sums: out[(term * gridDim.x + block) * 2 * MAX_PTS + 2 * t + limb]
 template <int NF>
-__device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, u64 *__restrict__ partial, u32 *lds)
+__device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 *__restrict__ partial, u32 *lds)
 {
+    const u64 n_pairs = td.n_pairs;
     constexpr int NP = NF + 1;
     E2 acc[NP];
 #pragma unroll
@@ -413,7 +424,10 @@ __device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, 
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             const FactorDesc &fd = td.f[f];
-            if (fd.pair) {
+            if (fd.pair == 2) {
+                cur[f] = tab_get(fd.c0, fd.c1, 0);
+                dl[f] = gl::neg(cur[f]);
+            } else if (fd.pair) {
                 U64x2 a = ld2(fd.c0 + 2 * i);
                 if (fd.c1) {
                     U64x2 b = ld2(fd.c1 + 2 * i);
@@ -452,19 +466,19 @@ __device__ __forceinline__ void eval_term_body(const TermDesc &td, u64 n_pairs, 
 }
 
 __global__ void __launch_bounds__(BLOCK)
-eval_terms_kernel(const TermDesc *__restrict__ terms, u64 n_pairs, u64 *__restrict__ partial, FinArgs fa)
+eval_terms_kernel(const TermDesc *__restrict__ terms, u64 *__restrict__ partial, FinArgs fa)
 {
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * MAX_PTS];
     __shared__ u64 res[2 * MAX_PTS];
     __shared__ int last_flag;
     const TermDesc &td = terms[blockIdx.y];
     switch (td.n_factors) {
-    case 1: eval_term_body<1>(td, n_pairs, partial, lds); break;
-    case 2: eval_term_body<2>(td, n_pairs, partial, lds); break;
-    case 3: eval_term_body<3>(td, n_pairs, partial, lds); break;
-    case 4: eval_term_body<4>(td, n_pairs, partial, lds); break;
-    case 5: eval_term_body<5>(td, n_pairs, partial, lds); break;
-    case 6: eval_term_body<6>(td, n_pairs, partial, lds); break;
+    case 1: eval_term_body<1>(td, partial, lds); break;
+    case 2: eval_term_body<2>(td, partial, lds); break;
+    case 3: eval_term_body<3>(td, partial, lds); break;
+    case 4: eval_term_body<4>(td, partial, lds); break;
+    case 5: eval_term_body<5>(td, partial, lds); break;
+    case 6: eval_term_body<6>(td, partial, lds); break;
     default: break;
     }
     if (take_ticket(fa.counter, fa.total_blocks, &last_flag)) finalize_block<MAX_PTS>(fa, lds, res);

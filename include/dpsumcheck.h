@@ -82,6 +82,13 @@ int32_t dps_tensor_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, dps
 int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, void *d_c1, uint64_t len, dps_mle **out);
 /* SmartSlice::Borrowed: a window [offset, offset + 2^n_vars) sharing storage */
 int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_vars, dps_mle **out);
+/* `src` read by a sumcheck as a table of n_vars variables that is 0 wherever one of
+ * the added (higher) variables is 1: DensePolynomial::zero_pad_num_vars on a view
+ * (zkml/src/poly_commit/prover.rs:214-226).  Nothing is copied or materialised;
+ * the final evaluation dps_sc_finish returns for it is that of the padded table,
+ * src(point_low) * prod (1 - point_high).  n_vars must equal the session's; the
+ * handle is accepted by dps_sc_begin, dps_mle_info, dps_mle_download and dps_mle_free only. */
+int32_t dps_mle_zero_pad(const dps_mle *src, uint32_t n_vars, dps_mle **out);
 int32_t dps_mle_info(const dps_mle *mle, int32_t *kind, uint64_t *len);
 /* copy back; c1 may be NULL for DPS_BASE / DPS_I64 */
 int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *c1);

@@ -259,3 +259,55 @@ def test_config3_shape_mid_size(dp, ctx, orc):
     gpu = [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(r)]
     ref = [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(r)]
     _check_prove(dp, ctx, orc, n, gpu, ref, [(ONE, [2, 0, 1])])
+
+
+def _materialise_zero_pad(tab, n):
+    out = np.zeros((1 << n, 2), dtype=np.uint64)
+    out[: tab.shape[0]] = tab
+    return out
+
+
+ZPAD_SHAPES = [
+    # (n, [(vars, zero-padded?)...], terms)
+    (5, [(5, False), (3, True)], [((1, 0), [0, 1])]),
+    (6, [(6, False), (0, True), (2, True)], [((3, 1), [0, 1]), ((2, 2), [0, 2]), ((5, 0), [1, 2])]),
+    (7, [(4, True), (4, True), (7, False), (3, False)], [((1, 0), [0, 1]), ((9, 4), [0, 2, 3]), ((1, 1), [2])]),
+    (9, [(9, True), (5, True), (1, True), (9, False)], [((1, 0), [0, 3]), ((7, 7), [1, 3]), ((2, 0), [2, 3]), ((3, 3), [1, 2])]),
+    (11, [(11, False), (10, True), (8, True), (11, False), (6, True)], [((1, 0), [0, 1]), ((1, 2), [2, 3]), ((4, 0), [4, 0])]),
+]
+
+
+@pytest.mark.parametrize("case", range(len(ZPAD_SHAPES)))
+def test_zero_padded_views_match_materialised_padding(dp, ctx, orc, case):
+    # DensePolynomial::zero_pad_num_vars (zkml/src/poly_commit/prover.rs:214-226): the GPU reads the short tables in
+    # place; the checker is handed the padded tables written out in full
+    n, tabs_spec, terms = ZPAD_SHAPES[case]
+    terms = [(np.array(c, dtype=np.uint64), f) for c, f in terms]
+    tabs = [rand_e2(1 << m, 9000 + 31 * case + k) for k, (m, _) in enumerate(tabs_spec)]
+    gpu, ref = [], []
+    for t, (m, z) in zip(tabs, tabs_spec):
+        h = ctx.mle_from_ext2(t)
+        gpu.append(h.zero_pad(n) if z else h)
+        ref.append(_materialise_zero_pad(t, n) if z else t)
+    _, point, finals = _check_prove(dp, ctx, orc, n, gpu, ref, terms)
+    # the final evaluation of a padded table is that of the short one times prod (1 - r_high)
+    for k, (m, z) in enumerate(tabs_spec):
+        if z:
+            v = to_E2(orc.mle_evaluate(tabs[k], point[:m]))[0]
+            for r in to_E2(point[m:]):
+                v = v * (E2(1) - r)
+            assert (finals[k] == from_E2([v])[0]).all()
+
+
+def test_zero_pad_errors(dp, ctx):
+    t = ctx.mle_from_ext2(rand_e2(8, 77))
+    with pytest.raises(dp.DpsError):
+        t.zero_pad(2)
+    z = t.zero_pad(5)
+    with pytest.raises(dp.DpsError):
+        z.evaluate(rand_e2(3, 1))
+    with pytest.raises(dp.DpsError):
+        z.view(0, 2)
+    one = np.array([1, 0], dtype=np.uint64)
+    with pytest.raises(dp.DpsError):
+        dp.Session(ctx, 6, [z], [(one, [0])])
