@@ -580,3 +580,53 @@ def logup_batch_verify(instances_meta, is_table, stream, transcript):
     rc = host.dph_logup_batch_verify(n, ncols, nvars, _ptr(cs), _ptr(bs), 1 if is_table else 0, _ptr(stream), stream.shape[0], transcript._t,
                                      _ptr(claims), _ptr(point))
     return rc, claims, point
+
+
+host.dph_claims_batching_prove.restype = _i32
+host.dph_claims_batching_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
+host.dph_claims_batching_verify.restype = _i32
+host.dph_claims_batching_verify.argtypes = [_u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp]
+
+
+def _flat_claims(claims):
+    pts = [np.ascontiguousarray(_e2(p).reshape(-1, 2)) for cls in claims for p, _ in cls]
+    points = np.ascontiguousarray(np.concatenate(pts)) if pts else np.zeros((0, 2), dtype=np.uint64)
+    evals = np.ascontiguousarray(np.stack([_e2(e) for cls in claims for _, e in cls]))
+    return points, evals
+
+
+def claims_batching_prove(ctx, polys, claims, transcript):
+    """Claims-batching sumcheck of the opening proof.  polys: per committed polynomial
+    the list of its chunk tables (Mle); claims: per polynomial a list of (point, eval).
+    Returns (proof[n, 3, 2], point[n, 2], chunk_evals[total_chunks, 2])."""
+    n = len(polys)
+    cpp = (_u32 * n)(*[len(c) for c in polys])
+    flat = [m.handle for c in polys for m in c]
+    chunks = (_vp * len(flat))(*flat)
+    npc = (_u32 * n)(*[len(c) for c in claims])
+    points, evals = _flat_claims(claims)
+    n_vars = max((len(c[0]).bit_length() - 1) for c in polys)
+    proof = np.zeros((n_vars, 3, 2), dtype=np.uint64)
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    out = np.zeros((len(flat), 2), dtype=np.uint64)
+    nv = _u32(0)
+    ctx._chk_host(host.dph_claims_batching_prove(ctx._c, n, cpp, chunks, npc, _ptr(points), _ptr(evals), transcript._t, _ptr(proof), _ptr(point),
+                                                 _ptr(out), C.byref(nv)), "dph_claims_batching_prove")
+    assert nv.value == n_vars
+    return proof, point, out
+
+
+def claims_batching_verify(shapes, claims, proof, chunk_evals, transcript):
+    """shapes: per polynomial (num_chunks, num_vars of the whole polynomial).
+    Returns (status, point); status 0 = accepted."""
+    n = len(shapes)
+    cpp = (_u32 * n)(*[s[0] for s in shapes])
+    pv = (_u32 * n)(*[s[1] for s in shapes])
+    npc = (_u32 * n)(*[len(c) for c in claims])
+    points, evals = _flat_claims(claims)
+    proof = np.ascontiguousarray(_e2(proof))
+    ce = np.ascontiguousarray(_e2(chunk_evals))
+    n_vars = proof.shape[0]
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    rc = host.dph_claims_batching_verify(n, cpp, pv, npc, _ptr(points), _ptr(evals), _ptr(proof), n_vars, _ptr(ce), transcript._t, _ptr(point))
+    return rc, point

@@ -91,6 +91,14 @@ public:
         ctx_->check(dps_mle_view(h_.get(), offset, n_vars, &h), "dps_mle_view");
         return DensePolynomial(*ctx_, h);
     }
+    // as_view() + zero_pad_num_vars(n) (zkml/src/poly_commit/prover.rs:214-226): the same storage, read by a
+    // sumcheck over n variables as 0 wherever an added variable is 1
+    DensePolynomial zero_pad_num_vars(uint32_t n_vars) const
+    {
+        dps_mle *h = nullptr;
+        ctx_->check(dps_mle_zero_pad(h_.get(), n_vars, &h), "dps_mle_zero_pad");
+        return DensePolynomial(*ctx_, h);
+    }
     uint64_t len() const
     {
         uint64_t l = 0;

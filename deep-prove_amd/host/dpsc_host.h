@@ -78,6 +78,22 @@ int32_t dph_logup_batch_verify(uint32_t n_inst, const uint32_t *n_cols, const ui
                                const uint64_t *betas, int32_t is_table, const uint64_t *stream, uint64_t n_elems,
                                dph_transcript *t, uint64_t *claims_out, uint64_t *point_out);
 
+/* Claims-batching sumcheck of the opening proof (zkml/src/poly_commit/prover.rs:140-255).
+ * Polynomial p is held as chunks_per_poly[p] chunk tables (handles in `chunks`, polynomial by
+ * polynomial) and has claims_per_poly[p] claims; `points` holds the claim points one after the
+ * other (2 limbs per coordinate, num_vars(p) coordinates each), `evals` 2 limbs per claim.
+ * Outputs: proof n_vars x 3 elements, point n_vars elements, one evaluation per chunk table. */
+int32_t dph_claims_batching_prove(dps_ctx *ctx, uint32_t n_polys, const uint32_t *chunks_per_poly, const dps_mle *const *chunks,
+                                  const uint32_t *claims_per_poly, const uint64_t *points, const uint64_t *evals,
+                                  dph_transcript *t, uint64_t *proof_out, uint64_t *point_out, uint64_t *evals_out,
+                                  uint32_t *n_vars_out);
+/* Verifier twin (zkml/src/poly_commit/verifier.rs:203-340): poly_vars[p] = variables of the whole
+ * polynomial.  Returns DPS_OK and the opening point when the proof verifies. */
+int32_t dph_claims_batching_verify(uint32_t n_polys, const uint32_t *chunks_per_poly, const uint32_t *poly_vars,
+                                   const uint32_t *claims_per_poly, const uint64_t *points, const uint64_t *evals,
+                                   const uint64_t *proof, uint32_t n_vars, const uint64_t *sumcheck_evals,
+                                   dph_transcript *t, uint64_t *point_out);
+
 #ifdef __cplusplus
 }
 #endif

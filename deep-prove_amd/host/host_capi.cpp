@@ -5,6 +5,7 @@
 
 #include "dpsc/einsum.hpp"
 #include "dpsc/logup.hpp"
+#include "dpsc/poly_commit.hpp"
 #include "dpsc/sumcheck.hpp"
 
 using namespace dpsc;
@@ -272,6 +273,99 @@ int32_t dph_logup_batch_verify(uint32_t n_inst, const uint32_t *n_cols, const ui
         for (size_t i = 0; i < res.point.size(); i++) {
             point_out[2 * i] = res.point[i].c0;
             point_out[2 * i + 1] = res.point[i].c1;
+        }
+    });
+}
+
+namespace {
+
+// claim lists from the flat arrays of the C interface; poly_vars[p] = variables of polynomial p
+std::vector<std::vector<poly_commit::Claim>> read_claims(uint32_t n_polys, const std::vector<size_t> &poly_vars, const uint32_t *claims_per_poly,
+                                                         const uint64_t *points, const uint64_t *evals)
+{
+    std::vector<std::vector<poly_commit::Claim>> claims(n_polys);
+    size_t pw = 0, ci = 0;
+    for (uint32_t p = 0; p < n_polys; p++)
+        for (uint32_t k = 0; k < claims_per_poly[p]; k++) {
+            poly_commit::Claim cl;
+            cl.point = from_limbs(points + pw, poly_vars[p]);
+            pw += 2 * poly_vars[p];
+            cl.eval = F(evals[2 * ci], evals[2 * ci + 1]);
+            ci++;
+            claims[p].push_back(std::move(cl));
+        }
+    return claims;
+}
+
+}  // namespace
+
+int32_t dph_claims_batching_prove(dps_ctx *ctx, uint32_t n_polys, const uint32_t *chunks_per_poly, const dps_mle *const *chunks,
+                                  const uint32_t *claims_per_poly, const uint64_t *points, const uint64_t *evals,
+                                  dph_transcript *t, uint64_t *proof_out, uint64_t *point_out, uint64_t *evals_out,
+                                  uint32_t *n_vars_out)
+{
+    return guarded([&] {
+        Context c(ctx);
+        std::vector<std::unique_ptr<DensePolynomial>> keep;
+        std::vector<poly_commit::CommittedPoly> polys(n_polys);
+        std::vector<size_t> poly_vars(n_polys);
+        size_t k = 0;
+        for (uint32_t p = 0; p < n_polys; p++) {
+            for (uint32_t j = 0; j < chunks_per_poly[p]; j++) {
+                uint64_t len = 0;
+                dps_mle_info(chunks[k], nullptr, &len);
+                dps_mle *v = nullptr;
+                c.check(dps_mle_view(chunks[k], 0, DensePolynomial::log2_strict(len), &v), "dps_mle_view");
+                keep.emplace_back(new DensePolynomial(c, v));
+                polys[p].chunks.push_back(keep.back().get());
+                k++;
+            }
+            if (polys[p].chunks.empty()) throw Error(DPS_ERR_INVALID, "a committed polynomial needs at least one chunk");
+            poly_vars[p] = polys[p].num_vars();
+        }
+        auto claims = read_claims(n_polys, poly_vars, claims_per_poly, points, evals);
+        auto proof = poly_commit::claims_batching_sumcheck(c, polys, claims, t->t);
+        size_t w = 0;
+        for (auto &m : proof.sumcheck_proof.proofs) {
+            if (m.evaluations.size() != 3) throw Error(DPS_ERR_INVALID, "claims batching round message is not degree 2");
+            for (auto &e : m.evaluations) {
+                proof_out[w++] = e.c0;
+                proof_out[w++] = e.c1;
+            }
+        }
+        for (size_t i = 0; i < proof.sumcheck_point.size(); i++) {
+            point_out[2 * i] = proof.sumcheck_point[i].c0;
+            point_out[2 * i + 1] = proof.sumcheck_point[i].c1;
+        }
+        for (size_t i = 0; i < proof.sumcheck_evals.size(); i++) {
+            evals_out[2 * i] = proof.sumcheck_evals[i].c0;
+            evals_out[2 * i + 1] = proof.sumcheck_evals[i].c1;
+        }
+        *n_vars_out = (uint32_t)proof.sumcheck_point.size();
+    });
+}
+
+int32_t dph_claims_batching_verify(uint32_t n_polys, const uint32_t *chunks_per_poly, const uint32_t *poly_vars,
+                                   const uint32_t *claims_per_poly, const uint64_t *points, const uint64_t *evals,
+                                   const uint64_t *proof, uint32_t n_vars, const uint64_t *sumcheck_evals,
+                                   dph_transcript *t, uint64_t *point_out)
+{
+    return guarded([&] {
+        std::vector<poly_commit::CommitmentShape> shapes;
+        std::vector<size_t> pv(n_polys);
+        size_t total_chunks = 0;
+        for (uint32_t p = 0; p < n_polys; p++) {
+            shapes.push_back(poly_commit::CommitmentShape{chunks_per_poly[p], poly_vars[p]});
+            pv[p] = poly_vars[p];
+            total_chunks += chunks_per_poly[p];
+        }
+        auto claims = read_claims(n_polys, pv, claims_per_poly, points, evals);
+        IOPProof pr;
+        for (uint32_t j = 0; j < n_vars; j++) pr.proofs.push_back(IOPProverMessage{from_limbs(proof + 6 * (size_t)j, 3)});
+        auto point = poly_commit::claims_batching_verify(shapes, claims, pr, from_limbs(sumcheck_evals, total_chunks), t->t);
+        for (size_t i = 0; i < point.size(); i++) {
+            point_out[2 * i] = point[i].c0;
+            point_out[2 * i + 1] = point[i].c1;
         }
     });
 }

@@ -431,5 +431,107 @@ def logup_batch_verify(instances_meta, is_table, stream, transcript):
     return rc, claims, point
 
 
+# ---- claims-batching sumcheck of the opening proof ----
+# Follows zkml/src/poly_commit/prover.rs:140-255 (prover), mod.rs:46-68,95-159 (chunk
+# coefficients, eq point, expression) and verifier.rs:203-340 (verifier).  The
+# zero-padded views the reference takes (prover.rs:214-226) are written out in full
+# here, straight from their definition: entries beyond the table's length are 0.
+def _pow_e2(x, k):
+    out = e2(1)
+    for _ in range(k):
+        out = e2_mul(out, x)
+    return out
+
+
+def chunk_batching_coefficients(num_chunks, point):
+    """mod.rs:46-58: C_c = identity_eval(point[-b:], bits_le(c)), b = log2(num_chunks)."""
+    point = _e2arr(point).reshape(-1, 2)
+    b = num_chunks.bit_length() - 1
+    assert 1 << b == num_chunks
+    coords = point[len(point) - b:]
+    out = []
+    for c in range(num_chunks):
+        bits = np.array([[(c >> j) & 1, 0] for j in range(b)], dtype=np.uint64).reshape(-1, 2)
+        out.append(identity_eval(coords, bits) if b else e2(1))
+    return out
+
+
+def _claims_batching_terms(polys_chunks, claims, challenge):
+    """mod.rs:95-159 flattened: one product chal^k * C_c * chunk_c * eq_k per (claim, chunk)."""
+    eq_offset = sum(polys_chunks)
+    terms, k, base = [], 0, 0
+    for nch, cls in zip(polys_chunks, claims):
+        for point, _ in cls:
+            ck = _pow_e2(challenge, k)
+            for c, coeff in enumerate(chunk_batching_coefficients(nch, point)):
+                terms.append((e2_mul(ck, coeff), [base + c, eq_offset + k]))
+            k += 1
+        base += nch
+    return terms
+
+
+def claims_batching_prove(polys, claims, transcript):
+    """polys: per committed polynomial, the list of its chunk tables ((2^m, 2) arrays);
+    claims: per polynomial, a list of (point, eval).  Returns (proof, point, chunk_evals)."""
+    chunk_tabs, eq_tabs = [], []
+    max_vars = 0
+    for chunks, cls in zip(polys, claims):
+        nch = len(chunks)
+        b = nch.bit_length() - 1
+        for point, ev in cls:
+            point = _e2arr(point).reshape(-1, 2)
+            transcript.append_scalars(_e2arr(ev).reshape(1, 2))
+            eq_tabs.append(eq_evals(point[: len(point) - b]))
+        chunk_tabs.extend(_e2arr(c).reshape(-1, 2) for c in chunks)
+        max_vars = max(max_vars, _nvars(_e2arr(chunks[0]).reshape(-1, 2)))
+
+    def padded(t):
+        out = np.zeros((1 << max_vars, 2), dtype=np.uint64)
+        out[: t.shape[0]] = t
+        return out
+
+    tables = [padded(t) for t in chunk_tabs + eq_tabs]
+    challenge = transcript.append_and_sample(b"model_batching")
+    terms = _claims_batching_terms([len(c) for c in polys], claims, challenge)
+    proof, point, finals = sc_prove(max_vars, tables, terms, transcript)
+    return proof, point, finals[: len(chunk_tabs)]
+
+
+def claims_batching_verify(shapes, claims, proof, chunk_evals, transcript):
+    """shapes: per polynomial (num_chunks, num_vars of the whole polynomial).
+    Returns (ok, point)."""
+    eq_points, evals = [], []
+    max_vars = 0
+    for (nch, nv), cls in zip(shapes, claims):
+        b = nch.bit_length() - 1
+        for point, ev in cls:
+            point = _e2arr(point).reshape(-1, 2)
+            transcript.append_scalars(_e2arr(ev).reshape(1, 2))
+            eq_points.append(point[: len(point) - b])
+            evals.append(_e2arr(ev))
+        max_vars = max(max_vars, nv - b)
+    challenge = transcript.append_and_sample(b"model_batching")
+    claimed, acc = e2(0), e2(1)
+    for ev in evals:
+        claimed = e2_add(claimed, e2_mul(acc, ev))
+        acc = e2_mul(acc, challenge)
+    proof = _e2arr(proof)
+    if proof.shape[0] != max_vars or proof.shape[1] != 3:
+        return False, None
+    bad, point, expected = sc_verify(claimed, proof, transcript)
+    if bad:
+        return False, point
+    wit = [_e2arr(v) for v in _e2arr(chunk_evals).reshape(-1, 2)]
+    for ep in eq_points:
+        v = identity_eval(point[: len(ep)], ep) if len(ep) else e2(1)
+        for r in point[len(ep):]:
+            v = e2_mul(v, e2_sub(e2(1), r))
+        wit.append(v)
+    total = e2(0)
+    for coeff, (a, b_) in _claims_batching_terms([s[0] for s in shapes], claims, challenge):
+        total = e2_add(total, e2_mul(coeff, e2_mul(wit[a], wit[b_])))
+    return bool((total == expected).all()), point
+
+
 def num_threads():
     return lib().orc_num_threads()
