@@ -630,3 +630,34 @@ def claims_batching_verify(shapes, claims, proof, chunk_evals, transcript):
     point = np.zeros((n_vars, 2), dtype=np.uint64)
     rc = host.dph_claims_batching_verify(n, cpp, pv, npc, _ptr(points), _ptr(evals), _ptr(proof), n_vars, _ptr(ce), transcript._t, _ptr(point))
     return rc, point
+
+
+host.dph_same_poly_prove.restype = _i32
+host.dph_same_poly_prove.argtypes = [_vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp]
+host.dph_same_poly_verify.restype = _i32
+host.dph_same_poly_verify.argtypes = [_u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp]
+
+
+def same_poly_prove(ctx, poly, claims, transcript):
+    """same_poly::Prover: claims is a list of (point, eval) on the table `poly`.
+    Returns (proof[n, 3, 2], point[n, 2], eval[2])."""
+    n_vars = len(poly).bit_length() - 1
+    points = np.ascontiguousarray(np.stack([_e2(p).reshape(n_vars, 2) for p, _ in claims]))
+    evals = np.ascontiguousarray(np.stack([_e2(e) for _, e in claims]))
+    proof = np.zeros((n_vars, 3, 2), dtype=np.uint64)
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    ev = np.zeros(2, dtype=np.uint64)
+    ctx._chk_host(host.dph_same_poly_prove(ctx._c, poly.handle, len(claims), _ptr(points), _ptr(evals), transcript._t, _ptr(proof), _ptr(point),
+                                           _ptr(ev)), "dph_same_poly_prove")
+    return proof, point, ev
+
+
+def same_poly_verify(n_vars, claims, proof, ev, transcript):
+    """same_poly::Verifier.  Returns (status, point); status 0 = accepted."""
+    points = np.ascontiguousarray(np.stack([_e2(p).reshape(n_vars, 2) for p, _ in claims]))
+    evals = np.ascontiguousarray(np.stack([_e2(e) for _, e in claims]))
+    proof = np.ascontiguousarray(_e2(proof))
+    ev = np.ascontiguousarray(_e2(ev))
+    point = np.zeros((n_vars, 2), dtype=np.uint64)
+    rc = host.dph_same_poly_verify(n_vars, len(claims), _ptr(points), _ptr(evals), _ptr(proof), _ptr(ev), transcript._t, _ptr(point))
+    return rc, point

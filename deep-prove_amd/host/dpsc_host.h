@@ -94,6 +94,15 @@ int32_t dph_claims_batching_verify(uint32_t n_polys, const uint32_t *chunks_per_
                                    const uint64_t *proof, uint32_t n_vars, const uint64_t *sumcheck_evals,
                                    dph_transcript *t, uint64_t *point_out);
 
+/* same_poly::Prover::prove (zkml/src/iop/same_poly.rs:84-114): n_claims claims (points of
+ * num_vars(poly) coordinates, 2 limbs each; evals 2 limbs each) on one polynomial.
+ * Outputs: proof num_vars x 3 elements, the merged claim's point and evaluation. */
+int32_t dph_same_poly_prove(dps_ctx *ctx, const dps_mle *poly, uint32_t n_claims, const uint64_t *points, const uint64_t *evals,
+                            dph_transcript *t, uint64_t *proof_out, uint64_t *point_out, uint64_t *eval_out);
+/* same_poly::Verifier::verify (same_poly.rs:140-169); DPS_OK when the proof verifies */
+int32_t dph_same_poly_verify(uint32_t num_vars, uint32_t n_claims, const uint64_t *points, const uint64_t *evals, const uint64_t *proof,
+                             const uint64_t *eval, dph_transcript *t, uint64_t *point_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,6 +6,7 @@
 #include "dpsc/einsum.hpp"
 #include "dpsc/logup.hpp"
 #include "dpsc/poly_commit.hpp"
+#include "dpsc/same_poly.hpp"
 #include "dpsc/sumcheck.hpp"
 
 using namespace dpsc;
@@ -366,6 +367,57 @@ int32_t dph_claims_batching_verify(uint32_t n_polys, const uint32_t *chunks_per_
         for (size_t i = 0; i < point.size(); i++) {
             point_out[2 * i] = point[i].c0;
             point_out[2 * i + 1] = point[i].c1;
+        }
+    });
+}
+
+int32_t dph_same_poly_prove(dps_ctx *ctx, const dps_mle *poly, uint32_t n_claims, const uint64_t *points, const uint64_t *evals,
+                            dph_transcript *t, uint64_t *proof_out, uint64_t *point_out, uint64_t *eval_out)
+{
+    return guarded([&] {
+        Context c(ctx);
+        uint64_t len = 0;
+        dps_mle_info(poly, nullptr, &len);
+        const uint32_t nv = DensePolynomial::log2_strict(len);
+        dps_mle *v = nullptr;
+        c.check(dps_mle_view(poly, 0, nv, &v), "dps_mle_view");
+        DensePolynomial p(c, v);
+        same_poly::Prover prover(p);
+        for (uint32_t i = 0; i < n_claims; i++)
+            prover.add_claim(same_poly::Claim{from_limbs(points + 2 * (size_t)nv * i, nv), F(evals[2 * i], evals[2 * i + 1])});
+        auto res = prover.prove(t->t);
+        size_t w = 0;
+        for (auto &m : res.first.sumcheck.proofs) {
+            if (m.evaluations.size() != 3) throw Error(DPS_ERR_INVALID, "same_poly round message is not degree 2");
+            for (auto &e : m.evaluations) {
+                proof_out[w++] = e.c0;
+                proof_out[w++] = e.c1;
+            }
+        }
+        for (size_t i = 0; i < res.second.point.size(); i++) {
+            point_out[2 * i] = res.second.point[i].c0;
+            point_out[2 * i + 1] = res.second.point[i].c1;
+        }
+        eval_out[0] = res.second.eval.c0;
+        eval_out[1] = res.second.eval.c1;
+    });
+}
+
+int32_t dph_same_poly_verify(uint32_t num_vars, uint32_t n_claims, const uint64_t *points, const uint64_t *evals, const uint64_t *proof,
+                             const uint64_t *eval, dph_transcript *t, uint64_t *point_out)
+{
+    return guarded([&] {
+        same_poly::Context sctx(num_vars);
+        same_poly::Verifier verifier(sctx);
+        for (uint32_t i = 0; i < n_claims; i++)
+            verifier.add_claim(same_poly::Claim{from_limbs(points + 2 * (size_t)num_vars * i, num_vars), F(evals[2 * i], evals[2 * i + 1])});
+        same_poly::Proof pr;
+        for (uint32_t j = 0; j < num_vars; j++) pr.sumcheck.proofs.push_back(IOPProverMessage{from_limbs(proof + 6 * (size_t)j, 3)});
+        pr.eval = F(eval[0], eval[1]);
+        auto claim = verifier.verify(pr, t->t);
+        for (size_t i = 0; i < claim.point.size(); i++) {
+            point_out[2 * i] = claim.point[i].c0;
+            point_out[2 * i + 1] = claim.point[i].c1;
         }
     });
 }

@@ -533,5 +533,34 @@ def claims_batching_verify(shapes, claims, proof, chunk_evals, transcript):
     return bool((total == expected).all()), point
 
 
+# ---- merging claims on one polynomial (zkml/src/iop/same_poly.rs:84-169) ----
+def same_poly_prove(poly, claims, transcript):
+    """claims: list of (point, eval).  Returns (proof, point, eval)."""
+    poly = _e2arr(poly).reshape(-1, 2)
+    a = transcript.read_challenges(len(claims))
+    tables = [poly] + [eq_evals(p) for p, _ in claims]
+    terms = [(a[i], [0, 1 + i]) for i in range(len(claims))]
+    proof, point, finals = sc_prove(_nvars(poly), tables, terms, transcript)
+    return proof, point, finals[0]
+
+
+def same_poly_verify(num_vars, claims, proof, eval_, transcript):
+    """Returns (ok, point)."""
+    a = transcript.read_challenges(len(claims))
+    y = e2(0)
+    for (_, ev), ai in zip(claims, a):
+        y = e2_add(y, e2_mul(_e2arr(ev), ai))
+    proof = _e2arr(proof)
+    if proof.shape[0] != num_vars or proof.shape[1] != 3:
+        return False, None
+    bad, point, expected = sc_verify(y, proof, transcript)
+    if bad:
+        return False, point
+    computed = e2(0)
+    for (pt, _), ai in zip(claims, a):
+        computed = e2_add(computed, e2_mul(ai, identity_eval(pt, point)))
+    return bool((e2_mul(_e2arr(eval_), computed) == expected).all()), point
+
+
 def num_threads():
     return lib().orc_num_threads()

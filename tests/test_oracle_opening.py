@@ -53,3 +53,24 @@ def test_claims_batching_round_trip(orc, chunk_vars):
     bad_proof = proof.copy()
     bad_proof[n - 1, 2, 1] ^= np.uint64(2)
     assert not orc.claims_batching_verify(shapes, claims, bad_proof, evals, orc.OracleTranscript(b"commit test"))[0]
+
+
+def test_same_poly_round_trip(orc):
+    # zkml/src/iop/same_poly.rs:190-229 (test_same_poly_proof): 14 claims on a 10-variable polynomial; the merged
+    # claim must be a true evaluation of the polynomial
+    n, k = 10, 14
+    poly = rand_e2(1 << n, 321)
+    claims = []
+    for i in range(k):
+        pt = rand_e2(n, 400 + i)
+        claims.append((pt, orc.mle_evaluate(poly, pt)))
+    tr = orc.OracleTranscript()
+    proof, point, ev = orc.same_poly_prove(poly, claims, tr)
+    assert (ev == orc.mle_evaluate(poly, point)).all()
+    vt = orc.OracleTranscript()
+    ok, vpoint = orc.same_poly_verify(n, claims, proof, ev, vt)
+    assert ok and (vpoint == point).all() and vt.state() == tr.state()
+    bad = [(p, e) for p, e in claims]
+    bad[5] = (bad[5][0], orc.e2_add(bad[5][1], orc.e2(1)))
+    assert not orc.same_poly_verify(n, bad, proof, ev, orc.OracleTranscript())[0]
+    assert not orc.same_poly_verify(n, claims, proof, orc.e2_add(ev, orc.e2(0, 1)), orc.OracleTranscript())[0]
