@@ -1151,6 +1151,14 @@ struct dps_sc {
     std::vector<dpk::ProdArgs> fast_args;  // per round
     std::vector<u32> fast_nb;              // base-field sources per round
     u32 max_blocks;
+    // fused multi-term path: groups of at most POLY_MAXT tables, one grid row each
+    bool poly;
+    std::vector<std::vector<u32>> poly_tabs;  // per group: session table indices, in slot order
+    std::vector<u32> poly_term_begin, poly_term_end;
+    std::vector<int> poly_owner;              // per session table: the group that writes its fold, -1 = in no group
+    u32 poly_max_tabs;                        // sizes the kernel's LDS
+    dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
+    dpk::PolyTerm *d_poly_terms;
 };
 
 namespace {
@@ -1210,6 +1218,36 @@ int32_t launch_prod_dispatch(dps_ctx *ctx, u32 nf, u32 nb, bool eq, bool fold, c
     PK(1, 0, true) PK(1, 1, true) PK(2, 0, true) PK(2, 1, true) PK(2, 2, true)
 #undef PK
     return fail(ctx, DPS_ERR_UNSUPPORTED, "no product kernel for %u tables, %u base, eq %d", nf, nb, (int)eq);
+}
+
+template <int NF>
+void launch_poly(dps_ctx *ctx, bool eq, bool skip1, const dpk::PolyArgs &a, dim3 grid, size_t lds, u64 *partial, const dpk::FastFin &ff)
+{
+    if (eq && skip1)
+        dpk::poly_kernel<NF, true, true><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
+    else if (eq)
+        dpk::poly_kernel<NF, true, false><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
+    else if (skip1)
+        dpk::poly_kernel<NF, false, true><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
+    else
+        dpk::poly_kernel<NF, false, false><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
+}
+
+int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dpk::PolyArgs &a, dim3 grid, u32 max_tabs, u64 *partial,
+                             const dpk::FastFin &ff)
+{
+    // value and slope of every table of a group, per thread
+    const size_t lds = (size_t)std::max<u32>(max_tabs, 1) * 4 * dpk::BLOCK * 8;
+    switch (nf) {
+    case 1: launch_poly<1>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    case 2: launch_poly<2>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    case 3: launch_poly<3>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    case 4: launch_poly<4>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    case 5: launch_poly<5>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    case 6: launch_poly<6>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
+    default: return fail(ctx, DPS_ERR_UNSUPPORTED, "no fused kernel for degree %u", nf);
+    }
+    return DPS_OK;
 }
 
 u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
@@ -1300,6 +1338,112 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         }
     }
 
+    // fused multi-term path: every table of every term is either full-size or constant in the low variables
+    sc->poly = false;
+    sc->poly_max_tabs = 0;
+    sc->d_poly_groups = nullptr;
+    sc->d_poly_terms = nullptr;
+    std::vector<dpk::PolyTerm> poly_terms;
+    if (!sc->fast && sc->n_terms >= 1 && n_vars >= 1) {
+        bool ok = true;
+        for (const dps_term &t : sc->terms)
+            for (u32 f = 0; f < t.n_factors; f++)
+                if (mles[t.factors[f]]->pad_vars && nv0[t.factors[f]] < n_vars) ok = false;
+        // an eq table that is a factor of every term exactly once comes out in closed form
+        int eq = -1;
+        if (ok) {
+            const dps_term &t0 = sc->terms[0];
+            for (u32 f = 0; f < t0.n_factors && eq < 0; f++) {
+                const u32 k = t0.factors[f];
+                const dps_mle *h = mles[k];
+                if (!(h->eq && h->eq->m == n_vars && h->kind == DPS_EXT2 && nv0[k] == n_vars)) continue;
+                bool all = true;
+                u32 inner = 0;
+                for (const dps_term &t : sc->terms) {
+                    u32 cnt = 0;
+                    for (u32 q = 0; q < t.n_factors; q++) cnt += t.factors[q] == k;
+                    if (cnt != 1) all = false;
+                    inner = std::max(inner, t.n_factors - 1);
+                }
+                if (all && inner >= 1) eq = (int)k;
+            }
+        }
+        u32 nf = 0;
+        for (const dps_term &t : sc->terms) nf = std::max(nf, eq >= 0 ? t.n_factors - 1 : t.n_factors);
+        if (nf < 1 || nf > 6) ok = false;
+        // terms in order, a new group whenever the tables no longer fit
+        std::vector<std::vector<u32>> groups;
+        std::vector<u32> tb, te;
+        if (ok) {
+            std::vector<u32> cur;
+            u32 begin = 0;
+            for (u32 ti = 0; ti < sc->n_terms && ok; ti++) {
+                const dps_term &t = sc->terms[ti];
+                std::vector<u32> need;
+                for (u32 f = 0; f < t.n_factors; f++) {
+                    const u32 k = t.factors[f];
+                    if ((int)k == eq) continue;
+                    if (std::find(need.begin(), need.end(), k) == need.end()) need.push_back(k);
+                }
+                if (need.size() > (size_t)dpk::POLY_MAXT) {
+                    ok = false;
+                    break;
+                }
+                std::vector<u32> merged = cur;
+                for (u32 k : need)
+                    if (std::find(merged.begin(), merged.end(), k) == merged.end()) merged.push_back(k);
+                if (merged.size() > (size_t)dpk::POLY_MAXT) {
+                    groups.push_back(cur);
+                    tb.push_back(begin);
+                    te.push_back(ti);
+                    begin = ti;
+                    merged = need;
+                }
+                cur = merged;
+            }
+            if (ok) {
+                groups.push_back(cur);
+                tb.push_back(begin);
+                te.push_back(sc->n_terms);
+            }
+        }
+        if (ok && groups.size() <= 65535) {
+            sc->poly = true;
+            sc->poly_tabs = groups;
+            sc->poly_term_begin = tb;
+            sc->poly_term_end = te;
+            sc->poly_owner.assign(n_mles, -1);
+            for (size_t g = 0; g < groups.size(); g++) {
+                sc->poly_max_tabs = std::max<u32>(sc->poly_max_tabs, (u32)groups[g].size());
+                for (u32 k : groups[g])
+                    if (sc->poly_owner[k] < 0) sc->poly_owner[k] = (int)g;
+            }
+            sc->fast_nf = nf;
+            sc->fast_coeff = gl::e2_one();
+            if (eq >= 0) {
+                sc->fast_eq = eq;
+                sc->eq_info = mles[eq]->eq;
+                sc->eq_c0 = mles[eq]->p0();
+                sc->eq_c1 = mles[eq]->p1();
+            }
+            for (size_t g = 0; g < groups.size(); g++)
+                for (u32 ti = tb[g]; ti < te[g]; ti++) {
+                    const dps_term &t = sc->terms[ti];
+                    dpk::PolyTerm pt;
+                    memset(&pt, 0, sizeof pt);
+                    pt.c0 = t.coeff[0];
+                    pt.c1 = t.coeff[1];
+                    pt.w = gl::mul_small(t.coeff[1], (u32)gl::W);
+                    for (u32 f = 0; f < t.n_factors; f++) {
+                        if ((int)t.factors[f] == eq) continue;
+                        const auto &gt = groups[g];
+                        pt.slot[pt.n_factors++] = (uint8_t)(std::find(gt.begin(), gt.end(), t.factors[f]) - gt.begin());
+                    }
+                    poly_terms.push_back(pt);
+                }
+        }
+    }
+
     // the last rounds run in one resident workgroup when every registered table belongs to the term
     if (sc->fast && n_vars >= 11 && n_mles == sc->terms[0].n_factors) sc->tail_j0 = n_vars - 8;  // 2^8 = TAIL_PAIRS pairs
 
@@ -1344,6 +1488,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     std::vector<dpk::TermDesc> tdescs;
     std::vector<SessMle> sim = sc->m;
     auto in_fast = [&](u32 k) {
+        if (sc->poly) return sc->poly_owner[k] >= 0;
         if (!sc->fast) return false;
         for (u32 f = 0; f < sc->fast_nf; f++)
             if (sc->fast_order[f] == k) return true;
@@ -1356,7 +1501,11 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->term_off.assign(n_vars + 2, 0);
     sc->fast_args.resize(n_vars + 2);
     sc->fast_nb.assign(n_vars + 2, 0);
+    std::vector<dpk::PolyGroup> poly_groups;  // [round][group]
+    std::vector<const u64 *> pre0(n_mles), pre1(n_mles);
+    std::vector<char> folded(n_mles);
     for (u32 j = 1; j <= n_vars + 1; j++) {
+        std::fill(folded.begin(), folded.end(), 0);
         // step j starts by folding, with the challenge of round j-1, the tables that were live-sized then
         if (j >= 2) {
             u32 prev_live = n_vars - (j - 1) + 1;
@@ -1396,6 +1545,9 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                 dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1), 0};
                 folds.push_back(d);
                 if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
+                pre0[k] = s.c0;
+                pre1[k] = s.c1;
+                folded[k] = 1;
                 s.c0 = d.d0;
                 s.c1 = d.d1;
                 s.nv -= 1;
@@ -1416,7 +1568,42 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             pa.n_pairs = 1ull << (n_vars - 1);
             sc->fast_nb[1] = nb;
         }
-        if (j <= n_vars && !sc->fast) {
+        if (j <= n_vars && sc->poly) {
+            const u32 live = n_vars - j + 1;
+            for (size_t g = 0; g < sc->poly_tabs.size(); g++) {
+                dpk::PolyGroup pg;
+                memset(&pg, 0, sizeof pg);
+                pg.n_tabs = (u32)sc->poly_tabs[g].size();
+                pg.term_begin = sc->poly_term_begin[g];
+                pg.term_end = sc->poly_term_end[g];
+                for (u32 sl = 0; sl < pg.n_tabs; sl++) {
+                    const u32 k = sc->poly_tabs[g][sl];
+                    const SessMle &s = sim[k];
+                    dpk::PolyTab &tb = pg.tab[sl];
+                    if (folded[k]) {
+                        // folds with the previous challenge on the way in; the owning group writes the result
+                        tb.mode = dpk::POLY_PAIR_FOLD;
+                        tb.s0 = pre0[k];
+                        tb.s1 = pre1[k];
+                        if (sc->poly_owner[k] == (int)g) {
+                            tb.d0 = const_cast<u64 *>(s.c0);
+                            tb.d1 = const_cast<u64 *>(s.c1);
+                        }
+                    } else if (s.nv >= live) {
+                        tb.mode = dpk::POLY_PAIR;
+                        tb.s0 = s.c0;
+                        tb.s1 = s.c1;
+                    } else {
+                        tb.mode = dpk::POLY_BCAST;
+                        tb.s0 = s.c0;
+                        tb.s1 = s.c1;
+                        tb.shift = live - 1 - s.nv;
+                    }
+                }
+                poly_groups.push_back(pg);
+            }
+        }
+        if (j <= n_vars && !sc->fast && !sc->poly) {
             u32 live = n_vars - j + 1;
             sc->term_off[j] = (u32)tdescs.size();
             for (const dps_term &t : sc->terms) {
@@ -1458,7 +1645,9 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     size_t bytes_gath = round_up(gath.size() * sizeof(dpk::GatherDesc), 256);
     size_t bytes_partial = round_up((size_t)std::max<u32>(sc->n_terms, 1) * sc->max_blocks * 2 * dpk::MAX_PTS * 8, 256);
     size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256) + 256;
-    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_partial + bytes_result;
+    size_t bytes_pg = round_up(poly_groups.size() * sizeof(dpk::PolyGroup), 256);
+    size_t bytes_pt = round_up(poly_terms.size() * sizeof(dpk::PolyTerm), 256);
+    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_partial + bytes_result;
     int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
     if (rc != DPS_OK) return cleanup(rc);
     char *p = (char *)sc->dev_block;
@@ -1472,12 +1661,16 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     p += bytes_fin;
     sc->d_gather = (dpk::GatherDesc *)p;
     p += bytes_gath;
+    sc->d_poly_groups = (dpk::PolyGroup *)p;
+    p += bytes_pg;
+    sc->d_poly_terms = (dpk::PolyTerm *)p;
+    p += bytes_pt;
     sc->d_partial = (u64 *)p;
     p += bytes_partial;
     sc->d_result = (u64 *)p;
     sc->d_counter = ctx->d_counter;
     // one staged upload of all descriptors
-    std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath, 0);
+    std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt, 0);
     char *q = stage.data();
     if (!folds.empty()) memcpy(q, folds.data(), folds.size() * sizeof(dpk::FoldDesc));
     q += bytes_fold;
@@ -1488,6 +1681,10 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     if (!fins.empty()) memcpy(q, fins.data(), fins.size() * sizeof(dpk::FinTerm));
     q += bytes_fin;
     if (!gath.empty()) memcpy(q, gath.data(), gath.size() * sizeof(dpk::GatherDesc));
+    q += bytes_gath;
+    if (!poly_groups.empty()) memcpy(q, poly_groups.data(), poly_groups.size() * sizeof(dpk::PolyGroup));
+    q += bytes_pg;
+    if (!poly_terms.empty()) memcpy(q, poly_terms.data(), poly_terms.size() * sizeof(dpk::PolyTerm));
     // a product session that ends in the resident kernel reads none of the descriptors
     const bool needs_descs = !(sc->fast && sc->tail_j0);
     if (!stage.empty() && needs_descs) {
@@ -1601,7 +1798,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         ProfScope ps(ctx, DPS_K_FINALIZE, 0.0);
         dpk::finalize_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(fa);
         HIPCHK(ctx, hipGetLastError());
-    } else if (sc->fast) {
+    } else if (sc->fast || sc->poly) {
         dpk::ProdArgs a = sc->fast_args[j];
         const bool has_eq = sc->fast_eq >= 0;
         const u32 nf = sc->fast_nf;
@@ -1722,6 +1919,29 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             sc->round = j;
             return DPS_OK;
         }
+        if (sc->poly) {
+            dpk::PolyArgs pa;
+            const u32 n_groups = (u32)sc->poly_tabs.size();
+            pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
+            pa.terms = sc->d_poly_terms;
+            pa.q0 = a.q0;
+            pa.q1 = a.q1;
+            pa.n_pairs = n_pairs;
+            pa.r0 = a.r0;
+            pa.r1 = a.r1;
+            ff.n_blocks = blocks * n_groups;
+            double pbytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
+            for (u32 k = 0; k < sc->n_mles; k++)
+                if (sc->poly_owner[k] >= 0) pbytes += (double)n_pairs * (j >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
+            ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
+            CHK(launch_poly_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(blocks, n_groups), sc->poly_max_tabs, sc->d_partial, ff));
+            HIPCHK(ctx, hipGetLastError());
+            CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
+            sc->last_msg.resize(sc->degree + 1);
+            for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
+            sc->round = j;
+            return DPS_OK;
+        }
         double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
         for (u32 f = 0; f < nf; f++) {
             double eb = a.s1[f] ? 16.0 : 8.0;
@@ -1788,7 +2008,7 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         sc->finished = true;
         return DPS_OK;
     }
-    if (sc->n_vars >= 1) CHK(launch_folds(sc, sc->n_vars + 1, sc->fast, challenge));
+    if (sc->n_vars >= 1) CHK(launch_folds(sc, sc->n_vars + 1, sc->fast || sc->poly, challenge));
     if (sc->n_mles) {
         if (2 * (size_t)sc->n_mles > ctx->res_off - 64) return fail(ctx, DPS_ERR_UNSUPPORTED, "too many tables in one session");
         dpk::gather_kernel<<<(sc->n_mles + 63) / 64, 64, 0, ctx->stream>>>(sc->d_gather, sc->n_mles, ctx->d_pinned);

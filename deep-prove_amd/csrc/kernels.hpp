@@ -980,6 +980,195 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
     if (threadIdx.x == 0) publish_words(a.out_host, HOST_FINALS_SLOT, res, 2 * NF, fin_seq);
 }
 
+// ---------------------------------------------------------------------------
+// fused kernel for sums of several product terms over shared tables
+//
+// A group is up to POLY_MAXT tables and the terms made of them.  Per pair a
+// thread loads every table of the group once (folding it with the previous
+// challenge on the way, and writing the folded pair when this group owns the
+// table), keeps value and slope of every table in LDS (the terms pick their
+// factors by index, which registers cannot do), and evaluates
+//     G(t) = sum_terms coeff * prod_factors table(t)
+// at t = 0..NF with the coefficients applied here, so one set of running sums
+// serves all terms.  An eq factor common to all terms is taken out in closed
+// form exactly as in prod_kernel (G is then the polynomial without it), and
+// t = 1 is skipped when the claim is known.  Output and finish are those of
+// prod_kernel: per-workgroup sums of G(t) (times R), then fast_finalize.
+// Groups are grid rows; their partials are simply added.
+// ---------------------------------------------------------------------------
+constexpr int POLY_MAXT = 7;
+constexpr u32 POLY_PAIR = 0, POLY_PAIR_FOLD = 1, POLY_BCAST = 2;
+
+struct PolyTab {
+    const u64 *s0;
+    const u64 *s1;  // nullptr: base-field source
+    u64 *d0;        // POLY_PAIR_FOLD: where the folded table goes; nullptr: another group writes it
+    u64 *d1;
+    u32 mode;
+    u32 shift;      // POLY_BCAST: entry index = pair index >> shift
+};
+
+struct PolyGroup {
+    PolyTab tab[POLY_MAXT];
+    u32 n_tabs;
+    u32 term_begin, term_end;
+    u32 pad;
+};
+
+struct PolyTerm {
+    u64 c0, c1, w;  // coefficient, prepared (w = 7 c1)
+    u32 n_factors;
+    uint8_t slot[DPS_MAX_FACTORS];  // table slots within the group
+    u32 pad;
+};
+
+struct PolyArgs {
+    const PolyGroup *groups;  // one per grid row, this round's
+    const PolyTerm *terms;
+    const u64 *q0;  // eq suffix table of this round (common eq factor only)
+    const u64 *q1;
+    u64 n_pairs;
+    u64 r0, r1;
+};
+
+template <int NF, bool EQ, bool SKIP1>
+__global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict__ partial, FastFin ff)
+{
+    constexpr int NP = NF + 1;
+    extern __shared__ u64 dyn[];  // [n_tabs][4][BLOCK]: value c0, c1, slope c0, c1
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
+    __shared__ u64 res[6 * MAX_PTS];
+    __shared__ int last_flag;
+    const PolyGroup &g = a.groups[blockIdx.y];
+    const u32 n_tabs = g.n_tabs;
+    const E2 r = gl::e2(a.r0, a.r1);
+    const gl::E2P rp = gl::prep(r);
+    const u32 tid = threadIdx.x;
+    auto cur0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 0) * BLOCK + tid]; };
+    auto cur1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 1) * BLOCK + tid]; };
+    auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
+    auto dl1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 3) * BLOCK + tid]; };
+
+    gl::E2Acc lz[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) lz[t] = gl::e2acc_zero();
+
+    for (u64 i = (u64)blockIdx.x * BLOCK + tid; i < a.n_pairs; i += (u64)gridDim.x * BLOCK) {
+        // all loads of the step first (statically indexed registers), then the arithmetic
+        U64x2 a0[POLY_MAXT], b0[POLY_MAXT], a1[POLY_MAXT], b1[POLY_MAXT];
+#pragma unroll
+        for (int k = 0; k < POLY_MAXT; k++) {
+            if ((u32)k < n_tabs) {
+                const PolyTab &tb = g.tab[k];
+                a0[k] = b0[k] = a1[k] = b1[k] = U64x2{0, 0};
+                if (tb.mode == POLY_PAIR_FOLD) {
+                    a0[k] = ld2(tb.s0 + 4 * i);
+                    b0[k] = ld2(tb.s0 + 4 * i + 2);
+                    if (tb.s1) {
+                        a1[k] = ld2(tb.s1 + 4 * i);
+                        b1[k] = ld2(tb.s1 + 4 * i + 2);
+                    }
+                } else if (tb.mode == POLY_PAIR) {
+                    a0[k] = ld2(tb.s0 + 2 * i);
+                    if (tb.s1) a1[k] = ld2(tb.s1 + 2 * i);
+                } else {
+                    const u64 e = i >> tb.shift;
+                    a0[k].x = tb.s0[e];
+                    if (tb.s1) a1[k].x = tb.s1[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < POLY_MAXT; k++) {
+            if ((u32)k < n_tabs) {
+                const PolyTab &tb = g.tab[k];
+                E2 lo, hi;
+                if (tb.mode == POLY_PAIR_FOLD) {
+                    if (tb.s1) {
+                        lo = fold1p(gl::e2(a0[k].x, a1[k].x), gl::e2(a0[k].y, a1[k].y), rp);
+                        hi = fold1p(gl::e2(b0[k].x, b1[k].x), gl::e2(b0[k].y, b1[k].y), rp);
+                    } else {
+                        lo = fold1_base(a0[k].x, a0[k].y, r);
+                        hi = fold1_base(b0[k].x, b0[k].y, r);
+                    }
+                    if (tb.d0) {
+                        st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
+                        st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
+                    }
+                } else if (tb.mode == POLY_PAIR) {
+                    lo = gl::e2(a0[k].x, a1[k].x);
+                    hi = gl::e2(a0[k].y, a1[k].y);
+                } else {
+                    lo = hi = gl::e2(a0[k].x, a1[k].x);
+                }
+                const E2 d = gl::sub(hi, lo);
+                cur0(k) = lo.c0;
+                cur1(k) = lo.c1;
+                dl0(k) = d.c0;
+                dl1(k) = d.c1;
+            }
+        }
+        gl::E2P restp = gl::prep(gl::e2_one());
+        if (EQ) restp = gl::prep(gl::e2(a.q0[i], a.q1[i]));
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            if (!(t == 1 && SKIP1)) {
+                gl::E2Acc G = gl::e2acc_zero();
+                for (u32 j = g.term_begin; j < g.term_end; j++) {
+                    const PolyTerm &tm = a.terms[j];
+                    E2 prod = gl::e2_one();
+                    if (tm.n_factors > 0) {
+                        const u32 s0 = tm.slot[0];
+                        prod = gl::e2(cur0(s0), cur1(s0));
+                        for (u32 f = 1; f < tm.n_factors; f++) {
+                            const u32 sl = tm.slot[f];
+                            prod = gl::mulp(prod, gl::prep(gl::e2(cur0(sl), cur1(sl))));
+                        }
+                    }
+                    gl::E2P cp;
+                    cp.c0 = tm.c0;
+                    cp.c1 = tm.c1;
+                    cp.w = tm.w;
+                    gl::acc_mul(G, prod, cp);
+                }
+                const E2 gsum = gl::acc_reduce(G);
+                if (EQ)
+                    gl::acc_mul(lz[t], gsum, restp);
+                else
+                    gl::acc_e2(lz[t], gsum);
+            }
+            if (t + 1 < NP) {
+                // on to t + 1 (the slope is added even when t = 1 is skipped: t = 2 needs it twice)
+                for (u32 k = 0; k < n_tabs; k++) {
+                    cur0(k) = gl::add(cur0(k), dl0(k));
+                    cur1(k) = gl::add(cur1(k), dl1(k));
+                }
+            }
+        }
+    }
+    E2 acc[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
+    block_reduce<NP>(acc, lds);
+    if (gridDim.x * gridDim.y == 1) {
+        fast_finalize<NF>(ff, acc, res);
+        return;
+    }
+    if (tid == 0) {
+        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            st_agent(o + 2 * t, acc[t].c0);
+            st_agent(o + 2 * t + 1, acc[t].c1);
+        }
+    }
+    if (take_ticket(ff.counter, gridDim.x * gridDim.y, &last_flag)) {
+        E2 q[NP];
+        gather_partials<NP>(ff, lds, q);
+        fast_finalize<NF>(ff, q, res);
+    }
+}
+
 // final evaluations: entry 0 of every table after the last fold
 struct GatherDesc {
     const u64 *c0;
