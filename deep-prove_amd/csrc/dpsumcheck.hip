@@ -1159,6 +1159,9 @@ struct dps_sc {
     u32 poly_max_tabs;                        // sizes the kernel's LDS
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
+    std::vector<dpk::PolyGroup> h_poly_groups;  // host copies: a single group travels in the kernel arguments
+    std::vector<dpk::PolyTerm> h_poly_terms;
+    std::vector<char> stage;                  // descriptor upload in flight (no wait at set-up)
 };
 
 namespace {
@@ -1237,7 +1240,7 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
                              const dpk::FastFin &ff)
 {
     // value and slope of every table of a group, per thread
-    const size_t lds = (size_t)std::max<u32>(max_tabs, 1) * 4 * dpk::BLOCK * 8;
+    const size_t lds = (size_t)std::max<u32>(max_tabs, 1) * 4 * dpk::BLOCK * 8;  // + 2.3 KB of static LDS in the kernel
     switch (nf) {
     case 1: launch_poly<1>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
     case 2: launch_poly<2>(ctx, eq, skip1, a, grid, lds, partial, ff); break;
@@ -1670,7 +1673,10 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->d_result = (u64 *)p;
     sc->d_counter = ctx->d_counter;
     // one staged upload of all descriptors
-    std::vector<char> stage(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt, 0);
+    std::vector<char> &stage = sc->stage;  // lives as long as the session: the upload is not waited for
+    stage.assign(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt, 0);
+    sc->h_poly_groups = poly_groups;
+    sc->h_poly_terms = poly_terms;
     char *q = stage.data();
     if (!folds.empty()) memcpy(q, folds.data(), folds.size() * sizeof(dpk::FoldDesc));
     q += bytes_fold;
@@ -1689,8 +1695,6 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     const bool needs_descs = !(sc->fast && sc->tail_j0);
     if (!stage.empty() && needs_descs) {
         hipError_t e = hipMemcpyAsync(sc->dev_block, stage.data(), stage.size(), hipMemcpyHostToDevice, ctx->stream);
-        // the staging vector dies with this call
-        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) return cleanup(fail(ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e)));
     }
     *out = sc.release();
@@ -1924,6 +1928,11 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u32 n_groups = (u32)sc->poly_tabs.size();
             pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
             pa.terms = sc->d_poly_terms;
+            if (n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS) {
+                pa.groups = nullptr;
+                pa.g0 = sc->h_poly_groups[j - 1];
+                std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+            }
             pa.q0 = a.q0;
             pa.q1 = a.q1;
             pa.n_pairs = n_pairs;

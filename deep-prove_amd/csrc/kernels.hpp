@@ -997,6 +997,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
 // Groups are grid rows; their partials are simply added.
 // ---------------------------------------------------------------------------
 constexpr int POLY_MAXT = 7;
+constexpr int POLY_LDS_TERMS = 48;  // terms of a group kept in LDS; further ones are read from device memory
 constexpr u32 POLY_PAIR = 0, POLY_PAIR_FOLD = 1, POLY_BCAST = 2;
 
 struct PolyTab {
@@ -1021,10 +1022,13 @@ struct PolyTerm {
     uint8_t slot[DPS_MAX_FACTORS];  // table slots within the group
     u32 pad;
 };
+static_assert(sizeof(PolyTerm) % 8 == 0 && sizeof(PolyGroup) % 8 == 0, "descriptors are copied as 64-bit words");
 
 struct PolyArgs {
-    const PolyGroup *groups;  // one per grid row, this round's
+    const PolyGroup *groups;  // one per grid row, this round's; nullptr: the single group and its terms are in g0 / t0
     const PolyTerm *terms;
+    PolyGroup g0;
+    PolyTerm t0[POLY_LDS_TERMS];
     const u64 *q0;  // eq suffix table of this round (common eq factor only)
     const u64 *q1;
     u64 n_pairs;
@@ -1039,11 +1043,28 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
-    const PolyGroup &g = a.groups[blockIdx.y];
+    // The group's descriptors come from device memory; read from there inside the loops every use would be
+    // a dependent load of its own (the small rounds are nothing but such latencies), so they are staged in LDS once.
+    __shared__ PolyGroup g;
+    __shared__ PolyTerm lterms[POLY_LDS_TERMS];
+    const u32 tid = threadIdx.x;
+    {
+        const bool inl = a.groups == nullptr;  // a single group handed over in the kernel arguments
+        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + blockIdx.y);
+        u64 *dst = reinterpret_cast<u64 *>(&g);
+        for (u32 w = tid; w < sizeof(PolyGroup) / 8; w += BLOCK) dst[w] = src[w];
+        __syncthreads();
+        const u32 nt = g.term_end - g.term_begin;
+        const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
+        const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
+        u64 *td = reinterpret_cast<u64 *>(lterms);
+        for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        __syncthreads();
+    }
     const u32 n_tabs = g.n_tabs;
+    const u32 n_terms = g.term_end - g.term_begin;
     const E2 r = gl::e2(a.r0, a.r1);
     const gl::E2P rp = gl::prep(r);
-    const u32 tid = threadIdx.x;
     auto cur0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 0) * BLOCK + tid]; };
     auto cur1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 1) * BLOCK + tid]; };
     auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
@@ -1114,8 +1135,8 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         for (int t = 0; t < NP; t++) {
             if (!(t == 1 && SKIP1)) {
                 gl::E2Acc G = gl::e2acc_zero();
-                for (u32 j = g.term_begin; j < g.term_end; j++) {
-                    const PolyTerm &tm = a.terms[j];
+                for (u32 j = 0; j < n_terms; j++) {
+                    const PolyTerm &tm = j < (u32)POLY_LDS_TERMS ? lterms[j] : a.terms[g.term_begin + j];
                     E2 prod = gl::e2_one();
                     if (tm.n_factors > 0) {
                         const u32 s0 = tm.slot[0];
