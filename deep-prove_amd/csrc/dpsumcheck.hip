@@ -1871,8 +1871,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         ff.out_host = fa.out_host;
         ff.seq = fa.seq;
         ff.counter = sc->d_counter;
-        if (sc->tail_j0 && j >= sc->tail_j0) {
-            // mail for the resident kernel: challenge, scales, claim; then the sequence number it waits for
+        // mail for a resident kernel: challenge, scales, claim; then the sequence number it waits for
+        auto post_mail = [&]() {
             u64 *mb = mailbox(ctx);
             mb[dpk::MAIL_R] = a.r0;
             mb[dpk::MAIL_R + 1] = a.r1;
@@ -1888,6 +1888,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             mb[dpk::MAIL_CONST + 1] = cst.c1;
             mb[dpk::MAIL_SKIP1] = a.skip1;
             send_mail(ctx, fa.seq);
+        };
+        if (sc->tail_j0 && j >= sc->tail_j0) {
+            post_mail();
             if (j == sc->tail_j0) {
                 dpk::TailArgs ta;
                 memset(&ta, 0, sizeof ta);
@@ -1924,6 +1927,32 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             return DPS_OK;
         }
         if (sc->poly) {
+            auto took_round = [&]() {
+                sc->last_msg.resize(sc->degree + 1);
+                for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
+                sc->round = j;
+            };
+            if (sc->tail_running) {
+                if (a.skip1) {
+                    // the resident launch of an earlier round runs this one
+                    post_mail();
+                    int32_t rc = wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
+                    if (rc != DPS_OK || j == sc->n_vars) {
+                        // it exits by itself after the last round
+                        sc->tail_running = false;
+                        ctx->tail_owner = nullptr;
+                    }
+                    CHK(rc);
+                    took_round();
+                    return DPS_OK;
+                }
+                // evaluating t = 1 after all is not compiled into the resident variant: end it and launch normally
+                __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
+                HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+                __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
+                sc->tail_running = false;
+                ctx->tail_owner = nullptr;
+            }
             dpk::PolyArgs pa;
             const u32 n_groups = (u32)sc->poly_tabs.size();
             pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
@@ -1938,6 +1967,20 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.n_pairs = n_pairs;
             pa.r0 = a.r0;
             pa.r1 = a.r1;
+            pa.j = j;
+            pa.last_round = 0;
+            pa.n_vars = sc->n_vars;
+            pa.spin_limit = 4000000;
+            pa.eq0 = sc->eq_c0;
+            pa.eq1 = sc->eq_c1;
+            pa.mail = ctx->d_pinned + (ctx->res_off - 64);
+            pa.seq = fa.seq;
+            // a single workgroup from here on: it stays for the remaining rounds
+            const bool reside = n_groups == 1 && blocks == 1 && a.skip1 && j < sc->n_vars;
+            if (reside) {
+                pa.groups = sc->d_poly_groups + (size_t)(j - 1);
+                pa.last_round = sc->n_vars;
+            }
             ff.n_blocks = blocks * n_groups;
             double pbytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
             for (u32 k = 0; k < sc->n_mles; k++)
@@ -1945,10 +1988,13 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
             CHK(launch_poly_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(blocks, n_groups), sc->poly_max_tabs, sc->d_partial, ff));
             HIPCHK(ctx, hipGetLastError());
+            if (reside) {
+                sc->tail_running = true;
+                sc->tail_seq0 = fa.seq;
+                ctx->tail_owner = sc;
+            }
             CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
-            sc->last_msg.resize(sc->degree + 1);
-            for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
-            sc->round = j;
+            took_round();
             return DPS_OK;
         }
         double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;

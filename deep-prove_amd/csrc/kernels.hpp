@@ -835,13 +835,13 @@ struct TailArgs {
 // the host link) fetches the whole mail; it is accepted when the sequence number
 // matches and the check word agrees with the payload, which makes a torn read
 // (the host still writing) look like no mail yet.  Returns false on abort or timeout.
-__device__ __forceinline__ bool tail_wait_mail(const TailArgs &a, u64 want, u64 *box, int *ok_lds)
+__device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, u64 want, u64 *box, int *ok_lds)
 {
     if (threadIdx.x < WAVE) {
         const u32 l = threadIdx.x;
         int ok = 0;
-        for (u32 spins = 0; spins < a.spin_limit; spins++) {
-            const u64 w = l < (u32)MAIL_WORDS ? ld_sys(a.mail + l) : 0;
+        for (u32 spins = 0; spins < spin_limit; spins++) {
+            const u64 w = l < (u32)MAIL_WORDS ? ld_sys(mail + l) : 0;
             u64 x = mail_mix(w, l);
 #pragma unroll
             for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
@@ -875,7 +875,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
     u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
     bool to_ping = true;  // destination of this round's folded tables
     for (u32 j = a.j0; j <= a.n_vars; j++) {
-        if (!tail_wait_mail(a, a.seq0 + (j - a.j0), box, &ok_flag)) return;
+        if (!tail_wait_mail(a.mail, a.spin_limit, a.seq0 + (j - a.j0), box, &ok_flag)) return;
         const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
         const gl::E2P rp = gl::prep(r);
         const bool skip1 = box[MAIL_SKIP1] != 0;
@@ -965,7 +965,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
     }
     // final evaluations: the last challenge folds the two remaining entries of every table
     const u64 fin_seq = a.seq0 + (a.n_vars - a.j0 + 1);
-    if (!tail_wait_mail(a, fin_seq, box, &ok_flag)) return;
+    if (!tail_wait_mail(a.mail, a.spin_limit, fin_seq, box, &ok_flag)) return;
     if (threadIdx.x < NF) {
         const int f = threadIdx.x;
         const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
@@ -1033,6 +1033,17 @@ struct PolyArgs {
     const u64 *q1;
     u64 n_pairs;
     u64 r0, r1;
+    // Resident rounds (single-workgroup launches only): after round j the workgroup stays, waits for the next
+    // challenge in the host's mailbox as tail_kernel does, and runs the following rounds up to last_round on the
+    // tables it folded itself.  `groups` then holds one descriptor per round, starting with this launch's.
+    u32 j;           // this launch's round (1-based)
+    u32 last_round;  // 0: exit after round j
+    u32 n_vars;
+    u32 spin_limit;
+    const u64 *eq0;  // eq storage, level 0 at entry 0 (common eq factor only)
+    const u64 *eq1;
+    const u64 *mail;
+    u64 seq;         // sequence number of round j; round j + k waits for mail seq + k
 };
 
 template <int NF, bool EQ, bool SKIP1>
@@ -1047,10 +1058,22 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     // a dependent load of its own (the small rounds are nothing but such latencies), so they are staged in LDS once.
     __shared__ PolyGroup g;
     __shared__ PolyTerm lterms[POLY_LDS_TERMS];
+    __shared__ u64 box[MAIL_WORDS];
+    __shared__ int ok_flag;
     const u32 tid = threadIdx.x;
+    auto cur0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 0) * BLOCK + tid]; };
+    auto cur1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 1) * BLOCK + tid]; };
+    auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
+    auto dl1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 3) * BLOCK + tid]; };
+    u32 j = a.j;
+    u64 n_pairs = a.n_pairs;
+    E2 r = gl::e2(a.r0, a.r1);
+    const u64 *q0 = a.q0, *q1 = a.q1;
+    FastFin cf = ff;
+  for (;;) {
     {
         const bool inl = a.groups == nullptr;  // a single group handed over in the kernel arguments
-        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + blockIdx.y);
+        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + (j - a.j) + blockIdx.y);
         u64 *dst = reinterpret_cast<u64 *>(&g);
         for (u32 w = tid; w < sizeof(PolyGroup) / 8; w += BLOCK) dst[w] = src[w];
         __syncthreads();
@@ -1058,23 +1081,19 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
         const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
         u64 *td = reinterpret_cast<u64 *>(lterms);
-        for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        if (j == a.j)
+            for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
         __syncthreads();
     }
     const u32 n_tabs = g.n_tabs;
     const u32 n_terms = g.term_end - g.term_begin;
-    const E2 r = gl::e2(a.r0, a.r1);
     const gl::E2P rp = gl::prep(r);
-    auto cur0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 0) * BLOCK + tid]; };
-    auto cur1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 1) * BLOCK + tid]; };
-    auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
-    auto dl1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 3) * BLOCK + tid]; };
 
     gl::E2Acc lz[NP];
 #pragma unroll
     for (int t = 0; t < NP; t++) lz[t] = gl::e2acc_zero();
 
-    for (u64 i = (u64)blockIdx.x * BLOCK + tid; i < a.n_pairs; i += (u64)gridDim.x * BLOCK) {
+    for (u64 i = (u64)blockIdx.x * BLOCK + tid; i < n_pairs; i += (u64)gridDim.x * BLOCK) {
         // all loads of the step first (statically indexed registers), then the arithmetic
         U64x2 a0[POLY_MAXT], b0[POLY_MAXT], a1[POLY_MAXT], b1[POLY_MAXT];
 #pragma unroll
@@ -1130,7 +1149,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
             }
         }
         gl::E2P restp = gl::prep(gl::e2_one());
-        if (EQ) restp = gl::prep(gl::e2(a.q0[i], a.q1[i]));
+        if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
 #pragma unroll
         for (int t = 0; t < NP; t++) {
             if (!(t == 1 && SKIP1)) {
@@ -1172,8 +1191,37 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
-        fast_finalize<NF>(ff, acc, res);
-        return;
+        fast_finalize<NF>(cf, acc, res);
+        if (a.last_round == 0 || j >= a.last_round) return;
+        // stay for the next round: its challenge and the scalars of its message arrive by mail
+        j++;
+        if (!tail_wait_mail(a.mail, a.spin_limit, a.seq + (j - a.j), box, &ok_flag)) return;
+        // a run-time switch to evaluating t = 1 is not compiled in: the host ends the residency instead
+        if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
+        r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+        n_pairs >>= 1;
+        if (EQ) {
+            const u64 off = (2ull << a.n_vars) - (2ull << (a.n_vars - j));
+            q0 = a.eq0 + off;
+            q1 = a.eq1 + off;
+        }
+#pragma unroll
+        for (int k = 0; k < 2 * MAX_PTS; k++) {
+            cf.scale[k] = box[MAIL_SCALE + k];
+            cf.cext[k] = box[MAIL_CEXT + k];
+        }
+        cf.k0 = box[MAIL_K];
+        cf.k1 = box[MAIL_K + 1];
+        cf.claim0 = box[MAIL_CLAIM];
+        cf.claim1 = box[MAIL_CLAIM + 1];
+        cf.const0 = box[MAIL_CONST];
+        cf.const1 = box[MAIL_CONST + 1];
+        cf.seq = a.seq + (j - a.j);
+        // the tables this workgroup folded and stored are read back by other lanes: stores done, then no stale L1 lines
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        continue;
     }
     if (tid == 0) {
         u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
@@ -1188,6 +1236,8 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         gather_partials<NP>(ff, lds, q);
         fast_finalize<NF>(ff, q, res);
     }
+    return;
+  }
 }
 
 // final evaluations: entry 0 of every table after the last fold
