@@ -36,6 +36,127 @@ def rand_base(n, seed):
     return np.where(v >= np.uint64(P), v - np.uint64(P), v)
 
 
+def _timed(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    ts = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        out = fn()
+        ts.append(time.perf_counter() - t0)
+    return 1e3 * sum(ts) / len(ts), 1e3 * min(ts), out
+
+
+def rand_i64(shape, seed):
+    return np.random.Generator(np.random.PCG64(seed)).integers(-2048, 2048, size=shape, dtype=np.int64)
+
+
+def other_config(args):
+    """The remaining configurations, one JSON line each: a step is one complete proof of that configuration
+    (tables resident in HBM where the interface takes handles; the einsum driver takes host tensors, so its
+    step includes their upload).  The CPU leg times the checker on the same statement where it has a driver."""
+    dp = importlib.import_module("deep-prove_amd")
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    orc = None
+    if not args.no_cpu:
+        import dpsc_oracle as orc
+
+        orc.select(True)
+    ctx = dp.Context(0)
+    one = np.array([1, 0], dtype=np.uint64)
+    cfg = args.config
+    cpu_ms, exact, extra = None, None, {}
+    if cfg == "1":
+        n = 16
+        f, g = rand_base(1 << n, 1), rand_base(1 << n, 2)
+        mf, mg = ctx.mle_from_base(f), ctx.mle_from_base(g)
+        terms = [(one, [0, 1])]
+        run = lambda: ctx.sumcheck_prove(n, [mf, mg], terms, dp.Transcript(b"bench"))
+        workload, metric = "cfg1: sum f*g, n=16, base field, degree 2", "sumcheck prove ms @ n=16 deg-2 base"
+        if orc:
+            tabs = [orc.embed_base(f), orc.embed_base(g)]
+            cpu_ms, _, ref = _timed(lambda: orc.sc_prove(n, tabs, terms, orc.OracleTranscript(b"bench")), 5, 1)
+            got = run()
+            exact = bool(all((a == b).all() for a, b in zip(got, ref)))
+    elif cfg in ("2", "4"):
+        if cfg == "2":
+            ops, lhs, rhs = [("ik", "kj", "ij")], rand_i64((512, 768), 11), [rand_i64((768, 3072), 12)]
+            workload, metric = "cfg2: A[512x768] @ W[768x3072], partial evaluation + 10-variable degree-2 sumcheck", "einsum prove ms (gpt2 mlp up-projection)"
+            nv_out = 9 + 12
+        else:
+            ops, lhs, rhs = [("hsd", "htd", "hst")], rand_i64((8, 512, 256), 13), [rand_i64((8, 512, 256), 14)]
+            workload, metric = "cfg4: Q,K[8x512x256] 'hsd,htd->hst', partial evaluation + 8-variable sumcheck over 16 tables", "einsum prove ms (attention scores)"
+            nv_out = 3 + 9 + 9
+        pt = np.stack([rand_base(nv_out, 5), rand_base(nv_out, 6)], axis=-1)
+        claims = [(pt, one)]  # timing only: the claimed value does not change the work
+        run = lambda: dp.einsum_prove(ctx, ops, lhs, rhs, claims, dp.Transcript(b"bench"))
+        extra["note"] = "the step includes the upload of the int64 tensors (the driver takes host tensors)"
+    elif cfg == "5":
+        log_l, log_t = 22, 16
+        rng = np.random.Generator(np.random.PCG64(600))
+        t_in = np.arange(1 << log_t, dtype=np.uint64)
+        t_out = (t_in * np.uint64(40503) + np.uint64(17)) & np.uint64(0xFFFF)
+        idx = rng.integers(0, 1 << log_t, size=1 << log_l)
+        mult = np.bincount(idx, minlength=1 << log_t).astype(np.uint64)
+        tr0 = dp.Transcript(b"bench")
+        c, beta = tr0.append_and_sample(b"c"), tr0.append_and_sample(b"beta")
+        look_cols = [t_in[idx], t_out[idx]]
+        look_d = [dict(cols=[ctx.mle_from_base(x) for x in look_cols], numer=None, c=c, beta=beta)]
+        tab_d = [dict(cols=[ctx.mle_from_base(t_in), ctx.mle_from_base(t_out)], numer=ctx.mle_from_base(mult), c=c, beta=beta)]
+
+        def run():
+            t = tr0.clone()
+            return dp.logup_batch_prove(ctx, look_d, t), dp.logup_batch_prove(ctx, tab_d, t)
+
+        workload = "cfg5: LogUp-GKR, 2^22 lookups (2 columns) into a 2^16-entry table with multiplicities; lookup batch + table batch"
+        metric = "logup-gkr prove ms @ 2^22 lookups"
+        if orc:
+            def cpu():
+                t = orc.OracleTranscript(b"bench")
+                t.append_and_sample(b"c"), t.append_and_sample(b"beta")
+                return (orc.logup_batch_prove([dict(cols=look_cols, numer=None, c=c, beta=beta)], t),
+                        orc.logup_batch_prove([dict(cols=[t_in, t_out], numer=mult, c=c, beta=beta)], t))
+
+            cpu_ms, _, ref = _timed(cpu, 1, 0)
+            got = run()
+            exact = bool((got[0] == ref[0]).all() and (got[1] == ref[1]).all())
+    else:
+        # the reference's test_poly_commit shape with chunks of 2^10 (zkml/src/poly_commit/mod.rs:224-409)
+        rng = np.random.Generator(np.random.PCG64(77))
+        sizes = [int(x) for x in rng.integers(10, 16, size=5)] + [int(x) for x in rng.integers(10, 14, size=9)]
+        polys_h, polys_d, claims = [], [], []
+        for i, nv in enumerate(sizes):
+            full = np.stack([rand_base(1 << nv, 100 + i), rand_base(1 << nv, 200 + i)], axis=-1)
+            m = min(nv, 10)
+            chunks = [full[k << m:(k + 1) << m] for k in range(1 << (nv - m))]
+            whole = ctx.mle_from_ext2(full)
+            polys_h.append(chunks)
+            polys_d.append([whole.view(k << m, m) for k in range(len(chunks))])
+            cls = []
+            for k in range(2 if (i < 5 and i % 2) else 1):
+                pt = np.stack([rand_base(nv, 300 + 10 * i + k), rand_base(nv, 400 + 10 * i + k)], axis=-1)
+                cls.append((pt, whole.evaluate(pt)))
+            claims.append(cls)
+        run = lambda: dp.claims_batching_prove(ctx, polys_d, claims, dp.Transcript(b"bench"))
+        workload = "claims-batching sumcheck of the opening proof: 14 polynomials of 10..15 variables in chunks of 2^10, 16 claims"
+        metric = "claims batching prove ms"
+        if orc:
+            cpu_ms, _, ref = _timed(lambda: orc.claims_batching_prove(polys_h, claims, orc.OracleTranscript(b"bench")), 3, 1)
+            got = run()
+            exact = bool(all((a == b).all() for a, b in zip(got, ref)))
+    ms, best, _ = _timed(run, args.steps, args.warmup)
+    out = {"metric": metric, "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(ms, 4), "min_step_ms": round(best, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "u64 (Goldilocks, ext2)", "data": "synthetic", "config": {"workload": workload}}
+    out.update(extra)
+    if cpu_ms is not None:
+        out["cpu_baseline"] = {"value": round(cpu_ms, 2), "unit": "ms", "cores": orc.num_threads(), "kind": "port",
+                               "sample": "the same statement, whole; C restatement with OpenMP"}
+        out["speedup_vs_cpu"] = round(cpu_ms / ms, 1)
+        out["bit_exact"] = exact
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -43,10 +164,15 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--nvars", type=int, default=24, help="variables of the sum (24 is the benchmark configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--config", default="3", choices=["1", "2", "3", "4", "5", "opening"],
+                    help="3 (default) is the benchmark configuration; the others time the remaining configurations the same way")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
+    if args.config != "3":
+        print(json.dumps(other_config(args)))
+        return
 
     dp = importlib.import_module("deep-prove_amd")
     n = args.nvars
