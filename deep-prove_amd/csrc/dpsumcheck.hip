@@ -959,7 +959,11 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         if (kinds[a] == DPS_AXIS_CONTRACTED) contraction *= unpadded_dims[a];
         if (kinds[a] == DPS_AXIS_STACKED) stacked *= unpadded_dims[a];
     }
-    if (padded_total > tensor->len) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: tensor shorter than its padded shape");
+    // the tensor is stored in its padded shape, or compactly in its unpadded shape (told apart by its length)
+    u64 unpadded_total = 1;
+    for (u32 a = 0; a < n_dims; a++) unpadded_total *= unpadded_dims[a];
+    const bool compact = tensor->len == unpadded_total && unpadded_total != padded_total;
+    if (!compact && padded_total > tensor->len) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: tensor shorter than its padded shape");
     if (stacked > out_cap) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: %llu tables do not fit out_cap", (unsigned long long)stacked);
 
     // current tensor: dims (unpadded sizes of the axes still present) and element strides
@@ -970,7 +974,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         u64 s = 1;
         for (int a = (int)n_dims - 1; a >= 0; a--) {
             strides[a] = s;
-            s *= padded_dims[a];
+            s *= compact ? unpadded_dims[a] : padded_dims[a];
             orig[a] = a;
         }
     }

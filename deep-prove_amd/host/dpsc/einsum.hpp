@@ -21,10 +21,13 @@ struct Claim {
 // A quantised tensor: row-major int64 values in the padded shape, resident on the GPU.
 struct Tensor {
     std::vector<uint64_t> padded_shape, unpadded_shape;
-    std::vector<int64_t> host;  // padded data (zeros outside the unpadded region)
-    DensePolynomial device;     // raw int64 tensor handle
+    const int64_t *data = nullptr;  // the caller's unpadded row-major values (borrowed)
+    uint64_t count = 0;
+    DensePolynomial device;         // raw int64 tensor on the device, stored compactly (unpadded)
 
-    static Tensor from_unpadded(const Context &ctx, const std::vector<int64_t> &data, const std::vector<uint64_t> &shape)
+    // The tensor goes to the device as it is: padding and the embedding into the field happen in the kernels
+    // that read it (einsum/prove.rs:66-94 materialises a padded Tensor<F> instead).
+    static Tensor from_unpadded(const Context &ctx, const int64_t *data, uint64_t n, const std::vector<uint64_t> &shape)
     {
         Tensor t;
         t.unpadded_shape = shape;
@@ -33,25 +36,37 @@ struct Tensor {
             while (p < d) p <<= 1;
             t.padded_shape.push_back(p);
         }
-        uint64_t total = 1, utotal = 1;
-        for (auto d : t.padded_shape) total *= d;
+        uint64_t utotal = 1;
         for (auto d : shape) utotal *= d;
-        if (data.size() != utotal) throw Error(DPS_ERR_INVALID, "Tensor: data does not match the shape");
-        t.host.assign(total, 0);
-        std::vector<uint64_t> idx(shape.size(), 0);
-        for (uint64_t flat = 0; flat < utotal; flat++) {
+        if (n != utotal) throw Error(DPS_ERR_INVALID, "Tensor: data does not match the shape");
+        t.data = data;
+        t.count = n;
+        dps_mle *h = nullptr;
+        ctx.check(dps_tensor_from_i64(ctx.raw(), data, n, &h), "dps_tensor_from_i64");
+        t.device = DensePolynomial(ctx, h);
+        return t;
+    }
+    static Tensor from_unpadded(const Context &ctx, const std::vector<int64_t> &data, const std::vector<uint64_t> &shape)
+    {
+        return from_unpadded(ctx, data.data(), data.size(), shape);
+    }
+    // padded row-major copy (zeros outside the unpadded region); only the aggregation sumcheck needs it
+    std::vector<int64_t> padded_host() const
+    {
+        uint64_t total = 1;
+        for (auto d : padded_shape) total *= d;
+        std::vector<int64_t> host(total, 0);
+        std::vector<uint64_t> idx(unpadded_shape.size(), 0);
+        for (uint64_t flat = 0; flat < count; flat++) {
             uint64_t dst = 0;
-            for (size_t a = 0; a < shape.size(); a++) dst = dst * t.padded_shape[a] + idx[a];
-            t.host[dst] = data[flat];
-            for (size_t a = shape.size(); a-- > 0;) {
-                if (++idx[a] < shape[a]) break;
+            for (size_t a = 0; a < unpadded_shape.size(); a++) dst = dst * padded_shape[a] + idx[a];
+            host[dst] = data[flat];
+            for (size_t a = unpadded_shape.size(); a-- > 0;) {
+                if (++idx[a] < unpadded_shape[a]) break;
                 idx[a] = 0;
             }
         }
-        dps_mle *h = nullptr;
-        ctx.check(dps_tensor_from_i64(ctx.raw(), t.host.data(), t.host.size(), &h), "dps_tensor_from_i64");
-        t.device = DensePolynomial(ctx, h);
-        return t;
+        return host;
     }
 };
 
@@ -262,7 +277,7 @@ inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> 
     Claim lhs_claim;
     if (R > 1) {
         // prove.rs:260-302: aggregate the R claims on the LHS with a second sumcheck
-        DensePolynomial input_mle = DensePolynomial::from_i64(ctx, lhs.host);
+        DensePolynomial input_mle = DensePolynomial::from_i64(ctx, lhs.padded_host());
         const uint32_t nv = input_mle.num_vars();
         std::vector<DensePolynomial> eq_polys;
         for (size_t r = 0; r < R; r++)

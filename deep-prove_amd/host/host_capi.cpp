@@ -138,11 +138,10 @@ int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels
         std::vector<einsum::Op> ops;
         std::vector<einsum::Tensor> rts;
         std::vector<einsum::Claim> claims;
-        einsum::Tensor lt = einsum::Tensor::from_unpadded(c, std::vector<int64_t>(lhs, lhs + count(lhs_shape, lhs_rank)),
-                                                          std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
+        einsum::Tensor lt = einsum::Tensor::from_unpadded(c, lhs, count(lhs_shape, lhs_rank), std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
         for (uint32_t r = 0; r < n_ops; r++) {
             ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
-            rts.push_back(einsum::Tensor::from_unpadded(c, std::vector<int64_t>(rhs[r], rhs[r] + count(rhs_shapes[r], rhs_ranks[r])),
+            rts.push_back(einsum::Tensor::from_unpadded(c, rhs[r], count(rhs_shapes[r], rhs_ranks[r]),
                                                         std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
             claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
         }

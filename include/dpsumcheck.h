@@ -107,7 +107,10 @@ int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point 
 int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*k */, uint32_t k, dps_mle **out);
 
 /* ---- FixedAxesMapping::mles_from_tensor (zkml/src/layers/einsum/axis.rs:1142-1234) ----
- * tensor: row-major with padded_dims; only the unpadded region is read.
+ * tensor: row-major, stored either with padded_dims (only the unpadded region is
+ * read) or compactly with unpadded_dims -- a raw quantised tensor as the model
+ * holds it, never padded or embedded by the caller; the two are told apart by
+ * the table's length.
  * kinds[a]: 0 contracted, 1 outer, 2 stacked.  points[a]: 2*log2(padded_dims[a])
  * limbs for outer axes (the claim-point slice of that axis), ignored otherwise.
  * Produces prod(stacked dims) tables of 2^ceil_log2(prod(contracted dims))
