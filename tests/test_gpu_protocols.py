@@ -49,6 +49,9 @@ PE_CASES = [
     ((512, 768), [O_, C_]),        # configuration 2, X
     ((768, 3072), [C_, O_]),       # configuration 2, W
     ((8, 512, 256), [S_, O_, C_]), # configuration 4, Q / K
+    ((5, 6), [O_, O_]),            # every axis fixed: Tensor::evaluate of the quantised tensor at a claim point
+    ((3, 4, 5), [O_, O_, O_]),
+    ((300, 350), [O_, O_]),
 ]
 
 
@@ -69,6 +72,11 @@ def test_partial_eval_matches_checker(ctx, orc, case):
     assert len(got2) == ref.shape[0]
     for g, r in zip(got2, ref):
         assert (g.download() == r).all()
+    if all(k == O_ for k in kinds):
+        # ... which is the padded tensor's multilinear extension at the point (last axis = lowest variables)
+        full_point = np.concatenate([points[a] for a in reversed(range(len(shape)))])
+        want = orc.mle_evaluate(orc.embed_i64(_padded(t).reshape(-1)), full_point)
+        assert len(got2) == 1 and (got2[0].download()[0] == want).all()
 
 
 def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec"):
