@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one round-2 launch at n = 24 from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, both
 # factors calibrated on the library's plain copy kernel); counters cannot be read from inside this script
-MEASURED_TRAFFIC_N24 = 604.5e6
+MEASURED_TRAFFIC_N24 = 604.4e6
 P = 0xFFFFFFFF00000001
 
 
