@@ -76,7 +76,7 @@ dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
-           "dps_partial_eval", "dps_sc_begin", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_free",
+           "dps_partial_eval", "dps_sc_begin", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
            "dps_sc_prove", "dps_logup_build", "dps_logup_num_layers", "dps_logup_layer", "dps_logup_outputs",
            "dps_logup_free", "dps_profile_enable", "dps_profile_reset", "dps_profile_read"]:
     getattr(dev, _f).restype = _i32
@@ -303,6 +303,9 @@ class Session:
         if getattr(self, "_h", None) and self.ctx._c:
             dev.dps_sc_free(self._h)
         self._h = None
+
+    def abort(self):
+        self.ctx._chk(dev.dps_sc_abort(self._h), "dps_sc_abort")
 
     def round(self, challenge=None):
         out = np.zeros((self.degree + 1, 2), dtype=np.uint64)

@@ -2085,6 +2085,16 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
     return DPS_OK;
 }
 
+extern "C" int32_t dps_sc_abort(dps_sc *sc)
+{
+    if (!sc) return DPS_ERR_INVALID;
+    dps_ctx *ctx = sc->ctx;
+    DeviceGuard g(ctx->device);
+    if (ctx->tail_owner == sc) tail_abort(ctx);
+    sc->broken = true;
+    return DPS_OK;
+}
+
 extern "C" int32_t dps_sc_free(dps_sc *sc)
 {
     if (!sc) return DPS_OK;

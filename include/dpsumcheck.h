@@ -144,6 +144,9 @@ int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
  * get_mle_flatten_final_evaluations (einsum/prove.rs:188): one element per table,
  * in registration order. */
 int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t *final_evals_out /* 2*n_mles */);
+/* give a session up part-way: a kernel of it that is resident on the GPU exits, further rounds fail with
+ * DPS_ERR_STATE; the handle remains to be freed */
+int32_t dps_sc_abort(dps_sc *sc);
 int32_t dps_sc_free(dps_sc *sc);
 
 /* Transcript hook: absorb `n_evals` extension elements of round `round`

@@ -237,6 +237,33 @@ def test_round_by_round_session_and_errors(dp, ctx, orc):
         ctx.session(n, gpu, [(ONE, [0] * 7)])  # degree above the compiled kernels
 
 
+def test_resident_kernel_gives_way(dp, ctx, orc):
+    # A product session of 12 variables runs its last 8 rounds in one kernel that stays on the GPU between rounds.
+    # Another call on the context makes that kernel exit (through its mailbox; nothing is killed), the interrupted
+    # session reports the failure, and the context keeps working.  dps_sc_abort does the same on request.
+    n = 12
+    f, g = rand_base(1 << n, 8100), rand_base(1 << n, 8101)
+    mf, mg = ctx.mle_from_base(f), ctx.mle_from_base(g)
+    terms = [(ONE, [0, 1])]
+    ref_proof, ref_point, _ = orc.sc_prove(n, [orc.embed_base(f), orc.embed_base(g)], terms, orc.OracleTranscript())
+    for how in ("other call", "abort"):
+        s = ctx.session(n, [mf, mg], terms)
+        chal = None
+        for j in range(6):  # rounds 4 to 6 are already inside the resident kernel
+            assert (s.round(chal) == ref_proof[j]).all()
+            chal = ref_point[j]
+        if how == "other call":
+            assert (ctx.mle_from_base(f).download()[:, 0] == f).all()  # an upload on the same context
+        else:
+            s.abort()
+        with pytest.raises(dp.DpsError):
+            s.round(chal)
+        del s
+        # the context is fine: the same proof from scratch
+        proof, point, _ = ctx.sumcheck_prove(n, [mf, mg], terms, dp.Transcript())
+        assert (proof == ref_proof).all() and (point == ref_point).all()
+
+
 def test_views_are_borrowed_halves(dp, ctx, orc):
     # SmartSlice::Borrowed halves as used by the LogUp layers (circuit.rs:260-271)
     n = 8
