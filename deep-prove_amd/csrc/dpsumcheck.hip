@@ -624,17 +624,6 @@ extern "C" int32_t dps_mle_free(dps_mle *mle)
 // ---------------------------------------------------------------------------
 namespace {
 
-// uploads `words` 64-bit words through the pinned buffer region [slot, slot+words)
-int32_t stage_words(dps_ctx *ctx, const u64 *src, size_t words, size_t slot, const u64 **dev)
-{
-    if (slot + words > ctx->res_off - 64) return fail(ctx, DPS_ERR_INVALID, "staging buffer too small");
-    // the buffer may still be read by queued kernels
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    memcpy(ctx->h_pinned + slot, src, words * 8);
-    *dev = ctx->d_pinned + slot;
-    return DPS_OK;
-}
-
 bool canonical(const u64 *v, size_t n)
 {
     for (size_t i = 0; i < n; i++)
@@ -648,11 +637,11 @@ u64 eq_level_off(u32 m, u32 l) { return (2ull << m) - (2ull << (m - l)); }
 // (2^(m+1) entries).  Levels of at most 2^16 entries come straight from the
 // definition in one launch, together with the 2^8-entry seeds eq(rho_{l..l+7}, .)
 // the larger levels need; level l > 2^16 entries is level l+8 expanded by seed l.
-int32_t eq_build_dev(dps_ctx *ctx, const u64 *d_point, u32 m, u64 *o0, u64 *o1)
+int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
 {
     dpk::EqJobs js;
     memset(&js, 0, sizeof js);
-    js.point = d_point;
+    if (m) memcpy(js.point, point, 16 * (size_t)m);
     js.o0 = o0;
     js.o1 = o1;
     u32 n_jobs = 0, max_bits = 0;
@@ -684,7 +673,7 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *d_point, u32 m, u64 *o0, u64 *o1)
         for (u32 base = 0; base < first_small && rc == DPS_OK; base += dpk::EQ_MAX_JOBS) {
             dpk::EqJobs ss;
             memset(&ss, 0, sizeof ss);
-            ss.point = d_point;
+            memcpy(ss.point, js.point, sizeof ss.point);
             ss.o0 = seed0;
             ss.o1 = seed1;
             u32 n = std::min<u32>(first_small - base, dpk::EQ_MAX_JOBS);
@@ -715,17 +704,14 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *d_point, u32 m, u64 *o0, u64 *o1)
 
 extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m, dps_mle **out)
 {
-    if (!ctx || !out || (m && !point) || m > 34) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: bad argument");
+    if (!ctx || !out || (m && !point) || m > dpk::EQ_MAX_VARS) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: bad argument");
     if (!canonical(point, 2 * (size_t)m)) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build: point not canonical");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
-    const u64 *d_point = nullptr;
-    u64 dummy[2] = {0, 0};
-    CHK(stage_words(ctx, m ? point : dummy, m ? 2 * (size_t)m : 2, 0, &d_point));
     dps_mle *t = nullptr;
     CHK(new_table(ctx, DPS_EXT2, 2ull << m, &t));
     t->len = 1ull << m;
-    int32_t rc = eq_build_dev(ctx, d_point, m, t->st->c0, t->st->c1);
+    int32_t rc = eq_build_dev(ctx, point, m, t->st->c0, t->st->c1);
     if (rc != DPS_OK) {
         delete t;
         return rc;
@@ -916,11 +902,8 @@ extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint6
     for (u32 j = 0; j < k && rc == DPS_OK; j++) {
         len >>= 1;
         dpk::FoldDesc d{s0, s1, bufs[w]->st->c0, bufs[w]->st->c1, len};
-        const u64 *dd = nullptr;
-        rc = stage_words(ctx, (const u64 *)&d, sizeof d / 8, 0, &dd);
-        if (rc != DPS_OK) break;
         ProfScope ps(ctx, DPS_K_FOLD, (double)len * (s1 ? 32.0 : 16.0) + (double)len * 16.0);
-        dpk::fold_kernel<<<dim3(grid_for(len), 1), dpk::BLOCK, 0, ctx->stream>>>((const dpk::FoldDesc *)dd, point[2 * j], point[2 * j + 1]);
+        dpk::fold_one_kernel<<<grid_for(len), dpk::BLOCK, 0, ctx->stream>>>(d, point[2 * j], point[2 * j + 1]);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "fold launch: %s", hipGetErrorString(e));
         s0 = bufs[w]->st->c0;

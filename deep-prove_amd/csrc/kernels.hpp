@@ -142,12 +142,13 @@ __device__ __forceinline__ void block_reduce(E2 (&acc)[NP], u32 *lds /* (BLOCK /
 // Small tables straight from the definition, many per launch.  Job k (blockIdx.y)
 // writes 2^n_bits entries: out[i] = prod_b (bit_b(i) ? r[first + b] : 1 - r[first + b]).
 constexpr int EQ_MAX_JOBS = 48;
+constexpr int EQ_MAX_VARS = 34;
 struct EqJob {
     u32 first, n_bits;
     u64 out_off;  // entries from the start of the output arrays
 };
 struct EqJobs {
-    const u64 *point;  // 2 limbs per coordinate
+    u64 point[2 * EQ_MAX_VARS];  // 2 limbs per coordinate, travels in the kernel arguments
     u64 *o0, *o1;
     EqJob job[EQ_MAX_JOBS];
 };
@@ -211,10 +212,8 @@ __device__ __forceinline__ E2 fold1_base(u64 lo, u64 hi, E2 r)
     return d;
 }
 
-__global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict__ descs, u64 r0, u64 r1)
+__device__ __forceinline__ void fold_body(const FoldDesc &d, E2 r)
 {
-    const FoldDesc d = descs[blockIdx.y];
-    const E2 r = gl::e2(r0, r1);
     if (d.single) {
         if (blockIdx.x == 0 && threadIdx.x == 0) {
             E2 v = fold1(gl::e2(d.s0[0], d.s1 ? d.s1[0] : 0), gl::e2_zero(), r);
@@ -236,6 +235,16 @@ __global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict_
         d.d1[i] = v.c1;
     }
 }
+
+// one table per grid row, descriptors in device-visible memory
+__global__ void __launch_bounds__(BLOCK) fold_kernel(const FoldDesc *__restrict__ descs, u64 r0, u64 r1)
+{
+    const FoldDesc d = descs[blockIdx.y];
+    fold_body(d, gl::e2(r0, r1));
+}
+
+// one table, descriptor in the kernel arguments
+__global__ void __launch_bounds__(BLOCK) fold_one_kernel(FoldDesc d, u64 r0, u64 r1) { fold_body(d, gl::e2(r0, r1)); }
 
 // ---------------------------------------------------------------------------
 // round result: the last workgroup of an evaluation launch sums the block
