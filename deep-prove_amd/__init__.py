@@ -20,7 +20,7 @@ LIB_DIR = os.path.join(_HERE, "lib")
 P = 0xFFFFFFFF00000001
 MAX_FACTORS = 8
 AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
-KIND_BASE, KIND_EXT2, KIND_I64 = 0, 1, 2
+KIND_BASE, KIND_EXT2, KIND_I64, KIND_I16 = 0, 1, 2, 3
 KERNELS = ["eval_first", "fold_eval", "eval_terms", "fold", "eq", "axis_dot", "logup", "finalize", "tail"]
 
 
@@ -67,6 +67,9 @@ for _f, _a in [("dph_tr_free", [_vp]), ("dph_tr_append_message", [_vp, C.c_char_
 # integer arguments are 64-bit so that ctypes does not truncate them
 dev.dps_mle_from_i64.argtypes = [_vp, _vp, _u64, _u32, _vp]
 dev.dps_tensor_from_i64.argtypes = [_vp, _vp, _u64, _vp]
+dev.dps_tensor_from_i16.argtypes = [_vp, _vp, _u64, _vp]
+dev.dps_mle_from_tensor.restype = _i32
+dev.dps_mle_from_tensor.argtypes = [_vp, _vp, _vp, _vp, _u32, _vp]
 dev.dps_mle_wrap_device.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_mle_view.argtypes = [_vp, _u64, _u32, _vp]
 dev.dps_mle_zero_pad.restype = _i32
@@ -225,7 +228,7 @@ class Mle:
         c0 = np.zeros(n, dtype=np.uint64)
         c1 = np.zeros(n, dtype=np.uint64)
         self.ctx._chk(dev.dps_mle_download(self._h, _ptr(c0), _ptr(c1)), "dps_mle_download")
-        if kind == KIND_I64:
+        if kind in (KIND_I64, KIND_I16):
             return c0.view(np.int64)
         return np.stack([c0, c1], axis=-1)
 
@@ -382,6 +385,26 @@ class Context:
         self._chk(dev.dps_tensor_from_i64(self._c, _ptr(v), v.size, C.byref(h)), "dps_tensor_from_i64")
         return Mle(self, h)
 
+    def tensor_from_i16(self, v):
+        """the quantised tensor in 16-bit storage (values must fit int16)"""
+        v = np.ascontiguousarray(v)
+        if v.dtype != np.int16:
+            if v.size and (v.min() < -32768 or v.max() > 32767):
+                raise ValueError("tensor_from_i16: values do not fit 16 bits")
+            v = v.astype(np.int16)
+        v = v.reshape(-1)
+        h = _vp()
+        self._chk(dev.dps_tensor_from_i16(self._c, _ptr(v), v.size, C.byref(h)), "dps_tensor_from_i16")
+        return Mle(self, h)
+
+    def mle_from_tensor(self, tensor, padded_dims, unpadded_dims):
+        """the padded tensor as a base-field table (zero outside the unpadded region), built on the device"""
+        nd = len(padded_dims)
+        pd, ud = (_u64 * nd)(*padded_dims), (_u64 * nd)(*unpadded_dims)
+        h = _vp()
+        self._chk(dev.dps_mle_from_tensor(self._c, tensor.handle, pd, ud, nd, C.byref(h)), "dps_mle_from_tensor")
+        return Mle(self, h)
+
     def wrap_device(self, kind, ptr_c0, ptr_c1, length):
         h = _vp()
         self._chk(dev.dps_mle_wrap_device(self._c, kind, ptr_c0, ptr_c1, length, C.byref(h)), "dps_mle_wrap_device")
@@ -482,6 +505,8 @@ class Context:
 # ---- einsum and LogUp drivers of the host mirror ----
 host.dph_einsum_prove.restype = _i32
 host.dph_einsum_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
+host.dph_einsum_prove_resident.restype = _i32
+host.dph_einsum_prove_resident.argtypes = host.dph_einsum_prove.argtypes
 host.dph_logup_batch_prove.restype = _i32
 host.dph_logup_batch_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
 host.dph_logup_batch_verify.restype = _i32
@@ -495,20 +520,52 @@ def _parse_proof(words, pos):
     return proof, pos + 2 * rounds * npts
 
 
+class Tensor:
+    """A quantised tensor kept on the device (unpadded, row-major): weights across
+    proofs, activations across the layers that read them.  bits: 64 or 16."""
+
+    def __init__(self, ctx, values, bits=64):
+        values = np.asarray(values)
+        self.shape = tuple(values.shape)
+        if bits == 64:
+            self.mle = ctx.tensor_from_i64(values)
+        elif bits == 16:
+            self.mle = ctx.tensor_from_i16(values)
+        else:
+            raise ValueError("Tensor: bits must be 64 or 16")
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+
 def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
     """EinSum::prove_internal.  ops: list of (lhs_labels, rhs_labels, out_labels);
     lhs: int64 ndarray (unpadded); rhs: list of int64 ndarrays; claims: list of
-    (point[k, 2], eval[2]) on the outputs.  Returns a dict with the sumcheck proof,
-    the final evaluations, the optional aggregation proof and the input claims."""
+    (point[k, 2], eval[2]) on the outputs.  lhs and every rhs may instead be
+    `Tensor`s already on the device (nothing is uploaded then).  Returns a dict with
+    the sumcheck proof, the final evaluations, the optional aggregation proof and
+    the input claims."""
     R = len(ops)
     lab = []
     for o in ops:
         lab += [s.encode() for s in o]
     labels = (C.c_char_p * (3 * R))(*lab)
-    lhs = np.ascontiguousarray(lhs, dtype=np.int64)
+    resident = isinstance(lhs, Tensor)
+    if resident != all(isinstance(x, Tensor) for x in rhs) or (not resident and any(isinstance(x, Tensor) for x in rhs)):
+        raise ValueError("einsum_prove: either every tensor is on the device or none is")
+    if resident:
+        rk = list(rhs)
+        rptr = (_vp * R)(*[x.mle.handle for x in rk])
+        lhs_arg = lhs.mle.handle
+        fn, fn_name = host.dph_einsum_prove_resident, "dph_einsum_prove_resident"
+    else:
+        lhs = np.ascontiguousarray(lhs, dtype=np.int64)
+        rk = [np.ascontiguousarray(x, dtype=np.int64) for x in rhs]
+        rptr = (_vp * R)(*[x.ctypes.data for x in rk])
+        lhs_arg = _ptr(lhs)
+        fn, fn_name = host.dph_einsum_prove, "dph_einsum_prove"
     lshape = (_u64 * lhs.ndim)(*lhs.shape)
-    rk = [np.ascontiguousarray(x, dtype=np.int64) for x in rhs]
-    rptr = (_vp * R)(*[x.ctypes.data for x in rk])
     rshapes_keep = [(_u64 * x.ndim)(*x.shape) for x in rk]
     rshapes = (_vp * R)(*[C.cast(s, _vp).value for s in rshapes_keep])
     rranks = (_u32 * R)(*[x.ndim for x in rk])
@@ -519,8 +576,8 @@ def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
     cap = 1 << 16
     out = np.zeros(cap, dtype=np.uint64)
     n = _u64(0)
-    ctx._chk_host(host.dph_einsum_prove(ctx._c, R, labels, _ptr(lhs), lshape, lhs.ndim, rptr, rshapes, rranks, pts, plens, _ptr(evals),
-                                        transcript._t, _ptr(out), cap, C.byref(n)), "dph_einsum_prove")
+    ctx._chk_host(fn(ctx._c, R, labels, lhs_arg, lshape, lhs.ndim, rptr, rshapes, rranks, pts, plens, _ptr(evals),
+                     transcript._t, _ptr(out), cap, C.byref(n)), fn_name)
     w = out[: n.value]
     res = {}
     res["proof"], pos = _parse_proof(w, 0)

@@ -285,6 +285,9 @@ struct dps_mle {
 namespace {
 
 bool is_pow2(u64 x) { return x && !(x & (x - 1)); }
+// raw quantised integers (not field elements): readable by the tensor kernels only
+bool is_raw(int32_t kind) { return kind == DPS_I64 || kind == DPS_I16; }
+int raw_bytes(int32_t kind) { return kind == DPS_I64 ? 8 : kind == DPS_I16 ? 2 : 0; }
 u32 log2u(u64 x)
 {
     u32 l = 0;
@@ -297,7 +300,7 @@ int32_t new_table(dps_ctx *ctx, int32_t kind, u64 len, dps_mle **out)
     auto st = std::make_shared<Storage>();
     st->ctx = ctx;
     void *p = nullptr;
-    CHK(pool_alloc(ctx, len * 8, &p));
+    CHK(pool_alloc(ctx, kind == DPS_I16 ? (len * 2 + 7) / 8 * 8 : len * 8, &p));
     st->c0 = (u64 *)p;
     if (kind == DPS_EXT2) {
         CHK(pool_alloc(ctx, len * 8, &p));
@@ -517,6 +520,26 @@ extern "C" int32_t dps_tensor_from_i64(dps_ctx *ctx, const int64_t *host, uint64
     return DPS_OK;
 }
 
+extern "C" int32_t dps_tensor_from_i16(dps_ctx *ctx, const int16_t *host, uint64_t len, dps_mle **out)
+{
+    if (!ctx || !out || (len && !host)) return fail(ctx, DPS_ERR_INVALID, "dps_tensor_from_i16: bad argument");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    dps_mle *m = nullptr;
+    CHK(new_table(ctx, DPS_I16, std::max<u64>(len, 1), &m));
+    m->len = len;
+    if (len) {
+        hipError_t e = hipMemcpyAsync(m->st->c0, host, len * 2, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            delete m;
+            return fail(ctx, DPS_ERR_HIP, "upload: %s", hipGetErrorString(e));
+        }
+    }
+    *out = m;
+    return DPS_OK;
+}
+
 extern "C" int32_t dps_mle_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, uint32_t n_vars, dps_mle **out)
 {
     if (!ctx || !out || n_vars > 40 || len > (1ull << n_vars) || (len && !host))
@@ -544,9 +567,55 @@ extern "C" int32_t dps_mle_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t 
     return DPS_OK;
 }
 
+extern "C" int32_t dps_mle_from_tensor(dps_ctx *ctx, const dps_mle *tensor, const uint64_t *padded_dims, const uint64_t *unpadded_dims,
+                                       uint32_t n_dims, dps_mle **out)
+{
+    if (!ctx || !tensor || !padded_dims || !unpadded_dims || !out || n_dims == 0 || n_dims > dpk::PAD_MAX_DIMS)
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_tensor: bad argument");
+    if (tensor->ctx != ctx || tensor->kind == DPS_EXT2 || tensor->pad_vars)
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_tensor: not a raw or base-field tensor of this context");
+    u64 padded_total = 1, unpadded_total = 1;
+    for (u32 a = 0; a < n_dims; a++) {
+        if (!is_pow2(padded_dims[a]) || unpadded_dims[a] == 0 || unpadded_dims[a] > padded_dims[a] || padded_total > (1ull << 40) / padded_dims[a])
+            return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_tensor: axis %u: sizes %llu (padded %llu)", a, (unsigned long long)unpadded_dims[a],
+                        (unsigned long long)padded_dims[a]);
+        padded_total *= padded_dims[a];
+        unpadded_total *= unpadded_dims[a];
+    }
+    // stored in its padded shape, or compactly in its unpadded shape (told apart by its length)
+    const bool compact = tensor->len == unpadded_total && unpadded_total != padded_total;
+    if (!compact && tensor->len < padded_total) return fail(ctx, DPS_ERR_INVALID, "dps_mle_from_tensor: tensor shorter than its padded shape");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    dpk::PadTensorArgs a;
+    memset(&a, 0, sizeof a);
+    a.in = tensor->kind == DPS_I16 ? (const void *)tensor->st->c0 : (const void *)tensor->p0();
+    a.in_int = raw_bytes(tensor->kind);
+    a.n_dims = n_dims;
+    u64 stride = 1;
+    for (int d = (int)n_dims - 1; d >= 0; d--) {
+        a.padded_dims[d] = padded_dims[d];
+        a.unpadded_dims[d] = unpadded_dims[d];
+        a.src_strides[d] = stride;
+        stride *= compact ? unpadded_dims[d] : padded_dims[d];
+    }
+    a.total = padded_total;
+    dps_mle *m = nullptr;
+    CHK(new_table(ctx, DPS_BASE, padded_total, &m));
+    a.out = m->st->c0;
+    dpk::pad_tensor_kernel<<<grid_for(padded_total), dpk::BLOCK, 0, ctx->stream>>>(a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        delete m;
+        return fail(ctx, DPS_ERR_HIP, "pad_tensor launch: %s", hipGetErrorString(e));
+    }
+    *out = m;
+    return DPS_OK;
+}
+
 extern "C" int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, void *d_c1, uint64_t len, dps_mle **out)
 {
-    if (!ctx || !out || !d_c0 || kind < DPS_BASE || kind > DPS_I64 || (kind == DPS_EXT2) != (d_c1 != nullptr))
+    if (!ctx || !out || !d_c0 || kind < DPS_BASE || kind > DPS_I16 || (kind == DPS_EXT2) != (d_c1 != nullptr))
         return fail(ctx, DPS_ERR_INVALID, "dps_mle_wrap_device: bad argument");
     if (((uintptr_t)d_c0 & 15) || ((uintptr_t)d_c1 & 15)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_wrap_device: pointers must be 16-byte aligned");
     auto st = std::make_shared<Storage>();
@@ -564,6 +633,7 @@ extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_
     dps_ctx *ctx = src->ctx;
     u64 len = 1ull << n_vars;
     if (src->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_view: the table is a zero-padded view");
+    if (src->kind == DPS_I16) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_view: no windows into int16 tensors");
     if (n_vars > 40 || offset > src->len || len > src->len - offset) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: window outside the table");
     // pair loads are 16 bytes wide
     if (n_vars >= 1 && ((src->offset + offset) & 1)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: offset must be even");
@@ -576,7 +646,7 @@ extern "C" int32_t dps_mle_zero_pad(const dps_mle *src, uint32_t n_vars, dps_mle
 {
     if (!src || !out) return DPS_ERR_INVALID;
     dps_ctx *ctx = src->ctx;
-    if (src->kind == DPS_I64 || !is_pow2(src->len)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: not a power-of-two field table");
+    if (is_raw(src->kind) || !is_pow2(src->len)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: not a power-of-two field table");
     if (n_vars > 40 || (1ull << n_vars) < src->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: %u variables are fewer than the table has", n_vars);
     *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset, src->len, nullptr, n_vars};
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
@@ -597,6 +667,14 @@ extern "C" int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (mle->kind == DPS_I16) {
+        // widened on the host: the caller's buffer holds len int64 values like a DPS_I64 tensor's
+        std::vector<int16_t> tmp(mle->len);
+        if (mle->len) HIPCHK(ctx, hipMemcpy(tmp.data(), mle->st->c0, mle->len * 2, hipMemcpyDeviceToHost));
+        for (u64 i = 0; i < mle->len; i++) c0[i] = (u64)(int64_t)tmp[i];
+        if (c1) memset(c1, 0, mle->len * 8);
+        return DPS_OK;
+    }
     if (mle->len) HIPCHK(ctx, hipMemcpy(c0, mle->p0(), mle->len * 8, hipMemcpyDeviceToHost));
     if (c1) {
         if (mle->kind == DPS_EXT2) {
@@ -730,7 +808,7 @@ namespace {
 
 struct AxisJob {
     const u64 *in0 = nullptr, *in1 = nullptr;
-    bool in_is_i64 = false;
+    int in_int = 0;  // bytes per raw integer entry, 0 for field elements
     const u64 *b0 = nullptr, *b1 = nullptr;
     u64 K = 1, stride_k = 1;
     std::vector<u64> pre_dims, pre_strides, post_dims, post_strides;
@@ -745,7 +823,7 @@ int32_t axis_dot(dps_ctx *ctx, const AxisJob &j)
         return fail(ctx, DPS_ERR_UNSUPPORTED, "tensor rank above %d", dpk::AX_MAX_DIMS);
     a.in0 = j.in0;
     a.in1 = j.in1;
-    a.in_is_i64 = j.in_is_i64;
+    a.in_int = j.in_int;
     a.b0 = j.b0;
     a.b1 = j.b1;
     a.K = j.K;
@@ -819,7 +897,7 @@ extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint
     AxisJob j;
     j.in0 = mle->p0();
     j.in1 = mle->p1();
-    j.in_is_i64 = mle->kind == DPS_I64;
+    j.in_int = raw_bytes(mle->kind);
     j.b0 = eq->p0();
     j.b1 = eq->p1();
     j.K = mle->len;
@@ -853,7 +931,7 @@ extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint
         AxisJob j;
         j.in0 = mle->p0();
         j.in1 = mle->p1();
-        j.in_is_i64 = mle->kind == DPS_I64;
+        j.in_int = raw_bytes(mle->kind);
         j.b0 = eq->p0();
         j.b1 = eq->p1();
         j.K = 1ull << k;
@@ -879,7 +957,7 @@ extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint6
 {
     if (!ctx || !mle || !out || (k && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: bad argument");
     if (mle->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_fix_low: the table is a zero-padded view");
-    if (!is_pow2(mle->len) || (1ull << k) > mle->len || mle->kind == DPS_I64)
+    if (!is_pow2(mle->len) || (1ull << k) > mle->len || is_raw(mle->kind))
         return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: needs a power-of-two field table and k <= log2(len)");
     if (!canonical(point, 2 * (size_t)k)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: point not canonical");
     DeviceGuard g(ctx->device);
@@ -962,7 +1040,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         }
     }
     const u64 *in0 = tensor->p0(), *in1 = tensor->p1();
-    bool in_is_i64 = tensor->kind == DPS_I64;
+    int in_int = raw_bytes(tensor->kind);
     dps_mle *cur = nullptr;  // owns the intermediate
     int32_t rc = DPS_OK;
     // the reference walks the axes from the last to the first (axis.rs:1152)
@@ -976,7 +1054,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         AxisJob j;
         j.in0 = in0;
         j.in1 = in1;
-        j.in_is_i64 = in_is_i64;
+        j.in_int = in_int;
         j.b0 = beta->p0();
         j.b1 = beta->p1();
         j.K = dims[a];  // evals(point)[..size]
@@ -1009,7 +1087,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         for (int d = (int)dims.size() - 2; d >= 0; d--) strides[d] = strides[d + 1] * dims[d + 1];
         in0 = cur->st->c0;
         in1 = cur->st->c1;
-        in_is_i64 = false;
+        in_int = 0;
     }
     if (rc != DPS_OK) {
         delete cur;
@@ -1040,7 +1118,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
                 AxisJob j;
                 j.in0 = in0;
                 j.in1 = in1;
-                j.in_is_i64 = in_is_i64;
+                j.in_int = in_int;
                 j.b0 = unit->p0();
                 j.b1 = unit->p1();
                 j.K = 1;
@@ -1265,7 +1343,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     for (u32 k = 0; k < n_mles; k++) {
         const dps_mle *t = mles[k];
         if (!t || t->ctx != ctx) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u belongs to another context", k);
-        if (t->kind == DPS_I64 || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
+        if (is_raw(t->kind) || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
         nv0[k] = log2u(t->len);
         if (nv0[k] > n_vars) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u has %u variables, the sum has %u", k, nv0[k], n_vars);
         if (t->pad_vars && t->pad_vars != n_vars)

@@ -1272,6 +1272,38 @@ embed_i64_kernel(const int64_t *__restrict__ in, u64 len, u64 padded_len, u64 *_
         out[i] = i < len ? gl::from_i64(in[i]) : 0;
 }
 
+// a raw tensor stored row-major in `src_dims` (its unpadded shape, or its padded one)
+// into the base-field table of its padded shape: entry (i_0..i_{n-1}) is the
+// embedded value when every i_a < unpadded_dims[a], else 0
+constexpr int PAD_MAX_DIMS = 6;
+struct PadTensorArgs {
+    const void *in;
+    int in_int;  // 8: int64, 2: int16, 0: base-field elements
+    u32 n_dims;
+    u64 padded_dims[PAD_MAX_DIMS], unpadded_dims[PAD_MAX_DIMS], src_strides[PAD_MAX_DIMS];
+    u64 total;
+    u64 *out;
+};
+__global__ void __launch_bounds__(BLOCK) pad_tensor_kernel(PadTensorArgs a)
+{
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.total; i += (u64)gridDim.x * BLOCK) {
+        u64 flat = i, off = 0;
+        bool inside = true;
+        for (int d = (int)a.n_dims - 1; d >= 0; d--) {
+            u64 q = flat / a.padded_dims[d], c = flat - q * a.padded_dims[d];
+            inside = inside && c < a.unpadded_dims[d];
+            off += c * a.src_strides[d];
+            flat = q;
+        }
+        u64 v = 0;
+        if (inside)
+            v = a.in_int == 8   ? gl::from_i64(((const int64_t *)a.in)[off])
+                : a.in_int == 2 ? gl::from_i64(((const int16_t *)a.in)[off])
+                                : ((const u64 *)a.in)[off];
+        a.out[i] = v;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // contraction of one tensor axis with a table beta (partial evaluation):
 //   out[pre][i] = sum_k in[off_pre(pre) + k * stride_k + off_post(i)] * beta[k]
@@ -1281,8 +1313,8 @@ embed_i64_kernel(const int64_t *__restrict__ in, u64 len, u64 padded_len, u64 *_
 constexpr int AX_MAX_DIMS = 6;
 struct AxisArgs {
     const u64 *in0;
-    const u64 *in1;  // nullptr: base field or raw int64
-    int in_is_i64;
+    const u64 *in1;  // nullptr: base field or raw integers
+    int in_int;      // 0: field elements; 8: raw int64; 2: raw int16 (embedded on load)
     const u64 *b0;
     const u64 *b1;
     u64 K, stride_k;
@@ -1309,7 +1341,8 @@ __device__ __forceinline__ u64 ax_offset(u64 flat, u32 n, const u64 *dims, const
 
 __device__ __forceinline__ E2 ax_load(const AxisArgs &a, u64 off)
 {
-    if (a.in_is_i64) return gl::e2(gl::from_i64(((const int64_t *)a.in0)[off]), 0);
+    if (a.in_int == 8) return gl::e2(gl::from_i64(((const int64_t *)a.in0)[off]), 0);
+    if (a.in_int == 2) return gl::e2(gl::from_i64(((const int16_t *)a.in0)[off]), 0);
     return gl::e2(a.in0[off], a.in1 ? a.in1[off] : 0);
 }
 

@@ -18,16 +18,14 @@ struct Claim {
     F eval;
 };
 
-// A quantised tensor: row-major int64 values in the padded shape, resident on the GPU.
+// A quantised tensor on the GPU: raw integers, row-major, stored compactly in the unpadded shape.  Padding and
+// the embedding into the field happen in the kernels that read it (einsum/prove.rs:66-94 materialises a padded
+// Tensor<F> instead).
 struct Tensor {
     std::vector<uint64_t> padded_shape, unpadded_shape;
-    const int64_t *data = nullptr;  // the caller's unpadded row-major values (borrowed)
-    uint64_t count = 0;
-    DensePolynomial device;         // raw int64 tensor on the device, stored compactly (unpadded)
+    DensePolynomial device;
 
-    // The tensor goes to the device as it is: padding and the embedding into the field happen in the kernels
-    // that read it (einsum/prove.rs:66-94 materialises a padded Tensor<F> instead).
-    static Tensor from_unpadded(const Context &ctx, const int64_t *data, uint64_t n, const std::vector<uint64_t> &shape)
+    static Tensor with_shape(const std::vector<uint64_t> &shape, uint64_t n)
     {
         Tensor t;
         t.unpadded_shape = shape;
@@ -39,8 +37,12 @@ struct Tensor {
         uint64_t utotal = 1;
         for (auto d : shape) utotal *= d;
         if (n != utotal) throw Error(DPS_ERR_INVALID, "Tensor: data does not match the shape");
-        t.data = data;
-        t.count = n;
+        return t;
+    }
+    // upload for the length of one proof
+    static Tensor from_unpadded(const Context &ctx, const int64_t *data, uint64_t n, const std::vector<uint64_t> &shape)
+    {
+        Tensor t = with_shape(shape, n);
         dps_mle *h = nullptr;
         ctx.check(dps_tensor_from_i64(ctx.raw(), data, n, &h), "dps_tensor_from_i64");
         t.device = DensePolynomial(ctx, h);
@@ -50,24 +52,20 @@ struct Tensor {
     {
         return from_unpadded(ctx, data.data(), data.size(), shape);
     }
-    // padded row-major copy (zeros outside the unpadded region); only the aggregation sumcheck needs it
-    std::vector<int64_t> padded_host() const
+    // a tensor the caller uploaded before (dps_tensor_from_i64 / dps_tensor_from_i16, unpadded) and keeps: weights
+    // stay on the device across proofs, activations go there once per layer
+    static Tensor resident(const Context &ctx, const dps_mle *handle, const std::vector<uint64_t> &shape)
     {
-        uint64_t total = 1;
-        for (auto d : padded_shape) total *= d;
-        std::vector<int64_t> host(total, 0);
-        std::vector<uint64_t> idx(unpadded_shape.size(), 0);
-        for (uint64_t flat = 0; flat < count; flat++) {
-            uint64_t dst = 0;
-            for (size_t a = 0; a < unpadded_shape.size(); a++) dst = dst * padded_shape[a] + idx[a];
-            host[dst] = data[flat];
-            for (size_t a = unpadded_shape.size(); a-- > 0;) {
-                if (++idx[a] < unpadded_shape[a]) break;
-                idx[a] = 0;
-            }
-        }
-        return host;
+        int32_t kind = 0;
+        uint64_t len = 0;
+        if (!handle || dps_mle_info(handle, &kind, &len) != DPS_OK) throw Error(DPS_ERR_INVALID, "Tensor: null handle");
+        if (kind != DPS_I64 && kind != DPS_I16) throw Error(DPS_ERR_INVALID, "Tensor: the handle is not a raw integer tensor");
+        Tensor t = with_shape(shape, len);
+        t.device = DensePolynomial::borrowed(ctx, handle);
+        return t;
     }
+    // the padded tensor as a base-field table (the aggregation sumcheck's input)
+    DensePolynomial padded_mle(const Context &ctx) const { return DensePolynomial::from_tensor(ctx, device, padded_shape, unpadded_shape); }
 };
 
 // Shape::split_point (zkml/src/shape.rs:475-496): the last dimension takes the lowest variables
@@ -277,7 +275,7 @@ inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> 
     Claim lhs_claim;
     if (R > 1) {
         // prove.rs:260-302: aggregate the R claims on the LHS with a second sumcheck
-        DensePolynomial input_mle = DensePolynomial::from_i64(ctx, lhs.padded_host());
+        DensePolynomial input_mle = lhs.padded_mle(ctx);
         const uint32_t nv = input_mle.num_vars();
         std::vector<DensePolynomial> eq_polys;
         for (size_t r = 0; r < R; r++)

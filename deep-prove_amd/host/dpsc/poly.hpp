@@ -48,6 +48,23 @@ class DensePolynomial {
 public:
     DensePolynomial() = default;
     DensePolynomial(const Context &ctx, dps_mle *h) : ctx_(&ctx), h_(h, &dps_mle_free) {}
+    // a handle the caller keeps alive and frees (tensors resident on the device across proofs)
+    static DensePolynomial borrowed(const Context &ctx, const dps_mle *h)
+    {
+        DensePolynomial p;
+        p.ctx_ = &ctx;
+        p.h_ = decltype(p.h_)(const_cast<dps_mle *>(h), [](dps_mle *) { return 0; });
+        return p;
+    }
+    // pad_next_power_of_two + to_field_mle of a raw tensor that is already on the device
+    static DensePolynomial from_tensor(const Context &ctx, const DensePolynomial &tensor, const std::vector<uint64_t> &padded_shape,
+                                       const std::vector<uint64_t> &unpadded_shape)
+    {
+        dps_mle *h = nullptr;
+        ctx.check(dps_mle_from_tensor(ctx.raw(), tensor.raw(), padded_shape.data(), unpadded_shape.data(), (uint32_t)padded_shape.size(), &h),
+                  "dps_mle_from_tensor");
+        return DensePolynomial(ctx, h);
+    }
 
     // DensePolynomial::new(Vec<F>) for base-field evaluations
     static DensePolynomial from_base(const Context &ctx, const std::vector<uint64_t> &evals)

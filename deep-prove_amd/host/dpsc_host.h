@@ -61,6 +61,17 @@ int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels
                          const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
                          uint64_t *n_words);
 
+/* The same proof over tensors that are already on the device: raw integer
+ * tensors made with dps_tensor_from_i64 / dps_tensor_from_i16 (unpadded,
+ * row-major) that the caller keeps — weights across proofs, activations
+ * across the layers that read them.  Nothing is uploaded per call. */
+int32_t dph_einsum_prove_resident(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const dps_mle *lhs,
+                                  const uint64_t *lhs_shape, uint32_t lhs_rank, const dps_mle *const *rhs,
+                                  const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                                  const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
+                                  const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
+                                  uint64_t *n_words);
+
 /* ---- new_batch_multiple_sizes_prove (zkml/src/lookup/logup_gkr/prover.rs:91-344) ----
  * Instance i has n_cols[i] base-field column tables (handles, flattened in
  * cols) and, for table instances, a multiplicity table numer[i] (numer is NULL

@@ -121,6 +121,49 @@ int32_t dph_sumcheck_verify(const uint64_t claimed_sum[2], const uint64_t *proof
     });
 }
 
+namespace {
+
+// the proof and the claims as 64-bit words, in the order the header states
+void write_einsum(const einsum::EinSumProofInfo &info, uint64_t *out, uint64_t out_cap, uint64_t *n_words)
+{
+    std::vector<uint64_t> w;
+    auto put = [&](const F &x) {
+        w.push_back(x.c0);
+        w.push_back(x.c1);
+    };
+    auto put_proof = [&](const IOPProof &p) {
+        w.push_back(p.proofs.size());
+        w.push_back(p.proofs.empty() ? 0 : p.proofs[0].evaluations.size());
+        for (auto &m : p.proofs)
+            for (auto &e : m.evaluations) put(e);
+    };
+    put_proof(info.proof.einsum_sumcheck);
+    w.push_back(info.proof.einsum_evaluations.size());
+    for (auto &e : info.proof.einsum_evaluations) put(e);
+    if (info.proof.has_aggregation)
+        put_proof(info.proof.input_aggregation_sumcheck);
+    else
+        w.push_back(0);
+    w.push_back(info.claims.size());
+    for (auto &cl : info.claims) {
+        w.push_back(cl.point.size());
+        for (auto &x : cl.point) put(x);
+        put(cl.eval);
+    }
+    if (w.size() > out_cap) throw Error(DPS_ERR_INVALID, "dph_einsum_prove: output buffer too small");
+    memcpy(out, w.data(), w.size() * 8);
+    *n_words = w.size();
+}
+
+uint64_t shape_count(const uint64_t *shape, uint32_t rank)
+{
+    uint64_t n = 1;
+    for (uint32_t i = 0; i < rank; i++) n *= shape[i];
+    return n;
+}
+
+}  // namespace
+
 int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const int64_t *lhs,
                          const uint64_t *lhs_shape, uint32_t lhs_rank, const int64_t *const *rhs,
                          const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
@@ -130,49 +173,39 @@ int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels
 {
     return guarded([&] {
         Context c(ctx);
-        auto count = [](const uint64_t *shape, uint32_t rank) {
-            uint64_t n = 1;
-            for (uint32_t i = 0; i < rank; i++) n *= shape[i];
-            return n;
-        };
         std::vector<einsum::Op> ops;
         std::vector<einsum::Tensor> rts;
         std::vector<einsum::Claim> claims;
-        einsum::Tensor lt = einsum::Tensor::from_unpadded(c, lhs, count(lhs_shape, lhs_rank), std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
+        einsum::Tensor lt = einsum::Tensor::from_unpadded(c, lhs, shape_count(lhs_shape, lhs_rank), std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
         for (uint32_t r = 0; r < n_ops; r++) {
             ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
-            rts.push_back(einsum::Tensor::from_unpadded(c, rhs[r], count(rhs_shapes[r], rhs_ranks[r]),
+            rts.push_back(einsum::Tensor::from_unpadded(c, rhs[r], shape_count(rhs_shapes[r], rhs_ranks[r]),
                                                         std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
             claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
         }
-        auto info = einsum::prove_internal(c, ops, lt, rts, claims, t->t);
-        std::vector<uint64_t> w;
-        auto put = [&](const F &x) {
-            w.push_back(x.c0);
-            w.push_back(x.c1);
-        };
-        auto put_proof = [&](const IOPProof &p) {
-            w.push_back(p.proofs.size());
-            w.push_back(p.proofs.empty() ? 0 : p.proofs[0].evaluations.size());
-            for (auto &m : p.proofs)
-                for (auto &e : m.evaluations) put(e);
-        };
-        put_proof(info.proof.einsum_sumcheck);
-        w.push_back(info.proof.einsum_evaluations.size());
-        for (auto &e : info.proof.einsum_evaluations) put(e);
-        if (info.proof.has_aggregation)
-            put_proof(info.proof.input_aggregation_sumcheck);
-        else
-            w.push_back(0);
-        w.push_back(info.claims.size());
-        for (auto &cl : info.claims) {
-            w.push_back(cl.point.size());
-            for (auto &x : cl.point) put(x);
-            put(cl.eval);
+        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t), out, out_cap, n_words);
+    });
+}
+
+int32_t dph_einsum_prove_resident(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const dps_mle *lhs,
+                                  const uint64_t *lhs_shape, uint32_t lhs_rank, const dps_mle *const *rhs,
+                                  const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                                  const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
+                                  const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
+                                  uint64_t *n_words)
+{
+    return guarded([&] {
+        Context c(ctx);
+        std::vector<einsum::Op> ops;
+        std::vector<einsum::Tensor> rts;
+        std::vector<einsum::Claim> claims;
+        einsum::Tensor lt = einsum::Tensor::resident(c, lhs, std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
+        for (uint32_t r = 0; r < n_ops; r++) {
+            ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
+            rts.push_back(einsum::Tensor::resident(c, rhs[r], std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
+            claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
         }
-        if (w.size() > out_cap) throw Error(DPS_ERR_INVALID, "dph_einsum_prove: output buffer too small");
-        memcpy(out, w.data(), w.size() * 8);
-        *n_words = w.size();
+        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t), out, out_cap, n_words);
     });
 }
 

@@ -50,7 +50,9 @@ typedef enum dps_status {
 typedef enum dps_kind {
     DPS_BASE = 0, /* uint64_t canonical base-field entries */
     DPS_EXT2 = 1, /* two limb arrays */
-    DPS_I64 = 2   /* raw quantised int64_t entries, embedded on load (zkml/src/quantization/mod.rs:262-266) */
+    DPS_I64 = 2,  /* raw quantised int64_t entries, embedded on load (zkml/src/quantization/mod.rs:262-266) */
+    DPS_I16 = 3   /* the same values stored as int16_t (quantised activations and weights fit 16 bits); a tensor
+                   * input of dps_partial_eval, dps_mle_evaluate and dps_mle_fix_high only */
 } dps_kind;
 
 typedef struct dps_ctx dps_ctx;
@@ -78,7 +80,16 @@ int32_t dps_mle_from_ext2(dps_ctx *ctx, const uint64_t *c0, const uint64_t *c1, 
 int32_t dps_mle_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, uint32_t n_vars, dps_mle **out);
 /* upload a raw quantised tensor of any length (input of dps_partial_eval) */
 int32_t dps_tensor_from_i64(dps_ctx *ctx, const int64_t *host, uint64_t len, dps_mle **out);
-/* borrow device memory the caller owns (kind DPS_BASE / DPS_I64: d_c1 is NULL) */
+/* the same tensor from 16-bit storage: a quarter of the bytes on the device and over PCIe */
+int32_t dps_tensor_from_i16(dps_ctx *ctx, const int16_t *host, uint64_t len, dps_mle **out);
+/* Tensor<Element>::pad_next_power_of_two + to_field_mle on a tensor that is already on the
+ * device (zkml/src/tensor/mod.rs:328-401, 812-990): the base-field table of the padded shape,
+ * zero outside the unpadded region.  `tensor` (DPS_I64, DPS_I16 or DPS_BASE) is stored row-major
+ * in its unpadded shape or in its padded one, as for dps_partial_eval.  Queued on the context's
+ * stream, no wait. */
+int32_t dps_mle_from_tensor(dps_ctx *ctx, const dps_mle *tensor, const uint64_t *padded_dims, const uint64_t *unpadded_dims,
+                            uint32_t n_dims, dps_mle **out);
+/* borrow device memory the caller owns (kind DPS_BASE / DPS_I64 / DPS_I16: d_c1 is NULL) */
 int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, void *d_c1, uint64_t len, dps_mle **out);
 /* SmartSlice::Borrowed: a window [offset, offset + 2^n_vars) sharing storage */
 int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_vars, dps_mle **out);
@@ -90,7 +101,7 @@ int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_vars, dps_m
  * handle is accepted by dps_sc_begin, dps_mle_info, dps_mle_download and dps_mle_free only. */
 int32_t dps_mle_zero_pad(const dps_mle *src, uint32_t n_vars, dps_mle **out);
 int32_t dps_mle_info(const dps_mle *mle, int32_t *kind, uint64_t *len);
-/* copy back; c1 may be NULL for DPS_BASE / DPS_I64 */
+/* copy back; c1 may be NULL for DPS_BASE / DPS_I64 / DPS_I16 (raw tensors come back as int64_t values in c0) */
 int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *c1);
 int32_t dps_mle_free(dps_mle *mle);
 

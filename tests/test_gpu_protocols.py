@@ -55,6 +55,44 @@ PE_CASES = [
 ]
 
 
+def test_int16_tensor_edges(dp, ctx, orc):
+    """extreme 16-bit values embed like their int64 counterparts; odd lengths; what int16 tensors refuse"""
+    v = np.array([-32768, 32767, -1, 0, 1, -12345, 777], dtype=np.int64)
+    t16 = ctx.tensor_from_i16(v)
+    assert t16.info() == (dp.KIND_I16, 7)
+    assert (t16.download() == v).all()
+    point = [rand_e2(3, 5)]
+    want = orc.partial_eval(_padded(v), [8], [7], [O_], point)
+    got = ctx.partial_eval(t16, [8], [7], [O_], point)
+    assert (got[0].download() == want[0]).all()
+    p8 = np.concatenate([v, [0]])
+    assert (ctx.tensor_from_i16(p8).evaluate(point[0]) == orc.mle_evaluate(orc.embed_i64(p8), point[0])).all()
+    with pytest.raises(ValueError):
+        ctx.tensor_from_i16(np.array([40000]))
+    with pytest.raises(dp.DpsError):
+        ctx.tensor_from_i16(p8).view(0, 2)
+    with pytest.raises(dp.DpsError):
+        ctx.tensor_from_i16(p8).zero_pad(4)
+    with pytest.raises(dp.DpsError):
+        ctx.session(3, [ctx.tensor_from_i16(p8)], [((1, 0), [0])])
+
+
+@pytest.mark.parametrize("shape", [(5,), (3, 5), (4, 8), (2, 3, 7), (300, 350)])
+def test_padded_table_from_resident_tensor(dp, ctx, orc, shape):
+    """dps_mle_from_tensor: the padded tensor's base-field table from compact or padded storage, 64- and 16-bit"""
+    t = rand_i64(shape, 77)
+    want = orc.embed_i64(_padded(t).reshape(-1))
+    for make in (ctx.tensor_from_i64, ctx.tensor_from_i16):
+        for stored in (t, _padded(t)):
+            got = ctx.mle_from_tensor(make(stored), _pad(shape), list(shape))
+            assert got.info() == (dp.KIND_BASE, want.shape[0])
+            assert (got.download() == want).all()
+    with pytest.raises(dp.DpsError):
+        ctx.mle_from_tensor(ctx.tensor_from_i64(t.reshape(-1)[:-1]), _pad(shape), list(shape))
+    with pytest.raises(dp.DpsError):
+        ctx.mle_from_tensor(ctx.tensor_from_i64(t), [d + 1 for d in _pad(shape)], list(shape))
+
+
 @pytest.mark.parametrize("case", range(len(PE_CASES)))
 def test_partial_eval_matches_checker(ctx, orc, case):
     shape, kinds = PE_CASES[case]
@@ -72,6 +110,14 @@ def test_partial_eval_matches_checker(ctx, orc, case):
     assert len(got2) == ref.shape[0]
     for g, r in zip(got2, ref):
         assert (g.download() == r).all()
+    # the same values in 16-bit storage, padded and compact
+    for stored in (_padded(t), t):
+        t16 = ctx.tensor_from_i16(stored)
+        assert (t16.download() == stored.reshape(-1)).all()
+        got3 = ctx.partial_eval(t16, pd, list(shape), kinds, points)
+        assert len(got3) == ref.shape[0]
+        for g, r in zip(got3, ref):
+            assert (g.download() == r).all()
     if all(k == O_ for k in kinds):
         # ... which is the padded tensor's multilinear extension at the point (last axis = lowest variables)
         full_point = np.concatenate([points[a] for a in reversed(range(len(shape)))])
@@ -179,6 +225,20 @@ def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed):
     for (gp, ge), (rp, re) in zip(got["claims"], ref["claims"]):
         assert (gp == rp).all() and (ge == re).all()
     assert tr.state() == otr.state()
+    # the same proof from tensors that stay on the device, in 64-bit and in 16-bit storage, proved twice from
+    # the same handles (nothing in a proof may change them)
+    for bits in (64, 16):
+        dl, dr = dp.Tensor(ctx, lhs, bits), [dp.Tensor(ctx, x, bits) for x in rhs]
+        for _ in range(2):
+            rt = dp.Transcript()
+            again = dp.einsum_prove(ctx, ops, dl, dr, claims, rt)
+            assert (again["proof"] == got["proof"]).all() and (again["evaluations"] == got["evaluations"]).all()
+            assert (again["aggregation_proof"] is None) == (got["aggregation_proof"] is None)
+            if got["aggregation_proof"] is not None:
+                assert (again["aggregation_proof"] == got["aggregation_proof"]).all()
+            for (gp, ge), (rp, re) in zip(again["claims"], got["claims"]):
+                assert (gp == rp).all() and (ge == re).all()
+            assert rt.state() == tr.state()
     # the proof proves the output claim: p_1(0) + p_1(1) = sum_r gamma^r claim_r
     vt = orc.OracleTranscript()
     gamma = vt.append_and_sample(b"batching_challenge")
