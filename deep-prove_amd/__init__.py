@@ -721,3 +721,72 @@ def same_poly_verify(n_vars, claims, proof, ev, transcript):
     point = np.zeros((n_vars, 2), dtype=np.uint64)
     rc = host.dph_same_poly_verify(n_vars, len(claims), _ptr(points), _ptr(evals), _ptr(proof), _ptr(ev), transcript._t, _ptr(point))
     return rc, point
+
+
+# ---- the sumcheck linking a lookup argument to its layer ----
+class _LinkingConfig(C.Structure):
+    _fields_ = [("variant", _i32), ("normalised_sum", _i32), ("has_weight", _i32), ("number_of_value_chunks", _u32),
+                ("number_of_zeroing_chunks", _u32), ("table_bit_size", _u32), ("table_is_signed", _i32), ("input_sign_negative", _i32),
+                ("min_output_value", C.c_int64), ("max_output_value", C.c_int64), ("rank", _u32), ("unpadded_input_shape", _vp)]
+
+
+host.dph_linking_prove.restype = _i32
+host.dph_linking_prove.argtypes = [_vp, _vp, _vp, _u32, _vp, _vp, _u32, _vp, _u32, _vp, _vp, _u64, _vp]
+host.dph_linking_verify.restype = _i32
+host.dph_linking_verify.argtypes = [_vp, _vp, _vp, _u32, _u32, _vp, _u32, _vp, _vp, _u32, _vp, _u32, _vp, _vp]
+LINKING_VARIANTS = {"standard": 0, "glu": 1, "softmax": 2, "normalisation": 3}
+
+
+def _linking_config(cfg):
+    shape = (_u64 * len(cfg["shape"]))(*cfg["shape"])
+    c = _LinkingConfig(LINKING_VARIANTS[cfg["variant"]], int(cfg.get("norm_sum", False)), int(cfg.get("has_weight", False)),
+                       cfg["value_chunks"], cfg["zero_chunks"], cfg["bit_size"], int(cfg["signed"]),
+                       int(cfg.get("input_sign", "positive") == "negative"), cfg.get("min_out", 0), cfg.get("max_out", 0), len(cfg["shape"]),
+                       C.cast(shape, _vp))
+    return c, shape
+
+
+def linking_prove(ctx, cfg, mles, transcript, last_claim_point, logup_point, weight=None):
+    """LookupInputConfig::prove_linking_sumcheck.  cfg: dict with variant ('standard', 'glu', 'softmax',
+    'normalisation'), shape (unpadded input shape), value_chunks, zero_chunks, bit_size, signed, min_out,
+    max_out, input_sign, norm_sum, has_weight.  mles: the witness tables in the expression's order.
+    Returns (proof[n, d+1, 2], point[n, 2], evaluations[len(mles), 2], weight evaluation or None, challenges)."""
+    c, keep = _linking_config(cfg)
+    hs = (_vp * max(1, len(mles)))(*[m.handle for m in mles])
+    lcp, lp = _e2(last_claim_point).reshape(-1, 2), _e2(logup_point).reshape(-1, 2)
+    cap = 1 << 16
+    out = np.zeros(cap, dtype=np.uint64)
+    n = _u64(0)
+    ctx._chk_host(host.dph_linking_prove(ctx._c, C.byref(c), hs, len(mles), None if weight is None else weight.handle, _ptr(lcp), lcp.shape[0],
+                                         _ptr(lp), lp.shape[0], transcript._t, _ptr(out), cap, C.byref(n)), "dph_linking_prove")
+    w = out[: n.value]
+    proof, pos = _parse_proof(w, 0)
+    ne = int(w[pos])
+    pos += 1
+    evals = w[pos:pos + 2 * ne].reshape(ne, 2).copy()
+    pos += 2 * ne
+    weight_eval = None
+    if int(w[pos]):
+        weight_eval = w[pos + 1:pos + 3].copy()
+        pos += 2
+    pos += 1
+    rounds = proof.shape[0]
+    point = w[pos:pos + 2 * rounds].reshape(rounds, 2).copy()
+    pos += 2 * rounds
+    nc = int(w[pos])
+    challenges = w[pos + 1:pos + 1 + 2 * nc].reshape(nc, 2).copy()
+    return proof, point, evals, weight_eval, challenges
+
+
+def linking_verify(cfg, initial_claim, proof, evaluations, weight_eval, transcript, last_claim_point, logup_point):
+    """LookupInputConfig::verify_linking_sumcheck from the claimed sum on.  Returns (status, point); status 0 = accepted."""
+    c, keep = _linking_config(cfg)
+    proof = np.ascontiguousarray(_e2(proof))
+    evaluations = np.ascontiguousarray(_e2(evaluations)).reshape(-1, 2)
+    lcp, lp = _e2(last_claim_point).reshape(-1, 2), _e2(logup_point).reshape(-1, 2)
+    claim = np.ascontiguousarray(_e2(initial_claim))
+    we = None if weight_eval is None else np.ascontiguousarray(_e2(weight_eval))
+    point = np.zeros((proof.shape[0], 2), dtype=np.uint64)
+    rc = host.dph_linking_verify(C.byref(c), _ptr(claim), _ptr(proof), proof.shape[0], proof.shape[1], _ptr(evaluations), evaluations.shape[0],
+                                 None if we is None else _ptr(we), _ptr(lcp), lcp.shape[0], _ptr(lp), lp.shape[0], transcript._t, _ptr(point))
+    return rc, point

@@ -114,6 +114,39 @@ int32_t dph_same_poly_prove(dps_ctx *ctx, const dps_mle *poly, uint32_t n_claims
 int32_t dph_same_poly_verify(uint32_t num_vars, uint32_t n_claims, const uint64_t *points, const uint64_t *evals, const uint64_t *proof,
                              const uint64_t *eval, dph_transcript *t, uint64_t *point_out);
 
+/* ---- the sumcheck linking a lookup argument to its layer ----
+ * LookupInputConfig::prove_linking_sumcheck (zkml/src/lookup/operation/inputs/proving.rs:26-114) with
+ * the expression of LookupVariant::build_full_sumcheck_expression (variant.rs:55-348).  The
+ * configuration carries what that expression reads from the layer: */
+typedef struct dph_linking_config {
+    int32_t variant;        /* 0 Standard, 1 GLU, 2 Softmax, 3 Normalisation */
+    int32_t normalised_sum; /* Normalisation: normalised_sum_value is Some */
+    int32_t has_weight;     /* Normalisation: has_weight */
+    uint32_t number_of_value_chunks, number_of_zeroing_chunks; /* ChunkingInfo */
+    uint32_t table_bit_size;                                   /* Table::table_bit_size */
+    int32_t table_is_signed;
+    int32_t input_sign_negative; /* unsigned tables: TableSign::Negative (else Positive) */
+    int64_t min_output_value, max_output_value;
+    uint32_t rank;
+    const uint64_t *unpadded_input_shape;
+} dph_linking_config;
+/* mles: the witness tables in the expression's order (per 2-D chunk its value chunks then its zeroing
+ * chunks; then, GLU: one table per chunk; Normalisation: the input chunks, then the scaling tables),
+ * each with the variables of the padded last two dimensions.  weight: the Normalisation weight table or
+ * NULL.  Points: 2 limbs per coordinate.  Output words: rounds, points per round, the round messages,
+ * n_evaluations, the evaluations of `mles` at the sumcheck point, has_weight_eval (0/1) [+ that
+ * evaluation], the sumcheck point (rounds elements), n_challenges, the batching challenges. */
+int32_t dph_linking_prove(dps_ctx *ctx, const dph_linking_config *cfg, const dps_mle *const *mles, uint32_t n_mles, const dps_mle *weight,
+                          const uint64_t *last_claim_point, uint32_t last_claim_len, const uint64_t *logup_point, uint32_t logup_len,
+                          dph_transcript *t, uint64_t *out, uint64_t out_cap, uint64_t *n_words);
+/* verify_linking_sumcheck (inputs/verifying.rs:236-330) from the initial claim on: the claimed sum
+ * (LookupVariant::prepare_sumcheck_verification's result) is the caller's.  DPS_OK and the sumcheck
+ * point when the proof verifies. */
+int32_t dph_linking_verify(const dph_linking_config *cfg, const uint64_t initial_claim[2], const uint64_t *proof, uint32_t n_rounds,
+                           uint32_t points_per_round, const uint64_t *evaluations, uint32_t n_evaluations, const uint64_t *weight_eval,
+                           const uint64_t *last_claim_point, uint32_t last_claim_len, const uint64_t *logup_point, uint32_t logup_len,
+                           dph_transcript *t, uint64_t *point_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,6 +5,7 @@
 
 #include "dpsc/einsum.hpp"
 #include "dpsc/logup.hpp"
+#include "dpsc/lookup_linking.hpp"
 #include "dpsc/poly_commit.hpp"
 #include "dpsc/same_poly.hpp"
 #include "dpsc/sumcheck.hpp"
@@ -450,6 +451,91 @@ int32_t dph_same_poly_verify(uint32_t num_vars, uint32_t n_claims, const uint64_
         for (size_t i = 0; i < claim.point.size(); i++) {
             point_out[2 * i] = claim.point[i].c0;
             point_out[2 * i + 1] = claim.point[i].c1;
+        }
+    });
+}
+
+namespace {
+
+lookup::LookupInputConfig linking_config(const dph_linking_config *cfg)
+{
+    if (!cfg || !cfg->unpadded_input_shape || cfg->rank == 0) throw Error(DPS_ERR_INVALID, "linking sumcheck: null configuration");
+    if (cfg->variant < 0 || cfg->variant > 3) throw Error(DPS_ERR_INVALID, "linking sumcheck: unknown variant");
+    lookup::ChunkingInfo ci;
+    ci.number_of_value_chunks = cfg->number_of_value_chunks;
+    ci.number_of_zeroing_chunks = cfg->number_of_zeroing_chunks;
+    ci.table_bit_size = cfg->table_bit_size;
+    ci.table_is_signed = cfg->table_is_signed != 0;
+    ci.min_output_value = cfg->min_output_value;
+    ci.max_output_value = cfg->max_output_value;
+    ci.input_sign = cfg->input_sign_negative ? lookup::TableSign::Negative : lookup::TableSign::Positive;
+    lookup::LookupVariant v;
+    v.kind = (lookup::Variant)cfg->variant;
+    v.normalised_sum = cfg->normalised_sum != 0;
+    v.has_weight = cfg->has_weight != 0;
+    return lookup::LookupInputConfig(ci, v, std::vector<uint64_t>(cfg->unpadded_input_shape, cfg->unpadded_input_shape + cfg->rank));
+}
+
+}  // namespace
+
+int32_t dph_linking_prove(dps_ctx *ctx, const dph_linking_config *cfg, const dps_mle *const *mles, uint32_t n_mles, const dps_mle *weight,
+                          const uint64_t *last_claim_point, uint32_t last_claim_len, const uint64_t *logup_point, uint32_t logup_len,
+                          dph_transcript *t, uint64_t *out, uint64_t out_cap, uint64_t *n_words)
+{
+    return guarded([&] {
+        Context c(ctx);
+        auto config = linking_config(cfg);
+        std::vector<DensePolynomial> tabs;
+        tabs.reserve(n_mles + 1);
+        for (uint32_t i = 0; i < n_mles; i++) tabs.push_back(DensePolynomial::borrowed(c, mles[i]));
+        if (weight) tabs.push_back(DensePolynomial::borrowed(c, weight));
+        std::vector<const DensePolynomial *> ptrs;
+        for (uint32_t i = 0; i < n_mles; i++) ptrs.push_back(&tabs[i]);
+        auto res = config.prove_linking_sumcheck(ptrs, t->t, from_limbs(last_claim_point, last_claim_len), from_limbs(logup_point, logup_len),
+                                                 weight ? &tabs.back() : nullptr);
+        std::vector<uint64_t> w;
+        auto put = [&](const F &x) {
+            w.push_back(x.c0);
+            w.push_back(x.c1);
+        };
+        const auto &pr = res.first;
+        w.push_back(pr.sumcheck_proof.proofs.size());
+        w.push_back(pr.sumcheck_proof.proofs.empty() ? 0 : pr.sumcheck_proof.proofs[0].evaluations.size());
+        for (auto &m : pr.sumcheck_proof.proofs)
+            for (auto &e : m.evaluations) put(e);
+        w.push_back(pr.evaluations.size());
+        for (auto &e : pr.evaluations) put(e);
+        w.push_back(pr.has_weight_eval ? 1 : 0);
+        if (pr.has_weight_eval) put(pr.weight_eval);
+        for (auto &x : pr.sumcheck_point) put(x);
+        w.push_back(res.second.size());
+        for (auto &x : res.second) put(x);
+        if (w.size() > out_cap) throw Error(DPS_ERR_INVALID, "dph_linking_prove: output buffer too small");
+        memcpy(out, w.data(), w.size() * 8);
+        *n_words = w.size();
+    });
+}
+
+int32_t dph_linking_verify(const dph_linking_config *cfg, const uint64_t initial_claim[2], const uint64_t *proof, uint32_t n_rounds,
+                           uint32_t points_per_round, const uint64_t *evaluations, uint32_t n_evaluations, const uint64_t *weight_eval,
+                           const uint64_t *last_claim_point, uint32_t last_claim_len, const uint64_t *logup_point, uint32_t logup_len,
+                           dph_transcript *t, uint64_t *point_out)
+{
+    return guarded([&] {
+        auto config = linking_config(cfg);
+        lookup::LookupSumcheckProof pr;
+        for (uint32_t j = 0; j < n_rounds; j++)
+            pr.sumcheck_proof.proofs.push_back(IOPProverMessage{from_limbs(proof + 2 * (size_t)points_per_round * j, points_per_round)});
+        pr.evaluations = from_limbs(evaluations, n_evaluations);
+        if (weight_eval) {
+            pr.has_weight_eval = true;
+            pr.weight_eval = F(weight_eval[0], weight_eval[1]);
+        }
+        auto res = config.verify_linking_sumcheck(pr, F(initial_claim[0], initial_claim[1]), t->t, from_limbs(last_claim_point, last_claim_len),
+                                                  from_limbs(logup_point, logup_len));
+        for (size_t i = 0; i < res.second.size(); i++) {
+            point_out[2 * i] = res.second[i].c0;
+            point_out[2 * i + 1] = res.second[i].c1;
         }
     });
 }

@@ -562,5 +562,225 @@ def same_poly_verify(num_vars, claims, proof, eval_, transcript):
     return bool((e2_mul(_e2arr(eval_), computed) == expected).all()), point
 
 
+# ---- sumcheck linking a lookup argument to its layer (zkml/src/lookup/operation) ----
+# The expression is built as a polynomial in the witness tables with the challenges
+# already substituted: a dict {sorted tuple of table indices: coefficient}.
+# Pinned by tests/test_oracle_linking.py: the sum the proof opens with equals the
+# protocol's statement recomputed entry by entry with Python integers.  Parity unpinned:
+# the degree the prover declares when the top-degree monomials' coefficients are zero
+# (here: the degree of the surviving monomials), and everything the sumcheck engine
+# itself leaves unpinned (message layout, transcript bytes, binding order).
+class _Poly:
+    def __init__(self, terms=None):
+        self.t = terms or {}
+
+    @staticmethod
+    def const(c):
+        return _Poly({(): _e2arr(c)})
+
+    @staticmethod
+    def const_i64(x):
+        return _Poly({(): e2(gl_from_i64(x))})
+
+    @staticmethod
+    def wit(i):
+        return _Poly({(i,): e2(1)})
+
+    def __add__(self, o):
+        out = dict(self.t)
+        for k, v in o.t.items():
+            out[k] = e2_add(out[k], v) if k in out else v
+        return _Poly(out)
+
+    def __neg__(self):
+        return _Poly({k: e2_sub(e2(0), v) for k, v in self.t.items()})
+
+    def __sub__(self, o):
+        return self + (-o)
+
+    def __mul__(self, o):
+        out = {}
+        for ka, va in self.t.items():
+            for kb, vb in o.t.items():
+                k = tuple(sorted(ka + kb))
+                v = e2_mul(va, vb)
+                out[k] = e2_add(out[k], v) if k in out else v
+        return _Poly(out)
+
+    def terms(self):
+        return [(v, list(k)) for k, v in sorted(self.t.items()) if v.any()]
+
+
+def split_point(padded_shape, point):
+    """Shape::split_point (zkml/src/shape.rs:475-496): the last dimension takes the lowest variables."""
+    point = _e2arr(point).reshape(-1, 2)
+    out, start = [None] * len(padded_shape), 0
+    for a in reversed(range(len(padded_shape))):
+        ln = max(0, (padded_shape[a] - 1).bit_length())
+        out[a] = point[start:start + ln]
+        start += ln
+    assert start == len(point)
+    return out
+
+
+def eq_point_and_batching_challenges(shape, point):
+    """Shape::compute_eq_point_and_batching_challenges (zkml/src/shape.rs:565-610): the variables of the last
+    two dimensions form the eq point; the leading dimensions turn into one coefficient per 2-D chunk."""
+    padded = [1 << max(0, (d - 1).bit_length()) for d in shape]
+    skip = max(0, len(shape) - 2)
+    eq_pt, bc = np.zeros((0, 2), dtype=np.uint64), [e2(1)]
+    for i, (dp, size) in enumerate(zip(split_point(padded, point), shape)):
+        if i < skip:
+            ev = eq_evals(dp)[:size]
+            bc = [e2_mul(c, e) for c in bc for e in ev]
+        else:
+            eq_pt = np.concatenate([dp, eq_pt])
+    return eq_pt, bc
+
+
+def _linking_chunks(cfg):
+    n = 1
+    for d in cfg["shape"][:max(0, len(cfg["shape"]) - 2)]:
+        n *= d
+    return n
+
+
+def _linking_extra_per_chunk(cfg):
+    return {"standard": 0, "softmax": 0, "glu": 1, "normalisation": 2}[cfg["variant"]]
+
+
+def linking_expression(cfg, ch):
+    """LookupVariant::build_full_sumcheck_expression with the challenges `ch` substituted
+    (zkml/src/lookup/operation/variant.rs:55-348, 475-522).  cfg: variant ('standard', 'glu', 'softmax',
+    'normalisation'), shape (unpadded input shape), value_chunks, zero_chunks, bit_size, signed, min_out,
+    max_out, input_sign ('positive' / 'negative', unsigned tables), norm_sum, has_weight."""
+    nvc, nz, bits = cfg["value_chunks"], cfg["zero_chunks"], cfg["bit_size"]
+    chunks = _linking_chunks(cfg)
+    per_chunk = nvc + nz
+    total_out = chunks * per_chunk
+    total_wit = chunks * _linking_extra_per_chunk(cfg) + total_out
+    one, W, K = _Poly.const(e2(1)), _Poly.wit, _Poly.const_i64
+    spow = lambda k: _Poly.const(_pow_e2(ch[0], k))
+    out_eq, logup_eq, norm_eq = W(total_wit), W(total_wit + 1), W(total_wit + 2)
+    final_dim_log = max(0, (cfg["shape"][-1] - 1).bit_length())
+    pow_two = K(1 << final_dim_log)
+    full = _Poly()
+    for c in range(chunks):
+        off = c * per_chunk
+        # the value the chunk's lookups stand for, and the start of the linear combination (variant.rs:475-522)
+        if nvc == 1:
+            value, total, wo, sco = W(off), W(off) * spow(1), off + 1, 2
+        else:
+            value, total = K(-(1 << (nvc * bits - 1))), _Poly()
+            for i in range(nvc):
+                value = value + K(1 << (bits * i)) * (W(off + i) + K(1 << (bits - 1)))
+                total = total + W(off + i) * spow(i + 1)
+            wo, sco = off + nvc, 1 + nvc
+        # zeroing chunks (variant.rs:95-220)
+        sq_clamp = _Poly()
+        if cfg["signed"]:
+            prod = one
+            for i in range(max(0, nz - 1)):
+                prod = prod * W(wo + i)
+                total = total + W(wo + i) * spow(sco + i)
+            if nz:
+                if nvc == 1:
+                    cmin, cmax = cfg["min_out"], cfg["max_out"]
+                else:
+                    cmin, cmax = -(1 << (nvc * bits - 1)), (1 << (nvc * bits - 1)) - 1
+                last, lower = W(wo - 1 + nz), prod
+                omt = one - last * last
+                prod = prod * omt
+                total = total + last * spow(sco - 1 + nz)
+                half = _Poly.const(e2_inv(e2(2)))
+                first = last * (last + one) * half + (omt - lower * omt)
+                second = last * (last - one) * half
+                clamp = first * K(cmax) + second * K(cmin)
+                if cfg["variant"] == "normalisation":
+                    sq_clamp = first * K(cmax) * K(cmax) + second * K(cmin) * K(cmin)
+            else:
+                clamp = _Poly()
+        else:
+            prod = one
+            for i in range(nz):
+                prod = prod * W(wo + i)
+                total = total + W(wo + i) * spow(sco + i)
+            # without zeroing chunks the reference's clamping term is the constant one (variant.rs:200-203)
+            clamp = K(cfg["max_out"] if cfg["input_sign"] == "positive" else cfg["min_out"]) if nz else one
+        prod_expr = clamp + prod * value
+        cc = _Poly.const(ch[1 + c])
+        v = cfg["variant"]
+        if v == "standard":
+            e = cc * (out_eq * prod_expr + logup_eq * total)
+        elif v == "glu":
+            e = cc * (out_eq * prod_expr * W(total_out + c) + logup_eq * total)
+        elif v == "softmax":
+            nc = _Poly.const(ch[1 + chunks]) * pow_two
+            e = cc * (out_eq * prod_expr + nc * (norm_eq * prod_expr) + logup_eq * total)
+        else:
+            sq_expr = sq_clamp + prod * value * value
+            sumsq_c = _Poly.const(ch[1 + chunks]) * pow_two
+            oeq = out_eq * W(total_wit + 3) if cfg["has_weight"] else out_eq
+            part = oeq * prod_expr
+            if cfg["norm_sum"]:
+                part = part + _Poly.const(_pow_e2(ch[1 + chunks], 2)) * pow_two * (norm_eq * prod_expr)
+            e = cc * (part + sumsq_c * (norm_eq * sq_expr)
+                      + logup_eq * (total + _Poly.const(ch[2 + chunks]) * (W(total_out + c) * W(total_out + chunks + c))))
+        full = full + e
+    return full.terms()
+
+
+def _linking_setup(cfg, last_claim_point, logup_point, transcript):
+    eq_pt, bc = eq_point_and_batching_challenges(cfg["shape"], last_claim_point)
+    ch = [transcript.append_and_sample(b"sum")] + bc
+    if cfg["variant"] in ("softmax", "normalisation"):
+        ch.append(transcript.append_and_sample(b"normalisation"))
+    if cfg["variant"] == "normalisation":
+        ch.append(transcript.append_and_sample(b"input"))
+    logup_point = _e2arr(logup_point).reshape(-1, 2)
+    eq_points = [eq_pt, logup_point]
+    if cfg["variant"] in ("softmax", "normalisation"):
+        fd = max(0, (cfg["shape"][-1] - 1).bit_length())
+        half = e2_inv(e2(2))
+        eq_points.append(np.concatenate([np.tile(half, (fd, 1)), logup_point[fd:]]))
+    return eq_pt, ch, eq_points
+
+
+def linking_prove(cfg, mles, transcript, last_claim_point, logup_point, weight=None):
+    """LookupInputConfig::prove_linking_sumcheck (zkml/src/lookup/operation/inputs/proving.rs:26-114).
+    Returns (proof, point, evaluations of `mles`, weight evaluation or None, batching challenges)."""
+    eq_pt, ch, eq_points = _linking_setup(cfg, last_claim_point, logup_point, transcript)
+    tables = [_e2arr(m).reshape(-1, 2) for m in mles] + [eq_evals(p) for p in eq_points]
+    if weight is not None:
+        tables.append(_e2arr(weight).reshape(-1, 2))
+    terms = linking_expression(cfg, ch)
+    proof, point, finals = sc_prove(len(eq_pt), tables, terms, transcript)
+    return proof, point, finals[:len(mles)], (finals[-1] if weight is not None else None), ch
+
+
+def linking_verify(cfg, initial_claim, proof, evaluations, weight_eval, transcript, last_claim_point, logup_point):
+    """LookupInputConfig::verify_linking_sumcheck (inputs/verifying.rs:236-330) from the initial claim on
+    (prepare_sumcheck_verification is the caller's).  Returns (ok, point, batching challenges)."""
+    eq_pt, ch, eq_points = _linking_setup(cfg, last_claim_point, logup_point, transcript)
+    terms = linking_expression(cfg, ch)
+    degree = max(len(f) for _, f in terms)
+    proof = _e2arr(proof)
+    if proof.shape[0] != len(eq_pt) or proof.shape[1] != degree + 1:
+        return False, None, ch
+    bad, point, expected = sc_verify(initial_claim, proof, transcript)
+    if bad:
+        return False, point, ch
+    wit = [_e2arr(v) for v in _e2arr(evaluations).reshape(-1, 2)] + [identity_eval(p, point) if len(p) else e2(1) for p in eq_points]
+    if weight_eval is not None:
+        wit.append(_e2arr(weight_eval))
+    total = e2(0)
+    for coeff, fs in terms:
+        v = coeff
+        for f in fs:
+            v = e2_mul(v, wit[f])
+        total = e2_add(total, v)
+    return bool((total == expected).all()), point, ch
+
+
 def num_threads():
     return lib().orc_num_threads()

@@ -117,6 +117,18 @@ def protocol_vectors():
     t = orc.OracleTranscript(b"golden")
     proof, point, ev = orc.same_poly_prove(poly, cl, t)
     out["same_poly"] = dict(poly_seed=40, point_seeds=[41, 42, 43], proof=hx(proof), point=hx(point), eval=hx(ev), state=st(t))
+    # the lookup-linking sumcheck: a signed table with one zeroing chunk (3 chunks), and the weighted normalisation variant
+    from linking_cases import CASES, make_instance as linking_instance
+
+    out["linking"] = []
+    for case, seed in ((1, 60), (9, 61)):
+        tabs, weight, lcp, lp = linking_instance(CASES[case], seed)
+        t = orc.OracleTranscript(b"golden")
+        proof, point, evals, weight_eval, ch = orc.linking_prove(CASES[case], [orc.embed_i64(x) for x in tabs], t, lcp, lp,
+                                                                 None if weight is None else orc.embed_i64(weight))
+        out["linking"].append(dict(instance=f"linking_cases.make_instance(CASES[{case}], {seed})", case=case, seed=seed, proof=hx(proof), point=hx(point),
+                                   evals=hx(evals), weight_eval=None if weight_eval is None else hx(weight_eval), challenges=hx(np.stack(ch)),
+                                   state=st(t)))
     return out
 
 

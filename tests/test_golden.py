@@ -133,3 +133,18 @@ def test_gpu_matches_protocol_vectors(dp, ctx, orc):
     t = dp.Transcript(b"golden")
     proof, point, ev = dp.same_poly_prove(ctx, ctx.mle_from_ext2(poly), cl, t)
     assert (proof.reshape(-1) == _u(sp["proof"])).all() and (ev == _u(sp["eval"])).all() and t.state()[0].hex() == sp["state"]["state"]
+
+    from linking_cases import CASES, chunk_vars, make_instance as linking_instance
+
+    for lk in pv["linking"]:
+        cfg = CASES[lk["case"]]
+        tabs, weight, lcp, lp = linking_instance(cfg, lk["seed"])
+        nv = chunk_vars(cfg)
+        t = dp.Transcript(b"golden")
+        proof, point, evals, weight_eval, ch = dp.linking_prove(ctx, cfg, [ctx.mle_from_i64(x, nv) for x in tabs], t, lcp, lp,
+                                                                None if weight is None else ctx.mle_from_i64(weight, nv))
+        assert (proof.reshape(-1) == _u(lk["proof"])).all() and (evals.reshape(-1) == _u(lk["evals"])).all()
+        assert (ch.reshape(-1) == _u(lk["challenges"])).all() and t.state()[0].hex() == lk["state"]["state"]
+        assert (weight_eval is None) == (lk["weight_eval"] is None)
+        if weight_eval is not None:
+            assert (weight_eval == _u(lk["weight_eval"])).all()
