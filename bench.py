@@ -129,6 +129,24 @@ def other_config(args):
             cpu_ms, _, ref = _timed(cpu, 1, 0)
             got = run()
             exact = bool((got[0] == ref[0]).all() and (got[1] == ref[1]).all())
+    elif cfg == "linking":
+        # the activation after GPT-2's MLP up-projection, [512 x 3072], through a signed 8-bit table with one zeroing chunk
+        lcfg = dict(variant="standard", shape=[512, 3072], value_chunks=1, zero_chunks=1, bit_size=8, signed=True, min_out=-128, max_out=127,
+                    input_sign="positive", norm_sum=False, has_weight=False)
+        nv = 9 + 12
+        rng = np.random.Generator(np.random.PCG64(91))
+        value = rng.integers(-128, 128, size=1 << nv, dtype=np.int64)
+        top = rng.integers(-1, 2, size=1 << nv, dtype=np.int64)
+        lcp, lp = np.stack([rand_base(nv, 92), rand_base(nv, 93)], axis=-1), np.stack([rand_base(nv, 94), rand_base(nv, 95)], axis=-1)
+        gpu = [ctx.mle_from_i64(value, nv), ctx.mle_from_i64(top, nv)]
+        run = lambda: dp.linking_prove(ctx, lcfg, gpu, dp.Transcript(b"bench"), lcp, lp)
+        workload = "lookup-linking sumcheck of a [512 x 3072] activation: signed 8-bit table, one value chunk + one zeroing chunk, 21 variables, degree 4"
+        metric = "lookup linking prove ms"
+        if orc:
+            tabs = [orc.embed_i64(value), orc.embed_i64(top)]
+            cpu_ms, _, ref = _timed(lambda: orc.linking_prove(lcfg, tabs, orc.OracleTranscript(b"bench"), lcp, lp), 2, 0)
+            got = run()
+            exact = bool((got[0] == ref[0]).all() and (got[2] == ref[2]).all())
     else:
         # the reference's test_poly_commit shape with chunks of 2^10 (zkml/src/poly_commit/mod.rs:224-409)
         rng = np.random.Generator(np.random.PCG64(77))
@@ -173,7 +191,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--nvars", type=int, default=24, help="variables of the sum (24 is the benchmark configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", default="3", choices=["1", "2", "3", "4", "5", "opening"],
+    ap.add_argument("--config", default="3", choices=["1", "2", "3", "4", "5", "opening", "linking"],
                     help="3 (default) is the benchmark configuration; the others time the remaining configurations the same way")
     args = ap.parse_args()
     if args.gpus != 1:

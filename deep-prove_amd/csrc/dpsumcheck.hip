@@ -1222,6 +1222,7 @@ struct dps_sc {
     std::vector<u32> poly_term_begin, poly_term_end;
     std::vector<int> poly_owner;              // per session table: the group that writes its fold, -1 = in no group
     u32 poly_max_tabs;                        // sizes the kernel's LDS
+    u32 poly_split_cap;                       // log2 of the most lanes a pair's work is worth spreading over
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
     std::vector<dpk::PolyGroup> h_poly_groups;  // host copies: a single group travels in the kernel arguments
@@ -1316,6 +1317,72 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
     default: return fail(ctx, DPS_ERR_UNSUPPORTED, "no fused kernel for degree %u", nf);
     }
     return DPS_OK;
+}
+
+// Rounds of at most this many pairs run on poly_split_kernel
+constexpr u64 POLY_SPLIT_MAX_PAIRS = 1ull << 16;
+
+// lanes per pair (log2) and grid of a split round: about 2^17 threads while that many items exist; a round
+// that fits one workgroup takes the lanes the workgroup has
+void poly_split_plan(u64 n_pairs, u32 cap, u32 *split_log, u32 *blocks)
+{
+    u32 lp = log2u(n_pairs);
+    u32 sl = n_pairs <= dpk::BLOCK ? log2u(dpk::BLOCK) - lp : (lp < 17 ? 17 - lp : 0);
+    sl = std::min(sl, cap);
+    *split_log = sl;
+    *blocks = (u32)std::max<u64>(1, (n_pairs << sl) / dpk::BLOCK);
+}
+
+template <int NF, bool EQ, bool SKIP1>
+int32_t launch_poly_split_one(dps_ctx *ctx, dpk::PolyArgs &a, dim3 grid, u32 max_tabs, bool want_state, u64 *partial, const dpk::FastFin &ff)
+{
+    // value and slope of every table, per pair; resident launches add the folded tables themselves
+    const size_t lds_vals = (size_t)std::max<u32>(max_tabs, 1) * 4 * dpk::BLOCK * 8;
+    const size_t lds_state = (size_t)std::max<u32>(max_tabs, 1) * 2 * 2 * dpk::BLOCK * 8;
+    size_t lds = lds_vals;
+    a.lds_state = 0;
+    a.state_off = (u32)(lds_vals / 8);
+    if (want_state) {
+        // more dynamic LDS than a launch gets by default: asked for once per kernel and device
+        static int granted[64] = {0};  // 0 not asked, 1 granted, 2 refused
+        int &gr = granted[ctx->device & 63];
+        if (gr == 0) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dpk::poly_split_kernel<NF, EQ, SKIP1>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(dpk::POLY_MAXT * 8 * dpk::BLOCK * 8));
+            gr = e == hipSuccess ? 1 : 2;
+            if (e != hipSuccess) (void)hipGetLastError();
+        }
+        if (gr == 1 || lds_vals + lds_state + 8192 <= 65536) {
+            a.lds_state = 1;
+            lds = lds_vals + lds_state;
+        }
+    }
+    dpk::poly_split_kernel<NF, EQ, SKIP1><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
+    return DPS_OK;
+}
+
+template <int NF>
+int32_t launch_poly_split(dps_ctx *ctx, bool eq, bool skip1, dpk::PolyArgs &a, dim3 grid, u32 max_tabs, bool want_state, u64 *partial,
+                          const dpk::FastFin &ff)
+{
+    if (eq && skip1) return launch_poly_split_one<NF, true, true>(ctx, a, grid, max_tabs, want_state, partial, ff);
+    if (eq) return launch_poly_split_one<NF, true, false>(ctx, a, grid, max_tabs, want_state, partial, ff);
+    if (skip1) return launch_poly_split_one<NF, false, true>(ctx, a, grid, max_tabs, want_state, partial, ff);
+    return launch_poly_split_one<NF, false, false>(ctx, a, grid, max_tabs, want_state, partial, ff);
+}
+
+int32_t launch_poly_split_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, dpk::PolyArgs &a, dim3 grid, u32 max_tabs, bool want_state,
+                                   u64 *partial, const dpk::FastFin &ff)
+{
+    switch (nf) {
+    case 1: return launch_poly_split<1>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    case 2: return launch_poly_split<2>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    case 3: return launch_poly_split<3>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    case 4: return launch_poly_split<4>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    case 5: return launch_poly_split<5>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    case 6: return launch_poly_split<6>(ctx, eq, skip1, a, grid, max_tabs, want_state, partial, ff);
+    default: return fail(ctx, DPS_ERR_UNSUPPORTED, "no fused kernel for degree %u", nf);
+    }
 }
 
 u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
@@ -1706,6 +1773,21 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     for (u32 k = 0; k < n_mles; k++) gath.push_back(dpk::GatherDesc{sim[k].c0, sim[k].c1});
 
     sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
+    sc->poly_split_cap = 0;
+    if (sc->poly) {
+        // items of a pair: (evaluation point, term) products; tables to fold
+        u32 most_terms = 0;
+        for (size_t g = 0; g < sc->poly_tabs.size(); g++) most_terms = std::max(most_terms, sc->poly_term_end[g] - sc->poly_term_begin[g]);
+        const u32 items = std::max<u32>(most_terms * std::max<u32>(sc->fast_nf, 1), sc->poly_max_tabs);
+        sc->poly_split_cap = std::min<u32>(4, log2u(std::max<u32>(items, 1)));
+        for (u32 j = 1; j <= n_vars; j++) {
+            const u64 np = 1ull << (n_vars - j);
+            if (np > POLY_SPLIT_MAX_PAIRS) continue;
+            u32 sl, bl;
+            poly_split_plan(np, sc->poly_split_cap, &sl, &bl);
+            sc->max_blocks = std::max(sc->max_blocks, bl);
+        }
+    }
     size_t bytes_fold = round_up(folds.size() * sizeof(dpk::FoldDesc), 256);
     size_t bytes_fold_x = round_up(folds_extra.size() * sizeof(dpk::FoldDesc), 256);
     size_t bytes_terms = round_up(tdescs.size() * sizeof(dpk::TermDesc), 256);
@@ -2040,18 +2122,27 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.eq1 = sc->eq_c1;
             pa.mail = ctx->d_pinned + (ctx->res_off - 64);
             pa.seq = fa.seq;
+            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = 0;
+            // few pairs: the work of a pair is spread over several lanes
+            const bool split = n_pairs <= POLY_SPLIT_MAX_PAIRS;
+            u32 sblocks = blocks;
+            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, &pa.split_log, &sblocks);
+            pa.split_cap = sc->poly_split_cap;
             // a single workgroup from here on: it stays for the remaining rounds
-            const bool reside = n_groups == 1 && blocks == 1 && a.skip1 && j < sc->n_vars;
+            const bool reside = split && n_groups == 1 && sblocks == 1 && a.skip1 && j < sc->n_vars;
             if (reside) {
                 pa.groups = sc->d_poly_groups + (size_t)(j - 1);
                 pa.last_round = sc->n_vars;
             }
-            ff.n_blocks = blocks * n_groups;
+            ff.n_blocks = sblocks * n_groups;
             double pbytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
             for (u32 k = 0; k < sc->n_mles; k++)
                 if (sc->poly_owner[k] >= 0) pbytes += (double)n_pairs * (j >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
             ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
-            CHK(launch_poly_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(blocks, n_groups), sc->poly_max_tabs, sc->d_partial, ff));
+            if (split)
+                CHK(launch_poly_split_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(sblocks, n_groups), sc->poly_max_tabs, reside, sc->d_partial, ff));
+            else
+                CHK(launch_poly_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(blocks, n_groups), sc->poly_max_tabs, sc->d_partial, ff));
             HIPCHK(ctx, hipGetLastError());
             if (reside) {
                 sc->tail_running = true;

@@ -1042,9 +1042,10 @@ struct PolyArgs {
     const u64 *q1;
     u64 n_pairs;
     u64 r0, r1;
-    // Resident rounds (single-workgroup launches only): after round j the workgroup stays, waits for the next
-    // challenge in the host's mailbox as tail_kernel does, and runs the following rounds up to last_round on the
-    // tables it folded itself.  `groups` then holds one descriptor per round, starting with this launch's.
+    // Resident rounds (poly_split_kernel, single-workgroup launches only): after round j the workgroup stays, waits
+    // for the next challenge in the host's mailbox as tail_kernel does, and runs the following rounds up to
+    // last_round on the tables it folded itself.  `groups` then holds one descriptor per round, starting with
+    // this launch's.
     u32 j;           // this launch's round (1-based)
     u32 last_round;  // 0: exit after round j
     u32 n_vars;
@@ -1053,6 +1054,10 @@ struct PolyArgs {
     const u64 *eq1;
     const u64 *mail;
     u64 seq;         // sequence number of round j; round j + k waits for mail seq + k
+    u32 split_log;   // 2^split_log lanes share a pair in round j
+    u32 split_cap;   // resident rounds: the share doubles as the pairs halve, up to 2^split_cap lanes
+    u32 lds_state;   // resident rounds: the folded tables stay in LDS (state_off words into the dynamic LDS)
+    u32 state_off;
 };
 
 template <int NF, bool EQ, bool SKIP1>
@@ -1067,22 +1072,17 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     // a dependent load of its own (the small rounds are nothing but such latencies), so they are staged in LDS once.
     __shared__ PolyGroup g;
     __shared__ PolyTerm lterms[POLY_LDS_TERMS];
-    __shared__ u64 box[MAIL_WORDS];
-    __shared__ int ok_flag;
     const u32 tid = threadIdx.x;
     auto cur0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 0) * BLOCK + tid]; };
     auto cur1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 1) * BLOCK + tid]; };
     auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
     auto dl1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 3) * BLOCK + tid]; };
-    u32 j = a.j;
-    u64 n_pairs = a.n_pairs;
-    E2 r = gl::e2(a.r0, a.r1);
+    const u64 n_pairs = a.n_pairs;
+    const E2 r = gl::e2(a.r0, a.r1);
     const u64 *q0 = a.q0, *q1 = a.q1;
-    FastFin cf = ff;
-  for (;;) {
     {
         const bool inl = a.groups == nullptr;  // a single group handed over in the kernel arguments
-        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + (j - a.j) + blockIdx.y);
+        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + blockIdx.y);
         u64 *dst = reinterpret_cast<u64 *>(&g);
         for (u32 w = tid; w < sizeof(PolyGroup) / 8; w += BLOCK) dst[w] = src[w];
         __syncthreads();
@@ -1090,8 +1090,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
         const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
         u64 *td = reinterpret_cast<u64 *>(lterms);
-        if (j == a.j)
-            for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
         __syncthreads();
     }
     const u32 n_tabs = g.n_tabs;
@@ -1200,6 +1199,205 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
+        fast_finalize<NF>(ff, acc, res);
+        return;
+    }
+    if (tid == 0) {
+        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
+#pragma unroll
+        for (int t = 0; t < NP; t++) {
+            st_agent(o + 2 * t, acc[t].c0);
+            st_agent(o + 2 * t + 1, acc[t].c1);
+        }
+    }
+    if (take_ticket(ff.counter, gridDim.x * gridDim.y, &last_flag)) {
+        E2 q[NP];
+        gather_partials<NP>(ff, lds, q);
+        fast_finalize<NF>(ff, q, res);
+    }
+}
+
+// The same sum for rounds of few pairs, where a launch is one serial chain per thread: the work of a pair is
+// spread over 2^split_log adjacent lanes.  First the pair's tables are divided among the lanes (each loads,
+// folds and stores its tables and leaves value and slope in LDS), then the (point, term) products are: lane l
+// takes every item q = point_position * n_terms + term with q = l mod 2^split_log, reading a factor at point t
+// as value + t * slope.  Sums are exact in the field, so the message is the one poly_kernel computes.
+// A single-workgroup launch stays resident as described at PolyArgs; with lds_state the tables it folds stay
+// in LDS from one round to the next (they still go to device memory, where the final evaluations are read).
+template <int NF, bool EQ, bool SKIP1>
+__global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__restrict__ partial, FastFin ff)
+{
+    constexpr int NP = NF + 1;
+    extern __shared__ u64 dyn[];  // [n_tabs][4][BLOCK] value c0, c1, slope c0, c1 per pair; at state_off [n_tabs][2][2 * BLOCK] folded tables
+    __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
+    __shared__ u64 res[6 * MAX_PTS];
+    __shared__ int last_flag;
+    __shared__ PolyGroup g;
+    __shared__ PolyTerm lterms[POLY_LDS_TERMS];
+    __shared__ u64 box[MAIL_WORDS];
+    __shared__ int ok_flag;
+    const u32 tid = threadIdx.x;
+    u32 j = a.j;
+    u64 n_pairs = a.n_pairs;
+    E2 r = gl::e2(a.r0, a.r1);
+    const u64 *q0 = a.q0, *q1 = a.q1;
+    FastFin cf = ff;
+    u32 sl = a.split_log;
+    u32 in_lds = 0;  // tables (bit per slot) whose current contents this workgroup holds in LDS
+    u64 *const state = dyn + a.state_off;
+  for (;;) {
+    {
+        const bool inl = a.groups == nullptr;
+        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + (j - a.j) + blockIdx.y);
+        u64 *dst = reinterpret_cast<u64 *>(&g);
+        for (u32 w = tid; w < sizeof(PolyGroup) / 8; w += BLOCK) dst[w] = src[w];
+        __syncthreads();
+        const u32 nt = g.term_end - g.term_begin;
+        const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
+        const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
+        u64 *td = reinterpret_cast<u64 *>(lterms);
+        if (j == a.j)
+            for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        __syncthreads();
+    }
+    const u32 n_tabs = g.n_tabs;
+    const u32 n_terms = g.term_end - g.term_begin;
+    const gl::E2P rp = gl::prep(r);
+    const u32 S = 1u << sl, sub = tid & (S - 1), pib = tid >> sl, ppb = BLOCK >> sl;
+    auto val = [&](u32 k, u32 c) -> u64 & { return dyn[(k * 4 + c) * BLOCK + pib]; };
+    u32 wrote = 0;  // tables this round folds and stores
+    for (u32 k = 0; k < n_tabs; k++)
+        if (g.tab[k].mode == POLY_PAIR_FOLD && g.tab[k].d0) wrote |= 1u << k;
+
+    gl::E2Acc lz[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) lz[t] = gl::e2acc_zero();
+
+    // the bounds are the same for every thread of the workgroup: the barriers inside are reached by all
+    for (u64 base = (u64)blockIdx.x * ppb; base < n_pairs; base += (u64)gridDim.x * ppb) {
+        const u64 i = base + pib;
+        const bool active = i < n_pairs;
+        // tables sub, sub + S, ... of the pair: all loads first
+        U64x2 a0[POLY_MAXT], b0[POLY_MAXT], a1[POLY_MAXT], b1[POLY_MAXT];
+#pragma unroll
+        for (int m = 0; m < POLY_MAXT; m++) {
+            const u32 k = sub + (u32)m * S;
+            a0[m] = b0[m] = a1[m] = b1[m] = U64x2{0, 0};
+            if (active && k < n_tabs) {
+                const PolyTab &tb = g.tab[k];
+                if (tb.mode == POLY_PAIR_FOLD) {
+                    if ((in_lds >> k) & 1) {
+                        const u64 *c0 = state + (size_t)(k * 2 + 0) * 2 * BLOCK, *c1 = state + (size_t)(k * 2 + 1) * 2 * BLOCK;
+                        a0[m] = U64x2{c0[4 * i], c0[4 * i + 1]};
+                        b0[m] = U64x2{c0[4 * i + 2], c0[4 * i + 3]};
+                        a1[m] = U64x2{c1[4 * i], c1[4 * i + 1]};
+                        b1[m] = U64x2{c1[4 * i + 2], c1[4 * i + 3]};
+                    } else {
+                        a0[m] = ld2(tb.s0 + 4 * i);
+                        b0[m] = ld2(tb.s0 + 4 * i + 2);
+                        if (tb.s1) {
+                            a1[m] = ld2(tb.s1 + 4 * i);
+                            b1[m] = ld2(tb.s1 + 4 * i + 2);
+                        }
+                    }
+                } else if (tb.mode == POLY_PAIR) {
+                    a0[m] = ld2(tb.s0 + 2 * i);
+                    if (tb.s1) a1[m] = ld2(tb.s1 + 2 * i);
+                } else {
+                    const u64 e = i >> tb.shift;
+                    a0[m].x = tb.s0[e];
+                    if (tb.s1) a1[m].x = tb.s1[e];
+                }
+            }
+        }
+        // the folded tables go where other lanes have just read: every read first
+        if (in_lds) __syncthreads();
+#pragma unroll
+        for (int m = 0; m < POLY_MAXT; m++) {
+            const u32 k = sub + (u32)m * S;
+            if (active && k < n_tabs) {
+                const PolyTab &tb = g.tab[k];
+                E2 lo, hi;
+                if (tb.mode == POLY_PAIR_FOLD) {
+                    if (tb.s1 || ((in_lds >> k) & 1)) {
+                        lo = fold1p(gl::e2(a0[m].x, a1[m].x), gl::e2(a0[m].y, a1[m].y), rp);
+                        hi = fold1p(gl::e2(b0[m].x, b1[m].x), gl::e2(b0[m].y, b1[m].y), rp);
+                    } else {
+                        lo = fold1_base(a0[m].x, a0[m].y, r);
+                        hi = fold1_base(b0[m].x, b0[m].y, r);
+                    }
+                    if (tb.d0) {
+                        st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
+                        st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
+                        if (a.lds_state) {
+                            u64 *c0 = state + (size_t)(k * 2 + 0) * 2 * BLOCK, *c1 = state + (size_t)(k * 2 + 1) * 2 * BLOCK;
+                            c0[2 * i] = lo.c0;
+                            c0[2 * i + 1] = hi.c0;
+                            c1[2 * i] = lo.c1;
+                            c1[2 * i + 1] = hi.c1;
+                        }
+                    }
+                } else if (tb.mode == POLY_PAIR) {
+                    lo = gl::e2(a0[m].x, a1[m].x);
+                    hi = gl::e2(a0[m].y, a1[m].y);
+                } else {
+                    lo = hi = gl::e2(a0[m].x, a1[m].x);
+                }
+                const E2 d = gl::sub(hi, lo);
+                val(k, 0) = lo.c0;
+                val(k, 1) = lo.c1;
+                val(k, 2) = d.c0;
+                val(k, 3) = d.c1;
+            }
+        }
+        __syncthreads();
+        if (active) {
+            gl::E2P restp = gl::prep(gl::e2_one());
+            if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
+            // items q = position of the point * n_terms + term; this lane's are sub, sub + S, ...  The point is a
+            // run-time value, so the lanes of a wavefront run the same instructions whatever item each one holds.
+            constexpr u32 NPE = SKIP1 ? NP - 1 : NP;
+            u32 tpos = 0, jj = sub;
+            while (jj >= n_terms && tpos < NPE) {
+                jj -= n_terms;
+                tpos++;
+            }
+            while (tpos < NPE) {
+                const u32 t = (SKIP1 && tpos >= 1) ? tpos + 1 : tpos;
+                auto at = [&](u32 k) {
+                    const E2 d = gl::mul_base(gl::e2(val(k, 2), val(k, 3)), (u64)t);
+                    return gl::add(gl::e2(val(k, 0), val(k, 1)), d);
+                };
+                const PolyTerm &tm = jj < (u32)POLY_LDS_TERMS ? lterms[jj] : a.terms[g.term_begin + jj];
+                gl::E2P cp;
+                cp.c0 = tm.c0;
+                cp.c1 = tm.c1;
+                cp.w = tm.w;
+                E2 w = gl::e2(tm.c0, tm.c1);
+                if (tm.n_factors > 0) {
+                    E2 prod = at(tm.slot[0]);
+                    for (u32 f = 1; f < tm.n_factors; f++) prod = gl::mulp(prod, gl::prep(at(tm.slot[f])));
+                    w = gl::mulp(prod, cp);
+                }
+                if (EQ) w = gl::mulp(w, restp);
+#pragma unroll
+                for (int tt = 0; tt < NP; tt++)
+                    if ((u32)tt == t) gl::acc_e2(lz[tt], w);
+                jj += S;
+                while (jj >= n_terms && tpos < NPE) {
+                    jj -= n_terms;
+                    tpos++;
+                }
+            }
+        }
+        // value and slope are overwritten by the next step
+        __syncthreads();
+    }
+    E2 acc[NP];
+#pragma unroll
+    for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
+    block_reduce<NP>(acc, lds);
+    if (gridDim.x * gridDim.y == 1) {
         fast_finalize<NF>(cf, acc, res);
         if (a.last_round == 0 || j >= a.last_round) return;
         // stay for the next round: its challenge and the scalars of its message arrive by mail
@@ -1209,6 +1407,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
         r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
         n_pairs >>= 1;
+        if (sl < a.split_cap && (n_pairs << (sl + 1)) <= (u64)BLOCK) sl++;
         if (EQ) {
             const u64 off = (2ull << a.n_vars) - (2ull << (a.n_vars - j));
             q0 = a.eq0 + off;
@@ -1226,10 +1425,15 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         cf.const0 = box[MAIL_CONST];
         cf.const1 = box[MAIL_CONST + 1];
         cf.seq = a.seq + (j - a.j);
-        // the tables this workgroup folded and stored are read back by other lanes: stores done, then no stale L1 lines
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (a.lds_state) {
+            in_lds = wrote;
+            __syncthreads();
+        } else {
+            // the tables this workgroup folded and stored are read back by other lanes: stores done, then no stale L1 lines
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        }
         continue;
     }
     if (tid == 0) {
