@@ -1223,6 +1223,8 @@ struct dps_sc {
     std::vector<int> poly_owner;              // per session table: the group that writes its fold, -1 = in no group
     u32 poly_max_tabs;                        // sizes the kernel's LDS
     u32 poly_split_cap;                       // log2 of the most lanes a pair's work is worth spreading over
+    bool descs_uploaded;                      // the descriptor block is on the device (uploaded when first needed)
+    bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
     std::vector<dpk::PolyGroup> h_poly_groups;  // host copies: a single group travels in the kernel arguments
@@ -1386,6 +1388,20 @@ int32_t launch_poly_split_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, dp
 }
 
 u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
+
+}  // namespace
+
+namespace {
+
+// one staged upload of all descriptors; not waited for (the staging vector lives as long as the session)
+int32_t ensure_descs(dps_sc *sc)
+{
+    if (sc->descs_uploaded || sc->stage.empty()) return DPS_OK;
+    hipError_t e = hipMemcpyAsync(sc->dev_block, sc->stage.data(), sc->stage.size(), hipMemcpyHostToDevice, sc->ctx->stream);
+    if (e != hipSuccess) return fail(sc->ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e));
+    sc->descs_uploaded = true;
+    return DPS_OK;
+}
 
 }  // namespace
 
@@ -1774,7 +1790,11 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
 
     sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
     sc->poly_split_cap = 0;
+    sc->poly_finish_in_kernel = false;
     if (sc->poly) {
+        sc->poly_finish_in_kernel = sc->poly_tabs.size() == 1;
+        for (u32 k = 0; k < n_mles; k++)
+            if (sc->poly_owner[k] != 0 && (int)k != sc->fast_eq) sc->poly_finish_in_kernel = false;
         // items of a pair: (evaluation point, term) products; tables to fold
         u32 most_terms = 0;
         for (size_t g = 0; g < sc->poly_tabs.size(); g++) most_terms = std::max(most_terms, sc->poly_term_end[g] - sc->poly_term_begin[g]);
@@ -1838,11 +1858,15 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     if (!poly_groups.empty()) memcpy(q, poly_groups.data(), poly_groups.size() * sizeof(dpk::PolyGroup));
     q += bytes_pg;
     if (!poly_terms.empty()) memcpy(q, poly_terms.data(), poly_terms.size() * sizeof(dpk::PolyTerm));
-    // a product session that ends in the resident kernel reads none of the descriptors
-    const bool needs_descs = !(sc->fast && sc->tail_j0);
-    if (!stage.empty() && needs_descs) {
-        hipError_t e = hipMemcpyAsync(sc->dev_block, stage.data(), stage.size(), hipMemcpyHostToDevice, ctx->stream);
-        if (e != hipSuccess) return cleanup(fail(ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e)));
+    // Sessions whose launches carry their descriptors themselves (a product session that ends in the resident kernel; a
+    // single group of terms, inline in the kernel arguments or staged in pinned memory for the resident launch) upload
+    // nothing unless a step outside that flow needs the block (ensure_descs).
+    sc->descs_uploaded = false;
+    const bool self_contained = (sc->fast && sc->tail_j0) ||
+                                (sc->poly && sc->poly_tabs.size() == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS);
+    if (!self_contained) {
+        rc = ensure_descs(sc.get());
+        if (rc != DPS_OK) return cleanup(rc);
     }
     *out = sc.release();
     return DPS_OK;
@@ -1862,6 +1886,7 @@ int32_t launch_folds(dps_sc *sc, u32 step, bool extra_only, const u64 *chal)
     dps_ctx *ctx = sc->ctx;
     u32 cnt = extra_only ? sc->fold_extra_cnt[step] : sc->fold_cnt[step];
     if (!cnt) return DPS_OK;
+    CHK(ensure_descs(sc));
     const dpk::FoldDesc *d = extra_only ? sc->d_fold_extra + sc->fold_extra_off[step] : sc->d_fold + sc->fold_off[step];
     // the grid is sized for the largest table that can fold in this step; smaller (zero-padded) ones leave blocks idle
     u32 prev_live = sc->n_vars - (step - 1) + 1;
@@ -1934,6 +1959,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
     fa.partial = sc->d_partial;
     fa.blocks_per_term = sc->n_terms ? blocks : 0;
     fa.n_terms = sc->n_terms;
+    if (!sc->fast && !sc->poly) CHK(ensure_descs(sc));
     fa.terms = sc->d_fin;
     fa.degree = sc->degree;
     fa.total_blocks = blocks * sc->n_terms;
@@ -2084,11 +2110,12 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                     // the resident launch of an earlier round runs this one
                     post_mail();
                     int32_t rc = wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
-                    if (rc != DPS_OK || j == sc->n_vars) {
-                        // it exits by itself after the last round
+                    if (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel)) {
+                        // without a finishing step of its own it exits after the last round
                         sc->tail_running = false;
                         ctx->tail_owner = nullptr;
                     }
+                    // else it waits for the last challenge (dps_sc_finish)
                     CHK(rc);
                     took_round();
                     return DPS_OK;
@@ -2104,10 +2131,14 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u32 n_groups = (u32)sc->poly_tabs.size();
             pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
             pa.terms = sc->d_poly_terms;
-            if (n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS) {
+            const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
+            if (inline_descs) {
                 pa.groups = nullptr;
+                pa.terms = nullptr;
                 pa.g0 = sc->h_poly_groups[j - 1];
                 std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+            } else {
+                CHK(ensure_descs(sc));
             }
             pa.q0 = a.q0;
             pa.q1 = a.q1;
@@ -2122,17 +2153,27 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.eq1 = sc->eq_c1;
             pa.mail = ctx->d_pinned + (ctx->res_off - 64);
             pa.seq = fa.seq;
-            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = 0;
+            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = pa.pad = 0;
+            pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
             // few pairs: the work of a pair is spread over several lanes
             const bool split = n_pairs <= POLY_SPLIT_MAX_PAIRS;
             u32 sblocks = blocks;
             if (split) poly_split_plan(n_pairs, sc->poly_split_cap, &pa.split_log, &sblocks);
             pa.split_cap = sc->poly_split_cap;
             // a single workgroup from here on: it stays for the remaining rounds
-            const bool reside = split && n_groups == 1 && sblocks == 1 && a.skip1 && j < sc->n_vars;
+            const bool reside = split && n_groups == 1 && sblocks == 1 && a.skip1 && j < sc->n_vars &&
+                                sc->n_vars - j + 1 <= (u32)dpk::POLY_RES_ROUNDS;
             if (reside) {
-                pa.groups = sc->d_poly_groups + (size_t)(j - 1);
                 pa.last_round = sc->n_vars;
+                if (inline_descs) {
+                    // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
+                    // before its first round, and this call returns only after that round's message has arrived
+                    const size_t words = (size_t)(sc->n_vars - j + 1) * sizeof(dpk::PolyGroup) / 8;
+                    memcpy(ctx->h_pinned, &sc->h_poly_groups[j - 1], words * 8);
+                    pa.groups = reinterpret_cast<const dpk::PolyGroup *>(ctx->d_pinned);
+                } else {
+                    pa.groups = sc->d_poly_groups + (size_t)(j - 1);
+                }
             }
             ff.n_blocks = sblocks * n_groups;
             double pbytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
@@ -2199,17 +2240,18 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         mb[dpk::MAIL_R] = challenge[0];
         mb[dpk::MAIL_R + 1] = challenge[1];
         send_mail(ctx, seq);
-        u64 fin[2 * 3];
-        int32_t rc = wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * sc->fast_nf, fin);
-        // the kernel exits right after publishing
-        hipError_t e = hipStreamSynchronize(ctx->stream);
+        u64 fin[2 * dpk::POLY_MAXT];
+        // the fused multi-term kernel publishes its group's tables in slot order, the single-product one its factors
+        const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[0].size() : sc->fast_nf;
+        int32_t rc = wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin);
+        // the kernel exits right after publishing and reads nothing more; whatever is launched next follows it on the stream
         sc->tail_running = false;
         ctx->tail_owner = nullptr;
         if (rc != DPS_OK) return rc;
-        if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "tail kernel: %s", hipGetErrorString(e));
-        for (u32 f = 0; f < sc->fast_nf; f++) {
-            final_evals_out[2 * sc->fast_order[f]] = fin[2 * f];
-            final_evals_out[2 * sc->fast_order[f] + 1] = fin[2 * f + 1];
+        for (u32 f = 0; f < n_fin; f++) {
+            const u32 k = sc->poly ? sc->poly_tabs[0][f] : sc->fast_order[f];
+            final_evals_out[2 * k] = fin[2 * f];
+            final_evals_out[2 * k + 1] = fin[2 * f + 1];
         }
         if (sc->fast_eq >= 0) {
             E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], gl::e2(challenge[0], challenge[1])));
@@ -2222,6 +2264,7 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
     if (sc->n_vars >= 1) CHK(launch_folds(sc, sc->n_vars + 1, sc->fast || sc->poly, challenge));
     if (sc->n_mles) {
         if (2 * (size_t)sc->n_mles > ctx->res_off - 64) return fail(ctx, DPS_ERR_UNSUPPORTED, "too many tables in one session");
+        CHK(ensure_descs(sc));
         dpk::gather_kernel<<<(sc->n_mles + 63) / 64, 64, 0, ctx->stream>>>(sc->d_gather, sc->n_mles, ctx->d_pinned);
         HIPCHK(ctx, hipGetLastError());
     }
@@ -2253,7 +2296,9 @@ extern "C" int32_t dps_sc_free(dps_sc *sc)
     dps_ctx *ctx = sc->ctx;
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
-    (void)hipStreamSynchronize(ctx->stream);
+    // a descriptor upload may still be reading the session's staging vector; the device blocks need no wait,
+    // whoever gets them next uses them in stream order
+    if (sc->descs_uploaded) (void)hipStreamSynchronize(ctx->stream);
     pool_free(ctx, sc->scratch);
     pool_free(ctx, sc->dev_block);
     delete sc;

@@ -1007,6 +1007,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
 // ---------------------------------------------------------------------------
 constexpr int POLY_MAXT = 7;
 constexpr int POLY_LDS_TERMS = 48;  // terms of a group kept in LDS; further ones are read from device memory
+constexpr int POLY_RES_ROUNDS = 9;  // rounds one resident launch can run: from 256 pairs down to one
 constexpr u32 POLY_PAIR = 0, POLY_PAIR_FOLD = 1, POLY_BCAST = 2;
 
 struct PolyTab {
@@ -1034,8 +1035,8 @@ struct PolyTerm {
 static_assert(sizeof(PolyTerm) % 8 == 0 && sizeof(PolyGroup) % 8 == 0, "descriptors are copied as 64-bit words");
 
 struct PolyArgs {
-    const PolyGroup *groups;  // one per grid row, this round's; nullptr: the single group and its terms are in g0 / t0
-    const PolyTerm *terms;
+    const PolyGroup *groups;  // one per grid row, this round's; nullptr: the single group is in g0
+    const PolyTerm *terms;    // nullptr: the terms are in t0
     PolyGroup g0;
     PolyTerm t0[POLY_LDS_TERMS];
     const u64 *q0;  // eq suffix table of this round (common eq factor only)
@@ -1058,6 +1059,8 @@ struct PolyArgs {
     u32 split_cap;   // resident rounds: the share doubles as the pairs halve, up to 2^split_cap lanes
     u32 lds_state;   // resident rounds: the folded tables stay in LDS (state_off words into the dynamic LDS)
     u32 state_off;
+    u32 finish;      // resident rounds: stay after the last round for the last challenge and publish the final evaluations
+    u32 pad;
 };
 
 template <int NF, bool EQ, bool SKIP1>
@@ -1232,7 +1235,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
-    __shared__ PolyGroup g;
+    __shared__ PolyGroup gall[POLY_RES_ROUNDS];  // the descriptors of every round this launch runs
     __shared__ PolyTerm lterms[POLY_LDS_TERMS];
     __shared__ u64 box[MAIL_WORDS];
     __shared__ int ok_flag;
@@ -1245,21 +1248,24 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     u32 sl = a.split_log;
     u32 in_lds = 0;  // tables (bit per slot) whose current contents this workgroup holds in LDS
     u64 *const state = dyn + a.state_off;
-  for (;;) {
     {
-        const bool inl = a.groups == nullptr;
-        const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + (j - a.j) + blockIdx.y);
-        u64 *dst = reinterpret_cast<u64 *>(&g);
-        for (u32 w = tid; w < sizeof(PolyGroup) / 8; w += BLOCK) dst[w] = src[w];
+        // Descriptors and terms are staged in LDS once: read where they lie (kernel arguments, device memory, or for a
+        // resident launch pinned host memory) every use would be a dependent load of its own.  A resident launch has
+        // a single group, whose descriptors for rounds j, j + 1, ... follow each other.
+        const u32 n_rounds = a.last_round ? a.last_round - a.j + 1 : 1;
+        const u64 *src = a.groups ? reinterpret_cast<const u64 *>(a.groups + blockIdx.y) : reinterpret_cast<const u64 *>(&a.g0);
+        u64 *dst = reinterpret_cast<u64 *>(gall);
+        for (u32 w = tid; w < n_rounds * (u32)(sizeof(PolyGroup) / 8); w += BLOCK) dst[w] = src[w];
         __syncthreads();
-        const u32 nt = g.term_end - g.term_begin;
+        const u32 nt = gall[0].term_end - gall[0].term_begin;
         const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
-        const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
+        const u64 *ts = a.terms ? reinterpret_cast<const u64 *>(a.terms + gall[0].term_begin) : reinterpret_cast<const u64 *>(a.t0);
         u64 *td = reinterpret_cast<u64 *>(lterms);
-        if (j == a.j)
-            for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
         __syncthreads();
     }
+  for (;;) {
+    const PolyGroup &g = gall[j - a.j];
     const u32 n_tabs = g.n_tabs;
     const u32 n_terms = g.term_end - g.term_begin;
     const gl::E2P rp = gl::prep(r);
@@ -1399,7 +1405,25 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
         fast_finalize<NF>(cf, acc, res);
-        if (a.last_round == 0 || j >= a.last_round) return;
+        if (a.last_round == 0) return;
+        if (j >= a.last_round) {
+            if (!a.finish) return;
+            // after the last round: the last challenge arrives, every table's remaining pair (value and slope are
+            // still in LDS, pair 0) is folded with it, and the final evaluations go to the host in slot order
+            const u64 fin_seq = a.seq + (j - a.j) + 1;
+            if (!tail_wait_mail(a.mail, a.spin_limit, fin_seq, box, &ok_flag)) return;
+            if (tid < n_tabs) {
+                const gl::E2P rl = gl::prep(gl::e2(box[MAIL_R], box[MAIL_R + 1]));
+                const E2 lo = gl::e2(dyn[(tid * 4 + 0) * BLOCK], dyn[(tid * 4 + 1) * BLOCK]);
+                const E2 d = gl::e2(dyn[(tid * 4 + 2) * BLOCK], dyn[(tid * 4 + 3) * BLOCK]);
+                const E2 v = gl::fma(d, rl, lo);
+                res[2 * tid] = v.c0;
+                res[2 * tid + 1] = v.c1;
+            }
+            __syncthreads();
+            if (tid == 0) publish_words(cf.out_host, HOST_FINALS_SLOT, res, 2 * n_tabs, fin_seq);
+            return;
+        }
         // stay for the next round: its challenge and the scalars of its message arrive by mail
         j++;
         if (!tail_wait_mail(a.mail, a.spin_limit, a.seq + (j - a.j), box, &ok_flag)) return;
