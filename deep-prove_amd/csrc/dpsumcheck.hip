@@ -1219,6 +1219,7 @@ struct dps_sc {
     // fused multi-term path: groups of at most POLY_MAXT tables, one grid row each
     bool poly;
     std::vector<std::vector<u32>> poly_tabs;  // per group: session table indices, in slot order
+    std::vector<u32> poly_op_begin, poly_op_end;  // per group: its nested program in h_poly_ops
     std::vector<u32> poly_term_begin, poly_term_end;
     std::vector<int> poly_owner;              // per session table: the group that writes its fold, -1 = in no group
     u32 poly_max_tabs;                        // sizes the kernel's LDS
@@ -1229,6 +1230,8 @@ struct dps_sc {
     dpk::PolyTerm *d_poly_terms;
     std::vector<dpk::PolyGroup> h_poly_groups;  // host copies: a single group travels in the kernel arguments
     std::vector<dpk::PolyTerm> h_poly_terms;
+    std::vector<dpk::PolyOp> h_poly_ops;      // nested programs of the groups (empty: term by term)
+    dpk::PolyOp *d_poly_ops;
     std::vector<char> stage;                  // descriptor upload in flight (no wait at set-up)
 };
 
@@ -1392,6 +1395,71 @@ u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
 }  // namespace
 
 namespace {
+
+// Nested (Horner) form of a group's terms: the table found in most of the remaining terms is factored out of
+// them, recursively.  Appends the program to `ops`; returns its number of products.
+struct HornerTerm {
+    E2 coeff;
+    std::vector<uint8_t> slots;  // remaining factors
+};
+
+u32 horner_build(std::vector<HornerTerm> ts, u32 depth, std::vector<dpk::PolyOp> &ops)
+{
+    auto make = [](u32 kind, u32 d, u32 slot, E2 c) {
+        dpk::PolyOp op;
+        memset(&op, 0, sizeof op);
+        op.c0 = c.c0;
+        op.c1 = c.c1;
+        op.w = gl::mul_small(c.c1, (u32)gl::W);
+        op.code = kind | d << 2 | slot << 8;
+        return op;
+    };
+    u32 products = 0;
+    // terms that end at this node were added to the node's constant by the caller
+    ts.erase(std::remove_if(ts.begin(), ts.end(), [](const HornerTerm &t) { return t.slots.empty(); }), ts.end());
+    while (!ts.empty()) {
+        u32 count[256] = {0};
+        for (const HornerTerm &t : ts) {
+            bool seen[256] = {false};
+            for (uint8_t sl : t.slots)
+                if (!seen[sl]) {
+                    seen[sl] = true;
+                    count[sl]++;
+                }
+        }
+        u32 best = 0;
+        for (u32 sl = 1; sl < 256; sl++)
+            if (count[sl] > count[best]) best = sl;
+        std::vector<HornerTerm> sub, rest;
+        for (HornerTerm &t : ts) {
+            auto it = std::find(t.slots.begin(), t.slots.end(), (uint8_t)best);
+            if (it == t.slots.end()) {
+                rest.push_back(std::move(t));
+            } else {
+                t.slots.erase(it);
+                sub.push_back(std::move(t));
+            }
+        }
+        E2 ends = gl::e2_zero();
+        bool inner = false;
+        for (const HornerTerm &t : sub) {
+            if (t.slots.empty())
+                ends = gl::add(ends, t.coeff);
+            else
+                inner = true;
+        }
+        if (!inner) {
+            ops.push_back(make(dpk::POLY_OP_LEAF, depth, best, ends));
+        } else {
+            ops.push_back(make(dpk::POLY_OP_ENTER, depth + 1, 0, ends));
+            products += horner_build(std::move(sub), depth + 1, ops);
+            ops.push_back(make(dpk::POLY_OP_LEAVE, depth + 1, best, gl::e2_zero()));
+        }
+        products++;
+        ts = std::move(rest);
+    }
+    return products;
+}
 
 // one staged upload of all descriptors; not waited for (the staging vector lives as long as the session)
 int32_t ensure_descs(dps_sc *sc)
@@ -1592,6 +1660,43 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                     }
                     poly_terms.push_back(pt);
                 }
+            // the nested form, where it saves products and fits the kernel's staging area
+            sc->poly_op_begin.assign(groups.size(), 0);
+            sc->poly_op_end.assign(groups.size(), 0);
+            bool use_ops = true;
+            std::vector<dpk::PolyOp> all_ops;
+            u32 plain = 0, nested = 0;
+            for (size_t g = 0; g < groups.size() && use_ops; g++) {
+                std::vector<HornerTerm> ts;
+                E2 root = gl::e2_zero();
+                for (u32 ti = tb[g]; ti < te[g]; ti++) {
+                    const dpk::PolyTerm &pt = poly_terms[ti];
+                    HornerTerm ht;
+                    ht.coeff = gl::e2(pt.c0, pt.c1);
+                    ht.slots.assign(pt.slot, pt.slot + pt.n_factors);
+                    if (ht.slots.empty()) root = gl::add(root, ht.coeff);
+                    plain += pt.n_factors;  // n_factors - 1 products and one for the coefficient
+                    ts.push_back(std::move(ht));
+                }
+                std::vector<dpk::PolyOp> ops;
+                dpk::PolyOp enter;
+                memset(&enter, 0, sizeof enter);
+                enter.c0 = root.c0;
+                enter.c1 = root.c1;
+                enter.code = dpk::POLY_OP_ENTER;
+                ops.push_back(enter);
+                nested += horner_build(std::move(ts), 0, ops);
+                if (ops.size() > (size_t)dpk::POLY_LDS_OPS) use_ops = false;
+                sc->poly_op_begin[g] = (u32)all_ops.size();
+                all_ops.insert(all_ops.end(), ops.begin(), ops.end());
+                sc->poly_op_end[g] = (u32)all_ops.size();
+            }
+            if (use_ops && nested < plain) {
+                sc->h_poly_ops = all_ops;
+            } else {
+                sc->poly_op_begin.assign(groups.size(), 0);
+                sc->poly_op_end.assign(groups.size(), 0);
+            }
         }
     }
 
@@ -1727,6 +1832,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                 pg.n_tabs = (u32)sc->poly_tabs[g].size();
                 pg.term_begin = sc->poly_term_begin[g];
                 pg.term_end = sc->poly_term_end[g];
+                pg.op_begin = sc->poly_op_begin[g];
+                pg.op_end = sc->poly_op_end[g];
                 for (u32 sl = 0; sl < pg.n_tabs; sl++) {
                     const u32 k = sc->poly_tabs[g][sl];
                     const SessMle &s = sim[k];
@@ -1817,7 +1924,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256) + 256;
     size_t bytes_pg = round_up(poly_groups.size() * sizeof(dpk::PolyGroup), 256);
     size_t bytes_pt = round_up(poly_terms.size() * sizeof(dpk::PolyTerm), 256);
-    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_partial + bytes_result;
+    size_t bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
+    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result;
     int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
     if (rc != DPS_OK) return cleanup(rc);
     char *p = (char *)sc->dev_block;
@@ -1835,13 +1943,15 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     p += bytes_pg;
     sc->d_poly_terms = (dpk::PolyTerm *)p;
     p += bytes_pt;
+    sc->d_poly_ops = (dpk::PolyOp *)p;
+    p += bytes_po;
     sc->d_partial = (u64 *)p;
     p += bytes_partial;
     sc->d_result = (u64 *)p;
     sc->d_counter = ctx->d_counter;
     // one staged upload of all descriptors
     std::vector<char> &stage = sc->stage;  // lives as long as the session: the upload is not waited for
-    stage.assign(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt, 0);
+    stage.assign(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po, 0);
     sc->h_poly_groups = poly_groups;
     sc->h_poly_terms = poly_terms;
     char *q = stage.data();
@@ -1858,6 +1968,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     if (!poly_groups.empty()) memcpy(q, poly_groups.data(), poly_groups.size() * sizeof(dpk::PolyGroup));
     q += bytes_pg;
     if (!poly_terms.empty()) memcpy(q, poly_terms.data(), poly_terms.size() * sizeof(dpk::PolyTerm));
+    q += bytes_pt;
+    if (!sc->h_poly_ops.empty()) memcpy(q, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
     // Sessions whose launches carry their descriptors themselves (a product session that ends in the resident kernel; a
     // single group of terms, inline in the kernel arguments or staged in pinned memory for the resident launch) upload
     // nothing unless a step outside that flow needs the block (ensure_descs).
@@ -2132,11 +2244,18 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
             pa.terms = sc->d_poly_terms;
             const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
+            // few pairs: the work of a pair is spread over several lanes (term by term); else one thread per pair
+            const bool split = n_pairs <= POLY_SPLIT_MAX_PAIRS;
+            pa.ops = sc->d_poly_ops;
             if (inline_descs) {
                 pa.groups = nullptr;
                 pa.terms = nullptr;
+                pa.ops = nullptr;
                 pa.g0 = sc->h_poly_groups[j - 1];
-                std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+                if (!split && !sc->h_poly_ops.empty())
+                    memcpy(pa.o0, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
+                else
+                    std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
             } else {
                 CHK(ensure_descs(sc));
             }
@@ -2155,8 +2274,6 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.seq = fa.seq;
             pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = pa.pad = 0;
             pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
-            // few pairs: the work of a pair is spread over several lanes
-            const bool split = n_pairs <= POLY_SPLIT_MAX_PAIRS;
             u32 sblocks = blocks;
             if (split) poly_split_plan(n_pairs, sc->poly_split_cap, &pa.split_log, &sblocks);
             pa.split_cap = sc->poly_split_cap;

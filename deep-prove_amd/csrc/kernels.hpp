@@ -1023,6 +1023,7 @@ struct PolyGroup {
     PolyTab tab[POLY_MAXT];
     u32 n_tabs;
     u32 term_begin, term_end;
+    u32 op_begin, op_end;  // the same terms as a nested (Horner) program, poly_kernel only; empty: evaluate term by term
     u32 pad;
 };
 
@@ -1032,13 +1033,33 @@ struct PolyTerm {
     uint8_t slot[DPS_MAX_FACTORS];  // table slots within the group
     u32 pad;
 };
+// The terms of a group in nested form: factoring the most frequent table out of the terms that contain it, again
+// and again, turns sum_k c_k prod table into a tree whose every edge is one product,
+//     G = c + sum_children table_child * G_child.
+// The tree is walked depth first with one running value per depth:
+//     ENTER d, c      acc[d] = c                          (a node with children; c = coefficient of the term ending here, or 0)
+//     LEAF  d, s, c   acc[d] += table_s * c               (a child without children)
+//     LEAVE d, s      acc[d - 1] += table_s * acc[d]      (back to the parent)
+// and G = acc[0].  One product per edge instead of one per factor and coefficient of every term.
+constexpr u32 POLY_OP_ENTER = 0, POLY_OP_LEAF = 1, POLY_OP_LEAVE = 2;
+struct PolyOp {
+    u64 c0, c1, w;  // coefficient, prepared (ENTER, LEAF)
+    u32 code;       // kind | depth << 2 | slot << 8
+    u32 pad;
+};
+constexpr int POLY_LDS_OPS = POLY_LDS_TERMS * 40 / 32;  // a program shares the terms' place in LDS and in the kernel arguments
+static_assert(sizeof(PolyTerm) == 40 && sizeof(PolyOp) == 32, "terms and operations share storage");
 static_assert(sizeof(PolyTerm) % 8 == 0 && sizeof(PolyGroup) % 8 == 0, "descriptors are copied as 64-bit words");
 
 struct PolyArgs {
     const PolyGroup *groups;  // one per grid row, this round's; nullptr: the single group is in g0
     const PolyTerm *terms;    // nullptr: the terms are in t0
+    const PolyOp *ops;        // poly_kernel, groups with a program: nullptr = the program is in t0 (instead of the terms)
     PolyGroup g0;
-    PolyTerm t0[POLY_LDS_TERMS];
+    union {
+        PolyTerm t0[POLY_LDS_TERMS];
+        PolyOp o0[POLY_LDS_OPS];
+    };
     const u64 *q0;  // eq suffix table of this round (common eq factor only)
     const u64 *q1;
     u64 n_pairs;
@@ -1093,100 +1114,136 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
         const u64 *ts = inl ? reinterpret_cast<const u64 *>(a.t0) : reinterpret_cast<const u64 *>(a.terms + g.term_begin);
         u64 *td = reinterpret_cast<u64 *>(lterms);
-        for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        const u32 no = g.op_end - g.op_begin;  // at most POLY_LDS_OPS
+        if (no) {
+            // a program in the kernel arguments is read from there
+            if (!inl) {
+                const u64 *os = reinterpret_cast<const u64 *>(a.ops + g.op_begin);
+                for (u32 w = tid; w < no * (sizeof(PolyOp) / 8); w += BLOCK) td[w] = os[w];
+            }
+        } else {
+            for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
+        }
         __syncthreads();
     }
     const u32 n_tabs = g.n_tabs;
     const u32 n_terms = g.term_end - g.term_begin;
+    const u32 n_ops = g.op_end - g.op_begin;
+    const PolyOp *lops = reinterpret_cast<const PolyOp *>(lterms);
     const gl::E2P rp = gl::prep(r);
 
-    gl::E2Acc lz[NP];
+    // Few live registers matter more here than loads in flight: the loop is arithmetic, and it is the number of
+    // wavefronts per SIMD that hides the latency of its dependent integer chains.  Tables are taken one at a time.
+    E2 lz[NP];
 #pragma unroll
-    for (int t = 0; t < NP; t++) lz[t] = gl::e2acc_zero();
+    for (int t = 0; t < NP; t++) lz[t] = gl::e2_zero();
+    const bool inl = a.groups == nullptr;
 
     for (u64 i = (u64)blockIdx.x * BLOCK + tid; i < n_pairs; i += (u64)gridDim.x * BLOCK) {
-        // all loads of the step first (statically indexed registers), then the arithmetic
-        U64x2 a0[POLY_MAXT], b0[POLY_MAXT], a1[POLY_MAXT], b1[POLY_MAXT];
-#pragma unroll
-        for (int k = 0; k < POLY_MAXT; k++) {
-            if ((u32)k < n_tabs) {
-                const PolyTab &tb = g.tab[k];
-                a0[k] = b0[k] = a1[k] = b1[k] = U64x2{0, 0};
-                if (tb.mode == POLY_PAIR_FOLD) {
-                    a0[k] = ld2(tb.s0 + 4 * i);
-                    b0[k] = ld2(tb.s0 + 4 * i + 2);
-                    if (tb.s1) {
-                        a1[k] = ld2(tb.s1 + 4 * i);
-                        b1[k] = ld2(tb.s1 + 4 * i + 2);
-                    }
-                } else if (tb.mode == POLY_PAIR) {
-                    a0[k] = ld2(tb.s0 + 2 * i);
-                    if (tb.s1) a1[k] = ld2(tb.s1 + 2 * i);
+        auto take = [&](const PolyTab &tb, u32 k) {
+            E2 lo, hi;
+            if (tb.mode == POLY_PAIR_FOLD) {
+                const U64x2 x0 = ld2(tb.s0 + 4 * i), y0 = ld2(tb.s0 + 4 * i + 2);
+                if (tb.s1) {
+                    const U64x2 x1 = ld2(tb.s1 + 4 * i), y1 = ld2(tb.s1 + 4 * i + 2);
+                    lo = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rp);
+                    hi = fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), rp);
                 } else {
-                    const u64 e = i >> tb.shift;
-                    a0[k].x = tb.s0[e];
-                    if (tb.s1) a1[k].x = tb.s1[e];
+                    lo = fold1_base(x0.x, x0.y, r);
+                    hi = fold1_base(y0.x, y0.y, r);
                 }
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < POLY_MAXT; k++) {
-            if ((u32)k < n_tabs) {
-                const PolyTab &tb = g.tab[k];
-                E2 lo, hi;
-                if (tb.mode == POLY_PAIR_FOLD) {
-                    if (tb.s1) {
-                        lo = fold1p(gl::e2(a0[k].x, a1[k].x), gl::e2(a0[k].y, a1[k].y), rp);
-                        hi = fold1p(gl::e2(b0[k].x, b1[k].x), gl::e2(b0[k].y, b1[k].y), rp);
-                    } else {
-                        lo = fold1_base(a0[k].x, a0[k].y, r);
-                        hi = fold1_base(b0[k].x, b0[k].y, r);
-                    }
-                    if (tb.d0) {
-                        st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
-                        st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
-                    }
-                } else if (tb.mode == POLY_PAIR) {
-                    lo = gl::e2(a0[k].x, a1[k].x);
-                    hi = gl::e2(a0[k].y, a1[k].y);
-                } else {
-                    lo = hi = gl::e2(a0[k].x, a1[k].x);
+                if (tb.d0) {
+                    st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
+                    st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
                 }
-                const E2 d = gl::sub(hi, lo);
-                cur0(k) = lo.c0;
-                cur1(k) = lo.c1;
-                dl0(k) = d.c0;
-                dl1(k) = d.c1;
+            } else if (tb.mode == POLY_PAIR) {
+                const U64x2 x0 = ld2(tb.s0 + 2 * i);
+                U64x2 x1 = U64x2{0, 0};
+                if (tb.s1) x1 = ld2(tb.s1 + 2 * i);
+                lo = gl::e2(x0.x, x1.x);
+                hi = gl::e2(x0.y, x1.y);
+            } else {
+                const u64 e = i >> tb.shift;
+                lo = hi = gl::e2(tb.s0[e], tb.s1 ? tb.s1[e] : 0);
             }
-        }
+            const E2 d = gl::sub(hi, lo);
+            cur0(k) = lo.c0;
+            cur1(k) = lo.c1;
+            dl0(k) = d.c0;
+            dl1(k) = d.c1;
+        };
+        // descriptors in the kernel arguments arrive in scalar registers
+        if (inl)
+            for (u32 k = 0; k < n_tabs; k++) take(a.g0.tab[k], k);
+        else
+            for (u32 k = 0; k < n_tabs; k++) take(g.tab[k], k);
         gl::E2P restp = gl::prep(gl::e2_one());
         if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
 #pragma unroll
         for (int t = 0; t < NP; t++) {
             if (!(t == 1 && SKIP1)) {
-                gl::E2Acc G = gl::e2acc_zero();
-                for (u32 j = 0; j < n_terms; j++) {
-                    const PolyTerm &tm = j < (u32)POLY_LDS_TERMS ? lterms[j] : a.terms[g.term_begin + j];
-                    E2 prod = gl::e2_one();
-                    if (tm.n_factors > 0) {
-                        const u32 s0 = tm.slot[0];
-                        prod = gl::e2(cur0(s0), cur1(s0));
-                        for (u32 f = 1; f < tm.n_factors; f++) {
-                            const u32 sl = tm.slot[f];
-                            prod = gl::mulp(prod, gl::prep(gl::e2(cur0(sl), cur1(sl))));
+                E2 gsum;
+                if (n_ops) {
+                    // the nested program: every index below is a compile-time constant inside its case.  Read from
+                    // the kernel arguments an operation arrives in scalar registers and its branches are uniform.
+                    E2 hv[NF + 2];
+#pragma unroll
+                    for (int d = 0; d < NF + 2; d++) hv[d] = gl::e2_zero();
+                    auto step = [&](const PolyOp &op) {
+                        const u32 kind = op.code & 3, dep = (op.code >> 2) & 7, sl = op.code >> 8;
+                        if (kind == POLY_OP_ENTER) {
+                            const E2 c = gl::e2(op.c0, op.c1);
+#pragma unroll
+                            for (int d = 0; d < NF + 1; d++)
+                                if (dep == (u32)d) hv[d] = c;
+                        } else if (kind == POLY_OP_LEAF) {
+                            gl::E2P cp;
+                            cp.c0 = op.c0;
+                            cp.c1 = op.c1;
+                            cp.w = op.w;
+                            const E2 p = gl::mulp(gl::e2(cur0(sl), cur1(sl)), cp);
+#pragma unroll
+                            for (int d = 0; d < NF + 1; d++)
+                                if (dep == (u32)d) hv[d] = gl::add(hv[d], p);
+                        } else {
+                            const gl::E2P vp = gl::prep(gl::e2(cur0(sl), cur1(sl)));
+                            E2 child = hv[1];
+#pragma unroll
+                            for (int d = 2; d < NF + 1; d++)
+                                if (dep == (u32)d) child = hv[d];
+                            const E2 p = gl::mulp(child, vp);
+#pragma unroll
+                            for (int d = 1; d < NF + 1; d++)
+                                if (dep == (u32)d) hv[d - 1] = gl::add(hv[d - 1], p);
                         }
+                    };
+                    if (inl)
+                        for (u32 o = 0; o < n_ops; o++) step(a.o0[o]);
+                    else
+                        for (u32 o = 0; o < n_ops; o++) step(lops[o]);
+                    gsum = hv[0];
+                } else {
+                    gl::E2Acc G = gl::e2acc_zero();
+                    for (u32 j = 0; j < n_terms; j++) {
+                        const PolyTerm &tm = j < (u32)POLY_LDS_TERMS ? lterms[j] : a.terms[g.term_begin + j];
+                        E2 prod = gl::e2_one();
+                        if (tm.n_factors > 0) {
+                            const u32 s0 = tm.slot[0];
+                            prod = gl::e2(cur0(s0), cur1(s0));
+                            for (u32 f = 1; f < tm.n_factors; f++) {
+                                const u32 sl = tm.slot[f];
+                                prod = gl::mulp(prod, gl::prep(gl::e2(cur0(sl), cur1(sl))));
+                            }
+                        }
+                        gl::E2P cp;
+                        cp.c0 = tm.c0;
+                        cp.c1 = tm.c1;
+                        cp.w = tm.w;
+                        gl::acc_mul(G, prod, cp);
                     }
-                    gl::E2P cp;
-                    cp.c0 = tm.c0;
-                    cp.c1 = tm.c1;
-                    cp.w = tm.w;
-                    gl::acc_mul(G, prod, cp);
+                    gsum = gl::acc_reduce(G);
                 }
-                const E2 gsum = gl::acc_reduce(G);
-                if (EQ)
-                    gl::acc_mul(lz[t], gsum, restp);
-                else
-                    gl::acc_e2(lz[t], gsum);
+                lz[t] = EQ ? gl::fma(gsum, restp, lz[t]) : gl::add(lz[t], gsum);
             }
             if (t + 1 < NP) {
                 // on to t + 1 (the slope is added even when t = 1 is skipped: t = 2 needs it twice)
@@ -1199,7 +1256,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     }
     E2 acc[NP];
 #pragma unroll
-    for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
+    for (int t = 0; t < NP; t++) acc[t] = lz[t];
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
         fast_finalize<NF>(ff, acc, res);
