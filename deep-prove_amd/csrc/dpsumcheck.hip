@@ -1343,7 +1343,8 @@ int32_t launch_poly_split_one(dps_ctx *ctx, dpk::PolyArgs &a, dim3 grid, u32 max
 {
     // value and slope of every table, per pair; resident launches add the folded tables themselves
     const size_t lds_vals = (size_t)std::max<u32>(max_tabs, 1) * 4 * dpk::BLOCK * 8;
-    const size_t lds_state = (size_t)std::max<u32>(max_tabs, 1) * 2 * 2 * dpk::BLOCK * 8;
+    // two buffers of POLY_MAXT tables: 2 * BLOCK and BLOCK entries per limb array
+    const size_t lds_state = (size_t)dpk::POLY_MAXT * 2 * 3 * dpk::BLOCK * 8;
     size_t lds = lds_vals;
     a.lds_state = 0;
     a.state_off = (u32)(lds_vals / 8);
@@ -1353,7 +1354,7 @@ int32_t launch_poly_split_one(dps_ctx *ctx, dpk::PolyArgs &a, dim3 grid, u32 max
         int &gr = granted[ctx->device & 63];
         if (gr == 0) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dpk::poly_split_kernel<NF, EQ, SKIP1>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(dpk::POLY_MAXT * 8 * dpk::BLOCK * 8));
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(dpk::POLY_MAXT * 10 * dpk::BLOCK * 8));
             gr = e == hipSuccess ? 1 : 2;
             if (e != hipSuccess) (void)hipGetLastError();
         }

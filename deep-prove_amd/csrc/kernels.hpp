@@ -1288,7 +1288,7 @@ template <int NF, bool EQ, bool SKIP1>
 __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__restrict__ partial, FastFin ff)
 {
     constexpr int NP = NF + 1;
-    extern __shared__ u64 dyn[];  // [n_tabs][4][BLOCK] value c0, c1, slope c0, c1 per pair; at state_off [n_tabs][2][2 * BLOCK] folded tables
+    extern __shared__ u64 dyn[];  // [n_tabs][4][BLOCK] value c0, c1, slope c0, c1 per pair; at state_off the folded tables
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
@@ -1304,7 +1304,11 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     FastFin cf = ff;
     u32 sl = a.split_log;
     u32 in_lds = 0;  // tables (bit per slot) whose current contents this workgroup holds in LDS
-    u64 *const state = dyn + a.state_off;
+    // resident rounds with lds_state: the folded tables, alternating between a buffer of 2 * BLOCK entries per limb
+    // array and one of BLOCK entries (every round halves them)
+    u64 *const state_a = dyn + a.state_off;
+    u64 *const state_b = state_a + (size_t)POLY_MAXT * 2 * 2 * BLOCK;
+    bool dst_is_a = true;
     {
         // Descriptors and terms are staged in LDS once: read where they lie (kernel arguments, device memory, or for a
         // resident launch pinned host memory) every use would be a dependent load of its own.  A resident launch has
@@ -1328,6 +1332,9 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     const gl::E2P rp = gl::prep(r);
     const u32 S = 1u << sl, sub = tid & (S - 1), pib = tid >> sl, ppb = BLOCK >> sl;
     auto val = [&](u32 k, u32 c) -> u64 & { return dyn[(k * 4 + c) * BLOCK + pib]; };
+    u64 *const state_dst = dst_is_a ? state_a : state_b;
+    const u64 *const state_src = dst_is_a ? state_b : state_a;
+    const u32 state_dst_len = dst_is_a ? 2 * BLOCK : BLOCK, state_src_len = dst_is_a ? BLOCK : 2 * BLOCK;
     u32 wrote = 0;  // tables this round folds and stores
     for (u32 k = 0; k < n_tabs; k++)
         if (g.tab[k].mode == POLY_PAIR_FOLD && g.tab[k].d0) wrote |= 1u << k;
@@ -1340,60 +1347,46 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     for (u64 base = (u64)blockIdx.x * ppb; base < n_pairs; base += (u64)gridDim.x * ppb) {
         const u64 i = base + pib;
         const bool active = i < n_pairs;
-        // tables sub, sub + S, ... of the pair: all loads first
-        U64x2 a0[POLY_MAXT], b0[POLY_MAXT], a1[POLY_MAXT], b1[POLY_MAXT];
-#pragma unroll
-        for (int m = 0; m < POLY_MAXT; m++) {
-            const u32 k = sub + (u32)m * S;
-            a0[m] = b0[m] = a1[m] = b1[m] = U64x2{0, 0};
-            if (active && k < n_tabs) {
-                const PolyTab &tb = g.tab[k];
-                if (tb.mode == POLY_PAIR_FOLD) {
-                    if ((in_lds >> k) & 1) {
-                        const u64 *c0 = state + (size_t)(k * 2 + 0) * 2 * BLOCK, *c1 = state + (size_t)(k * 2 + 1) * 2 * BLOCK;
-                        a0[m] = U64x2{c0[4 * i], c0[4 * i + 1]};
-                        b0[m] = U64x2{c0[4 * i + 2], c0[4 * i + 3]};
-                        a1[m] = U64x2{c1[4 * i], c1[4 * i + 1]};
-                        b1[m] = U64x2{c1[4 * i + 2], c1[4 * i + 3]};
-                    } else {
-                        a0[m] = ld2(tb.s0 + 4 * i);
-                        b0[m] = ld2(tb.s0 + 4 * i + 2);
-                        if (tb.s1) {
-                            a1[m] = ld2(tb.s1 + 4 * i);
-                            b1[m] = ld2(tb.s1 + 4 * i + 2);
-                        }
-                    }
-                } else if (tb.mode == POLY_PAIR) {
-                    a0[m] = ld2(tb.s0 + 2 * i);
-                    if (tb.s1) a1[m] = ld2(tb.s1 + 2 * i);
-                } else {
-                    const u64 e = i >> tb.shift;
-                    a0[m].x = tb.s0[e];
-                    if (tb.s1) a1[m].x = tb.s1[e];
-                }
-            }
-        }
-        // the folded tables go where other lanes have just read: every read first
-        if (in_lds) __syncthreads();
-#pragma unroll
-        for (int m = 0; m < POLY_MAXT; m++) {
-            const u32 k = sub + (u32)m * S;
-            if (active && k < n_tabs) {
+        // tables sub, sub + S, ... of the pair, one at a time (few live registers).  In resident rounds a folded table
+        // is read from one LDS buffer and written to the other, so no lane overwrites what another still has to read.
+        if (active) {
+            for (u32 k = sub; k < n_tabs; k += S) {
                 const PolyTab &tb = g.tab[k];
                 E2 lo, hi;
                 if (tb.mode == POLY_PAIR_FOLD) {
-                    if (tb.s1 || ((in_lds >> k) & 1)) {
-                        lo = fold1p(gl::e2(a0[m].x, a1[m].x), gl::e2(a0[m].y, a1[m].y), rp);
-                        hi = fold1p(gl::e2(b0[m].x, b1[m].x), gl::e2(b0[m].y, b1[m].y), rp);
+                    E2 x0, x1, y0, y1;
+                    bool ext = true;
+                    if ((in_lds >> k) & 1) {
+                        const u64 *c0 = state_src + (size_t)(k * 2 + 0) * state_src_len, *c1 = state_src + (size_t)(k * 2 + 1) * state_src_len;
+                        x0 = gl::e2(c0[4 * i], c1[4 * i]);
+                        x1 = gl::e2(c0[4 * i + 1], c1[4 * i + 1]);
+                        y0 = gl::e2(c0[4 * i + 2], c1[4 * i + 2]);
+                        y1 = gl::e2(c0[4 * i + 3], c1[4 * i + 3]);
                     } else {
-                        lo = fold1_base(a0[m].x, a0[m].y, r);
-                        hi = fold1_base(b0[m].x, b0[m].y, r);
+                        const U64x2 p0 = ld2(tb.s0 + 4 * i), q0v = ld2(tb.s0 + 4 * i + 2);
+                        U64x2 p1 = U64x2{0, 0}, q1v = U64x2{0, 0};
+                        ext = tb.s1 != nullptr;
+                        if (ext) {
+                            p1 = ld2(tb.s1 + 4 * i);
+                            q1v = ld2(tb.s1 + 4 * i + 2);
+                        }
+                        x0 = gl::e2(p0.x, p1.x);
+                        x1 = gl::e2(p0.y, p1.y);
+                        y0 = gl::e2(q0v.x, q1v.x);
+                        y1 = gl::e2(q0v.y, q1v.y);
+                    }
+                    if (ext) {
+                        lo = fold1p(x0, x1, rp);
+                        hi = fold1p(y0, y1, rp);
+                    } else {
+                        lo = fold1_base(x0.c0, x1.c0, r);
+                        hi = fold1_base(y0.c0, y1.c0, r);
                     }
                     if (tb.d0) {
                         st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
                         st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
                         if (a.lds_state) {
-                            u64 *c0 = state + (size_t)(k * 2 + 0) * 2 * BLOCK, *c1 = state + (size_t)(k * 2 + 1) * 2 * BLOCK;
+                            u64 *c0 = state_dst + (size_t)(k * 2 + 0) * state_dst_len, *c1 = state_dst + (size_t)(k * 2 + 1) * state_dst_len;
                             c0[2 * i] = lo.c0;
                             c0[2 * i + 1] = hi.c0;
                             c1[2 * i] = lo.c1;
@@ -1401,10 +1394,14 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
                         }
                     }
                 } else if (tb.mode == POLY_PAIR) {
-                    lo = gl::e2(a0[m].x, a1[m].x);
-                    hi = gl::e2(a0[m].y, a1[m].y);
+                    const U64x2 p0 = ld2(tb.s0 + 2 * i);
+                    U64x2 p1 = U64x2{0, 0};
+                    if (tb.s1) p1 = ld2(tb.s1 + 2 * i);
+                    lo = gl::e2(p0.x, p1.x);
+                    hi = gl::e2(p0.y, p1.y);
                 } else {
-                    lo = hi = gl::e2(a0[m].x, a1[m].x);
+                    const u64 e = i >> tb.shift;
+                    lo = hi = gl::e2(tb.s0[e], tb.s1 ? tb.s1[e] : 0);
                 }
                 const E2 d = gl::sub(hi, lo);
                 val(k, 0) = lo.c0;
@@ -1508,6 +1505,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         cf.seq = a.seq + (j - a.j);
         if (a.lds_state) {
             in_lds = wrote;
+            dst_is_a = !dst_is_a;
             __syncthreads();
         } else {
             // the tables this workgroup folded and stored are read back by other lanes: stores done, then no stale L1 lines
