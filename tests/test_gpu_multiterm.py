@@ -1,0 +1,103 @@
+"""GPU parity of sums of several product terms over shared tables (the fused multi-term kernels) against
+the CPU checker, on seeded random expressions that reach every way such a session can run: rounds of more
+than 2^16 pairs and of few pairs, resident rounds and the finish inside the resident launch, a common eq
+factor or none, more than one group of tables, more terms than are staged on chip, repeated factors,
+tables with fewer variables, tables no term uses, and a round whose claim cannot replace the evaluation at 1."""
+import importlib
+
+import numpy as np
+import pytest
+
+from util import py_rng, rand_base, rand_e2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dp():
+    return importlib.import_module("deep-prove_amd")
+
+
+@pytest.fixture(scope="module")
+def ctx(dp):
+    c = dp.Context(0)
+    yield c
+    c.close()
+
+
+def _instance(ctx, orc, seed, n, table_vars, base, n_terms, max_deg, with_eq, unused=0, eq_point=None):
+    """table_vars: variables of each table (n = full size, fewer = constant in the low variables);
+    base: indices of base-field tables.  Returns (gpu tables, checker tables, terms)."""
+    rng = py_rng(seed)
+    gpu, host = [], []
+    for k, m in enumerate(table_vars):
+        if k in base:
+            v = rand_base(1 << m, seed * 50 + k)
+            gpu.append(ctx.mle_from_base(v))
+            host.append(orc.embed_base(v))
+        else:
+            v = rand_e2(1 << m, seed * 50 + k)
+            gpu.append(ctx.mle_from_ext2(v))
+            host.append(v)
+    used = len(table_vars) - unused
+    terms = []
+    for _ in range(n_terms):
+        deg = rng.randint(1, max_deg)
+        fs = [rng.randrange(used) for _ in range(deg)]
+        coeff = np.array([rng.randrange(1, 1 << 62), rng.randrange(0, 1 << 62)], dtype=np.uint64)
+        terms.append((coeff, fs))
+    if with_eq:
+        pt = rand_e2(n, seed * 50 + 49) if eq_point is None else eq_point
+        gpu.append(ctx.eq_build(pt))
+        host.append(orc.eq_evals(pt))
+        e = len(gpu) - 1
+        terms = [(c, fs + [e]) for c, fs in terms]
+    return gpu, host, terms
+
+
+def _check(dp, ctx, orc, n, gpu, host, terms):
+    tr, otr = dp.Transcript(b"multi"), orc.OracleTranscript(b"multi")
+    proof, point, finals = ctx.sumcheck_prove(n, gpu, terms, tr)
+    oproof, opoint, ofinals = orc.sc_prove(n, host, terms, otr)
+    assert (proof == oproof).all() and (point == opoint).all() and (finals == ofinals).all()
+    assert tr.state() == otr.state()
+
+
+CASES = [
+    # n, table_vars, base, n_terms, max_deg, with_eq, unused
+    dict(n=18, table_vars=[18] * 5, base=[], n_terms=12, max_deg=4, with_eq=True),          # large rounds, nested form, resident finish
+    dict(n=18, table_vars=[18] * 6, base=[0, 1], n_terms=70, max_deg=3, with_eq=False),     # more terms than are staged on chip
+    dict(n=17, table_vars=[17] * 12, base=[3], n_terms=20, max_deg=3, with_eq=True),        # two groups of tables
+    dict(n=12, table_vars=[12] * 8, base=[], n_terms=10, max_deg=3, with_eq=True, unused=1),  # a table no term uses: finish outside
+    dict(n=19, table_vars=[19, 19, 19, 10, 0, 19], base=[0, 1, 2], n_terms=9, max_deg=5, with_eq=False),  # fewer-variable tables, repeats
+    dict(n=9, table_vars=[9] * 4, base=[], n_terms=6, max_deg=3, with_eq=True),             # resident from the first launch
+    dict(n=10, table_vars=[10] * 3, base=[1], n_terms=5, max_deg=6, with_eq=False),          # degree 6
+    dict(n=13, table_vars=[13] * 7, base=[], n_terms=48, max_deg=2, with_eq=True),          # a full group, as many terms as fit
+    dict(n=1, table_vars=[1, 1], base=[], n_terms=3, max_deg=2, with_eq=True),
+    dict(n=2, table_vars=[2, 2, 0], base=[], n_terms=4, max_deg=3, with_eq=False),
+]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_random_expressions_match_checker(dp, ctx, orc, case):
+    c = dict(CASES[case])
+    n = c.pop("n")
+    gpu, host, terms = _instance(ctx, orc, 300 + case, n, **c)
+    _check(dp, ctx, orc, n, gpu, host, terms)
+    # a second proof from the same tables: nothing in a session may change them
+    _check(dp, ctx, orc, n, gpu, host, terms)
+
+
+@pytest.mark.parametrize("n,zero_at", [(10, 0), (10, 4), (12, 9), (12, 11), (6, 2)])
+def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
+    """eq(rho, .) with rho_v = 0 makes the message of round v + 1 vanish at 1: that round must evaluate t = 1
+    itself instead of deriving it from the claim, also when it falls among the resident rounds."""
+    pt = rand_e2(n, 777 + n + zero_at)
+    pt[zero_at] = 0
+    gpu, host, terms = _instance(ctx, orc, 400 + n + zero_at, n, [n] * 4, [], 6, 3, True, eq_point=pt)
+    _check(dp, ctx, orc, n, gpu, host, terms)
+    # the single-product path with the same point
+    f, g = rand_base(1 << n, 5), rand_base(1 << n, 6)
+    one = np.array([1, 0], dtype=np.uint64)
+    _check(dp, ctx, orc, n, [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(pt)],
+           [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(pt)], [(one, [2, 0, 1])])
