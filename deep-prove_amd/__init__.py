@@ -72,6 +72,8 @@ dev.dps_mle_from_tensor.restype = _i32
 dev.dps_mle_from_tensor.argtypes = [_vp, _vp, _vp, _vp, _u32, _vp]
 dev.dps_mle_wrap_device.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_mle_view.argtypes = [_vp, _u64, _u32, _vp]
+dev.dps_eq_build_many.restype = _i32
+dev.dps_eq_build_many.argtypes = [_vp, _vp, _vp, _u32, _vp]
 dev.dps_mle_zero_pad.restype = _i32
 dev.dps_mle_zero_pad.argtypes = [_vp, _u32, _vp]
 dev.dps_debug_field_op.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
@@ -415,6 +417,16 @@ class Context:
         h = _vp()
         self._chk(dev.dps_eq_build(self._c, _ptr(point), point.shape[0], C.byref(h)), "dps_eq_build")
         return Mle(self, h)
+
+    def eq_build_many(self, points):
+        """one eq table per point; the small ones come out of a single launch"""
+        pts = [np.ascontiguousarray(_e2(p).reshape(-1, 2)) for p in points]
+        n = len(pts)
+        ptrs = (_vp * max(1, n))(*[p.ctypes.data for p in pts])
+        ms = (_u32 * max(1, n))(*[p.shape[0] for p in pts])
+        hs = (_vp * max(1, n))()
+        self._chk(dev.dps_eq_build_many(self._c, ptrs, ms, n, hs), "dps_eq_build_many")
+        return [Mle(self, _vp(hs[i])) for i in range(n)]
 
     def partial_eval(self, tensor, padded_dims, unpadded_dims, kinds, points):
         nd = len(padded_dims)

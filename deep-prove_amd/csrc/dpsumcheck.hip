@@ -60,6 +60,8 @@ struct dps_ctx {
     u64 *h_pinned = nullptr;    // host-visible result buffer
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
+    hipEvent_t stage_event = nullptr;  // recorded after a launch that reads the staging region of the pinned buffer
+    bool stage_pending = false;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
     u64 seq = 0;                // last sequence number handed to a launch
     struct dps_sc *tail_owner = nullptr;  // session whose tail kernel is resident on the stream
@@ -385,7 +387,8 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
     if (hipMemcpy(ctx->d_lagrange, lag.data(), lag.size() * 8, hipMemcpyHostToDevice) != hipSuccess) return bail(DPS_ERR_HIP);
     ctx->d_counter = (u32 *)((char *)ctx->d_lagrange + lag_bytes);
     if (hipMemset(ctx->d_counter, 0, 256) != hipSuccess) return bail(DPS_ERR_HIP);
-    ctx->pinned_words = 4096;
+    ctx->pinned_words = 16384;
+    if (hipEventCreateWithFlags(&ctx->stage_event, hipEventDisableTiming) != hipSuccess) return bail(DPS_ERR_HIP);
     // fine-grained host memory: a kernel's system-scope stores become visible to the polling host while the kernel runs
     if (hipHostMalloc((void **)&ctx->h_pinned, ctx->pinned_words * 8, hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess) {
         (void)hipGetLastError();
@@ -406,6 +409,7 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
     (void)hipStreamSynchronize(ctx->stream);
     prof_collect(ctx);
     for (auto e : ctx->ev_pool) (void)hipEventDestroy(e);
+    if (ctx->stage_event) (void)hipEventDestroy(ctx->stage_event);
     for (auto &kv : ctx->free_blocks) (void)hipFree(kv.second);
     for (auto &kv : ctx->live_blocks) (void)hipFree(kv.first);
     if (ctx->d_lagrange) (void)hipFree(ctx->d_lagrange);
@@ -798,6 +802,84 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     t->eq->m = m;
     for (u32 i = 0; i < m; i++) t->eq->point.push_back(gl::e2(point[2 * i], point[2 * i + 1]));
     *out = t;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points, const uint32_t *m, uint32_t count, dps_mle **out)
+{
+    if (!ctx || !out || (count && (!points || !m))) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build_many: bad argument");
+    for (u32 i = 0; i < count; i++) {
+        out[i] = nullptr;
+        if ((m[i] && !points[i]) || m[i] > dpk::EQ_MAX_VARS) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build_many: bad argument (table %u)", i);
+        if (!canonical(points[i], 2 * (size_t)m[i])) return fail(ctx, DPS_ERR_INVALID, "dps_eq_build_many: point %u not canonical", i);
+    }
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    auto undo = [&](int32_t rc) {
+        for (u32 i = 0; i < count; i++) {
+            delete out[i];
+            out[i] = nullptr;
+        }
+        return rc;
+    };
+    // staging region of the pinned buffer: job descriptors, then the points
+    const size_t stage_lo = 1024, stage_hi = ctx->pinned_words / 2;
+    std::vector<dpk::EqJobM> jobs;
+    std::vector<u64> pts;
+    u32 max_bits = 0;
+    auto flush = [&]() -> int32_t {
+        if (jobs.empty()) return DPS_OK;
+        // the previous launch that read the region must be done with it
+        if (ctx->stage_pending) {
+            HIPCHK(ctx, hipEventSynchronize(ctx->stage_event));
+            ctx->stage_pending = false;
+        }
+        const size_t job_words = jobs.size() * sizeof(dpk::EqJobM) / 8;
+        memcpy(ctx->h_pinned + stage_lo, jobs.data(), job_words * 8);
+        memcpy(ctx->h_pinned + stage_lo + job_words, pts.data(), pts.size() * 8);
+        ProfScope ps(ctx, DPS_K_EQ, 0.0);
+        dpk::eq_define_many_kernel<<<dim3((u32)(((1ull << max_bits) + dpk::BLOCK - 1) / dpk::BLOCK), (u32)jobs.size()), dpk::BLOCK, 0, ctx->stream>>>(
+            reinterpret_cast<const dpk::EqJobM *>(ctx->d_pinned + stage_lo), ctx->d_pinned + stage_lo + job_words);
+        HIPCHK(ctx, hipGetLastError());
+        HIPCHK(ctx, hipEventRecord(ctx->stage_event, ctx->stream));
+        ctx->stage_pending = true;
+        jobs.clear();
+        pts.clear();
+        max_bits = 0;
+        return DPS_OK;
+    };
+    for (u32 i = 0; i < count; i++) {
+        dps_mle *t = nullptr;
+        int32_t rc = new_table(ctx, DPS_EXT2, 2ull << m[i], &t);
+        if (rc != DPS_OK) return undo(rc);
+        out[i] = t;
+        t->len = 1ull << m[i];
+        t->eq = std::make_shared<EqInfo>();
+        t->eq->m = m[i];
+        for (u32 k = 0; k < m[i]; k++) t->eq->point.push_back(gl::e2(points[i][2 * k], points[i][2 * k + 1]));
+        if (m[i] > 16) {
+            // large tables are built by expansion, one at a time
+            rc = eq_build_dev(ctx, points[i], m[i], t->st->c0, t->st->c1);
+            if (rc != DPS_OK) return undo(rc);
+            continue;
+        }
+        const size_t need = ((jobs.size() + m[i] + 1) * sizeof(dpk::EqJobM)) / 8 + pts.size() + 2 * (size_t)m[i];
+        if (stage_lo + need > stage_hi || jobs.size() + m[i] + 1 > 65535) {
+            rc = flush();
+            if (rc != DPS_OK) return undo(rc);
+        }
+        // every level eq(rho_{l..m-1}, .), l = 0..m, straight from the definition
+        const u32 point_off = (u32)pts.size();
+        pts.insert(pts.end(), points[i], points[i] + 2 * (size_t)m[i]);
+        for (u32 l = 0; l <= m[i]; l++) {
+            const u64 off = eq_level_off(m[i], l);
+            jobs.push_back(dpk::EqJobM{t->st->c0 + off, t->st->c1 + off, l, m[i] - l, point_off, 0});
+            max_bits = std::max(max_bits, m[i] - l);
+        }
+    }
+    // the point offsets are relative to the start of the points, which follow the jobs of the same launch
+    int32_t rc = flush();
+    if (rc != DPS_OK) return undo(rc);
     return DPS_OK;
 }
 
@@ -1328,11 +1410,11 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
 constexpr u64 POLY_SPLIT_MAX_PAIRS = 1ull << 16;
 
 // lanes per pair (log2) and grid of a split round: about 2^17 threads while that many items exist; a round
-// that fits one workgroup takes the lanes the workgroup has
-void poly_split_plan(u64 n_pairs, u32 cap, u32 *split_log, u32 *blocks)
+// that fits one workgroup takes the lanes the workgroup has when it can stay resident (a single group)
+void poly_split_plan(u64 n_pairs, u32 cap, bool may_reside, u32 *split_log, u32 *blocks)
 {
     u32 lp = log2u(n_pairs);
-    u32 sl = n_pairs <= dpk::BLOCK ? log2u(dpk::BLOCK) - lp : (lp < 17 ? 17 - lp : 0);
+    u32 sl = (may_reside && n_pairs <= dpk::BLOCK) ? log2u(dpk::BLOCK) - lp : (lp < 17 ? 17 - lp : 0);
     sl = std::min(sl, cap);
     *split_log = sl;
     *blocks = (u32)std::max<u64>(1, (n_pairs << sl) / dpk::BLOCK);
@@ -1419,17 +1501,18 @@ u32 horner_build(std::vector<HornerTerm> ts, u32 depth, std::vector<dpk::PolyOp>
     // terms that end at this node were added to the node's constant by the caller
     ts.erase(std::remove_if(ts.begin(), ts.end(), [](const HornerTerm &t) { return t.slots.empty(); }), ts.end());
     while (!ts.empty()) {
-        u32 count[256] = {0};
+        // slots are positions within a group: fewer than POLY_MAXT
+        u32 count[dpk::POLY_MAXT] = {0};
         for (const HornerTerm &t : ts) {
-            bool seen[256] = {false};
+            u32 seen = 0;
             for (uint8_t sl : t.slots)
-                if (!seen[sl]) {
-                    seen[sl] = true;
+                if (!((seen >> sl) & 1)) {
+                    seen |= 1u << sl;
                     count[sl]++;
                 }
         }
         u32 best = 0;
-        for (u32 sl = 1; sl < 256; sl++)
+        for (u32 sl = 1; sl < (u32)dpk::POLY_MAXT; sl++)
             if (count[sl] > count[best]) best = sl;
         std::vector<HornerTerm> sub, rest;
         for (HornerTerm &t : ts) {
@@ -1912,7 +1995,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             const u64 np = 1ull << (n_vars - j);
             if (np > POLY_SPLIT_MAX_PAIRS) continue;
             u32 sl, bl;
-            poly_split_plan(np, sc->poly_split_cap, &sl, &bl);
+            poly_split_plan(np, sc->poly_split_cap, sc->poly_tabs.size() == 1, &sl, &bl);
             sc->max_blocks = std::max(sc->max_blocks, bl);
         }
     }
@@ -2276,7 +2359,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = pa.pad = 0;
             pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
             u32 sblocks = blocks;
-            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, &pa.split_log, &sblocks);
+            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, n_groups == 1, &pa.split_log, &sblocks);
             pa.split_cap = sc->poly_split_cap;
             // a single workgroup from here on: it stays for the remaining rounds
             const bool reside = split && n_groups == 1 && sblocks == 1 && a.skip1 && j < sc->n_vars &&

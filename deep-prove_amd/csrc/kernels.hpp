@@ -167,6 +167,29 @@ __global__ void __launch_bounds__(BLOCK) eq_define_kernel(EqJobs js)
     js.o1[j.out_off + i] = acc.c1;
 }
 
+// The same for jobs of several tables at once (many small eq tables, each with its own point): descriptors and
+// points lie in host-visible memory, written just before the launch.
+struct EqJobM {
+    u64 *o0, *o1;     // where the job's entries go
+    u32 first, n_bits;
+    u32 point_off;    // words from `points` to the table's point
+    u32 pad;
+};
+__global__ void __launch_bounds__(BLOCK) eq_define_many_kernel(const EqJobM *__restrict__ jobs, const u64 *__restrict__ points)
+{
+    const EqJobM j = jobs[blockIdx.y];
+    const u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= ((u64)1 << j.n_bits)) return;
+    const u64 *pt = points + j.point_off;
+    E2 acc = gl::e2_one();
+    for (u32 b = 0; b < j.n_bits; b++) {
+        E2 r = gl::e2(pt[2 * (j.first + b)], pt[2 * (j.first + b) + 1]);
+        acc = gl::mul(acc, ((i >> b) & 1) ? r : gl::sub(gl::e2_one(), r));
+    }
+    j.o0[i] = acc.c0;
+    j.o1[i] = acc.c1;
+}
+
 // Expansion: out[h * 2^b + l] = hi[h] * lo[l], lo has 2^b <= 256 entries.  Each
 // thread keeps one lo entry in registers and walks hi entries; stores of one
 // wavefront cover 512 contiguous bytes per limb array.

@@ -277,9 +277,9 @@ inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> 
         // prove.rs:260-302: aggregate the R claims on the LHS with a second sumcheck
         DensePolynomial input_mle = lhs.padded_mle(ctx);
         const uint32_t nv = input_mle.num_vars();
-        std::vector<DensePolynomial> eq_polys;
-        for (size_t r = 0; r < R; r++)
-            eq_polys.push_back(DensePolynomial::eq(ctx, reconstruct_full_point(lhs_fixes[r], info.einsum_sumcheck_point, lhs.padded_shape)));
+        std::vector<std::vector<F>> eq_points;
+        for (size_t r = 0; r < R; r++) eq_points.push_back(reconstruct_full_point(lhs_fixes[r], info.einsum_sumcheck_point, lhs.padded_shape));
+        std::vector<DensePolynomial> eq_polys = DensePolynomial::eq_many(ctx, eq_points);
         F input_batching = transcript.append_and_sample("input_batching_challenge");
         std::vector<const DensePolynomial *> am{&input_mle};
         for (auto &p : eq_polys) am.push_back(&p);

@@ -110,35 +110,46 @@ private:
     }
     static std::vector<Monomial> expand(const Node &n, const std::vector<F> &ch)
     {
+        std::vector<Monomial> out;
+        expand_into(n, F::one(), ch, out);
+        return out;
+    }
+    // appends scale * (the node's monomials) to `out`: long sums (one `+` per term, as the provers build them)
+    // cost one pass, not one copy of everything so far per `+`
+    static void expand_into(const Node &n, const F &scale, const std::vector<F> &ch, std::vector<Monomial> &out)
+    {
+        if (scale.is_zero()) return;
         switch (n.kind) {
-        case Kind::WitIn: return {Monomial{F::one(), {n.id}}};
-        case Kind::Constant: return {Monomial{n.scalar, {}}};
-        case Kind::Challenge: return {Monomial{challenge_value(n, ch), {}}};
-        case Kind::Neg: {
-            auto v = expand(*n.a, ch);
-            for (auto &m : v) m.coeff = -m.coeff;
-            return v;
+        case Kind::WitIn: out.push_back(Monomial{scale, {n.id}}); return;
+        case Kind::Constant:
+            if (!n.scalar.is_zero()) out.push_back(Monomial{scale * n.scalar, {}});
+            return;
+        case Kind::Challenge: {
+            const F c = challenge_value(n, ch);
+            if (!c.is_zero()) out.push_back(Monomial{scale * c, {}});
+            return;
         }
-        case Kind::Sum: {
-            auto v = expand(*n.a, ch), w = expand(*n.b, ch);
-            v.insert(v.end(), w.begin(), w.end());
-            return v;
-        }
+        case Kind::Neg: expand_into(*n.a, -scale, ch, out); return;
+        case Kind::Sum:
+            expand_into(*n.a, scale, ch, out);
+            expand_into(*n.b, scale, ch, out);
+            return;
         case Kind::Product: {
-            auto v = expand(*n.a, ch), w = expand(*n.b, ch);
-            std::vector<Monomial> out;
-            out.reserve(v.size() * w.size());
+            std::vector<Monomial> v, w;
+            expand_into(*n.a, F::one(), ch, v);
+            expand_into(*n.b, scale, ch, w);
+            out.reserve(out.size() + v.size() * w.size());
             for (auto &x : v)
                 for (auto &y : w) {
                     Monomial m{x.coeff * y.coeff, x.wits};
+                    if (m.coeff.is_zero()) continue;
                     m.wits.insert(m.wits.end(), y.wits.begin(), y.wits.end());
                     std::sort(m.wits.begin(), m.wits.end());
-                    if (!m.coeff.is_zero()) out.push_back(std::move(m));
+                    out.push_back(std::move(m));
                 }
-            return out;
+            return;
         }
         }
-        return {};
     }
     static F eval(const Node &n, const std::vector<F> &w, const std::vector<F> &ch)
     {

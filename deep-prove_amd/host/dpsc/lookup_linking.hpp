@@ -245,8 +245,7 @@ public:
         if (logup_point.size() != eb.first.size()) throw Error(DPS_ERR_INVALID, "linking sumcheck: LogUp point length does not match the chunk");
         const std::vector<F> ch = batching_challenges(eb.second, transcript);
         const Context &ctx = mles[0]->context();
-        std::vector<DensePolynomial> eqs;
-        for (auto &p : eq_points(eb.first, logup_point)) eqs.push_back(DensePolynomial::eq(ctx, p));
+        std::vector<DensePolynomial> eqs = DensePolynomial::eq_many(ctx, eq_points(eb.first, logup_point));
         std::vector<const DensePolynomial *> all(mles);
         for (auto &e : eqs) all.push_back(&e);
         if (weight_mle) all.push_back(weight_mle);

@@ -101,6 +101,25 @@ public:
         ctx.check(dps_eq_build(ctx.raw(), limbs.data(), (uint32_t)point.size(), &h), "dps_eq_build");
         return DensePolynomial(ctx, h);
     }
+    // several eq tables built together (one launch for all the small ones)
+    static std::vector<DensePolynomial> eq_many(const Context &ctx, const std::vector<std::vector<F>> &points)
+    {
+        std::vector<std::vector<uint64_t>> limbs;
+        std::vector<const uint64_t *> ptrs;
+        std::vector<uint32_t> m;
+        limbs.reserve(points.size());
+        for (auto &p : points) {
+            limbs.push_back(to_limbs(p));
+            m.push_back((uint32_t)p.size());
+        }
+        for (auto &l : limbs) ptrs.push_back(l.data());
+        std::vector<dps_mle *> hs(points.size(), nullptr);
+        ctx.check(dps_eq_build_many(ctx.raw(), ptrs.data(), m.data(), (uint32_t)points.size(), hs.data()), "dps_eq_build_many");
+        std::vector<DensePolynomial> out;
+        out.reserve(hs.size());
+        for (auto *h : hs) out.emplace_back(ctx, h);
+        return out;
+    }
     // new_from_smart_slice(SmartSlice::Borrowed(&evals[offset..offset + 2^n_vars]))
     DensePolynomial view(uint64_t offset, uint32_t n_vars) const
     {

@@ -93,7 +93,7 @@ inline ClaimsBatchingProof claims_batching_sumcheck(const Context &ctx, const st
                                                     const std::vector<std::vector<Claim>> &claims, Transcript &transcript)
 {
     if (polys.size() != claims.size() || polys.empty()) throw Error(DPS_ERR_INVALID, "claims_batching_sumcheck: one claim list per polynomial");
-    std::vector<DensePolynomial> eq_polys;
+    std::vector<std::vector<F>> eq_points;
     std::vector<const DensePolynomial *> committed;
     std::vector<ChunkedCommittedPolyInfo> infos;
     size_t max_num_vars = 0;
@@ -103,13 +103,15 @@ inline ClaimsBatchingProof claims_batching_sumcheck(const Context &ctx, const st
         for (const Claim &cl : claims[p]) {
             if (cl.point.size() != poly.num_vars()) throw Error(DPS_ERR_INVALID, "claim point does not match the polynomial");
             transcript.append_scalars(&cl.eval, 1);
-            eq_polys.push_back(DensePolynomial::eq(ctx, eq_point_per_chunk(poly.num_chunks(), cl.point)));
+            eq_points.push_back(eq_point_per_chunk(poly.num_chunks(), cl.point));
             info.batching_coefficients.push_back(batching_coefficients_for_chunks(poly.num_chunks(), cl.point));
         }
         for (auto *c : poly.chunks) committed.push_back(c);
         max_num_vars = std::max(max_num_vars, poly.num_vars_for_chunk());
         infos.push_back(std::move(info));
     }
+    // one eq table per claim (prover.rs:176-181), built together
+    std::vector<DensePolynomial> eq_polys = DensePolynomial::eq_many(ctx, eq_points);
     Expression expr = build_sumcheck_expression(infos);
 
     // zero-padded views of every table, chunk tables first, then the eq tables

@@ -38,9 +38,9 @@ public:
     std::pair<Proof, Claim> prove(Transcript &t) const
     {
         const std::vector<F> challenges = t.read_challenges(claims_.size());
-        std::vector<DensePolynomial> beta_evals;
-        beta_evals.reserve(claims_.size());
-        for (auto &c : claims_) beta_evals.push_back(DensePolynomial::eq(poly_->context(), c.point));
+        std::vector<std::vector<F>> points;
+        for (auto &c : claims_) points.push_back(c.point);
+        std::vector<DensePolynomial> beta_evals = DensePolynomial::eq_many(poly_->context(), points);
         const size_t num_vars = poly_->num_vars();
         VirtualPolynomialsBuilder builder(optimal_sumcheck_threads(num_vars), num_vars);
         Expression poly_expr = builder.lift(*poly_);

@@ -108,6 +108,9 @@ int32_t dps_mle_free(dps_mle *mle);
 /* ---- poly::eq::evals (zkml/src/layers/hadamard.rs:103, zkml/src/layers/einsum/axis.rs:1032,
  *      zkml/src/lookup/logup_gkr/prover.rs:247-249): out[i] = prod_j (bit_j(i) ? r_j : 1 - r_j) ---- */
 int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point /* 2*m */, uint32_t m, dps_mle **out);
+/* `count` eq tables, table i at points[i] of m[i] coordinates (zkml/src/poly_commit/prover.rs:176-181 and
+ * zkml/src/iop/same_poly.rs:88-91 build one per claim): every table of at most 2^16 entries comes out of one launch. */
+int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points, const uint32_t *m, uint32_t count, dps_mle **out);
 
 /* ---- DensePolynomial::{evaluate, fix_low_variables, fix_high_variables}
  *      (zkml/src/layers/einsum/prove.rs:208, zkml/src/tensor/mod.rs:1892, zkml/src/iop/prover.rs:448,509) ---- */

@@ -338,3 +338,30 @@ def test_zero_pad_errors(dp, ctx):
     one = np.array([1, 0], dtype=np.uint64)
     with pytest.raises(dp.DpsError):
         dp.Session(ctx, 6, [z], [(one, [0])])
+
+
+def test_eq_tables_built_together(dp, ctx, orc):
+    """dps_eq_build_many: every table equals the one built alone, including the suffix levels a sumcheck reads
+    when the table is a factor of every term; sizes on both sides of the one-launch limit, the empty point"""
+    ms = [0, 1, 5, 10, 16, 17, 3, 10]
+    points = [rand_e2(m, 900 + i) for i, m in enumerate(ms)]
+    tabs = ctx.eq_build_many(points)
+    assert len(tabs) == len(ms)
+    for t, p, m in zip(tabs, points, ms):
+        assert t.info() == (dp.KIND_EXT2, 1 << m)
+        assert (t.download() == orc.eq_evals(p)).all()
+    assert ctx.eq_build_many([]) == []
+    # as the common eq factor of a product (closed form over the suffix tables)
+    n = 10
+    f, g = rand_base(1 << n, 950), rand_base(1 << n, 951)
+    one = np.array([1, 0], dtype=np.uint64)
+    for k in (3, 7):
+        _check_prove(dp, ctx, orc, n, [ctx.mle_from_base(f), ctx.mle_from_base(g), tabs[k]],
+                     [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(points[k])], [(one, [2, 0, 1])])
+    # many tables: more than one launch's worth of staging is split, not refused
+    many = [rand_e2(12, 2000 + i) for i in range(80)]
+    got = ctx.eq_build_many(many)
+    for t, p in zip(got[::13], many[::13]):
+        assert (t.download() == orc.eq_evals(p)).all()
+    with pytest.raises(dp.DpsError):
+        ctx.eq_build_many([np.array([[dp.P, 0]], dtype=np.uint64)])
