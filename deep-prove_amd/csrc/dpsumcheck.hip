@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -1307,6 +1308,7 @@ struct dps_sc {
     u32 poly_max_tabs;                        // sizes the kernel's LDS
     u32 poly_split_cap;                       // log2 of the most lanes a pair's work is worth spreading over
     bool descs_uploaded;                      // the descriptor block is on the device (uploaded when first needed)
+    bool poly_raw;                            // the resident launch has one workgroup per group; the host adds their sums
     bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
@@ -1406,6 +1408,10 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
     return DPS_OK;
 }
 
+// Several groups resident side by side publish into 64-word slots of the pinned buffer from here on
+constexpr u32 POLY_RAW_MAX_GROUPS = 32;
+size_t poly_raw_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64; }
+
 // Rounds of at most this many pairs run on poly_split_kernel
 constexpr u64 POLY_SPLIT_MAX_PAIRS = 1ull << 16;
 
@@ -1420,6 +1426,24 @@ void poly_split_plan(u64 n_pairs, u32 cap, bool may_reside, u32 *split_log, u32 
     *blocks = (u32)std::max<u64>(1, (n_pairs << sl) / dpk::BLOCK);
 }
 
+// Resident launches keep the folded tables in LDS, which takes more dynamic LDS than a launch gets by default:
+// asked for once per kernel and device.
+template <int NF, bool EQ, bool SKIP1>
+bool poly_split_state_granted(dps_ctx *ctx)
+{
+    static std::atomic<int> granted[64];  // 0 not asked, 1 granted, 2 refused
+    std::atomic<int> &gr = granted[ctx->device & 63];
+    int v = gr.load();
+    if (v == 0) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dpk::poly_split_kernel<NF, EQ, SKIP1>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)(dpk::POLY_MAXT * 10 * dpk::BLOCK * 8));
+        if (e != hipSuccess) (void)hipGetLastError();
+        v = e == hipSuccess ? 1 : 2;
+        gr.store(v);
+    }
+    return v == 1;
+}
+
 template <int NF, bool EQ, bool SKIP1>
 int32_t launch_poly_split_one(dps_ctx *ctx, dpk::PolyArgs &a, dim3 grid, u32 max_tabs, bool want_state, u64 *partial, const dpk::FastFin &ff)
 {
@@ -1430,21 +1454,12 @@ int32_t launch_poly_split_one(dps_ctx *ctx, dpk::PolyArgs &a, dim3 grid, u32 max
     size_t lds = lds_vals;
     a.lds_state = 0;
     a.state_off = (u32)(lds_vals / 8);
-    if (want_state) {
-        // more dynamic LDS than a launch gets by default: asked for once per kernel and device
-        static int granted[64] = {0};  // 0 not asked, 1 granted, 2 refused
-        int &gr = granted[ctx->device & 63];
-        if (gr == 0) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dpk::poly_split_kernel<NF, EQ, SKIP1>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(dpk::POLY_MAXT * 10 * dpk::BLOCK * 8));
-            gr = e == hipSuccess ? 1 : 2;
-            if (e != hipSuccess) (void)hipGetLastError();
-        }
-        if (gr == 1 || lds_vals + lds_state + 8192 <= 65536) {
-            a.lds_state = 1;
-            lds = lds_vals + lds_state;
-        }
+    if (want_state && poly_split_state_granted<NF, EQ, SKIP1>(ctx)) {
+        a.lds_state = 1;
+        lds = lds_vals + lds_state;
     }
+    // several resident groups must not read each other's stores: without the tables in LDS they cannot stay
+    if (a.raw_out && !a.lds_state) return fail(ctx, DPS_ERR_HIP, "resident groups need the larger LDS allocation");
     dpk::poly_split_kernel<NF, EQ, SKIP1><<<grid, dpk::BLOCK, lds, ctx->stream>>>(a, partial, ff);
     return DPS_OK;
 }
@@ -1457,6 +1472,29 @@ int32_t launch_poly_split(dps_ctx *ctx, bool eq, bool skip1, dpk::PolyArgs &a, d
     if (eq) return launch_poly_split_one<NF, true, false>(ctx, a, grid, max_tabs, want_state, partial, ff);
     if (skip1) return launch_poly_split_one<NF, false, true>(ctx, a, grid, max_tabs, want_state, partial, ff);
     return launch_poly_split_one<NF, false, false>(ctx, a, grid, max_tabs, want_state, partial, ff);
+}
+
+template <int NF>
+bool poly_split_state_ok_nf(dps_ctx *ctx, bool eq, bool skip1)
+{
+    if (eq && skip1) return poly_split_state_granted<NF, true, true>(ctx);
+    if (eq) return poly_split_state_granted<NF, true, false>(ctx);
+    if (skip1) return poly_split_state_granted<NF, false, true>(ctx);
+    return poly_split_state_granted<NF, false, false>(ctx);
+}
+
+// can a resident launch of this kernel keep its tables in LDS?
+bool poly_split_state_ok(dps_ctx *ctx, u32 nf, bool eq, bool skip1)
+{
+    switch (nf) {
+    case 1: return poly_split_state_ok_nf<1>(ctx, eq, skip1);
+    case 2: return poly_split_state_ok_nf<2>(ctx, eq, skip1);
+    case 3: return poly_split_state_ok_nf<3>(ctx, eq, skip1);
+    case 4: return poly_split_state_ok_nf<4>(ctx, eq, skip1);
+    case 5: return poly_split_state_ok_nf<5>(ctx, eq, skip1);
+    case 6: return poly_split_state_ok_nf<6>(ctx, eq, skip1);
+    default: return false;
+    }
 }
 
 int32_t launch_poly_split_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, dpk::PolyArgs &a, dim3 grid, u32 max_tabs, bool want_state,
@@ -1983,9 +2021,11 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->poly_split_cap = 0;
     sc->poly_finish_in_kernel = false;
     if (sc->poly) {
-        sc->poly_finish_in_kernel = sc->poly_tabs.size() == 1;
+        // every table is in a group (or is the closed-form eq): the resident launch can publish all final evaluations
+        sc->poly_finish_in_kernel = true;
         for (u32 k = 0; k < n_mles; k++)
-            if (sc->poly_owner[k] != 0 && (int)k != sc->fast_eq) sc->poly_finish_in_kernel = false;
+            if (sc->poly_owner[k] < 0 && (int)k != sc->fast_eq) sc->poly_finish_in_kernel = false;
+        sc->poly_raw = false;
         // items of a pair: (evaluation point, term) products; tables to fold
         u32 most_terms = 0;
         for (size_t g = 0; g < sc->poly_tabs.size(); g++) most_terms = std::max(most_terms, sc->poly_term_end[g] - sc->poly_term_begin[g]);
@@ -1995,7 +2035,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             const u64 np = 1ull << (n_vars - j);
             if (np > POLY_SPLIT_MAX_PAIRS) continue;
             u32 sl, bl;
-            poly_split_plan(np, sc->poly_split_cap, sc->poly_tabs.size() == 1, &sl, &bl);
+            poly_split_plan(np, sc->poly_split_cap, sc->poly_tabs.size() <= POLY_RAW_MAX_GROUPS, &sl, &bl);
             sc->max_blocks = std::max(sc->max_blocks, bl);
         }
     }
@@ -2105,9 +2145,13 @@ namespace {
 // word; the words are accepted once the check word agrees with them, since the
 // kernel's stores may land in any order.  If the result does not arrive the
 // stream is queried to surface the error.
-int32_t wait_result(dps_ctx *ctx, u64 seq, u32 slot0, u32 n, u64 *out)
+int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out);
+int32_t wait_result(dps_ctx *ctx, u64 seq, u32 slot0, u32 n, u64 *out) { return wait_result_at(ctx, ctx->res_off, seq, slot0, n, out); }
+
+// the same hand-off in another 64-word area of the pinned buffer
+int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out)
 {
-    volatile u64 *base = ctx->h_pinned + ctx->res_off;
+    volatile u64 *base = ctx->h_pinned + base_off;
     volatile u64 *flag = base + dpk::HOST_SEQ_SLOT;
     auto take = [&]() {
         if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) return false;
@@ -2258,6 +2302,31 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             mb[dpk::MAIL_SKIP1] = a.skip1;
             send_mail(ctx, fa.seq);
         };
+        // several resident groups: their sums q(t) added, then the message as fast_finalize forms it
+        auto take_raw_round = [&]() -> int32_t {
+            const u32 n_groups = (u32)sc->poly_tabs.size(), np = nf + 1;
+            E2 q[dpk::MAX_PTS];
+            for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+            for (u32 g = 0; g < n_groups; g++) {
+                u64 w[2 * dpk::MAX_PTS];
+                CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
+                for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
+            }
+            E2 msg[dpk::MAX_PTS + 1];
+            for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(ff.scale[2 * t], ff.scale[2 * t + 1]), q[t]), cst);
+            if (a.skip1) msg[1] = gl::sub(sc->claim, msg[0]);
+            if (has_eq) {
+                E2 e = gl::add(gl::e2(ff.k0, ff.k1), cst);
+                for (u32 i = 0; i < np; i++)
+                    if (!(a.skip1 && i == 1)) e = gl::add(e, gl::mul(gl::e2(ff.cext[2 * i], ff.cext[2 * i + 1]), q[i]));
+                msg[np] = e;
+            }
+            for (u32 t = 0; t <= sc->degree; t++) {
+                evals_out[2 * t] = msg[t].c0;
+                evals_out[2 * t + 1] = msg[t].c1;
+            }
+            return DPS_OK;
+        };
         if (sc->tail_j0 && j >= sc->tail_j0) {
             post_mail();
             if (j == sc->tail_j0) {
@@ -2305,7 +2374,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 if (a.skip1) {
                     // the resident launch of an earlier round runs this one
                     post_mail();
-                    int32_t rc = wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
+                    int32_t rc = sc->poly_raw ? take_raw_round() : wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
                     if (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel)) {
                         // without a finishing step of its own it exits after the last round
                         sc->tail_running = false;
@@ -2356,17 +2425,27 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             pa.eq1 = sc->eq_c1;
             pa.mail = ctx->d_pinned + (ctx->res_off - 64);
             pa.seq = fa.seq;
-            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = pa.pad = 0;
+            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = 0;
             pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
+            pa.group_stride = 1;
+            pa.raw_out = nullptr;
             u32 sblocks = blocks;
-            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, n_groups == 1, &pa.split_log, &sblocks);
+            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, n_groups <= POLY_RAW_MAX_GROUPS, &pa.split_log, &sblocks);
             pa.split_cap = sc->poly_split_cap;
             // a single workgroup from here on: it stays for the remaining rounds
-            const bool reside = split && n_groups == 1 && sblocks == 1 && a.skip1 && j < sc->n_vars &&
-                                sc->n_vars - j + 1 <= (u32)dpk::POLY_RES_ROUNDS;
+            // (several groups stay only with their tables in LDS: they must not read each other's stores)
+            const bool reside = split && n_groups <= POLY_RAW_MAX_GROUPS && sblocks == 1 && a.skip1 && j < sc->n_vars &&
+                                sc->n_vars - j + 1 <= (u32)dpk::POLY_RES_ROUNDS &&
+                                (n_groups == 1 || poly_split_state_ok(ctx, nf, has_eq, true));
             if (reside) {
                 pa.last_round = sc->n_vars;
-                if (inline_descs) {
+                if (n_groups > 1) {
+                    // one resident workgroup per group, each publishing its own sums
+                    CHK(ensure_descs(sc));
+                    pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
+                    pa.group_stride = n_groups;
+                    pa.raw_out = ctx->d_pinned + poly_raw_off(ctx);
+                } else if (inline_descs) {
                     // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
                     // before its first round, and this call returns only after that round's message has arrived
                     const size_t words = (size_t)(sc->n_vars - j + 1) * sizeof(dpk::PolyGroup) / 8;
@@ -2390,8 +2469,12 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 sc->tail_running = true;
                 sc->tail_seq0 = fa.seq;
                 ctx->tail_owner = sc;
+                sc->poly_raw = n_groups > 1;
             }
-            CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
+            if (reside && n_groups > 1)
+                CHK(take_raw_round());
+            else
+                CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
             took_round();
             return DPS_OK;
         }
@@ -2442,18 +2525,26 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         mb[dpk::MAIL_R + 1] = challenge[1];
         send_mail(ctx, seq);
         u64 fin[2 * dpk::POLY_MAXT];
-        // the fused multi-term kernel publishes its group's tables in slot order, the single-product one its factors
-        const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[0].size() : sc->fast_nf;
-        int32_t rc = wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin);
+        // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
+        // groups are resident), the single-product one its factors
+        int32_t rc = DPS_OK;
+        const u32 n_areas = sc->poly ? (u32)sc->poly_tabs.size() : 1;
+        for (u32 g = 0; g < n_areas && rc == DPS_OK; g++) {
+            const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[g].size() : sc->fast_nf;
+            rc = sc->poly_raw ? wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin)
+                              : wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin);
+            for (u32 f = 0; f < n_fin && rc == DPS_OK; f++) {
+                const u32 k = sc->poly ? sc->poly_tabs[g][f] : sc->fast_order[f];
+                // a table shared by several groups is folded by each; the owner's copy counts
+                if (sc->poly && sc->poly_owner[k] != (int)g) continue;
+                final_evals_out[2 * k] = fin[2 * f];
+                final_evals_out[2 * k + 1] = fin[2 * f + 1];
+            }
+        }
         // the kernel exits right after publishing and reads nothing more; whatever is launched next follows it on the stream
         sc->tail_running = false;
         ctx->tail_owner = nullptr;
         if (rc != DPS_OK) return rc;
-        for (u32 f = 0; f < n_fin; f++) {
-            const u32 k = sc->poly ? sc->poly_tabs[0][f] : sc->fast_order[f];
-            final_evals_out[2 * k] = fin[2 * f];
-            final_evals_out[2 * k + 1] = fin[2 * f + 1];
-        }
         if (sc->fast_eq >= 0) {
             E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], gl::e2(challenge[0], challenge[1])));
             final_evals_out[2 * sc->fast_eq] = v.c0;

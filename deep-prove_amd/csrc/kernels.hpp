@@ -1104,7 +1104,11 @@ struct PolyArgs {
     u32 lds_state;   // resident rounds: the folded tables stay in LDS (state_off words into the dynamic LDS)
     u32 state_off;
     u32 finish;      // resident rounds: stay after the last round for the last challenge and publish the final evaluations
-    u32 pad;
+    u32 group_stride;  // resident rounds: descriptors of consecutive rounds of one group lie this many apart
+    // Several groups resident side by side (one workgroup each, gridDim.y of them): a workgroup cannot finish the
+    // message, which is the sum over the groups, so each publishes its own sums q(t) (and later its tables' final
+    // evaluations) to its 64-word slot raw_out + 64 * blockIdx.y, laid out like the main result area, and the host adds.
+    u64 *raw_out;    // nullptr: a single workgroup finishes the message itself
 };
 
 template <int NF, bool EQ, bool SKIP1>
@@ -1337,9 +1341,13 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         // resident launch pinned host memory) every use would be a dependent load of its own.  A resident launch has
         // a single group, whose descriptors for rounds j, j + 1, ... follow each other.
         const u32 n_rounds = a.last_round ? a.last_round - a.j + 1 : 1;
+        constexpr u32 GW = sizeof(PolyGroup) / 8;
         const u64 *src = a.groups ? reinterpret_cast<const u64 *>(a.groups + blockIdx.y) : reinterpret_cast<const u64 *>(&a.g0);
         u64 *dst = reinterpret_cast<u64 *>(gall);
-        for (u32 w = tid; w < n_rounds * (u32)(sizeof(PolyGroup) / 8); w += BLOCK) dst[w] = src[w];
+        for (u32 w = tid; w < n_rounds * GW; w += BLOCK) {
+            const u32 rr = w / GW;
+            dst[w] = src[(size_t)rr * a.group_stride * GW + (w - rr * GW)];
+        }
         __syncthreads();
         const u32 nt = gall[0].term_end - gall[0].term_begin;
         const u32 staged = nt < (u32)POLY_LDS_TERMS ? nt : (u32)POLY_LDS_TERMS;
@@ -1358,9 +1366,11 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     u64 *const state_dst = dst_is_a ? state_a : state_b;
     const u64 *const state_src = dst_is_a ? state_b : state_a;
     const u32 state_dst_len = dst_is_a ? 2 * BLOCK : BLOCK, state_src_len = dst_is_a ? BLOCK : 2 * BLOCK;
-    u32 wrote = 0;  // tables this round folds and stores
+    // tables this round folds: with lds_state every one of them is kept in LDS, also a table another group owns
+    // (only the owner writes it to device memory), so that resident groups never read each other's stores
+    u32 wrote = 0;
     for (u32 k = 0; k < n_tabs; k++)
-        if (g.tab[k].mode == POLY_PAIR_FOLD && g.tab[k].d0) wrote |= 1u << k;
+        if (g.tab[k].mode == POLY_PAIR_FOLD) wrote |= 1u << k;
 
     gl::E2Acc lz[NP];
 #pragma unroll
@@ -1408,13 +1418,13 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
                     if (tb.d0) {
                         st2_stream(tb.d0 + 2 * i, lo.c0, hi.c0);
                         st2_stream(tb.d1 + 2 * i, lo.c1, hi.c1);
-                        if (a.lds_state) {
-                            u64 *c0 = state_dst + (size_t)(k * 2 + 0) * state_dst_len, *c1 = state_dst + (size_t)(k * 2 + 1) * state_dst_len;
-                            c0[2 * i] = lo.c0;
-                            c0[2 * i + 1] = hi.c0;
-                            c1[2 * i] = lo.c1;
-                            c1[2 * i + 1] = hi.c1;
-                        }
+                    }
+                    if (a.lds_state) {
+                        u64 *c0 = state_dst + (size_t)(k * 2 + 0) * state_dst_len, *c1 = state_dst + (size_t)(k * 2 + 1) * state_dst_len;
+                        c0[2 * i] = lo.c0;
+                        c0[2 * i + 1] = hi.c0;
+                        c1[2 * i] = lo.c1;
+                        c1[2 * i + 1] = hi.c1;
                     }
                 } else if (tb.mode == POLY_PAIR) {
                     const U64x2 p0 = ld2(tb.s0 + 2 * i);
@@ -1480,8 +1490,21 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
     block_reduce<NP>(acc, lds);
-    if (gridDim.x * gridDim.y == 1) {
-        fast_finalize<NF>(cf, acc, res);
+    const bool raw = a.raw_out != nullptr;  // then gridDim.x == 1
+    if (gridDim.x * gridDim.y == 1 || raw) {
+        u64 *const my_out = raw ? a.raw_out + 64 * blockIdx.y : cf.out_host;
+        if (raw) {
+            if (tid == 0) {
+#pragma unroll
+                for (int t = 0; t < NP; t++) {
+                    res[2 * t] = acc[t].c0;
+                    res[2 * t + 1] = acc[t].c1;
+                }
+                publish_words(my_out, 0, res, 2 * NP, a.seq + (j - a.j));
+            }
+        } else {
+            fast_finalize<NF>(cf, acc, res);
+        }
         if (a.last_round == 0) return;
         if (j >= a.last_round) {
             if (!a.finish) return;
@@ -1498,7 +1521,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
                 res[2 * tid + 1] = v.c1;
             }
             __syncthreads();
-            if (tid == 0) publish_words(cf.out_host, HOST_FINALS_SLOT, res, 2 * n_tabs, fin_seq);
+            if (tid == 0) publish_words(my_out, HOST_FINALS_SLOT, res, 2 * n_tabs, fin_seq);
             return;
         }
         // stay for the next round: its challenge and the scalars of its message arrive by mail
