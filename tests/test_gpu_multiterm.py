@@ -88,6 +88,27 @@ def test_random_expressions_match_checker(dp, ctx, orc, case):
     _check(dp, ctx, orc, n, gpu, host, terms)
 
 
+@pytest.mark.parametrize("n_terms,with_eq", [(40, False), (12, True), (33, True)])
+def test_many_groups(dp, ctx, orc, n_terms, with_eq):
+    """every term over tables of its own: as many groups as terms -- up to 32 of them stay resident side by side
+    (one workgroup each, the host adds their sums), more run a launch per round"""
+    n, per_term = 8, 5
+    tabs = [rand_e2(1 << n, 6000 + k) for k in range(n_terms * per_term)]
+    gpu = [ctx.mle_from_ext2(t) for t in tabs]
+    host = list(tabs)
+    rng = py_rng(n_terms)
+    terms = []
+    for t in range(n_terms):
+        coeff = np.array([rng.randrange(1, 1 << 62), rng.randrange(0, 1 << 62)], dtype=np.uint64)
+        terms.append((coeff, [t * per_term + f for f in range(per_term)]))
+    if with_eq:
+        pt = rand_e2(n, 6500 + n_terms)
+        gpu.append(ctx.eq_build(pt))
+        host.append(orc.eq_evals(pt))
+        terms = [(c, fs + [len(gpu) - 1]) for c, fs in terms]
+    _check(dp, ctx, orc, n, gpu, host, terms)
+
+
 @pytest.mark.parametrize("n,zero_at", [(10, 0), (10, 4), (12, 9), (12, 11), (6, 2)])
 def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
     """eq(rho, .) with rho_v = 0 makes the message of round v + 1 vanish at 1: that round must evaluate t = 1
@@ -95,6 +116,9 @@ def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
     pt = rand_e2(n, 777 + n + zero_at)
     pt[zero_at] = 0
     gpu, host, terms = _instance(ctx, orc, 400 + n + zero_at, n, [n] * 4, [], 6, 3, True, eq_point=pt)
+    _check(dp, ctx, orc, n, gpu, host, terms)
+    # the same with more tables than one group holds
+    gpu, host, terms = _instance(ctx, orc, 500 + n + zero_at, n, [n] * 11, [], 9, 2, True, eq_point=pt)
     _check(dp, ctx, orc, n, gpu, host, terms)
     # the single-product path with the same point
     f, g = rand_base(1 << n, 5), rand_base(1 << n, 6)
