@@ -1823,7 +1823,14 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     }
 
     // the last rounds run in one resident workgroup when every registered table belongs to the term
-    if (sc->fast && n_vars >= 11 && n_mles == sc->terms[0].n_factors) sc->tail_j0 = n_vars - 8;  // 2^8 = TAIL_PAIRS pairs
+    // (from the round of 2^8 = TAIL_PAIRS pairs on, or from round 2 in a smaller sum; the tail kernel reads extension
+    // tables, which every table is once folded, so a start in round 2 needs extension tables to begin with)
+    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
+        const u32 j0 = n_vars > 10 ? n_vars - 8 : 2;
+        bool all_ext = true;
+        for (u32 f = 0; f < sc->fast_nf; f++) all_ext = all_ext && mles[sc->fast_order[f]]->kind == DPS_EXT2;
+        if (j0 >= 3 || all_ext) sc->tail_j0 = j0;
+    }
 
     // scratch: two ping-pong buffers per table, extension limbs
     size_t scratch_words = 0;
