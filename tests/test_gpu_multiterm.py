@@ -125,3 +125,32 @@ def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
     one = np.array([1, 0], dtype=np.uint64)
     _check(dp, ctx, orc, n, [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(pt)],
            [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(pt)], [(one, [2, 0, 1])])
+
+
+@pytest.mark.parametrize("n_tabs", [4, 11])
+def test_resident_groups_give_way(dp, ctx, orc, n_tabs):
+    """A multi-term session stays on the GPU from the round of 256 pairs on (one workgroup, or one per group of
+    tables).  Another call on the context makes the resident launch exit through its mailbox, the interrupted
+    session reports it, an unfinished session can simply be dropped, and the context keeps working."""
+    n = 11
+    gpu, host, terms = _instance(ctx, orc, 700 + n_tabs, n, [n] * n_tabs, [], 2 * n_tabs, 2, True)
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
+    for how in ("other call", "abort", "dropped", "finish by hand"):
+        s = ctx.session(n, gpu, terms)
+        chal = None
+        rounds = n if how == "finish by hand" else 6  # rounds 3 and later run inside the resident launch
+        for j in range(rounds):
+            assert (s.round(chal) == ref_proof[j]).all()
+            chal = ref_point[j]
+        if how == "other call":
+            assert (ctx.eq_build(ref_point[:3]).download() == orc.eq_evals(ref_point[:3])).all()
+            with pytest.raises(dp.DpsError):
+                s.round(chal)
+        elif how == "abort":
+            s.abort()
+            with pytest.raises(dp.DpsError):
+                s.round(chal)
+        elif how == "finish by hand":
+            assert (s.finish(chal) == ref_finals).all()
+        del s
+        _check(dp, ctx, orc, n, gpu, host, terms)
