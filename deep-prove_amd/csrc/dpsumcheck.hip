@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -1309,6 +1310,11 @@ struct dps_sc {
     u32 poly_split_cap;                       // log2 of the most lanes a pair's work is worth spreading over
     bool descs_uploaded;                      // the descriptor block is on the device (uploaded when first needed)
     bool poly_raw;                            // the resident launch has one workgroup per group; the host adds their sums
+    bool wait_stays;                          // the launch waiting for mail stays for the rounds after the one it waits for
+    bool wait_skip1;                          // ... and was compiled to take p(1) from the claim
+    bool wait_fresh;                          // ... and has not been sent a mail yet (ending it loses nothing)
+    bool no_ahead;                            // a launch made ahead was in another call's way once: make no more
+    std::chrono::steady_clock::time_point ahead_at;  // when the launch that has had no mail yet was made
     bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
@@ -1341,7 +1347,12 @@ void tail_abort(dps_ctx *ctx)
     (void)hipStreamSynchronize(ctx->stream);
     __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
     owner->tail_running = false;
-    owner->broken = true;
+    // a launch that has had no mail yet has changed nothing: its session goes on with ordinary launches
+    if (owner->wait_fresh)
+        owner->no_ahead = true;
+    else
+        owner->broken = true;
+    owner->wait_fresh = false;
     ctx->tail_owner = nullptr;
 }
 
@@ -1411,6 +1422,12 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
 // Several groups resident side by side publish into 64-word slots of the pinned buffer from here on
 constexpr u32 POLY_RAW_MAX_GROUPS = 32;
 size_t poly_raw_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64; }
+
+// A round's launch is made ahead of time only with at most this many workgroups: each of them polls the mailbox
+constexpr u32 POLY_AHEAD_MAX_WORKGROUPS = 64;
+// ... and is trusted to be still waiting for its mail for this long (its own patience: spin_limit polls of pinned
+// memory, at least a few hundred milliseconds)
+constexpr int POLY_AHEAD_PATIENCE_MS = 20;
 
 // Rounds of at most this many pairs run on poly_split_kernel
 constexpr u64 POLY_SPLIT_MAX_PAIRS = 1ull << 16;
@@ -1645,6 +1662,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->tail_j0 = 0;
     sc->tail_running = false;
     sc->tail_seq0 = 0;
+    sc->wait_stays = sc->wait_skip1 = sc->wait_fresh = sc->no_ahead = false;
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
@@ -2377,111 +2395,184 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
                 sc->round = j;
             };
-            if (sc->tail_running) {
-                if (a.skip1) {
-                    // the resident launch of an earlier round runs this one
-                    post_mail();
-                    int32_t rc = sc->poly_raw ? take_raw_round() : wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
-                    if (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel)) {
-                        // without a finishing step of its own it exits after the last round
-                        sc->tail_running = false;
-                        ctx->tail_owner = nullptr;
-                    }
-                    // else it waits for the last challenge (dps_sc_finish)
-                    CHK(rc);
-                    took_round();
-                    return DPS_OK;
+            const u32 n_groups = (u32)sc->poly_tabs.size();
+            const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
+            // What a launch for round jj looks like: the kernel, its grid, whether it stays for the later rounds.
+            // Nothing here depends on a challenge, so a launch can be planned (and made) before its round begins.
+            struct Plan {
+                bool split, reside;
+                u32 split_log, blocks;
+                u64 n_pairs;
+            };
+            auto plan_round = [&](u32 jj, bool skip1_jj) {
+                Plan p;
+                p.n_pairs = 1ull << (sc->n_vars - jj);
+                p.split = p.n_pairs <= POLY_SPLIT_MAX_PAIRS;
+                p.split_log = 0;
+                p.blocks = blocks_for_pairs(p.n_pairs);
+                if (p.split) poly_split_plan(p.n_pairs, sc->poly_split_cap, n_groups <= POLY_RAW_MAX_GROUPS, &p.split_log, &p.blocks);
+                // a single workgroup (per group) from here on: it stays for the remaining rounds
+                // (several groups stay only with their tables in LDS: they must not read each other's stores)
+                p.reside = p.split && n_groups <= POLY_RAW_MAX_GROUPS && p.blocks == 1 && skip1_jj && jj < sc->n_vars &&
+                           sc->n_vars - jj + 1 <= (u32)dpk::POLY_RES_ROUNDS && (n_groups == 1 || poly_split_state_ok(ctx, nf, has_eq, true));
+                return p;
+            };
+            // Launches the kernel of round jj.  `ahead`: round jj has not begun (its challenge is not known); the kernel
+            // waits for the mail of sequence number `seq_jj` and takes the challenge and the message's scalars from it.
+            auto launch_round = [&](u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj) -> int32_t {
+                dpk::PolyArgs pa;
+                pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
+                pa.terms = sc->d_poly_terms;
+                pa.ops = sc->d_poly_ops;
+                if (inline_descs) {
+                    pa.groups = nullptr;
+                    pa.terms = nullptr;
+                    pa.ops = nullptr;
+                    pa.g0 = sc->h_poly_groups[jj - 1];
+                    if (!p.split && !sc->h_poly_ops.empty())
+                        memcpy(pa.o0, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
+                    else
+                        std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+                } else {
+                    CHK(ensure_descs(sc));
                 }
-                // evaluating t = 1 after all is not compiled into the resident variant: end it and launch normally
+                pa.q0 = pa.q1 = nullptr;
+                if (has_eq) {
+                    const u64 off = eq_level_off(sc->n_vars, jj);
+                    pa.q0 = sc->eq_c0 + off;
+                    pa.q1 = sc->eq_c1 + off;
+                }
+                pa.n_pairs = p.n_pairs;
+                pa.r0 = ahead ? 0 : a.r0;
+                pa.r1 = ahead ? 0 : a.r1;
+                pa.j = jj;
+                pa.last_round = 0;
+                pa.n_vars = sc->n_vars;
+                pa.spin_limit = 4000000;
+                pa.eq0 = sc->eq_c0;
+                pa.eq1 = sc->eq_c1;
+                pa.mail = ctx->d_pinned + (ctx->res_off - 64);
+                pa.seq = seq_jj;
+                pa.split_log = p.split_log;
+                pa.split_cap = sc->poly_split_cap;
+                pa.lds_state = pa.state_off = pa.pad = 0;
+                pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
+                pa.group_stride = 1;
+                pa.raw_out = nullptr;
+                pa.wait_first = ahead ? 1 : 0;
+                if (p.reside) {
+                    pa.last_round = sc->n_vars;
+                    if (n_groups > 1) {
+                        // one resident workgroup per group, each publishing its own sums
+                        CHK(ensure_descs(sc));
+                        pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
+                        pa.group_stride = n_groups;
+                        pa.raw_out = ctx->d_pinned + poly_raw_off(ctx);
+                    } else if (inline_descs) {
+                        // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
+                        // before anything else (and before it looks for mail); the area is not written again before a
+                        // message of this launch has arrived
+                        const size_t words = (size_t)(sc->n_vars - jj + 1) * sizeof(dpk::PolyGroup) / 8;
+                        memcpy(ctx->h_pinned, &sc->h_poly_groups[jj - 1], words * 8);
+                        pa.groups = reinterpret_cast<const dpk::PolyGroup *>(ctx->d_pinned);
+                    } else {
+                        pa.groups = sc->d_poly_groups + (size_t)(jj - 1);
+                    }
+                }
+                dpk::FastFin fl = ff;  // an early launch gets this round's scalars by mail
+                fl.seq = seq_jj;
+                fl.skip1 = skip1_jj ? 1 : 0;
+                fl.n_blocks = p.blocks * n_groups;
+                double pbytes = has_eq ? (double)p.n_pairs * 16.0 : 0.0;
+                for (u32 k = 0; k < sc->n_mles; k++)
+                    if (sc->poly_owner[k] >= 0) pbytes += (double)p.n_pairs * (jj >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
+                ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
+                if (p.split)
+                    CHK(launch_poly_split_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, p.reside, sc->d_partial, fl));
+                else
+                    CHK(launch_poly_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, sc->d_partial, fl));
+                HIPCHK(ctx, hipGetLastError());
+                return DPS_OK;
+            };
+            auto end_waiting_launch = [&]() -> int32_t {
                 __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
                 HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
                 __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
                 sc->tail_running = false;
+                sc->wait_fresh = false;
                 ctx->tail_owner = nullptr;
+                return DPS_OK;
+            };
+            // a launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an
+            // earlier round, or one made ahead during the previous round
+            bool on_gpu = sc->tail_running;
+            if (on_gpu && ((a.skip1 != 0) != sc->wait_skip1)) {
+                // it was compiled for the other way of getting p(1): end it and launch normally
+                CHK(end_waiting_launch());
+                on_gpu = false;
             }
-            dpk::PolyArgs pa;
-            const u32 n_groups = (u32)sc->poly_tabs.size();
-            pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
-            pa.terms = sc->d_poly_terms;
-            const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
-            // few pairs: the work of a pair is spread over several lanes (term by term); else one thread per pair
-            const bool split = n_pairs <= POLY_SPLIT_MAX_PAIRS;
-            pa.ops = sc->d_poly_ops;
-            if (inline_descs) {
-                pa.groups = nullptr;
-                pa.terms = nullptr;
-                pa.ops = nullptr;
-                pa.g0 = sc->h_poly_groups[j - 1];
-                if (!split && !sc->h_poly_ops.empty())
-                    memcpy(pa.o0, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
-                else
-                    std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+            if (on_gpu && sc->wait_fresh && std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS)) {
+                // the caller took its time: the launch made ahead may have given up waiting (it polls for much longer
+                // than this, so up to here it certainly has not)
+                CHK(end_waiting_launch());
+                on_gpu = false;
+            }
+            bool stays, raw_now;
+            if (on_gpu) {
+                post_mail();
+                sc->wait_fresh = false;
+                stays = sc->wait_stays;
+                raw_now = sc->poly_raw;
             } else {
-                CHK(ensure_descs(sc));
-            }
-            pa.q0 = a.q0;
-            pa.q1 = a.q1;
-            pa.n_pairs = n_pairs;
-            pa.r0 = a.r0;
-            pa.r1 = a.r1;
-            pa.j = j;
-            pa.last_round = 0;
-            pa.n_vars = sc->n_vars;
-            pa.spin_limit = 4000000;
-            pa.eq0 = sc->eq_c0;
-            pa.eq1 = sc->eq_c1;
-            pa.mail = ctx->d_pinned + (ctx->res_off - 64);
-            pa.seq = fa.seq;
-            pa.split_log = pa.split_cap = pa.lds_state = pa.state_off = 0;
-            pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
-            pa.group_stride = 1;
-            pa.raw_out = nullptr;
-            u32 sblocks = blocks;
-            if (split) poly_split_plan(n_pairs, sc->poly_split_cap, n_groups <= POLY_RAW_MAX_GROUPS, &pa.split_log, &sblocks);
-            pa.split_cap = sc->poly_split_cap;
-            // a single workgroup from here on: it stays for the remaining rounds
-            // (several groups stay only with their tables in LDS: they must not read each other's stores)
-            const bool reside = split && n_groups <= POLY_RAW_MAX_GROUPS && sblocks == 1 && a.skip1 && j < sc->n_vars &&
-                                sc->n_vars - j + 1 <= (u32)dpk::POLY_RES_ROUNDS &&
-                                (n_groups == 1 || poly_split_state_ok(ctx, nf, has_eq, true));
-            if (reside) {
-                pa.last_round = sc->n_vars;
-                if (n_groups > 1) {
-                    // one resident workgroup per group, each publishing its own sums
-                    CHK(ensure_descs(sc));
-                    pa.groups = sc->d_poly_groups + (size_t)(j - 1) * n_groups;
-                    pa.group_stride = n_groups;
-                    pa.raw_out = ctx->d_pinned + poly_raw_off(ctx);
-                } else if (inline_descs) {
-                    // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
-                    // before its first round, and this call returns only after that round's message has arrived
-                    const size_t words = (size_t)(sc->n_vars - j + 1) * sizeof(dpk::PolyGroup) / 8;
-                    memcpy(ctx->h_pinned, &sc->h_poly_groups[j - 1], words * 8);
-                    pa.groups = reinterpret_cast<const dpk::PolyGroup *>(ctx->d_pinned);
-                } else {
-                    pa.groups = sc->d_poly_groups + (size_t)(j - 1);
+                const Plan p = plan_round(j, a.skip1 != 0);
+                CHK(launch_round(j, p, a.skip1 != 0, false, fa.seq));
+                stays = p.reside;
+                raw_now = p.reside && n_groups > 1;
+                if (p.reside) {
+                    sc->tail_running = true;
+                    sc->tail_seq0 = fa.seq;
+                    ctx->tail_owner = sc;
+                    sc->poly_raw = raw_now;
+                    sc->wait_stays = true;
+                    sc->wait_skip1 = true;
+                    sc->wait_fresh = false;
                 }
             }
-            ff.n_blocks = sblocks * n_groups;
-            double pbytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
-            for (u32 k = 0; k < sc->n_mles; k++)
-                if (sc->poly_owner[k] >= 0) pbytes += (double)n_pairs * (j >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
-            ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
-            if (split)
-                CHK(launch_poly_split_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(sblocks, n_groups), sc->poly_max_tabs, reside, sc->d_partial, ff));
-            else
-                CHK(launch_poly_dispatch(ctx, nf, has_eq, a.skip1 != 0, pa, dim3(blocks, n_groups), sc->poly_max_tabs, sc->d_partial, ff));
-            HIPCHK(ctx, hipGetLastError());
-            if (reside) {
-                sc->tail_running = true;
-                sc->tail_seq0 = fa.seq;
-                ctx->tail_owner = sc;
-                sc->poly_raw = n_groups > 1;
+            if (!stays) {
+                // the launch of this round ends with it
+                sc->tail_running = false;
+                ctx->tail_owner = nullptr;
+                // The next round's launch is made now, behind this one: by the time this round's message has crossed to
+                // the host and the challenge is drawn, it is already on the GPU looking for its mail.  Only for rounds
+                // of few workgroups (every workgroup polls the mailbox), and not while launches are being timed.
+                if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
+                    // p(1) comes from the claim unless the scale vanishes at 1, i.e. unless the eq point is 0 there
+                    bool skip1_next = true;
+                    if (has_eq) {
+                        const E2 rho = sc->eq_info->point[j];
+                        skip1_next = !(rho.c0 == 0 && rho.c1 == 0);
+                    }
+                    const Plan pn = plan_round(j + 1, skip1_next);
+                    if (pn.split && pn.blocks * n_groups <= POLY_AHEAD_MAX_WORKGROUPS) {
+                        CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
+                        sc->tail_running = true;
+                        sc->tail_seq0 = ctx->seq + 1;
+                        ctx->tail_owner = sc;
+                        sc->wait_stays = pn.reside;
+                        sc->wait_skip1 = skip1_next;
+                        sc->wait_fresh = true;
+                        sc->ahead_at = std::chrono::steady_clock::now();
+                        sc->poly_raw = pn.reside && n_groups > 1;
+                    }
+                }
             }
-            if (reside && n_groups > 1)
-                CHK(take_raw_round());
-            else
-                CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
+            int32_t rc = raw_now ? take_raw_round() : wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
+            if (stays && (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel))) {
+                // (without a finishing step of its own a resident launch exits after the last round)
+                sc->tail_running = false;
+                ctx->tail_owner = nullptr;
+            }
+            CHK(rc);
             took_round();
             return DPS_OK;
         }

@@ -1105,6 +1105,8 @@ struct PolyArgs {
     u32 state_off;
     u32 finish;      // resident rounds: stay after the last round for the last challenge and publish the final evaluations
     u32 group_stride;  // resident rounds: descriptors of consecutive rounds of one group lie this many apart
+    u32 wait_first;  // launched ahead of its round: the challenge and the scalars of round j also arrive by mail (seq)
+    u32 pad;
     // Several groups resident side by side (one workgroup each, gridDim.y of them): a workgroup cannot finish the
     // message, which is the sum over the groups, so each publishes its own sums q(t) (and later its tables' final
     // evaluations) to its 64-word slot raw_out + 64 * blockIdx.y, laid out like the main result area, and the host adds.
@@ -1356,6 +1358,28 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
         __syncthreads();
     }
+    // the challenge of a round and the scalars of its message, from the mail the host posted for it
+    auto take_mail = [&](u64 seq) -> bool {
+        if (!tail_wait_mail(a.mail, a.spin_limit, seq, box, &ok_flag)) return false;
+        // a run-time switch to evaluating t = 1 (or not) is not compiled in: the host ends the launch instead
+        if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
+        r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+#pragma unroll
+        for (int k = 0; k < 2 * MAX_PTS; k++) {
+            cf.scale[k] = box[MAIL_SCALE + k];
+            cf.cext[k] = box[MAIL_CEXT + k];
+        }
+        cf.k0 = box[MAIL_K];
+        cf.k1 = box[MAIL_K + 1];
+        cf.claim0 = box[MAIL_CLAIM];
+        cf.claim1 = box[MAIL_CLAIM + 1];
+        cf.const0 = box[MAIL_CONST];
+        cf.const1 = box[MAIL_CONST + 1];
+        cf.seq = seq;
+        return true;
+    };
+    // launched while the previous round was still running: everything that depends on its challenge comes by mail
+    if (a.wait_first && !take_mail(a.seq)) return;
   for (;;) {
     const PolyGroup &g = gall[j - a.j];
     const u32 n_tabs = g.n_tabs;
@@ -1526,10 +1550,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         }
         // stay for the next round: its challenge and the scalars of its message arrive by mail
         j++;
-        if (!tail_wait_mail(a.mail, a.spin_limit, a.seq + (j - a.j), box, &ok_flag)) return;
-        // a run-time switch to evaluating t = 1 is not compiled in: the host ends the residency instead
-        if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
-        r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+        if (!take_mail(a.seq + (j - a.j))) return;
         n_pairs >>= 1;
         if (sl < a.split_cap && (n_pairs << (sl + 1)) <= (u64)BLOCK) sl++;
         if (EQ) {
@@ -1537,18 +1558,6 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
             q0 = a.eq0 + off;
             q1 = a.eq1 + off;
         }
-#pragma unroll
-        for (int k = 0; k < 2 * MAX_PTS; k++) {
-            cf.scale[k] = box[MAIL_SCALE + k];
-            cf.cext[k] = box[MAIL_CEXT + k];
-        }
-        cf.k0 = box[MAIL_K];
-        cf.k1 = box[MAIL_K + 1];
-        cf.claim0 = box[MAIL_CLAIM];
-        cf.claim1 = box[MAIL_CLAIM + 1];
-        cf.const0 = box[MAIL_CONST];
-        cf.const1 = box[MAIL_CONST + 1];
-        cf.seq = a.seq + (j - a.j);
         if (a.lds_state) {
             in_lds = wrote;
             dst_is_a = !dst_is_a;
@@ -1572,7 +1581,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     if (take_ticket(ff.counter, gridDim.x * gridDim.y, &last_flag)) {
         E2 q[NP];
         gather_partials<NP>(ff, lds, q);
-        fast_finalize<NF>(ff, q, res);
+        fast_finalize<NF>(cf, q, res);
     }
     return;
   }

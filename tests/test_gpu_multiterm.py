@@ -154,3 +154,29 @@ def test_resident_groups_give_way(dp, ctx, orc, n_tabs):
             assert (s.finish(chal) == ref_finals).all()
         del s
         _check(dp, ctx, orc, n, gpu, host, terms)
+
+
+@pytest.mark.parametrize("n_tabs", [4, 11])
+def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
+    """Rounds of few workgroups are launched during the round before and wait for their challenge.  Such a launch
+    has changed nothing yet: when another call needs the context, or the caller is slow, it ends, and the session
+    carries on with ordinary launches and the same messages."""
+    import time
+    n = 14
+    gpu, host, terms = _instance(ctx, orc, 900 + n_tabs, n, [n] * n_tabs, [], 2 * n_tabs, 2, True)
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
+    for after in (1, 3, 4, 5):  # up to round 5 no launch has stayed for later rounds (that takes n - j + 1 <= 9)
+        for how in ("other call", "slow caller"):
+            s = ctx.session(n, gpu, terms)
+            chal = None
+            for j in range(n):
+                assert (s.round(chal) == ref_proof[j]).all(), (after, how, j)
+                chal = ref_point[j]
+                if j + 1 == after:
+                    if how == "other call":
+                        assert (ctx.eq_build(ref_point[:3]).download() == orc.eq_evals(ref_point[:3])).all()
+                    else:
+                        time.sleep(0.05)
+            assert (s.finish(chal) == ref_finals).all()
+            del s
+    _check(dp, ctx, orc, n, gpu, host, terms)
