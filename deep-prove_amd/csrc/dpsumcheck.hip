@@ -2246,6 +2246,13 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         const u32 nf = sc->fast_nf;
         dpk::FastFin ff;
         memset(&ff, 0, sizeof ff);
+        // the kernels hand over the sums q(t); the message is formed from them here (take_sums)
+        struct {
+            u64 scale[2 * dpk::MAX_PTS];  // p(t) = scale(t) q(t) + const, t = 0..nf
+            u64 cext[2 * dpk::MAX_PTS];   // eq factor: p(nf + 1) = sum_i cext_i q(i) + k + const
+            u64 k0, k1;
+        } hf;
+        memset(&hf, 0, sizeof hf);
         if (j >= 2) {
             const E2 r = gl::e2(challenge[0], challenge[1]);
             a.r0 = r.c0;
@@ -2268,44 +2275,36 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
         for (u32 t = 0; t <= sc->degree; t++) {
             E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
-            ff.scale[2 * t] = sc_t.c0;
-            ff.scale[2 * t + 1] = sc_t.c1;
+            hf.scale[2 * t] = sc_t.c0;
+            hf.scale[2 * t + 1] = sc_t.c1;
         }
-        E2 s1 = gl::e2(ff.scale[2], ff.scale[3]);
+        E2 s1 = gl::e2(hf.scale[2], hf.scale[3]);
         const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
         a.skip1 = skip1 ? 1 : 0;
-        ff.claim0 = sc->claim.c0;
-        ff.claim1 = sc->claim.c1;
         if (has_eq) {
             const u64 off = eq_level_off(sc->n_vars, j);
             a.q0 = sc->eq_c0 + off;
             a.q1 = sc->eq_c1 + off;
             // p(nf + 1) = sum_i cext_i q(i) + k + const
-            const E2 s_top = gl::e2(ff.scale[2 * (nf + 1)], ff.scale[2 * (nf + 1) + 1]);
+            const E2 s_top = gl::e2(hf.scale[2 * (nf + 1)], hf.scale[2 * (nf + 1) + 1]);
             E2 cext[dpk::MAX_PTS];
             for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
             if (skip1) {
                 // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
                 const E2 A = gl::mul(cext[1], h_e2_inv(s1));
-                cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(ff.scale[0], ff.scale[1])));
+                cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(hf.scale[0], hf.scale[1])));
                 const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
-                ff.k0 = kk.c0;
-                ff.k1 = kk.c1;
+                hf.k0 = kk.c0;
+                hf.k1 = kk.c1;
                 cext[1] = gl::e2_zero();
             }
             for (u32 i = 0; i <= nf; i++) {
-                ff.cext[2 * i] = cext[i].c0;
-                ff.cext[2 * i + 1] = cext[i].c1;
+                hf.cext[2 * i] = cext[i].c0;
+                hf.cext[2 * i + 1] = cext[i].c1;
             }
         }
         ff.partial = sc->d_partial;
         ff.n_blocks = blocks;
-        ff.degree = sc->degree;
-        ff.has_eq = has_eq ? 1 : 0;
-        ff.skip1 = a.skip1;
-        ff.const0 = cst.c0;
-        ff.const1 = cst.c1;
-        ff.out_dev = sc->d_result;
         ff.out_host = fa.out_host;
         ff.seq = fa.seq;
         ff.counter = sc->d_counter;
@@ -2314,41 +2313,41 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             u64 *mb = mailbox(ctx);
             mb[dpk::MAIL_R] = a.r0;
             mb[dpk::MAIL_R + 1] = a.r1;
-            for (u32 k = 0; k < 2 * dpk::MAX_PTS; k++) {
-                mb[dpk::MAIL_SCALE + k] = ff.scale[k];
-                mb[dpk::MAIL_CEXT + k] = ff.cext[k];
-            }
-            mb[dpk::MAIL_K] = ff.k0;
-            mb[dpk::MAIL_K + 1] = ff.k1;
-            mb[dpk::MAIL_CLAIM] = ff.claim0;
-            mb[dpk::MAIL_CLAIM + 1] = ff.claim1;
-            mb[dpk::MAIL_CONST] = cst.c0;
-            mb[dpk::MAIL_CONST + 1] = cst.c1;
             mb[dpk::MAIL_SKIP1] = a.skip1;
             send_mail(ctx, fa.seq);
         };
-        // several resident groups: their sums q(t) added, then the message as fast_finalize forms it
-        auto take_raw_round = [&]() -> int32_t {
-            const u32 n_groups = (u32)sc->poly_tabs.size(), np = nf + 1;
+        // Waits for the sums q(t), t = 0..nf, of this round (one set, or one per resident group, which are added) and
+        // forms the message: p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was skipped; with an eq factor
+        // p(nf + 1) by extrapolation of q (coefficients above).
+        auto take_sums = [&](bool per_group) -> int32_t {
+            const u32 np = nf + 1;
             E2 q[dpk::MAX_PTS];
-            for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
-            for (u32 g = 0; g < n_groups; g++) {
-                u64 w[2 * dpk::MAX_PTS];
-                CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
-                for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
+            u64 w[2 * dpk::MAX_PTS];
+            if (per_group) {
+                const u32 n_groups = (u32)sc->poly_tabs.size();
+                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+                for (u32 g = 0; g < n_groups; g++) {
+                    CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
+                    for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
+                }
+            } else {
+                CHK(wait_result(ctx, fa.seq, 0, 2 * np, w));
+                for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
             }
             E2 msg[dpk::MAX_PTS + 1];
-            for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(ff.scale[2 * t], ff.scale[2 * t + 1]), q[t]), cst);
+            for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(hf.scale[2 * t], hf.scale[2 * t + 1]), q[t]), cst);
             if (a.skip1) msg[1] = gl::sub(sc->claim, msg[0]);
             if (has_eq) {
-                E2 e = gl::add(gl::e2(ff.k0, ff.k1), cst);
+                E2 e = gl::add(gl::e2(hf.k0, hf.k1), cst);
                 for (u32 i = 0; i < np; i++)
-                    if (!(a.skip1 && i == 1)) e = gl::add(e, gl::mul(gl::e2(ff.cext[2 * i], ff.cext[2 * i + 1]), q[i]));
+                    if (!(a.skip1 && i == 1)) e = gl::add(e, gl::mul(gl::e2(hf.cext[2 * i], hf.cext[2 * i + 1]), q[i]));
                 msg[np] = e;
             }
+            sc->last_msg.resize(sc->degree + 1);
             for (u32 t = 0; t <= sc->degree; t++) {
                 evals_out[2 * t] = msg[t].c0;
                 evals_out[2 * t + 1] = msg[t].c1;
+                sc->last_msg[t] = msg[t];
             }
             return DPS_OK;
         };
@@ -2365,11 +2364,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 ta.eq1 = sc->eq_c1;
                 ta.n_vars = sc->n_vars;
                 ta.j0 = j;
-                ta.degree = sc->degree;
-                ta.has_eq = has_eq ? 1 : 0;
                 ta.mail = ctx->d_pinned + (ctx->res_off - 64);
                 ta.out_host = fa.out_host;
-                ta.out_dev = sc->d_result;
                 ta.seq0 = fa.seq;
                 sc->tail_seq0 = fa.seq;
                 ta.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
@@ -2383,18 +2379,11 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 sc->tail_running = true;
                 ctx->tail_owner = sc;
             }
-            CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
-            sc->last_msg.resize(sc->degree + 1);
-            for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
+            CHK(take_sums(false));
             sc->round = j;
             return DPS_OK;
         }
         if (sc->poly) {
-            auto took_round = [&]() {
-                sc->last_msg.resize(sc->degree + 1);
-                for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
-                sc->round = j;
-            };
             const u32 n_groups = (u32)sc->poly_tabs.size();
             const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
             // What a launch for round jj looks like: the kernel, its grid, whether it stays for the later rounds.
@@ -2479,9 +2468,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                         pa.groups = sc->d_poly_groups + (size_t)(jj - 1);
                     }
                 }
-                dpk::FastFin fl = ff;  // an early launch gets this round's scalars by mail
+                dpk::FastFin fl = ff;
                 fl.seq = seq_jj;
-                fl.skip1 = skip1_jj ? 1 : 0;
                 fl.n_blocks = p.blocks * n_groups;
                 double pbytes = has_eq ? (double)p.n_pairs * 16.0 : 0.0;
                 for (u32 k = 0; k < sc->n_mles; k++)
@@ -2566,14 +2554,14 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                     }
                 }
             }
-            int32_t rc = raw_now ? take_raw_round() : wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out);
+            int32_t rc = take_sums(raw_now);
             if (stays && (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel))) {
                 // (without a finishing step of its own a resident launch exits after the last round)
                 sc->tail_running = false;
                 ctx->tail_owner = nullptr;
             }
             CHK(rc);
-            took_round();
+            sc->round = j;
             return DPS_OK;
         }
         double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
@@ -2586,6 +2574,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j], has_eq, j >= 2, a, blocks, sc->d_partial, ff));
             HIPCHK(ctx, hipGetLastError());
         }
+        CHK(take_sums(false));
+        sc->round = j;
+        return DPS_OK;
     } else {
         if (j >= 2) CHK(launch_folds(sc, j, false, challenge));
         for (u32 base = 0; base < sc->n_terms; base += 65535) {
@@ -2597,10 +2588,6 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         }
     }
     CHK(wait_result(ctx, fa.seq, 0, 2 * (sc->degree + 1), evals_out));
-    if (sc->fast) {
-        sc->last_msg.resize(sc->degree + 1);
-        for (u32 t = 0; t <= sc->degree; t++) sc->last_msg[t] = gl::e2(evals_out[2 * t], evals_out[2 * t + 1]);
-    }
     sc->round = j;
     return DPS_OK;
 }

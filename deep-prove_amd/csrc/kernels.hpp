@@ -548,30 +548,14 @@ struct ProdArgs {
     u32 skip1;    // 1: t = 1 is not evaluated (the launch picks the kernel variant accordingly)
 };
 
-// What the last workgroup needs to turn the sums q(t), t = 0..NF, into the round
-// message p(t) = scale(t) q(t) + const, t = 0..degree.
-//
-// With an eq factor the message has one point more than the kernel sums:
-// q(NF + 1) = sum_i ext_i q(i) (Lagrange over the nodes 0..NF), so
-// p(NF + 1) = sum_i cext_i q(i) + const with cext_i = scale(NF + 1) ext_i.
-//
-// skip1: the caller knows claim = p(0) + p(1); the kernel did not sum q(1).
-// Then p(1) = claim - p(0), and q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
-// is folded into the coefficients by the host: with A = cext_1 / scale(1),
-// cext_0 becomes cext_0 - A scale(0), and k = A (claim - 2 const) is added.
-// Every product is then independent of the others: one lane each.
+// The kernels hand the host the sums q(t), t = 0..NF (q(1) left at zero when t = 1 was skipped), not the round
+// message: p(t) = scale(t) q(t) + const, the extra point p(NF + 1) of a sum with an eq factor, and p(1) from the
+// claim are a dozen field products, which one GPU lane takes about 2 us over and a CPU core 0.1 us, while the
+// kernel of the next round cannot start before the host has drawn its challenge anyway.
 struct FastFin {
-    const u64 *partial;
+    const u64 *partial;  // word k of workgroup b at partial[k * n_blocks + b]
     u32 n_blocks;
-    u32 degree;       // of the message: NF, or NF + 1 with an eq factor
-    u32 has_eq;
-    u32 skip1;
-    u64 scale[2 * MAX_PTS];  // scale(t) for t = 0..degree, extension elements
-    u64 cext[2 * MAX_PTS];   // coefficient of q(i) in p(NF + 1), i = 0..NF (eq factor only; entry 1 unused when skip1)
-    u64 k0, k1;              // constant part of p(NF + 1) (eq factor and skip1 only, else 0)
-    u64 claim0, claim1;      // p(0) + p(1), used when skip1
-    u64 const0, const1;      // constant terms summed over the remaining hypercube
-    u64 *out_dev;
+    u32 pad;
     u64 *out_host;
     u64 seq;
     u32 *counter;
@@ -583,73 +567,46 @@ __device__ __forceinline__ void gather_partials(const FastFin &ff, u32 *lds, E2 
 {
 #pragma unroll
     for (int t = 0; t < NP; t++) q[t] = gl::e2_zero();
-    for (u32 b = threadIdx.x; b < ff.n_blocks; b += BLOCK) {
-        const u64 *p = ff.partial + (u64)b * 2 * MAX_PTS;
+    // Word k of workgroup b is at partial[k * n_blocks + b]: a wavefront's load reads 64 adjacent words.  (With a
+    // workgroup's words side by side every lane touched a cache line of its own, and the gather of 768 workgroups took
+    // 5 to 7 us.)  A thread issues the loads of all its workgroups before it adds: one wait, not one per workgroup.
+    constexpr int AHEAD = 4;
+    for (u32 b0 = threadIdx.x; b0 < ff.n_blocks; b0 += AHEAD * BLOCK) {
+        u64 w[AHEAD][2 * NP];
 #pragma unroll
-        for (int t = 0; t < NP; t++) {
-            q[t].c0 = gl::add(q[t].c0, ld_agent(p + 2 * t));
-            q[t].c1 = gl::add(q[t].c1, ld_agent(p + 2 * t + 1));
+        for (int u = 0; u < AHEAD; u++) {
+            const u32 b = b0 + u * BLOCK;
+            const u64 *p = ff.partial + b;
+#pragma unroll
+            for (int k = 0; k < 2 * NP; k++) w[u][k] = b < ff.n_blocks ? ld_agent(p + (u64)k * ff.n_blocks) : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+#pragma unroll
+            for (int t = 0; t < NP; t++) {
+                q[t].c0 = gl::add(q[t].c0, w[u][2 * t]);
+                q[t].c1 = gl::add(q[t].c1, w[u][2 * t + 1]);
+            }
         }
     }
     block_reduce<NP>(q, lds);
 }
 
-// sums[t] = q(t) for t = 0..NF, valid in thread 0.  res: 6 * MAX_PTS words of LDS.
-template <int NF>
-__device__ __forceinline__ void fast_finalize(const FastFin &ff, const E2 (&sums)[NF + 1], u64 *res)
+// sums[t] = q(t) for t = 0..NP - 1, valid in thread 0: to the host as 2 * NP words, and the ticket counter back to zero
+template <int NP>
+__device__ __forceinline__ void publish_sums(u64 *out_host, u64 seq, u32 *counter, const E2 (&sums)[NP])
 {
-    constexpr int NP = NF + 1;
-    u64 *q = res;                  // 2 * NP words
-    u64 *prod = res + 2 * MAX_PTS; // 2 * (2 * NP) words
-    u64 *out = res + 2 * MAX_PTS;  // reused for the message after the products are consumed
     if (threadIdx.x == 0) {
+        if (counter) *counter = 0;
+        u64 chk = seq;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            q[2 * t] = sums[t].c0;
-            q[2 * t + 1] = sums[t].c1;
+            chk ^= rotl64(sums[t].c0, 2 * t + 1) ^ rotl64(sums[t].c1, 2 * t + 2);
+            st_sys(out_host + 2 * t, sums[t].c0);
+            st_sys(out_host + 2 * t + 1, sums[t].c1);
         }
-    }
-    __syncthreads();
-    // lane t < NP: scale(t) q(t); lane NP + i: cext_i q(i)
-    if (threadIdx.x < 2 * NP) {
-        const u32 l = threadIdx.x, i = l < NP ? l : l - NP;
-        const bool needed = !(ff.skip1 && i == 1) && (l < NP || ff.has_eq);
-        E2 v = gl::e2_zero();
-        if (needed) {
-            // the coefficient is picked with constant indices so that it stays in registers
-            E2 c = gl::e2_zero();
-#pragma unroll
-            for (int k = 0; k < NP; k++) {
-                if (l == (u32)k) c = gl::e2(ff.scale[2 * k], ff.scale[2 * k + 1]);
-                if (l == (u32)(NP + k)) c = gl::e2(ff.cext[2 * k], ff.cext[2 * k + 1]);
-            }
-            v = gl::mul(gl::e2(q[2 * i], q[2 * i + 1]), c);
-        }
-        prod[2 * l] = v.c0;
-        prod[2 * l + 1] = v.c1;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        E2 msg[NP + 1];
-        const E2 cst = gl::e2(ff.const0, ff.const1);
-#pragma unroll
-        for (int t = 0; t < NP; t++) msg[t] = gl::add(gl::e2(prod[2 * t], prod[2 * t + 1]), cst);
-        if (ff.skip1) msg[1] = gl::sub(gl::e2(ff.claim0, ff.claim1), msg[0]);
-        E2 e = gl::add(gl::e2(ff.k0, ff.k1), cst);
-#pragma unroll
-        for (int i = 0; i < NP; i++) e = gl::add(e, gl::e2(prod[2 * (NP + i)], prod[2 * (NP + i) + 1]));
-        msg[NP] = e;
-#pragma unroll
-        for (int t = 0; t <= NP; t++) {
-            if ((u32)t <= ff.degree) {
-                out[2 * t] = msg[t].c0;
-                out[2 * t + 1] = msg[t].c1;
-                ff.out_dev[2 * t] = msg[t].c0;
-                ff.out_dev[2 * t + 1] = msg[t].c1;
-            }
-        }
-        if (ff.counter) *ff.counter = 0;
-        publish_words(ff.out_host, 0, out, 2 * (ff.degree + 1), ff.seq);
+        st_sys(out_host + HOST_CHK_SLOT, chk);
+        st_sys(out_host + HOST_SEQ_SLOT, seq);
     }
 }
 
@@ -658,7 +615,6 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 {
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
-    __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
     const E2 r = gl::e2(a.r0, a.r1);
     const gl::E2P rp = gl::prep(r);
@@ -809,21 +765,22 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     block_reduce<NP>(acc, lds);
     if (gridDim.x == 1) {
         // a single workgroup: its sums are the round's sums, no partials and no ticket
-        fast_finalize<NF>(ff, acc, res);
+        publish_sums<NP>(ff.out_host, ff.seq, ff.counter, acc);
         return;
     }
     if (threadIdx.x == 0) {
-        u64 *o = partial + (u64)blockIdx.x * 2 * MAX_PTS;
+        u64 *o = partial + blockIdx.x;
+        const u64 total = gridDim.x;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            st_agent(o + 2 * t, acc[t].c0);
-            st_agent(o + 2 * t + 1, acc[t].c1);
+            st_agent(o + (2 * t) * total, acc[t].c0);
+            st_agent(o + (2 * t + 1) * total, acc[t].c1);
         }
     }
     if (take_ticket(ff.counter, gridDim.x, &last_flag)) {
         E2 q[NP];
         gather_partials<NP>(ff, lds, q);
-        fast_finalize<NF>(ff, q, res);
+        publish_sums<NP>(ff.out_host, ff.seq, ff.counter, q);
     }
 }
 
@@ -840,8 +797,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 // ---------------------------------------------------------------------------
 constexpr int TAIL_PAIRS = 256;
 // mailbox words; MAIL_SEQ == MAIL_ABORT_SEQ tells the kernel to exit
-constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SCALE = 4, MAIL_CEXT = MAIL_SCALE + 2 * MAX_PTS, MAIL_K = MAIL_CEXT + 2 * MAX_PTS,
-              MAIL_CLAIM = MAIL_K + 2, MAIL_CONST = MAIL_CLAIM + 2, MAIL_SKIP1 = MAIL_CONST + 2, MAIL_WORDS = MAIL_SKIP1 + 1;
+constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_WORDS = 5;
 static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
 constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
 
@@ -854,10 +810,8 @@ struct TailArgs {
     const u64 *eq0;    // eq storage (level 0 at entry 0), eq factor only
     const u64 *eq1;
     u32 n_vars, j0;    // the sum's variables, first round handled here (1-based)
-    u32 degree, has_eq;
     const u64 *mail;   // host mailbox, MAIL_WORDS words
-    u64 *out_host;     // message limbs, HOST_SEQ_SLOT, HOST_FINALS_SLOT
-    u64 *out_dev;
+    u64 *out_host;     // the sums q(t), HOST_SEQ_SLOT, HOST_FINALS_SLOT
     u64 seq0;          // sequence number of round j0; round j uses seq0 + (j - j0), the final evaluations seq0 + (n_vars - j0 + 1)
     u32 spin_limit;
 };
@@ -971,26 +925,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
             }
         }
         block_reduce<NP>(acc, lds);
-        // the round message, as in the per-round kernels
-        FastFin ff;
-        ff.degree = a.degree;
-        ff.has_eq = a.has_eq;
-        ff.skip1 = skip1 ? 1 : 0;
-#pragma unroll
-        for (int k = 0; k < 2 * MAX_PTS; k++) ff.scale[k] = box[MAIL_SCALE + k];
-        ff.claim0 = box[MAIL_CLAIM];
-        ff.claim1 = box[MAIL_CLAIM + 1];
-        ff.k0 = box[MAIL_K];
-        ff.k1 = box[MAIL_K + 1];
-#pragma unroll
-        for (int k = 0; k < 2 * MAX_PTS; k++) ff.cext[k] = box[MAIL_CEXT + k];
-        ff.const0 = box[MAIL_CONST];
-        ff.const1 = box[MAIL_CONST + 1];
-        ff.out_dev = a.out_dev;
-        ff.out_host = a.out_host;
-        ff.seq = a.seq0 + (j - a.j0);
-        ff.counter = nullptr;
-        fast_finalize<NF>(ff, acc, res);
+        publish_sums<NP>(a.out_host, a.seq0 + (j - a.j0), nullptr, acc);
         __syncthreads();
         to_ping = !to_ping;
         n_pairs >>= 1;
@@ -1110,7 +1045,7 @@ struct PolyArgs {
     // Several groups resident side by side (one workgroup each, gridDim.y of them): a workgroup cannot finish the
     // message, which is the sum over the groups, so each publishes its own sums q(t) (and later its tables' final
     // evaluations) to its 64-word slot raw_out + 64 * blockIdx.y, laid out like the main result area, and the host adds.
-    u64 *raw_out;    // nullptr: a single workgroup finishes the message itself
+    u64 *raw_out;    // nullptr: a single workgroup, which publishes to the main result area
 };
 
 template <int NF, bool EQ, bool SKIP1>
@@ -1119,7 +1054,6 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     constexpr int NP = NF + 1;
     extern __shared__ u64 dyn[];  // [n_tabs][4][BLOCK]: value c0, c1, slope c0, c1
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
-    __shared__ u64 res[6 * MAX_PTS];
     __shared__ int last_flag;
     // The group's descriptors come from device memory; read from there inside the loops every use would be
     // a dependent load of its own (the small rounds are nothing but such latencies), so they are staged in LDS once.
@@ -1288,21 +1222,22 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     for (int t = 0; t < NP; t++) acc[t] = lz[t];
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
-        fast_finalize<NF>(ff, acc, res);
+        publish_sums<NP>(ff.out_host, ff.seq, ff.counter, acc);
         return;
     }
     if (tid == 0) {
-        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
+        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x);
+        const u64 total = (u64)gridDim.x * gridDim.y;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            st_agent(o + 2 * t, acc[t].c0);
-            st_agent(o + 2 * t + 1, acc[t].c1);
+            st_agent(o + (2 * t) * total, acc[t].c0);
+            st_agent(o + (2 * t + 1) * total, acc[t].c1);
         }
     }
     if (take_ticket(ff.counter, gridDim.x * gridDim.y, &last_flag)) {
         E2 q[NP];
         gather_partials<NP>(ff, lds, q);
-        fast_finalize<NF>(ff, q, res);
+        publish_sums<NP>(ff.out_host, ff.seq, ff.counter, q);
     }
 }
 
@@ -1330,7 +1265,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     u64 n_pairs = a.n_pairs;
     E2 r = gl::e2(a.r0, a.r1);
     const u64 *q0 = a.q0, *q1 = a.q1;
-    FastFin cf = ff;
+    u64 cf_seq = ff.seq;  // sequence number of the round being worked on
     u32 sl = a.split_log;
     u32 in_lds = 0;  // tables (bit per slot) whose current contents this workgroup holds in LDS
     // resident rounds with lds_state: the folded tables, alternating between a buffer of 2 * BLOCK entries per limb
@@ -1358,24 +1293,13 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         for (u32 w = tid; w < staged * (sizeof(PolyTerm) / 8); w += BLOCK) td[w] = ts[w];
         __syncthreads();
     }
-    // the challenge of a round and the scalars of its message, from the mail the host posted for it
+    // the challenge of a round, from the mail the host posted for it
     auto take_mail = [&](u64 seq) -> bool {
         if (!tail_wait_mail(a.mail, a.spin_limit, seq, box, &ok_flag)) return false;
         // a run-time switch to evaluating t = 1 (or not) is not compiled in: the host ends the launch instead
         if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
         r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
-#pragma unroll
-        for (int k = 0; k < 2 * MAX_PTS; k++) {
-            cf.scale[k] = box[MAIL_SCALE + k];
-            cf.cext[k] = box[MAIL_CEXT + k];
-        }
-        cf.k0 = box[MAIL_K];
-        cf.k1 = box[MAIL_K + 1];
-        cf.claim0 = box[MAIL_CLAIM];
-        cf.claim1 = box[MAIL_CLAIM + 1];
-        cf.const0 = box[MAIL_CONST];
-        cf.const1 = box[MAIL_CONST + 1];
-        cf.seq = seq;
+        cf_seq = seq;
         return true;
     };
     // launched while the previous round was still running: everything that depends on its challenge comes by mail
@@ -1516,19 +1440,8 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
     block_reduce<NP>(acc, lds);
     const bool raw = a.raw_out != nullptr;  // then gridDim.x == 1
     if (gridDim.x * gridDim.y == 1 || raw) {
-        u64 *const my_out = raw ? a.raw_out + 64 * blockIdx.y : cf.out_host;
-        if (raw) {
-            if (tid == 0) {
-#pragma unroll
-                for (int t = 0; t < NP; t++) {
-                    res[2 * t] = acc[t].c0;
-                    res[2 * t + 1] = acc[t].c1;
-                }
-                publish_words(my_out, 0, res, 2 * NP, a.seq + (j - a.j));
-            }
-        } else {
-            fast_finalize<NF>(cf, acc, res);
-        }
+        u64 *const my_out = raw ? a.raw_out + 64 * blockIdx.y : ff.out_host;
+        publish_sums<NP>(my_out, cf_seq, raw ? nullptr : ff.counter, acc);
         if (a.last_round == 0) return;
         if (j >= a.last_round) {
             if (!a.finish) return;
@@ -1571,17 +1484,18 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         continue;
     }
     if (tid == 0) {
-        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x) * 2 * MAX_PTS;
+        u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x);
+        const u64 total = (u64)gridDim.x * gridDim.y;
 #pragma unroll
         for (int t = 0; t < NP; t++) {
-            st_agent(o + 2 * t, acc[t].c0);
-            st_agent(o + 2 * t + 1, acc[t].c1);
+            st_agent(o + (2 * t) * total, acc[t].c0);
+            st_agent(o + (2 * t + 1) * total, acc[t].c1);
         }
     }
     if (take_ticket(ff.counter, gridDim.x * gridDim.y, &last_flag)) {
         E2 q[NP];
         gather_partials<NP>(ff, lds, q);
-        fast_finalize<NF>(cf, q, res);
+        publish_sums<NP>(ff.out_host, cf_seq, ff.counter, q);
     }
     return;
   }
