@@ -2258,51 +2258,59 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             a.r0 = r.c0;
             a.r1 = r.c1;
             CHK(launch_folds(sc, j, true, challenge));
-            // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
-            const u32 d = sc->degree;
-            E2 acc = gl::e2_zero();
-            for (u32 k = 0; k <= d; k++) {
-                E2 num = gl::e2_one();
-                for (u32 m = 0; m <= d; m++)
-                    if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
-                acc = gl::add(acc, gl::mul(gl::mul_base(num, ctx->h_inv_den[d][k]), sc->last_msg[k]));
-            }
-            sc->claim = acc;
             if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
         }
-        // scale(t) = coeff * S * eq1(rho_{j-1}, t)
+        // scale(t) = coeff * S * eq1(rho_{j-1}, t).  Only whether scale(1) vanishes matters to the kernel (it then has to
+        // evaluate t = 1); everything else about the message is worked out while the kernel runs (prepare_message).
         E2 base_scale = sc->fast_coeff;
         if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
-        for (u32 t = 0; t <= sc->degree; t++) {
-            E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
-            hf.scale[2 * t] = sc_t.c0;
-            hf.scale[2 * t + 1] = sc_t.c1;
-        }
-        E2 s1 = gl::e2(hf.scale[2], hf.scale[3]);
+        const E2 s1 = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2_one())) : base_scale;
         const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
         a.skip1 = skip1 ? 1 : 0;
         if (has_eq) {
             const u64 off = eq_level_off(sc->n_vars, j);
             a.q0 = sc->eq_c0 + off;
             a.q1 = sc->eq_c1 + off;
-            // p(nf + 1) = sum_i cext_i q(i) + k + const
-            const E2 s_top = gl::e2(hf.scale[2 * (nf + 1)], hf.scale[2 * (nf + 1) + 1]);
-            E2 cext[dpk::MAX_PTS];
-            for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
-            if (skip1) {
-                // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
-                const E2 A = gl::mul(cext[1], h_e2_inv(s1));
-                cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(hf.scale[0], hf.scale[1])));
-                const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
-                hf.k0 = kk.c0;
-                hf.k1 = kk.c1;
-                cext[1] = gl::e2_zero();
-            }
-            for (u32 i = 0; i <= nf; i++) {
-                hf.cext[2 * i] = cext[i].c0;
-                hf.cext[2 * i + 1] = cext[i].c1;
-            }
         }
+        auto prepare_message = [&]() {
+            if (j >= 2) {
+                // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
+                const E2 r = gl::e2(challenge[0], challenge[1]);
+                const u32 d = sc->degree;
+                E2 acc = gl::e2_zero();
+                for (u32 k = 0; k <= d; k++) {
+                    E2 num = gl::e2_one();
+                    for (u32 m = 0; m <= d; m++)
+                        if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+                    acc = gl::add(acc, gl::mul(gl::mul_base(num, ctx->h_inv_den[d][k]), sc->last_msg[k]));
+                }
+                sc->claim = acc;
+            }
+            for (u32 t = 0; t <= sc->degree; t++) {
+                E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
+                hf.scale[2 * t] = sc_t.c0;
+                hf.scale[2 * t + 1] = sc_t.c1;
+            }
+            if (has_eq) {
+                // p(nf + 1) = sum_i cext_i q(i) + k + const
+                const E2 s_top = gl::e2(hf.scale[2 * (nf + 1)], hf.scale[2 * (nf + 1) + 1]);
+                E2 cext[dpk::MAX_PTS];
+                for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
+                if (skip1) {
+                    // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
+                    const E2 A = gl::mul(cext[1], h_e2_inv(s1));
+                    cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(hf.scale[0], hf.scale[1])));
+                    const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
+                    hf.k0 = kk.c0;
+                    hf.k1 = kk.c1;
+                    cext[1] = gl::e2_zero();
+                }
+                for (u32 i = 0; i <= nf; i++) {
+                    hf.cext[2 * i] = cext[i].c0;
+                    hf.cext[2 * i + 1] = cext[i].c1;
+                }
+            }
+        };
         ff.partial = sc->d_partial;
         ff.n_blocks = blocks;
         ff.out_host = fa.out_host;
@@ -2320,6 +2328,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         // forms the message: p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was skipped; with an eq factor
         // p(nf + 1) by extrapolation of q (coefficients above).
         auto take_sums = [&](bool per_group) -> int32_t {
+            prepare_message();
             const u32 np = nf + 1;
             E2 q[dpk::MAX_PTS];
             u64 w[2 * dpk::MAX_PTS];
