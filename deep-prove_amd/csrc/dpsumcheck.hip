@@ -1312,6 +1312,7 @@ struct dps_sc {
     bool poly_raw;                            // the resident launch has one workgroup per group; the host adds their sums
     bool wait_stays;                          // the launch waiting for mail stays for the rounds after the one it waits for
     bool wait_skip1;                          // ... and was compiled to take p(1) from the claim
+    bool wait_any_skip1;                      // ... or takes p(1) either way (the tail kernel)
     bool wait_fresh;                          // ... and has not been sent a mail yet (ending it loses nothing)
     bool no_ahead;                            // a launch made ahead was in another call's way once: make no more
     std::chrono::steady_clock::time_point ahead_at;  // when the launch that has had no mail yet was made
@@ -1662,7 +1663,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->tail_j0 = 0;
     sc->tail_running = false;
     sc->tail_seq0 = 0;
-    sc->wait_stays = sc->wait_skip1 = sc->wait_fresh = sc->no_ahead = false;
+    sc->wait_stays = sc->wait_skip1 = sc->wait_any_skip1 = sc->wait_fresh = sc->no_ahead = false;
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
@@ -2360,34 +2361,61 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             }
             return DPS_OK;
         };
-        if (sc->tail_j0 && j >= sc->tail_j0) {
-            post_mail();
-            if (j == sc->tail_j0) {
-                dpk::TailArgs ta;
-                memset(&ta, 0, sizeof ta);
-                for (u32 f = 0; f < nf; f++) {
-                    ta.s0[f] = a.s0[f];
-                    ta.s1[f] = a.s1[f];
-                }
-                ta.eq0 = sc->eq_c0;
-                ta.eq1 = sc->eq_c1;
-                ta.n_vars = sc->n_vars;
-                ta.j0 = j;
-                ta.mail = ctx->d_pinned + (ctx->res_off - 64);
-                ta.out_host = fa.out_host;
-                ta.seq0 = fa.seq;
-                sc->tail_seq0 = fa.seq;
-                ta.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
-                ProfScope ps(ctx, DPS_K_TAIL, 0.0);
-                if (has_eq && nf == 1) launch_tail<1, true>(ctx, ta);
-                else if (has_eq && nf == 2) launch_tail<2, true>(ctx, ta);
-                else if (!has_eq && nf == 2) launch_tail<2, false>(ctx, ta);
-                else if (!has_eq && nf == 3) launch_tail<3, false>(ctx, ta);
-                else return fail(ctx, DPS_ERR_UNSUPPORTED, "no tail kernel for %u tables, eq %d", nf, (int)has_eq);
-                HIPCHK(ctx, hipGetLastError());
-                sc->tail_running = true;
-                ctx->tail_owner = sc;
+        // A launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an earlier
+        // round, or one made ahead during the previous round.  It cannot be used when it was compiled for the other way
+        // of getting p(1) (wait_any_skip1: the tail kernel, which takes either), or when it has had no mail yet and the
+        // caller took its time: it may have given up waiting (it polls for much longer than the limit here, so up to
+        // that limit it certainly has not).  Then it is ended and the round is launched normally.
+        auto end_waiting_launch = [&]() -> int32_t {
+            __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
+            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
+            sc->tail_running = false;
+            sc->wait_fresh = false;
+            ctx->tail_owner = nullptr;
+            return DPS_OK;
+        };
+        if (sc->tail_running && !sc->wait_any_skip1 && ((a.skip1 != 0) != sc->wait_skip1)) CHK(end_waiting_launch());
+        if (sc->tail_running && sc->wait_fresh &&
+            std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS))
+            CHK(end_waiting_launch());
+        // the launch of the tail kernel, whose first round is j0 and has the sequence number seq0
+        auto launch_tail_at = [&](u32 j0, u64 seq0) -> int32_t {
+            const dpk::ProdArgs &a0 = sc->fast_args[j0];
+            dpk::TailArgs ta;
+            memset(&ta, 0, sizeof ta);
+            for (u32 f = 0; f < nf; f++) {
+                ta.s0[f] = a0.s0[f];
+                ta.s1[f] = a0.s1[f];
             }
+            ta.eq0 = sc->eq_c0;
+            ta.eq1 = sc->eq_c1;
+            ta.n_vars = sc->n_vars;
+            ta.j0 = j0;
+            ta.mail = ctx->d_pinned + (ctx->res_off - 64);
+            ta.out_host = fa.out_host;
+            ta.seq0 = seq0;
+            sc->tail_seq0 = seq0;
+            ta.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
+            ProfScope ps(ctx, DPS_K_TAIL, 0.0);
+            if (has_eq && nf == 1) launch_tail<1, true>(ctx, ta);
+            else if (has_eq && nf == 2) launch_tail<2, true>(ctx, ta);
+            else if (!has_eq && nf == 2) launch_tail<2, false>(ctx, ta);
+            else if (!has_eq && nf == 3) launch_tail<3, false>(ctx, ta);
+            else return fail(ctx, DPS_ERR_UNSUPPORTED, "no tail kernel for %u tables, eq %d", nf, (int)has_eq);
+            HIPCHK(ctx, hipGetLastError());
+            sc->tail_running = true;
+            sc->wait_any_skip1 = true;
+            ctx->tail_owner = sc;
+            return DPS_OK;
+        };
+        if (sc->tail_j0 && j >= sc->tail_j0) {
+            if (!sc->tail_running) {
+                if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
+                CHK(launch_tail_at(j, fa.seq));
+            }
+            post_mail();
+            sc->wait_fresh = false;
             CHK(take_sums(false));
             sc->round = j;
             return DPS_OK;
@@ -2491,29 +2519,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 HIPCHK(ctx, hipGetLastError());
                 return DPS_OK;
             };
-            auto end_waiting_launch = [&]() -> int32_t {
-                __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
-                HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-                __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
-                sc->tail_running = false;
-                sc->wait_fresh = false;
-                ctx->tail_owner = nullptr;
-                return DPS_OK;
-            };
             // a launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an
             // earlier round, or one made ahead during the previous round
-            bool on_gpu = sc->tail_running;
-            if (on_gpu && ((a.skip1 != 0) != sc->wait_skip1)) {
-                // it was compiled for the other way of getting p(1): end it and launch normally
-                CHK(end_waiting_launch());
-                on_gpu = false;
-            }
-            if (on_gpu && sc->wait_fresh && std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS)) {
-                // the caller took its time: the launch made ahead may have given up waiting (it polls for much longer
-                // than this, so up to here it certainly has not)
-                CHK(end_waiting_launch());
-                on_gpu = false;
-            }
+            const bool on_gpu = sc->tail_running;
             bool stays, raw_now;
             if (on_gpu) {
                 post_mail();
@@ -2573,15 +2581,65 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             sc->round = j;
             return DPS_OK;
         }
-        double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
-        for (u32 f = 0; f < nf; f++) {
-            double eb = a.s1[f] ? 16.0 : 8.0;
-            bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
-        }
-        {
+        if (sc->tail_running) {
+            // launched during the previous round
+            post_mail();
+            sc->wait_fresh = false;
+        } else {
+            double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
+            for (u32 f = 0; f < nf; f++) {
+                double eb = a.s1[f] ? 16.0 : 8.0;
+                bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
+            }
             ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
+            a.wait_first = 0;
             CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j], has_eq, j >= 2, a, blocks, sc->d_partial, ff));
             HIPCHK(ctx, hipGetLastError());
+        }
+        // this round's launch ends with the round
+        sc->tail_running = false;
+        ctx->tail_owner = nullptr;
+        // The next round's launch is made now, behind this one (see the fused multi-term path below... the same reasons):
+        // the tail kernel, or a product kernel of few workgroups, which then waits for its challenge by mail.
+        if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
+            const u64 next_seq = ctx->seq + 1;
+            bool made = false;
+            if (sc->tail_j0 && j + 1 == sc->tail_j0) {
+                CHK(launch_tail_at(j + 1, next_seq));
+                made = true;
+            } else if (blocks_for_pairs(n_pairs >> 1) <= POLY_AHEAD_MAX_WORKGROUPS) {
+                // p(1) comes from the claim unless the scale vanishes at 1
+                bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
+                if (has_eq) {
+                    const E2 rho = sc->eq_info->point[j];
+                    skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
+                }
+                dpk::ProdArgs an = sc->fast_args[j + 1];
+                if (has_eq) {
+                    const u64 off = eq_level_off(sc->n_vars, j + 1);
+                    an.q0 = sc->eq_c0 + off;
+                    an.q1 = sc->eq_c1 + off;
+                }
+                an.r0 = an.r1 = 0;
+                an.skip1 = skip1_next ? 1 : 0;
+                an.wait_first = 1;
+                an.spin_limit = 4000000;
+                an.mail = ctx->d_pinned + (ctx->res_off - 64);
+                dpk::FastFin fn = ff;
+                fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
+                fn.seq = next_seq;
+                CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j + 1], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
+                HIPCHK(ctx, hipGetLastError());
+                sc->wait_any_skip1 = false;
+                sc->wait_skip1 = skip1_next;
+                made = true;
+            }
+            if (made) {
+                sc->tail_running = true;
+                sc->wait_fresh = true;
+                sc->ahead_at = std::chrono::steady_clock::now();
+                ctx->tail_owner = sc;
+            }
         }
         CHK(take_sums(false));
         sc->round = j;

@@ -313,6 +313,12 @@ __device__ __forceinline__ void st_agent(u64 *p, u64 v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// a value that is the same in every lane, moved to scalar registers
+__device__ __forceinline__ u64 uniform64(u64 v)
+{
+    const u32 lo = __builtin_amdgcn_readfirstlane((u32)v), hi = __builtin_amdgcn_readfirstlane((u32)(v >> 32));
+    return ((u64)hi << 32) | lo;
+}
 // host-visible (fine-grained pinned) memory
 __device__ __forceinline__ u64 ld_sys(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
 __device__ __forceinline__ void st_sys(u64 *p, u64 v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); }
@@ -517,6 +523,49 @@ eval_terms_kernel(const TermDesc *__restrict__ terms, u64 *__restrict__ partial,
 }
 
 // ---------------------------------------------------------------------------
+// mailbox: how a kernel that is already on the GPU is handed a challenge.  The host writes the words to fine-grained
+// pinned memory, the kernel polls them with system-scope loads.  Used by the resident kernels for every round after
+// their first, and by launches made ahead of their round for the first one as well.
+// ---------------------------------------------------------------------------
+// mailbox words; MAIL_SEQ == MAIL_ABORT_SEQ tells the kernel to exit
+constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_WORDS = 5;
+static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
+constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
+
+// check word of a mailbox: seq ^ xor over the payload words of rotl(word_i, i)
+__host__ __device__ __forceinline__ u64 mail_mix(u64 w, u32 i) { return (i >= (u32)MAIL_R && i < (u32)MAIL_WORDS) ? rotl64(w, i) : 0; }
+
+// Waits for mail number `want` and copies it to `box` (LDS).  The first wavefront
+// polls: every lane loads one mailbox word, so one load instruction (one trip over
+// the host link) fetches the whole mail; it is accepted when the sequence number
+// matches and the check word agrees with the payload, which makes a torn read
+// (the host still writing) look like no mail yet.  Returns false on abort or timeout.
+__device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, u64 want, u64 *box, int *ok_lds)
+{
+    if (threadIdx.x < WAVE) {
+        const u32 l = threadIdx.x;
+        int ok = 0;
+        for (u32 spins = 0; spins < spin_limit; spins++) {
+            const u64 w = l < (u32)MAIL_WORDS ? ld_sys(mail + l) : 0;
+            u64 x = mail_mix(w, l);
+#pragma unroll
+            for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
+            const u64 seq = __shfl(w, MAIL_SEQ, WAVE), chk = __shfl(w, MAIL_CHK, WAVE);
+            if (seq == MAIL_ABORT_SEQ) break;
+            if (seq == want && chk == (x ^ seq)) {
+                if (l < (u32)MAIL_WORDS) box[l] = w;
+                ok = 1;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        if (l == 0) *ok_lds = ok;
+    }
+    __syncthreads();
+    return *ok_lds != 0;
+}
+
+// ---------------------------------------------------------------------------
 // fused product kernels: one term, NF full-size tables (the first NB of them
 // base-field in the source), optionally times an eq(rho, x) factor.
 //
@@ -546,6 +595,11 @@ struct ProdArgs {
     u64 n_pairs;  // pairs evaluated this round
     u64 r0, r1;   // fold challenge
     u32 skip1;    // 1: t = 1 is not evaluated (the launch picks the kernel variant accordingly)
+    // A launch made before its round began (wait_first): the challenge is not in r0, r1; the kernel waits for the mail
+    // with the launch's sequence number and takes it from there.
+    u32 wait_first;
+    u32 spin_limit;
+    const u64 *mail;
 };
 
 // The kernels hand the host the sums q(t), t = 0..NF (q(1) left at zero when t = 1 was skipped), not the round
@@ -616,7 +670,16 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ int last_flag;
-    const E2 r = gl::e2(a.r0, a.r1);
+    E2 r = gl::e2(a.r0, a.r1);
+    if (a.wait_first) {
+        __shared__ u64 box[MAIL_WORDS];
+        __shared__ int ok_flag;
+        if (!tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag)) return;
+        // the other way of getting p(1) is not compiled into this variant: the host ends the launch instead
+        if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
+        // (kept in scalar registers, as the kernel argument would be)
+        r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
+    }
     const gl::E2P rp = gl::prep(r);
     // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
     constexpr bool skip1 = SKIP1;
@@ -796,14 +859,6 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 // gives up after `spin_limit` polls and exits.
 // ---------------------------------------------------------------------------
 constexpr int TAIL_PAIRS = 256;
-// mailbox words; MAIL_SEQ == MAIL_ABORT_SEQ tells the kernel to exit
-constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_WORDS = 5;
-static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
-constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
-
-// check word of a mailbox: seq ^ xor over the payload words of rotl(word_i, i)
-__host__ __device__ __forceinline__ u64 mail_mix(u64 w, u32 i) { return (i >= (u32)MAIL_R && i < (u32)MAIL_WORDS) ? rotl64(w, i) : 0; }
-
 struct TailArgs {
     const u64 *s0[3];
     const u64 *s1[3];  // extension tables of the first tail round, 4 * n_pairs0 entries each
@@ -815,36 +870,6 @@ struct TailArgs {
     u64 seq0;          // sequence number of round j0; round j uses seq0 + (j - j0), the final evaluations seq0 + (n_vars - j0 + 1)
     u32 spin_limit;
 };
-
-// Waits for mail number `want` and copies it to `box` (LDS).  The first wavefront
-// polls: every lane loads one mailbox word, so one load instruction (one trip over
-// the host link) fetches the whole mail; it is accepted when the sequence number
-// matches and the check word agrees with the payload, which makes a torn read
-// (the host still writing) look like no mail yet.  Returns false on abort or timeout.
-__device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, u64 want, u64 *box, int *ok_lds)
-{
-    if (threadIdx.x < WAVE) {
-        const u32 l = threadIdx.x;
-        int ok = 0;
-        for (u32 spins = 0; spins < spin_limit; spins++) {
-            const u64 w = l < (u32)MAIL_WORDS ? ld_sys(mail + l) : 0;
-            u64 x = mail_mix(w, l);
-#pragma unroll
-            for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
-            const u64 seq = __shfl(w, MAIL_SEQ, WAVE), chk = __shfl(w, MAIL_CHK, WAVE);
-            if (seq == MAIL_ABORT_SEQ) break;
-            if (seq == want && chk == (x ^ seq)) {
-                if (l < (u32)MAIL_WORDS) box[l] = w;
-                ok = 1;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-        }
-        if (l == 0) *ok_lds = ok;
-    }
-    __syncthreads();
-    return *ok_lds != 0;
-}
 
 template <int NF, bool EQ>
 __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)

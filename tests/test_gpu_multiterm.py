@@ -180,3 +180,35 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
             assert (s.finish(chal) == ref_finals).all()
             del s
     _check(dp, ctx, orc, n, gpu, host, terms)
+
+
+@pytest.mark.parametrize("with_eq", [True, False])
+def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq):
+    """The same for a single product of full-size tables: its small rounds and the resident kernel of its last
+    rounds (first round 6 of 14 here) are launched during the round before."""
+    import time
+    n = 14
+    f, g = rand_base(1 << n, 31), rand_e2(1 << n, 32)
+    gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
+    if with_eq:
+        pt = rand_e2(n, 33)
+        gpu.append(ctx.eq_build(pt))
+        host.append(orc.eq_evals(pt))
+        fs = [2, 0, 1]
+    terms = [(np.array([3, 5], dtype=np.uint64), fs)]
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
+    for after in (1, 2, 4, 5):
+        for how in ("other call", "slow caller"):
+            s = ctx.session(n, gpu, terms)
+            chal = None
+            for j in range(n):
+                assert (s.round(chal) == ref_proof[j]).all(), (after, how, j)
+                chal = ref_point[j]
+                if j + 1 == after:
+                    if how == "other call":
+                        assert (ctx.eq_build(ref_point[:3]).download() == orc.eq_evals(ref_point[:3])).all()
+                    else:
+                        time.sleep(0.05)
+            assert (s.finish(chal) == ref_finals).all()
+            del s
+    _check(dp, ctx, orc, n, gpu, host, terms)
