@@ -1314,6 +1314,7 @@ struct dps_sc {
     bool wait_skip1;                          // ... and was compiled to take p(1) from the claim
     bool wait_any_skip1;                      // ... or takes p(1) either way (the tail kernel)
     bool wait_fresh;                          // ... and has not been sent a mail yet (ending it loses nothing)
+    u32 wait_slots;                           // ... and publishes to this many result areas of its own (0: the main one)
     bool no_ahead;                            // a launch made ahead was in another call's way once: make no more
     std::chrono::steady_clock::time_point ahead_at;  // when the launch that has had no mail yet was made
     bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
@@ -1423,6 +1424,10 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
 // Several groups resident side by side publish into 64-word slots of the pinned buffer from here on
 constexpr u32 POLY_RAW_MAX_GROUPS = 32;
 size_t poly_raw_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64; }
+// a launch of this many workgroups publishes per workgroup (FastFin::slots) rather than through the last one
+constexpr u32 SLOT_MAX_WORKGROUPS = 16;
+static_assert(SLOT_MAX_WORKGROUPS <= POLY_RAW_MAX_GROUPS, "the per-workgroup result areas are those of the resident groups");
+u32 slots_for(u32 workgroups) { return workgroups > 1 && workgroups <= SLOT_MAX_WORKGROUPS ? workgroups : 0; }
 
 // A round's launch is made ahead of time only with at most this many workgroups: each of them polls the mailbox
 constexpr u32 POLY_AHEAD_MAX_WORKGROUPS = 64;
@@ -1664,6 +1669,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->tail_running = false;
     sc->tail_seq0 = 0;
     sc->wait_stays = sc->wait_skip1 = sc->wait_any_skip1 = sc->wait_fresh = sc->no_ahead = false;
+    sc->wait_slots = 0;
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
@@ -2325,18 +2331,18 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             mb[dpk::MAIL_SKIP1] = a.skip1;
             send_mail(ctx, fa.seq);
         };
-        // Waits for the sums q(t), t = 0..nf, of this round (one set, or one per resident group, which are added) and
+        // Waits for the sums q(t), t = 0..nf, of this round (one set in the main result area, or n_slots sets in areas
+        // of their own -- resident groups, or the workgroups of a small launch -- which are added) and
         // forms the message: p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was skipped; with an eq factor
         // p(nf + 1) by extrapolation of q (coefficients above).
-        auto take_sums = [&](bool per_group) -> int32_t {
+        auto take_sums = [&](u32 n_slots) -> int32_t {
             prepare_message();
             const u32 np = nf + 1;
             E2 q[dpk::MAX_PTS];
             u64 w[2 * dpk::MAX_PTS];
-            if (per_group) {
-                const u32 n_groups = (u32)sc->poly_tabs.size();
+            if (n_slots) {
                 for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
-                for (u32 g = 0; g < n_groups; g++) {
+                for (u32 g = 0; g < n_slots; g++) {
                     CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
                     for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
                 }
@@ -2406,6 +2412,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             HIPCHK(ctx, hipGetLastError());
             sc->tail_running = true;
             sc->wait_any_skip1 = true;
+            sc->wait_slots = 0;
             ctx->tail_owner = sc;
             return DPS_OK;
         };
@@ -2416,7 +2423,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             }
             post_mail();
             sc->wait_fresh = false;
-            CHK(take_sums(false));
+            CHK(take_sums(0));
             sc->round = j;
             return DPS_OK;
         }
@@ -2508,6 +2515,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 dpk::FastFin fl = ff;
                 fl.seq = seq_jj;
                 fl.n_blocks = p.blocks * n_groups;
+                fl.slots = !p.reside && slots_for(fl.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
                 double pbytes = has_eq ? (double)p.n_pairs * 16.0 : 0.0;
                 for (u32 k = 0; k < sc->n_mles; k++)
                     if (sc->poly_owner[k] >= 0) pbytes += (double)p.n_pairs * (jj >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
@@ -2522,22 +2530,26 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             // a launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an
             // earlier round, or one made ahead during the previous round
             const bool on_gpu = sc->tail_running;
-            bool stays, raw_now;
+            // result areas the launch of this round publishes to, 0 = the main one
+            auto slots_of = [&](const Plan &p) { return p.reside ? (n_groups > 1 ? n_groups : 0) : slots_for(p.blocks * n_groups); };
+            bool stays;
+            u32 slots_now;
             if (on_gpu) {
                 post_mail();
                 sc->wait_fresh = false;
                 stays = sc->wait_stays;
-                raw_now = sc->poly_raw;
+                slots_now = sc->wait_slots;
             } else {
                 const Plan p = plan_round(j, a.skip1 != 0);
                 CHK(launch_round(j, p, a.skip1 != 0, false, fa.seq));
                 stays = p.reside;
-                raw_now = p.reside && n_groups > 1;
+                slots_now = slots_of(p);
                 if (p.reside) {
                     sc->tail_running = true;
                     sc->tail_seq0 = fa.seq;
                     ctx->tail_owner = sc;
-                    sc->poly_raw = raw_now;
+                    sc->poly_raw = n_groups > 1;
+                    sc->wait_slots = slots_now;
                     sc->wait_stays = true;
                     sc->wait_skip1 = true;
                     sc->wait_fresh = false;
@@ -2568,10 +2580,11 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                         sc->wait_fresh = true;
                         sc->ahead_at = std::chrono::steady_clock::now();
                         sc->poly_raw = pn.reside && n_groups > 1;
+                        sc->wait_slots = slots_of(pn);
                     }
                 }
             }
-            int32_t rc = take_sums(raw_now);
+            int32_t rc = take_sums(slots_now);
             if (stays && (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel))) {
                 // (without a finishing step of its own a resident launch exits after the last round)
                 sc->tail_running = false;
@@ -2581,11 +2594,14 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             sc->round = j;
             return DPS_OK;
         }
+        u32 slots_now = sc->wait_slots;
         if (sc->tail_running) {
             // launched during the previous round
             post_mail();
             sc->wait_fresh = false;
         } else {
+            slots_now = slots_for(blocks);
+            ff.slots = slots_now ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
             double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
             for (u32 f = 0; f < nf; f++) {
                 double eb = a.s1[f] ? 16.0 : 8.0;
@@ -2628,6 +2644,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 dpk::FastFin fn = ff;
                 fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
                 fn.seq = next_seq;
+                fn.slots = slots_for(fn.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
+                sc->wait_slots = slots_for(fn.n_blocks);
                 CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j + 1], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
                 HIPCHK(ctx, hipGetLastError());
                 sc->wait_any_skip1 = false;
@@ -2641,7 +2659,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 ctx->tail_owner = sc;
             }
         }
-        CHK(take_sums(false));
+        CHK(take_sums(slots_now));
         sc->round = j;
         return DPS_OK;
     } else {

@@ -613,6 +613,10 @@ struct FastFin {
     u64 *out_host;
     u64 seq;
     u32 *counter;
+    // Few workgroups: each publishes its own sums to a 64-word area of its own (slots + 64 * workgroup, laid out like
+    // out_host) and the host adds them; this spares the round the ticket and the gathering, two trips through device
+    // memory one after the other.  nullptr: the last workgroup gathers and publishes to out_host.
+    u64 *slots;
 };
 
 // sums of the workgroups' partials, valid in thread 0
@@ -671,16 +675,20 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ int last_flag;
     E2 r = gl::e2(a.r0, a.r1);
-    if (a.wait_first) {
+    gl::E2P rp = gl::prep(r);
+    // A launch made ahead of its round waits here for its challenge, with the operands of its first step already
+    // requested (they do not depend on the challenge).  False: no mail came, or the mail asks for the other way of
+    // getting p(1), which is not compiled into this variant; the host then ends the launch.
+    auto take_challenge = [&]() -> bool {
         __shared__ u64 box[MAIL_WORDS];
         __shared__ int ok_flag;
-        if (!tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag)) return;
-        // the other way of getting p(1) is not compiled into this variant: the host ends the launch instead
-        if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
+        if (!tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag)) return false;
+        if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
         // (kept in scalar registers, as the kernel argument would be)
         r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
-    }
-    const gl::E2P rp = gl::prep(r);
+        rp = gl::prep(r);
+        return true;
+    };
     // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
     constexpr bool skip1 = SKIP1;
     // running sums, reduced once after the loop
@@ -804,6 +812,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     if (FOLD) {
         Raw w;
         if (i < a.n_pairs) load_raw(i, w);
+        if (a.wait_first && !take_challenge()) return;
         for (; i < a.n_pairs; i += stride) {
             step(i, w);
             if (i + stride < a.n_pairs) load_raw(i + stride, w);
@@ -829,6 +838,10 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     if (gridDim.x == 1) {
         // a single workgroup: its sums are the round's sums, no partials and no ticket
         publish_sums<NP>(ff.out_host, ff.seq, ff.counter, acc);
+        return;
+    }
+    if (ff.slots) {
+        publish_sums<NP>(ff.slots + 64 * (u64)blockIdx.x, ff.seq, nullptr, acc);
         return;
     }
     if (threadIdx.x == 0) {
@@ -1250,6 +1263,10 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         publish_sums<NP>(ff.out_host, ff.seq, ff.counter, acc);
         return;
     }
+    if (ff.slots) {
+        publish_sums<NP>(ff.slots + 64 * ((u64)blockIdx.y * gridDim.x + blockIdx.x), ff.seq, nullptr, acc);
+        return;
+    }
     if (tid == 0) {
         u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x);
         const u64 total = (u64)gridDim.x * gridDim.y;
@@ -1507,6 +1524,10 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         }
         continue;
+    }
+    if (ff.slots) {
+        publish_sums<NP>(ff.slots + 64 * ((u64)blockIdx.y * gridDim.x + blockIdx.x), cf_seq, nullptr, acc);
+        return;
     }
     if (tid == 0) {
         u64 *o = partial + ((u64)blockIdx.y * gridDim.x + blockIdx.x);
