@@ -1315,6 +1315,7 @@ struct dps_sc {
     bool wait_any_skip1;                      // ... or takes p(1) either way (the tail kernel)
     bool wait_fresh;                          // ... and has not been sent a mail yet (ending it loses nothing)
     u32 wait_slots;                           // ... and publishes to this many result areas of its own (0: the main one)
+    u64 pairs_seq;                            // nonzero: the last round's launch also published the tables' last pairs, under this number
     bool no_ahead;                            // a launch made ahead was in another call's way once: make no more
     std::chrono::steady_clock::time_point ahead_at;  // when the launch that has had no mail yet was made
     bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
@@ -1670,6 +1671,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->tail_seq0 = 0;
     sc->wait_stays = sc->wait_skip1 = sc->wait_any_skip1 = sc->wait_fresh = sc->no_ahead = false;
     sc->wait_slots = 0;
+    sc->pairs_seq = 0;
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
@@ -2177,14 +2179,15 @@ namespace {
 // word; the words are accepted once the check word agrees with them, since the
 // kernel's stores may land in any order.  If the result does not arrive the
 // stream is queried to surface the error.
-int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out);
+int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out, int seq_slot = dpk::HOST_SEQ_SLOT,
+                       int chk_slot = dpk::HOST_CHK_SLOT);
 int32_t wait_result(dps_ctx *ctx, u64 seq, u32 slot0, u32 n, u64 *out) { return wait_result_at(ctx, ctx->res_off, seq, slot0, n, out); }
 
 // the same hand-off in another 64-word area of the pinned buffer
-int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out)
+int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out, int seq_slot, int chk_slot)
 {
     volatile u64 *base = ctx->h_pinned + base_off;
-    volatile u64 *flag = base + dpk::HOST_SEQ_SLOT;
+    volatile u64 *flag = base + seq_slot;
     auto take = [&]() {
         if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) return false;
         u64 chk = seq;
@@ -2192,7 +2195,7 @@ int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n,
             out[i] = base[slot0 + i];
             chk ^= dpk::rotl64(out[i], i + 1);
         }
-        return chk == base[dpk::HOST_CHK_SLOT];
+        return chk == base[chk_slot];
     };
     for (u64 spins = 0;; spins++) {
         if (take()) return DPS_OK;
@@ -2423,7 +2426,14 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             }
             post_mail();
             sc->wait_fresh = false;
-            CHK(take_sums(0));
+            const int32_t rc = take_sums(0);
+            if (j == sc->n_vars || rc != DPS_OK) {
+                // with its last round the kernel publishes the tables' last pairs and exits
+                sc->tail_running = false;
+                ctx->tail_owner = nullptr;
+                if (rc == DPS_OK) sc->pairs_seq = fa.seq;
+            }
+            CHK(rc);
             sc->round = j;
             return DPS_OK;
         }
@@ -2585,10 +2595,11 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 }
             }
             int32_t rc = take_sums(slots_now);
-            if (stays && (rc != DPS_OK || (j == sc->n_vars && !sc->poly_finish_in_kernel))) {
-                // (without a finishing step of its own a resident launch exits after the last round)
+            if (stays && (rc != DPS_OK || j == sc->n_vars)) {
+                // a resident launch exits after the last round; one that can finish has published the tables' last pairs with it
                 sc->tail_running = false;
                 ctx->tail_owner = nullptr;
+                if (rc == DPS_OK && sc->poly_finish_in_kernel) sc->pairs_seq = fa.seq;
             }
             CHK(rc);
             sc->round = j;
@@ -2687,36 +2698,29 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
     if (sc->broken) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: the session was interrupted by another call on its context");
     DeviceGuard g(ctx->device);
     if (ctx->tail_owner != sc) tail_abort(ctx);
-    if (sc->tail_running) {
-        // the resident kernel folds with the last challenge and publishes the final evaluations
-        u64 *mb = mailbox(ctx);
-        const u64 seq = ++ctx->seq;
-        mb[dpk::MAIL_R] = challenge[0];
-        mb[dpk::MAIL_R + 1] = challenge[1];
-        send_mail(ctx, seq);
-        u64 fin[2 * dpk::POLY_MAXT];
+    if (sc->pairs_seq) {
+        // the resident launch published value and slope of every table's last pair with its last round: the final
+        // evaluations are value + r * slope
+        const E2 r = gl::e2(challenge[0], challenge[1]);
+        u64 w[4 * dpk::POLY_MAXT];
         // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
         // groups are resident), the single-product one its factors
-        int32_t rc = DPS_OK;
         const u32 n_areas = sc->poly ? (u32)sc->poly_tabs.size() : 1;
-        for (u32 g = 0; g < n_areas && rc == DPS_OK; g++) {
+        for (u32 g = 0; g < n_areas; g++) {
             const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[g].size() : sc->fast_nf;
-            rc = sc->poly_raw ? wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin)
-                              : wait_result(ctx, seq, dpk::HOST_FINALS_SLOT, 2 * n_fin, fin);
-            for (u32 f = 0; f < n_fin && rc == DPS_OK; f++) {
+            const size_t base = sc->poly_raw ? poly_raw_off(ctx) + 64 * (size_t)g : ctx->res_off;
+            CHK(wait_result_at(ctx, base, sc->pairs_seq, dpk::HOST_FINALS_SLOT, 4 * n_fin, w, dpk::HOST_PAIRS_SEQ_SLOT, dpk::HOST_PAIRS_CHK_SLOT));
+            for (u32 f = 0; f < n_fin; f++) {
                 const u32 k = sc->poly ? sc->poly_tabs[g][f] : sc->fast_order[f];
                 // a table shared by several groups is folded by each; the owner's copy counts
                 if (sc->poly && sc->poly_owner[k] != (int)g) continue;
-                final_evals_out[2 * k] = fin[2 * f];
-                final_evals_out[2 * k + 1] = fin[2 * f + 1];
+                const E2 v = gl::add(gl::e2(w[4 * f], w[4 * f + 1]), gl::mul(r, gl::e2(w[4 * f + 2], w[4 * f + 3])));
+                final_evals_out[2 * k] = v.c0;
+                final_evals_out[2 * k + 1] = v.c1;
             }
         }
-        // the kernel exits right after publishing and reads nothing more; whatever is launched next follows it on the stream
-        sc->tail_running = false;
-        ctx->tail_owner = nullptr;
-        if (rc != DPS_OK) return rc;
         if (sc->fast_eq >= 0) {
-            E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], gl::e2(challenge[0], challenge[1])));
+            E2 v = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[sc->n_vars - 1], r));
             final_evals_out[2 * sc->fast_eq] = v.c0;
             final_evals_out[2 * sc->fast_eq + 1] = v.c1;
         }

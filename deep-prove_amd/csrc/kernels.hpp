@@ -299,6 +299,11 @@ struct FinArgs {
 constexpr int HOST_SEQ_SLOT = 2 * MAX_PTS;
 constexpr int HOST_CHK_SLOT = HOST_SEQ_SLOT + 1;
 constexpr int HOST_FINALS_SLOT = HOST_SEQ_SLOT + 8;
+// A second hand-off in the same 64-word area, with a sequence and a check word of its own: with its last round a
+// resident kernel also publishes value and slope of the last pair of every table (4 words per table from
+// HOST_FINALS_SLOT on); the final evaluations are then value + r * slope, which the host works out when the last
+// challenge is drawn -- no further trip to the GPU.
+constexpr int HOST_PAIRS_SEQ_SLOT = 62, HOST_PAIRS_CHK_SLOT = 63;
 
 // Block partials cross XCDs (each XCD has its own L2).  They are written and read
 // with agent-scope accesses, which go through to the coherence point, so that no
@@ -333,7 +338,8 @@ __host__ __device__ __forceinline__ u64 rotl64(u64 x, u32 k)
 // word and the sequence number the host polls.  Nothing waits for a store to be
 // acknowledged, and the order in which the stores land does not matter: the
 // host accepts the words only when  check == seq ^ xor_i rotl(word_i, i + 1).
-__device__ __forceinline__ void publish_words(u64 *out_host, u32 slot0, const u64 *words, u32 n, u64 seq)
+__device__ __forceinline__ void publish_words(u64 *out_host, u32 slot0, const u64 *words, u32 n, u64 seq, int seq_slot = HOST_SEQ_SLOT,
+                                              int chk_slot = HOST_CHK_SLOT)
 {
     u64 chk = seq;
     for (u32 i = 0; i < n; i++) {
@@ -341,8 +347,8 @@ __device__ __forceinline__ void publish_words(u64 *out_host, u32 slot0, const u6
         chk ^= rotl64(w, i + 1);
         st_sys(out_host + slot0 + i, w);
     }
-    st_sys(out_host + HOST_CHK_SLOT, chk);
-    st_sys(out_host + HOST_SEQ_SLOT, seq);
+    st_sys(out_host + chk_slot, chk);
+    st_sys(out_host + seq_slot, seq);
 }
 
 // Called by every thread of one workgroup once all partials are visible.
@@ -968,21 +974,21 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
         to_ping = !to_ping;
         n_pairs >>= 1;
     }
-    // final evaluations: the last challenge folds the two remaining entries of every table
-    const u64 fin_seq = a.seq0 + (a.n_vars - a.j0 + 1);
-    if (!tail_wait_mail(a.mail, a.spin_limit, fin_seq, box, &ok_flag)) return;
+    // with the last round: value and slope of the remaining pair of every table (the host folds them with the last challenge)
     if (threadIdx.x < NF) {
         const int f = threadIdx.x;
-        const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
         // the last round wrote its pair to the buffer `to_ping` now points away from
         const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
         const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
-        E2 v = fold1(gl::e2(c0[0], c1[0]), gl::e2(c0[1], c1[1]), r);
-        res[2 * f] = v.c0;
-        res[2 * f + 1] = v.c1;
+        const E2 lo = gl::e2(c0[0], c1[0]), d = gl::sub(gl::e2(c0[1], c1[1]), lo);
+        res[4 * f] = lo.c0;
+        res[4 * f + 1] = lo.c1;
+        res[4 * f + 2] = d.c0;
+        res[4 * f + 3] = d.c1;
     }
     __syncthreads();
-    if (threadIdx.x == 0) publish_words(a.out_host, HOST_FINALS_SLOT, res, 2 * NF, fin_seq);
+    if (threadIdx.x == 0)
+        publish_words(a.out_host, HOST_FINALS_SLOT, res, 4 * NF, a.seq0 + (a.n_vars - a.j0), HOST_PAIRS_SEQ_SLOT, HOST_PAIRS_CHK_SLOT);
 }
 
 // ---------------------------------------------------------------------------
@@ -1045,6 +1051,7 @@ struct PolyOp {
 };
 constexpr int POLY_LDS_OPS = POLY_LDS_TERMS * 40 / 32;  // a program shares the terms' place in LDS and in the kernel arguments
 static_assert(sizeof(PolyTerm) == 40 && sizeof(PolyOp) == 32, "terms and operations share storage");
+static_assert(HOST_FINALS_SLOT + 4 * POLY_MAXT <= HOST_PAIRS_SEQ_SLOT && 4 * POLY_MAXT <= 6 * MAX_PTS, "last pairs of a group fit its result area");
 static_assert(sizeof(PolyTerm) % 8 == 0 && sizeof(PolyGroup) % 8 == 0, "descriptors are copied as 64-bit words");
 
 struct PolyArgs {
@@ -1487,20 +1494,14 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         if (a.last_round == 0) return;
         if (j >= a.last_round) {
             if (!a.finish) return;
-            // after the last round: the last challenge arrives, every table's remaining pair (value and slope are
-            // still in LDS, pair 0) is folded with it, and the final evaluations go to the host in slot order
-            const u64 fin_seq = a.seq + (j - a.j) + 1;
-            if (!tail_wait_mail(a.mail, a.spin_limit, fin_seq, box, &ok_flag)) return;
+            // with the last round: value and slope of every table's remaining pair (still in LDS, pair 0), in slot order;
+            // the host folds them with the last challenge
             if (tid < n_tabs) {
-                const gl::E2P rl = gl::prep(gl::e2(box[MAIL_R], box[MAIL_R + 1]));
-                const E2 lo = gl::e2(dyn[(tid * 4 + 0) * BLOCK], dyn[(tid * 4 + 1) * BLOCK]);
-                const E2 d = gl::e2(dyn[(tid * 4 + 2) * BLOCK], dyn[(tid * 4 + 3) * BLOCK]);
-                const E2 v = gl::fma(d, rl, lo);
-                res[2 * tid] = v.c0;
-                res[2 * tid + 1] = v.c1;
+#pragma unroll
+                for (int k = 0; k < 4; k++) res[4 * tid + k] = dyn[(tid * 4 + k) * BLOCK];
             }
             __syncthreads();
-            if (tid == 0) publish_words(my_out, HOST_FINALS_SLOT, res, 2 * n_tabs, fin_seq);
+            if (tid == 0) publish_words(my_out, HOST_FINALS_SLOT, res, 4 * n_tabs, cf_seq, HOST_PAIRS_SEQ_SLOT, HOST_PAIRS_CHK_SLOT);
             return;
         }
         // stay for the next round: its challenge and the scalars of its message arrive by mail
