@@ -271,6 +271,7 @@ struct Storage {
 // level j in round j instead of folding the full table.
 struct EqInfo {
     u32 m;
+    u32 fact_levels = 0;  // levels 1..fact_levels have a low table behind the levels (eq_low_off)
     std::vector<E2> point;
 };
 
@@ -716,6 +717,12 @@ bool canonical(const u64 *v, size_t n)
 }
 
 u64 eq_level_off(u32 m, u32 l) { return (2ull << m) - (2ull << (m - l)); }
+// Behind the levels: for every level l = 1..m-16 (those of at least 2^16 entries) the table eq(rho_{l..l+15}, .) of its 16 lowest
+// variables.  Level l is then the product  level_{l+16}[i >> 16] * low_l[i & 65535], which the product kernels use in their
+// large rounds instead of streaming level l.
+u32 eq_fact_levels(u32 m) { return m > dpk::EQ_LO_BITS ? m - dpk::EQ_LO_BITS : 0; }
+u64 eq_low_off(u32 m, u32 l) { return (2ull << m) + ((u64)(l - 1) << dpk::EQ_LO_BITS); }
+u64 eq_storage_entries(u32 m) { return (2ull << m) + ((u64)eq_fact_levels(m) << dpk::EQ_LO_BITS); }
 
 // Builds eq(rho, .) and every level eq(rho_{l..m-1}, .), l = 1..m, into o0/o1
 // (2^(m+1) entries).  Levels of at most 2^16 entries come straight from the
@@ -733,6 +740,11 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
     for (u32 l = first_small; l <= m; l++) {
         js.job[n_jobs++] = dpk::EqJob{l, m - l, eq_level_off(m, l)};
         max_bits = std::max(max_bits, m - l);
+    }
+    // the low tables of the large levels (the caller allocated eq_storage_entries(m))
+    for (u32 l = 1; l <= eq_fact_levels(m); l++) {
+        js.job[n_jobs++] = dpk::EqJob{l, dpk::EQ_LO_BITS, eq_low_off(m, l)};
+        max_bits = std::max(max_bits, dpk::EQ_LO_BITS);
     }
     // seeds live in a scratch block behind nothing: a separate allocation
     void *seed_block = nullptr;
@@ -793,7 +805,7 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
     dps_mle *t = nullptr;
-    CHK(new_table(ctx, DPS_EXT2, 2ull << m, &t));
+    CHK(new_table(ctx, DPS_EXT2, eq_storage_entries(m), &t));
     t->len = 1ull << m;
     int32_t rc = eq_build_dev(ctx, point, m, t->st->c0, t->st->c1);
     if (rc != DPS_OK) {
@@ -802,6 +814,7 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     }
     t->eq = std::make_shared<EqInfo>();
     t->eq->m = m;
+    t->eq->fact_levels = eq_fact_levels(m);
     for (u32 i = 0; i < m; i++) t->eq->point.push_back(gl::e2(point[2 * i], point[2 * i + 1]));
     *out = t;
     return DPS_OK;
@@ -852,12 +865,13 @@ extern "C" int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points
     };
     for (u32 i = 0; i < count; i++) {
         dps_mle *t = nullptr;
-        int32_t rc = new_table(ctx, DPS_EXT2, 2ull << m[i], &t);
+        int32_t rc = new_table(ctx, DPS_EXT2, eq_storage_entries(m[i]), &t);
         if (rc != DPS_OK) return undo(rc);
         out[i] = t;
         t->len = 1ull << m[i];
         t->eq = std::make_shared<EqInfo>();
         t->eq->m = m[i];
+        t->eq->fact_levels = eq_fact_levels(m[i]);  // (only tables of more than 16 variables have any: built by eq_build_dev)
         for (u32 k = 0; k < m[i]; k++) t->eq->point.push_back(gl::e2(points[i][2 * k], points[i][2 * k + 1]));
         if (m[i] > 16) {
             // large tables are built by expansion, one at a time
@@ -1368,6 +1382,18 @@ void launch_tail(dps_ctx *ctx, const dpk::TailArgs &a)
 template <int NF, int NB, bool EQ>
 void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial, const dpk::FastFin &ff)
 {
+    if constexpr (EQ) {
+        if (a.lq0) {
+            // large round: eq weights as a product of a small low table and a later level
+            if (fold && a.skip1)
+                dpk::prod_kernel<NF, NB, true, true, true, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+            else if (fold)
+                dpk::prod_kernel<NF, NB, true, true, false, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+            else
+                dpk::prod_kernel<NF, NB, false, true, false, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+            return;
+        }
+    }
     if (fold && a.skip1)
         dpk::prod_kernel<NF, NB, true, EQ, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
     else if (fold)
@@ -2281,6 +2307,14 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u64 off = eq_level_off(sc->n_vars, j);
             a.q0 = sc->eq_c0 + off;
             a.q1 = sc->eq_c1 + off;
+            // (the factored form needs a grid whose stride is a multiple of the low table's size)
+            if (sc->fast && j <= sc->eq_info->fact_levels && ((u64)blocks * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
+                const u64 lo = eq_low_off(sc->n_vars, j), hi = eq_level_off(sc->n_vars, j + dpk::EQ_LO_BITS);
+                a.lq0 = sc->eq_c0 + lo;
+                a.lq1 = sc->eq_c1 + lo;
+                a.hq0 = sc->eq_c0 + hi;
+                a.hq1 = sc->eq_c1 + hi;
+            }
         }
         auto prepare_message = [&]() {
             if (j >= 2) {
@@ -2613,7 +2647,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         } else {
             slots_now = slots_for(blocks);
             ff.slots = slots_now ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
-            double bytes = has_eq ? (double)n_pairs * 16.0 : 0.0;
+            // (in the factored form the eq weights are one entry per thread and one per workgroup and step: not counted)
+            double bytes = has_eq && !a.lq0 ? (double)n_pairs * 16.0 : 0.0;
             for (u32 f = 0; f < nf; f++) {
                 double eb = a.s1[f] ? 16.0 : 8.0;
                 bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;

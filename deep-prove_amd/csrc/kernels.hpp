@@ -606,7 +606,13 @@ struct ProdArgs {
     u32 wait_first;
     u32 spin_limit;
     const u64 *mail;
+    // FACT variants (rounds of at least 2^EQ_LO_BITS pairs): R is not streamed.  R(i) = hi[i >> EQ_LO_BITS] * lo[i & mask],
+    // lo = eq over the EQ_LO_BITS lowest live variables, hi = R of EQ_LO_BITS rounds later.  The grid's stride is a
+    // multiple of 2^EQ_LO_BITS, so a thread's pairs all have the same low part: it weights its running sums with hi only
+    // (one entry per workgroup and step: scalar loads) and multiplies them by its entry of lo once, at the end.
+    const u64 *lq0, *lq1, *hq0, *hq1;
 };
+constexpr u32 EQ_LO_BITS = 16;
 
 // The kernels hand the host the sums q(t), t = 0..NF (q(1) left at zero when t = 1 was skipped), not the round
 // message: p(t) = scale(t) q(t) + const, the extra point p(NF + 1) of a sum with an eq factor, and p(1) from the
@@ -674,9 +680,10 @@ __device__ __forceinline__ void publish_sums(u64 *out_host, u64 seq, u32 *counte
     }
 }
 
-template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1>
+template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT = false>
 __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial, FastFin ff)
 {
+    static_assert(!FACT || EQ, "factored weights belong to the eq factor");
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ int last_flag;
@@ -725,8 +732,15 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             }
         }
         if (EQ) {
-            w.q0 = a.q0[i];
-            w.q1 = a.q1[i];
+            if (FACT) {
+                // the same entry for the whole workgroup (BLOCK divides 2^EQ_LO_BITS)
+                const u32 hi = __builtin_amdgcn_readfirstlane((u32)(i >> EQ_LO_BITS));
+                w.q0 = a.hq0[hi];
+                w.q1 = a.hq1[hi];
+            } else {
+                w.q0 = a.q0[i];
+                w.q1 = a.q1[i];
+            }
         }
     };
     // one loop step on loaded operands
@@ -840,6 +854,14 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     E2 acc[NP];
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = gl::acc_reduce(lz[t]);
+    if (FACT) {
+        // the low part of the weight, the same for all pairs of this thread
+        const u64 lo = ((u64)blockIdx.x * BLOCK + threadIdx.x) & ((1u << EQ_LO_BITS) - 1);
+        const gl::E2P lp = gl::prep(gl::e2(a.lq0[lo], a.lq1[lo]));
+#pragma unroll
+        for (int t = 0; t < NP; t++)
+            if (!(t == 1 && skip1)) acc[t] = gl::mulp(acc[t], lp);
+    }
     block_reduce<NP>(acc, lds);
     if (gridDim.x == 1) {
         // a single workgroup: its sums are the round's sums, no partials and no ticket
