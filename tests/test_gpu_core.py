@@ -288,6 +288,31 @@ def test_config3_shape_mid_size(dp, ctx, orc):
     _check_prove(dp, ctx, orc, n, gpu, ref, [(ONE, [2, 0, 1])])
 
 
+@pytest.mark.parametrize("n,kinds,zero_at", [(17, "ee", None), (18, "be", 1), (17, "e", None), (18, "b", 0), (19, "bb", 2)])
+def test_large_rounds_take_eq_weights_from_two_small_tables(dp, ctx, orc, n, kinds, zero_at):
+    """In rounds of at least 2^16 pairs a product with an eq factor does not stream the eq weights: they are the
+    product of an entry of a 2^16-entry table (per thread) and one of a later level (per workgroup and step).
+    One and two tables, base-field and extension sources, and an eq point with a zero coordinate in such a round
+    (then the evaluation at 1 cannot come from the claim)."""
+    tabs_gpu, tabs_ref = [], []
+    for k, kind in enumerate(kinds):
+        if kind == "b":
+            v = rand_base(1 << n, 8100 + k)
+            tabs_gpu.append(ctx.mle_from_base(v))
+            tabs_ref.append(orc.embed_base(v))
+        else:
+            v = rand_e2(1 << n, 8100 + k)
+            tabs_gpu.append(ctx.mle_from_ext2(v))
+            tabs_ref.append(v)
+    r = rand_e2(n, 8110)
+    if zero_at is not None:
+        r[zero_at] = 0
+    tabs_gpu.append(ctx.eq_build(r))
+    tabs_ref.append(orc.eq_evals(r))
+    e = len(kinds)
+    _check_prove(dp, ctx, orc, n, tabs_gpu, tabs_ref, [(np.array([7, 3], dtype=np.uint64), [e] + list(range(e)))])
+
+
 def _materialise_zero_pad(tab, n):
     out = np.zeros((1 << n, 2), dtype=np.uint64)
     out[: tab.shape[0]] = tab
