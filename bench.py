@@ -275,7 +275,7 @@ def main():
     survey_total = float(2 * (1 << n) * 32 + (1 << (n + 1)) * 16 * 3)
     roofline = {
         "bound": "hbm",
-        "kernel": "prod_kernel<2,2,true,true,true> (round 2: fold f,g + evaluate; eq factor in closed form)",
+        "kernel": "prod_kernel<2,2,true,true,true,true> (round 2: fold f,g + evaluate; eq factor in closed form, its weights from two small tables)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

@@ -2303,19 +2303,21 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         const E2 s1 = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2_one())) : base_scale;
         const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
         a.skip1 = skip1 ? 1 : 0;
-        if (has_eq) {
-            const u64 off = eq_level_off(sc->n_vars, j);
-            a.q0 = sc->eq_c0 + off;
-            a.q1 = sc->eq_c1 + off;
-            // (the factored form needs a grid whose stride is a multiple of the low table's size)
-            if (sc->fast && j <= sc->eq_info->fact_levels && ((u64)blocks * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
-                const u64 lo = eq_low_off(sc->n_vars, j), hi = eq_level_off(sc->n_vars, j + dpk::EQ_LO_BITS);
-                a.lq0 = sc->eq_c0 + lo;
-                a.lq1 = sc->eq_c1 + lo;
-                a.hq0 = sc->eq_c0 + hi;
-                a.hq1 = sc->eq_c1 + hi;
+        // where round jj finds its eq weights: level jj, or for the large rounds of a product (a grid whose stride is a
+        // multiple of the low table's size) the low table of level jj and level jj + 16
+        auto set_eq_weights = [&](dpk::ProdArgs &pa, u32 jj, u32 blocks_jj) {
+            const u64 off = eq_level_off(sc->n_vars, jj);
+            pa.q0 = sc->eq_c0 + off;
+            pa.q1 = sc->eq_c1 + off;
+            if (sc->fast && jj <= sc->eq_info->fact_levels && ((u64)blocks_jj * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
+                const u64 lo = eq_low_off(sc->n_vars, jj), hi = eq_level_off(sc->n_vars, jj + dpk::EQ_LO_BITS);
+                pa.lq0 = sc->eq_c0 + lo;
+                pa.lq1 = sc->eq_c1 + lo;
+                pa.hq0 = sc->eq_c0 + hi;
+                pa.hq1 = sc->eq_c1 + hi;
             }
-        }
+        };
+        if (has_eq) set_eq_weights(a, j, blocks);
         auto prepare_message = [&]() {
             if (j >= 2) {
                 // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
@@ -2669,7 +2671,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             if (sc->tail_j0 && j + 1 == sc->tail_j0) {
                 CHK(launch_tail_at(j + 1, next_seq));
                 made = true;
-            } else if (blocks_for_pairs(n_pairs >> 1) <= POLY_AHEAD_MAX_WORKGROUPS) {
+            } else {
+                // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
                 // p(1) comes from the claim unless the scale vanishes at 1
                 bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
                 if (has_eq) {
@@ -2677,16 +2680,13 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                     skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
                 }
                 dpk::ProdArgs an = sc->fast_args[j + 1];
-                if (has_eq) {
-                    const u64 off = eq_level_off(sc->n_vars, j + 1);
-                    an.q0 = sc->eq_c0 + off;
-                    an.q1 = sc->eq_c1 + off;
-                }
+                if (has_eq) set_eq_weights(an, j + 1, blocks_for_pairs(n_pairs >> 1));
                 an.r0 = an.r1 = 0;
                 an.skip1 = skip1_next ? 1 : 0;
                 an.wait_first = 1;
                 an.spin_limit = 4000000;
                 an.mail = ctx->d_pinned + (ctx->res_off - 64);
+                an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 128) : nullptr;
                 dpk::FastFin fn = ff;
                 fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
                 fn.seq = next_seq;

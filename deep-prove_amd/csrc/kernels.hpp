@@ -606,6 +606,9 @@ struct ProdArgs {
     u32 wait_first;
     u32 spin_limit;
     const u64 *mail;
+    // A launch of many workgroups made ahead: only workgroup 0 polls the host's mailbox; it copies the mail to these
+    // MAIL_WORDS words of device memory, where the other workgroups look for it.  nullptr: every workgroup polls the mailbox.
+    u64 *relay;
     // FACT variants (rounds of at least 2^EQ_LO_BITS pairs): R is not streamed.  R(i) = hi[i >> EQ_LO_BITS] * lo[i & mask],
     // lo = eq over the EQ_LO_BITS lowest live variables, hi = R of EQ_LO_BITS rounds later.  The grid's stride is a
     // multiple of 2^EQ_LO_BITS, so a thread's pairs all have the same low part: it weights its running sums with hi only
@@ -695,7 +698,29 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     auto take_challenge = [&]() -> bool {
         __shared__ u64 box[MAIL_WORDS];
         __shared__ int ok_flag;
-        if (!tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag)) return false;
+        bool ok;
+        if (a.relay == nullptr) {
+            ok = tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag);
+        } else if (blockIdx.x == 0) {
+            ok = tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag);
+            if (threadIdx.x == 0) {
+                u64 w[MAIL_WORDS];
+#pragma unroll
+                for (int k = 0; k < MAIL_WORDS; k++) w[k] = box[k];
+                if (!ok) {
+                    // no mail came: pass on a mail of this number that this variant does not accept, so that every workgroup exits
+                    w[MAIL_SEQ] = ff.seq;
+                    w[MAIL_R] = w[MAIL_R + 1] = 0;
+                    w[MAIL_SKIP1] = SKIP1 ? 0 : 1;
+                    w[MAIL_CHK] = ff.seq ^ mail_mix(w[MAIL_SKIP1], MAIL_SKIP1);
+                }
+#pragma unroll
+                for (int k = 0; k < MAIL_WORDS; k++) st_sys(a.relay + k, w[k]);
+            }
+        } else {
+            ok = tail_wait_mail(a.relay, a.spin_limit, ff.seq, box, &ok_flag);
+        }
+        if (!ok) return false;
         if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
         // (kept in scalar registers, as the kernel argument would be)
         r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));

@@ -182,12 +182,12 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     _check(dp, ctx, orc, n, gpu, host, terms)
 
 
-@pytest.mark.parametrize("with_eq", [True, False])
-def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq):
-    """The same for a single product of full-size tables: its small rounds and the resident kernel of its last
-    rounds (first round 6 of 14 here) are launched during the round before."""
+@pytest.mark.parametrize("with_eq,n", [(True, 14), (False, 14), (True, 19), (False, 18)])
+def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
+    """The same for a single product of full-size tables: every round after the first and the resident kernel of
+    its last rounds (first round 6 of 14) are launched during the round before.  In a launch of more than 64
+    workgroups (n = 18, 19) only the first workgroup looks for the mail and passes it on to the others."""
     import time
-    n = 14
     f, g = rand_base(1 << n, 31), rand_e2(1 << n, 32)
     gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
     if with_eq:
