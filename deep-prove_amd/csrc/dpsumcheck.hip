@@ -1345,6 +1345,8 @@ struct dps_sc {
 namespace {
 
 u64 *mailbox(dps_ctx *ctx) { return ctx->h_pinned + ctx->res_off - 64; }
+// device memory through which the first workgroup of a large launch made ahead passes the mail on (behind the ticket counter)
+u64 *mail_relay(dps_ctx *ctx) { return reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 128); }
 
 // completes a mail: check word over the payload as it stands, then the sequence number the kernel waits for
 void send_mail(dps_ctx *ctx, u64 seq)
@@ -1456,7 +1458,8 @@ constexpr u32 SLOT_MAX_WORKGROUPS = 16;
 static_assert(SLOT_MAX_WORKGROUPS <= POLY_RAW_MAX_GROUPS, "the per-workgroup result areas are those of the resident groups");
 u32 slots_for(u32 workgroups) { return workgroups > 1 && workgroups <= SLOT_MAX_WORKGROUPS ? workgroups : 0; }
 
-// A round's launch is made ahead of time only with at most this many workgroups: each of them polls the mailbox
+// In a launch made ahead of its round every workgroup polls the host's mailbox up to this many workgroups; in a larger
+// one only the first does and passes the mail on through device memory
 constexpr u32 POLY_AHEAD_MAX_WORKGROUPS = 64;
 // ... and is trusted to be still waiting for its mail for this long (its own patience: spin_limit polls of pinned
 // memory, at least a few hundred milliseconds)
@@ -2539,6 +2542,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 pa.group_stride = 1;
                 pa.raw_out = nullptr;
                 pa.wait_first = ahead ? 1 : 0;
+                // (more workgroups than should poll the host's memory: the first one polls and passes the mail on)
+                pa.relay = ahead && p.blocks * n_groups > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
                 if (p.reside) {
                     pa.last_round = sc->n_vars;
                     if (n_groups > 1) {
@@ -2616,7 +2621,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                         skip1_next = !(rho.c0 == 0 && rho.c1 == 0);
                     }
                     const Plan pn = plan_round(j + 1, skip1_next);
-                    if (pn.split && pn.blocks * n_groups <= POLY_AHEAD_MAX_WORKGROUPS) {
+                    {
                         CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
                         sc->tail_running = true;
                         sc->tail_seq0 = ctx->seq + 1;
@@ -2686,7 +2691,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 an.wait_first = 1;
                 an.spin_limit = 4000000;
                 an.mail = ctx->d_pinned + (ctx->res_off - 64);
-                an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 128) : nullptr;
+                an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
                 dpk::FastFin fn = ff;
                 fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
                 fn.seq = next_seq;

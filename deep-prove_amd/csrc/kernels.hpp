@@ -571,6 +571,32 @@ __device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, 
     return *ok_lds != 0;
 }
 
+// The first mail of a launch made ahead of its round.  With few workgroups each polls the host's mailbox (relay ==
+// nullptr).  With many, only the first one does (first_wg) and copies the mail to MAIL_WORDS words of device memory, where
+// the others look for it; when no mail comes it passes on a mail of this number with `reject_skip1` in the skip word, a
+// value the calling variant does not accept, so that every workgroup leaves.  True: the mail is in `box`.
+__device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, bool first_wg, u32 spin_limit, u64 seq, u64 reject_skip1, u64 *box,
+                                                int *ok_lds)
+{
+    if (relay == nullptr) return tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
+    if (!first_wg) return tail_wait_mail(relay, spin_limit, seq, box, ok_lds);
+    const bool ok = tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
+    if (threadIdx.x == 0) {
+        u64 w[MAIL_WORDS];
+#pragma unroll
+        for (int k = 0; k < MAIL_WORDS; k++) w[k] = box[k];
+        if (!ok) {
+            w[MAIL_SEQ] = seq;
+            w[MAIL_R] = w[MAIL_R + 1] = 0;
+            w[MAIL_SKIP1] = reject_skip1;
+            w[MAIL_CHK] = seq ^ mail_mix(reject_skip1, MAIL_SKIP1);
+        }
+#pragma unroll
+        for (int k = 0; k < MAIL_WORDS; k++) st_sys(relay + k, w[k]);
+    }
+    return ok;
+}
+
 // ---------------------------------------------------------------------------
 // fused product kernels: one term, NF full-size tables (the first NB of them
 // base-field in the source), optionally times an eq(rho, x) factor.
@@ -698,28 +724,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     auto take_challenge = [&]() -> bool {
         __shared__ u64 box[MAIL_WORDS];
         __shared__ int ok_flag;
-        bool ok;
-        if (a.relay == nullptr) {
-            ok = tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag);
-        } else if (blockIdx.x == 0) {
-            ok = tail_wait_mail(a.mail, a.spin_limit, ff.seq, box, &ok_flag);
-            if (threadIdx.x == 0) {
-                u64 w[MAIL_WORDS];
-#pragma unroll
-                for (int k = 0; k < MAIL_WORDS; k++) w[k] = box[k];
-                if (!ok) {
-                    // no mail came: pass on a mail of this number that this variant does not accept, so that every workgroup exits
-                    w[MAIL_SEQ] = ff.seq;
-                    w[MAIL_R] = w[MAIL_R + 1] = 0;
-                    w[MAIL_SKIP1] = SKIP1 ? 0 : 1;
-                    w[MAIL_CHK] = ff.seq ^ mail_mix(w[MAIL_SKIP1], MAIL_SKIP1);
-                }
-#pragma unroll
-                for (int k = 0; k < MAIL_WORDS; k++) st_sys(a.relay + k, w[k]);
-            }
-        } else {
-            ok = tail_wait_mail(a.relay, a.spin_limit, ff.seq, box, &ok_flag);
-        }
+        const bool ok = wait_first_mail(a.mail, a.relay, blockIdx.x == 0, a.spin_limit, ff.seq, SKIP1 ? 0 : 1, box, &ok_flag);
         if (!ok) return false;
         if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
         // (kept in scalar registers, as the kernel argument would be)
@@ -1132,8 +1137,9 @@ struct PolyArgs {
     u32 state_off;
     u32 finish;      // resident rounds: stay after the last round for the last challenge and publish the final evaluations
     u32 group_stride;  // resident rounds: descriptors of consecutive rounds of one group lie this many apart
-    u32 wait_first;  // launched ahead of its round: the challenge and the scalars of round j also arrive by mail (seq)
+    u32 wait_first;  // launched ahead of its round: the challenge of round j also arrives by mail (seq)
     u32 pad;
+    u64 *relay;      // ... through these words of device memory for all workgroups but the first (see wait_first_mail); or nullptr
     // Several groups resident side by side (one workgroup each, gridDim.y of them): a workgroup cannot finish the
     // message, which is the sum over the groups, so each publishes its own sums q(t) (and later its tables' final
     // evaluations) to its 64-word slot raw_out + 64 * blockIdx.y, laid out like the main result area, and the host adds.
@@ -1157,7 +1163,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     auto dl0 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 2) * BLOCK + tid]; };
     auto dl1 = [&](u32 k) -> u64 & { return dyn[(k * 4 + 3) * BLOCK + tid]; };
     const u64 n_pairs = a.n_pairs;
-    const E2 r = gl::e2(a.r0, a.r1);
+    E2 r = gl::e2(a.r0, a.r1);
     const u64 *q0 = a.q0, *q1 = a.q1;
     {
         const bool inl = a.groups == nullptr;  // a single group handed over in the kernel arguments
@@ -1185,6 +1191,15 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     const u32 n_terms = g.term_end - g.term_begin;
     const u32 n_ops = g.op_end - g.op_begin;
     const PolyOp *lops = reinterpret_cast<const PolyOp *>(lterms);
+    if (a.wait_first) {
+        // launched while the previous round was still running: the challenge comes by mail
+        __shared__ u64 box[MAIL_WORDS];
+        __shared__ int ok_flag;
+        if (!wait_first_mail(a.mail, a.relay, blockIdx.x == 0 && blockIdx.y == 0, a.spin_limit, ff.seq, SKIP1 ? 0 : 1, box, &ok_flag)) return;
+        // the other way of getting p(1) is not compiled into this variant: the host ends the launch instead
+        if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
+        r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
+    }
     const gl::E2P rp = gl::prep(r);
 
     // Few live registers matter more here than loads in flight: the loop is arithmetic, and it is the number of
@@ -1390,8 +1405,11 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         __syncthreads();
     }
     // the challenge of a round, from the mail the host posted for it
-    auto take_mail = [&](u64 seq) -> bool {
-        if (!tail_wait_mail(a.mail, a.spin_limit, seq, box, &ok_flag)) return false;
+    auto take_mail = [&](u64 seq, bool first) -> bool {
+        // (only the first mail of a launch made ahead can concern several workgroups)
+        const bool ok = first ? wait_first_mail(a.mail, a.relay, blockIdx.x == 0 && blockIdx.y == 0, a.spin_limit, seq, SKIP1 ? 0 : 1, box, &ok_flag)
+                              : tail_wait_mail(a.mail, a.spin_limit, seq, box, &ok_flag);
+        if (!ok) return false;
         // a run-time switch to evaluating t = 1 (or not) is not compiled in: the host ends the launch instead
         if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
         r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
@@ -1399,7 +1417,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         return true;
     };
     // launched while the previous round was still running: everything that depends on its challenge comes by mail
-    if (a.wait_first && !take_mail(a.seq)) return;
+    if (a.wait_first && !take_mail(a.seq, true)) return;
   for (;;) {
     const PolyGroup &g = gall[j - a.j];
     const u32 n_tabs = g.n_tabs;
@@ -1553,7 +1571,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         }
         // stay for the next round: its challenge and the scalars of its message arrive by mail
         j++;
-        if (!take_mail(a.seq + (j - a.j))) return;
+        if (!take_mail(a.seq + (j - a.j), false)) return;
         n_pairs >>= 1;
         if (sl < a.split_cap && (n_pairs << (sl + 1)) <= (u64)BLOCK) sl++;
         if (EQ) {
