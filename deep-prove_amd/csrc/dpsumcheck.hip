@@ -271,7 +271,8 @@ struct Storage {
 // level j in round j instead of folding the full table.
 struct EqInfo {
     u32 m;
-    u32 fact_levels = 0;  // levels 1..fact_levels have a low table behind the levels (eq_low_off)
+    u32 fact_levels = 0;  // levels 1..fact_levels have room for a low table behind the levels (eq_low_off)
+    bool fact_built = false;  // ... and the low tables are there (built when a product session first wants them)
     std::vector<E2> point;
 };
 
@@ -741,11 +742,6 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
         js.job[n_jobs++] = dpk::EqJob{l, m - l, eq_level_off(m, l)};
         max_bits = std::max(max_bits, m - l);
     }
-    // the low tables of the large levels (the caller allocated eq_storage_entries(m))
-    for (u32 l = 1; l <= eq_fact_levels(m); l++) {
-        js.job[n_jobs++] = dpk::EqJob{l, dpk::EQ_LO_BITS, eq_low_off(m, l)};
-        max_bits = std::max(max_bits, dpk::EQ_LO_BITS);
-    }
     // seeds live in a scratch block behind nothing: a separate allocation
     void *seed_block = nullptr;
     u64 *seed0 = nullptr, *seed1 = nullptr;
@@ -797,6 +793,27 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
 }
 
 }  // namespace
+
+// the low tables of the large levels of an eq table (storage of eq_storage_entries(m) entries), one launch
+int32_t eq_build_low(dps_ctx *ctx, const EqInfo &info, u64 *o0, u64 *o1)
+{
+    const u32 m = info.m;
+    if (!eq_fact_levels(m)) return DPS_OK;
+    dpk::EqJobs js;
+    memset(&js, 0, sizeof js);
+    for (u32 i = 0; i < m; i++) {
+        js.point[2 * i] = info.point[i].c0;
+        js.point[2 * i + 1] = info.point[i].c1;
+    }
+    js.o0 = o0;
+    js.o1 = o1;
+    u32 n_jobs = 0;
+    for (u32 l = 1; l <= eq_fact_levels(m); l++) js.job[n_jobs++] = dpk::EqJob{l, dpk::EQ_LO_BITS, eq_low_off(m, l)};
+    ProfScope ps(ctx, DPS_K_EQ, (double)n_jobs * (double)(1u << dpk::EQ_LO_BITS) * 16.0);
+    dpk::eq_define_kernel<<<dim3((1u << dpk::EQ_LO_BITS) / dpk::BLOCK, n_jobs), dpk::BLOCK, 0, ctx->stream>>>(js);
+    HIPCHK(ctx, hipGetLastError());
+    return DPS_OK;
+}
 
 extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m, dps_mle **out)
 {
@@ -1881,6 +1898,12 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     // the last rounds run in one resident workgroup when every registered table belongs to the term
     // (from the round of 2^8 = TAIL_PAIRS pairs on, or from round 2 in a smaller sum; the tail kernel reads extension
     // tables, which every table is once folded, so a start in round 2 needs extension tables to begin with)
+    // a product with an eq factor reads the eq weights of its large rounds as products of two small tables: the low ones are
+    // built now if this eq table has not served such a session before (they lie behind its levels; the table itself is not touched)
+    if (sc->fast && sc->fast_eq >= 0 && sc->eq_info->fact_levels && !sc->eq_info->fact_built) {
+        CHK(eq_build_low(ctx, *sc->eq_info, const_cast<u64 *>(sc->eq_c0), const_cast<u64 *>(sc->eq_c1)));
+        sc->eq_info->fact_built = true;
+    }
     if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
         const u32 j0 = n_vars > 10 ? n_vars - 8 : 2;
         bool all_ext = true;
@@ -2312,7 +2335,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u64 off = eq_level_off(sc->n_vars, jj);
             pa.q0 = sc->eq_c0 + off;
             pa.q1 = sc->eq_c1 + off;
-            if (sc->fast && jj <= sc->eq_info->fact_levels && ((u64)blocks_jj * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
+            if (sc->fast && sc->eq_info->fact_built && jj <= sc->eq_info->fact_levels && ((u64)blocks_jj * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
                 const u64 lo = eq_low_off(sc->n_vars, jj), hi = eq_level_off(sc->n_vars, jj + dpk::EQ_LO_BITS);
                 pa.lq0 = sc->eq_c0 + lo;
                 pa.lq1 = sc->eq_c1 + lo;
