@@ -81,7 +81,7 @@ dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
-           "dps_partial_eval", "dps_sc_begin", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
+           "dps_partial_eval", "dps_sc_begin", "dps_sc_set_claim", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
            "dps_sc_prove", "dps_logup_build", "dps_logup_num_layers", "dps_logup_layer", "dps_logup_outputs",
            "dps_logup_free", "dps_profile_enable", "dps_profile_reset", "dps_profile_read"]:
     getattr(dev, _f).restype = _i32
@@ -100,6 +100,7 @@ dev.dps_mle_fix_high.argtypes = [_vp, _vp, _vp, _u32, _vp]
 dev.dps_partial_eval.argtypes = [_vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _u32, _vp]
 dev.dps_sc_begin.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp]
 dev.dps_sc_degree.argtypes = [_vp, _vp]
+dev.dps_sc_set_claim.argtypes = [_vp, _vp]
 dev.dps_sc_round.argtypes = [_vp, _vp, _vp]
 dev.dps_sc_finish.argtypes = [_vp, _vp, _vp]
 dev.dps_sc_free.argtypes = [_vp]
@@ -308,6 +309,11 @@ class Session:
         if getattr(self, "_h", None) and self.ctx._c:
             dev.dps_sc_free(self._h)
         self._h = None
+
+    def set_claim(self, claim):
+        """The value of the whole sum, if known: round 1 then takes p(1) from it (dps_sc_set_claim)."""
+        c = _e2(claim)
+        self.ctx._chk(dev.dps_sc_set_claim(self._h, _ptr(c)), "dps_sc_set_claim")
 
     def abort(self):
         self.ctx._chk(dev.dps_sc_abort(self._h), "dps_sc_abort")

@@ -1308,7 +1308,8 @@ struct dps_sc {
     const u64 *eq_c0, *eq_c1;  // its storage (level 0 at entry 0)
     E2 fast_coeff;
     E2 eq_scalar;       // product of eq1(rho_i, r_{i+1}) over the bound variables
-    E2 claim;           // p(0) + p(1) expected from the next message (valid from round 2)
+    E2 claim;           // p(0) + p(1) expected from the next message (valid from round 2; from round 1 with dps_sc_set_claim)
+    bool have_claim;    // the caller said what the whole sum is
     std::vector<E2> last_msg;
     bool broken;        // its tail kernel was interrupted by another call on the context
     u32 tail_j0;        // first round run by the resident tail kernel, 0 = none
@@ -1408,6 +1409,8 @@ void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u6
                 dpk::prod_kernel<NF, NB, true, true, true, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
             else if (fold)
                 dpk::prod_kernel<NF, NB, true, true, false, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+            else if (a.skip1)
+                dpk::prod_kernel<NF, NB, false, true, true, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
             else
                 dpk::prod_kernel<NF, NB, false, true, false, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
             return;
@@ -1721,6 +1724,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->fast_eq = -1;
     sc->eq_scalar = gl::e2_one();
     sc->claim = gl::e2_zero();
+    sc->have_claim = false;
     if (sc->n_terms == 1 && sc->terms[0].n_factors >= 2 && sc->terms[0].n_factors <= 3 && n_vars >= 1) {
         const dps_term &t = sc->terms[0];
         bool ok = true;
@@ -2194,6 +2198,17 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     return DPS_OK;
 }
 
+extern "C" int32_t dps_sc_set_claim(dps_sc *sc, const uint64_t *claim)
+{
+    if (!sc || !claim) return DPS_ERR_INVALID;
+    dps_ctx *ctx = sc->ctx;
+    if (sc->round != 0 || sc->finished) return fail(ctx, DPS_ERR_STATE, "dps_sc_set_claim: the session has started");
+    if (!canonical(claim, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_set_claim: claim not canonical");
+    sc->claim = gl::e2(claim[0], claim[1]);
+    sc->have_claim = true;
+    return DPS_OK;
+}
+
 extern "C" int32_t dps_sc_degree(const dps_sc *sc, uint32_t *degree)
 {
     if (!sc || !degree) return DPS_ERR_INVALID;
@@ -2327,7 +2342,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         E2 base_scale = sc->fast_coeff;
         if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
         const E2 s1 = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2_one())) : base_scale;
-        const bool skip1 = j >= 2 && !(s1.c0 == 0 && s1.c1 == 0);
+        const bool skip1 = (j >= 2 || sc->have_claim) && !(s1.c0 == 0 && s1.c1 == 0);
         a.skip1 = skip1 ? 1 : 0;
         // where round jj finds its eq weights: level jj, or for the large rounds of a product (a grid whose stride is a
         // multiple of the low table's size) the low table of level jj and level jj + 16

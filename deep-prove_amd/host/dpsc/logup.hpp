@@ -275,7 +275,7 @@ inline LogUpBatchProof new_batch_multiple_sizes_prove(const Context &ctx, const 
         for (auto &m : eq_mles) all.push_back(&m);
         auto builder = VirtualPolynomialsBuilder::new_with_mles(optimal_sumcheck_threads(current_layer_vars), current_layer_vars, all);
         auto vp = builder.to_virtual_polys({full}, {alpha, lambda});
-        auto res = IOPProverState::prove(vp, transcript);
+        auto res = IOPProverState::prove(vp, transcript, &current_claim);
 
         // prover.rs:278-296
         sumcheck_point = res.second.collect_raw_challenges();

@@ -48,7 +48,10 @@ public:
         for (size_t i = 0; i < beta_evals.size(); i++)
             sum_expr = sum_expr + Expression::Challenge((uint16_t)i, 1, F::one(), F::zero()) * builder.lift(beta_evals[i]);
         auto vp = builder.to_virtual_polys({poly_expr * sum_expr}, challenges);
-        auto res = IOPProverState::prove(vp, t);
+        // the sum the proof is about: sum_i challenge_i * claim_i (same_poly.rs:226-227)
+        F claimed = F::zero();
+        for (size_t i = 0; i < claims_.size(); i++) claimed += challenges[i] * claims_[i].eval;
+        auto res = IOPProverState::prove(vp, t, &claimed);
         const F eval = res.second.get_mle_flatten_final_evaluations()[0];
         return {Proof{std::move(res.first), eval}, Claim{res.second.collect_raw_challenges(), eval}};
     }

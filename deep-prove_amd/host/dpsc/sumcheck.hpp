@@ -108,7 +108,9 @@ public:
     // the d+1 evaluations; the challenge of a round is squeezed right after its
     // message.  Runs the whole protocol; the returned state holds the challenges
     // and the final evaluation of every registered table.
-    static std::pair<IOPProof, IOPProverState> prove(const VirtualPolynomials &vp, Transcript &transcript)
+    // `claimed_sum`: the value of the whole sum when the caller knows it (the reference's callers put it on the transcript
+    // before this call); round 1 then need not evaluate the polynomial at 1.
+    static std::pair<IOPProof, IOPProverState> prove(const VirtualPolynomials &vp, Transcript &transcript, const F *claimed_sum = nullptr)
     {
         const Context &ctx = *vp.ctx;
         const std::vector<const dps_mle *> &handles = vp.mles;
@@ -117,6 +119,10 @@ public:
                                (uint32_t)vp.terms.size(), &sc),
                   "dps_sc_begin");
         std::unique_ptr<dps_sc, int32_t (*)(dps_sc *)> guard(sc, &dps_sc_free);
+        if (claimed_sum) {
+            const uint64_t limbs[2] = {claimed_sum->c0, claimed_sum->c1};
+            ctx.check(dps_sc_set_claim(sc, limbs), "dps_sc_set_claim");
+        }
         uint32_t degree = 0;
         dps_sc_degree(sc, &degree);
         transcript.append_u64(vp.num_vars);

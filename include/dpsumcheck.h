@@ -150,6 +150,11 @@ typedef struct dps_term {
 int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
                      const dps_term *terms, uint32_t n_terms, dps_sc **out);
 int32_t dps_sc_degree(const dps_sc *sc, uint32_t *degree);
+/* Optional, before round 1: the value of the whole sum, when the caller knows it (the reference's callers do: they put
+ * it on the transcript before they call prove, e.g. current_claim at logup_gkr/prover.rs:257-261).  Round 1 then takes
+ * p(1) = claim - p(0) instead of evaluating at 1, as every later round does with the claim it derives itself.  The
+ * messages are the same bits as without the call if the claim is the true sum; with a wrong claim the proof is wrong. */
+int32_t dps_sc_set_claim(dps_sc *sc, const uint64_t *claim /* 2 limbs */);
 /* One round: fold with the previous round's challenge (NULL in round 1), then
  * evaluate.  evals_out receives degree+1 extension elements, p(0..degree).  Only
  * these cross to the host. */

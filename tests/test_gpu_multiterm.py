@@ -212,3 +212,49 @@ def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
             assert (s.finish(chal) == ref_finals).all()
             del s
     _check(dp, ctx, orc, n, gpu, host, terms)
+
+
+def _fadd(a, b):
+    """sum of two extension elements given as limb pairs"""
+    P = 0xFFFFFFFF00000001
+    return np.array([(int(a[0]) + int(b[0])) % P, (int(a[1]) + int(b[1])) % P], dtype=np.uint64)
+
+
+@pytest.mark.parametrize("shape", ["product n=6", "product n=14", "product n=19", "product n=12 no eq", "terms n=8", "terms n=13", "terms n=18"])
+def test_claim_known_before_round_one(dp, ctx, orc, shape):
+    """With the value of the whole sum given (dps_sc_set_claim) round 1 takes p(1) from it like every later round;
+    the messages and final evaluations are the same bits.  Covers the single-product kernels (small, with the resident
+    last rounds, with factored eq weights) and the multi-term ones (resident from round 1, launched, large rounds)."""
+    kind, rest = shape.split(" ", 1)
+    n = int(rest.split("=")[1].split()[0])
+    if kind == "product":
+        f, g = rand_base(1 << n, 41), rand_e2(1 << n, 42)
+        gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
+        if "no eq" not in shape:
+            pt = rand_e2(n, 43)
+            gpu.append(ctx.eq_build(pt))
+            host.append(orc.eq_evals(pt))
+            fs = [2, 0, 1]
+        terms = [(np.array([3, 5], dtype=np.uint64), fs)]
+    else:
+        gpu, host, terms = _instance(ctx, orc, 1200 + n, n, [n] * 5, [1], 9, 3, True)
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
+    s = ctx.session(n, gpu, terms)
+    s.set_claim(_fadd(ref_proof[0][0], ref_proof[0][1]))
+    chal = None
+    for j in range(n):
+        assert (s.round(chal) == ref_proof[j]).all(), (shape, j)
+        chal = ref_point[j]
+    assert (s.finish(chal) == ref_finals).all()
+    # too late once the session has started
+    with pytest.raises(dp.DpsError):
+        s.set_claim(ref_proof[0][0])
+    del s
+    # a wrong claim gives a first message that sums to it (and no longer the true one)
+    s = ctx.session(n, gpu, terms)
+    wrong = _fadd(_fadd(ref_proof[0][0], ref_proof[0][1]), np.array([1, 0], dtype=np.uint64))
+    s.set_claim(wrong)
+    m = s.round(None)
+    assert (m[0] == ref_proof[0][0]).all() and (_fadd(m[0], m[1]) == wrong).all()
+    del s
+    _check(dp, ctx, orc, n, gpu, host, terms)
