@@ -1350,7 +1350,7 @@ struct dps_sc {
     u64 pairs_seq;                            // nonzero: the last round's launch also published the tables' last pairs, under this number
     bool no_ahead;                            // a launch made ahead was in another call's way once: make no more
     std::chrono::steady_clock::time_point ahead_at;  // when the launch that has had no mail yet was made
-    bool poly_finish_in_kernel;               // every table is in the single group (or is the closed-form eq): the resident kernel finishes
+    bool poly_finish_in_kernel;               // every table is in a group (or is the closed-form eq): the resident kernel hands over the last pairs
     dpk::PolyGroup *d_poly_groups;            // [round 1..n_vars][group]
     dpk::PolyTerm *d_poly_terms;
     std::vector<dpk::PolyGroup> h_poly_groups;  // host copies: a single group travels in the kernel arguments
@@ -2403,7 +2403,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         ff.out_host = fa.out_host;
         ff.seq = fa.seq;
         ff.counter = sc->d_counter;
-        // mail for a resident kernel: challenge, scales, claim; then the sequence number it waits for
+        // mail for a kernel that waits on the GPU: challenge, whether t = 1 is skipped; then the sequence number it waits for
         auto post_mail = [&]() {
             u64 *mb = mailbox(ctx);
             mb[dpk::MAIL_R] = a.r0;

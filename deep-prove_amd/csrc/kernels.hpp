@@ -611,10 +611,10 @@ __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, boo
 // eq1(a, b) = a b + (1 - a)(1 - b), and R = eq(rho_{v+1..}, .) a table of half this
 // round's size, prepared when the eq table was built.  The kernel sums
 // q(t) = sum_{x'} R(x') prod_f table_f(t, x') at t = 0..NF; the round message
-// p(t) = coeff * S * eq1(rho_v, t) * q(t) at t = 0..NF+1 is finished by the last
-// workgroup (q has degree NF, so q(NF+1) follows from the NF+1 sums).
+// p(t) = coeff * S * eq1(rho_v, t) * q(t) at t = 0..NF+1 is formed by the host
+// from the sums (q has degree NF, so q(NF+1) follows from the NF+1 sums).
 //
-// From round 2 on the caller knows the claim p(0) + p(1); then t = 1 is skipped
+// From round 2 on the host knows the claim p(0) + p(1); then t = 1 is skipped
 // in the loop and q(1) is solved from the claim.
 // ---------------------------------------------------------------------------
 struct ProdArgs {
@@ -1055,8 +1055,8 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
 // at t = 0..NF with the coefficients applied here, so one set of running sums
 // serves all terms.  An eq factor common to all terms is taken out in closed
 // form exactly as in prod_kernel (G is then the polynomial without it), and
-// t = 1 is skipped when the claim is known.  Output and finish are those of
-// prod_kernel: per-workgroup sums of G(t) (times R), then fast_finalize.
+// t = 1 is skipped when the claim is known.  Output is that of prod_kernel:
+// per-workgroup sums of G(t) (times R), gathered by the last workgroup and handed to the host.
 // Groups are grid rows; their partials are simply added.
 // ---------------------------------------------------------------------------
 constexpr int POLY_MAXT = 7;
@@ -1135,7 +1135,7 @@ struct PolyArgs {
     u32 split_cap;   // resident rounds: the share doubles as the pairs halve, up to 2^split_cap lanes
     u32 lds_state;   // resident rounds: the folded tables stay in LDS (state_off words into the dynamic LDS)
     u32 state_off;
-    u32 finish;      // resident rounds: stay after the last round for the last challenge and publish the final evaluations
+    u32 finish;      // resident rounds: with the last round, also publish value and slope of every table's last pair
     u32 group_stride;  // resident rounds: descriptors of consecutive rounds of one group lie this many apart
     u32 wait_first;  // launched ahead of its round: the challenge of round j also arrives by mail (seq)
     u32 pad;
@@ -1569,7 +1569,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
             if (tid == 0) publish_words(my_out, HOST_FINALS_SLOT, res, 4 * n_tabs, cf_seq, HOST_PAIRS_SEQ_SLOT, HOST_PAIRS_CHK_SLOT);
             return;
         }
-        // stay for the next round: its challenge and the scalars of its message arrive by mail
+        // stay for the next round: its challenge arrives by mail
         j++;
         if (!take_mail(a.seq + (j - a.j), false)) return;
         n_pairs >>= 1;
