@@ -1484,6 +1484,9 @@ constexpr u32 POLY_AHEAD_MAX_WORKGROUPS = 64;
 // ... and is trusted to be still waiting for its mail for this long (its own patience: spin_limit polls of pinned
 // memory, at least a few hundred milliseconds)
 constexpr int POLY_AHEAD_PATIENCE_MS = 20;
+// Polls of the host's mailbox (2.5 us each) after which a launch made ahead gives up: about 150 ms, so that a caller who
+// went away does not leave up to 768 waiting workgroups on the GPU for long (a resident kernel, one workgroup, waits seconds)
+constexpr u32 AHEAD_SPIN_LIMIT = 60000;
 
 // Rounds of at most this many pairs run on poly_split_kernel
 constexpr u64 POLY_SPLIT_MAX_PAIRS = 1ull << 16;
@@ -2580,6 +2583,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 pa.group_stride = 1;
                 pa.raw_out = nullptr;
                 pa.wait_first = ahead ? 1 : 0;
+                if (ahead && !p.reside) pa.spin_limit = AHEAD_SPIN_LIMIT;
                 // (more workgroups than should poll the host's memory: the first one polls and passes the mail on)
                 pa.relay = ahead && p.blocks * n_groups > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
                 if (p.reside) {
@@ -2727,7 +2731,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 an.r0 = an.r1 = 0;
                 an.skip1 = skip1_next ? 1 : 0;
                 an.wait_first = 1;
-                an.spin_limit = 4000000;
+                an.spin_limit = AHEAD_SPIN_LIMIT;
                 an.mail = ctx->d_pinned + (ctx->res_off - 64);
                 an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
                 dpk::FastFin fn = ff;

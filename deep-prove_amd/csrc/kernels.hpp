@@ -579,7 +579,8 @@ __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, boo
                                                 int *ok_lds)
 {
     if (relay == nullptr) return tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
-    if (!first_wg) return tail_wait_mail(relay, spin_limit, seq, box, ok_lds);
+    // (the others outlast the first workgroup, which always passes something on: their polls of device memory are quicker)
+    if (!first_wg) return tail_wait_mail(relay, spin_limit > (1u << 25) ? ~0u : spin_limit << 6, seq, box, ok_lds);
     const bool ok = tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
     if (threadIdx.x == 0) {
         u64 w[MAIL_WORDS];

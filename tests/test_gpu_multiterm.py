@@ -176,7 +176,8 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
                     if how == "other call":
                         assert (ctx.eq_build(ref_point[:3]).download() == orc.eq_evals(ref_point[:3])).all()
                     else:
-                        time.sleep(0.05)
+                        # longer than the host trusts the launch to wait; the first time, longer than the launch waits
+                        time.sleep(0.3 if after == 1 else 0.05)
             assert (s.finish(chal) == ref_finals).all()
             del s
     _check(dp, ctx, orc, n, gpu, host, terms)
@@ -208,7 +209,8 @@ def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
                     if how == "other call":
                         assert (ctx.eq_build(ref_point[:3]).download() == orc.eq_evals(ref_point[:3])).all()
                     else:
-                        time.sleep(0.05)
+                        # longer than the host trusts the launch to wait; the first time, longer than the launch waits
+                        time.sleep(0.3 if after == 1 else 0.05)
             assert (s.finish(chal) == ref_finals).all()
             del s
     _check(dp, ctx, orc, n, gpu, host, terms)
