@@ -1215,8 +1215,15 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
     u32 nv = log2u(contraction);
     u64 tl = 1ull << nv;
     dps_mle *all = nullptr;
-    rc = new_table(ctx, DPS_EXT2, stacked * tl, &all);
-    if (rc == DPS_OK) {
+    // rows that are a power of two long already: the result is the table as it stands
+    const bool as_it_stands = cur && contraction == tl && cur->kind == DPS_EXT2 && cur->offset == 0 && cur->len == stacked * tl;
+    if (as_it_stands) {
+        all = cur;
+        cur = nullptr;
+    } else {
+        rc = new_table(ctx, DPS_EXT2, stacked * tl, &all);
+    }
+    if (rc == DPS_OK && !as_it_stands) {
         if (cur) {
             dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(cur->st->c0, cur->st->c1, stacked, contraction, tl,
                                                                                     all->st->c0, all->st->c1);
@@ -1255,8 +1262,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
             delete flat;
         }
     }
-    hipError_t e = hipStreamSynchronize(ctx->stream);
-    if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "partial eval: %s", hipGetErrorString(e));
+    // (no wait for the stream: the blocks given back are reused in stream order, and whoever consumes the result waits)
     delete cur;
     if (rc != DPS_OK) {
         delete all;
