@@ -134,7 +134,9 @@ int32_t pool_alloc(dps_ctx *ctx, size_t bytes, void **out)
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
     if (e != hipSuccess) {
-        // give cached blocks back to the driver and retry once
+        // give cached blocks back to the driver and retry once (queued work may still use them: blocks are handed
+        // back to the pool without waiting for the stream)
+        (void)hipStreamSynchronize(ctx->stream);
         for (auto &kv : ctx->free_blocks) (void)hipFree(kv.second);
         ctx->free_blocks.clear();
         e = hipMalloc(&p, bytes);
@@ -697,10 +699,9 @@ extern "C" int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *
 extern "C" int32_t dps_mle_free(dps_mle *mle)
 {
     if (!mle) return DPS_OK;
-    DeviceGuard g(mle->ctx->device);
-    tail_abort(mle->ctx);
-    // work that still reads the storage may be queued
-    (void)hipStreamSynchronize(mle->ctx->stream);
+    // No wait for the stream: when this was the last handle of its storage the block goes back to the context's pool,
+    // whose next user runs on the same stream, after whatever is still queued; a session holds on to the storage of its
+    // tables by itself.
     delete mle;
     return DPS_OK;
 }
@@ -1188,8 +1189,6 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
             j.o1 = next->st->c1;
             rc = axis_dot(ctx, j);
         }
-        hipError_t e = hipStreamSynchronize(ctx->stream);
-        if (rc == DPS_OK && e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "partial eval: %s", hipGetErrorString(e));
         delete beta;
         delete cur;
         cur = next;
@@ -2958,7 +2957,6 @@ extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uin
             HIPCHK(ctx, hipGetLastError());
         }
     }
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     *out = lg.release();
     return DPS_OK;
 }
@@ -3003,10 +3001,7 @@ extern "C" int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8])
 extern "C" int32_t dps_logup_free(dps_logup *lg)
 {
     if (!lg) return DPS_OK;
-    DeviceGuard g(lg->ctx->device);
-    tail_abort(lg->ctx);
-    (void)hipStreamSynchronize(lg->ctx->stream);
-    delete lg;
+    delete lg;  // (the arena goes back to the context's pool; see dps_mle_free)
     return DPS_OK;
 }
 
@@ -3022,6 +3017,7 @@ extern "C" int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *
     void *p = nullptr;
     CHK(pool_alloc(ctx, 6 * n * 8, &p));
     u64 *d = (u64 *)p;
+    (void)hipStreamSynchronize(ctx->stream);  // the copies below do not run on the stream; the block may have a queued user
     hipError_t e = hipMemcpy(d, a, 2 * n * 8, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(d + 2 * n, b, 2 * n * 8, hipMemcpyHostToDevice);
     if (e == hipSuccess) {
