@@ -701,7 +701,12 @@ extern "C" int32_t dps_mle_free(dps_mle *mle)
     if (!mle) return DPS_OK;
     // No wait for the stream: when this was the last handle of its storage the block goes back to the context's pool,
     // whose next user runs on the same stream, after whatever is still queued; a session holds on to the storage of its
-    // tables by itself.
+    // tables by itself.  Memory the caller owns is different: the caller may free or overwrite it once this returns.
+    if (mle->st && !mle->st->owned) {
+        DeviceGuard g(mle->ctx->device);
+        tail_abort(mle->ctx);
+        (void)hipStreamSynchronize(mle->ctx->stream);
+    }
     delete mle;
     return DPS_OK;
 }

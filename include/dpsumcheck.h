@@ -89,7 +89,8 @@ int32_t dps_tensor_from_i16(dps_ctx *ctx, const int16_t *host, uint64_t len, dps
  * stream, no wait. */
 int32_t dps_mle_from_tensor(dps_ctx *ctx, const dps_mle *tensor, const uint64_t *padded_dims, const uint64_t *unpadded_dims,
                             uint32_t n_dims, dps_mle **out);
-/* borrow device memory the caller owns (kind DPS_BASE / DPS_I64 / DPS_I16: d_c1 is NULL) */
+/* borrow device memory the caller owns (kind DPS_BASE / DPS_I64 / DPS_I16: d_c1 is NULL); dps_mle_free of such a
+ * handle waits for the context's queued work, after which the memory is the caller's again */
 int32_t dps_mle_wrap_device(dps_ctx *ctx, int32_t kind, void *d_c0, void *d_c1, uint64_t len, dps_mle **out);
 /* SmartSlice::Borrowed: a window [offset, offset + 2^n_vars) sharing storage */
 int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_vars, dps_mle **out);
