@@ -958,6 +958,11 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
     u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
     bool to_ping = true;  // destination of this round's folded tables
     for (u32 j = a.j0; j <= a.n_vars; j++) {
+        // this thread's eq weight of the round does not depend on the challenge: requested before the wait for the mail,
+        // it is there when the mail is (n_pairs <= BLOCK: a thread has at most one pair per round)
+        const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) : 0;
+        E2 rest_ahead = gl::e2_one();
+        if (EQ && threadIdx.x < n_pairs) rest_ahead = gl::e2(a.eq0[eq_off + threadIdx.x], a.eq1[eq_off + threadIdx.x]);
         if (!tail_wait_mail(a.mail, a.spin_limit, a.seq0 + (j - a.j0), box, &ok_flag)) return;
         const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
         const gl::E2P rp = gl::prep(r);
@@ -965,7 +970,6 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
         E2 acc[NP];
 #pragma unroll
         for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
-        const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) : 0;
         for (u64 i = threadIdx.x; i < n_pairs; i += BLOCK) {
             E2 lo[NF], hi[NF];
 #pragma unroll
@@ -997,7 +1001,7 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
                 d1[2 * i + 1] = hi[f].c1;
             }
             gl::E2P restp = gl::prep(gl::e2_one());
-            if (EQ) restp = gl::prep(gl::e2(a.eq0[eq_off + i], a.eq1[eq_off + i]));
+            if (EQ) restp = gl::prep(i == threadIdx.x ? rest_ahead : gl::e2(a.eq0[eq_off + i], a.eq1[eq_off + i]));
             E2 dl[NF], cur[NF];
 #pragma unroll
             for (int f = 0; f < NF; f++) {
@@ -1417,8 +1421,23 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         cf_seq = seq;
         return true;
     };
+    // The eq weight of a thread's first pair of a round does not depend on the challenge: before a wait for mail it is
+    // requested for the round to come, so that it is there when the mail is (rest_ahead_i: the pair it belongs to).
+    E2 rest_ahead = gl::e2_one();
+    u64 rest_ahead_i = ~(u64)0;
+    auto request_rest = [&](const u64 *e0, const u64 *e1, u64 pairs, u32 split) {
+        rest_ahead_i = ~(u64)0;
+        const u64 pi = (u64)blockIdx.x * (BLOCK >> split) + (tid >> split);
+        if (EQ && pi < pairs) {
+            rest_ahead = gl::e2(e0[pi], e1[pi]);
+            rest_ahead_i = pi;
+        }
+    };
     // launched while the previous round was still running: everything that depends on its challenge comes by mail
-    if (a.wait_first && !take_mail(a.seq, true)) return;
+    if (a.wait_first) {
+        request_rest(q0, q1, n_pairs, sl);
+        if (!take_mail(a.seq, true)) return;
+    }
   for (;;) {
     const PolyGroup &g = gall[j - a.j];
     const u32 n_tabs = g.n_tabs;
@@ -1509,7 +1528,7 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         __syncthreads();
         if (active) {
             gl::E2P restp = gl::prep(gl::e2_one());
-            if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
+            if (EQ) restp = gl::prep(i == rest_ahead_i ? rest_ahead : gl::e2(q0[i], q1[i]));
             // items q = position of the point * n_terms + term; this lane's are sub, sub + S, ...  The point is a
             // run-time value, so the lanes of a wavefront run the same instructions whatever item each one holds.
             constexpr u32 NPE = SKIP1 ? NP - 1 : NP;
@@ -1572,7 +1591,6 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         }
         // stay for the next round: its challenge arrives by mail
         j++;
-        if (!take_mail(a.seq + (j - a.j), false)) return;
         n_pairs >>= 1;
         if (sl < a.split_cap && (n_pairs << (sl + 1)) <= (u64)BLOCK) sl++;
         if (EQ) {
@@ -1580,6 +1598,8 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
             q0 = a.eq0 + off;
             q1 = a.eq1 + off;
         }
+        request_rest(q0, q1, n_pairs, sl);
+        if (!take_mail(a.seq + (j - a.j), false)) return;
         if (a.lds_state) {
             in_lds = wrote;
             dst_is_a = !dst_is_a;
