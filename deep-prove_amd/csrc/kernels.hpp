@@ -957,6 +957,18 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
 
     u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
     bool to_ping = true;  // destination of this round's folded tables
+    // the first round's entries of this thread's pair, requested before the wait for the first mail (the kernel is launched
+    // ahead of its first round; the tables are complete by then, the launch follows their last writer on the stream)
+    U64x2 first[NF][4];
+    if (threadIdx.x < n_pairs) {
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            first[f][0] = ld2(a.s0[f] + 4 * (u64)threadIdx.x);
+            first[f][1] = ld2(a.s0[f] + 4 * (u64)threadIdx.x + 2);
+            first[f][2] = ld2(a.s1[f] + 4 * (u64)threadIdx.x);
+            first[f][3] = ld2(a.s1[f] + 4 * (u64)threadIdx.x + 2);
+        }
+    }
     for (u32 j = a.j0; j <= a.n_vars; j++) {
         // this thread's eq weight of the round does not depend on the challenge: requested before the wait for the mail,
         // it is there when the mail is (n_pairs <= BLOCK: a thread has at most one pair per round)
@@ -976,8 +988,9 @@ __global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
             for (int f = 0; f < NF; f++) {
                 E2 x0, x1, x2, x3;
                 if (j == a.j0) {
-                    U64x2 p0 = ld2(a.s0[f] + 4 * i), q0 = ld2(a.s0[f] + 4 * i + 2);
-                    U64x2 p1 = ld2(a.s1[f] + 4 * i), q1 = ld2(a.s1[f] + 4 * i + 2);
+                    const bool mine = i == threadIdx.x;
+                    U64x2 p0 = mine ? first[f][0] : ld2(a.s0[f] + 4 * i), q0 = mine ? first[f][1] : ld2(a.s0[f] + 4 * i + 2);
+                    U64x2 p1 = mine ? first[f][2] : ld2(a.s1[f] + 4 * i), q1 = mine ? first[f][3] : ld2(a.s1[f] + 4 * i + 2);
                     x0 = gl::e2(p0.x, p1.x);
                     x1 = gl::e2(p0.y, p1.y);
                     x2 = gl::e2(q0.x, q1.x);
