@@ -1447,8 +1447,26 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
         }
     };
     // launched while the previous round was still running: everything that depends on its challenge comes by mail
+    // Likewise the entries of the first table this lane takes in its first step of a launch made ahead (a table that is
+    // folded on the way in, read from device memory): four 16-byte loads that are then not waited for after the mail.
+    U64x2 tab_ahead[4];
+    u64 tab_ahead_i = ~(u64)0;
     if (a.wait_first) {
         request_rest(q0, q1, n_pairs, sl);
+        const u32 sub0 = tid & ((1u << sl) - 1);
+        const u64 pi = (u64)blockIdx.x * (BLOCK >> sl) + (tid >> sl);
+        if (pi < n_pairs && sub0 < gall[0].n_tabs && gall[0].tab[sub0].mode == POLY_PAIR_FOLD) {
+            const PolyTab &tb = gall[0].tab[sub0];
+            tab_ahead[0] = ld2(tb.s0 + 4 * pi);
+            tab_ahead[1] = ld2(tb.s0 + 4 * pi + 2);
+            if (tb.s1) {
+                tab_ahead[2] = ld2(tb.s1 + 4 * pi);
+                tab_ahead[3] = ld2(tb.s1 + 4 * pi + 2);
+            } else {
+                tab_ahead[2] = tab_ahead[3] = U64x2{0, 0};
+            }
+            tab_ahead_i = pi;
+        }
         if (!take_mail(a.seq, true)) return;
     }
   for (;;) {
@@ -1491,12 +1509,14 @@ __global__ void __launch_bounds__(BLOCK) poly_split_kernel(PolyArgs a, u64 *__re
                         y0 = gl::e2(c0[4 * i + 2], c1[4 * i + 2]);
                         y1 = gl::e2(c0[4 * i + 3], c1[4 * i + 3]);
                     } else {
-                        const U64x2 p0 = ld2(tb.s0 + 4 * i), q0v = ld2(tb.s0 + 4 * i + 2);
+                        // (requested before the mail came: the first table of the first step of a launch made ahead)
+                        const bool had = j == a.j && k == sub && i == tab_ahead_i;
+                        const U64x2 p0 = had ? tab_ahead[0] : ld2(tb.s0 + 4 * i), q0v = had ? tab_ahead[1] : ld2(tb.s0 + 4 * i + 2);
                         U64x2 p1 = U64x2{0, 0}, q1v = U64x2{0, 0};
                         ext = tb.s1 != nullptr;
                         if (ext) {
-                            p1 = ld2(tb.s1 + 4 * i);
-                            q1v = ld2(tb.s1 + 4 * i + 2);
+                            p1 = had ? tab_ahead[2] : ld2(tb.s1 + 4 * i);
+                            q1v = had ? tab_ahead[3] : ld2(tb.s1 + 4 * i + 2);
                         }
                         x0 = gl::e2(p0.x, p1.x);
                         x1 = gl::e2(p0.y, p1.y);
