@@ -104,14 +104,19 @@ int32_t fail(dps_ctx *ctx, int32_t code, const char *fmt, ...)
 
 struct DeviceGuard {
     int prev = -1;
+    bool changed = false;
     explicit DeviceGuard(int dev)
     {
         if (hipGetDevice(&prev) != hipSuccess) prev = -1;
-        if (prev != dev) (void)hipSetDevice(dev);
+        if (prev != dev) {
+            (void)hipSetDevice(dev);
+            changed = true;
+        }
     }
     ~DeviceGuard()
     {
-        if (prev >= 0) (void)hipSetDevice(prev);
+        // (nothing to restore in the usual case: a call per round that is not made)
+        if (changed && prev >= 0) (void)hipSetDevice(prev);
     }
 };
 
