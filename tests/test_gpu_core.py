@@ -313,6 +313,20 @@ def test_large_rounds_take_eq_weights_from_two_small_tables(dp, ctx, orc, n, kin
     _check_prove(dp, ctx, orc, n, tabs_gpu, tabs_ref, [(np.array([7, 3], dtype=np.uint64), [e] + list(range(e)))])
 
 
+def test_prepared_prover_gives_the_same_proofs(dp, ctx, orc):
+    """sumcheck_prover marshals handles and terms once; each call is the proof sumcheck_prove gives."""
+    n = 11
+    f, g = rand_base(1 << n, 8200), rand_e2(1 << n, 8201)
+    r = rand_e2(n, 8202)
+    gpu = [ctx.mle_from_base(f), ctx.mle_from_ext2(g), ctx.eq_build(r)]
+    terms = [(ONE, [2, 0, 1])]
+    want = ctx.sumcheck_prove(n, gpu, terms, dp.Transcript(b"p"))
+    prover = ctx.sumcheck_prover(n, gpu, terms)
+    for _ in range(3):
+        got = prover(dp.Transcript(b"p"))
+        assert all((a == b).all() for a, b in zip(got, want))
+
+
 def _materialise_zero_pad(tab, n):
     out = np.zeros((1 << n, 2), dtype=np.uint64)
     out[: tab.shape[0]] = tab
