@@ -1880,7 +1880,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             // the nested form, where it saves products and fits the kernel's staging area
             sc->poly_op_begin.assign(groups.size(), 0);
             sc->poly_op_end.assign(groups.size(), 0);
-            bool use_ops = true;
+            // (only the kernel of the rounds of more than 2^16 pairs runs it: a smaller sum has no use for it)
+            bool use_ops = n_vars >= 1 && (1ull << (n_vars - 1)) > POLY_SPLIT_MAX_PAIRS;
             std::vector<dpk::PolyOp> all_ops;
             u32 plain = 0, nested = 0;
             for (size_t g = 0; g < groups.size() && use_ops; g++) {
