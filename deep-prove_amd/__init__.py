@@ -95,6 +95,8 @@ dev.dps_mle_download.argtypes = [_vp, _vp, _vp]
 dev.dps_mle_free.argtypes = [_vp]
 dev.dps_eq_build.argtypes = [_vp, _vp, _u32, _vp]
 dev.dps_mle_evaluate.argtypes = [_vp, _vp, _vp, _u32, _vp]
+dev.dps_mle_evaluate_noalloc.restype = _i32
+dev.dps_mle_evaluate_noalloc.argtypes = [_vp, _vp, _vp, _u32, _vp]
 dev.dps_mle_fix_low.argtypes = [_vp, _vp, _vp, _u32, _vp]
 dev.dps_mle_fix_high.argtypes = [_vp, _vp, _vp, _u32, _vp]
 dev.dps_partial_eval.argtypes = [_vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _u32, _vp]
@@ -250,6 +252,13 @@ class Mle:
         point = _e2(point).reshape(-1, 2)
         out = np.zeros(2, dtype=np.uint64)
         self.ctx._chk(dev.dps_mle_evaluate(self.ctx._c, self._h, _ptr(point), point.shape[0], _ptr(out)), "dps_mle_evaluate")
+        return out
+
+    def evaluate_noalloc(self, point):
+        """the same value through the entry point that allocates nothing (dps_mle_evaluate_noalloc)"""
+        point = _e2(point).reshape(-1, 2)
+        out = np.zeros(2, dtype=np.uint64)
+        self.ctx._chk(dev.dps_mle_evaluate_noalloc(self.ctx._c, self._h, _ptr(point), point.shape[0], _ptr(out)), "dps_mle_evaluate_noalloc")
         return out
 
     def fix_low(self, point):

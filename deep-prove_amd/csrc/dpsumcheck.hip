@@ -14,6 +14,7 @@
 #include <cstring>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -23,6 +24,12 @@
 using gl::E2;
 using gl::u32;
 using gl::u64;
+
+// Work area of dps_mle_evaluate_noalloc, the one entry point that allocates nothing: eq tables of the two halves of
+// the point, per-workgroup partial sums and a ticket counter (dpk::WS_WORDS words, 144 KiB).  File-scope device
+// memory: every GPU the library runs on holds its own copy, at its own address, until the process ends.  In host
+// code the name below is only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+static __device__ __align__(256) uint64_t scratch[dpk::WS_WORDS];
 
 namespace {
 
@@ -67,6 +74,7 @@ struct dps_ctx {
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
     u64 seq = 0;                // last sequence number handed to a launch
     struct dps_sc *tail_owner = nullptr;  // session whose tail kernel is resident on the stream
+    u64 *ws = nullptr;          // this device's copy of the allocation-free entry point's work area
     bool profiling = false;
     std::vector<ProfRec> recs;
     std::vector<hipEvent_t> ev_pool;
@@ -121,6 +129,26 @@ struct DeviceGuard {
 };
 
 size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Address of `scratch` on a device, asked for once per device with that device current (every GPU has its own copy).
+constexpr int WS_MAX_DEVICES = 64;
+int32_t work_area_of_device(int device, u64 **out)
+{
+    static std::mutex mu;
+    static u64 *ptr_of[WS_MAX_DEVICES] = {};
+    if (device < 0 || device >= WS_MAX_DEVICES) return DPS_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr_of[device]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return DPS_ERR_HIP;
+        }
+        ptr_of[device] = static_cast<u64 *>(p);
+    }
+    *out = ptr_of[device];
+    return DPS_OK;
+}
 
 // A resident tail kernel blocks the stream until its session finishes.  Any other
 // use of the context first makes that kernel exit (its session is then failed).
@@ -372,6 +400,8 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
         return rc;
     };
     if (hipStreamCreate(&ctx->stream) != hipSuccess) return bail(DPS_ERR_HIP);
+    // (the context's device is current here)
+    if (int32_t rc = work_area_of_device(device, &ctx->ws); rc != DPS_OK) return bail(rc);
     // Lagrange weights: a polynomial of degree k known at 0..k, evaluated at t <= 8
     std::vector<u64> lag(9 * 9 * 9, 0);
     for (u32 k = 0; k <= 8; k++)
@@ -2887,6 +2917,71 @@ extern "C" int32_t dps_sc_prove(dps_sc *sc, dps_round_fn fn, void *user, uint64_
         point_out[2 * (j - 1) + 1] = chal[1];
     }
     return dps_sc_finish(sc, sc->n_vars ? chal : nullptr, final_evals_out);
+}
+
+// ---------------------------------------------------------------------------
+// DensePolynomial::evaluate for callers that must not allocate (code under HIP graph capture, tight serving loops):
+// the same value as dps_mle_evaluate, with everything beyond the table and the result kept in `scratch`.
+// No hipMalloc, hipFree, stream wait or host allocation on the way; the result crosses through the context's
+// pinned result area like a round message.
+// ---------------------------------------------------------------------------
+namespace {
+
+template <int KIND>
+void launch_ws_dot(dps_ctx *ctx, bool full, u32 blocks, const void *t0, const u64 *t1, u32 lo, u32 hi, const dpk::FastFin &ff)
+{
+    if (full)
+        dpk::ws_dot_kernel<KIND, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(t0, t1, lo, hi, ctx->ws, ff);
+    else
+        dpk::ws_dot_kernel<KIND, false><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(t0, t1, lo, hi, ctx->ws, ff);
+}
+
+}  // namespace
+
+extern "C" int32_t dps_mle_evaluate_noalloc(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point, uint32_t n, uint64_t out[2])
+{
+    if (!ctx || !mle || !out || (n && !point)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: bad argument");
+    if (mle->ctx != ctx) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: the table belongs to another context");
+    if (mle->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_evaluate_noalloc: the table is a zero-padded view");
+    if (n > 40 || !is_pow2(mle->len) || (1ull << n) != mle->len)
+        return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: point length does not match the table");
+    if (n > dpk::WS_MAX_VARS)
+        return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_mle_evaluate_noalloc: a table of %u variables is beyond the work area's limit of %u (use dps_mle_evaluate)", n,
+                    dpk::WS_MAX_VARS);
+    if (!canonical(point, 2 * (size_t)n)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: point not canonical");
+    if (!ctx->ws) return fail(ctx, DPS_ERR_STATE, "dps_mle_evaluate_noalloc: the context has no work area");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    dpk::WsPoint pt;
+    memset(&pt, 0, sizeof pt);
+    if (n) memcpy(pt.p, point, 16 * (size_t)n);
+    pt.n = n;
+    pt.lo = std::min<u32>(n, dpk::WS_LO_BITS);
+    const u32 lo = pt.lo, hi = n - lo;
+    const u32 eq_entries = (1u << lo) + (1u << hi);
+    dpk::ws_eq_kernel<<<(eq_entries + dpk::BLOCK - 1) / dpk::BLOCK, dpk::BLOCK, 0, ctx->stream>>>(pt, ctx->ws);
+    HIPCHK(ctx, hipGetLastError());
+    const u32 blocks = std::min<u32>(1u << hi, MAX_BLOCKS);
+    static_assert(MAX_BLOCKS <= dpk::WS_MAX_BLOCKS, "one partial per workgroup fits the work area");
+    dpk::FastFin ff;
+    memset(&ff, 0, sizeof ff);
+    ff.partial = ctx->ws + dpk::WS_OFF_PARTIAL;
+    ff.n_blocks = blocks;
+    ff.out_host = ctx->d_pinned + ctx->res_off;
+    ff.seq = ++ctx->seq;
+    ff.counter = reinterpret_cast<u32 *>(ctx->ws + dpk::WS_OFF_COUNTER);
+    const bool full = lo == dpk::WS_LO_BITS;
+    const void *t0 = mle->kind == DPS_I16 ? (const void *)mle->st->c0 : (const void *)mle->p0();
+    // (no timing events here: creating one is an allocation of the runtime's)
+    switch (mle->kind) {
+    case DPS_BASE: launch_ws_dot<0>(ctx, full, blocks, t0, nullptr, lo, hi, ff); break;
+    case DPS_EXT2: launch_ws_dot<1>(ctx, full, blocks, t0, mle->p1(), lo, hi, ff); break;
+    case DPS_I64: launch_ws_dot<8>(ctx, full, blocks, t0, nullptr, lo, hi, ff); break;
+    case DPS_I16: launch_ws_dot<2>(ctx, full, blocks, t0, nullptr, lo, hi, ff); break;
+    default: return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: unknown table kind");
+    }
+    HIPCHK(ctx, hipGetLastError());
+    return wait_result(ctx, ff.seq, 0, 2, out);
 }
 
 // ---------------------------------------------------------------------------

@@ -1823,6 +1823,139 @@ __global__ void __launch_bounds__(BLOCK) axis_dot_row_kernel(AxisArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------
+// evaluation of a table at a point without any memory of its own making: everything beyond the table and the two
+// result words lives in one work area the caller of the kernels passes in (`ws`, WS_WORDS words)
+//
+//   value = sum_h eq_hi[h] * ( sum_l eq_lo[l] * table[h * 2^lo + l] ),   eq_lo over the lo lowest coordinates of the
+// point, eq_hi over the others: two tables of at most 2^WS_LO_BITS entries instead of one of 2^n.  ws_eq_kernel
+// writes them (and zeroes the ticket counter); ws_dot_kernel streams the table once, one row h per workgroup and
+// step, a thread's eq_lo weights staying in registers across its rows, every sum unreduced until its end.
+// ---------------------------------------------------------------------------
+constexpr u32 WS_MAX_VARS = 24;
+constexpr u32 WS_LO_BITS = 12;
+constexpr u32 WS_MAX_BLOCKS = 1024;
+// layout of the work area, in 64-bit words
+constexpr u32 WS_OFF_COUNTER = 0;  // ticket counter (32 bits used)
+constexpr u32 WS_OFF_LO0 = 32, WS_OFF_LO1 = WS_OFF_LO0 + (1u << WS_LO_BITS);
+constexpr u32 WS_OFF_HI0 = WS_OFF_LO1 + (1u << WS_LO_BITS), WS_OFF_HI1 = WS_OFF_HI0 + (1u << WS_LO_BITS);
+constexpr u32 WS_OFF_PARTIAL = WS_OFF_HI1 + (1u << WS_LO_BITS);  // 2 words per workgroup, word-major
+constexpr u32 WS_WORDS = WS_OFF_PARTIAL + 2 * WS_MAX_BLOCKS;
+
+struct WsPoint {
+    u64 p[2 * WS_MAX_VARS];  // 2 limbs per coordinate
+    u32 n, lo;               // coordinates; how many of them eq_lo covers
+};
+
+__global__ void __launch_bounds__(BLOCK) ws_eq_kernel(WsPoint pt, u64 *__restrict__ ws)
+{
+    const u32 i = blockIdx.x * BLOCK + threadIdx.x;
+    // the ticket counter of the launch that follows starts at zero whatever an earlier call left behind
+    if (i == 0) *reinterpret_cast<u32 *>(ws + WS_OFF_COUNTER) = 0;
+    const u32 n_lo = 1u << pt.lo, n_hi = 1u << (pt.n - pt.lo);
+    u32 first, bits, e;
+    u64 *o0, *o1;
+    if (i < n_lo) {
+        first = 0, bits = pt.lo, e = i, o0 = ws + WS_OFF_LO0, o1 = ws + WS_OFF_LO1;
+    } else if (i - n_lo < n_hi) {
+        first = pt.lo, bits = pt.n - pt.lo, e = i - n_lo, o0 = ws + WS_OFF_HI0, o1 = ws + WS_OFF_HI1;
+    } else {
+        return;
+    }
+    E2 acc = gl::e2_one();
+    for (u32 b = 0; b < bits; b++) {
+        const E2 r = gl::e2(pt.p[2 * (first + b)], pt.p[2 * (first + b) + 1]);
+        acc = gl::mul(acc, ((e >> b) & 1) ? r : gl::sub(gl::e2_one(), r));
+    }
+    o0[e] = acc.c0;
+    o1[e] = acc.c1;
+}
+
+// KIND: 0 base-field entries, 1 extension entries, 8 raw int64, 2 raw int16.  FULL: rows of exactly 2^WS_LO_BITS entries
+// (a thread's weights then sit in registers and its loads are 16 bytes wide).
+template <int KIND, bool FULL>
+__global__ void __launch_bounds__(BLOCK) ws_dot_kernel(const void *__restrict__ t0, const u64 *__restrict__ t1, u32 lo, u32 hi, u64 *ws, FastFin ff)
+{
+    __shared__ u32 lds[(BLOCK / WAVE) * 6];
+    __shared__ int last_flag;
+    const u64 *lo0 = ws + WS_OFF_LO0, *lo1 = ws + WS_OFF_LO1, *hi0 = ws + WS_OFF_HI0, *hi1 = ws + WS_OFF_HI1;
+    const u32 rows = 1u << hi, cols = 1u << lo, tid = threadIdx.x;
+    auto entry = [&](u64 i) -> E2 {
+        if (KIND == 8) return gl::e2(gl::from_i64(reinterpret_cast<const int64_t *>(t0)[i]), 0);
+        if (KIND == 2) return gl::e2(gl::from_i64(reinterpret_cast<const int16_t *>(t0)[i]), 0);
+        if (KIND == 1) return gl::e2(reinterpret_cast<const u64 *>(t0)[i], t1[i]);
+        return gl::e2(reinterpret_cast<const u64 *>(t0)[i], 0);
+    };
+    gl::E2Acc total = gl::e2acc_zero();
+    if (FULL) {
+        // columns 2 (tid + BLOCK k), 2 (tid + BLOCK k) + 1 for k = 0..STEPS-1
+        constexpr int STEPS = (1 << WS_LO_BITS) / (2 * BLOCK);
+        E2 w[2 * STEPS];
+#pragma unroll
+        for (int k = 0; k < STEPS; k++) {
+            const U64x2 a = ld2(lo0 + 2 * (tid + BLOCK * k)), b = ld2(lo1 + 2 * (tid + BLOCK * k));
+            w[2 * k] = gl::e2(a.x, b.x);
+            w[2 * k + 1] = gl::e2(a.y, b.y);
+        }
+        for (u32 row = blockIdx.x; row < rows; row += gridDim.x) {
+            const u64 base = (u64)row << WS_LO_BITS;
+            E2 v[2 * STEPS];
+#pragma unroll
+            for (int k = 0; k < STEPS; k++) {
+                const u64 i = base + 2 * (tid + BLOCK * k);
+                if (KIND == 0 || KIND == 1) {
+                    const U64x2 a = ld2(reinterpret_cast<const u64 *>(t0) + i);
+                    U64x2 b = U64x2{0, 0};
+                    if (KIND == 1) b = ld2(t1 + i);
+                    v[2 * k] = gl::e2(a.x, b.x);
+                    v[2 * k + 1] = gl::e2(a.y, b.y);
+                } else {
+                    v[2 * k] = entry(i);
+                    v[2 * k + 1] = entry(i + 1);
+                }
+            }
+            gl::E2Acc a = gl::e2acc_zero();
+#pragma unroll
+            for (int k = 0; k < 2 * STEPS; k++) {
+                if (KIND == 1)
+                    gl::acc_mul(a, v[k], gl::prep(w[k]));
+                else
+                    gl::acc_mul_base(a, w[k], v[k].c0);
+            }
+            gl::acc_mul(total, gl::acc_reduce(a), gl::prep(gl::e2(hi0[row], hi1[row])));
+        }
+    } else {
+        for (u32 row = blockIdx.x; row < rows; row += gridDim.x) {
+            const u64 base = (u64)row << lo;
+            gl::E2Acc a = gl::e2acc_zero();
+            for (u32 l = tid; l < cols; l += BLOCK) {
+                const E2 wv = gl::e2(lo0[l], lo1[l]), v = entry(base + l);
+                if (KIND == 1)
+                    gl::acc_mul(a, v, gl::prep(wv));
+                else
+                    gl::acc_mul_base(a, wv, v.c0);
+            }
+            gl::acc_mul(total, gl::acc_reduce(a), gl::prep(gl::e2(hi0[row], hi1[row])));
+        }
+    }
+    E2 acc[1] = {gl::acc_reduce(total)};
+    block_reduce<1>(acc, lds);
+    if (gridDim.x == 1) {
+        publish_sums<1>(ff.out_host, ff.seq, ff.counter, acc);
+        return;
+    }
+    if (tid == 0) {
+        u64 *o = ws + WS_OFF_PARTIAL + blockIdx.x;
+        st_agent(o, acc[0].c0);
+        st_agent(o + gridDim.x, acc[0].c1);
+    }
+    if (take_ticket(ff.counter, gridDim.x, &last_flag)) {
+        E2 q[1];
+        gather_partials<1>(ff, lds, q);
+        publish_sums<1>(ff.out_host, ff.seq, ff.counter, q);
+    }
+}
+
 // sum the k-slices: out[j] = sum_s in[s * n + j]
 __global__ void __launch_bounds__(BLOCK)
 slice_sum_kernel(const u64 *__restrict__ i0, const u64 *__restrict__ i1, u64 n, u32 n_slices, u64 *__restrict__ o0,

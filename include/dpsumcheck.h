@@ -116,6 +116,13 @@ int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points, const uin
 /* ---- DensePolynomial::{evaluate, fix_low_variables, fix_high_variables}
  *      (zkml/src/layers/einsum/prove.rs:208, zkml/src/tensor/mod.rs:1892, zkml/src/iop/prover.rs:448,509) ---- */
 int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*n */, uint32_t n, uint64_t out[2]);
+/* The same evaluation for callers that cannot allocate.  No counterpart in the reference: it is for code under HIP
+ * graph capture, tight serving loops and harnesses that forbid hipMalloc.  The call makes no hipMalloc, hipFree or
+ * host allocation and waits for no stream; its eq tables, partial sums and ticket counter live in a file-scope
+ * device array of the library (144 KiB per GPU, held until the process ends).  At most 24 variables
+ * (DPS_ERR_UNSUPPORTED beyond).  Every call on one GPU shares that GPU's array: calls that overlap on one GPU,
+ * from this or another context, race. */
+int32_t dps_mle_evaluate_noalloc(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*n */, uint32_t n, uint64_t out[2]);
 /* point[j] binds variable j */
 int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*k */, uint32_t k, dps_mle **out);
 /* point[j] binds variable n-k+j */
