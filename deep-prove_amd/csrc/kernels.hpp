@@ -717,22 +717,10 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ int last_flag;
+    __shared__ u64 box[MAIL_WORDS];  // the mail of a launch made ahead
+    __shared__ int ok_flag;
     E2 r = gl::e2(a.r0, a.r1);
     gl::E2P rp = gl::prep(r);
-    // A launch made ahead of its round waits here for its challenge, with the operands of its first step already
-    // requested (they do not depend on the challenge).  False: no mail came, or the mail asks for the other way of
-    // getting p(1), which is not compiled into this variant; the host then ends the launch.
-    auto take_challenge = [&]() -> bool {
-        __shared__ u64 box[MAIL_WORDS];
-        __shared__ int ok_flag;
-        const bool ok = wait_first_mail(a.mail, a.relay, blockIdx.x == 0, a.spin_limit, ff.seq, SKIP1 ? 0 : 1, box, &ok_flag);
-        if (!ok) return false;
-        if ((box[MAIL_SKIP1] != 0) != SKIP1) return false;
-        // (kept in scalar registers, as the kernel argument would be)
-        r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
-        rp = gl::prep(r);
-        return true;
-    };
     // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
     constexpr bool skip1 = SKIP1;
     // running sums, reduced once after the loop
@@ -743,9 +731,11 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     // Raw operands of one loop step.  The first-round kernel has little arithmetic
     // per byte, so it loads the next step's operands before working on the
     // current ones; the fold kernels are arithmetic-bound and keep one set.
+    // (Members a variant never loads -- the second limbs of base-field sources, the weights without an eq factor -- keep
+    // their zeros and are never read.)
     struct Raw {
-        U64x2 a0[NF], b0[NF], a1[NF], b1[NF];
-        u64 q0, q1;
+        U64x2 a0[NF] = {}, b0[NF] = {}, a1[NF] = {}, b1[NF] = {};
+        u64 q0 = 0, q1 = 0;
     };
     auto load_raw = [&](u64 i, Raw &w) {
 #pragma unroll
@@ -863,7 +853,16 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     if (FOLD) {
         Raw w;
         if (i < a.n_pairs) load_raw(i, w);
-        if (a.wait_first && !take_challenge()) return;
+        if (a.wait_first) {
+            // A launch made ahead of its round waits here for its challenge, with the operands of its first step already
+            // requested (they do not depend on the challenge).  It leaves when no mail comes, or when the mail asks for the
+            // other way of getting p(1), which is not compiled into this variant; the host then ends the launch.
+            if (!wait_first_mail(a.mail, a.relay, blockIdx.x == 0, a.spin_limit, ff.seq, SKIP1 ? 0 : 1, box, &ok_flag)) return;
+            if ((box[MAIL_SKIP1] != 0) != SKIP1) return;
+            // (kept in scalar registers, as the kernel argument would be)
+            r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
+            rp = gl::prep(r);
+        }
         for (; i < a.n_pairs; i += stride) {
             step(i, w);
             if (i + stride < a.n_pairs) load_raw(i + stride, w);

@@ -1,0 +1,229 @@
+// prod_kernel (the fused fold + evaluate kernel of a product sumcheck) run on the CPU: one workgroup at a time, one host
+// thread per lane, through tests/cpp/emu/hip/hip_runtime.h.  Built with the host sanitizers (address, undefined
+// behaviour) and with a fill pattern for uninitialised locals (-ftrivial-auto-var-init=pattern, or =zero for a second
+// opinion): a kernel body that reads something it never wrote then gives sums that differ from build to build and
+// from the sums worked out here with plain loops.  tests/test_kernel_emulation.py builds and runs the quick set; the
+// full set (no argument) takes a few minutes, most of it thread hand-offs.  Covers every way the kernel hands over
+// its result (single workgroup, per-workgroup result areas, partials + ticket + gather), both evaluation modes, the
+// eq weights streamed and taken from two small tables, and a launch that waits for its challenge by mail (directly
+// and through the relay).
+#include <chrono>
+#include <thread>
+#include <vector>
+
+#include "dpsumcheck.h"
+#include "kernels.hpp"
+
+using gl::E2;
+using gl::u32;
+using gl::u64;
+
+static u64 sm_state = 12345;
+static u64 splitmix()
+{
+    sm_state += 0x9E3779B97F4A7C15ull;
+    u64 z = sm_state;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static u64 felt()
+{
+    for (;;) {
+        const u64 v = splitmix();
+        if (v < gl::P) return v;
+    }
+}
+
+template <class K, class... A>
+static void launch(u32 blocks, K kernel, A... args)
+{
+    gridDim = dim3(blocks);
+    blockDim = dim3(dpk::BLOCK);
+    for (u32 b = 0; b < blocks; b++) {
+        emu::block_barrier.reset(dpk::BLOCK);
+        for (int w = 0; w < dpk::BLOCK / dpk::WAVE; w++) emu::wave_barrier[w].reset(dpk::WAVE);
+        std::vector<std::thread> th;
+        for (u32 t = 0; t < (u32)dpk::BLOCK; t++)
+            th.emplace_back([=] {
+                threadIdx = dim3(t);
+                blockIdx = dim3(b);
+                kernel(args...);
+            });
+        for (auto &x : th) x.join();
+    }
+}
+
+static int failures = 0;
+
+struct Case {
+    const char *name;
+    u64 n_pairs;
+    u32 blocks;
+    bool slots;       // per-workgroup result areas
+    int wait;         // 0: challenge in the arguments, 1: by mail, every workgroup polling, 2: by mail through the relay
+};
+
+template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT>
+static void run_case(const Case &c)
+{
+    constexpr int NP = NF + 1;
+    const u64 np = c.n_pairs;
+    const u64 src_len = FOLD ? 4 * np : 2 * np;
+    std::vector<std::vector<u64>> s0(NF), s1(NF), d0(NF), d1(NF);
+    for (int f = 0; f < NF; f++) {
+        s0[f].resize(src_len);
+        for (auto &x : s0[f]) x = felt();
+        if (f >= NB) {
+            s1[f].resize(src_len);
+            for (auto &x : s1[f]) x = felt();
+        }
+        d0[f].assign(2 * np, 0);
+        d1[f].assign(2 * np, 0);
+    }
+    // eq weights: streamed (one per pair), or factored into a low table of 2^16 entries and a high one
+    std::vector<u64> q0, q1, lq0, lq1, hq0, hq1;
+    auto weight = [&](u64 i) -> E2 {
+        if (!EQ) return gl::e2_one();
+        if (FACT) return gl::mul(gl::e2(hq0[i >> dpk::EQ_LO_BITS], hq1[i >> dpk::EQ_LO_BITS]), gl::e2(lq0[i & 65535], lq1[i & 65535]));
+        return gl::e2(q0[i], q1[i]);
+    };
+    if (EQ && FACT) {
+        lq0.resize(65536), lq1.resize(65536);
+        for (auto &x : lq0) x = felt();
+        for (auto &x : lq1) x = felt();
+        const u64 nh = (np + 65535) >> 16;
+        hq0.resize(nh), hq1.resize(nh);
+        for (auto &x : hq0) x = felt();
+        for (auto &x : hq1) x = felt();
+    } else if (EQ) {
+        q0.resize(np), q1.resize(np);
+        for (auto &x : q0) x = felt();
+        for (auto &x : q1) x = felt();
+    }
+    const E2 r = gl::e2(felt(), felt());
+
+    // what the launch has to produce, by plain loops
+    E2 want[NP];
+    for (int t = 0; t < NP; t++) want[t] = gl::e2_zero();
+    std::vector<std::vector<E2>> folded(NF, std::vector<E2>(FOLD ? 2 * np : 0));
+    for (u64 i = 0; i < np; i++) {
+        E2 lo[NF], hi[NF];
+        for (int f = 0; f < NF; f++) {
+            auto at = [&](u64 k) { return gl::e2(s0[f][k], f >= NB ? s1[f][k] : 0); };
+            if (FOLD) {
+                lo[f] = gl::add(at(4 * i), gl::mul(r, gl::sub(at(4 * i + 1), at(4 * i))));
+                hi[f] = gl::add(at(4 * i + 2), gl::mul(r, gl::sub(at(4 * i + 3), at(4 * i + 2))));
+                folded[f][2 * i] = lo[f];
+                folded[f][2 * i + 1] = hi[f];
+            } else {
+                lo[f] = at(2 * i);
+                hi[f] = at(2 * i + 1);
+            }
+        }
+        for (int t = 0; t < NP; t++) {
+            if (t == 1 && SKIP1) continue;
+            E2 prod = weight(i);
+            for (int f = 0; f < NF; f++) prod = gl::mul(prod, gl::add(lo[f], gl::mul_base(gl::sub(hi[f], lo[f]), (u64)t)));
+            want[t] = gl::add(want[t], prod);
+        }
+    }
+
+    dpk::ProdArgs a;
+    memset(&a, 0, sizeof a);
+    for (int f = 0; f < NF; f++) {
+        a.s0[f] = s0[f].data();
+        a.s1[f] = f >= NB ? s1[f].data() : nullptr;
+        a.d0[f] = d0[f].data();
+        a.d1[f] = d1[f].data();
+    }
+    a.q0 = q0.data(), a.q1 = q1.data();
+    a.lq0 = lq0.empty() ? nullptr : lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
+    a.n_pairs = np;
+    a.skip1 = SKIP1;
+    std::vector<u64> mail(64, 0), relay(64, 0), out_host(64, 0), slots(64 * 64, 0), partial(2 * NP * (size_t)c.blocks + 64, 0);
+    u32 counter = 0;
+    const u64 seq = 77;
+    dpk::FastFin ff;
+    memset(&ff, 0, sizeof ff);
+    ff.partial = partial.data();
+    ff.n_blocks = c.blocks;
+    ff.out_host = out_host.data();
+    ff.seq = seq;
+    ff.counter = &counter;
+    ff.slots = c.slots ? slots.data() : nullptr;
+    std::thread host;
+    if (c.wait) {
+        a.wait_first = 1;
+        a.spin_limit = 1u << 30;
+        a.mail = mail.data();
+        a.relay = c.wait == 2 ? relay.data() : nullptr;
+        // the host's side: the mail arrives while the workgroups are waiting (the first of them, run one after the other here)
+        host = std::thread([&] {
+            std::this_thread::sleep_for(std::chrono::milliseconds(30));
+            mail[dpk::MAIL_R] = r.c0;
+            mail[dpk::MAIL_R + 1] = r.c1;
+            mail[dpk::MAIL_SKIP1] = SKIP1;
+            u64 chk = seq;
+            for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
+            mail[dpk::MAIL_CHK] = chk;
+            __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
+        });
+    } else {
+        a.r0 = r.c0, a.r1 = r.c1;
+    }
+    launch(c.blocks, dpk::prod_kernel<NF, NB, FOLD, EQ, SKIP1, FACT>, a, partial.data(), ff);
+    if (host.joinable()) host.join();
+
+    E2 got[NP];
+    for (int t = 0; t < NP; t++) got[t] = gl::e2_zero();
+    bool handed = true;
+    auto take = [&](const u64 *area) {
+        u64 chk = seq;
+        for (int k = 0; k < 2 * NP; k++) chk ^= dpk::rotl64(area[k], k + 1);
+        if (area[dpk::HOST_SEQ_SLOT] != seq || area[dpk::HOST_CHK_SLOT] != chk) handed = false;
+        for (int t = 0; t < NP; t++) got[t] = gl::add(got[t], gl::e2(area[2 * t], area[2 * t + 1]));
+    };
+    if (c.slots && c.blocks > 1)
+        for (u32 b = 0; b < c.blocks; b++) take(slots.data() + 64 * (size_t)b);
+    else
+        take(out_host.data());
+    bool ok = handed && counter == 0;
+    for (int t = 0; t < NP; t++) ok = ok && gl::eq(got[t], want[t]);
+    if (FOLD)
+        for (int f = 0; f < NF && ok; f++)
+            for (u64 k = 0; k < 2 * np && ok; k++) ok = d0[f][k] == folded[f][k].c0 && d1[f][k] == folded[f][k].c1;
+    printf("%-58s NF=%d NB=%d fold=%d eq=%d skip1=%d fact=%d pairs=%llu workgroups=%u : %s\n", c.name, NF, NB, (int)FOLD, (int)EQ, (int)SKIP1, (int)FACT,
+           (unsigned long long)np, c.blocks, ok ? "ok" : "MISMATCH");
+    // the sums are printed so that builds with different fills for uninitialised locals can be compared
+    for (int t = 0; t < NP; t++) printf("    q(%d) = %016llx %016llx\n", t, (unsigned long long)got[t].c0, (unsigned long long)got[t].c1);
+    if (!ok) failures++;
+}
+
+int main(int argc, char **argv)
+{
+    // "quick": without the three-table variants and the two 256-workgroup cases (the suite's CPU run)
+    const bool quick = argc > 1 && !strcmp(argv[1], "quick");
+    // first round (sources read as they are), base-field and mixed sources
+    run_case<2, 2, false, false, false, false>({"first round, single workgroup", 200, 1, false, 0});
+    run_case<2, 2, false, false, false, false>({"first round, ragged pairs, ticket and gather", 5000, 19, false, 0});
+    run_case<2, 1, false, true, false, false>({"first round with streamed eq weights, result areas", 3000, 5, true, 0});
+    if (!quick) run_case<3, 1, false, false, true, false>({"first round, three tables, p(1) from the claim", 777, 2, true, 0});
+    // fold + evaluate
+    run_case<2, 2, true, false, true, false>({"fold of base-field sources", 4100, 18, false, 0});
+    run_case<2, 0, true, false, true, false>({"fold of extension sources", 2500, 3, true, 0});
+    run_case<2, 0, true, true, true, false>({"fold with streamed eq weights", 1000, 1, false, 0});
+    run_case<2, 1, true, true, false, false>({"fold, mixed sources, t = 1 evaluated", 1500, 17, false, 0});
+    run_case<1, 0, true, true, true, false>({"one table times eq", 900, 2, true, 0});
+    if (!quick) run_case<3, 0, true, false, false, false>({"three extension tables", 600, 4, false, 0});
+    // the challenge arrives by mail: every workgroup polls / the first one relays it
+    run_case<2, 0, true, false, true, false>({"launch made ahead, every workgroup polls the mailbox", 1200, 3, true, 1});
+    run_case<2, 2, true, false, true, false>({"launch made ahead, mail relayed by the first workgroup", 4500, 18, false, 2});
+    // eq weights as a product of two small tables (the grid's stride is a multiple of 2^16 pairs)
+    if (!quick) {
+        run_case<2, 2, false, true, false, true>({"first round, eq weights from two small tables", 3ull << 16, 256, false, 0});
+        run_case<2, 2, true, true, true, true>({"fold, eq weights from two small tables", 1ull << 17, 256, false, 0});
+    }
+    printf("%s\n", failures ? "FAILED" : "all cases ok");
+    return failures ? 1 : 0;
+}
