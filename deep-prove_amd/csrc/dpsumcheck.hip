@@ -66,6 +66,7 @@ struct dps_ctx {
     std::vector<u64> h_lagrange;
     u64 h_inv_den[9][9] = {};   // [d][k]: 1 / prod_{m != k, m <= d} (k - m), the Lagrange denominators over the nodes 0..d
     u32 *d_counter = nullptr;   // ticket counter of the evaluation launches; every launch leaves it at zero
+    u64 *d_slice_ctr = nullptr; // sum counters of a resident launch of several workgroups (zero between trips), its ticket behind them
     u64 *h_pinned = nullptr;    // host-visible result buffer
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
@@ -129,6 +130,10 @@ struct DeviceGuard {
 };
 
 size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Behind the Lagrange weights: the ticket counter (and at +128 the words through which a launch's first workgroup
+// passes the mail on), then the sum counters of a resident launch of several workgroups and their ticket.
+constexpr size_t COUNTER_BYTES = 256 + 4 * dpk::SL_MAX_SUMS * 8 + 256;
 
 // Address of `scratch` on a device, asked for once per device with that device current (every GPU has its own copy).
 constexpr int WS_MAX_DEVICES = 64;
@@ -424,10 +429,11 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
             ctx->h_inv_den[d][k] = h_inv(den);
         }
     const size_t lag_bytes = round_up(lag.size() * 8, 256);
-    if (hipMalloc((void **)&ctx->d_lagrange, lag_bytes + 256) != hipSuccess) return bail(DPS_ERR_OOM);
+    if (hipMalloc((void **)&ctx->d_lagrange, lag_bytes + COUNTER_BYTES) != hipSuccess) return bail(DPS_ERR_OOM);
     if (hipMemcpy(ctx->d_lagrange, lag.data(), lag.size() * 8, hipMemcpyHostToDevice) != hipSuccess) return bail(DPS_ERR_HIP);
     ctx->d_counter = (u32 *)((char *)ctx->d_lagrange + lag_bytes);
-    if (hipMemset(ctx->d_counter, 0, 256) != hipSuccess) return bail(DPS_ERR_HIP);
+    ctx->d_slice_ctr = (u64 *)((char *)ctx->d_counter + 256);
+    if (hipMemset(ctx->d_counter, 0, COUNTER_BYTES) != hipSuccess) return bail(DPS_ERR_HIP);
     ctx->pinned_words = 16384;
     if (hipEventCreateWithFlags(&ctx->stage_event, hipEventDisableTiming) != hipSuccess) return bail(DPS_ERR_HIP);
     // fine-grained host memory: a kernel's system-scope stores become visible to the polling host while the kernel runs
@@ -1357,7 +1363,20 @@ struct dps_sc {
     bool have_claim;    // the caller said what the whole sum is
     std::vector<E2> last_msg;
     bool broken;        // its tail kernel was interrupted by another call on the context
-    u32 tail_j0;        // first round run by the resident tail kernel, 0 = none
+    // Resident rounds of a product session (slice_kernel): from round tail_j0 on the tables live in LDS, in one launch of
+    // one workgroup, or a launch of several followed by one of one.  A trip to the GPU covers one round or two.
+    struct Stage {
+        u32 W, j0, pend0, n_trips, dbl_mask, cap;
+        u64 src_len;
+        u64 *h0[3], *h1[3];  // several workgroups: where they leave their last entries (the next stage's source)
+    };
+    std::vector<Stage> stages;
+    std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip
+    E2 prev_chal;                     // the challenge of the call before this one
+    E2 stash[dpk::SL_MAX_SUMS];       // a trip of two rounds: the second round's sums as a polynomial in the first round's challenge
+    u64 last_trip_seq;
+    u32 fin_len;                      // entries per table the last trip leaves to the host (2, or 4 after a trip of two rounds)
+    u32 tail_j0;        // first resident round, 0 = none
     bool tail_running;
     u64 tail_seq0;
     void *scratch;      // one pool block holding every ping-pong buffer
@@ -1421,6 +1440,11 @@ void send_mail(dps_ctx *ctx, u64 seq)
     __atomic_store_n(mb + dpk::MAIL_SEQ, seq, __ATOMIC_RELEASE);
 }
 
+// After launches that were waiting on the GPU have been told to leave (and the stream has drained): the ticket
+// counters and sum counters back to zero, whatever a launch that gave up part-way left in them, and the relayed mail
+// gone -- it says "leave" under a sequence number that the launch made in its place will wait for again.
+void reset_device_words(dps_ctx *ctx) { (void)hipMemsetAsync(ctx->d_counter, 0, COUNTER_BYTES, ctx->stream); }
+
 void tail_abort(dps_ctx *ctx)
 {
     dps_sc *owner = ctx->tail_owner;
@@ -1428,6 +1452,7 @@ void tail_abort(dps_ctx *ctx)
     __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
     (void)hipStreamSynchronize(ctx->stream);
     __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
+    reset_device_words(ctx);
     owner->tail_running = false;
     // a launch that has had no mail yet has changed nothing: its session goes on with ordinary launches
     if (owner->wait_fresh)
@@ -1438,10 +1463,13 @@ void tail_abort(dps_ctx *ctx)
     ctx->tail_owner = nullptr;
 }
 
+// result area of the resident product launches (dpk::SL_AREA_WORDS words of the pinned buffer, behind the areas of resident groups)
+size_t slice_area_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64 + 64 * 32; }
+
 template <int NF, bool EQ>
-void launch_tail(dps_ctx *ctx, const dpk::TailArgs &a)
+void launch_slice(dps_ctx *ctx, u32 workgroups, u32 cap, const dpk::SliceArgs &a)
 {
-    dpk::tail_kernel<NF, EQ><<<1, dpk::BLOCK, 0, ctx->stream>>>(a);
+    dpk::slice_kernel<NF, EQ><<<workgroups, dpk::BLOCK, dpk::slice_lds_words(NF, cap) * 8, ctx->stream>>>(a);
 }
 
 template <int NF, int NB, bool EQ>
@@ -1517,6 +1545,7 @@ int32_t launch_poly_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, const dp
 
 // Several groups resident side by side publish into 64-word slots of the pinned buffer from here on
 constexpr u32 POLY_RAW_MAX_GROUPS = 32;
+static_assert(POLY_RAW_MAX_GROUPS == 32, "slice_area_off lies behind the result areas of the resident groups");
 size_t poly_raw_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64; }
 // a launch of this many workgroups publishes per workgroup (FastFin::slots) rather than through the last one
 constexpr u32 SLOT_MAX_WORKGROUPS = 16;
@@ -1712,6 +1741,64 @@ int32_t ensure_descs(dps_sc *sc)
     if (e != hipSuccess) return fail(sc->ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e));
     sc->descs_uploaded = true;
     return DPS_OK;
+}
+
+}  // namespace
+
+namespace {
+
+// pairs a workgroup of a resident launch takes in its first round (its LDS holds twice as many entries per table, and half of that again)
+u32 slice_pairs_per_workgroup(u32 nf) { return nf <= 2 ? 512 : 256; }
+constexpr u32 SLICE_MAX_WORKGROUPS = 256;
+
+// Which rounds of a product session are resident, in which launches, and how they pair up into trips.  `first_ok`: the
+// first round whose source tables are extension tables.  A trip covers two rounds when the second one's p(1) can come
+// from the claim (its eq coordinate is not zero) and the workgroups still hold a quad each.
+void plan_resident_rounds(dps_sc *sc, u32 first_ok)
+{
+    const u32 n = sc->n_vars, nf = sc->fast_nf;
+    const bool has_eq = sc->fast_eq >= 0;
+    if (first_ok > n) return;
+    auto claim_gives_p1 = [&](u32 round) {
+        if (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0) return false;
+        if (!has_eq) return true;
+        const E2 rho = sc->eq_info->point[round - 1];
+        return !(rho.c0 == 0 && rho.c1 == 0);
+    };
+    const u32 per_wg = slice_pairs_per_workgroup(nf);
+    auto pairs_of = [&](u32 round) { return (u64)1 << (n - round); };
+    u32 j = first_ok;
+    while (pairs_of(j) > (u64)per_wg * SLICE_MAX_WORKGROUPS) j++;
+    sc->tail_j0 = j;
+    u64 entries = (u64)1 << (n - j + 2);  // of the tables the stage to come starts from (before its pending folds)
+    u32 pend = 1;
+    auto add_stage = [&](u32 W) {
+        dps_sc::Stage st;
+        memset(&st, 0, sizeof st);
+        st.W = W;
+        st.j0 = j;
+        st.pend0 = pend;
+        st.src_len = entries;
+        u64 len = (entries / W) >> pend;  // entries per table and workgroup in the trip's first round
+        st.cap = (u32)len;
+        for (;;) {
+            const bool dbl = len >= 4 && j + 1 <= n && claim_gives_p1(j + 1);
+            if (dbl) st.dbl_mask |= 1u << st.n_trips;
+            st.n_trips++;
+            sc->round_kind[j] = dbl ? 2 : 1;
+            if (dbl) sc->round_kind[j + 1] = 3;
+            pend = dbl ? 2 : 1;
+            j += pend;
+            // several workgroups go on while each still has a pair after the pending folds; one goes on to the last round
+            if (j > n || (W > 1 && (len >> pend) < 2) || st.n_trips == (u32)dpk::SL_MAX_TRIPS) break;
+            len >>= pend;
+        }
+        entries = len * W;
+        sc->fin_len = (u32)len;
+        sc->stages.push_back(st);
+    };
+    if (pairs_of(j) > per_wg) add_stage((u32)(pairs_of(j) / per_wg));
+    while (j <= n) add_stage(1);
 }
 
 }  // namespace
@@ -1957,11 +2044,14 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         CHK(eq_build_low(ctx, *sc->eq_info, const_cast<u64 *>(sc->eq_c0), const_cast<u64 *>(sc->eq_c1)));
         sc->eq_info->fact_built = true;
     }
+    sc->round_kind.assign(n_vars + 2, 0);
+    sc->last_trip_seq = 0;
+    sc->fin_len = 0;
+    sc->prev_chal = gl::e2_zero();
     if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
-        const u32 j0 = n_vars > 10 ? n_vars - 8 : 2;
         bool all_ext = true;
         for (u32 f = 0; f < sc->fast_nf; f++) all_ext = all_ext && mles[sc->fast_order[f]]->kind == DPS_EXT2;
-        if (j0 >= 3 || all_ext) sc->tail_j0 = j0;
+        plan_resident_rounds(sc.get(), all_ext ? 2 : 3);
     }
 
     // scratch: two ping-pong buffers per table, extension limbs
@@ -2188,7 +2278,10 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     size_t bytes_pg = round_up(poly_groups.size() * sizeof(dpk::PolyGroup), 256);
     size_t bytes_pt = round_up(poly_terms.size() * sizeof(dpk::PolyTerm), 256);
     size_t bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
-    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result;
+    // what a resident stage that does not run to the last round leaves for the next: two limb arrays per table
+    size_t bytes_hand = 0;
+    for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * sc->fast_nf;
+    size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result + bytes_hand;
     int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
     if (rc != DPS_OK) return cleanup(rc);
     char *p = (char *)sc->dev_block;
@@ -2211,6 +2304,16 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->d_partial = (u64 *)p;
     p += bytes_partial;
     sc->d_result = (u64 *)p;
+    p += bytes_result;
+    for (size_t i = 0; i + 1 < sc->stages.size(); i++) {
+        const size_t limb = round_up((size_t)sc->stages[i + 1].src_len * 8, 256);
+        for (u32 f = 0; f < sc->fast_nf; f++) {
+            sc->stages[i].h0[f] = (u64 *)p;
+            p += limb;
+            sc->stages[i].h1[f] = (u64 *)p;
+            p += limb;
+        }
+    }
     sc->d_counter = ctx->d_counter;
     // one staged upload of all descriptors
     std::vector<char> &stage = sc->stage;  // lives as long as the session: the upload is not waited for
@@ -2457,6 +2560,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             u64 *mb = mailbox(ctx);
             mb[dpk::MAIL_R] = a.r0;
             mb[dpk::MAIL_R + 1] = a.r1;
+            mb[dpk::MAIL_RA] = sc->prev_chal.c0;
+            mb[dpk::MAIL_RA + 1] = sc->prev_chal.c1;
             mb[dpk::MAIL_SKIP1] = a.skip1;
             send_mail(ctx, fa.seq);
         };
@@ -2464,21 +2569,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         // of their own -- resident groups, or the workgroups of a small launch -- which are added) and
         // forms the message: p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was skipped; with an eq factor
         // p(nf + 1) by extrapolation of q (coefficients above).
-        auto take_sums = [&](u32 n_slots) -> int32_t {
-            prepare_message();
+        // the message from the sums q(0..nf) (prepare_message has run)
+        auto form_message = [&](const E2 *q) {
             const u32 np = nf + 1;
-            E2 q[dpk::MAX_PTS];
-            u64 w[2 * dpk::MAX_PTS];
-            if (n_slots) {
-                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
-                for (u32 g = 0; g < n_slots; g++) {
-                    CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
-                    for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
-                }
-            } else {
-                CHK(wait_result(ctx, fa.seq, 0, 2 * np, w));
-                for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
-            }
             E2 msg[dpk::MAX_PTS + 1];
             for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(hf.scale[2 * t], hf.scale[2 * t + 1]), q[t]), cst);
             if (a.skip1) msg[1] = gl::sub(sc->claim, msg[0]);
@@ -2494,6 +2587,23 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 evals_out[2 * t + 1] = msg[t].c1;
                 sc->last_msg[t] = msg[t];
             }
+        };
+        auto take_sums = [&](u32 n_slots) -> int32_t {
+            prepare_message();
+            const u32 np = nf + 1;
+            E2 q[dpk::MAX_PTS];
+            u64 w[2 * dpk::MAX_PTS];
+            if (n_slots) {
+                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+                for (u32 g = 0; g < n_slots; g++) {
+                    CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
+                    for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
+                }
+            } else {
+                CHK(wait_result(ctx, fa.seq, 0, 2 * np, w));
+                for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
+            }
+            form_message(q);
             return DPS_OK;
         };
         // A launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an earlier
@@ -2505,6 +2615,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
             HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
             __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
+            reset_device_words(ctx);
             sc->tail_running = false;
             sc->wait_fresh = false;
             ctx->tail_owner = nullptr;
@@ -2514,31 +2625,48 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         if (sc->tail_running && sc->wait_fresh &&
             std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS))
             CHK(end_waiting_launch());
-        // the launch of the tail kernel, whose first round is j0 and has the sequence number seq0
-        auto launch_tail_at = [&](u32 j0, u64 seq0) -> int32_t {
-            const dpk::ProdArgs &a0 = sc->fast_args[j0];
-            dpk::TailArgs ta;
-            memset(&ta, 0, sizeof ta);
-            for (u32 f = 0; f < nf; f++) {
-                ta.s0[f] = a0.s0[f];
-                ta.s1[f] = a0.s1[f];
+        // The launches of the resident rounds, queued one behind the other: the trip that starts at the first resident
+        // round has the sequence number seq0 (a round's call takes one number whether or not it makes a trip).
+        auto launch_stages_at = [&](u64 seq0) -> int32_t {
+            const u32 first = sc->tail_j0;
+            for (size_t si = 0; si < sc->stages.size(); si++) {
+                const dps_sc::Stage &st = sc->stages[si];
+                dpk::SliceArgs sa;
+                memset(&sa, 0, sizeof sa);
+                for (u32 f = 0; f < nf; f++) {
+                    // the first stage reads what the launch of the round before it wrote (or the session's own tables)
+                    sa.s0[f] = si == 0 ? sc->fast_args[first].s0[f] : sc->stages[si - 1].h0[f];
+                    sa.s1[f] = si == 0 ? sc->fast_args[first].s1[f] : sc->stages[si - 1].h1[f];
+                    sa.h0[f] = st.h0[f];
+                    sa.h1[f] = st.h1[f];
+                }
+                sa.src_len = st.src_len;
+                sa.pend0 = st.pend0;
+                sa.n_vars = sc->n_vars;
+                sa.j0 = st.j0;
+                sa.n_trips = st.n_trips;
+                sa.dbl_mask = st.dbl_mask;
+                sa.eq0 = sc->eq_c0;
+                sa.eq1 = sc->eq_c1;
+                sa.mail = ctx->d_pinned + (ctx->res_off - 64);
+                // (several workgroups: the first polls the host's mailbox and passes each mail on through device memory; with
+                // all 256 of them polling host memory a trip took 90 us instead of 18)
+                sa.relay = mail_relay(ctx);
+                sa.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
+                sa.finish = si + 1 == sc->stages.size() ? 1 : 0;
+                sa.out_host = ctx->d_pinned + slice_area_off(ctx);
+                sa.seq0 = seq0 + (st.j0 - first);
+                sa.ctr = ctx->d_slice_ctr;
+                sa.ticket = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
+                ProfScope ps(ctx, DPS_K_TAIL, 0.0);
+                if (has_eq && nf == 1) launch_slice<1, true>(ctx, st.W, st.cap, sa);
+                else if (has_eq && nf == 2) launch_slice<2, true>(ctx, st.W, st.cap, sa);
+                else if (!has_eq && nf == 2) launch_slice<2, false>(ctx, st.W, st.cap, sa);
+                else if (!has_eq && nf == 3) launch_slice<3, false>(ctx, st.W, st.cap, sa);
+                else return fail(ctx, DPS_ERR_UNSUPPORTED, "no resident kernel for %u tables, eq %d", nf, (int)has_eq);
+                HIPCHK(ctx, hipGetLastError());
             }
-            ta.eq0 = sc->eq_c0;
-            ta.eq1 = sc->eq_c1;
-            ta.n_vars = sc->n_vars;
-            ta.j0 = j0;
-            ta.mail = ctx->d_pinned + (ctx->res_off - 64);
-            ta.out_host = fa.out_host;
-            ta.seq0 = seq0;
             sc->tail_seq0 = seq0;
-            ta.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
-            ProfScope ps(ctx, DPS_K_TAIL, 0.0);
-            if (has_eq && nf == 1) launch_tail<1, true>(ctx, ta);
-            else if (has_eq && nf == 2) launch_tail<2, true>(ctx, ta);
-            else if (!has_eq && nf == 2) launch_tail<2, false>(ctx, ta);
-            else if (!has_eq && nf == 3) launch_tail<3, false>(ctx, ta);
-            else return fail(ctx, DPS_ERR_UNSUPPORTED, "no tail kernel for %u tables, eq %d", nf, (int)has_eq);
-            HIPCHK(ctx, hipGetLastError());
             sc->tail_running = true;
             sc->wait_any_skip1 = true;
             sc->wait_slots = 0;
@@ -2546,18 +2674,61 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             return DPS_OK;
         };
         if (sc->tail_j0 && j >= sc->tail_j0) {
-            if (!sc->tail_running) {
-                if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
-                CHK(launch_tail_at(j, fa.seq));
+            const u32 kind = sc->round_kind[j];
+            const u32 np = nf + 1;
+            E2 q[dpk::MAX_PTS];
+            int32_t rc = DPS_OK;
+            if (kind == 3) {
+                // Second round of a trip: the kernel handed over this round's sums as a polynomial in the challenge that has
+                // now been drawn (values at 0..nf-1 and the leading coefficient, per point t = 0, 2, .., nf); p(1) comes
+                // from the claim.  Nothing goes to the GPU.
+                const E2 r = gl::e2(challenge[0], challenge[1]);
+                E2 vanish = gl::e2_one(), basis[dpk::MAX_PTS];
+                for (u32 k = 0; k < nf; k++) {
+                    E2 num = gl::e2_one();
+                    for (u32 m = 0; m < nf; m++)
+                        if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+                    basis[k] = gl::mul_base(num, ctx->h_inv_den[nf - 1][k]);
+                    vanish = gl::mul(vanish, gl::sub(r, gl::e2(k, 0)));
+                }
+                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+                for (u32 ti = 0; ti < nf; ti++) {
+                    E2 v = gl::mul(vanish, sc->stash[nf * nf + ti]);
+                    for (u32 k = 0; k < nf; k++) v = gl::add(v, gl::mul(basis[k], sc->stash[k * nf + ti]));
+                    q[ti == 0 ? 0 : ti + 1] = v;
+                }
+                prepare_message();
+                form_message(q);
+            } else {
+                if (!sc->tail_running) {
+                    if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
+                    CHK(launch_stages_at(fa.seq));
+                }
+                post_mail();
+                sc->wait_fresh = false;
+                prepare_message();
+                // sums of this round, and with a trip of two rounds those of the next
+                const u32 ns = kind == 2 ? np + np * nf : np;
+                u64 w[2 * dpk::SL_MAX_SUMS];
+                rc = wait_result_at(ctx, slice_area_off(ctx), fa.seq, 0, 2 * ns, w, dpk::SL_SEQ_SLOT, dpk::SL_CHK_SLOT);
+                if (rc == DPS_OK) {
+                    for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
+                    for (u32 i = np; i < ns; i++) sc->stash[i - np] = gl::e2(w[2 * i], w[2 * i + 1]);
+                    form_message(q);
+                    sc->last_trip_seq = fa.seq;
+                }
             }
-            post_mail();
-            sc->wait_fresh = false;
-            const int32_t rc = take_sums(0);
+            if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
             if (j == sc->n_vars || rc != DPS_OK) {
-                // with its last round the kernel publishes the tables' last pairs and exits
+                // with its last trip the kernel publishes what is left of the tables and exits
                 sc->tail_running = false;
                 ctx->tail_owner = nullptr;
-                if (rc == DPS_OK) sc->pairs_seq = fa.seq;
+                if (rc == DPS_OK) sc->pairs_seq = sc->last_trip_seq;
+            }
+            if (rc != DPS_OK) {
+                // the launch left without publishing (it gave up waiting, or the stream failed): nothing of it can be used again
+                sc->broken = true;
+                reset_device_words(ctx);
             }
             CHK(rc);
             sc->round = j;
@@ -2724,6 +2895,11 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 }
             }
             int32_t rc = take_sums(slots_now);
+            if (rc != DPS_OK) {
+                // a launch that left without publishing may have taken some of its tickets and written some of its tables
+                sc->broken = true;
+                reset_device_words(ctx);
+            }
             if (stays && (rc != DPS_OK || j == sc->n_vars)) {
                 // a resident launch exits after the last round; one that can finish has published the tables' last pairs with it
                 sc->tail_running = false;
@@ -2762,7 +2938,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u64 next_seq = ctx->seq + 1;
             bool made = false;
             if (sc->tail_j0 && j + 1 == sc->tail_j0) {
-                CHK(launch_tail_at(j + 1, next_seq));
+                CHK(launch_stages_at(next_seq));
                 made = true;
             } else {
                 // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
@@ -2798,7 +2974,12 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 ctx->tail_owner = sc;
             }
         }
-        CHK(take_sums(slots_now));
+        if (const int32_t rc = take_sums(slots_now); rc != DPS_OK) {
+            sc->broken = true;
+            reset_device_words(ctx);
+            return rc;
+        }
+        if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
         sc->round = j;
         return DPS_OK;
     } else {
@@ -2833,7 +3014,21 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         u64 w[4 * dpk::POLY_MAXT];
         // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
         // groups are resident), the single-product one its factors
-        const u32 n_areas = sc->poly ? (u32)sc->poly_tabs.size() : 1;
+        if (!sc->poly) {
+            // a product session: the resident launch left 2 entries per table, or 4 when its last trip covered two rounds
+            // (the challenge between them is the one the last round's call brought)
+            const u32 L = sc->fin_len;
+            CHK(wait_result_at(ctx, slice_area_off(ctx), sc->pairs_seq, dpk::SL_FIN_SLOT, 2 * L * sc->fast_nf, w, dpk::SL_FIN_SEQ_SLOT, dpk::SL_FIN_CHK_SLOT));
+            for (u32 f = 0; f < sc->fast_nf; f++) {
+                auto at = [&](u32 e) { return gl::e2(w[2 * (f * L + e)], w[2 * (f * L + e) + 1]); };
+                auto fold = [](E2 lo, E2 hi, E2 c) { return gl::add(lo, gl::mul(c, gl::sub(hi, lo))); };
+                const E2 v = L == 4 ? fold(fold(at(0), at(1), sc->prev_chal), fold(at(2), at(3), sc->prev_chal), r) : fold(at(0), at(1), r);
+                const u32 k = sc->fast_order[f];
+                final_evals_out[2 * k] = v.c0;
+                final_evals_out[2 * k + 1] = v.c1;
+            }
+        }
+        const u32 n_areas = sc->poly ? (u32)sc->poly_tabs.size() : 0;
         for (u32 g = 0; g < n_areas; g++) {
             const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[g].size() : sc->fast_nf;
             const size_t base = sc->poly_raw ? poly_raw_off(ctx) + 64 * (size_t)g : ctx->res_off;

@@ -534,7 +534,11 @@ eval_terms_kernel(const TermDesc *__restrict__ terms, u64 *__restrict__ partial,
 // their first, and by launches made ahead of their round for the first one as well.
 // ---------------------------------------------------------------------------
 // mailbox words; MAIL_SEQ == MAIL_ABORT_SEQ tells the kernel to exit
-constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_WORDS = 5;
+// MAIL_R: the challenge of the round before the one the mail starts; MAIL_RA: the one before that (read by a kernel
+// that has two folds pending because its last result covered two rounds).  MAIL_SKIP1: 0 / 1, or MAIL_SKIP1_LEAVE when
+// the first workgroup of a launch passes on that no mail came.
+constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_RA = 5, MAIL_WORDS = 7;
+constexpr u64 MAIL_SKIP1_LEAVE = 2;
 static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
 constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
 
@@ -587,8 +591,9 @@ __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, boo
 #pragma unroll
         for (int k = 0; k < MAIL_WORDS; k++) w[k] = box[k];
         if (!ok) {
+#pragma unroll
+            for (int k = 0; k < MAIL_WORDS; k++) w[k] = 0;
             w[MAIL_SEQ] = seq;
-            w[MAIL_R] = w[MAIL_R + 1] = 0;
             w[MAIL_SKIP1] = reject_skip1;
             w[MAIL_CHK] = seq ^ mail_mix(reject_skip1, MAIL_SKIP1);
         }
@@ -919,145 +924,329 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 }
 
 // ---------------------------------------------------------------------------
-// tail kernel: the last rounds of a product sumcheck in one launch
+// slice kernel: the rounds of a product sumcheck that are latency, not bytes
 //
-// Once a round has at most TAIL_PAIRS pairs a launch per round is pure latency
-// (dispatch, a single wavefront's instruction stream, the result hand-off).  One
-// workgroup then stays resident for all remaining rounds: the tables live in LDS,
-// each round's message goes to host-visible memory as before, and the workgroup
-// waits for the next challenge in a mailbox the host writes (fine-grained pinned
-// memory, system-scope loads).  The wait is bounded: without mail the kernel
-// gives up after `spin_limit` polls and exits.
+// Once a round moves a few megabytes a launch per round is pure latency (dispatch, a wavefront's instruction stream,
+// the hand-off to the host and back).  From there on the tables live in LDS: every workgroup of this launch owns a
+// contiguous slice of every table -- binding the lowest variable turns entries 2i, 2i+1 into entry i, so what a
+// workgroup needs in the next round is what it has just made -- and stays on the GPU, waiting for each challenge in
+// the host's mailbox.  With one workgroup it runs to the last round; with several it runs until a workgroup is down to
+// an entry or two per table, leaves them in device memory (`h0/h1`) and a single-workgroup launch queued behind it goes on.
+//
+// A trip to the host can cover two rounds.  With S the state of round j (pairs (S[2i], S[2i+1])), the tables of round
+// j+1 are S[2i] + r_j (S[2i+1] - S[2i]): linear in the challenge r_j that is not known yet, so the sums of round j+1
+//     q_{j+1}(t) = sum_x R_{j+1}(x) prod_f f_{j+1}(t, x)
+// are a polynomial of degree NF in r_j.  Besides q_j(t) the kernel hands over that polynomial's values at r_j = 0..NF-1
+// and its leading coefficient (each is the same sum over quads of S with the pair (S[4i], S[4i+2]), (S[4i+1], S[4i+3]),
+// ... or the differences in place of the folded pair).  The host draws r_j from message j, evaluates the polynomial
+// there, forms message j+1 and draws r_{j+1} without the GPU; the next mail carries both challenges and the kernel
+// folds twice.  Same field elements as one round at a time; half the trips.
+//
+// Sums are added up as plain integers: a lane's canonical sums are cut into 32-bit halves and added into 64-bit
+// counters, per wavefront in LDS, then per launch in device memory (agent-scope atomics, one ticket per workgroup);
+// whoever takes the last ticket recombines and publishes.
 // ---------------------------------------------------------------------------
-constexpr int TAIL_PAIRS = 256;
-struct TailArgs {
+constexpr int SL_MAX_SUMS = 16;  // (NF + 1)^2 extension sums per trip at NF = 3
+constexpr int SL_SEQ_SLOT = 2 * SL_MAX_SUMS, SL_CHK_SLOT = SL_SEQ_SLOT + 1;
+// with the last trip of a run to the last round: the entries every table still has (2, or 4 after a trip of two rounds)
+constexpr int SL_FIN_SLOT = 40, SL_FIN_SEQ_SLOT = 64, SL_FIN_CHK_SLOT = 65, SL_AREA_WORDS = 128;
+constexpr int SL_MAX_TRIPS = 32;
+struct SliceArgs {
     const u64 *s0[3];
-    const u64 *s1[3];  // extension tables of the first tail round, 4 * n_pairs0 entries each
-    const u64 *eq0;    // eq storage (level 0 at entry 0), eq factor only
+    const u64 *s1[3];  // the tables before the folds that are pending when the launch starts: src_len entries each
+    u64 src_len;
+    u32 pend0;         // folds pending at the first trip: 1 (the challenge of the round before), or 2
+    u32 n_vars, j0;    // the sum's variables; first round evaluated here (1-based)
+    u32 n_trips;
+    u32 dbl_mask;      // bit k: trip k covers two rounds
+    const u64 *eq0;    // eq storage, level 0 at entry 0 (eq factor only)
     const u64 *eq1;
-    u32 n_vars, j0;    // the sum's variables, first round handled here (1-based)
-    const u64 *mail;   // host mailbox, MAIL_WORDS words
-    u64 *out_host;     // the sums q(t), HOST_SEQ_SLOT, HOST_FINALS_SLOT
-    u64 seq0;          // sequence number of round j0; round j uses seq0 + (j - j0), the final evaluations seq0 + (n_vars - j0 + 1)
+    const u64 *mail;   // host mailbox
+    u64 *relay;        // several workgroups: the first passes each mail on through these words of device memory
     u32 spin_limit;
+    u32 finish;        // a single workgroup that runs to the last round: the remaining entries go to the host with the last
+                       // trip; else they go to h0 / h1
+    u64 *out_host;     // result area of SL_AREA_WORDS words
+    u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
+    u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero between trips
+    u32 *ticket;       // ... and their ticket counter
+    u64 *h0[3];        // not finishing: where each workgroup leaves its last state (workgroup-major), to be folded by the next launch
+    u64 *h1[3];
 };
 
-template <int NF, bool EQ>
-__global__ void __launch_bounds__(BLOCK) tail_kernel(TailArgs a)
-{
-    constexpr int NP = NF + 1;
-    // ping: tables after the first tail round (2 * TAIL_PAIRS entries), pong: half of that
-    __shared__ u64 ping[NF][2][2 * TAIL_PAIRS];
-    __shared__ u64 pong[NF][2][TAIL_PAIRS];
-    __shared__ u64 box[MAIL_WORDS];
-    __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
-    __shared__ u64 res[6 * MAX_PTS];
-    __shared__ int ok_flag;
+// dynamic LDS of slice_kernel, in 64-bit words: counters per wavefront, mailbox copy, flags, then the two table buffers
+constexpr u32 SL_LDS_CTR = 0, SL_LDS_BOX = (BLOCK / WAVE) * 4 * SL_MAX_SUMS, SL_LDS_FLAGS = SL_LDS_BOX + 8, SL_LDS_TABLES = SL_LDS_FLAGS + 2;
+__host__ __device__ constexpr u32 slice_lds_words(u32 nf, u32 cap) { return SL_LDS_TABLES + nf * 2 * (cap + cap / 2); }
 
-    u64 n_pairs = (u64)1 << (a.n_vars - a.j0);
-    bool to_ping = true;  // destination of this round's folded tables
-    // the first round's entries of this thread's pair, requested before the wait for the first mail (the kernel is launched
-    // ahead of its first round; the tables are complete by then, the launch follows their last writer on the stream)
-    U64x2 first[NF][4];
-    if (threadIdx.x < n_pairs) {
-#pragma unroll
-        for (int f = 0; f < NF; f++) {
-            first[f][0] = ld2(a.s0[f] + 4 * (u64)threadIdx.x);
-            first[f][1] = ld2(a.s0[f] + 4 * (u64)threadIdx.x + 2);
-            first[f][2] = ld2(a.s1[f] + 4 * (u64)threadIdx.x);
-            first[f][3] = ld2(a.s1[f] + 4 * (u64)threadIdx.x + 2);
-        }
-    }
-    for (u32 j = a.j0; j <= a.n_vars; j++) {
-        // this thread's eq weight of the round does not depend on the challenge: requested before the wait for the mail,
-        // it is there when the mail is (n_pairs <= BLOCK: a thread has at most one pair per round)
-        const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) : 0;
-        E2 rest_ahead = gl::e2_one();
-        if (EQ && threadIdx.x < n_pairs) rest_ahead = gl::e2(a.eq0[eq_off + threadIdx.x], a.eq1[eq_off + threadIdx.x]);
-        if (!tail_wait_mail(a.mail, a.spin_limit, a.seq0 + (j - a.j0), box, &ok_flag)) return;
-        const E2 r = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
-        const gl::E2P rp = gl::prep(r);
+template <int NF, bool EQ>
+__global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
+{
+    constexpr int NP = NF + 1;          // sums of the trip's first round: q(0..NF), q(1) left zero when it comes from the claim
+    constexpr int NPT = NF;             // points of its second round: t = 0, 2, .., NF
+    constexpr int NSMP = NF + 1;        // samples of that round's sums as a polynomial in the challenge: 0..NF-1, leading coefficient
+    constexpr int NS = NP + NSMP * NPT; // extension sums per trip
+    static_assert(NS <= SL_MAX_SUMS, "sums per trip fit the result area");
+    extern __shared__ u64 dyn[];
+    u64 *const ctr = dyn + SL_LDS_CTR;  // [wavefront][4 * SL_MAX_SUMS]
+    u64 *const box = dyn + SL_LDS_BOX;
+    int *const ok_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS);
+    int *const last_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS + 1);
+    const u32 tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const u32 W = gridDim.x, wg = blockIdx.x;
+    const u64 src_wg = a.src_len / W;             // this workgroup's share of the source
+    u32 len = (u32)(src_wg >> a.pend0);           // entries per table once the pending folds are done
+    const u32 cap = len;
+    // two buffers per limb array: `cap` entries and half of that; a fold reads one and writes the other
+    u64 *const buf_big = dyn + SL_LDS_TABLES, *const buf_small = buf_big + (size_t)NF * 2 * cap;
+    bool in_big = true;  // where the current state is
+    auto tab = [&](bool big, int f, int limb) -> u64 * { return big ? buf_big + (size_t)(f * 2 + limb) * cap : buf_small + (size_t)(f * 2 + limb) * (cap / 2); };
+
+    u32 j = a.j0, pend = a.pend0;
+    u64 trip_seq = a.seq0;
+    for (u32 k = 0; k < a.n_trips; k++) {
+        const bool dbl = (a.dbl_mask >> k) & 1;
+        trip_seq = a.seq0 + (j - a.j0);
+        if (!wait_first_mail(a.mail, W > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
+        if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
         const bool skip1 = box[MAIL_SKIP1] != 0;
-        E2 acc[NP];
+        const gl::E2P rb = gl::prep(gl::e2(box[MAIL_R], box[MAIL_R + 1])), ra = gl::prep(gl::e2(box[MAIL_RA], box[MAIL_RA + 1]));
+        // ---- the pending folds ----
+        if (k == 0) {
+            // from device memory: entry i of the state is made of the source's entries 2i, 2i+1 (one fold) or 4i..4i+3 (two)
+            const u64 base = (u64)wg * src_wg;
+            for (u32 i = tid; i < len; i += BLOCK) {
 #pragma unroll
-        for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
-        for (u64 i = threadIdx.x; i < n_pairs; i += BLOCK) {
-            E2 lo[NF], hi[NF];
-#pragma unroll
-            for (int f = 0; f < NF; f++) {
-                E2 x0, x1, x2, x3;
-                if (j == a.j0) {
-                    const bool mine = i == threadIdx.x;
-                    U64x2 p0 = mine ? first[f][0] : ld2(a.s0[f] + 4 * i), q0 = mine ? first[f][1] : ld2(a.s0[f] + 4 * i + 2);
-                    U64x2 p1 = mine ? first[f][2] : ld2(a.s1[f] + 4 * i), q1 = mine ? first[f][3] : ld2(a.s1[f] + 4 * i + 2);
-                    x0 = gl::e2(p0.x, p1.x);
-                    x1 = gl::e2(p0.y, p1.y);
-                    x2 = gl::e2(q0.x, q1.x);
-                    x3 = gl::e2(q0.y, q1.y);
-                } else {
-                    // the source is the other LDS buffer
-                    const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
-                    const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
-                    x0 = gl::e2(c0[4 * i], c1[4 * i]);
-                    x1 = gl::e2(c0[4 * i + 1], c1[4 * i + 1]);
-                    x2 = gl::e2(c0[4 * i + 2], c1[4 * i + 2]);
-                    x3 = gl::e2(c0[4 * i + 3], c1[4 * i + 3]);
+                for (int f = 0; f < NF; f++) {
+                    E2 v;
+                    if (pend == 1) {
+                        const U64x2 x0 = ld2(a.s0[f] + base + 2 * (u64)i), x1 = ld2(a.s1[f] + base + 2 * (u64)i);
+                        v = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb);
+                    } else {
+                        const U64x2 x0 = ld2(a.s0[f] + base + 4 * (u64)i), y0 = ld2(a.s0[f] + base + 4 * (u64)i + 2);
+                        const U64x2 x1 = ld2(a.s1[f] + base + 4 * (u64)i), y1 = ld2(a.s1[f] + base + 4 * (u64)i + 2);
+                        v = fold1p(fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), ra), fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), ra), rb);
+                    }
+                    tab(true, f, 0)[i] = v.c0;
+                    tab(true, f, 1)[i] = v.c1;
                 }
-                lo[f] = fold1p(x0, x1, rp);
-                hi[f] = fold1p(x2, x3, rp);
-                u64 *d0 = to_ping ? ping[f][0] : pong[f][0];
-                u64 *d1 = to_ping ? ping[f][1] : pong[f][1];
-                d0[2 * i] = lo[f].c0;
-                d0[2 * i + 1] = hi[f].c0;
-                d1[2 * i] = lo[f].c1;
-                d1[2 * i + 1] = hi[f].c1;
             }
-            gl::E2P restp = gl::prep(gl::e2_one());
-            if (EQ) restp = gl::prep(i == threadIdx.x ? rest_ahead : gl::e2(a.eq0[eq_off + i], a.eq1[eq_off + i]));
-            E2 dl[NF], cur[NF];
+        } else {
+            len >>= pend;
+            for (u32 i = tid; i < len; i += BLOCK) {
 #pragma unroll
-            for (int f = 0; f < NF; f++) {
-                dl[f] = gl::sub(hi[f], lo[f]);
-                cur[f] = lo[f];
-            }
-#pragma unroll
-            for (int t = 0; t < NP; t++) {
-                if (!(t == 1 && skip1)) {
-                    E2 prod = cur[0];
-#pragma unroll
-                    for (int f = 1; f < NF; f++) prod = gl::mul(prod, cur[f]);
-                    if (EQ)
-                        acc[t] = gl::fma(prod, restp, acc[t]);
+                for (int f = 0; f < NF; f++) {
+                    const u64 *c0 = tab(in_big, f, 0), *c1 = tab(in_big, f, 1);
+                    E2 v;
+                    if (pend == 1)
+                        v = fold1p(gl::e2(c0[2 * i], c1[2 * i]), gl::e2(c0[2 * i + 1], c1[2 * i + 1]), rb);
                     else
-                        acc[t] = gl::add(acc[t], prod);
+                        v = fold1p(fold1p(gl::e2(c0[4 * i], c1[4 * i]), gl::e2(c0[4 * i + 1], c1[4 * i + 1]), ra),
+                                   fold1p(gl::e2(c0[4 * i + 2], c1[4 * i + 2]), gl::e2(c0[4 * i + 3], c1[4 * i + 3]), ra), rb);
+                    tab(!in_big, f, 0)[i] = v.c0;
+                    tab(!in_big, f, 1)[i] = v.c1;
                 }
-                if (t + 1 < NP) {
+            }
+            in_big = !in_big;
+        }
+        // this wavefront's counters start the trip at zero
+        for (u32 c = lane; c < 4 * (u32)NS; c += WAVE) ctr[wave * 4 * SL_MAX_SUMS + c] = 0;
+        __syncthreads();
+        const u64 *c0[NF], *c1[NF];
 #pragma unroll
-                    for (int f = 0; f < NF; f++) cur[f] = (t == 0) ? hi[f] : gl::add(cur[f], dl[f]);
+        for (int f = 0; f < NF; f++) c0[f] = tab(in_big, f, 0), c1[f] = tab(in_big, f, 1);
+        // adds a lane's canonical sum into the counters of extension sum `idx`
+        auto flush = [&](u32 idx, E2 v) {
+            u64 *c = ctr + wave * 4 * SL_MAX_SUMS + 4 * idx;
+            atomicAdd(reinterpret_cast<unsigned long long *>(c + 0), (unsigned long long)(u32)v.c0);
+            atomicAdd(reinterpret_cast<unsigned long long *>(c + 1), (unsigned long long)(v.c0 >> 32));
+            atomicAdd(reinterpret_cast<unsigned long long *>(c + 2), (unsigned long long)(u32)v.c1);
+            atomicAdd(reinterpret_cast<unsigned long long *>(c + 3), (unsigned long long)(v.c1 >> 32));
+        };
+        // ---- round j: pairs of the state; taken from the last thread down, so that with few pairs and quads they meet different lanes ----
+        {
+            const u32 n_pairs = len >> 1;
+            const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) + (u64)wg * n_pairs : 0;
+            E2 acc[NP];
+#pragma unroll
+            for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+            bool any = false;
+            for (u32 p = BLOCK - 1 - tid; p < n_pairs; p += BLOCK) {
+                any = true;
+                gl::E2P wp = gl::prep(gl::e2_one());
+                if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + p], a.eq1[eq_off + p]));
+                E2 lo[NF], hi[NF], dl[NF], cur[NF];
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    lo[f] = gl::e2(c0[f][2 * p], c1[f][2 * p]);
+                    hi[f] = gl::e2(c0[f][2 * p + 1], c1[f][2 * p + 1]);
+                    dl[f] = gl::sub(hi[f], lo[f]);
+                    cur[f] = lo[f];
                 }
+#pragma unroll
+                for (int t = 0; t < NP; t++) {
+                    if (!(t == 1 && skip1)) {
+                        E2 prod = cur[0];
+#pragma unroll
+                        for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
+                        acc[t] = EQ ? gl::fma(prod, wp, acc[t]) : gl::add(acc[t], prod);
+                    }
+                    if (t + 1 < NP) {
+#pragma unroll
+                        for (int f = 0; f < NF; f++) cur[f] = (t == 0) ? hi[f] : gl::add(cur[f], dl[f]);
+                    }
+                }
+            }
+            if (any) {
+#pragma unroll
+                for (int t = 0; t < NP; t++)
+                    if (!(t == 1 && skip1)) flush(t, acc[t]);
             }
         }
-        block_reduce<NP>(acc, lds);
-        publish_sums<NP>(a.out_host, a.seq0 + (j - a.j0), nullptr, acc);
+        // ---- round j + 1 as a polynomial in the challenge of round j: quads of the state ----
+        if (dbl) {
+            const u32 n_quads = len >> 2;
+            const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - (j + 1)))) + (u64)wg * n_quads : 0;
+            // a lane keeps one sample: NSMP adjacent lanes share a quad
+            const u32 smp = tid % NSMP, slot = tid / NSMP, n_slots = BLOCK / NSMP;
+            E2 acc[NPT];
+#pragma unroll
+            for (int t = 0; t < NPT; t++) acc[t] = gl::e2_zero();
+            bool any = false;
+            if (slot < n_slots) {
+                for (u32 u = slot; u < n_quads; u += n_slots) {
+                    any = true;
+                    gl::E2P wp = gl::prep(gl::e2_one());
+                    if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + u], a.eq1[eq_off + u]));
+                    E2 lo[NF], dl[NF], cur[NF];
+#pragma unroll
+                    for (int f = 0; f < NF; f++) {
+                        const E2 e0 = gl::e2(c0[f][4 * u], c1[f][4 * u]), e1 = gl::e2(c0[f][4 * u + 1], c1[f][4 * u + 1]);
+                        const E2 e2_ = gl::e2(c0[f][4 * u + 2], c1[f][4 * u + 2]), e3 = gl::e2(c0[f][4 * u + 3], c1[f][4 * u + 3]);
+                        const E2 d01 = gl::sub(e1, e0), d23 = gl::sub(e3, e2_);
+                        E2 hi;
+                        if (smp == (u32)NF) {
+                            // leading coefficient: the slopes in place of the folded entries
+                            lo[f] = d01;
+                            hi = d23;
+                        } else {
+                            // the pair folded with the challenge at smp: e0 + smp (e1 - e0), e2 + smp (e3 - e2)
+                            lo[f] = e0;
+                            hi = e2_;
+                            for (u32 m = 0; m < smp; m++) {
+                                lo[f] = gl::add(lo[f], d01);
+                                hi = gl::add(hi, d23);
+                            }
+                        }
+                        dl[f] = gl::sub(hi, lo[f]);
+                        cur[f] = lo[f];
+                    }
+                    // points t = 0, 2, .., NF
+#pragma unroll
+                    for (int ti = 0; ti < NPT; ti++) {
+                        if (ti == 1) {
+#pragma unroll
+                            for (int f = 0; f < NF; f++) cur[f] = gl::add(gl::add(lo[f], dl[f]), dl[f]);
+                        } else if (ti > 1) {
+#pragma unroll
+                            for (int f = 0; f < NF; f++) cur[f] = gl::add(cur[f], dl[f]);
+                        }
+                        E2 prod = cur[0];
+#pragma unroll
+                        for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
+                        acc[ti] = EQ ? gl::fma(prod, wp, acc[ti]) : gl::add(acc[ti], prod);
+                    }
+                }
+            }
+            if (any) {
+#pragma unroll
+                for (int ti = 0; ti < NPT; ti++) flush(NP + smp * NPT + ti, acc[ti]);
+            }
+        }
         __syncthreads();
-        to_ping = !to_ping;
-        n_pairs >>= 1;
+        // ---- hand the sums over ----
+        bool publish = W == 1;
+        if (W > 1) {
+            // the counters of the four wavefronts, added into the launch's counters in device memory
+            if (wave == 0) {
+                for (u32 c = lane; c < 4 * (u32)NS; c += WAVE) {
+                    u64 v = 0;
+#pragma unroll
+                    for (int w = 0; w < BLOCK / WAVE; w++) v += ctr[w * 4 * SL_MAX_SUMS + c];
+                    if (v) __hip_atomic_fetch_add(a.ctr + c, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            publish = take_ticket(a.ticket, W, last_flag);
+        }
+        if (publish && wave == 0) {
+            // word w of the result (limb w & 1 of sum w >> 1) is counters 2w (low halves) and 2w + 1 (high halves)
+            u64 word = 0;
+            const bool mine = lane < 2 * (u32)NS;
+            if (mine) {
+                u64 lo_h = 0, hi_h = 0;
+                if (W > 1) {
+                    lo_h = ld_agent(a.ctr + 2 * lane);
+                    hi_h = ld_agent(a.ctr + 2 * lane + 1);
+                    st_agent(a.ctr + 2 * lane, 0);
+                    st_agent(a.ctr + 2 * lane + 1, 0);
+                } else {
+#pragma unroll
+                    for (int w = 0; w < BLOCK / WAVE; w++) {
+                        lo_h += ctr[w * 4 * SL_MAX_SUMS + 2 * lane];
+                        hi_h += ctr[w * 4 * SL_MAX_SUMS + 2 * lane + 1];
+                    }
+                }
+                const unsigned __int128 t = (unsigned __int128)lo_h + ((unsigned __int128)hi_h << 32);
+                word = gl::reduce128((u64)t, (u64)(t >> 64));
+            }
+            if (W > 1) {
+                // the counters and the ticket are back at zero before the host can answer
+                // (stores that go through to where the other workgroups' atomics operate, like the counters' above)
+                if (lane == 0) __hip_atomic_store(a.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_s_waitcnt(0);
+            }
+            u64 x = mine ? rotl64(word, lane + 1) : 0;
+#pragma unroll
+            for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
+            if (mine) st_sys(a.out_host + lane, word);
+            if (lane == 0) {
+                st_sys(a.out_host + SL_CHK_SLOT, x ^ trip_seq);
+                st_sys(a.out_host + SL_SEQ_SLOT, trip_seq);
+            }
+        }
+        pend = dbl ? 2 : 1;
+        j += pend;
+        __syncthreads();
     }
-    // with the last round: value and slope of the remaining pair of every table (the host folds them with the last challenge)
-    if (threadIdx.x < NF) {
-        const int f = threadIdx.x;
-        // the last round wrote its pair to the buffer `to_ping` now points away from
-        const u64 *c0 = to_ping ? pong[f][0] : ping[f][0];
-        const u64 *c1 = to_ping ? pong[f][1] : ping[f][1];
-        const E2 lo = gl::e2(c0[0], c1[0]), d = gl::sub(gl::e2(c0[1], c1[1]), lo);
-        res[4 * f] = lo.c0;
-        res[4 * f + 1] = lo.c1;
-        res[4 * f + 2] = d.c0;
-        res[4 * f + 3] = d.c1;
+    // ---- what is left of the tables ----
+    const bool big = in_big;
+    if (!a.finish) {
+        // to device memory, for the launch queued behind this one (which starts with this launch's pending folds)
+        for (u32 i = tid; i < len; i += BLOCK) {
+#pragma unroll
+            for (int f = 0; f < NF; f++) {
+                a.h0[f][(u64)wg * len + i] = tab(big, f, 0)[i];
+                a.h1[f][(u64)wg * len + i] = tab(big, f, 1)[i];
+            }
+        }
+    } else if (wave == 0) {
+        // to the host, which does the last fold or two: entry e of table f at words 2 (f len + e), + 1
+        const u32 n_words = (u32)NF * len * 2;
+        const bool mine = lane < n_words;
+        u64 word = 0;
+        if (mine) {
+            const u32 f = lane / (2 * len), e = (lane >> 1) % len;
+            word = tab(big, f, lane & 1)[e];
+        }
+        u64 x = mine ? rotl64(word, lane + 1) : 0;
+#pragma unroll
+        for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
+        if (mine) st_sys(a.out_host + SL_FIN_SLOT + lane, word);
+        if (lane == 0) {
+            st_sys(a.out_host + SL_FIN_CHK_SLOT, x ^ trip_seq);
+            st_sys(a.out_host + SL_FIN_SEQ_SLOT, trip_seq);
+        }
     }
-    __syncthreads();
-    if (threadIdx.x == 0)
-        publish_words(a.out_host, HOST_FINALS_SLOT, res, 4 * NF, a.seq0 + (a.n_vars - a.j0), HOST_PAIRS_SEQ_SLOT, HOST_PAIRS_CHK_SLOT);
 }
 
 // ---------------------------------------------------------------------------

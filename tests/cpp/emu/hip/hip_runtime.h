@@ -52,25 +52,40 @@ struct Barrier {
         }
     }
 };
-inline Barrier block_barrier;
-inline Barrier wave_barrier[MAX_THREADS / WAVE];
-inline uint64_t xchg[MAX_THREADS];
+// what the threads of one workgroup share.  Kernels whose LDS is all dynamic (none of the __shared__ statics above) can
+// have several workgroups running at once, each with a context of its own.
+struct Group {
+    Barrier block_barrier;
+    Barrier wave_barrier[MAX_THREADS / WAVE];
+    uint64_t xchg[MAX_THREADS];
+    uint64_t *dyn = nullptr;  // dynamic LDS
+    void reset(int threads)
+    {
+        block_barrier.reset(threads);
+        for (int w = 0; w < threads / WAVE; w++) wave_barrier[w].reset(WAVE);
+    }
+};
+inline Group default_group;
+inline thread_local Group *group = &default_group;
+inline uint64_t *dyn_lds() { return group->dyn; }
 }  // namespace emu
 
 inline thread_local dim3 threadIdx, blockIdx;
 inline dim3 gridDim, blockDim;
 
-inline void __syncthreads() { emu::block_barrier.wait(); }
+inline void __syncthreads() { emu::group->block_barrier.wait(); }
+inline unsigned long long atomicAdd(unsigned long long *p, unsigned long long v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
 
 namespace emu {
 // value of `v` in lane `src` of the caller's wavefront (every lane of the wavefront calls this together)
 inline uint64_t lane_read(uint64_t v, int src)
 {
     const int t = (int)threadIdx.x, w = t / WAVE;
-    xchg[t] = v;
-    wave_barrier[w].wait();
-    const uint64_t r = xchg[w * WAVE + src];
-    wave_barrier[w].wait();
+    Group &g = *group;
+    g.xchg[t] = v;
+    g.wave_barrier[w].wait();
+    const uint64_t r = g.xchg[w * WAVE + src];
+    g.wave_barrier[w].wait();
     return r;
 }
 // v_mov_b32 with a DPP control, as __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl) of gfx9:

@@ -41,8 +41,7 @@ static void launch(u32 blocks, K kernel, A... args)
     gridDim = dim3(blocks);
     blockDim = dim3(dpk::BLOCK);
     for (u32 b = 0; b < blocks; b++) {
-        emu::block_barrier.reset(dpk::BLOCK);
-        for (int w = 0; w < dpk::BLOCK / dpk::WAVE; w++) emu::wave_barrier[w].reset(dpk::WAVE);
+        emu::default_group.reset(dpk::BLOCK);
         std::vector<std::thread> th;
         for (u32 t = 0; t < (u32)dpk::BLOCK; t++)
             th.emplace_back([=] {

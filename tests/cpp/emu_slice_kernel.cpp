@@ -1,0 +1,380 @@
+// slice_kernel (the LDS-resident rounds of a product sumcheck, one or two rounds per trip to the host, one or several
+// workgroups) run on the CPU through tests/cpp/emu/hip/hip_runtime.h: every workgroup of a launch at once, one host
+// thread per lane, and a thread that plays the host's side of the mailbox.  Every trip's sums are checked against
+// sums worked out from the definitions on a reference copy of the tables: the round's q(t) by plain loops, the next
+// round's sums at the sample challenges by actually folding the reference tables with 0, 1, .. and summing, the
+// leading coefficient by finite differences.  Then the algebra the host relies on: the polynomial through those
+// samples, evaluated at the real challenge, equals the next round's sums computed directly.  Built with the host
+// sanitizers and a fill pattern for uninitialised locals by tests/test_kernel_emulation.py.
+#include <chrono>
+#include <memory>
+#include <thread>
+#include <vector>
+
+#include "dpsumcheck.h"
+#include "kernels.hpp"
+
+using gl::E2;
+using gl::u32;
+using gl::u64;
+
+static u64 sm_state = 777;
+static u64 splitmix()
+{
+    sm_state += 0x9E3779B97F4A7C15ull;
+    u64 z = sm_state;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static u64 felt()
+{
+    for (;;) {
+        const u64 v = splitmix();
+        if (v < gl::P) return v;
+    }
+}
+static E2 felt2() { return gl::e2(felt(), felt()); }
+static u64 h_pow(u64 a, u64 e)
+{
+    u64 r = 1;
+    while (e) {
+        if (e & 1) r = gl::mul(r, a);
+        a = gl::mul(a, a);
+        e >>= 1;
+    }
+    return r;
+}
+static u64 h_inv(u64 a) { return h_pow(a, gl::P - 2); }
+
+typedef std::vector<E2> Table;
+static Table fold(const Table &s, E2 r)
+{
+    Table o(s.size() / 2);
+    for (size_t i = 0; i < o.size(); i++) o[i] = gl::add(s[2 * i], gl::mul(r, gl::sub(s[2 * i + 1], s[2 * i])));
+    return o;
+}
+
+// every workgroup of a launch at once
+template <class K, class A>
+static std::vector<std::thread> launch_all(u32 blocks, size_t lds_words, K kernel, A args, std::vector<std::unique_ptr<emu::Group>> &groups,
+                                           std::vector<std::vector<u64>> &lds)
+{
+    gridDim = dim3(blocks);
+    blockDim = dim3(dpk::BLOCK);
+    std::vector<std::thread> th;
+    for (u32 b = 0; b < blocks; b++) {
+        groups.emplace_back(new emu::Group());
+        lds.emplace_back(lds_words, 0xAAAAAAAAAAAAAAAAull);
+        groups.back()->reset(dpk::BLOCK);
+        groups.back()->dyn = lds.back().data();
+        emu::Group *g = groups.back().get();
+        for (u32 t = 0; t < (u32)dpk::BLOCK; t++)
+            th.emplace_back([=] {
+                emu::group = g;
+                threadIdx = dim3(t);
+                blockIdx = dim3(b);
+                kernel(args);
+            });
+    }
+    return th;
+}
+
+static int failures = 0;
+
+struct Stage {
+    u32 W, j0, pend0;
+    u64 src_len;
+    std::vector<std::pair<u32, bool>> trips;  // first round, covers two rounds
+};
+
+// NF tables, sum of n_vars variables, resident from round j0 on; `wide`: workgroups of the first stage (1: a single stage);
+// `single_rounds`: rounds that must start a trip of their own with t = 1 evaluated (an eq point with a zero coordinate there)
+template <int NF, bool EQ>
+static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pairs, std::vector<u32> single_rounds = {})
+{
+    constexpr int NP = NF + 1, NPT = NF, NSMP = NF + 1, NS = NP + NSMP * NPT;
+    auto is_single = [&](u32 j) {
+        for (u32 x : single_rounds)
+            if (x == j) return true;
+        return false;
+    };
+    // reference tables: the state before round j0's pending fold, and the challenges of every round
+    std::vector<Table> ref(NF, Table((size_t)1 << (n_vars - j0 + 2)));
+    for (auto &t : ref)
+        for (auto &x : t) x = felt2();
+    std::vector<E2> chal(n_vars + 1);
+    for (auto &c : chal) c = felt2();
+    // eq storage: level l at (2 << n) - (2 << (n - l)), eq(rho_{l..n-1}, .)
+    std::vector<E2> rho(n_vars);
+    for (auto &x : rho) x = felt2();
+    std::vector<u64> eq0((size_t)2 << n_vars, 0), eq1((size_t)2 << n_vars, 0);
+    auto eq_level = [&](u32 l, u64 i) { return gl::e2(eq0[((size_t)2 << n_vars) - ((size_t)2 << (n_vars - l)) + i], eq1[((size_t)2 << n_vars) - ((size_t)2 << (n_vars - l)) + i]); };
+    if (EQ)
+        for (u32 l = 0; l <= n_vars; l++)
+            for (u64 i = 0; i < ((u64)1 << (n_vars - l)); i++) {
+                E2 v = gl::e2_one();
+                for (u32 b = 0; b < n_vars - l; b++) v = gl::mul(v, ((i >> b) & 1) ? rho[l + b] : gl::sub(gl::e2_one(), rho[l + b]));
+                const size_t off = ((size_t)2 << n_vars) - ((size_t)2 << (n_vars - l)) + i;
+                eq0[off] = v.c0, eq1[off] = v.c1;
+            }
+    // the plan: stages and their trips (what the library's session planner does)
+    std::vector<Stage> stages;
+    {
+        u32 j = j0;
+        u64 entries = (u64)1 << (n_vars - j0 + 2);  // of the state the next stage starts from
+        u32 pend = 1;
+        if (wide > 1) {
+            Stage st{wide, j, pend, entries, {}};
+            u64 len_wg = (entries / wide) >> pend;
+            for (;;) {
+                const bool dbl = len_wg >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1);
+                st.trips.push_back({j, dbl});
+                pend = dbl ? 2 : 1;
+                j += pend;
+                if ((len_wg >> pend) < 2 || j > n_vars) break;
+                len_wg >>= pend;
+            }
+            entries = len_wg * wide;
+            stages.push_back(st);
+        }
+        Stage st{1, j, pend, entries, {}};
+        u64 len = entries >> pend;
+        while (j <= n_vars) {
+            const bool dbl = len >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1);
+            st.trips.push_back({j, dbl});
+            const u32 p = dbl ? 2 : 1;
+            j += p;
+            len >>= p;
+        }
+        stages.push_back(st);
+    }
+    (void)cap_pairs;
+
+    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
+    u32 ticket = 0;
+    const u64 seq_first = 1000;
+    bool ok = true;
+    // device-side tables of the stage to come
+    std::vector<std::vector<u64>> d0(NF), d1(NF);
+    for (int f = 0; f < NF; f++) {
+        d0[f].resize(ref[f].size()), d1[f].resize(ref[f].size());
+        for (size_t i = 0; i < ref[f].size(); i++) d0[f][i] = ref[f][i].c0, d1[f][i] = ref[f][i].c1;
+    }
+    std::vector<Table> state = ref;  // reference state, folded as the challenges are "drawn"
+    u32 folded_through = j0 - 2;     // the state has been folded with the challenges of rounds <= folded_through
+    auto fold_to = [&](u32 round) {  // bring the reference state to the tables of `round`
+        while (folded_through < round - 1) {
+            folded_through++;
+            for (auto &t : state) t = fold(t, chal[folded_through]);
+        }
+    };
+    // q(t) of a round from its tables, by the definition
+    auto round_sums = [&](const std::vector<Table> &tabs, u32 round, E2 *q /* NF + 1 */) {
+        for (int t = 0; t <= NF; t++) q[t] = gl::e2_zero();
+        for (size_t p = 0; p < tabs[0].size() / 2; p++)
+            for (int t = 0; t <= NF; t++) {
+                E2 prod = EQ ? eq_level(round, p) : gl::e2_one();
+                for (int f = 0; f < NF; f++) prod = gl::mul(prod, gl::add(tabs[f][2 * p], gl::mul_base(gl::sub(tabs[f][2 * p + 1], tabs[f][2 * p]), (u64)t)));
+                q[t] = gl::add(q[t], prod);
+            }
+    };
+
+    for (size_t si = 0; si < stages.size() && ok; si++) {
+        const Stage &st = stages[si];
+        dpk::SliceArgs a;
+        memset(&a, 0, sizeof a);
+        std::vector<std::vector<u64>> h0(NF), h1(NF);
+        for (int f = 0; f < NF; f++) {
+            a.s0[f] = d0[f].data();
+            a.s1[f] = d1[f].data();
+            h0[f].assign(st.src_len, 0);
+            h1[f].assign(st.src_len, 0);
+            a.h0[f] = h0[f].data();
+            a.h1[f] = h1[f].data();
+        }
+        a.src_len = st.src_len;
+        a.pend0 = st.pend0;
+        a.n_vars = n_vars;
+        a.j0 = st.j0;
+        a.n_trips = (u32)st.trips.size();
+        for (size_t k = 0; k < st.trips.size(); k++)
+            if (st.trips[k].second) a.dbl_mask |= 1u << k;
+        a.eq0 = eq0.data(), a.eq1 = eq1.data();
+        a.mail = mail.data();
+        a.relay = relay.data();
+        a.spin_limit = 1u << 24;
+        a.finish = si + 1 == stages.size();
+        a.out_host = area.data();
+        a.seq0 = seq_first + (st.j0 - j0);
+        a.ctr = gctr.data();
+        a.ticket = &ticket;
+        const u32 cap = (u32)((st.src_len / st.W) >> st.pend0);
+        std::vector<std::unique_ptr<emu::Group>> groups;
+        std::vector<std::vector<u64>> lds;
+        auto threads = launch_all(st.W, dpk::slice_lds_words(NF, cap), dpk::slice_kernel<NF, EQ>, a, groups, lds);
+        // ---- the host's side ----
+        u32 len_after = 0;
+        for (size_t k = 0; k < st.trips.size() && ok; k++) {
+            const u32 j = st.trips[k].first;
+            const bool dbl = st.trips[k].second;
+            const u64 seq = seq_first + (j - j0);
+            const bool skip1 = !is_single(j);
+            mail[dpk::MAIL_R] = chal[j - 1].c0, mail[dpk::MAIL_R + 1] = chal[j - 1].c1;
+            mail[dpk::MAIL_RA] = j >= 2 ? chal[j - 2].c0 : 0, mail[dpk::MAIL_RA + 1] = j >= 2 ? chal[j - 2].c1 : 0;
+            mail[dpk::MAIL_SKIP1] = skip1;
+            u64 chk = seq;
+            for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
+            mail[dpk::MAIL_CHK] = chk;
+            __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
+            // the result
+            u64 w[2 * dpk::SL_MAX_SUMS];
+            const auto t0 = std::chrono::steady_clock::now();
+            for (;;) {
+                if (__atomic_load_n(&area[dpk::SL_SEQ_SLOT], __ATOMIC_SEQ_CST) == seq) {
+                    u64 c = seq;
+                    for (int i = 0; i < 2 * NS; i++) {
+                        w[i] = __atomic_load_n(&area[i], __ATOMIC_SEQ_CST);
+                        c ^= dpk::rotl64(w[i], i + 1);
+                    }
+                    if (c == __atomic_load_n(&area[dpk::SL_CHK_SLOT], __ATOMIC_SEQ_CST)) break;
+                }
+                if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(60)) {
+                    printf("%s: no result for the trip of round %u\n", name, j);
+                    ok = false;
+                    break;
+                }
+                std::this_thread::sleep_for(std::chrono::microseconds(200));
+            }
+            if (!ok) break;
+            auto sum_at = [&](int idx) { return gl::e2(w[2 * idx], w[2 * idx + 1]); };
+            // round j by the definition
+            fold_to(j);
+            E2 q[NF + 1];
+            round_sums(state, j, q);
+            for (int t = 0; t <= NF; t++) {
+                const E2 want = (t == 1 && skip1) ? gl::e2_zero() : q[t];
+                if (!gl::eq(sum_at(t), want)) {
+                    printf("%s: round %u q(%d) differs\n", name, j, t);
+                    ok = false;
+                }
+            }
+            if (dbl) {
+                // round j + 1 with the challenge at 0, 1, .., NF: fold the reference tables with each and sum
+                E2 c[NF + 1][NF + 1];
+                for (int s = 0; s <= NF; s++) {
+                    std::vector<Table> tmp;
+                    for (auto &t : state) tmp.push_back(fold(t, gl::e2((u64)s, 0)));
+                    round_sums(tmp, j + 1, c[s]);
+                }
+                const int pts[3] = {0, 2, 3};
+                for (int ti = 0; ti < NPT && ok; ti++) {
+                    const int t = pts[ti];
+                    for (int s = 0; s < NF; s++)
+                        if (!gl::eq(sum_at(NP + s * NPT + ti), c[s][t])) {
+                            printf("%s: round %u sample %d point %d differs\n", name, j + 1, s, t);
+                            ok = false;
+                        }
+                    // leading coefficient = NF-th finite difference / NF!
+                    E2 lead = gl::e2_zero();
+                    u64 binom = 1, fact = 1;
+                    for (int kk = 0; kk <= NF; kk++) {
+                        const E2 term = gl::mul_base(c[kk][t], binom);
+                        lead = ((NF - kk) & 1) ? gl::sub(lead, term) : gl::add(lead, term);
+                        binom = binom * (u64)(NF - kk) / (u64)(kk + 1);
+                    }
+                    for (int kk = 2; kk <= NF; kk++) fact *= (u64)kk;
+                    lead = gl::mul_base(lead, h_inv(fact));
+                    if (!gl::eq(sum_at(NP + NF * NPT + ti), lead)) {
+                        printf("%s: round %u leading coefficient at point %d differs\n", name, j + 1, t);
+                        ok = false;
+                    }
+                    // what the host does with them: the polynomial at the real challenge = the round's sum computed directly
+                    const E2 r = chal[j];
+                    E2 val = gl::e2_zero(), vanish = gl::e2_one();
+                    for (int kk = 0; kk < NF; kk++) {
+                        E2 num = gl::e2_one();
+                        u64 den = 1;
+                        for (int m = 0; m < NF; m++)
+                            if (m != kk) {
+                                num = gl::mul(num, gl::sub(r, gl::e2((u64)m, 0)));
+                                den = gl::mul(den, gl::sub((u64)kk, (u64)m));
+                            }
+                        val = gl::add(val, gl::mul(gl::mul_base(num, h_inv(den)), sum_at(NP + kk * NPT + ti)));
+                        vanish = gl::mul(vanish, gl::sub(r, gl::e2((u64)kk, 0)));
+                    }
+                    val = gl::add(val, gl::mul(vanish, sum_at(NP + NF * NPT + ti)));
+                    std::vector<Table> next;
+                    for (auto &tb : state) next.push_back(fold(tb, r));
+                    E2 q2[NF + 1];
+                    round_sums(next, j + 1, q2);
+                    if (!gl::eq(val, q2[t])) {
+                        printf("%s: round %u point %d: interpolation at the challenge differs from the direct sum\n", name, j + 1, t);
+                        ok = false;
+                    }
+                }
+            }
+            len_after = dbl ? 4 : 2;
+        }
+        if (!ok) {
+            // let the launch leave: the abort sequence number, as the library does
+            __atomic_store_n(&mail[dpk::MAIL_SEQ], dpk::MAIL_ABORT_SEQ, __ATOMIC_SEQ_CST);
+        }
+        for (auto &t : threads) t.join();
+        if (!ok) break;
+        if (ticket != 0) ok = false, printf("%s: ticket counter left at %u\n", name, ticket);
+        for (u64 c : gctr)
+            if (c) ok = false;
+        const auto &last = st.trips.back();
+        const u32 pend = last.second ? 2 : 1;
+        if (si + 1 < stages.size()) {
+            // what the stage left behind is the reference state of its last trip's round
+            fold_to(last.first);
+            const u64 left = state[0].size();
+            if (left != stages[si + 1].src_len) ok = false, printf("%s: stage leaves %llu entries, the next expects %llu\n", name, (unsigned long long)left, (unsigned long long)stages[si + 1].src_len);
+            for (int f = 0; f < NF && ok; f++) {
+                d0[f].assign(left, 0), d1[f].assign(left, 0);
+                for (u64 i = 0; i < left; i++) {
+                    if (h0[f][i] != state[f][i].c0 || h1[f][i] != state[f][i].c1) {
+                        printf("%s: handed-over entry %llu of table %d differs\n", name, (unsigned long long)i, f);
+                        ok = false;
+                        break;
+                    }
+                    d0[f][i] = h0[f][i], d1[f][i] = h1[f][i];
+                }
+            }
+            if (stages[si + 1].pend0 != pend) ok = false, printf("%s: pending folds disagree\n", name);
+        } else {
+            // the last entries of every table, published with the last trip
+            fold_to(last.first);
+            const u64 seq = seq_first + (last.first - j0);
+            u64 c = seq;
+            const u32 n_words = NF * len_after * 2;
+            for (u32 i = 0; i < n_words; i++) c ^= dpk::rotl64(area[dpk::SL_FIN_SLOT + i], i + 1);
+            if (area[dpk::SL_FIN_SEQ_SLOT] != seq || area[dpk::SL_FIN_CHK_SLOT] != c) ok = false, printf("%s: last entries not handed over\n", name);
+            if (state[0].size() != len_after) ok = false, printf("%s: %zu entries left, %u expected\n", name, state[0].size(), len_after);
+            for (int f = 0; f < NF && ok; f++)
+                for (u32 e = 0; e < len_after; e++)
+                    if (area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e)] != state[f][e].c0 || area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e) + 1] != state[f][e].c1)
+                        ok = false, printf("%s: last entry %u of table %d differs\n", name, e, f);
+        }
+    }
+    size_t n_trips = 0;
+    for (auto &s : stages) n_trips += s.trips.size();
+    printf("%-60s NF=%d eq=%d n=%u from round %u, %zu stage(s), %zu trips for %u rounds : %s\n", name, NF, (int)EQ, n_vars, j0, stages.size(), n_trips,
+           n_vars - j0 + 1, ok ? "ok" : "MISMATCH");
+    if (!ok) failures++;
+}
+
+int main()
+{
+    run_case<2, true>("two tables and eq, one workgroup, trips of two rounds", 9, 2, 1, 0);
+    run_case<2, true>("odd number of rounds: the last trip covers one", 10, 2, 1, 0);
+    run_case<1, true>("one table and eq", 7, 2, 1, 0);
+    run_case<3, false>("three tables, no eq", 8, 3, 1, 0);
+    run_case<2, false>("two tables, rounds that must go alone (t = 1 evaluated)", 9, 2, 1, 0, {4, 7});
+    run_case<2, true>("four workgroups, then one", 12, 3, 4, 0);
+    run_case<2, true>("two workgroups down to one entry each, rounds that must go alone", 11, 3, 2, 0, {6});
+    printf("%s\n", failures ? "FAILED" : "all cases ok");
+    return failures ? 1 : 0;
+}

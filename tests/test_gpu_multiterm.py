@@ -185,9 +185,11 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
 
 @pytest.mark.parametrize("with_eq,n", [(True, 14), (False, 14), (True, 19), (False, 18)])
 def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
-    """The same for a single product of full-size tables: every round after the first and the resident kernel of
-    its last rounds (first round 6 of 14) are launched during the round before.  In a launch of more than 64
-    workgroups (n = 18, 19) only the first workgroup looks for the mail and passes it on to the others."""
+    """The same for a single product of full-size tables: round 2 and the resident launches of the rounds from 3 on
+    (several workgroups, then one) are made during the round before.  In a launch of more than 64 workgroups
+    (round 2 at n = 18, 19) only the first workgroup looks for the mail and passes it on to the others; the resident
+    launch of several workgroups always does so.  Once a resident launch has had its first mail another call on the
+    context ends the session (test_resident_kernel_gives_way)."""
     import time
     f, g = rand_base(1 << n, 31), rand_e2(1 << n, 32)
     gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
@@ -198,7 +200,7 @@ def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
         fs = [2, 0, 1]
     terms = [(np.array([3, 5], dtype=np.uint64), fs)]
     ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
-    for after in (1, 2, 4, 5):
+    for after in (1, 2):
         for how in ("other call", "slow caller"):
             s = ctx.session(n, gpu, terms)
             chal = None
@@ -213,6 +215,16 @@ def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
                         time.sleep(0.3 if after == 1 else 0.05)
             assert (s.finish(chal) == ref_finals).all()
             del s
+    # a slow caller in the resident rounds is waited for (the resident launches poll for seconds, not milliseconds)
+    s = ctx.session(n, gpu, terms)
+    chal = None
+    for j in range(n):
+        assert (s.round(chal) == ref_proof[j]).all(), j
+        chal = ref_point[j]
+        if j + 1 in (4, 5, n - 1):
+            time.sleep(0.05)
+    assert (s.finish(chal) == ref_finals).all()
+    del s
     _check(dp, ctx, orc, n, gpu, host, terms)
 
 
