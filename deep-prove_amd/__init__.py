@@ -117,6 +117,8 @@ dev.dps_profile_reset.argtypes = [_vp]
 dev.dps_profile_read.argtypes = [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]
 host.dph_sumcheck_prove.restype = _i32
 host.dph_sumcheck_prove.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]
+host.dph_sumcheck_prove_claimed.restype = _i32
+host.dph_sumcheck_prove_claimed.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp]
 host.dph_sumcheck_verify.restype = _i32
 host.dph_sumcheck_verify.argtypes = [_vp, _vp, _u32, _u32, _vp, _vp, _vp]
 
@@ -477,9 +479,10 @@ class Context:
                                                _ptr(finals), C.byref(d)), "dph_sumcheck_prove")
         return proof, point, finals[: len(mles)]
 
-    def sumcheck_prover(self, n_vars, mles, terms):
+    def sumcheck_prover(self, n_vars, mles, terms, claim=None):
         """The same proof called repeatedly: returns prove(transcript) with the handles and terms already marshalled
-        (a caller in a compiled language has no such per-call cost; from Python it is 10 us a proof)."""
+        (a caller in a compiled language has no such per-call cost; from Python it is 10 us a proof).
+        `claim`: the value of the whole sum when the caller holds it (the claim a layer prover is reducing)."""
         hs = (_vp * max(1, len(mles)))(*[m.handle for m in mles])
         tarr, nt = make_terms(terms)
         degree = max((len(f) for _, f in terms), default=0)
@@ -487,16 +490,18 @@ class Context:
         keep = list(mles)
         d = _u32(0)
         dref = C.byref(d)
+        cl = None if claim is None else np.ascontiguousarray(_e2(claim))
+        clp = None if cl is None else cl.ctypes.data
 
         def prove(transcript):
             proof = np.zeros((n_vars, degree + 1, 2), dtype=np.uint64)
             point = np.zeros((n_vars, 2), dtype=np.uint64)
             finals = np.zeros((max(1, n_mles), 2), dtype=np.uint64)
-            self._chk_host(host.dph_sumcheck_prove(self._c, n_vars, hs, n_mles, tarr, nt, transcript._t, proof.ctypes.data, point.ctypes.data,
-                                                   finals.ctypes.data, dref), "dph_sumcheck_prove")
+            self._chk_host(host.dph_sumcheck_prove_claimed(self._c, n_vars, hs, n_mles, tarr, nt, clp, transcript._t, proof.ctypes.data,
+                                                           point.ctypes.data, finals.ctypes.data, dref), "dph_sumcheck_prove")
             return proof, point, finals[:n_mles]
 
-        prove.keep = keep
+        prove.keep = (keep, cl)
         return prove
 
     def sumcheck_verify(self, claimed_sum, proof, transcript):

@@ -309,10 +309,15 @@ struct Storage {
 // eq(rho, .) the storage holds the tables eq(rho_{l..m-1}, .) for l = 1..m (2^(m-l)
 // entries each, level l at entry offset 2^(m+1) - 2^(m-l+1)): the sumcheck reads
 // level j in round j instead of folding the full table.
+// Nothing of it is written before somebody reads it: a product or multi-term session takes the eq factor in closed
+// form and reads suffix levels only (a product of 24 variables: levels 7..24 and the low tables; levels 0..6 are 2^25
+// entries, half a gigabyte of writes, that it never touches), while a download, a view, an evaluation or a session
+// that reads the table as an ordinary factor needs level 0.  `built` says which levels are there.
 struct EqInfo {
     u32 m;
     u32 fact_levels = 0;  // levels 1..fact_levels have room for a low table behind the levels (eq_low_off)
     bool fact_built = false;  // ... and the low tables are there (built when a product session first wants them)
+    u64 built = 0;        // bit l: level l is materialised
     std::vector<E2> point;
 };
 
@@ -329,6 +334,8 @@ struct dps_mle {
 };
 
 namespace {
+
+int32_t plain_ready(const dps_mle *t);
 
 bool is_pow2(u64 x) { return x && !(x & (x - 1)); }
 // raw quantised integers (not field elements): readable by the tensor kernels only
@@ -688,6 +695,12 @@ extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_
     if (n_vars > 40 || offset > src->len || len > src->len - offset) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: window outside the table");
     // pair loads are 16 bytes wide
     if (n_vars >= 1 && ((src->offset + offset) & 1)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_view: offset must be even");
+    // a window into an eq table shares its level 0 (a window over the whole table stays an eq table, built as its readers ask)
+    if (src->eq && !(offset == 0 && len == src->len)) {
+        DeviceGuard g(ctx->device);
+        tail_abort(ctx);
+        CHK(plain_ready(src));
+    }
     *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len, nullptr};
     if (*out && offset == 0 && len == src->len) (*out)->eq = src->eq;
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
@@ -699,6 +712,11 @@ extern "C" int32_t dps_mle_zero_pad(const dps_mle *src, uint32_t n_vars, dps_mle
     dps_ctx *ctx = src->ctx;
     if (is_raw(src->kind) || !is_pow2(src->len)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: not a power-of-two field table");
     if (n_vars > 40 || (1ull << n_vars) < src->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_zero_pad: %u variables are fewer than the table has", n_vars);
+    if (src->eq) {
+        DeviceGuard g(ctx->device);
+        tail_abort(ctx);
+        CHK(plain_ready(src));
+    }
     *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset, src->len, nullptr, n_vars};
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
 }
@@ -717,6 +735,7 @@ extern "C" int32_t dps_mle_download(const dps_mle *mle, uint64_t *c0, uint64_t *
     dps_ctx *ctx = mle->ctx;
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(mle));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     if (mle->kind == DPS_I16) {
         // widened on the host: the caller's buffer holds len int64 values like a DPS_I64 tensor's
@@ -769,59 +788,78 @@ u64 eq_level_off(u32 m, u32 l) { return (2ull << m) - (2ull << (m - l)); }
 // variables.  Level l is then the product  level_{l+16}[i >> 16] * low_l[i & 65535], which the product kernels use in their
 // large rounds instead of streaming level l.
 u32 eq_fact_levels(u32 m) { return m > dpk::EQ_LO_BITS ? m - dpk::EQ_LO_BITS : 0; }
+u32 eq_first_direct(u32 m) { return m > dpk::EQ_DIRECT_BITS ? m - dpk::EQ_DIRECT_BITS : 0; }
 u64 eq_low_off(u32 m, u32 l) { return (2ull << m) + ((u64)(l - 1) << dpk::EQ_LO_BITS); }
 u64 eq_storage_entries(u32 m) { return (2ull << m) + ((u64)eq_fact_levels(m) << dpk::EQ_LO_BITS); }
 
-// Builds eq(rho, .) and every level eq(rho_{l..m-1}, .), l = 1..m, into o0/o1
-// (2^(m+1) entries).  Levels of at most 2^16 entries come straight from the
-// definition in one launch, together with the 2^8-entry seeds eq(rho_{l..l+7}, .)
-// the larger levels need; level l > 2^16 entries is level l+8 expanded by seed l.
-int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
+// Materialises the levels in `need` (bit l: level l = eq(rho_{l..m-1}, .), 2^(m-l) entries at eq_level_off) that are not
+// there yet, and with `need_low` the low tables.  Levels of at most 2^16 entries come straight from the definition, in
+// one launch together with the low tables and the 2^8-entry seeds eq(rho_{l..l+7}, .) the larger levels need; a larger
+// level l is level l + 8 expanded by seed l (so asking for level 0 of a 24-variable table builds levels 0, 8, 16 only).
+int32_t eq_ensure(dps_ctx *ctx, EqInfo &info, u64 *o0, u64 *o1, u64 need, bool need_low)
 {
-    dpk::EqJobs js;
-    memset(&js, 0, sizeof js);
-    if (m) memcpy(js.point, point, 16 * (size_t)m);
-    js.o0 = o0;
-    js.o1 = o1;
-    u32 n_jobs = 0, max_bits = 0;
-    const u32 first_small = m > 16 ? m - 16 : 0;  // levels first_small..m have at most 16 variables
-    for (u32 l = first_small; l <= m; l++) {
-        js.job[n_jobs++] = dpk::EqJob{l, m - l, eq_level_off(m, l)};
-        max_bits = std::max(max_bits, m - l);
-    }
-    // seeds live in a scratch block behind nothing: a separate allocation
+    const u32 m = info.m;
+    const u32 first_small = eq_first_direct(m);  // levels first_small..m come straight from the definition
+    need &= (2ull << m) - 1;
+    u64 todo = need & ~info.built;
+    // a large level needs level l + 8
+    for (u32 l = 0; l < first_small; l++)
+        if (((todo >> l) & 1) && !((info.built >> (l + 8)) & 1)) todo |= 1ull << (l + 8);
+    const bool low = need_low && info.fact_levels && !info.fact_built;
+    if (!todo && !low) return DPS_OK;
+    std::vector<dpk::EqJob> jobs;
+    u32 n_large = 0;
+    for (u32 l = first_small; l <= m; l++)
+        if ((todo >> l) & 1) jobs.push_back(dpk::EqJob{l, m - l, eq_level_off(m, l)});
+    if (low)
+        for (u32 l = 1; l <= info.fact_levels; l++) jobs.push_back(dpk::EqJob{l, dpk::EQ_LO_BITS, eq_low_off(m, l)});
+    for (u32 l = 0; l < first_small; l++)
+        if ((todo >> l) & 1) n_large++;
+    // seeds live in a scratch block of their own, read by the expansions queued right behind
     void *seed_block = nullptr;
     u64 *seed0 = nullptr, *seed1 = nullptr;
-    if (first_small > 0) {
+    if (n_large) {
         CHK(pool_alloc(ctx, (size_t)first_small * 256 * 16, &seed_block));
         seed0 = (u64 *)seed_block;
         seed1 = seed0 + (size_t)first_small * 256;
     }
-    {
-        ProfScope ps(ctx, DPS_K_EQ, (double)(1ull << std::min<u32>(m, 16)) * 32.0);
-        dpk::eq_define_kernel<<<dim3((u32)(((1ull << max_bits) + dpk::BLOCK - 1) / dpk::BLOCK), n_jobs), dpk::BLOCK, 0, ctx->stream>>>(js);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) {
-            pool_free(ctx, seed_block);
-            return fail(ctx, DPS_ERR_HIP, "eq_define launch: %s", hipGetErrorString(e));
-        }
-    }
+    // the seeds of the large levels to build, in the same launch
+    for (u32 l = 0; l < first_small; l++)
+        if ((todo >> l) & 1) jobs.push_back(dpk::EqJob{l, 8, ((u64)l * 256) | dpk::EQ_JOB_SECOND});
     int32_t rc = DPS_OK;
-    if (first_small > 0) {
-        // seeds, up to EQ_MAX_JOBS per launch
-        for (u32 base = 0; base < first_small && rc == DPS_OK; base += dpk::EQ_MAX_JOBS) {
-            dpk::EqJobs ss;
-            memset(&ss, 0, sizeof ss);
-            memcpy(ss.point, js.point, sizeof ss.point);
-            ss.o0 = seed0;
-            ss.o1 = seed1;
-            u32 n = std::min<u32>(first_small - base, dpk::EQ_MAX_JOBS);
-            for (u32 k = 0; k < n; k++) ss.job[k] = dpk::EqJob{base + k, 8, (u64)(base + k) * 256};
-            dpk::eq_define_kernel<<<dim3(1, n), dpk::BLOCK, 0, ctx->stream>>>(ss);
+    auto run_jobs = [&](const std::vector<dpk::EqJob> &js_in, u64 *d0, u64 *d1) {
+        for (size_t base = 0; base < js_in.size() && rc == DPS_OK; base += dpk::EQ_MAX_JOBS) {
+            dpk::EqJobs js;
+            memset(&js, 0, sizeof js);
+            for (u32 i = 0; i < m; i++) {
+                js.point[2 * i] = info.point[i].c0;
+                js.point[2 * i + 1] = info.point[i].c1;
+            }
+            js.o0 = d0;
+            js.o1 = d1;
+            js.s0 = seed0;
+            js.s1 = seed1;
+            const u32 n = (u32)std::min<size_t>(js_in.size() - base, dpk::EQ_MAX_JOBS);
+            u32 max_bits = 0;
+            double entries = 0;
+            for (u32 k = 0; k < n; k++) {
+                js.job[k] = js_in[base + k];
+                max_bits = std::max(max_bits, js.job[k].n_bits);
+                entries += (double)(1ull << js.job[k].n_bits);
+            }
+            ProfScope ps(ctx, DPS_K_EQ, entries * 16.0);
+            // up to 16 workgroups share a job's rows of 256 entries
+            const u32 rows = max_bits > 8 ? 1u << (max_bits - 8) : 1;
+            dpk::eq_define_kernel<<<dim3(std::min<u32>(rows, 16), n), dpk::BLOCK, 0, ctx->stream>>>(js);
             hipError_t e = hipGetLastError();
-            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq seed launch: %s", hipGetErrorString(e));
+            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq_define launch: %s", hipGetErrorString(e));
         }
+    };
+    run_jobs(jobs, o0, o1);
+    if (n_large && rc == DPS_OK) {
+        // highest level first: level l reads level l + 8
         for (u32 l = first_small; l-- > 0 && rc == DPS_OK;) {
+            if (!((todo >> l) & 1)) continue;
             const u64 n_hi = 1ull << (m - l - 8);
             const u64 hi_off = eq_level_off(m, l + 8), out_off = eq_level_off(m, l);
             u32 blocks = (u32)std::min<u64>(n_hi, MAX_BLOCKS * 4);
@@ -836,31 +874,21 @@ int32_t eq_build_dev(dps_ctx *ctx, const u64 *point, u32 m, u64 *o0, u64 *o1)
     }
     // stream order makes the block reusable by later launches on this stream
     pool_free(ctx, seed_block);
+    if (rc == DPS_OK) {
+        info.built |= todo;
+        if (low) info.fact_built = true;
+    }
     return rc;
 }
 
-}  // namespace
-
-// the low tables of the large levels of an eq table (storage of eq_storage_entries(m) entries), one launch
-int32_t eq_build_low(dps_ctx *ctx, const EqInfo &info, u64 *o0, u64 *o1)
+// a table about to be read as ordinary entries: if it is an eq table, its level 0 has to be there
+int32_t plain_ready(const dps_mle *t)
 {
-    const u32 m = info.m;
-    if (!eq_fact_levels(m)) return DPS_OK;
-    dpk::EqJobs js;
-    memset(&js, 0, sizeof js);
-    for (u32 i = 0; i < m; i++) {
-        js.point[2 * i] = info.point[i].c0;
-        js.point[2 * i + 1] = info.point[i].c1;
-    }
-    js.o0 = o0;
-    js.o1 = o1;
-    u32 n_jobs = 0;
-    for (u32 l = 1; l <= eq_fact_levels(m); l++) js.job[n_jobs++] = dpk::EqJob{l, dpk::EQ_LO_BITS, eq_low_off(m, l)};
-    ProfScope ps(ctx, DPS_K_EQ, (double)n_jobs * (double)(1u << dpk::EQ_LO_BITS) * 16.0);
-    dpk::eq_define_kernel<<<dim3((1u << dpk::EQ_LO_BITS) / dpk::BLOCK, n_jobs), dpk::BLOCK, 0, ctx->stream>>>(js);
-    HIPCHK(ctx, hipGetLastError());
-    return DPS_OK;
+    if (!t || !t->eq || (t->eq->built & 1)) return DPS_OK;
+    return eq_ensure(t->ctx, *t->eq, t->st->c0, t->st->c1, 1, false);
 }
+
+}  // namespace
 
 extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m, dps_mle **out)
 {
@@ -871,15 +899,19 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     dps_mle *t = nullptr;
     CHK(new_table(ctx, DPS_EXT2, eq_storage_entries(m), &t));
     t->len = 1ull << m;
-    int32_t rc = eq_build_dev(ctx, point, m, t->st->c0, t->st->c1);
-    if (rc != DPS_OK) {
-        delete t;
-        return rc;
-    }
     t->eq = std::make_shared<EqInfo>();
     t->eq->m = m;
     t->eq->fact_levels = eq_fact_levels(m);
     for (u32 i = 0; i < m; i++) t->eq->point.push_back(gl::e2(point[2 * i], point[2 * i + 1]));
+    // Up to 17 variables everything comes out of one launch.  Of a larger table only the levels of at most 2^17 entries
+    // and the low tables are built now, in that one launch (what a product session reads, 13 MB at 24 variables); the
+    // large levels wait for whoever reads them.
+    const u64 small = ((2ull << m) - 1) & ~((1ull << eq_first_direct(m)) - 1);
+    int32_t rc = eq_ensure(ctx, *t->eq, t->st->c0, t->st->c1, small, true);
+    if (rc != DPS_OK) {
+        delete t;
+        return rc;
+    }
     *out = t;
     return DPS_OK;
 }
@@ -939,10 +971,12 @@ extern "C" int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points
         for (u32 k = 0; k < m[i]; k++) t->eq->point.push_back(gl::e2(points[i][2 * k], points[i][2 * k + 1]));
         if (m[i] > 16) {
             // large tables are built by expansion, one at a time
-            rc = eq_build_dev(ctx, points[i], m[i], t->st->c0, t->st->c1);
+            const u64 small = ((2ull << m[i]) - 1) & ~((1ull << eq_first_direct(m[i])) - 1);
+            rc = eq_ensure(ctx, *t->eq, t->st->c0, t->st->c1, small, true);
             if (rc != DPS_OK) return undo(rc);
             continue;
         }
+        t->eq->built = (2ull << m[i]) - 1;  // every level, by the launch below
         const size_t need = ((jobs.size() + m[i] + 1) * sizeof(dpk::EqJobM)) / 8 + pts.size() + 2 * (size_t)m[i];
         if (stage_lo + need > stage_hi || jobs.size() + m[i] + 1 > 65535) {
             rc = flush();
@@ -1054,8 +1088,13 @@ extern "C" int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint
     if (!is_pow2(mle->len) || (1ull << n) != mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate: point length does not match the table");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(mle));
     dps_mle *eq = nullptr;
     CHK(dps_eq_build(ctx, point, n, &eq));
+    if (int32_t rc_ = plain_ready(eq); rc_ != DPS_OK) {
+        delete eq;
+        return rc_;
+    }
     AxisJob j;
     j.in0 = mle->p0();
     j.in1 = mle->p1();
@@ -1084,8 +1123,13 @@ extern "C" int32_t dps_mle_fix_high(dps_ctx *ctx, const dps_mle *mle, const uint
     if (!is_pow2(mle->len) || (1ull << k) > mle->len) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_high: too many variables");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(mle));
     dps_mle *eq = nullptr;
     CHK(dps_eq_build(ctx, point, k, &eq));
+    if (int32_t rc_ = plain_ready(eq); rc_ != DPS_OK) {
+        delete eq;
+        return rc_;
+    }
     u64 rest = mle->len >> k;
     dps_mle *res = nullptr;
     int32_t rc = new_table(ctx, DPS_EXT2, rest, &res);
@@ -1124,6 +1168,7 @@ extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint6
     if (!canonical(point, 2 * (size_t)k)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_fix_low: point not canonical");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(mle));
     if (k == 0) return dps_mle_view(mle, 0, log2u(mle->len), out);
     // ping-pong between two buffers; the last one written becomes the result
     u64 len = mle->len;
@@ -1172,6 +1217,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
     if (tensor->pad_vars) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_partial_eval: the tensor is a zero-padded view");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(tensor));
     u64 padded_total = 1, contraction = 1, stacked = 1;
     for (u32 a = 0; a < n_dims; a++) {
         if (unpadded_dims[a] == 0 || unpadded_dims[a] > padded_dims[a]) return fail(ctx, DPS_ERR_INVALID, "dps_partial_eval: dimension %u", a);
@@ -1212,7 +1258,11 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         u32 m = log2u(padded_dims[oa]);
         dps_mle *beta = nullptr;
         rc = dps_eq_build(ctx, points[oa], m, &beta);
-        if (rc != DPS_OK) break;
+        if (rc == DPS_OK) rc = plain_ready(beta);
+        if (rc != DPS_OK) {
+            delete beta;
+            break;
+        }
         AxisJob j;
         j.in0 = in0;
         j.in1 = in1;
@@ -2040,10 +2090,6 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     // tables, which every table is once folded, so a start in round 2 needs extension tables to begin with)
     // a product with an eq factor reads the eq weights of its large rounds as products of two small tables: the low ones are
     // built now if this eq table has not served such a session before (they lie behind its levels; the table itself is not touched)
-    if (sc->fast && sc->fast_eq >= 0 && sc->eq_info->fact_levels && !sc->eq_info->fact_built) {
-        CHK(eq_build_low(ctx, *sc->eq_info, const_cast<u64 *>(sc->eq_c0), const_cast<u64 *>(sc->eq_c1)));
-        sc->eq_info->fact_built = true;
-    }
     sc->round_kind.assign(n_vars + 2, 0);
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
@@ -2052,6 +2098,22 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         bool all_ext = true;
         for (u32 f = 0; f < sc->fast_nf; f++) all_ext = all_ext && mles[sc->fast_order[f]]->kind == DPS_EXT2;
         plan_resident_rounds(sc.get(), all_ext ? 2 : 3);
+    }
+    // What this session reads of its tables: an eq table taken in closed form is read level by level -- level j in round j,
+    // except in the large rounds of a product, which take the low table of level j and level j + 16 instead -- and
+    // anything else as ordinary entries.  Whatever of that an eq table has not built yet is built now, on the stream.
+    for (u32 k = 0; k < n_mles; k++) {
+        if ((int)k == sc->fast_eq) {
+            u32 first_level = 1;
+            if (sc->fast) {
+                first_level = sc->eq_info->fact_levels + 1;
+                if (sc->tail_j0) first_level = std::min(first_level, sc->tail_j0);
+            }
+            const u64 need = ((2ull << n_vars) - 1) & ~((1ull << first_level) - 1);
+            CHK(eq_ensure(ctx, *sc->eq_info, const_cast<u64 *>(sc->eq_c0), const_cast<u64 *>(sc->eq_c1), need, sc->fast));
+        } else {
+            CHK(plain_ready(mles[k]));
+        }
     }
 
     // scratch: two ping-pong buffers per table, extension limbs
@@ -3147,6 +3209,7 @@ extern "C" int32_t dps_mle_evaluate_noalloc(dps_ctx *ctx, const dps_mle *mle, co
     if (!ctx->ws) return fail(ctx, DPS_ERR_STATE, "dps_mle_evaluate_noalloc: the context has no work area");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    CHK(plain_ready(mle));  // (an eq table that nobody has read yet: launches into its own storage, no allocation)
     dpk::WsPoint pt;
     memset(&pt, 0, sizeof pt);
     if (n) memcpy(pt.p, point, 16 * (size_t)n);

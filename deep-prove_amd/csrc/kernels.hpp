@@ -145,26 +145,51 @@ constexpr int EQ_MAX_JOBS = 48;
 constexpr int EQ_MAX_VARS = 34;
 struct EqJob {
     u32 first, n_bits;
-    u64 out_off;  // entries from the start of the output arrays
+    u64 out_off;  // entries from the start of the output arrays; bit 63: of the second pair of arrays (s0, s1)
 };
+constexpr u64 EQ_JOB_SECOND = 1ull << 63;
 struct EqJobs {
     u64 point[2 * EQ_MAX_VARS];  // 2 limbs per coordinate, travels in the kernel arguments
     u64 *o0, *o1;
+    u64 *s0, *s1;  // a second pair of output arrays (the seeds of an expansion live apart from the table)
     EqJob job[EQ_MAX_JOBS];
 };
 
+// A table of up to EQ_DIRECT_BITS variables is the outer product of the table of its 8 lowest variables (one entry per
+// thread, in a register) and the table of the others (worked out by the workgroup into LDS): about one product per
+// entry instead of one per entry and variable.  The workgroups of a job (gridDim.x of them) share its rows of 256 entries.
+constexpr u32 EQ_DIRECT_BITS = 17;
 __global__ void __launch_bounds__(BLOCK) eq_define_kernel(EqJobs js)
 {
+    static_assert(BLOCK == 256, "a row is the 8 lowest variables");
+    constexpr u32 HI_MAX = 1u << (EQ_DIRECT_BITS - 8);
+    __shared__ u64 hi0[HI_MAX], hi1[HI_MAX];
     const EqJob j = js.job[blockIdx.y];
-    const u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
-    if (i >= ((u64)1 << j.n_bits)) return;
-    E2 acc = gl::e2_one();
-    for (u32 b = 0; b < j.n_bits; b++) {
-        E2 r = gl::e2(js.point[2 * (j.first + b)], js.point[2 * (j.first + b) + 1]);
-        acc = gl::mul(acc, ((i >> b) & 1) ? r : gl::sub(gl::e2_one(), r));
+    const u32 lo_bits = j.n_bits < 8 ? j.n_bits : 8, hi_bits = j.n_bits - lo_bits, n_hi = 1u << hi_bits;
+    if (blockIdx.x >= n_hi) return;  // (the whole workgroup)
+    auto factor = [&](u32 var, u32 bit) {
+        const E2 r = gl::e2(js.point[2 * var], js.point[2 * var + 1]);
+        return bit ? r : gl::sub(gl::e2_one(), r);
+    };
+    const u32 t = threadIdx.x;
+    E2 lo = gl::e2_one();
+    for (u32 b = 0; b < lo_bits; b++) lo = gl::mul(lo, factor(j.first + b, (t >> b) & 1));
+    for (u32 h = t; h < n_hi; h += BLOCK) {
+        E2 v = gl::e2_one();
+        for (u32 b = 0; b < hi_bits; b++) v = gl::mul(v, factor(j.first + lo_bits + b, (h >> b) & 1));
+        hi0[h] = v.c0;
+        hi1[h] = v.c1;
     }
-    js.o0[j.out_off + i] = acc.c0;
-    js.o1[j.out_off + i] = acc.c1;
+    __syncthreads();
+    if (t >= (1u << lo_bits)) return;
+    const bool second = (j.out_off & EQ_JOB_SECOND) != 0;
+    u64 *o0 = (second ? js.s0 : js.o0) + (j.out_off & ~EQ_JOB_SECOND), *o1 = (second ? js.s1 : js.o1) + (j.out_off & ~EQ_JOB_SECOND);
+    const gl::E2P lp = gl::prep(lo);
+    for (u32 h = blockIdx.x; h < n_hi; h += gridDim.x) {
+        const E2 v = gl::mulp(gl::e2(hi0[h], hi1[h]), lp);
+        o0[((u64)h << lo_bits) | t] = v.c0;
+        o1[((u64)h << lo_bits) | t] = v.c1;
+    }
 }
 
 // The same for jobs of several tables at once (many small eq tables, each with its own point): descriptors and

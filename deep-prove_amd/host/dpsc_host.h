@@ -41,6 +41,11 @@ const char *dph_last_error(void);
 int32_t dph_sumcheck_prove(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
                            const dps_term *terms, uint32_t n_terms, dph_transcript *t, uint64_t *proof_out,
                            uint64_t *point_out, uint64_t *finals_out, uint32_t *degree_out);
+/* the same with the value of the whole sum stated by the caller, who holds it as the claim being reduced
+ * (zkml/src/layers/hadamard.rs:117-121): round 1 then takes p(1) from it, same messages */
+int32_t dph_sumcheck_prove_claimed(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
+                                   const dps_term *terms, uint32_t n_terms, const uint64_t claimed_sum[2], dph_transcript *t,
+                                   uint64_t *proof_out, uint64_t *point_out, uint64_t *finals_out, uint32_t *degree_out);
 /* IOPVerifierState::verify; returns 0 or DPS_ERR_INVALID when a round fails */
 int32_t dph_sumcheck_verify(const uint64_t claimed_sum[2], const uint64_t *proof, uint32_t n_vars, uint32_t degree,
                             dph_transcript *t, uint64_t *point_out, uint64_t expected_out[2]);

@@ -74,6 +74,13 @@ int32_t dph_sumcheck_prove(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *
                            const dps_term *terms, uint32_t n_terms, dph_transcript *t, uint64_t *proof_out,
                            uint64_t *point_out, uint64_t *finals_out, uint32_t *degree_out)
 {
+    return dph_sumcheck_prove_claimed(ctx, n_vars, mles, n_mles, terms, n_terms, nullptr, t, proof_out, point_out, finals_out, degree_out);
+}
+
+int32_t dph_sumcheck_prove_claimed(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
+                                   const dps_term *terms, uint32_t n_terms, const uint64_t claimed_sum[2], dph_transcript *t,
+                                   uint64_t *proof_out, uint64_t *point_out, uint64_t *finals_out, uint32_t *degree_out)
+{
     return guarded([&] {
         Context c(ctx);
         VirtualPolynomials vp;
@@ -81,7 +88,9 @@ int32_t dph_sumcheck_prove(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *
         vp.num_vars = n_vars;
         vp.mles.assign(mles, mles + n_mles);
         vp.terms.assign(terms, terms + n_terms);
-        auto res = IOPProverState::prove(vp, t->t);
+        F claim;
+        if (claimed_sum) claim = F(claimed_sum[0], claimed_sum[1]);
+        auto res = IOPProverState::prove(vp, t->t, claimed_sum ? &claim : nullptr);
         size_t npts = res.first.proofs.empty() ? 0 : res.first.proofs[0].evaluations.size();
         if (degree_out) *degree_out = npts ? (uint32_t)npts - 1 : 0;
         size_t w = 0;
