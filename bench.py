@@ -24,10 +24,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes of one round-2 launch at n = 24 from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, both
-# factors calibrated on the library's plain copy kernel); counters cannot be read from inside this script
-MEASURED_TRAFFIC_N24 = 540.2e6
 P = 0xFFFFFFFF00000001
+# Counters cannot be read from inside this script: the HBM bytes of one round-2 launch at n = 24 (rocprofv3 FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for the library's plain copy kernel) and the vector-ALU issue
+# shares of rounds 1 and 2 are taken from the committed summaries of those runs, as "key: value" lines.
+TRAFFIC_PROFILE = "profiles/prod_kernel_cfg3_n24_hbm_traffic.txt"
+VALU_PROFILE = "profiles/prod_kernel_cfg3_n24_valu.txt"
+
+
+def profile_value(path, key):
+    """the number on the line 'key: number' of a committed profile summary, or None"""
+    try:
+        for line in open(os.path.join(ROOT, path)):
+            if line.strip().startswith(key + ":"):
+                return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def rand_base(n, seed):
@@ -234,6 +247,14 @@ def main():
         tr = dp.Transcript(b"bench")
         return prover(tr), tr
 
+    def timed_loop(fn, steps):
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        ctx.sync()
+        return 1e3 * (time.perf_counter() - t0) / steps
+
     for _ in range(args.warmup):
         prove()
     ctx.sync()
@@ -250,6 +271,34 @@ def main():
     # every step proves the same statement: all proofs must be identical
     repeatable = all((q == proofs[0]).all() for q in proofs)
 
+    # The caller of the reference's hadamard prover holds the value of the sum (the claim it reduces, hadamard.rs:117-121);
+    # stated to the engine, round 1 takes p(1) from it.  Same proof; reported beside the headline, which does not use it.
+    p10 = [int(x) for x in proof[0][0]], [int(x) for x in proof[0][1]]
+    claim = np.array([(p10[0][0] + p10[1][0]) % P, (p10[0][1] + p10[1][1]) % P], dtype=np.uint64)
+    claimed = ctx.sumcheck_prover(n, [mf, mg, me], terms, claim=claim)
+    same_with_claim = bool((claimed(dp.Transcript(b"bench"))[0] == proofs[0]).all())
+    for _ in range(args.warmup):
+        claimed(dp.Transcript(b"bench"))
+    claimed_ms = timed_loop(lambda: claimed(dp.Transcript(b"bench")), args.steps)
+
+    # A fresh point every step, as in the reference's flow (hadamard.rs:103-115 builds the eq table for each proof): the eq
+    # build is inside the timed region.  The statement changes with the point, so these proofs are not compared.
+    points = [np.stack([rand_base(n, 1000 + 2 * k), rand_base(n, 1001 + 2 * k)], axis=-1) for k in range(args.steps + 2)]
+
+    def fresh(k):
+        e = ctx.eq_build(points[k])
+        out = ctx.sumcheck_prove(n, [mf, mg, e], terms, dp.Transcript(b"bench"))
+        e.free()
+        return out
+
+    fresh(args.steps), fresh(args.steps + 1)
+    ctx.sync()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        fresh(k)
+    ctx.sync()
+    fresh_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
     # same steps again with the library's HIP events on, for per-kernel durations
     ctx.profile(True)
     ctx.profile_reset()
@@ -261,9 +310,11 @@ def main():
     def gbs(by, ms):
         return by / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
 
-    # plain device copy moving as many bytes as the dominant launch does (half read, half written)
+    # plain device copy moving as many bytes as the dominant launch does (half read, half written), and a launch that
+    # only reads as many bytes as round 1 does
     copy_bytes = 8 * (1 << n) * 2
     copy_ms = ctx.copy_ms(copy_bytes, 10)
+    read_ms = ctx.read_ms(copy_bytes, 10)
 
     fe, ef = stats["fold_eval"], stats["eval_first"]
     # dominant kernel: the fused fold+evaluate launch of round 2.  It reads f and g
@@ -284,7 +335,8 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": MEASURED_TRAFFIC_N24 if n == 24 else None,
+        "traffic": profile_value(TRAFFIC_PROFILE, "round2_traffic_bytes") if n == 24 else None,
+        "traffic_source": TRAFFIC_PROFILE if n == 24 else None,
         "algorithmic_bytes_per_launch": dom_bytes,
         "avg_launch_ms": round(dom_ms, 5),
         "survey_bytes_per_launch": survey_round2,
@@ -292,6 +344,11 @@ def main():
         "copy_kernel_gbs": round(gbs(2 * copy_bytes, copy_ms), 1),
         "frac_of_copy_kernel": round(achieved / gbs(2 * copy_bytes, copy_ms), 4),
         "first_round_kernel_gbs": round(gbs(ef["bytes"], ef["ms"]), 1),
+        "read_kernel_gbs": round(gbs(copy_bytes, read_ms), 1),
+        "first_round_frac_of_read_kernel": round(gbs(ef["bytes"], ef["ms"]) / gbs(copy_bytes, read_ms), 4),
+        "valu_issue_share_round1": profile_value(VALU_PROFILE, "valu_issue_share_round1") if n == 24 else None,
+        "valu_issue_share_round2": profile_value(VALU_PROFILE, "valu_issue_share_round2") if n == 24 else None,
+        "valu_source": VALU_PROFILE if n == 24 else None,
         "all_rounds_algorithmic_bytes": stream_bytes,
         "all_rounds_survey_bytes": survey_total,
         "all_rounds_kernel_ms": round(stream_ms, 4),
@@ -319,6 +376,9 @@ def main():
         "field_elements_per_s": round(element_visits / (ms_per_step * 1e-3), 1),
         "min_step_ms": round(1e3 * min(per_step), 4),
         "eq_build_ms": round(eq_ms, 4),
+        "prove_with_fresh_eq_ms": round(fresh_ms, 4),
+        "prove_with_claim_ms": round(claimed_ms, 4),
+        "same_proof_with_claim": same_with_claim,
         "all_steps_identical": bool(repeatable),
         "upload_s": round(upload_s, 4),
         "roofline": roofline,

@@ -79,6 +79,8 @@ dev.dps_mle_zero_pad.argtypes = [_vp, _u32, _vp]
 dev.dps_debug_field_op.argtypes = [_vp, _i32, _vp, _vp, _u64, _vp]
 dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
+dev.dps_debug_read.restype = _i32
+dev.dps_debug_read.argtypes = [_vp, _u64, _u32, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
            "dps_partial_eval", "dps_sc_begin", "dps_sc_set_claim", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
@@ -554,6 +556,16 @@ class Context:
         ms = C.c_double(0)
         self._chk(dev.dps_debug_copy(self._c, n_bytes, reps, C.byref(ms)), "dps_debug_copy")
         return ms.value
+
+
+def _read_ms(self, n_bytes, reps=10):
+    """average duration of a launch that only streams n_bytes in (the yardstick of read-only launches)"""
+    ms = C.c_double(0)
+    self._chk(dev.dps_debug_read(self._c, n_bytes, reps, C.byref(ms)), "dps_debug_read")
+    return ms.value
+
+
+Context.read_ms = _read_ms
 
 
 # ---- einsum and LogUp drivers of the host mirror ----

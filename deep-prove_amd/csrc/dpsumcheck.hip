@@ -3434,3 +3434,39 @@ extern "C" int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps,
     if (avg_ms_out) *avg_ms_out = (double)ms / reps;
     return DPS_OK;
 }
+
+// the same for reads only: `reps` launches of a kernel that streams n_bytes in and writes nothing
+extern "C" int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out)
+{
+    if (!ctx || n_bytes == 0 || (n_bytes & 15) || reps == 0) return fail(ctx, DPS_ERR_INVALID, "dps_debug_read: bad argument");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, n_bytes + 8 * MAX_BLOCKS * 4, &p));
+    const uint4 *src = (const uint4 *)p;
+    u32 *sink = (u32 *)((char *)p + n_bytes);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipMemsetAsync(p, 0x5a, n_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    const u64 n16 = n_bytes / 16;
+    const u32 blocks = (u32)std::min<u64>((n16 + dpk::BLOCK - 1) / dpk::BLOCK, 8 * MAX_BLOCKS);
+    if (e == hipSuccess) {
+        dpk::read_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(src, n16, sink);  // untimed first touch
+        e = hipEventRecord(e0, ctx->stream);
+    }
+    for (u32 r = 0; r < reps && e == hipSuccess; r++) {
+        dpk::read_kernel<<<blocks, dpk::BLOCK, 0, ctx->stream>>>(src, n16, sink);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    pool_free(ctx, p);
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "read: %s", hipGetErrorString(e));
+    if (avg_ms_out) *avg_ms_out = (double)ms / reps;
+    return DPS_OK;
+}

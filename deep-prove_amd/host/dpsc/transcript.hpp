@@ -104,10 +104,14 @@ private:
         head[61] = (uint8_t)(n_rounds_ >> 16);
         head[62] = (uint8_t)(n_rounds_ >> 8);
         head[63] = (uint8_t)n_rounds_;
-        Blake3 h;
-        h.update(head, 64);
-        if (len) h.update(payload, len);
-        h.finalize(state_);
+        if (len <= 64) {
+            Blake3::hash_block_and(head, payload, len, state_);
+        } else {
+            Blake3 h;
+            h.update(head, 64);
+            h.update(payload, len);
+            h.finalize(state_);
+        }
         n_rounds_++;
     }
 };

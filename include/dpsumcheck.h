@@ -232,6 +232,8 @@ int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *a, const ui
  * counterpart in the reference; it is what the evaluation kernels' bandwidth
  * and the profiler's memory counters are read against. */
 int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
+/* the same for a launch that only reads n_bytes (what a round's first evaluation is read against) */
+int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
 
 #ifdef __cplusplus
 }

@@ -72,3 +72,30 @@ def test_expression_flattening_cpp(tmp_path):
     subprocess.check_call(["g++", "-O1", "-std=c++17", "-o", str(exe), os.path.join(ROOT, "tests", "cpp", "test_expression.cpp")])
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
+
+
+def test_blake3_vector_and_portable_compressions_agree(dp):
+    """The host mirror hashes with a 512-bit-permute compression where the CPU has AVX-512 and with a portable loop
+    elsewhere (DPSC_BLAKE3_PORTABLE forces the loop): same digests and the same transcript on both."""
+    import sys
+
+    script = (
+        "import importlib, sys, numpy as np\n"
+        "sys.path.insert(0, %r)\n"
+        "dp = importlib.import_module('deep-prove_amd')\n"
+        "out = [dp.blake3(bytes(range(256)) * k)[:8].hex() for k in (0, 1, 3, 5, 9)]\n"
+        "t = dp.Transcript(b'paths')\n"
+        "t.append_u64(7); t.append_bytes(b'x' * 100)\n"
+        "t.append_scalars(np.arange(10, dtype=np.uint64).reshape(5, 2))\n"
+        "out.append(t.append_and_sample(b'c').tolist()); out.append(t.state()[0].hex())\n"
+        "print(out)\n" % ROOT)
+    runs = []
+    for portable in (False, True):
+        env = dict(os.environ)
+        env.pop("DPSC_BLAKE3_PORTABLE", None)
+        if portable:
+            env["DPSC_BLAKE3_PORTABLE"] = "1"
+        res = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, env=env)
+        assert res.returncode == 0, res.stderr
+        runs.append(res.stdout.strip())
+    assert runs[0] == runs[1] and runs[0].startswith("['")
