@@ -1418,7 +1418,7 @@ struct dps_sc {
     struct Stage {
         u32 W, j0, pend0, n_trips, dbl_mask, cap;
         u64 src_len;
-        u64 *h0[3], *h1[3];  // several workgroups: where they leave their last entries (the next stage's source)
+        u64 *h0[dpk::SL_MAX_TABS], *h1[dpk::SL_MAX_TABS];  // where a stage that is not the last leaves its entries (the next stage's source)
     };
     std::vector<Stage> stages;
     std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip
@@ -1516,10 +1516,25 @@ void tail_abort(dps_ctx *ctx)
 // result area of the resident product launches (dpk::SL_AREA_WORDS words of the pinned buffer, behind the areas of resident groups)
 size_t slice_area_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64 + 64 * 32; }
 
-template <int NF, bool EQ>
-void launch_slice(dps_ctx *ctx, u32 workgroups, u32 cap, const dpk::SliceArgs &a)
+template <int NF, bool EQ, bool TERMS>
+void launch_slice(dps_ctx *ctx, u32 workgroups, u32 n_tabs, u32 cap, const dpk::SliceArgs &a)
 {
-    dpk::slice_kernel<NF, EQ><<<workgroups, dpk::BLOCK, dpk::slice_lds_words(NF, cap) * 8, ctx->stream>>>(a);
+    dpk::slice_kernel<NF, EQ, TERMS><<<workgroups, dpk::BLOCK, dpk::slice_lds_words(n_tabs, cap) * 8, ctx->stream>>>(a);
+}
+
+// the compiled variants: a product of 1 or 2 tables times eq, of 2 or 3 without; sums of several terms up to degree 4
+int32_t launch_slice_dispatch(dps_ctx *ctx, bool terms, u32 nf, bool eq, u32 workgroups, u32 n_tabs, u32 cap, const dpk::SliceArgs &a)
+{
+#define SK(NF_, EQ_, T_)                                                  \
+    if (terms == T_ && nf == NF_ && eq == EQ_) {                          \
+        launch_slice<NF_, EQ_, T_>(ctx, workgroups, n_tabs, cap, a);      \
+        return DPS_OK;                                                    \
+    }
+    SK(1, true, false) SK(2, true, false) SK(2, false, false) SK(3, false, false)
+    SK(1, true, true) SK(2, true, true) SK(3, true, true) SK(4, true, true)
+    SK(1, false, true) SK(2, false, true) SK(3, false, true) SK(4, false, true)
+#undef SK
+    return fail(ctx, DPS_ERR_UNSUPPORTED, "no resident kernel for degree %u, eq %d, several terms %d", nf, (int)eq, (int)terms);
 }
 
 template <int NF, int NB, bool EQ>
@@ -1797,31 +1812,38 @@ int32_t ensure_descs(dps_sc *sc)
 
 namespace {
 
-// pairs a workgroup of a resident launch takes in its first round (its LDS holds twice as many entries per table, and half of that again)
-u32 slice_pairs_per_workgroup(u32 nf) { return nf <= 2 ? 512 : 256; }
+// Pairs a workgroup of a resident launch takes in its first round: its LDS holds twice as many entries per table and half
+// of that again, within the 64 KB a launch gets without asking; a sum of several terms does several times a product's
+// arithmetic per pair, so its workgroups take fewer.
+u32 slice_pairs_per_workgroup(u32 n_tabs, bool terms)
+{
+    u32 cap = 1024;
+    while (dpk::slice_lds_words(n_tabs, cap) * 8 > 65536) cap >>= 1;
+    return terms ? std::min<u32>(cap / 2, 128) : cap / 2;
+}
 constexpr u32 SLICE_MAX_WORKGROUPS = 256;
 
-// Which rounds of a product session are resident, in which launches, and how they pair up into trips.  `first_ok`: the
-// first round whose source tables are extension tables.  A trip covers two rounds when the second one's p(1) can come
-// from the claim (its eq coordinate is not zero) and the workgroups still hold a quad each.
-void plan_resident_rounds(dps_sc *sc, u32 first_ok)
+// Which rounds of a session are resident, in which launches, and how they pair up into trips.  `n_tabs`: tables in LDS.
+// A trip covers two rounds when the second one's p(1) can come from the claim (its eq coordinate is not zero) and the
+// workgroups still hold a quad each.  The first resident round is the first whose pairs fit 256 workgroups.
+void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
 {
-    const u32 n = sc->n_vars, nf = sc->fast_nf;
+    const u32 n = sc->n_vars;
     const bool has_eq = sc->fast_eq >= 0;
-    if (first_ok > n) return;
+    const u32 first_ok = 1;
     auto claim_gives_p1 = [&](u32 round) {
         if (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0) return false;
         if (!has_eq) return true;
         const E2 rho = sc->eq_info->point[round - 1];
         return !(rho.c0 == 0 && rho.c1 == 0);
     };
-    const u32 per_wg = slice_pairs_per_workgroup(nf);
+    const u32 per_wg = slice_pairs_per_workgroup(n_tabs, sc->poly);
     auto pairs_of = [&](u32 round) { return (u64)1 << (n - round); };
     u32 j = first_ok;
     while (pairs_of(j) > (u64)per_wg * SLICE_MAX_WORKGROUPS) j++;
     sc->tail_j0 = j;
-    u64 entries = (u64)1 << (n - j + 2);  // of the tables the stage to come starts from (before its pending folds)
-    u32 pend = 1;
+    u32 pend = j == 1 ? 0 : 1;                   // a launch that starts with round 1 has nothing to fold first
+    u64 entries = (u64)1 << (n - j + 1 + pend);  // of the tables the stage to come starts from (before its pending folds)
     auto add_stage = [&](u32 W) {
         dps_sc::Stage st;
         memset(&st, 0, sizeof st);
@@ -2094,10 +2116,12 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
     sc->prev_chal = gl::e2_zero();
-    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
-        bool all_ext = true;
-        for (u32 f = 0; f < sc->fast_nf; f++) all_ext = all_ext && mles[sc->fast_order[f]]->kind == DPS_EXT2;
-        plan_resident_rounds(sc.get(), all_ext ? 2 : 3);
+    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) plan_resident_rounds(sc.get(), sc->fast_nf);
+    // a sum of several terms over one group of full-size tables (a fraction-sum layer, a claim merge): the same launches
+    if (sc->poly && sc->poly_tabs.size() == 1 && sc->fast_nf <= 4 && sc->n_terms <= (u32)dpk::SL_MAX_TERMS) {
+        bool ok = n_mles == sc->poly_tabs[0].size() + (sc->fast_eq >= 0 ? 1 : 0);
+        for (u32 k : sc->poly_tabs[0]) ok = ok && nv0[k] == n_vars && !mles[k]->pad_vars;
+        if (ok) plan_resident_rounds(sc.get(), (u32)sc->poly_tabs[0].size());
     }
     // What this session reads of its tables: an eq table taken in closed form is read level by level -- level j in round j,
     // except in the large rounds of a product, which take the low table of level j and level j + 16 instead -- and
@@ -2342,7 +2366,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     size_t bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
     // what a resident stage that does not run to the last round leaves for the next: two limb arrays per table
     size_t bytes_hand = 0;
-    for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * sc->fast_nf;
+    const u32 slice_tabs = sc->poly ? (sc->poly_tabs.empty() ? 0u : (u32)sc->poly_tabs[0].size()) : sc->fast_nf;
+    for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * slice_tabs;
     size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result + bytes_hand;
     int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
     if (rc != DPS_OK) return cleanup(rc);
@@ -2369,7 +2394,7 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     p += bytes_result;
     for (size_t i = 0; i + 1 < sc->stages.size(); i++) {
         const size_t limb = round_up((size_t)sc->stages[i + 1].src_len * 8, 256);
-        for (u32 f = 0; f < sc->fast_nf; f++) {
+        for (u32 f = 0; f < slice_tabs; f++) {
             sc->stages[i].h0[f] = (u64 *)p;
             p += limb;
             sc->stages[i].h1[f] = (u64 *)p;
@@ -2695,12 +2720,33 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 const dps_sc::Stage &st = sc->stages[si];
                 dpk::SliceArgs sa;
                 memset(&sa, 0, sizeof sa);
-                for (u32 f = 0; f < nf; f++) {
+                const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : nf;
+                for (u32 f = 0; f < n_tabs; f++) {
                     // the first stage reads what the launch of the round before it wrote (or the session's own tables)
-                    sa.s0[f] = si == 0 ? sc->fast_args[first].s0[f] : sc->stages[si - 1].h0[f];
-                    sa.s1[f] = si == 0 ? sc->fast_args[first].s1[f] : sc->stages[si - 1].h1[f];
+                    if (si > 0) {
+                        sa.s0[f] = sc->stages[si - 1].h0[f];
+                        sa.s1[f] = sc->stages[si - 1].h1[f];
+                    } else if (sc->poly) {
+                        const dpk::PolyTab &tb = sc->h_poly_groups[first - 1].tab[f];
+                        sa.s0[f] = tb.s0;
+                        sa.s1[f] = tb.s1;
+                    } else {
+                        sa.s0[f] = sc->fast_args[first].s0[f];
+                        sa.s1[f] = sc->fast_args[first].s1[f];
+                    }
                     sa.h0[f] = st.h0[f];
                     sa.h1[f] = st.h1[f];
+                }
+                sa.n_tabs = n_tabs;
+                if (sc->poly) {
+                    sa.n_terms = (u32)sc->h_poly_terms.size();
+                    for (u32 m = 0; m < sa.n_terms; m++) {
+                        const dpk::PolyTerm &pt = sc->h_poly_terms[m];
+                        dpk::SliceTerm &tm = sa.terms[m];
+                        tm.c0 = pt.c0, tm.c1 = pt.c1, tm.w = pt.w;
+                        tm.n_factors = pt.n_factors;
+                        memcpy(tm.slot, pt.slot, sizeof tm.slot);
+                    }
                 }
                 sa.src_len = st.src_len;
                 sa.pend0 = st.pend0;
@@ -2721,11 +2767,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 sa.ctr = ctx->d_slice_ctr;
                 sa.ticket = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
                 ProfScope ps(ctx, DPS_K_TAIL, 0.0);
-                if (has_eq && nf == 1) launch_slice<1, true>(ctx, st.W, st.cap, sa);
-                else if (has_eq && nf == 2) launch_slice<2, true>(ctx, st.W, st.cap, sa);
-                else if (!has_eq && nf == 2) launch_slice<2, false>(ctx, st.W, st.cap, sa);
-                else if (!has_eq && nf == 3) launch_slice<3, false>(ctx, st.W, st.cap, sa);
-                else return fail(ctx, DPS_ERR_UNSUPPORTED, "no resident kernel for %u tables, eq %d", nf, (int)has_eq);
+                CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
                 HIPCHK(ctx, hipGetLastError());
             }
             sc->tail_seq0 = seq0;
@@ -2942,7 +2984,12 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                         skip1_next = !(rho.c0 == 0 && rho.c1 == 0);
                     }
                     const Plan pn = plan_round(j + 1, skip1_next);
-                    {
+                    if (sc->tail_j0 && j + 1 == sc->tail_j0) {
+                        // the rounds from here on are resident: their launches are queued now and wait for their first mail
+                        CHK(launch_stages_at(ctx->seq + 1));
+                        sc->wait_fresh = true;
+                        sc->ahead_at = std::chrono::steady_clock::now();
+                    } else {
                         CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
                         sc->tail_running = true;
                         sc->tail_seq0 = ctx->seq + 1;
@@ -3073,24 +3120,25 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         // the resident launch published value and slope of every table's last pair with its last round: the final
         // evaluations are value + r * slope
         const E2 r = gl::e2(challenge[0], challenge[1]);
-        u64 w[4 * dpk::POLY_MAXT];
+        u64 w[8 * dpk::SL_MAX_TABS];
         // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
         // groups are resident), the single-product one its factors
-        if (!sc->poly) {
-            // a product session: the resident launch left 2 entries per table, or 4 when its last trip covered two rounds
-            // (the challenge between them is the one the last round's call brought)
+        if (!sc->stages.empty()) {
+            // the resident launch left 2 entries per table, or 4 when its last trip covered two rounds (the challenge
+            // between them is the one the last round's call brought)
             const u32 L = sc->fin_len;
-            CHK(wait_result_at(ctx, slice_area_off(ctx), sc->pairs_seq, dpk::SL_FIN_SLOT, 2 * L * sc->fast_nf, w, dpk::SL_FIN_SEQ_SLOT, dpk::SL_FIN_CHK_SLOT));
-            for (u32 f = 0; f < sc->fast_nf; f++) {
+            const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : sc->fast_nf;
+            CHK(wait_result_at(ctx, slice_area_off(ctx), sc->pairs_seq, dpk::SL_FIN_SLOT, 2 * L * n_tabs, w, dpk::SL_FIN_SEQ_SLOT, dpk::SL_FIN_CHK_SLOT));
+            for (u32 f = 0; f < n_tabs; f++) {
                 auto at = [&](u32 e) { return gl::e2(w[2 * (f * L + e)], w[2 * (f * L + e) + 1]); };
                 auto fold = [](E2 lo, E2 hi, E2 c) { return gl::add(lo, gl::mul(c, gl::sub(hi, lo))); };
                 const E2 v = L == 4 ? fold(fold(at(0), at(1), sc->prev_chal), fold(at(2), at(3), sc->prev_chal), r) : fold(at(0), at(1), r);
-                const u32 k = sc->fast_order[f];
+                const u32 k = sc->poly ? sc->poly_tabs[0][f] : sc->fast_order[f];
                 final_evals_out[2 * k] = v.c0;
                 final_evals_out[2 * k + 1] = v.c1;
             }
         }
-        const u32 n_areas = sc->poly ? (u32)sc->poly_tabs.size() : 0;
+        const u32 n_areas = sc->poly && sc->stages.empty() ? (u32)sc->poly_tabs.size() : 0;
         for (u32 g = 0; g < n_areas; g++) {
             const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[g].size() : sc->fast_nf;
             const size_t base = sc->poly_raw ? poly_raw_off(ctx) + 64 * (size_t)g : ctx->res_off;

@@ -971,16 +971,27 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 // counters, per wavefront in LDS, then per launch in device memory (agent-scope atomics, one ticket per workgroup);
 // whoever takes the last ticket recombines and publishes.
 // ---------------------------------------------------------------------------
-constexpr int SL_MAX_SUMS = 16;  // (NF + 1)^2 extension sums per trip at NF = 3
+constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
 constexpr int SL_SEQ_SLOT = 2 * SL_MAX_SUMS, SL_CHK_SLOT = SL_SEQ_SLOT + 1;
 // with the last trip of a run to the last round: the entries every table still has (2, or 4 after a trip of two rounds)
-constexpr int SL_FIN_SLOT = 40, SL_FIN_SEQ_SLOT = 64, SL_FIN_CHK_SLOT = 65, SL_AREA_WORDS = 128;
+constexpr int SL_FIN_SLOT = 56, SL_FIN_SEQ_SLOT = 112, SL_FIN_CHK_SLOT = 113, SL_AREA_WORDS = 128;
 constexpr int SL_MAX_TRIPS = 32;
+constexpr int SL_MAX_TABS = 7;    // tables of a sum of several terms (a product has at most 3)
+constexpr int SL_MAX_TERMS = 24;
+static_assert(SL_FIN_SLOT + 2 * 4 * SL_MAX_TABS <= SL_FIN_SEQ_SLOT && 2 * 4 * SL_MAX_TABS <= WAVE, "the last entries of every table fit the result area and one wavefront");
+// a term of a sum of several terms: coefficient (prepared: w = 7 c1) times the tables in `slot`
+struct SliceTerm {
+    u64 c0, c1, w;
+    u32 n_factors;
+    uint8_t slot[DPS_MAX_FACTORS];
+    u32 pad;
+};
 struct SliceArgs {
-    const u64 *s0[3];
-    const u64 *s1[3];  // the tables before the folds that are pending when the launch starts: src_len entries each
+    const u64 *s0[SL_MAX_TABS];
+    const u64 *s1[SL_MAX_TABS];  // the tables before the folds that are pending when the launch starts: src_len entries each
+                                 // (nullptr: base-field entries; only tables nothing has folded yet are)
     u64 src_len;
-    u32 pend0;         // folds pending at the first trip: 1 (the challenge of the round before), or 2
+    u32 pend0;         // folds pending at the first trip: 0 (the launch starts with round 1), 1, or 2
     u32 n_vars, j0;    // the sum's variables; first round evaluated here (1-based)
     u32 n_trips;
     u32 dbl_mask;      // bit k: trip k covers two rounds
@@ -995,36 +1006,51 @@ struct SliceArgs {
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
     u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero between trips
     u32 *ticket;       // ... and their ticket counter
-    u64 *h0[3];        // not finishing: where each workgroup leaves its last state (workgroup-major), to be folded by the next launch
-    u64 *h1[3];
+    u64 *h0[SL_MAX_TABS];  // not finishing: where each workgroup leaves its last state (workgroup-major), to be folded by the next launch
+    u64 *h1[SL_MAX_TABS];
+    // a sum of several terms (TERMS): the tables are those of all terms, the polynomial summed is sum_k coeff_k prod table
+    u32 n_tabs, n_terms;
+    SliceTerm terms[SL_MAX_TERMS];
 };
 
-// dynamic LDS of slice_kernel, in 64-bit words: counters per wavefront, mailbox copy, flags, then the two table buffers
-constexpr u32 SL_LDS_CTR = 0, SL_LDS_BOX = (BLOCK / WAVE) * 4 * SL_MAX_SUMS, SL_LDS_FLAGS = SL_LDS_BOX + 8, SL_LDS_TABLES = SL_LDS_FLAGS + 2;
-__host__ __device__ constexpr u32 slice_lds_words(u32 nf, u32 cap) { return SL_LDS_TABLES + nf * 2 * (cap + cap / 2); }
+// dynamic LDS of slice_kernel, in 64-bit words: counters per wavefront, mailbox copy, flags, the terms, then the two table buffers
+constexpr u32 SL_LDS_CTR = 0, SL_LDS_BOX = (BLOCK / WAVE) * 4 * SL_MAX_SUMS, SL_LDS_FLAGS = SL_LDS_BOX + 8, SL_LDS_TERMS = SL_LDS_FLAGS + 2;
+constexpr u32 SL_LDS_TABLES = SL_LDS_TERMS + SL_MAX_TERMS * (sizeof(SliceTerm) / 8);
+static_assert(sizeof(SliceTerm) % 8 == 0, "terms are copied as 64-bit words");
+__host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap) { return SL_LDS_TABLES + n_tabs * 2 * (cap + cap / 2); }
 
-template <int NF, bool EQ>
+// NF: tables of the product, or with TERMS the largest number of factors of a term (the degree of the polynomial summed)
+template <int NF, bool EQ, bool TERMS>
 __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
 {
     constexpr int NP = NF + 1;          // sums of the trip's first round: q(0..NF), q(1) left zero when it comes from the claim
     constexpr int NPT = NF;             // points of its second round: t = 0, 2, .., NF
     constexpr int NSMP = NF + 1;        // samples of that round's sums as a polynomial in the challenge: 0..NF-1, leading coefficient
     constexpr int NS = NP + NSMP * NPT; // extension sums per trip
+    constexpr int MAXT = TERMS ? SL_MAX_TABS : NF;
     static_assert(NS <= SL_MAX_SUMS, "sums per trip fit the result area");
     extern __shared__ u64 dyn[];
     u64 *const ctr = dyn + SL_LDS_CTR;  // [wavefront][4 * SL_MAX_SUMS]
     u64 *const box = dyn + SL_LDS_BOX;
     int *const ok_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS);
     int *const last_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS + 1);
+    const SliceTerm *const lterms = reinterpret_cast<const SliceTerm *>(dyn + SL_LDS_TERMS);
     const u32 tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const u32 W = gridDim.x, wg = blockIdx.x;
+    const u32 nt = TERMS ? a.n_tabs : (u32)NF;  // tables
     const u64 src_wg = a.src_len / W;             // this workgroup's share of the source
     u32 len = (u32)(src_wg >> a.pend0);           // entries per table once the pending folds are done
     const u32 cap = len;
     // two buffers per limb array: `cap` entries and half of that; a fold reads one and writes the other
-    u64 *const buf_big = dyn + SL_LDS_TABLES, *const buf_small = buf_big + (size_t)NF * 2 * cap;
+    u64 *const buf_big = dyn + SL_LDS_TABLES, *const buf_small = buf_big + (size_t)nt * 2 * cap;
     bool in_big = true;  // where the current state is
-    auto tab = [&](bool big, int f, int limb) -> u64 * { return big ? buf_big + (size_t)(f * 2 + limb) * cap : buf_small + (size_t)(f * 2 + limb) * (cap / 2); };
+    auto tab = [&](bool big, u32 f, int limb) -> u64 * { return big ? buf_big + (size_t)(f * 2 + limb) * cap : buf_small + (size_t)(f * 2 + limb) * (cap / 2); };
+    if (TERMS) {
+        // the terms are read per pair and point: staged in LDS once (visible after the first wait's barrier)
+        const u64 *src = reinterpret_cast<const u64 *>(a.terms);
+        u64 *dst = dyn + SL_LDS_TERMS;
+        for (u32 w = tid; w < a.n_terms * (u32)(sizeof(SliceTerm) / 8); w += BLOCK) dst[w] = src[w];
+    }
 
     u32 j = a.j0, pend = a.pend0;
     u64 trip_seq = a.seq0;
@@ -1034,21 +1060,32 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
         if (!wait_first_mail(a.mail, W > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
         if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
         const bool skip1 = box[MAIL_SKIP1] != 0;
-        const gl::E2P rb = gl::prep(gl::e2(box[MAIL_R], box[MAIL_R + 1])), ra = gl::prep(gl::e2(box[MAIL_RA], box[MAIL_RA + 1]));
+        const E2 rb_ = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+        const gl::E2P rb = gl::prep(rb_), ra = gl::prep(gl::e2(box[MAIL_RA], box[MAIL_RA + 1]));
         // ---- the pending folds ----
         if (k == 0) {
-            // from device memory: entry i of the state is made of the source's entries 2i, 2i+1 (one fold) or 4i..4i+3 (two)
+            // from device memory: entry i of the state is the source's entry i (nothing pending), or is made of its entries
+            // 2i, 2i+1 (one fold) or 4i..4i+3 (two)
             const u64 base = (u64)wg * src_wg;
             for (u32 i = tid; i < len; i += BLOCK) {
 #pragma unroll
-                for (int f = 0; f < NF; f++) {
+                for (u32 f = 0; f < (u32)MAXT; f++) {
+                    if (f >= nt) break;
+                    const u64 *p0 = a.s0[f], *p1 = a.s1[f];
                     E2 v;
-                    if (pend == 1) {
-                        const U64x2 x0 = ld2(a.s0[f] + base + 2 * (u64)i), x1 = ld2(a.s1[f] + base + 2 * (u64)i);
-                        v = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb);
+                    if (pend == 0) {
+                        v = gl::e2(p0[base + i], p1 ? p1[base + i] : 0);
+                    } else if (pend == 1) {
+                        const U64x2 x0 = ld2(p0 + base + 2 * (u64)i);
+                        if (p1) {
+                            const U64x2 x1 = ld2(p1 + base + 2 * (u64)i);
+                            v = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb);
+                        } else {
+                            v = fold1_base(x0.x, x0.y, rb_);
+                        }
                     } else {
-                        const U64x2 x0 = ld2(a.s0[f] + base + 4 * (u64)i), y0 = ld2(a.s0[f] + base + 4 * (u64)i + 2);
-                        const U64x2 x1 = ld2(a.s1[f] + base + 4 * (u64)i), y1 = ld2(a.s1[f] + base + 4 * (u64)i + 2);
+                        const U64x2 x0 = ld2(p0 + base + 4 * (u64)i), y0 = ld2(p0 + base + 4 * (u64)i + 2);
+                        const U64x2 x1 = ld2(p1 + base + 4 * (u64)i), y1 = ld2(p1 + base + 4 * (u64)i + 2);
                         v = fold1p(fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), ra), fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), ra), rb);
                     }
                     tab(true, f, 0)[i] = v.c0;
@@ -1059,7 +1096,8 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
             len >>= pend;
             for (u32 i = tid; i < len; i += BLOCK) {
 #pragma unroll
-                for (int f = 0; f < NF; f++) {
+                for (u32 f = 0; f < (u32)MAXT; f++) {
+                    if (f >= nt) break;
                     const u64 *c0 = tab(in_big, f, 0), *c1 = tab(in_big, f, 1);
                     E2 v;
                     if (pend == 1)
@@ -1076,9 +1114,7 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
         // this wavefront's counters start the trip at zero
         for (u32 c = lane; c < 4 * (u32)NS; c += WAVE) ctr[wave * 4 * SL_MAX_SUMS + c] = 0;
         __syncthreads();
-        const u64 *c0[NF], *c1[NF];
-#pragma unroll
-        for (int f = 0; f < NF; f++) c0[f] = tab(in_big, f, 0), c1[f] = tab(in_big, f, 1);
+        const bool big = in_big;
         // adds a lane's canonical sum into the counters of extension sum `idx`
         auto flush = [&](u32 idx, E2 v) {
             u64 *c = ctr + wave * 4 * SL_MAX_SUMS + 4 * idx;
@@ -1086,6 +1122,44 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
             atomicAdd(reinterpret_cast<unsigned long long *>(c + 1), (unsigned long long)(v.c0 >> 32));
             atomicAdd(reinterpret_cast<unsigned long long *>(c + 2), (unsigned long long)(u32)v.c1);
             atomicAdd(reinterpret_cast<unsigned long long *>(c + 3), (unsigned long long)(v.c1 >> 32));
+        };
+        // entry e of table f of the state
+        auto ent = [&](u32 f, u32 e) { return gl::e2(tab(big, f, 0)[e], tab(big, f, 1)[e]); };
+        // the polynomial summed, from its tables' values: the product of all tables, or sum_k coeff_k prod table (a table's
+        // value is asked for by `val(f)`, each time a term names it: the values live in LDS, not in registers a term
+        // could not index)
+        // `top_only`: only the terms of NF factors (the leading coefficient in the challenge belongs to them alone)
+        auto poly_of = [&](auto &&val, bool top_only = false) -> E2 {
+            if (!TERMS) {
+                E2 prod = val(0);
+#pragma unroll
+                for (u32 f = 1; f < (u32)NF; f++) prod = gl::mulp(prod, gl::prep(val(f)));
+                return prod;
+            }
+            gl::E2Acc G = gl::e2acc_zero();
+            for (u32 m = 0; m < a.n_terms; m++) {
+                const SliceTerm &tm = lterms[m];
+                if (top_only && tm.n_factors < (u32)NF) continue;
+                gl::E2P cp;
+                cp.c0 = tm.c0;
+                cp.c1 = tm.c1;
+                cp.w = tm.w;
+                E2 prod = gl::e2_one();
+                if (tm.n_factors > 0) {
+                    prod = val(tm.slot[0]);
+                    for (u32 f = 1; f < tm.n_factors; f++) prod = gl::mulp(prod, gl::prep(val(tm.slot[f])));
+                }
+                gl::acc_mul(G, prod, cp);
+            }
+            return gl::acc_reduce(G);
+        };
+        // lo + t (hi - lo) for the small t of the evaluation points
+        auto line_at = [](E2 lo, E2 hi, u32 t) {
+            if (t == 0) return lo;
+            const E2 d = gl::sub(hi, lo);
+            E2 v = hi;
+            for (u32 m = 1; m < t; m++) v = gl::add(v, d);
+            return v;
         };
         // ---- round j: pairs of the state; taken from the last thread down, so that with few pairs and quads they meet different lanes ----
         {
@@ -1099,26 +1173,11 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
                 any = true;
                 gl::E2P wp = gl::prep(gl::e2_one());
                 if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + p], a.eq1[eq_off + p]));
-                E2 lo[NF], hi[NF], dl[NF], cur[NF];
-#pragma unroll
-                for (int f = 0; f < NF; f++) {
-                    lo[f] = gl::e2(c0[f][2 * p], c1[f][2 * p]);
-                    hi[f] = gl::e2(c0[f][2 * p + 1], c1[f][2 * p + 1]);
-                    dl[f] = gl::sub(hi[f], lo[f]);
-                    cur[f] = lo[f];
-                }
 #pragma unroll
                 for (int t = 0; t < NP; t++) {
-                    if (!(t == 1 && skip1)) {
-                        E2 prod = cur[0];
-#pragma unroll
-                        for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
-                        acc[t] = EQ ? gl::fma(prod, wp, acc[t]) : gl::add(acc[t], prod);
-                    }
-                    if (t + 1 < NP) {
-#pragma unroll
-                        for (int f = 0; f < NF; f++) cur[f] = (t == 0) ? hi[f] : gl::add(cur[f], dl[f]);
-                    }
+                    if (t == 1 && skip1) continue;
+                    const E2 g = poly_of([&](u32 f) { return line_at(ent(f, 2 * p), ent(f, 2 * p + 1), (u32)t); });
+                    acc[t] = EQ ? gl::fma(g, wp, acc[t]) : gl::add(acc[t], g);
                 }
             }
             if (any) {
@@ -1142,43 +1201,19 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
                     any = true;
                     gl::E2P wp = gl::prep(gl::e2_one());
                     if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + u], a.eq1[eq_off + u]));
-                    E2 lo[NF], dl[NF], cur[NF];
-#pragma unroll
-                    for (int f = 0; f < NF; f++) {
-                        const E2 e0 = gl::e2(c0[f][4 * u], c1[f][4 * u]), e1 = gl::e2(c0[f][4 * u + 1], c1[f][4 * u + 1]);
-                        const E2 e2_ = gl::e2(c0[f][4 * u + 2], c1[f][4 * u + 2]), e3 = gl::e2(c0[f][4 * u + 3], c1[f][4 * u + 3]);
-                        const E2 d01 = gl::sub(e1, e0), d23 = gl::sub(e3, e2_);
-                        E2 hi;
-                        if (smp == (u32)NF) {
-                            // leading coefficient: the slopes in place of the folded entries
-                            lo[f] = d01;
-                            hi = d23;
-                        } else {
-                            // the pair folded with the challenge at smp: e0 + smp (e1 - e0), e2 + smp (e3 - e2)
-                            lo[f] = e0;
-                            hi = e2_;
-                            for (u32 m = 0; m < smp; m++) {
-                                lo[f] = gl::add(lo[f], d01);
-                                hi = gl::add(hi, d23);
-                            }
-                        }
-                        dl[f] = gl::sub(hi, lo[f]);
-                        cur[f] = lo[f];
-                    }
+                    // a table's pair of round j + 1 with the challenge of round j at this lane's sample: e0 + smp (e1 - e0) and
+                    // e2 + smp (e3 - e2); for the leading coefficient the slopes e1 - e0, e3 - e2 in their place
+                    auto sampled = [&](u32 f, u32 t) {
+                        const E2 e0 = ent(f, 4 * u), e1 = ent(f, 4 * u + 1), e2_ = ent(f, 4 * u + 2), e3 = ent(f, 4 * u + 3);
+                        if (smp == (u32)NF) return line_at(gl::sub(e1, e0), gl::sub(e3, e2_), t);
+                        return line_at(line_at(e0, e1, smp), line_at(e2_, e3, smp), t);
+                    };
                     // points t = 0, 2, .., NF
 #pragma unroll
                     for (int ti = 0; ti < NPT; ti++) {
-                        if (ti == 1) {
-#pragma unroll
-                            for (int f = 0; f < NF; f++) cur[f] = gl::add(gl::add(lo[f], dl[f]), dl[f]);
-                        } else if (ti > 1) {
-#pragma unroll
-                            for (int f = 0; f < NF; f++) cur[f] = gl::add(cur[f], dl[f]);
-                        }
-                        E2 prod = cur[0];
-#pragma unroll
-                        for (int f = 1; f < NF; f++) prod = gl::mulp(prod, gl::prep(cur[f]));
-                        acc[ti] = EQ ? gl::fma(prod, wp, acc[ti]) : gl::add(acc[ti], prod);
+                        const u32 t = ti == 0 ? 0 : (u32)ti + 1;
+                        const E2 g = poly_of([&](u32 f) { return sampled(f, t); }, smp == (u32)NF);
+                        acc[ti] = EQ ? gl::fma(g, wp, acc[ti]) : gl::add(acc[ti], g);
                     }
                 }
             }
@@ -1248,15 +1283,14 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
     if (!a.finish) {
         // to device memory, for the launch queued behind this one (which starts with this launch's pending folds)
         for (u32 i = tid; i < len; i += BLOCK) {
-#pragma unroll
-            for (int f = 0; f < NF; f++) {
+            for (u32 f = 0; f < nt; f++) {
                 a.h0[f][(u64)wg * len + i] = tab(big, f, 0)[i];
                 a.h1[f][(u64)wg * len + i] = tab(big, f, 1)[i];
             }
         }
     } else if (wave == 0) {
         // to the host, which does the last fold or two: entry e of table f at words 2 (f len + e), + 1
-        const u32 n_words = (u32)NF * len * 2;
+        const u32 n_words = nt * len * 2;
         const bool mine = lane < n_words;
         u64 word = 0;
         if (mine) {

@@ -88,21 +88,36 @@ struct Stage {
     std::vector<std::pair<u32, bool>> trips;  // first round, covers two rounds
 };
 
-// NF tables, sum of n_vars variables, resident from round j0 on; `wide`: workgroups of the first stage (1: a single stage);
-// `single_rounds`: rounds that must start a trip of their own with t = 1 evaluated (an eq point with a zero coordinate there)
-template <int NF, bool EQ>
-static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pairs, std::vector<u32> single_rounds = {})
+struct Term {
+    E2 coeff;
+    std::vector<u32> tabs;
+};
+
+// A sum of n_vars variables, resident from round j0 on (j0 = 1: from the start, nothing folded yet); `wide`: workgroups of
+// the first stage (1: a single stage); `single_rounds`: rounds that must start a trip of their own with t = 1 evaluated (an
+// eq point with a zero coordinate there).  TERMS = false: the product of NF tables.  TERMS = true: sum_k coeff_k prod tables
+// over `n_tabs` tables, NF the largest number of factors; `base_tabs` of the tables are base-field ones (j0 <= 2 only).
+template <int NF, bool EQ, bool TERMS = false>
+static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_in, std::vector<u32> single_rounds = {}, std::vector<Term> terms = {},
+                     u32 base_tabs = 0)
 {
     constexpr int NP = NF + 1, NPT = NF, NSMP = NF + 1, NS = NP + NSMP * NPT;
+    const u32 NT = TERMS ? n_tabs_in : (u32)NF;
+    if (!TERMS) {
+        Term t{gl::e2_one(), {}};
+        for (u32 f = 0; f < NT; f++) t.tabs.push_back(f);
+        terms = {t};
+    }
+    const u32 first_pend = j0 == 1 ? 0 : 1;
     auto is_single = [&](u32 j) {
         for (u32 x : single_rounds)
             if (x == j) return true;
         return false;
     };
     // reference tables: the state before round j0's pending fold, and the challenges of every round
-    std::vector<Table> ref(NF, Table((size_t)1 << (n_vars - j0 + 2)));
-    for (auto &t : ref)
-        for (auto &x : t) x = felt2();
+    std::vector<Table> ref(NT, Table((size_t)1 << (n_vars - j0 + 1 + first_pend)));
+    for (u32 f = 0; f < NT; f++)
+        for (auto &x : ref[f]) x = f < base_tabs ? gl::e2(felt(), 0) : felt2();
     std::vector<E2> chal(n_vars + 1);
     for (auto &c : chal) c = felt2();
     // eq storage: level l at (2 << n) - (2 << (n - l)), eq(rho_{l..n-1}, .)
@@ -122,8 +137,8 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
     std::vector<Stage> stages;
     {
         u32 j = j0;
-        u64 entries = (u64)1 << (n_vars - j0 + 2);  // of the state the next stage starts from
-        u32 pend = 1;
+        u64 entries = (u64)1 << (n_vars - j0 + 1 + first_pend);  // of the state the next stage starts from
+        u32 pend = first_pend;
         if (wide > 1) {
             Stage st{wide, j, pend, entries, {}};
             u64 len_wg = (entries / wide) >> pend;
@@ -149,20 +164,19 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
         }
         stages.push_back(st);
     }
-    (void)cap_pairs;
 
     std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
     u32 ticket = 0;
     const u64 seq_first = 1000;
     bool ok = true;
     // device-side tables of the stage to come
-    std::vector<std::vector<u64>> d0(NF), d1(NF);
-    for (int f = 0; f < NF; f++) {
+    std::vector<std::vector<u64>> d0(NT), d1(NT);
+    for (u32 f = 0; f < NT; f++) {
         d0[f].resize(ref[f].size()), d1[f].resize(ref[f].size());
         for (size_t i = 0; i < ref[f].size(); i++) d0[f][i] = ref[f][i].c0, d1[f][i] = ref[f][i].c1;
     }
     std::vector<Table> state = ref;  // reference state, folded as the challenges are "drawn"
-    u32 folded_through = j0 - 2;     // the state has been folded with the challenges of rounds <= folded_through
+    u32 folded_through = j0 - 1 - first_pend;  // the state has been folded with the challenges of rounds <= folded_through
     auto fold_to = [&](u32 round) {  // bring the reference state to the tables of `round`
         while (folded_through < round - 1) {
             folded_through++;
@@ -174,9 +188,13 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
         for (int t = 0; t <= NF; t++) q[t] = gl::e2_zero();
         for (size_t p = 0; p < tabs[0].size() / 2; p++)
             for (int t = 0; t <= NF; t++) {
-                E2 prod = EQ ? eq_level(round, p) : gl::e2_one();
-                for (int f = 0; f < NF; f++) prod = gl::mul(prod, gl::add(tabs[f][2 * p], gl::mul_base(gl::sub(tabs[f][2 * p + 1], tabs[f][2 * p]), (u64)t)));
-                q[t] = gl::add(q[t], prod);
+                E2 g = gl::e2_zero();
+                for (auto &tm : terms) {
+                    E2 prod = tm.coeff;
+                    for (u32 f : tm.tabs) prod = gl::mul(prod, gl::add(tabs[f][2 * p], gl::mul_base(gl::sub(tabs[f][2 * p + 1], tabs[f][2 * p]), (u64)t)));
+                    g = gl::add(g, prod);
+                }
+                q[t] = gl::add(q[t], EQ ? gl::mul(g, eq_level(round, p)) : g);
             }
     };
 
@@ -184,10 +202,11 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
         const Stage &st = stages[si];
         dpk::SliceArgs a;
         memset(&a, 0, sizeof a);
-        std::vector<std::vector<u64>> h0(NF), h1(NF);
-        for (int f = 0; f < NF; f++) {
+        std::vector<std::vector<u64>> h0(NT), h1(NT);
+        for (u32 f = 0; f < NT; f++) {
             a.s0[f] = d0[f].data();
-            a.s1[f] = d1[f].data();
+            // a table nothing has folded yet may be a base-field one (no second limb array)
+            a.s1[f] = (si == 0 && f < base_tabs) ? nullptr : d1[f].data();
             h0[f].assign(st.src_len, 0);
             h1[f].assign(st.src_len, 0);
             a.h0[f] = h0[f].data();
@@ -209,10 +228,18 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
         a.seq0 = seq_first + (st.j0 - j0);
         a.ctr = gctr.data();
         a.ticket = &ticket;
+        a.n_tabs = NT;
+        a.n_terms = TERMS ? (u32)terms.size() : 0;
+        for (size_t m = 0; TERMS && m < terms.size(); m++) {
+            a.terms[m].c0 = terms[m].coeff.c0, a.terms[m].c1 = terms[m].coeff.c1;
+            a.terms[m].w = gl::mul_small(terms[m].coeff.c1, (u32)gl::W);
+            a.terms[m].n_factors = (u32)terms[m].tabs.size();
+            for (size_t f = 0; f < terms[m].tabs.size(); f++) a.terms[m].slot[f] = (uint8_t)terms[m].tabs[f];
+        }
         const u32 cap = (u32)((st.src_len / st.W) >> st.pend0);
         std::vector<std::unique_ptr<emu::Group>> groups;
         std::vector<std::vector<u64>> lds;
-        auto threads = launch_all(st.W, dpk::slice_lds_words(NF, cap), dpk::slice_kernel<NF, EQ>, a, groups, lds);
+        auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap), dpk::slice_kernel<NF, EQ, TERMS>, a, groups, lds);
         // ---- the host's side ----
         u32 len_after = 0;
         for (size_t k = 0; k < st.trips.size() && ok; k++) {
@@ -220,7 +247,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
             const bool dbl = st.trips[k].second;
             const u64 seq = seq_first + (j - j0);
             const bool skip1 = !is_single(j);
-            mail[dpk::MAIL_R] = chal[j - 1].c0, mail[dpk::MAIL_R + 1] = chal[j - 1].c1;
+            mail[dpk::MAIL_R] = j >= 1 ? chal[j - 1].c0 : 0, mail[dpk::MAIL_R + 1] = j >= 1 ? chal[j - 1].c1 : 0;
             mail[dpk::MAIL_RA] = j >= 2 ? chal[j - 2].c0 : 0, mail[dpk::MAIL_RA + 1] = j >= 2 ? chal[j - 2].c1 : 0;
             mail[dpk::MAIL_SKIP1] = skip1;
             u64 chk = seq;
@@ -267,7 +294,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
                     for (auto &t : state) tmp.push_back(fold(t, gl::e2((u64)s, 0)));
                     round_sums(tmp, j + 1, c[s]);
                 }
-                const int pts[3] = {0, 2, 3};
+                const int pts[4] = {0, 2, 3, 4};
                 for (int ti = 0; ti < NPT && ok; ti++) {
                     const int t = pts[ti];
                     for (int s = 0; s < NF; s++)
@@ -332,11 +359,11 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
             fold_to(last.first);
             const u64 left = state[0].size();
             if (left != stages[si + 1].src_len) ok = false, printf("%s: stage leaves %llu entries, the next expects %llu\n", name, (unsigned long long)left, (unsigned long long)stages[si + 1].src_len);
-            for (int f = 0; f < NF && ok; f++) {
+            for (u32 f = 0; f < NT && ok; f++) {
                 d0[f].assign(left, 0), d1[f].assign(left, 0);
                 for (u64 i = 0; i < left; i++) {
                     if (h0[f][i] != state[f][i].c0 || h1[f][i] != state[f][i].c1) {
-                        printf("%s: handed-over entry %llu of table %d differs\n", name, (unsigned long long)i, f);
+                        printf("%s: handed-over entry %llu of table %u differs\n", name, (unsigned long long)i, f);
                         ok = false;
                         break;
                     }
@@ -349,19 +376,19 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 cap_pai
             fold_to(last.first);
             const u64 seq = seq_first + (last.first - j0);
             u64 c = seq;
-            const u32 n_words = NF * len_after * 2;
+            const u32 n_words = NT * len_after * 2;
             for (u32 i = 0; i < n_words; i++) c ^= dpk::rotl64(area[dpk::SL_FIN_SLOT + i], i + 1);
             if (area[dpk::SL_FIN_SEQ_SLOT] != seq || area[dpk::SL_FIN_CHK_SLOT] != c) ok = false, printf("%s: last entries not handed over\n", name);
             if (state[0].size() != len_after) ok = false, printf("%s: %zu entries left, %u expected\n", name, state[0].size(), len_after);
-            for (int f = 0; f < NF && ok; f++)
+            for (u32 f = 0; f < NT && ok; f++)
                 for (u32 e = 0; e < len_after; e++)
                     if (area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e)] != state[f][e].c0 || area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e) + 1] != state[f][e].c1)
-                        ok = false, printf("%s: last entry %u of table %d differs\n", name, e, f);
+                        ok = false, printf("%s: last entry %u of table %u differs\n", name, e, f);
         }
     }
     size_t n_trips = 0;
     for (auto &s : stages) n_trips += s.trips.size();
-    printf("%-60s NF=%d eq=%d n=%u from round %u, %zu stage(s), %zu trips for %u rounds : %s\n", name, NF, (int)EQ, n_vars, j0, stages.size(), n_trips,
+    printf("%-60s degree %d eq=%d n=%u from round %u, %zu stage(s), %zu trips for %u rounds : %s\n", name, NF, (int)EQ, n_vars, j0, stages.size(), n_trips,
            n_vars - j0 + 1, ok ? "ok" : "MISMATCH");
     if (!ok) failures++;
 }
@@ -375,6 +402,15 @@ int main()
     run_case<2, false>("two tables, rounds that must go alone (t = 1 evaluated)", 9, 2, 1, 0, {4, 7});
     run_case<2, true>("four workgroups, then one", 12, 3, 4, 0);
     run_case<2, true>("two workgroups down to one entry each, rounds that must go alone", 11, 3, 2, 0, {6});
+    run_case<2, true>("from round 1 (nothing folded yet)", 8, 1, 1, 0);
+    // sums of several terms: a LogUp layer eq (a d + b c + lambda c d), then higher degrees, base-field tables, constants
+    const Term la{felt2(), {0, 3}}, lb{felt2(), {1, 2}}, lc{felt2(), {2, 3}};
+    run_case<2, true, true>("fraction-sum layer: 4 tables, 3 terms, from round 1", 7, 1, 1, 4, {}, {la, lb, lc});
+    run_case<2, true, true>("the same over 4 workgroups, then one", 11, 2, 4, 4, {}, {la, lb, lc});
+    run_case<3, false, true>("degree 3 without eq: repeated and single factors, a constant term", 8, 2, 1, 5, {5},
+                             {Term{felt2(), {0, 1, 2}}, Term{felt2(), {3, 3, 4}}, Term{felt2(), {4}}, Term{felt2(), {}}});
+    run_case<4, false, true>("degree 4, base-field tables, from round 1", 6, 1, 1, 3, {}, {Term{felt2(), {0, 0, 1, 2}}, Term{felt2(), {1, 2}}}, 2);
+    run_case<2, true, true>("base-field tables folded once on the way in (from round 2)", 9, 2, 2, 3, {}, {Term{felt2(), {0, 1}}, Term{felt2(), {1, 2}}}, 2);
     printf("%s\n", failures ? "FAILED" : "all cases ok");
     return failures ? 1 : 0;
 }

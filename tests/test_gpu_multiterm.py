@@ -162,10 +162,13 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     has changed nothing yet: when another call needs the context, or the caller is slow, it ends, and the session
     carries on with ordinary launches and the same messages."""
     import time
-    n = 14
+    # 11 tables are several groups: launches of their own up to round 5 (a launch stays for the later rounds from
+    # n - j + 1 <= 9 on).  4 tables are one group, whose rounds are resident from the first that fits 256 workgroups of 128
+    # pairs (round 3 of 18): rounds 1 and 2 are launches, and the resident launches are queued during round 2.
+    n, afters = (14, (1, 3, 4, 5)) if n_tabs > 7 else (18, (1, 2))
     gpu, host, terms = _instance(ctx, orc, 900 + n_tabs, n, [n] * n_tabs, [], 2 * n_tabs, 2, True)
     ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
-    for after in (1, 3, 4, 5):  # up to round 5 no launch has stayed for later rounds (that takes n - j + 1 <= 9)
+    for after in afters:
         for how in ("other call", "slow caller"):
             s = ctx.session(n, gpu, terms)
             chal = None
@@ -183,13 +186,14 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     _check(dp, ctx, orc, n, gpu, host, terms)
 
 
-@pytest.mark.parametrize("with_eq,n", [(True, 14), (False, 14), (True, 19), (False, 18)])
+@pytest.mark.parametrize("with_eq,n", [(True, 20), (False, 20), (True, 21)])
 def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
-    """The same for a single product of full-size tables: round 2 and the resident launches of the rounds from 3 on
-    (several workgroups, then one) are made during the round before.  In a launch of more than 64 workgroups
-    (round 2 at n = 18, 19) only the first workgroup looks for the mail and passes it on to the others; the resident
-    launch of several workgroups always does so.  Once a resident launch has had its first mail another call on the
-    context ends the session (test_resident_kernel_gives_way)."""
+    """The same for a single product of full-size tables.  Its rounds are resident from the first that fits 256
+    workgroups of 512 pairs (round 3 of 20, round 4 of 21); the rounds before are launches, each made during the round
+    before it, and so are the resident launches (several workgroups, then one).  In a launch of more than 64
+    workgroups only the first workgroup looks for the mail and passes it on to the others; the resident launch of
+    several workgroups always does so.  Once a resident launch has had its first mail another call on the context ends
+    the session (test_resident_kernel_gives_way)."""
     import time
     f, g = rand_base(1 << n, 31), rand_e2(1 << n, 32)
     gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
