@@ -1422,6 +1422,8 @@ struct dps_sc {
     };
     std::vector<Stage> stages;
     std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip
+    std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip)
+    u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
     E2 prev_chal;                     // the challenge of the call before this one
     E2 stash[dpk::SL_MAX_SUMS];       // a trip of two rounds: the second round's sums as a polynomial in the first round's challenge
     u64 last_trip_seq;
@@ -1516,13 +1518,36 @@ void tail_abort(dps_ctx *ctx)
 // result area of the resident product launches (dpk::SL_AREA_WORDS words of the pinned buffer, behind the areas of resident groups)
 size_t slice_area_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 64 + 64 * 32; }
 
+// A workgroup of a resident launch may take most of a compute unit's LDS (it is alone there: 1024 threads); more than
+// 64 KB has to be asked for, once per kernel and device.  What a launch of this kernel can have, in bytes.
+constexpr u32 SLICE_LDS_DEFAULT = 64 * 1024, SLICE_LDS_LARGE = 160 * 1024;
+template <int NF, bool EQ, bool TERMS>
+u32 slice_lds_granted(dps_ctx *ctx)
+{
+    static std::atomic<int> granted[64];  // 0 not asked, 1 granted, 2 refused
+    std::atomic<int> &gr = granted[ctx->device & 63];
+    int v = gr.load();
+    if (v == 0) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&dpk::slice_kernel<NF, EQ, TERMS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)SLICE_LDS_LARGE);
+        if (e != hipSuccess) (void)hipGetLastError();
+        v = e == hipSuccess ? 1 : 2;
+        gr.store(v);
+    }
+    return v == 1 ? SLICE_LDS_LARGE : SLICE_LDS_DEFAULT;
+}
+
 template <int NF, bool EQ, bool TERMS>
 void launch_slice(dps_ctx *ctx, u32 workgroups, u32 n_tabs, u32 cap, const dpk::SliceArgs &a)
 {
-    dpk::slice_kernel<NF, EQ, TERMS><<<workgroups, dpk::BLOCK, dpk::slice_lds_words(n_tabs, cap) * 8, ctx->stream>>>(a);
+    dpk::slice_kernel<NF, EQ, TERMS><<<workgroups, dpk::SL_BLOCK, dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8, ctx->stream>>>(a);
 }
 
 // the compiled variants: a product of 1 or 2 tables times eq, of 2 or 3 without; sums of several terms up to degree 4
+#define SLICE_VARIANTS(SK)                                                              \
+    SK(1, true, false) SK(2, true, false) SK(2, false, false) SK(3, false, false)       \
+    SK(1, true, true) SK(2, true, true) SK(3, true, true) SK(4, true, true)             \
+    SK(1, false, true) SK(2, false, true) SK(3, false, true) SK(4, false, true)
 int32_t launch_slice_dispatch(dps_ctx *ctx, bool terms, u32 nf, bool eq, u32 workgroups, u32 n_tabs, u32 cap, const dpk::SliceArgs &a)
 {
 #define SK(NF_, EQ_, T_)                                                  \
@@ -1530,11 +1555,18 @@ int32_t launch_slice_dispatch(dps_ctx *ctx, bool terms, u32 nf, bool eq, u32 wor
         launch_slice<NF_, EQ_, T_>(ctx, workgroups, n_tabs, cap, a);      \
         return DPS_OK;                                                    \
     }
-    SK(1, true, false) SK(2, true, false) SK(2, false, false) SK(3, false, false)
-    SK(1, true, true) SK(2, true, true) SK(3, true, true) SK(4, true, true)
-    SK(1, false, true) SK(2, false, true) SK(3, false, true) SK(4, false, true)
+    SLICE_VARIANTS(SK)
 #undef SK
     return fail(ctx, DPS_ERR_UNSUPPORTED, "no resident kernel for degree %u, eq %d, several terms %d", nf, (int)eq, (int)terms);
+}
+// LDS a launch of the variant can have; 0: no such variant
+u32 slice_lds_limit(dps_ctx *ctx, bool terms, u32 nf, bool eq)
+{
+#define SK(NF_, EQ_, T_) \
+    if (terms == T_ && nf == NF_ && eq == EQ_) return slice_lds_granted<NF_, EQ_, T_>(ctx);
+    SLICE_VARIANTS(SK)
+#undef SK
+    return 0;
 }
 
 template <int NF, int NB, bool EQ>
@@ -1812,15 +1844,16 @@ int32_t ensure_descs(dps_sc *sc)
 
 namespace {
 
-// Pairs a workgroup of a resident launch takes in its first round: its LDS holds twice as many entries per table and half
-// of that again, within the 64 KB a launch gets without asking; a sum of several terms does several times a product's
-// arithmetic per pair, so its workgroups take fewer.
-u32 slice_pairs_per_workgroup(u32 n_tabs, bool terms)
+// Most pairs a workgroup of a resident launch can take in its first round: its LDS holds twice as many entries per table
+// and half of that again.
+u32 slice_pairs_per_workgroup(u32 n_tabs, u32 lds_bytes)
 {
-    u32 cap = 1024;
-    while (dpk::slice_lds_words(n_tabs, cap) * 8 > 65536) cap >>= 1;
-    return terms ? std::min<u32>(cap / 2, 128) : cap / 2;
+    u32 cap = 4096;
+    while (cap > 2 && dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8 > lds_bytes) cap >>= 1;
+    return cap / 2;
 }
+// ... and the fewest it is given when the sum is small enough for that: shorter chains of work per lane, more workgroups
+constexpr u32 SLICE_MIN_PAIRS = 128;
 constexpr u32 SLICE_MAX_WORKGROUPS = 256;
 
 // Which rounds of a session are resident, in which launches, and how they pair up into trips.  `n_tabs`: tables in LDS.
@@ -1837,10 +1870,15 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
         const E2 rho = sc->eq_info->point[round - 1];
         return !(rho.c0 == 0 && rho.c1 == 0);
     };
-    const u32 per_wg = slice_pairs_per_workgroup(n_tabs, sc->poly);
+    const u32 lds_bytes = slice_lds_limit(sc->ctx, sc->poly, sc->fast_nf, has_eq);
+    if (lds_bytes == 0) return;
+    // (more pairs per workgroup would make more rounds resident, but a trip's arithmetic is a workgroup's alone: with 512
+    // pairs of a 3-term sum the first trip took 75 us where a launch for the round and a trip of 128 pairs take 66)
+    const u32 per_wg_max = std::min<u32>(slice_pairs_per_workgroup(n_tabs, lds_bytes), sc->poly ? 128 : 512);
     auto pairs_of = [&](u32 round) { return (u64)1 << (n - round); };
     u32 j = first_ok;
-    while (pairs_of(j) > (u64)per_wg * SLICE_MAX_WORKGROUPS) j++;
+    while (pairs_of(j) > (u64)per_wg_max * SLICE_MAX_WORKGROUPS) j++;
+    const u32 per_wg = (u32)std::min<u64>(per_wg_max, std::max<u64>(SLICE_MIN_PAIRS, pairs_of(j) / SLICE_MAX_WORKGROUPS));
     sc->tail_j0 = j;
     u32 pend = j == 1 ? 0 : 1;                   // a launch that starts with round 1 has nothing to fold first
     u64 entries = (u64)1 << (n - j + 1 + pend);  // of the tables the stage to come starts from (before its pending folds)
@@ -1858,6 +1896,7 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
             if (dbl) st.dbl_mask |= 1u << st.n_trips;
             st.n_trips++;
             sc->round_kind[j] = dbl ? 2 : 1;
+            sc->round_wide[j] = W > 1;
             if (dbl) sc->round_kind[j + 1] = 3;
             pend = dbl ? 2 : 1;
             j += pend;
@@ -2113,6 +2152,8 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     // a product with an eq factor reads the eq weights of its large rounds as products of two small tables: the low ones are
     // built now if this eq table has not served such a session before (they lie behind its levels; the table itself is not touched)
     sc->round_kind.assign(n_vars + 2, 0);
+    sc->round_wide.assign(n_vars + 2, 0);
+    memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
     sc->prev_chal = gl::e2_zero();
@@ -2517,6 +2558,42 @@ int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n,
     }
 }
 
+// The sums of a trip of a resident launch: the four counters of each of `n_sums` sums, one word each at the start of the
+// launch's result area, whole once it carries the trip's tag (dpk::sl_tag) in its top byte.  `skip1`: the counters of
+// q(1) do not come (zeros are returned for them).  The tags are cleared as the words are taken, so that a word of 128
+// trips ago cannot pass for this trip's.
+int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u64 *out)
+{
+    volatile u64 *base = ctx->h_pinned + slice_area_off(ctx);
+    const u64 tag = dpk::sl_tag(seq);
+    u32 c = 0;
+    const u32 n = 4 * n_sums;
+    auto take = [&]() {
+        for (; c < n; c++) {
+            if (skip1 && c >= 4 && c < 8) {
+                out[c] = 0;
+                continue;
+            }
+            const u64 v = __atomic_load_n(base + c, __ATOMIC_ACQUIRE);
+            if ((v >> 56) != tag) return false;
+            out[c] = v & dpk::SL_CTR_MASK;
+            base[c] = 0;
+        }
+        return true;
+    };
+    for (u64 spins = 0;; spins++) {
+        if (take()) return DPS_OK;
+        if ((spins & 0xFFFFF) == 0xFFFFF) {
+            hipError_t q = hipStreamQuery(ctx->stream);
+            if (q == hipSuccess) {
+                if (take()) return DPS_OK;
+                return fail(ctx, DPS_ERR_HIP, "round result was not published");
+            }
+            if (q != hipErrorNotReady) return fail(ctx, DPS_ERR_HIP, "stream error while waiting for a round: %s", hipGetErrorString(q));
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
@@ -2718,6 +2795,10 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             const u32 first = sc->tail_j0;
             for (size_t si = 0; si < sc->stages.size(); si++) {
                 const dps_sc::Stage &st = sc->stages[si];
+                // a stage of several workgroups and the single-workgroup stage that runs to the last round are one launch:
+                // the first workgroup takes the others' entries up and goes on alone
+                const bool merged = st.W > 1 && si + 2 == sc->stages.size() && sc->stages[si + 1].W == 1 && sc->stages[si + 1].cap <= st.cap;
+                const size_t last_si = merged ? si + 1 : si;
                 dpk::SliceArgs sa;
                 memset(&sa, 0, sizeof sa);
                 const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : nf;
@@ -2754,6 +2835,10 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 sa.j0 = st.j0;
                 sa.n_trips = st.n_trips;
                 sa.dbl_mask = st.dbl_mask;
+                if (merged) {
+                    sa.n_trips2 = sc->stages[si + 1].n_trips;
+                    sa.dbl_mask2 = sc->stages[si + 1].dbl_mask;
+                }
                 sa.eq0 = sc->eq_c0;
                 sa.eq1 = sc->eq_c1;
                 sa.mail = ctx->d_pinned + (ctx->res_off - 64);
@@ -2761,15 +2846,21 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 // all 256 of them polling host memory a trip took 90 us instead of 18)
                 sa.relay = mail_relay(ctx);
                 sa.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
-                sa.finish = si + 1 == sc->stages.size() ? 1 : 0;
+                sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
                 sa.out_host = ctx->d_pinned + slice_area_off(ctx);
                 sa.seq0 = seq0 + (st.j0 - first);
                 sa.ctr = ctx->d_slice_ctr;
-                sa.ticket = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
+                sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
                 ProfScope ps(ctx, DPS_K_TAIL, 0.0);
                 CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
                 HIPCHK(ctx, hipGetLastError());
+                // a launch of several workgroups that nobody takes over from inside leaves its counters as they are
+                if (st.W > 1 && !merged) reset_device_words(ctx);
+                si = last_si;
             }
+            memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
+            // no resident launch of this context is running now: whatever an abandoned one left in the result area goes
+            for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
             sc->tail_seq0 = seq0;
             sc->tail_running = true;
             sc->wait_any_skip1 = true;
@@ -2813,9 +2904,23 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
                 prepare_message();
                 // sums of this round, and with a trip of two rounds those of the next
                 const u32 ns = kind == 2 ? np + np * nf : np;
-                u64 w[2 * dpk::SL_MAX_SUMS];
-                rc = wait_result_at(ctx, slice_area_off(ctx), fa.seq, 0, 2 * ns, w, dpk::SL_SEQ_SLOT, dpk::SL_CHK_SLOT);
+                u64 cnt[4 * dpk::SL_MAX_SUMS];
+                rc = wait_slice_sums(ctx, fa.seq, ns, a.skip1 != 0, cnt);
                 if (rc == DPS_OK) {
+                    // several workgroups: the counters run on from trip to trip of the launch
+                    if (sc->round_wide[j])
+                        for (u32 c = 0; c < 4 * ns; c++) {
+                            if (a.skip1 && c >= 4 && c < 8) continue;
+                            const u64 now = cnt[c];
+                            cnt[c] = now - sc->ctr_seen[c];
+                            sc->ctr_seen[c] = now;
+                        }
+                    // limb w & 1 of sum w >> 1: counters 2w (low halves) and 2w + 1 (high halves)
+                    u64 w[2 * dpk::SL_MAX_SUMS];
+                    for (u32 i = 0; i < 2 * ns; i++) {
+                        const unsigned __int128 t = (unsigned __int128)cnt[2 * i] + ((unsigned __int128)cnt[2 * i + 1] << 32);
+                        w[i] = gl::reduce128((u64)t, (u64)(t >> 64));
+                    }
                     for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
                     for (u32 i = np; i < ns; i++) sc->stash[i - np] = gl::e2(w[2 * i], w[2 * i + 1]);
                     form_message(q);

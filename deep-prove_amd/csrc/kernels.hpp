@@ -968,13 +968,22 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 // folds twice.  Same field elements as one round at a time; half the trips.
 //
 // Sums are added up as plain integers: a lane's canonical sums are cut into 32-bit halves and added into 64-bit
-// counters, per wavefront in LDS, then per launch in device memory (agent-scope atomics, one ticket per workgroup);
-// whoever takes the last ticket recombines and publishes.
+// counters, per wavefront in LDS, then per launch in device memory: one agent-scope atomic add per workgroup and counter,
+// which adds the workgroup's share to the low 56 bits and one to the top byte.  The counters are never cleared during a
+// launch (the host subtracts what the trip before left there; 2^10 lanes x 2^8 workgroups x 2^5 trips of 32-bit values stay
+// below 2^56), so the top byte counts the adds: the workgroup whose add makes it a multiple of the number of workgroups has
+// been handed, by that same atomic, the sum of everyone else's shares, and passes the total straight on to the host.  No
+// ticket, no fence, no second trip through device memory.  The host recombines the halves and reduces.
 // ---------------------------------------------------------------------------
 constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
-constexpr int SL_SEQ_SLOT = 2 * SL_MAX_SUMS, SL_CHK_SLOT = SL_SEQ_SLOT + 1;
+// A trip's result: the 4 counters of every sum (32-bit halves of both limbs, added up as integers), one word each in the
+// first 4 * SL_MAX_SUMS words of the result area: the count in the low 56 bits, the trip's tag in the top byte.  A word
+// is one store, so it is whole when its tag is there; the host clears the tags it has taken.
+constexpr u64 SL_CTR_MASK = (1ull << 56) - 1, SL_CTR_ONE = 1ull << 56;
+__host__ __device__ __forceinline__ u64 sl_tag(u64 trip_seq) { return 0x80 | (trip_seq & 0x7F); }
 // with the last trip of a run to the last round: the entries every table still has (2, or 4 after a trip of two rounds)
-constexpr int SL_FIN_SLOT = 56, SL_FIN_SEQ_SLOT = 112, SL_FIN_CHK_SLOT = 113, SL_AREA_WORDS = 128;
+constexpr int SL_FIN_SLOT = 104, SL_FIN_SEQ_SLOT = 160, SL_FIN_CHK_SLOT = 161, SL_AREA_WORDS = 192;
+static_assert(4 * SL_MAX_SUMS <= SL_FIN_SLOT, "the counters lie before the last entries");
 constexpr int SL_MAX_TRIPS = 32;
 constexpr int SL_MAX_TABS = 7;    // tables of a sum of several terms (a product has at most 3)
 constexpr int SL_MAX_TERMS = 24;
@@ -995,6 +1004,10 @@ struct SliceArgs {
     u32 n_vars, j0;    // the sum's variables; first round evaluated here (1-based)
     u32 n_trips;
     u32 dbl_mask;      // bit k: trip k covers two rounds
+    // several workgroups: after their n_trips trips the tables (an entry or a few per workgroup) go to h0 / h1, the first
+    // workgroup waits for all of them at the gate, takes them up with the pending folds and goes on alone for n_trips2 trips
+    u32 n_trips2;
+    u32 dbl_mask2;
     const u64 *eq0;    // eq storage, level 0 at entry 0 (eq factor only)
     const u64 *eq1;
     const u64 *mail;   // host mailbox
@@ -1004,36 +1017,44 @@ struct SliceArgs {
                        // trip; else they go to h0 / h1
     u64 *out_host;     // result area of SL_AREA_WORDS words
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
-    u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero between trips
-    u32 *ticket;       // ... and their ticket counter
-    u64 *h0[SL_MAX_TABS];  // not finishing: where each workgroup leaves its last state (workgroup-major), to be folded by the next launch
-    u64 *h1[SL_MAX_TABS];
+    u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero when the launch starts
+    u32 *gate;         // ... and the count of workgroups that have left their tables in h0 / h1 (zero when the launch starts)
+    u64 *h0[SL_MAX_TABS];  // where each workgroup leaves its last state (workgroup-major): for the first workgroup to go on with,
+    u64 *h1[SL_MAX_TABS];  // or (a launch that ends before the last round) for the launch queued behind this one
     // a sum of several terms (TERMS): the tables are those of all terms, the polynomial summed is sum_k coeff_k prod table
     u32 n_tabs, n_terms;
     SliceTerm terms[SL_MAX_TERMS];
 };
 
 // dynamic LDS of slice_kernel, in 64-bit words: counters per wavefront, mailbox copy, flags, the terms, then the two table buffers
-constexpr u32 SL_LDS_CTR = 0, SL_LDS_BOX = (BLOCK / WAVE) * 4 * SL_MAX_SUMS, SL_LDS_FLAGS = SL_LDS_BOX + 8, SL_LDS_TERMS = SL_LDS_FLAGS + 2;
-constexpr u32 SL_LDS_TABLES = SL_LDS_TERMS + SL_MAX_TERMS * (sizeof(SliceTerm) / 8);
+// (`blk`: threads of a workgroup)
+constexpr u32 SL_LDS_CTR = 0;
+__host__ __device__ constexpr u32 sl_lds_box(u32 blk) { return (blk / WAVE) * 4 * SL_MAX_SUMS; }
+__host__ __device__ constexpr u32 sl_lds_flags(u32 blk) { return sl_lds_box(blk) + 8; }
+__host__ __device__ constexpr u32 sl_lds_terms(u32 blk) { return sl_lds_flags(blk) + 2; }
+__host__ __device__ constexpr u32 sl_lds_tables(u32 blk) { return sl_lds_terms(blk) + SL_MAX_TERMS * (sizeof(SliceTerm) / 8); }
 static_assert(sizeof(SliceTerm) % 8 == 0, "terms are copied as 64-bit words");
-__host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap) { return SL_LDS_TABLES + n_tabs * 2 * (cap + cap / 2); }
+__host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap, u32 blk) { return sl_lds_tables(blk) + n_tabs * 2 * (cap + cap / 2); }
+// A workgroup of these launches is 1024 threads: what a round costs here is the longest chain of dependent field
+// multiplications in any one lane, and with more lanes each has fewer units of work behind one another.
+constexpr int SL_BLOCK = 1024;
 
 // NF: tables of the product, or with TERMS the largest number of factors of a term (the degree of the polynomial summed)
-template <int NF, bool EQ, bool TERMS>
-__global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
+// BLK: threads of a workgroup (SL_BLOCK in the library; the kernel's CPU test runs smaller ones)
+template <int NF, bool EQ, bool TERMS, int BLK = SL_BLOCK>
+__global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
 {
+    constexpr int BLOCK = BLK;
+    constexpr u32 SL_LDS_BOX = sl_lds_box(BLK), SL_LDS_FLAGS = sl_lds_flags(BLK), SL_LDS_TERMS = sl_lds_terms(BLK), SL_LDS_TABLES = sl_lds_tables(BLK);
     constexpr int NP = NF + 1;          // sums of the trip's first round: q(0..NF), q(1) left zero when it comes from the claim
     constexpr int NPT = NF;             // points of its second round: t = 0, 2, .., NF
     constexpr int NSMP = NF + 1;        // samples of that round's sums as a polynomial in the challenge: 0..NF-1, leading coefficient
     constexpr int NS = NP + NSMP * NPT; // extension sums per trip
-    constexpr int MAXT = TERMS ? SL_MAX_TABS : NF;
-    static_assert(NS <= SL_MAX_SUMS, "sums per trip fit the result area");
+    static_assert(NS <= SL_MAX_SUMS && 4 * NS <= BLK, "sums per trip fit the result area, their counters one lane each");
     extern __shared__ u64 dyn[];
     u64 *const ctr = dyn + SL_LDS_CTR;  // [wavefront][4 * SL_MAX_SUMS]
     u64 *const box = dyn + SL_LDS_BOX;
     int *const ok_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS);
-    int *const last_flag = reinterpret_cast<int *>(dyn + SL_LDS_FLAGS + 1);
     const SliceTerm *const lterms = reinterpret_cast<const SliceTerm *>(dyn + SL_LDS_TERMS);
     const u32 tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const u32 W = gridDim.x, wg = blockIdx.x;
@@ -1041,6 +1062,7 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
     const u64 src_wg = a.src_len / W;             // this workgroup's share of the source
     u32 len = (u32)(src_wg >> a.pend0);           // entries per table once the pending folds are done
     const u32 cap = len;
+    u32 len_log = (u32)__builtin_ctz(len);      // a workgroup's share is a power of two
     // two buffers per limb array: `cap` entries and half of that; a fold reads one and writes the other
     u64 *const buf_big = dyn + SL_LDS_TABLES, *const buf_small = buf_big + (size_t)nt * 2 * cap;
     bool in_big = true;  // where the current state is
@@ -1052,62 +1074,100 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
         for (u32 w = tid; w < a.n_terms * (u32)(sizeof(SliceTerm) / 8); w += BLOCK) dst[w] = src[w];
     }
 
+    // lanes that share a pair (a quad) at one evaluation point split the terms among them
+    const u32 p_split = TERMS ? a.n_terms : 1u;
+    const u32 q_split = TERMS ? (a.n_terms * (u32)(NPT * NSMP) <= (u32)BLOCK ? a.n_terms : 1u) : 1u;
     u32 j = a.j0, pend = a.pend0;
     u64 trip_seq = a.seq0;
-    for (u32 k = 0; k < a.n_trips; k++) {
-        const bool dbl = (a.dbl_mask >> k) & 1;
+    u32 Wc = W;  // workgroups still at work
+    for (u32 k = 0; k < a.n_trips + a.n_trips2; k++) {
+        const bool regroup = k > 0 && k == a.n_trips;
+        const bool dbl = ((k < a.n_trips ? a.dbl_mask >> k : a.dbl_mask2 >> (k - a.n_trips)) & 1) != 0;
+        u64 src_each = src_wg;  // entries of the source a workgroup takes up (k == 0, or the first workgroup when regrouping)
+        if (regroup) {
+            // every workgroup leaves its entries in device memory: stores that go through to where every compute unit
+            // reads (a release fence at device scope would write back the whole L2, from every wavefront of the launch:
+            // 30 us at 256 workgroups), acknowledged to each lane before the workgroup is counted at the gate
+            for (u32 u = tid; u < (nt << len_log); u += BLOCK) {
+                const u32 f = u >> len_log, i = u & (len - 1);
+                st_agent(a.h0[f] + (u64)wg * len + i, tab(in_big, f, 0)[i]);
+                st_agent(a.h1[f] + (u64)wg * len + i, tab(in_big, f, 1)[i]);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            if (tid == 0) __hip_atomic_fetch_add(a.gate, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (wg != 0) return;
+            if (tid == 0) {
+                int ok = 0;
+                for (u32 spins = 0; spins < a.spin_limit; spins++) {
+                    if (__hip_atomic_load(a.gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Wc) {
+                        ok = 1;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                *ok_flag = ok;
+            }
+            __syncthreads();
+            if (*ok_flag == 0) return;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            // every workgroup has made its last add: counters and gate go back to zero for the launch after this one
+            for (u32 c = tid; c < 4 * (u32)SL_MAX_SUMS; c += BLOCK) st_agent(a.ctr + c, 0);
+            if (tid == 0) __hip_atomic_store(a.gate, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            src_each = (u64)Wc * len;
+            len = (u32)(src_each >> pend);
+            len_log = (u32)__builtin_ctz(len);
+            Wc = 1;
+            in_big = true;
+        }
         trip_seq = a.seq0 + (j - a.j0);
-        if (!wait_first_mail(a.mail, W > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
+        if (!wait_first_mail(a.mail, Wc > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
         if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
         const bool skip1 = box[MAIL_SKIP1] != 0;
         const E2 rb_ = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
         const gl::E2P rb = gl::prep(rb_), ra = gl::prep(gl::e2(box[MAIL_RA], box[MAIL_RA + 1]));
         // ---- the pending folds ----
-        if (k == 0) {
+        if (k == 0 || regroup) {
             // from device memory: entry i of the state is the source's entry i (nothing pending), or is made of its entries
             // 2i, 2i+1 (one fold) or 4i..4i+3 (two)
-            const u64 base = (u64)wg * src_wg;
-            for (u32 i = tid; i < len; i += BLOCK) {
-#pragma unroll
-                for (u32 f = 0; f < (u32)MAXT; f++) {
-                    if (f >= nt) break;
-                    const u64 *p0 = a.s0[f], *p1 = a.s1[f];
-                    E2 v;
-                    if (pend == 0) {
-                        v = gl::e2(p0[base + i], p1 ? p1[base + i] : 0);
-                    } else if (pend == 1) {
-                        const U64x2 x0 = ld2(p0 + base + 2 * (u64)i);
-                        if (p1) {
-                            const U64x2 x1 = ld2(p1 + base + 2 * (u64)i);
-                            v = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb);
-                        } else {
-                            v = fold1_base(x0.x, x0.y, rb_);
-                        }
+            const u64 base = (u64)wg * src_each;
+            for (u32 u = tid; u < (nt << len_log); u += BLOCK) {
+                const u32 f = u >> len_log, i = u & (len - 1);
+                const u64 *p0 = regroup ? a.h0[f] : a.s0[f], *p1 = regroup ? a.h1[f] : a.s1[f];
+                E2 v;
+                if (pend == 0) {
+                    v = gl::e2(p0[base + i], p1 ? p1[base + i] : 0);
+                } else if (pend == 1) {
+                    const U64x2 x0 = ld2(p0 + base + 2 * (u64)i);
+                    if (p1) {
+                        const U64x2 x1 = ld2(p1 + base + 2 * (u64)i);
+                        v = fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb);
                     } else {
-                        const U64x2 x0 = ld2(p0 + base + 4 * (u64)i), y0 = ld2(p0 + base + 4 * (u64)i + 2);
-                        const U64x2 x1 = ld2(p1 + base + 4 * (u64)i), y1 = ld2(p1 + base + 4 * (u64)i + 2);
-                        v = fold1p(fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), ra), fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), ra), rb);
+                        v = fold1_base(x0.x, x0.y, rb_);
                     }
-                    tab(true, f, 0)[i] = v.c0;
-                    tab(true, f, 1)[i] = v.c1;
+                } else {
+                    const U64x2 x0 = ld2(p0 + base + 4 * (u64)i), y0 = ld2(p0 + base + 4 * (u64)i + 2);
+                    const U64x2 x1 = ld2(p1 + base + 4 * (u64)i), y1 = ld2(p1 + base + 4 * (u64)i + 2);
+                    v = fold1p(fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), ra), fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), ra), rb);
                 }
+                tab(true, f, 0)[i] = v.c0;
+                tab(true, f, 1)[i] = v.c1;
             }
         } else {
             len >>= pend;
-            for (u32 i = tid; i < len; i += BLOCK) {
-#pragma unroll
-                for (u32 f = 0; f < (u32)MAXT; f++) {
-                    if (f >= nt) break;
-                    const u64 *c0 = tab(in_big, f, 0), *c1 = tab(in_big, f, 1);
-                    E2 v;
-                    if (pend == 1)
-                        v = fold1p(gl::e2(c0[2 * i], c1[2 * i]), gl::e2(c0[2 * i + 1], c1[2 * i + 1]), rb);
-                    else
-                        v = fold1p(fold1p(gl::e2(c0[4 * i], c1[4 * i]), gl::e2(c0[4 * i + 1], c1[4 * i + 1]), ra),
-                                   fold1p(gl::e2(c0[4 * i + 2], c1[4 * i + 2]), gl::e2(c0[4 * i + 3], c1[4 * i + 3]), ra), rb);
-                    tab(!in_big, f, 0)[i] = v.c0;
-                    tab(!in_big, f, 1)[i] = v.c1;
-                }
+            len_log -= pend;
+            for (u32 u = tid; u < (nt << len_log); u += BLOCK) {
+                const u32 f = u >> len_log, i = u & (len - 1);
+                const u64 *c0 = tab(in_big, f, 0), *c1 = tab(in_big, f, 1);
+                E2 v;
+                if (pend == 1)
+                    v = fold1p(gl::e2(c0[2 * i], c1[2 * i]), gl::e2(c0[2 * i + 1], c1[2 * i + 1]), rb);
+                else
+                    v = fold1p(fold1p(gl::e2(c0[4 * i], c1[4 * i]), gl::e2(c0[4 * i + 1], c1[4 * i + 1]), ra),
+                               fold1p(gl::e2(c0[4 * i + 2], c1[4 * i + 2]), gl::e2(c0[4 * i + 3], c1[4 * i + 3]), ra), rb);
+                tab(!in_big, f, 0)[i] = v.c0;
+                tab(!in_big, f, 1)[i] = v.c1;
             }
             in_big = !in_big;
         }
@@ -1129,7 +1189,8 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
         // value is asked for by `val(f)`, each time a term names it: the values live in LDS, not in registers a term
         // could not index)
         // `top_only`: only the terms of NF factors (the leading coefficient in the challenge belongs to them alone)
-        auto poly_of = [&](auto &&val, bool top_only = false) -> E2 {
+        // `m0`, `step`: the terms m0, m0 + step, ... only (lanes that share a pair split its terms; their sums add up)
+        auto poly_of = [&](auto &&val, bool top_only, u32 m0, u32 step) -> E2 {
             if (!TERMS) {
                 E2 prod = val(0);
 #pragma unroll
@@ -1137,7 +1198,7 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
                 return prod;
             }
             gl::E2Acc G = gl::e2acc_zero();
-            for (u32 m = 0; m < a.n_terms; m++) {
+            for (u32 m = m0; m < a.n_terms; m += step) {
                 const SliceTerm &tm = lterms[m];
                 if (top_only && tm.n_factors < (u32)NF) continue;
                 gl::E2P cp;
@@ -1161,118 +1222,66 @@ __global__ void __launch_bounds__(BLOCK) slice_kernel(SliceArgs a)
             for (u32 m = 1; m < t; m++) v = gl::add(v, d);
             return v;
         };
-        // ---- round j: pairs of the state; taken from the last thread down, so that with few pairs and quads they meet different lanes ----
+        // Late rounds have a pair or two per table and hundreds of lanes: a field multiplication is a chain of a hundred
+        // dependent instructions, so the work of a pair is cut into units of one evaluation point (and one term) each
+        // and spread over the lanes; every unit's value goes into the point's counters, where the pieces add up.
+        // ---- round j: pairs of the state; units taken from the last thread down, those of the quads from the first up ----
         {
             const u32 n_pairs = len >> 1;
             const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) + (u64)wg * n_pairs : 0;
-            E2 acc[NP];
-#pragma unroll
-            for (int t = 0; t < NP; t++) acc[t] = gl::e2_zero();
+            const u32 rt = BLOCK - 1 - tid;
+            const u32 m0 = rt % p_split, t = (rt / p_split) % (u32)NP, slot = rt / (p_split * (u32)NP), n_slots = BLOCK / (p_split * (u32)NP);
+            E2 acc = gl::e2_zero();
             bool any = false;
-            for (u32 p = BLOCK - 1 - tid; p < n_pairs; p += BLOCK) {
-                any = true;
-                gl::E2P wp = gl::prep(gl::e2_one());
-                if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + p], a.eq1[eq_off + p]));
-#pragma unroll
-                for (int t = 0; t < NP; t++) {
-                    if (t == 1 && skip1) continue;
-                    const E2 g = poly_of([&](u32 f) { return line_at(ent(f, 2 * p), ent(f, 2 * p + 1), (u32)t); });
-                    acc[t] = EQ ? gl::fma(g, wp, acc[t]) : gl::add(acc[t], g);
+            if (slot < n_slots && !(t == 1 && skip1)) {
+                for (u32 p = slot; p < n_pairs; p += n_slots) {
+                    any = true;
+                    const E2 g = poly_of([&](u32 f) { return line_at(ent(f, 2 * p), ent(f, 2 * p + 1), t); }, false, m0, p_split);
+                    acc = EQ ? gl::fma(g, gl::prep(gl::e2(a.eq0[eq_off + p], a.eq1[eq_off + p])), acc) : gl::add(acc, g);
                 }
             }
-            if (any) {
-#pragma unroll
-                for (int t = 0; t < NP; t++)
-                    if (!(t == 1 && skip1)) flush(t, acc[t]);
-            }
+            if (any) flush(t, acc);
         }
         // ---- round j + 1 as a polynomial in the challenge of round j: quads of the state ----
         if (dbl) {
             const u32 n_quads = len >> 2;
             const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - (j + 1)))) + (u64)wg * n_quads : 0;
-            // a lane keeps one sample: NSMP adjacent lanes share a quad
-            const u32 smp = tid % NSMP, slot = tid / NSMP, n_slots = BLOCK / NSMP;
-            E2 acc[NPT];
-#pragma unroll
-            for (int t = 0; t < NPT; t++) acc[t] = gl::e2_zero();
+            // a lane keeps one sample at one point (of some of the terms)
+            const u32 m0 = tid % q_split, ti = (tid / q_split) % (u32)NPT, smp = (tid / (q_split * (u32)NPT)) % (u32)NSMP;
+            const u32 slot = tid / (q_split * (u32)(NPT * NSMP)), n_slots = BLOCK / (q_split * (u32)(NPT * NSMP));
+            const u32 t = ti == 0 ? 0 : ti + 1;  // points t = 0, 2, .., NF
+            E2 acc = gl::e2_zero();
             bool any = false;
             if (slot < n_slots) {
                 for (u32 u = slot; u < n_quads; u += n_slots) {
                     any = true;
-                    gl::E2P wp = gl::prep(gl::e2_one());
-                    if (EQ) wp = gl::prep(gl::e2(a.eq0[eq_off + u], a.eq1[eq_off + u]));
                     // a table's pair of round j + 1 with the challenge of round j at this lane's sample: e0 + smp (e1 - e0) and
                     // e2 + smp (e3 - e2); for the leading coefficient the slopes e1 - e0, e3 - e2 in their place
-                    auto sampled = [&](u32 f, u32 t) {
+                    auto sampled = [&](u32 f) {
                         const E2 e0 = ent(f, 4 * u), e1 = ent(f, 4 * u + 1), e2_ = ent(f, 4 * u + 2), e3 = ent(f, 4 * u + 3);
                         if (smp == (u32)NF) return line_at(gl::sub(e1, e0), gl::sub(e3, e2_), t);
                         return line_at(line_at(e0, e1, smp), line_at(e2_, e3, smp), t);
                     };
-                    // points t = 0, 2, .., NF
-#pragma unroll
-                    for (int ti = 0; ti < NPT; ti++) {
-                        const u32 t = ti == 0 ? 0 : (u32)ti + 1;
-                        const E2 g = poly_of([&](u32 f) { return sampled(f, t); }, smp == (u32)NF);
-                        acc[ti] = EQ ? gl::fma(g, wp, acc[ti]) : gl::add(acc[ti], g);
-                    }
+                    const E2 g = poly_of(sampled, smp == (u32)NF, m0, q_split);
+                    acc = EQ ? gl::fma(g, gl::prep(gl::e2(a.eq0[eq_off + u], a.eq1[eq_off + u])), acc) : gl::add(acc, g);
                 }
             }
-            if (any) {
-#pragma unroll
-                for (int ti = 0; ti < NPT; ti++) flush(NP + smp * NPT + ti, acc[ti]);
-            }
+            if (any) flush(NP + smp * NPT + ti, acc);
         }
         __syncthreads();
-        // ---- hand the sums over ----
-        bool publish = W == 1;
-        if (W > 1) {
-            // the counters of the four wavefronts, added into the launch's counters in device memory
-            if (wave == 0) {
-                for (u32 c = lane; c < 4 * (u32)NS; c += WAVE) {
-                    u64 v = 0;
+        // ---- hand the sums over: one counter per lane ----
+        if (tid < 4 * (u32)NS && !(skip1 && tid >= 4 && tid < 8)) {
+            const u32 c = tid;
+            u64 v = 0;
 #pragma unroll
-                    for (int w = 0; w < BLOCK / WAVE; w++) v += ctr[w * 4 * SL_MAX_SUMS + c];
-                    if (v) __hip_atomic_fetch_add(a.ctr + c, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+            for (int w = 0; w < BLOCK / WAVE; w++) v += ctr[w * 4 * SL_MAX_SUMS + c];
+            bool mine = true;
+            if (Wc > 1) {
+                const u64 before = __hip_atomic_fetch_add(a.ctr + c, v + SL_CTR_ONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                mine = ((((before >> 56) + 1) & (u64)(Wc - 1)) == 0);
+                v = (before + v) & SL_CTR_MASK;
             }
-            publish = take_ticket(a.ticket, W, last_flag);
-        }
-        if (publish && wave == 0) {
-            // word w of the result (limb w & 1 of sum w >> 1) is counters 2w (low halves) and 2w + 1 (high halves)
-            u64 word = 0;
-            const bool mine = lane < 2 * (u32)NS;
-            if (mine) {
-                u64 lo_h = 0, hi_h = 0;
-                if (W > 1) {
-                    lo_h = ld_agent(a.ctr + 2 * lane);
-                    hi_h = ld_agent(a.ctr + 2 * lane + 1);
-                    st_agent(a.ctr + 2 * lane, 0);
-                    st_agent(a.ctr + 2 * lane + 1, 0);
-                } else {
-#pragma unroll
-                    for (int w = 0; w < BLOCK / WAVE; w++) {
-                        lo_h += ctr[w * 4 * SL_MAX_SUMS + 2 * lane];
-                        hi_h += ctr[w * 4 * SL_MAX_SUMS + 2 * lane + 1];
-                    }
-                }
-                const unsigned __int128 t = (unsigned __int128)lo_h + ((unsigned __int128)hi_h << 32);
-                word = gl::reduce128((u64)t, (u64)(t >> 64));
-            }
-            if (W > 1) {
-                // the counters and the ticket are back at zero before the host can answer
-                // (stores that go through to where the other workgroups' atomics operate, like the counters' above)
-                if (lane == 0) __hip_atomic_store(a.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                __builtin_amdgcn_s_waitcnt(0);
-            }
-            u64 x = mine ? rotl64(word, lane + 1) : 0;
-#pragma unroll
-            for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
-            if (mine) st_sys(a.out_host + lane, word);
-            if (lane == 0) {
-                st_sys(a.out_host + SL_CHK_SLOT, x ^ trip_seq);
-                st_sys(a.out_host + SL_SEQ_SLOT, trip_seq);
-            }
+            if (mine) st_sys(a.out_host + c, v | (sl_tag(trip_seq) << 56));
         }
         pend = dbl ? 2 : 1;
         j += pend;

@@ -11,6 +11,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <thread>
 
 #define __host__
 #define __device__
@@ -120,7 +121,8 @@ inline int update_dpp(int old, int src, int ctrl, int row_mask, int /*bank_mask*
 #define __builtin_amdgcn_readfirstlane(x) (x)
 #define __builtin_amdgcn_fence(order, scope) std::atomic_thread_fence(std::memory_order_seq_cst)
 #define __builtin_amdgcn_s_waitcnt(x) ((void)0)
-#define __builtin_amdgcn_s_sleep(x) ((void)0)
+// (a polling lane gives the other host threads a turn: a workgroup here is hundreds of threads on a few cores)
+#define __builtin_amdgcn_s_sleep(x) std::this_thread::yield()
 #define __HIP_MEMORY_SCOPE_AGENT 0
 #define __HIP_MEMORY_SCOPE_SYSTEM 0
 #define __hip_atomic_load(p, order, scope) __atomic_load_n(p, __ATOMIC_SEQ_CST)

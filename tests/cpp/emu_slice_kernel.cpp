@@ -1,5 +1,5 @@
 // slice_kernel (the LDS-resident rounds of a product sumcheck, one or two rounds per trip to the host, one or several
-// workgroups) run on the CPU through tests/cpp/emu/hip/hip_runtime.h: every workgroup of a launch at once, one host
+// workgroups, the first of which takes the others' entries up and goes on alone) run on the CPU through tests/cpp/emu/hip/hip_runtime.h: every workgroup of a launch at once, one host
 // thread per lane, and a thread that plays the host's side of the mailbox.  Every trip's sums are checked against
 // sums worked out from the definitions on a reference copy of the tables: the round's q(t) by plain loops, the next
 // round's sums at the sample challenges by actually folding the reference tables with 0, 1, .. and summing, the
@@ -97,9 +97,11 @@ struct Term {
 // the first stage (1: a single stage); `single_rounds`: rounds that must start a trip of their own with t = 1 evaluated (an
 // eq point with a zero coordinate there).  TERMS = false: the product of NF tables.  TERMS = true: sum_k coeff_k prod tables
 // over `n_tabs` tables, NF the largest number of factors; `base_tabs` of the tables are base-field ones (j0 <= 2 only).
+// `separate`: the stage of several workgroups and the single workgroup after it are two launches (as when the rounds left
+// are more than one launch can run); otherwise they are one.
 template <int NF, bool EQ, bool TERMS = false>
 static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_in, std::vector<u32> single_rounds = {}, std::vector<Term> terms = {},
-                     u32 base_tabs = 0)
+                     u32 base_tabs = 0, bool separate = false)
 {
     constexpr int NP = NF + 1, NPT = NF, NSMP = NF + 1, NS = NP + NSMP * NPT;
     const u32 NT = TERMS ? n_tabs_in : (u32)NF;
@@ -166,7 +168,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
     }
 
     std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
-    u32 ticket = 0;
+    u32 gate = 0;
     const u64 seq_first = 1000;
     bool ok = true;
     // device-side tables of the stage to come
@@ -198,8 +200,10 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
             }
     };
 
-    for (size_t si = 0; si < stages.size() && ok; si++) {
+    for (size_t si = 0; si < stages.size() && ok;) {
         const Stage &st = stages[si];
+        const bool merged = st.W > 1 && !separate;
+        const size_t last_si = merged ? si + 1 : si;
         dpk::SliceArgs a;
         memset(&a, 0, sizeof a);
         std::vector<std::vector<u64>> h0(NT), h1(NT);
@@ -219,15 +223,20 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         a.n_trips = (u32)st.trips.size();
         for (size_t k = 0; k < st.trips.size(); k++)
             if (st.trips[k].second) a.dbl_mask |= 1u << k;
+        if (merged) {
+            a.n_trips2 = (u32)stages[si + 1].trips.size();
+            for (size_t k = 0; k < stages[si + 1].trips.size(); k++)
+                if (stages[si + 1].trips[k].second) a.dbl_mask2 |= 1u << k;
+        }
         a.eq0 = eq0.data(), a.eq1 = eq1.data();
         a.mail = mail.data();
         a.relay = relay.data();
         a.spin_limit = 1u << 24;
-        a.finish = si + 1 == stages.size();
+        a.finish = last_si + 1 == stages.size();
         a.out_host = area.data();
         a.seq0 = seq_first + (st.j0 - j0);
         a.ctr = gctr.data();
-        a.ticket = &ticket;
+        a.gate = &gate;
         a.n_tabs = NT;
         a.n_terms = TERMS ? (u32)terms.size() : 0;
         for (size_t m = 0; TERMS && m < terms.size(); m++) {
@@ -239,109 +248,129 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         const u32 cap = (u32)((st.src_len / st.W) >> st.pend0);
         std::vector<std::unique_ptr<emu::Group>> groups;
         std::vector<std::vector<u64>> lds;
-        auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap), dpk::slice_kernel<NF, EQ, TERMS>, a, groups, lds);
+        auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap, dpk::BLOCK), dpk::slice_kernel<NF, EQ, TERMS, dpk::BLOCK>, a, groups, lds);
         // ---- the host's side ----
         u32 len_after = 0;
-        for (size_t k = 0; k < st.trips.size() && ok; k++) {
-            const u32 j = st.trips[k].first;
-            const bool dbl = st.trips[k].second;
-            const u64 seq = seq_first + (j - j0);
-            const bool skip1 = !is_single(j);
-            mail[dpk::MAIL_R] = j >= 1 ? chal[j - 1].c0 : 0, mail[dpk::MAIL_R + 1] = j >= 1 ? chal[j - 1].c1 : 0;
-            mail[dpk::MAIL_RA] = j >= 2 ? chal[j - 2].c0 : 0, mail[dpk::MAIL_RA + 1] = j >= 2 ? chal[j - 2].c1 : 0;
-            mail[dpk::MAIL_SKIP1] = skip1;
-            u64 chk = seq;
-            for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
-            mail[dpk::MAIL_CHK] = chk;
-            __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
-            // the result
-            u64 w[2 * dpk::SL_MAX_SUMS];
-            const auto t0 = std::chrono::steady_clock::now();
-            for (;;) {
-                if (__atomic_load_n(&area[dpk::SL_SEQ_SLOT], __ATOMIC_SEQ_CST) == seq) {
-                    u64 c = seq;
-                    for (int i = 0; i < 2 * NS; i++) {
-                        w[i] = __atomic_load_n(&area[i], __ATOMIC_SEQ_CST);
-                        c ^= dpk::rotl64(w[i], i + 1);
+        std::vector<u64> seen(4 * dpk::SL_MAX_SUMS, 0);  // the counters of several workgroups run on from trip to trip
+        for (size_t sj = si; sj <= last_si && ok; sj++) {
+            const Stage &sx = stages[sj];
+            for (size_t k = 0; k < sx.trips.size() && ok; k++) {
+                const u32 j = sx.trips[k].first;
+                const bool dbl = sx.trips[k].second;
+                const u64 seq = seq_first + (j - j0);
+                const bool skip1 = !is_single(j);
+                mail[dpk::MAIL_R] = j >= 1 ? chal[j - 1].c0 : 0, mail[dpk::MAIL_R + 1] = j >= 1 ? chal[j - 1].c1 : 0;
+                mail[dpk::MAIL_RA] = j >= 2 ? chal[j - 2].c0 : 0, mail[dpk::MAIL_RA + 1] = j >= 2 ? chal[j - 2].c1 : 0;
+                mail[dpk::MAIL_SKIP1] = skip1;
+                u64 chk = seq;
+                for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
+                mail[dpk::MAIL_CHK] = chk;
+                __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
+                // the result: every counter of the trip's sums, tagged with the trip
+                const int ns = dbl ? NS : NP;
+                u64 cnt[4 * dpk::SL_MAX_SUMS];
+                const auto t0 = std::chrono::steady_clock::now();
+                for (int c = 0; c < 4 * ns && ok;) {
+                    if (skip1 && c >= 4 && c < 8) {
+                        cnt[c++] = 0;
+                        continue;
                     }
-                    if (c == __atomic_load_n(&area[dpk::SL_CHK_SLOT], __ATOMIC_SEQ_CST)) break;
+                    const u64 v = __atomic_load_n(&area[c], __ATOMIC_SEQ_CST);
+                    if ((v >> 56) == dpk::sl_tag(seq)) {
+                        cnt[c] = v & dpk::SL_CTR_MASK;
+                        if (sx.W > 1) {
+                            const u64 now = cnt[c];
+                            cnt[c] = now - seen[c];
+                            seen[c] = now;
+                        }
+                        area[c] = 0;
+                        c++;
+                        continue;
+                    }
+                    if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(60)) {
+                        printf("%s: no result for the trip of round %u (counter %d)\n", name, j, c);
+                        ok = false;
+                        break;
+                    }
+                    std::this_thread::sleep_for(std::chrono::microseconds(200));
                 }
-                if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(60)) {
-                    printf("%s: no result for the trip of round %u\n", name, j);
-                    ok = false;
-                    break;
+                if (!ok) break;
+                auto sum_at = [&](int idx) {
+                    u64 limb[2];
+                    for (int l = 0; l < 2; l++) {
+                        const unsigned __int128 t = (unsigned __int128)cnt[4 * idx + 2 * l] + ((unsigned __int128)cnt[4 * idx + 2 * l + 1] << 32);
+                        limb[l] = gl::reduce128((u64)t, (u64)(t >> 64));
+                    }
+                    return gl::e2(limb[0], limb[1]);
+                };
+                // round j by the definition
+                fold_to(j);
+                E2 q[NF + 1];
+                round_sums(state, j, q);
+                for (int t = 0; t <= NF; t++) {
+                    const E2 want = (t == 1 && skip1) ? gl::e2_zero() : q[t];
+                    if (!gl::eq(sum_at(t), want)) {
+                        printf("%s: round %u q(%d) differs\n", name, j, t);
+                        ok = false;
+                    }
                 }
-                std::this_thread::sleep_for(std::chrono::microseconds(200));
-            }
-            if (!ok) break;
-            auto sum_at = [&](int idx) { return gl::e2(w[2 * idx], w[2 * idx + 1]); };
-            // round j by the definition
-            fold_to(j);
-            E2 q[NF + 1];
-            round_sums(state, j, q);
-            for (int t = 0; t <= NF; t++) {
-                const E2 want = (t == 1 && skip1) ? gl::e2_zero() : q[t];
-                if (!gl::eq(sum_at(t), want)) {
-                    printf("%s: round %u q(%d) differs\n", name, j, t);
-                    ok = false;
-                }
-            }
-            if (dbl) {
-                // round j + 1 with the challenge at 0, 1, .., NF: fold the reference tables with each and sum
-                E2 c[NF + 1][NF + 1];
-                for (int s = 0; s <= NF; s++) {
-                    std::vector<Table> tmp;
-                    for (auto &t : state) tmp.push_back(fold(t, gl::e2((u64)s, 0)));
-                    round_sums(tmp, j + 1, c[s]);
-                }
-                const int pts[4] = {0, 2, 3, 4};
-                for (int ti = 0; ti < NPT && ok; ti++) {
-                    const int t = pts[ti];
-                    for (int s = 0; s < NF; s++)
-                        if (!gl::eq(sum_at(NP + s * NPT + ti), c[s][t])) {
-                            printf("%s: round %u sample %d point %d differs\n", name, j + 1, s, t);
+                if (dbl) {
+                    // round j + 1 with the challenge at 0, 1, .., NF: fold the reference tables with each and sum
+                    E2 c[NF + 1][NF + 1];
+                    for (int s = 0; s <= NF; s++) {
+                        std::vector<Table> tmp;
+                        for (auto &t : state) tmp.push_back(fold(t, gl::e2((u64)s, 0)));
+                        round_sums(tmp, j + 1, c[s]);
+                    }
+                    const int pts[4] = {0, 2, 3, 4};
+                    for (int ti = 0; ti < NPT && ok; ti++) {
+                        const int t = pts[ti];
+                        for (int s = 0; s < NF; s++)
+                            if (!gl::eq(sum_at(NP + s * NPT + ti), c[s][t])) {
+                                printf("%s: round %u sample %d point %d differs\n", name, j + 1, s, t);
+                                ok = false;
+                            }
+                        // leading coefficient = NF-th finite difference / NF!
+                        E2 lead = gl::e2_zero();
+                        u64 binom = 1, fact = 1;
+                        for (int kk = 0; kk <= NF; kk++) {
+                            const E2 term = gl::mul_base(c[kk][t], binom);
+                            lead = ((NF - kk) & 1) ? gl::sub(lead, term) : gl::add(lead, term);
+                            binom = binom * (u64)(NF - kk) / (u64)(kk + 1);
+                        }
+                        for (int kk = 2; kk <= NF; kk++) fact *= (u64)kk;
+                        lead = gl::mul_base(lead, h_inv(fact));
+                        if (!gl::eq(sum_at(NP + NF * NPT + ti), lead)) {
+                            printf("%s: round %u leading coefficient at point %d differs\n", name, j + 1, t);
                             ok = false;
                         }
-                    // leading coefficient = NF-th finite difference / NF!
-                    E2 lead = gl::e2_zero();
-                    u64 binom = 1, fact = 1;
-                    for (int kk = 0; kk <= NF; kk++) {
-                        const E2 term = gl::mul_base(c[kk][t], binom);
-                        lead = ((NF - kk) & 1) ? gl::sub(lead, term) : gl::add(lead, term);
-                        binom = binom * (u64)(NF - kk) / (u64)(kk + 1);
-                    }
-                    for (int kk = 2; kk <= NF; kk++) fact *= (u64)kk;
-                    lead = gl::mul_base(lead, h_inv(fact));
-                    if (!gl::eq(sum_at(NP + NF * NPT + ti), lead)) {
-                        printf("%s: round %u leading coefficient at point %d differs\n", name, j + 1, t);
-                        ok = false;
-                    }
-                    // what the host does with them: the polynomial at the real challenge = the round's sum computed directly
-                    const E2 r = chal[j];
-                    E2 val = gl::e2_zero(), vanish = gl::e2_one();
-                    for (int kk = 0; kk < NF; kk++) {
-                        E2 num = gl::e2_one();
-                        u64 den = 1;
-                        for (int m = 0; m < NF; m++)
-                            if (m != kk) {
-                                num = gl::mul(num, gl::sub(r, gl::e2((u64)m, 0)));
-                                den = gl::mul(den, gl::sub((u64)kk, (u64)m));
-                            }
-                        val = gl::add(val, gl::mul(gl::mul_base(num, h_inv(den)), sum_at(NP + kk * NPT + ti)));
-                        vanish = gl::mul(vanish, gl::sub(r, gl::e2((u64)kk, 0)));
-                    }
-                    val = gl::add(val, gl::mul(vanish, sum_at(NP + NF * NPT + ti)));
-                    std::vector<Table> next;
-                    for (auto &tb : state) next.push_back(fold(tb, r));
-                    E2 q2[NF + 1];
-                    round_sums(next, j + 1, q2);
-                    if (!gl::eq(val, q2[t])) {
-                        printf("%s: round %u point %d: interpolation at the challenge differs from the direct sum\n", name, j + 1, t);
-                        ok = false;
+                        // what the host does with them: the polynomial at the real challenge = the round's sum computed directly
+                        const E2 r = chal[j];
+                        E2 val = gl::e2_zero(), vanish = gl::e2_one();
+                        for (int kk = 0; kk < NF; kk++) {
+                            E2 num = gl::e2_one();
+                            u64 den = 1;
+                            for (int m = 0; m < NF; m++)
+                                if (m != kk) {
+                                    num = gl::mul(num, gl::sub(r, gl::e2((u64)m, 0)));
+                                    den = gl::mul(den, gl::sub((u64)kk, (u64)m));
+                                }
+                            val = gl::add(val, gl::mul(gl::mul_base(num, h_inv(den)), sum_at(NP + kk * NPT + ti)));
+                            vanish = gl::mul(vanish, gl::sub(r, gl::e2((u64)kk, 0)));
+                        }
+                        val = gl::add(val, gl::mul(vanish, sum_at(NP + NF * NPT + ti)));
+                        std::vector<Table> next;
+                        for (auto &tb : state) next.push_back(fold(tb, r));
+                        E2 q2[NF + 1];
+                        round_sums(next, j + 1, q2);
+                        if (!gl::eq(val, q2[t])) {
+                            printf("%s: round %u point %d: interpolation at the challenge differs from the direct sum\n", name, j + 1, t);
+                            ok = false;
+                        }
                     }
                 }
+                len_after = dbl ? 4 : 2;
             }
-            len_after = dbl ? 4 : 2;
         }
         if (!ok) {
             // let the launch leave: the abort sequence number, as the library does
@@ -349,20 +378,31 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         }
         for (auto &t : threads) t.join();
         if (!ok) break;
-        if (ticket != 0) ok = false, printf("%s: ticket counter left at %u\n", name, ticket);
+        if (st.W > 1 && !merged) {
+            // nobody took over inside the launch: its counters stay as they are, the library clears them behind it
+            for (auto &c : gctr) c = 0;
+        }
+        if (gate != 0) ok = false, printf("%s: gate left at %u\n", name, gate);
         for (u64 c : gctr)
-            if (c) ok = false;
-        const auto &last = st.trips.back();
-        const u32 pend = last.second ? 2 : 1;
-        if (si + 1 < stages.size()) {
-            // what the stage left behind is the reference state of its last trip's round
-            fold_to(last.first);
-            const u64 left = state[0].size();
+            if (c) ok = false, printf("%s: a counter was left at %llx\n", name, (unsigned long long)c);
+        if (st.W > 1) {
+            // what the workgroups left behind (for the first of them, or for the next launch) is the reference state of
+            // their last trip's round
+            std::vector<Table> at_last = ref;
+            {
+                // fold a copy of the reference from the start (the state itself may be further on already)
+                u32 through = j0 - 1 - first_pend;
+                while (through < st.trips.back().first - 1) {
+                    through++;
+                    for (auto &t : at_last) t = fold(t, chal[through]);
+                }
+            }
+            const u64 left = at_last[0].size();
             if (left != stages[si + 1].src_len) ok = false, printf("%s: stage leaves %llu entries, the next expects %llu\n", name, (unsigned long long)left, (unsigned long long)stages[si + 1].src_len);
             for (u32 f = 0; f < NT && ok; f++) {
                 d0[f].assign(left, 0), d1[f].assign(left, 0);
                 for (u64 i = 0; i < left; i++) {
-                    if (h0[f][i] != state[f][i].c0 || h1[f][i] != state[f][i].c1) {
+                    if (h0[f][i] != at_last[f][i].c0 || h1[f][i] != at_last[f][i].c1) {
                         printf("%s: handed-over entry %llu of table %u differs\n", name, (unsigned long long)i, f);
                         ok = false;
                         break;
@@ -370,9 +410,11 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
                     d0[f][i] = h0[f][i], d1[f][i] = h1[f][i];
                 }
             }
-            if (stages[si + 1].pend0 != pend) ok = false, printf("%s: pending folds disagree\n", name);
-        } else {
+            if (stages[si + 1].pend0 != (st.trips.back().second ? 2u : 1u)) ok = false, printf("%s: pending folds disagree\n", name);
+        }
+        if (last_si + 1 == stages.size()) {
             // the last entries of every table, published with the last trip
+            const auto &last = stages[last_si].trips.back();
             fold_to(last.first);
             const u64 seq = seq_first + (last.first - j0);
             u64 c = seq;
@@ -385,6 +427,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
                     if (area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e)] != state[f][e].c0 || area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e) + 1] != state[f][e].c1)
                         ok = false, printf("%s: last entry %u of table %u differs\n", name, e, f);
         }
+        si = last_si + 1;
     }
     size_t n_trips = 0;
     for (auto &s : stages) n_trips += s.trips.size();
@@ -402,6 +445,7 @@ int main()
     run_case<2, false>("two tables, rounds that must go alone (t = 1 evaluated)", 9, 2, 1, 0, {4, 7});
     run_case<2, true>("four workgroups, then one", 12, 3, 4, 0);
     run_case<2, true>("two workgroups down to one entry each, rounds that must go alone", 11, 3, 2, 0, {6});
+    run_case<2, true>("four workgroups and the single one as two launches", 12, 3, 4, 0, {}, {}, 0, true);
     run_case<2, true>("from round 1 (nothing folded yet)", 8, 1, 1, 0);
     // sums of several terms: a LogUp layer eq (a d + b c + lambda c d), then higher degrees, base-field tables, constants
     const Term la{felt2(), {0, 3}}, lb{felt2(), {1, 2}}, lc{felt2(), {2, 3}};

@@ -163,9 +163,9 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     carries on with ordinary launches and the same messages."""
     import time
     # 11 tables are several groups: launches of their own up to round 5 (a launch stays for the later rounds from
-    # n - j + 1 <= 9 on).  4 tables are one group, whose rounds are resident from the first that fits 256 workgroups of 128
-    # pairs (round 3 of 18): rounds 1 and 2 are launches, and the resident launches are queued during round 2.
-    n, afters = (14, (1, 3, 4, 5)) if n_tabs > 7 else (18, (1, 2))
+    # n - j + 1 <= 9 on).  4 tables are one group, whose rounds are resident from the first that fits 256 workgroups of 512
+    # pairs (round 3 of 20): rounds 1 and 2 are launches, and the resident launches are queued during round 2.
+    n, afters = (14, (1, 3, 4, 5)) if n_tabs > 7 else (20, (1, 2))
     gpu, host, terms = _instance(ctx, orc, 900 + n_tabs, n, [n] * n_tabs, [], 2 * n_tabs, 2, True)
     ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
     for after in afters:
@@ -186,10 +186,10 @@ def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     _check(dp, ctx, orc, n, gpu, host, terms)
 
 
-@pytest.mark.parametrize("with_eq,n", [(True, 20), (False, 20), (True, 21)])
+@pytest.mark.parametrize("with_eq,n", [(True, 21), (False, 21), (True, 22)])
 def test_product_launch_made_ahead_steps_aside(dp, ctx, orc, with_eq, n):
     """The same for a single product of full-size tables.  Its rounds are resident from the first that fits 256
-    workgroups of 512 pairs (round 3 of 20, round 4 of 21); the rounds before are launches, each made during the round
+    workgroups of 1024 pairs (round 3 of 21, round 4 of 22); the rounds before are launches, each made during the round
     before it, and so are the resident launches (several workgroups, then one).  In a launch of more than 64
     workgroups only the first workgroup looks for the mail and passes it on to the others; the resident launch of
     several workgroups always does so.  Once a resident launch has had its first mail another call on the context ends
