@@ -848,9 +848,9 @@ int32_t eq_ensure(dps_ctx *ctx, EqInfo &info, u64 *o0, u64 *o1, u64 need, bool n
                 entries += (double)(1ull << js.job[k].n_bits);
             }
             ProfScope ps(ctx, DPS_K_EQ, entries * 16.0);
-            // up to 16 workgroups share a job's rows of 256 entries
+            // up to 128 workgroups share a job's rows of 256 entries (4 rows each in the largest job)
             const u32 rows = max_bits > 8 ? 1u << (max_bits - 8) : 1;
-            dpk::eq_define_kernel<<<dim3(std::min<u32>(rows, 16), n), dpk::BLOCK, 0, ctx->stream>>>(js);
+            dpk::eq_define_kernel<<<dim3(std::min<u32>(rows, 128), n), dpk::BLOCK, 0, ctx->stream>>>(js);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "eq_define launch: %s", hipGetErrorString(e));
         }

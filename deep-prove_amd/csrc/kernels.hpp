@@ -156,37 +156,58 @@ struct EqJobs {
 };
 
 // A table of up to EQ_DIRECT_BITS variables is the outer product of the table of its 8 lowest variables (one entry per
-// thread, in a register) and the table of the others (worked out by the workgroup into LDS): about one product per
-// entry instead of one per entry and variable.  The workgroups of a job (gridDim.x of them) share its rows of 256 entries.
+// thread, in a register) and the table of the others, of which a workgroup works out the rows it writes (the workgroups of
+// a job, gridDim.x of them, share its rows of 256 entries).  Both are outer products themselves, of two tables of at
+// most 5 variables each; the four small tables are made by one wavefront each, at the same time.  What a launch costs
+// is its longest chain of field multiplications (a fifth of a microsecond each, whatever else the lane could do
+// meanwhile): at most 5 for a small table, 1 for the thread's low entry and the workgroup's rows, 1 per row written.
 constexpr u32 EQ_DIRECT_BITS = 17;
 __global__ void __launch_bounds__(BLOCK) eq_define_kernel(EqJobs js)
 {
-    static_assert(BLOCK == 256, "a row is the 8 lowest variables");
+    static_assert(BLOCK == 256 && WAVE == 64, "a row is the 8 lowest variables; four wavefronts make the four small tables");
     constexpr u32 HI_MAX = 1u << (EQ_DIRECT_BITS - 8);
+    __shared__ u64 part0[4][32], part1[4][32];
     __shared__ u64 hi0[HI_MAX], hi1[HI_MAX];
     const EqJob j = js.job[blockIdx.y];
     const u32 lo_bits = j.n_bits < 8 ? j.n_bits : 8, hi_bits = j.n_bits - lo_bits, n_hi = 1u << hi_bits;
     if (blockIdx.x >= n_hi) return;  // (the whole workgroup)
-    auto factor = [&](u32 var, u32 bit) {
-        const E2 r = gl::e2(js.point[2 * var], js.point[2 * var + 1]);
-        return bit ? r : gl::sub(gl::e2_one(), r);
-    };
-    const u32 t = threadIdx.x;
-    E2 lo = gl::e2_one();
-    for (u32 b = 0; b < lo_bits; b++) lo = gl::mul(lo, factor(j.first + b, (t >> b) & 1));
-    for (u32 h = t; h < n_hi; h += BLOCK) {
+    const u32 t = threadIdx.x, w = t / WAVE, lane = t % WAVE;
+    // variables of the four small tables: the low 8 as la + lb, the others as ha + hb
+    const u32 la = lo_bits / 2, lb = lo_bits - la, ha = hi_bits / 2, hb = hi_bits - ha;
+    const u32 bits_w = w == 0 ? la : w == 1 ? lb : w == 2 ? ha : hb;
+    const u32 first_w = j.first + (w == 0 ? 0 : w == 1 ? la : w == 2 ? lo_bits : lo_bits + ha);
+    if (lane < (1u << bits_w)) {
         E2 v = gl::e2_one();
-        for (u32 b = 0; b < hi_bits; b++) v = gl::mul(v, factor(j.first + lo_bits + b, (h >> b) & 1));
-        hi0[h] = v.c0;
-        hi1[h] = v.c1;
+        for (u32 b = 0; b < bits_w; b++) {
+            const E2 r = gl::e2(js.point[2 * (first_w + b)], js.point[2 * (first_w + b) + 1]);
+            v = gl::mul(v, ((lane >> b) & 1) ? r : gl::sub(gl::e2_one(), r));
+        }
+        part0[w][lane] = v.c0;
+        part1[w][lane] = v.c1;
+    }
+    __syncthreads();
+    // the rows of this workgroup: blockIdx.x, + gridDim.x, ...
+    const u32 n_rows = (n_hi - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    for (u32 k = t; k < n_rows; k += BLOCK) {
+        const u32 h = blockIdx.x + k * gridDim.x;
+        const u32 a = h & ((1u << ha) - 1), b = h >> ha;
+        const E2 v = gl::mul(gl::e2(part0[2][a], part1[2][a]), gl::e2(part0[3][b], part1[3][b]));
+        hi0[k] = v.c0;
+        hi1[k] = v.c1;
+    }
+    E2 lo = gl::e2_one();
+    if (t < (1u << lo_bits)) {
+        const u32 a = t & ((1u << la) - 1), b = t >> la;
+        lo = gl::mul(gl::e2(part0[0][a], part1[0][a]), gl::e2(part0[1][b], part1[1][b]));
     }
     __syncthreads();
     if (t >= (1u << lo_bits)) return;
     const bool second = (j.out_off & EQ_JOB_SECOND) != 0;
     u64 *o0 = (second ? js.s0 : js.o0) + (j.out_off & ~EQ_JOB_SECOND), *o1 = (second ? js.s1 : js.o1) + (j.out_off & ~EQ_JOB_SECOND);
     const gl::E2P lp = gl::prep(lo);
-    for (u32 h = blockIdx.x; h < n_hi; h += gridDim.x) {
-        const E2 v = gl::mulp(gl::e2(hi0[h], hi1[h]), lp);
+    for (u32 k = 0; k < n_rows; k++) {
+        const u32 h = blockIdx.x + k * gridDim.x;
+        const E2 v = gl::mulp(gl::e2(hi0[k], hi1[k]), lp);
         o0[((u64)h << lo_bits) | t] = v.c0;
         o1[((u64)h << lo_bits) | t] = v.c1;
     }
