@@ -570,7 +570,7 @@ Context.read_ms = _read_ms
 
 # ---- einsum and LogUp drivers of the host mirror ----
 host.dph_einsum_prove.restype = _i32
-host.dph_einsum_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
+host.dph_einsum_prove.argtypes = [_vp, _u32, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp]
 host.dph_einsum_prove_resident.restype = _i32
 host.dph_einsum_prove_resident.argtypes = host.dph_einsum_prove.argtypes
 host.dph_logup_batch_prove.restype = _i32
@@ -605,19 +605,27 @@ class Tensor:
         return len(self.shape)
 
 
-def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
-    """EinSum::prove_internal.  ops: list of (lhs_labels, rhs_labels, out_labels);
+def einsum_prove(ctx, ops, lhs, rhs, claims, transcript, biases=None):
+    """EinSum::prove_internal.  ops: list of (lhs_labels, rhs_labels, out_labels) or, for an
+    output with a bias, (lhs_labels, rhs_labels, out_labels, bias_labels);
     lhs: int64 ndarray (unpadded); rhs: list of int64 ndarrays; claims: list of
-    (point[k, 2], eval[2]) on the outputs.  lhs and every rhs may instead be
-    `Tensor`s already on the device (nothing is uploaded then).  Returns a dict with
-    the sumcheck proof, the final evaluations, the optional aggregation proof and
-    the input claims."""
+    (point[k, 2], eval[2]) on the outputs; biases: None, or one entry per op (None where
+    the op has no bias).  lhs, every rhs and every bias may instead be `Tensor`s already on
+    the device (nothing is uploaded then).  Returns a dict with the sumcheck proof, the
+    final evaluations, the optional aggregation proof, the input claims and the bias
+    claims (output index, point, evaluation)."""
     R = len(ops)
     lab = []
     for o in ops:
-        lab += [s.encode() for s in o]
-    labels = (C.c_char_p * (3 * R))(*lab)
+        lab += [s.encode() for s in o] + ([b""] if len(o) == 3 else [])
+    labels = (C.c_char_p * (4 * R))(*lab)
     resident = isinstance(lhs, Tensor)
+    bk = list(biases) if biases is not None else None
+    if bk is not None:
+        if len(bk) != R or any((b is None) != (len(o) == 3 or not o[3]) for b, o in zip(bk, ops)):
+            raise ValueError("einsum_prove: one bias per op that names bias labels")
+        if any(b is not None and isinstance(b, Tensor) != resident for b in bk):
+            raise ValueError("einsum_prove: either every tensor is on the device or none is")
     if resident != all(isinstance(x, Tensor) for x in rhs) or (not resident and any(isinstance(x, Tensor) for x in rhs)):
         raise ValueError("einsum_prove: either every tensor is on the device or none is")
     if resident:
@@ -635,6 +643,16 @@ def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
     rshapes_keep = [(_u64 * x.ndim)(*x.shape) for x in rk]
     rshapes = (_vp * R)(*[C.cast(s, _vp).value for s in rshapes_keep])
     rranks = (_u32 * R)(*[x.ndim for x in rk])
+    bptr = bshapes = branks = None
+    if bk is not None:
+        if not resident:
+            bk = [None if b is None else np.ascontiguousarray(b, dtype=np.int64) for b in bk]
+            bptr = (_vp * R)(*[None if b is None else b.ctypes.data for b in bk])
+        else:
+            bptr = (_vp * R)(*[None if b is None else b.mle.handle for b in bk])
+        bshapes_keep = [None if b is None else (_u64 * b.ndim)(*b.shape) for b in bk]
+        bshapes = (_vp * R)(*[None if s_ is None else C.cast(s_, _vp).value for s_ in bshapes_keep])
+        branks = (_u32 * R)(*[0 if b is None else b.ndim for b in bk])
     pts_keep = [_e2(p).reshape(-1, 2) for p, _ in claims]
     pts = (_vp * R)(*[p.ctypes.data for p in pts_keep])
     plens = (_u32 * R)(*[p.shape[0] for p in pts_keep])
@@ -642,7 +660,7 @@ def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
     cap = 1 << 16
     out = np.zeros(cap, dtype=np.uint64)
     n = _u64(0)
-    ctx._chk_host(fn(ctx._c, R, labels, lhs_arg, lshape, lhs.ndim, rptr, rshapes, rranks, pts, plens, _ptr(evals),
+    ctx._chk_host(fn(ctx._c, R, labels, lhs_arg, lshape, lhs.ndim, rptr, rshapes, rranks, bptr, bshapes, branks, pts, plens, _ptr(evals),
                      transcript._t, _ptr(out), cap, C.byref(n)), fn_name)
     w = out[: n.value]
     res = {}
@@ -665,6 +683,16 @@ def einsum_prove(ctx, ops, lhs, rhs, claims, transcript):
         point = w[pos:pos + 2 * pl].reshape(pl, 2).copy()
         pos += 2 * pl
         res["claims"].append((point, w[pos:pos + 2].copy()))
+        pos += 2
+    nb = int(w[pos])
+    pos += 1
+    res["bias_claims"] = []
+    for _ in range(nb):
+        output, pl = int(w[pos]), int(w[pos + 1])
+        pos += 2
+        point = w[pos:pos + 2 * pl].reshape(pl, 2).copy()
+        pos += 2 * pl
+        res["bias_claims"].append((output, point, w[pos:pos + 2].copy()))
         pos += 2
     return res
 

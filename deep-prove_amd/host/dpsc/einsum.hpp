@@ -1,8 +1,11 @@
 // Einsum / matmul proof, host side: axis classification, partial evaluation of
 // the quantised inputs on the GPU, the batched degree-2 sumcheck and the input
 // claims.  Follows zkml/src/layers/einsum/{axis.rs:478-580,1016-1259, prove.rs:46-361,
-// op_info.rs:137-199}.  Biases are not handled here (the reference evaluates
-// them with DensePolynomial::evaluate, which DensePolynomial::evaluate covers).
+// op_info.rs:137-199}.  A bias added to an output gives a claim of its own: the bias tensor's
+// multilinear extension at the part of the output claim's point that its axes name
+// (prove.rs:191-214, axis.rs:582-637), evaluated on the GPU.  Constant tensors (weights)
+// are ordinary right-hand sides here: they arrive unpadded like every tensor and are padded
+// by the kernels that read them (prove.rs:66-94 pads them on the host).
 #pragma once
 #include <string>
 
@@ -89,9 +92,10 @@ struct FixedAxis {
     std::vector<F> point;  // empty for contracted axes
 };
 
-// One batched operation: lhs labels, rhs labels -> output labels, e.g. "ik","kj","ij"
+// One batched operation: lhs labels, rhs labels -> output labels, e.g. "ik","kj","ij"; `bias`: the labels of the bias
+// tensor added to the output (a subset of the output's, "A(ij)@B(kj)->C(ik)+BIAS(k)" has "k"), empty when there is none
 struct Op {
-    std::string lhs, rhs, out;
+    std::string lhs, rhs, out, bias;
 };
 
 inline AxisType classify(const Op &op, char label)
@@ -101,6 +105,19 @@ inline AxisType classify(const Op &op, char label)
     if (l && r && !o) return AxisType::Contracted;
     if ((l != r) && o) return AxisType::Outer;
     throw Error(DPS_ERR_UNSUPPORTED, std::string("einsum axis '") + label + "' is neither stacked, contracted nor outer");
+}
+
+// bias_evaluation_point (axis.rs:582-637): the slices of the output claim's point that belong to the bias tensor's
+// axes, the last axis first (it takes the lowest variables)
+inline std::vector<F> bias_evaluation_point(const Op &op, const std::vector<std::vector<F>> &out_slices)
+{
+    std::vector<F> point;
+    for (size_t a = op.bias.size(); a-- > 0;) {
+        const size_t pos = op.out.find(op.bias[a]);
+        if (pos == std::string::npos) throw Error(DPS_ERR_INVALID, std::string("Bias tensor has an axis '") + op.bias[a] + "' that is not present in the output tensor");
+        point.insert(point.end(), out_slices[pos].begin(), out_slices[pos].end());
+    }
+    return point;
 }
 
 // reconstruct_full_point (prove.rs:337-361)
@@ -178,6 +195,7 @@ inline Expression build_einsum_expression(const std::vector<std::vector<F>> &coe
 }
 
 struct EinSumProof {
+    std::vector<F> bias_evals;  // one per output that has a bias, in output order
     IOPProof einsum_sumcheck;
     std::vector<F> einsum_evaluations;
     bool has_aggregation = false;
@@ -186,18 +204,22 @@ struct EinSumProof {
 
 struct EinSumProofInfo {
     std::vector<Claim> claims;  // lhs first, then one per rhs
+    std::vector<std::pair<size_t, Claim>> bias_claims;  // (output, claim on its bias tensor): the constant-polynomial claims of prove.rs:254-258
     EinSumProof proof;
     std::vector<F> einsum_sumcheck_point;
     std::vector<std::vector<F>> stacking_coeffs;
 };
 
 // EinSum::prove_internal (prove.rs:46-333).  ops[r] contracts the one LHS with
-// rhs[r] into output r; last_claims[r] is the claim on output r.
+// rhs[r] into output r; last_claims[r] is the claim on output r; biases[r] is the
+// tensor added to output r (nullptr: none; `biases` may be empty when no output has one).
 inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> &ops, const Tensor &lhs, const std::vector<Tensor> &rhs,
-                                      const std::vector<Claim> &last_claims, Transcript &transcript)
+                                      const std::vector<Claim> &last_claims, Transcript &transcript, const std::vector<const Tensor *> &biases = {})
 {
     const size_t R = ops.size();
     if (R == 0 || rhs.size() != R || last_claims.size() != R) throw Error(DPS_ERR_INVALID, "prove_internal: mismatched number of inputs and claims");
+    if (!biases.empty() && biases.size() != R) throw Error(DPS_ERR_INVALID, "prove_internal: one bias slot per output");
+    std::vector<std::vector<F>> bias_points(R);
     std::vector<std::vector<FixedAxis>> lhs_fixes(R), rhs_fixes(R);
     uint64_t contraction_size = 0, stacking_size = 0;
     for (size_t r = 0; r < R; r++) {
@@ -216,6 +238,15 @@ inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> 
                 throw Error(DPS_ERR_INVALID, "prove_internal: output axis not found in any input tensor");
         }
         auto slices = split_point(out_shape, last_claims[r].point);
+        const Tensor *bias = biases.empty() ? nullptr : biases[r];
+        if ((bias != nullptr) != !op.bias.empty()) throw Error(DPS_ERR_INVALID, "prove_internal: bias labels and bias tensor do not go together");
+        if (bias) {
+            if (bias->padded_shape.size() != op.bias.size()) throw Error(DPS_ERR_INVALID, "prove_internal: bias rank does not match its labels");
+            bias_points[r] = bias_evaluation_point(op, slices);
+            size_t nv = 0;
+            for (auto d : bias->padded_shape) nv += ceil_log2(d);
+            if (nv != bias_points[r].size()) throw Error(DPS_ERR_INVALID, "prove_internal: bias shape does not match the output's");
+        }
         auto fix = [&](const std::string &labels) {
             std::vector<FixedAxis> fa(labels.size());
             for (size_t a = 0; a < labels.size(); a++) {
@@ -261,6 +292,15 @@ inline EinSumProofInfo prove_internal(const Context &ctx, const std::vector<Op> 
     info.proof.einsum_sumcheck = std::move(res.first);
     info.proof.einsum_evaluations = res.second.get_mle_flatten_final_evaluations();
     info.einsum_sumcheck_point = res.second.collect_raw_challenges();
+    // prove.rs:191-222: the bias tensors at their points
+    for (size_t r = 0; r < R && !biases.empty(); r++) {
+        if (!biases[r]) continue;
+        Claim c;
+        c.point = bias_points[r];
+        c.eval = biases[r]->padded_mle(ctx).evaluate(c.point);
+        info.proof.bias_evals.push_back(c.eval);
+        info.bias_claims.emplace_back(r, std::move(c));
+    }
     const auto &ev = info.proof.einsum_evaluations;
     const size_t half = ev.size() / 2;
     // prove.rs:224-253: one claim per RHS

@@ -51,17 +51,22 @@ int32_t dph_sumcheck_verify(const uint64_t claimed_sum[2], const uint64_t *proof
                             dph_transcript *t, uint64_t *point_out, uint64_t expected_out[2]);
 
 /* ---- EinSum::prove_internal (zkml/src/layers/einsum/prove.rs:46-333) ----
- * n_ops batched operations share one LHS.  labels: 3*n_ops C strings (lhs, rhs,
- * out per operation, e.g. "ik","kj","ij").  Tensors arrive unpadded, row-major.
+ * n_ops batched operations share one LHS.  labels: 4*n_ops C strings (lhs, rhs,
+ * out, bias per operation, e.g. "ik","kj","ij","j"; bias "" = the output has no
+ * bias).  Tensors arrive unpadded, row-major.  biases: NULL when no output has a
+ * bias, else n_ops entries (NULL where the bias labels are ""), with their shapes
+ * and ranks alongside (prove.rs:191-214: every bias gives a claim of its own).
  * claim_points[r]: 2*len limbs of the claim point on output r, claim_evals 2 per op.
  * The result is written as 64-bit words:
  *   rounds, points_per_round, proof limbs..., n_evals, eval limbs...,
  *   agg_rounds (0 = none), agg proof limbs (3 points per round)...,
- *   n_claims, then per claim: point_len, point limbs..., eval limbs
+ *   n_claims, then per claim: point_len, point limbs..., eval limbs,
+ *   n_bias_claims, then per bias claim: output index, point_len, point limbs..., eval limbs
  * Returns DPS_OK and the word count through *n_words. */
 int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const int64_t *lhs,
                          const uint64_t *lhs_shape, uint32_t lhs_rank, const int64_t *const *rhs,
                          const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                         const int64_t *const *biases, const uint64_t *const *bias_shapes, const uint32_t *bias_ranks,
                          const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
                          const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
                          uint64_t *n_words);
@@ -73,6 +78,7 @@ int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels
 int32_t dph_einsum_prove_resident(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const dps_mle *lhs,
                                   const uint64_t *lhs_shape, uint32_t lhs_rank, const dps_mle *const *rhs,
                                   const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                                  const dps_mle *const *biases, const uint64_t *const *bias_shapes, const uint32_t *bias_ranks,
                                   const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
                                   const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
                                   uint64_t *n_words);

@@ -160,6 +160,13 @@ void write_einsum(const einsum::EinSumProofInfo &info, uint64_t *out, uint64_t o
         for (auto &x : cl.point) put(x);
         put(cl.eval);
     }
+    w.push_back(info.bias_claims.size());
+    for (auto &bc : info.bias_claims) {
+        w.push_back(bc.first);
+        w.push_back(bc.second.point.size());
+        for (auto &x : bc.second.point) put(x);
+        put(bc.second.eval);
+    }
     if (w.size() > out_cap) throw Error(DPS_ERR_INVALID, "dph_einsum_prove: output buffer too small");
     memcpy(out, w.data(), w.size() * 8);
     *n_words = w.size();
@@ -177,6 +184,7 @@ uint64_t shape_count(const uint64_t *shape, uint32_t rank)
 int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const int64_t *lhs,
                          const uint64_t *lhs_shape, uint32_t lhs_rank, const int64_t *const *rhs,
                          const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                         const int64_t *const *biases, const uint64_t *const *bias_shapes, const uint32_t *bias_ranks,
                          const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
                          const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
                          uint64_t *n_words)
@@ -186,20 +194,28 @@ int32_t dph_einsum_prove(dps_ctx *ctx, uint32_t n_ops, const char *const *labels
         std::vector<einsum::Op> ops;
         std::vector<einsum::Tensor> rts;
         std::vector<einsum::Claim> claims;
+        std::vector<std::unique_ptr<einsum::Tensor>> bts(n_ops);
+        std::vector<const einsum::Tensor *> bptr;
         einsum::Tensor lt = einsum::Tensor::from_unpadded(c, lhs, shape_count(lhs_shape, lhs_rank), std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
         for (uint32_t r = 0; r < n_ops; r++) {
-            ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
+            ops.push_back(einsum::Op{labels[4 * r], labels[4 * r + 1], labels[4 * r + 2], labels[4 * r + 3]});
             rts.push_back(einsum::Tensor::from_unpadded(c, rhs[r], shape_count(rhs_shapes[r], rhs_ranks[r]),
                                                         std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
             claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
+            if (biases && biases[r])
+                bts[r].reset(new einsum::Tensor(einsum::Tensor::from_unpadded(c, biases[r], shape_count(bias_shapes[r], bias_ranks[r]),
+                                                                               std::vector<uint64_t>(bias_shapes[r], bias_shapes[r] + bias_ranks[r]))));
         }
-        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t), out, out_cap, n_words);
+        if (biases)
+            for (auto &b : bts) bptr.push_back(b.get());
+        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t, bptr), out, out_cap, n_words);
     });
 }
 
 int32_t dph_einsum_prove_resident(dps_ctx *ctx, uint32_t n_ops, const char *const *labels, const dps_mle *lhs,
                                   const uint64_t *lhs_shape, uint32_t lhs_rank, const dps_mle *const *rhs,
                                   const uint64_t *const *rhs_shapes, const uint32_t *rhs_ranks,
+                                  const dps_mle *const *biases, const uint64_t *const *bias_shapes, const uint32_t *bias_ranks,
                                   const uint64_t *const *claim_points, const uint32_t *claim_point_lens,
                                   const uint64_t *claim_evals, dph_transcript *t, uint64_t *out, uint64_t out_cap,
                                   uint64_t *n_words)
@@ -209,13 +225,19 @@ int32_t dph_einsum_prove_resident(dps_ctx *ctx, uint32_t n_ops, const char *cons
         std::vector<einsum::Op> ops;
         std::vector<einsum::Tensor> rts;
         std::vector<einsum::Claim> claims;
+        std::vector<std::unique_ptr<einsum::Tensor>> bts(n_ops);
+        std::vector<const einsum::Tensor *> bptr;
         einsum::Tensor lt = einsum::Tensor::resident(c, lhs, std::vector<uint64_t>(lhs_shape, lhs_shape + lhs_rank));
         for (uint32_t r = 0; r < n_ops; r++) {
-            ops.push_back(einsum::Op{labels[3 * r], labels[3 * r + 1], labels[3 * r + 2]});
+            ops.push_back(einsum::Op{labels[4 * r], labels[4 * r + 1], labels[4 * r + 2], labels[4 * r + 3]});
             rts.push_back(einsum::Tensor::resident(c, rhs[r], std::vector<uint64_t>(rhs_shapes[r], rhs_shapes[r] + rhs_ranks[r])));
             claims.push_back(einsum::Claim{from_limbs(claim_points[r], claim_point_lens[r]), F(claim_evals[2 * r], claim_evals[2 * r + 1])});
+            if (biases && biases[r])
+                bts[r].reset(new einsum::Tensor(einsum::Tensor::resident(c, biases[r], std::vector<uint64_t>(bias_shapes[r], bias_shapes[r] + bias_ranks[r]))));
         }
-        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t), out, out_cap, n_words);
+        if (biases)
+            for (auto &b : bts) bptr.push_back(b.get());
+        write_einsum(einsum::prove_internal(c, ops, lt, rts, claims, t->t, bptr), out, out_cap, n_words);
     });
 }
 

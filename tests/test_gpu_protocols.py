@@ -125,8 +125,10 @@ def test_partial_eval_matches_checker(ctx, orc, case):
         assert len(got2) == 1 and (got2[0].download()[0] == want).all()
 
 
-def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec"):
-    """prove_internal restated with the checker's pieces (einsum/prove.rs:138-316), one or more RHS."""
+def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec", biases=None):
+    """prove_internal restated with the checker's pieces (einsum/prove.rs:138-316), one or more RHS; a bias gives a
+    claim of its own, its padded tensor's MLE at the slices of the output claim's point that its axes name
+    (prove.rs:191-214, axis.rs:582-637)."""
     R = len(ops)
     tr = orc.OracleTranscript(label)
     lp, lpad = _padded(lhs), _pad(lhs.shape)
@@ -154,11 +156,15 @@ def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec"):
                 out.append(pts[a])
         return np.concatenate(out) if out else np.zeros((0, 2), np.uint64)
 
-    lfix, rfix, lpts, rpts, ltabs, rtabs, coeffs = [], [], [], [], [], [], []
+    lfix, rfix, lpts, rpts, ltabs, rtabs, coeffs, bias_claims = [], [], [], [], [], [], [], []
     for r, op in enumerate(ops):
         rpad = _pad(rhs[r].shape)
         out_shape = [lpad[op[0].index(c)] if c in op[0] else rpad[op[1].index(c)] for c in op[2]]
         sl = split(out_shape, claims[r][0])
+        if biases is not None and biases[r] is not None:
+            bpt = [sl[op[2].index(c)] for c in reversed(op[3])]
+            bpt = np.concatenate(bpt) if bpt else np.zeros((0, 2), np.uint64)
+            bias_claims.append((r, bpt, orc.mle_evaluate(orc.embed_i64(_padded(biases[r]).reshape(-1)), bpt)))
         lk = [classify(op, c) for c in op[0]]
         rk = [classify(op, c) for c in op[1]]
         lpt = [None if k == C_ else sl[op[2].index(c)] for c, k in zip(op[0], lk)]
@@ -200,21 +206,31 @@ def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec"):
         for j in range(S):
             ev = orc.e2_add(ev, orc.e2_mul(coeffs[0][j], finals[j]))
         lhs_claim = (reconstruct(lfix[0], lpts[0], point, lpad), ev)
-    return dict(proof=proof, evaluations=finals, aggregation_proof=agg, claims=[lhs_claim] + out_claims), tr
+    return dict(proof=proof, evaluations=finals, aggregation_proof=agg, claims=[lhs_claim] + out_claims, bias_claims=bias_claims), tr
 
 
-def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed):
-    # output claims: the true MLE evaluations of the integer results
-    claims = []
+def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed, biases=None):
+    # output claims: the true MLE evaluations of the integer results (with the bias added where there is one)
+    claims, bias_parts = [], []
     for r, op in enumerate(ops):
         out = np.einsum(f"{op[0]},{op[1]}->{op[2]}", lhs, rhs[r])
+        added = np.zeros_like(out)
+        if biases is not None and biases[r] is not None:
+            # broadcast over the output axes the bias does not have
+            added = np.broadcast_to(biases[r].reshape([out.shape[op[2].index(c)] if c in op[3] else 1 for c in op[2]]), out.shape).copy()
+            assert [c for c in op[2] if c in op[3]] == list(op[3])  # (the reshape above takes the bias axes in output order)
         nvars = sum(max(0, (d - 1).bit_length()) for d in _pad(out.shape))
         pt = rand_e2(nvars, seed + r)
-        ev = orc.mle_evaluate(orc.embed_i64(_padded(out).reshape(-1)), pt)
+        ev = orc.mle_evaluate(orc.embed_i64(_padded(out + added).reshape(-1)), pt)
         claims.append((pt, ev))
+        # what the verifier takes off the claim: the broadcast bias (zero in the padding) at the claim's point
+        bias_parts.append(orc.mle_evaluate(orc.embed_i64(_padded(added).reshape(-1)), pt))
     tr = dp.Transcript()
-    got = dp.einsum_prove(ctx, ops, lhs, rhs, claims, tr)
-    ref, otr = _oracle_einsum(orc, ops, lhs, rhs, claims)
+    got = dp.einsum_prove(ctx, ops, lhs, rhs, claims, tr, biases)
+    ref, otr = _oracle_einsum(orc, ops, lhs, rhs, claims, biases=biases)
+    assert len(got["bias_claims"]) == len(ref["bias_claims"])
+    for (go, gp, ge), (ro, rp, re) in zip(got["bias_claims"], ref["bias_claims"]):
+        assert go == ro and (gp == rp).all() and (ge == re).all()
     assert (got["proof"] == ref["proof"]).all()
     assert (got["evaluations"] == ref["evaluations"]).all()
     if ref["aggregation_proof"] is None:
@@ -229,9 +245,12 @@ def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed):
     # the same handles (nothing in a proof may change them)
     for bits in (64, 16):
         dl, dr = dp.Tensor(ctx, lhs, bits), [dp.Tensor(ctx, x, bits) for x in rhs]
+        db = None if biases is None else [None if b is None else dp.Tensor(ctx, b, bits) for b in biases]
         for _ in range(2):
             rt = dp.Transcript()
-            again = dp.einsum_prove(ctx, ops, dl, dr, claims, rt)
+            again = dp.einsum_prove(ctx, ops, dl, dr, claims, rt, db)
+            for (go, gp, ge), (ro, rp, re) in zip(again["bias_claims"], got["bias_claims"]):
+                assert go == ro and (gp == rp).all() and (ge == re).all()
             assert (again["proof"] == got["proof"]).all() and (again["evaluations"] == got["evaluations"]).all()
             assert (again["aggregation_proof"] is None) == (got["aggregation_proof"] is None)
             if got["aggregation_proof"] is not None:
@@ -243,8 +262,8 @@ def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed):
     vt = orc.OracleTranscript()
     gamma = vt.append_and_sample(b"batching_challenge")
     acc, gp = E2(0), E2(1)
-    for _, ev in claims:
-        acc = acc + gp * to_E2(ev)[0]
+    for (_, ev), part in zip(claims, bias_parts):
+        acc = acc + gp * (to_E2(ev)[0] - to_E2(part)[0])
         gp = gp * to_E2(gamma)[0]
     p1 = to_E2(got["proof"][0])
     assert p1[0] + p1[1] == acc
@@ -262,6 +281,21 @@ def test_einsum_matmul_small(dp, ctx, orc):
 def test_einsum_matmul_reference_test_sizes(dp, ctx, orc):
     # zkml/src/layers/einsum/mod.rs:700-722: 300 x 350 x 256
     _check_einsum(dp, ctx, orc, [("ik", "kj", "ij")], rand_i64((300, 350), 3), [rand_i64((350, 256), 4)], 310)
+
+
+def test_einsum_transposed_matmul_with_bias(dp, ctx, orc):
+    # zkml/src/layers/einsum/mod.rs:699-722: "A(ij)@B(kj)->C(ik)+BIAS(k)", 300 x 350 times the transpose of 256 x 350
+    _check_einsum(dp, ctx, orc, [("ij", "kj", "ik", "k")], rand_i64((300, 350), 21), [rand_i64((256, 350), 22)], 360,
+                  biases=[rand_i64((256,), 23)])
+
+
+def test_einsum_bias_on_some_outputs(dp, ctx, orc):
+    # three weights against one input, a bias over both output axes on the first, over the rows on the last, none in
+    # between (unpadded sizes: the padding of a broadcast bias is zero, which the statement check below relies on)
+    x = rand_i64((6, 7), 24)
+    ws = [rand_i64((7, 5), 25 + k) for k in range(3)]
+    _check_einsum(dp, ctx, orc, [("ik", "kj", "ij", "ij"), ("ik", "kj", "ij"), ("ik", "kj", "ij", "i")], x, ws, 370,
+                  biases=[rand_i64((6, 5), 28), None, rand_i64((6,), 29)])
 
 
 def test_einsum_stacked(dp, ctx, orc):
