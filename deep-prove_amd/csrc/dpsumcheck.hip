@@ -1042,9 +1042,11 @@ int32_t axis_dot(dps_ctx *ctx, const AxisJob &j)
     const bool col = a.C >= 32;
     // split k over workgroups when there are too few outputs to fill the chip
     const u64 out_blocks = col ? a.P * ((a.C + dpk::WAVE - 1) / dpk::WAVE) : outputs;
-    const u64 k_unit = col ? 64 : 1024;  // k values one workgroup should at least own
+    // k values one workgroup should at least own (two trips of four per wavefront, or one per lane); a few thousand workgroups
+    // keep enough loads in flight to hide the latency of a launch that is a few megabytes in all
+    const u64 k_unit = col ? 32 : 1024;
     u32 n_slices = 1;
-    if (out_blocks < 1024 && a.K > k_unit) n_slices = (u32)std::min<u64>((a.K + k_unit - 1) / k_unit, std::max<u64>(1, 2048 / out_blocks));
+    if (out_blocks < 2048 && a.K > k_unit) n_slices = (u32)std::min<u64>((a.K + k_unit - 1) / k_unit, std::max<u64>(1, 4096 / out_blocks));
     if (n_slices > 65535) n_slices = 65535;
     a.k_per_slice = (a.K + n_slices - 1) / n_slices;
     n_slices = (u32)((a.K + a.k_per_slice - 1) / a.k_per_slice);

@@ -2055,11 +2055,18 @@ __global__ void __launch_bounds__(BLOCK) axis_dot_col_kernel(AxisArgs a)
         const u64 base = ax_offset(pre, a.n_pre, a.pre_dims, a.pre_strides) + ax_offset(i, a.n_post, a.post_dims, a.post_strides);
         u64 k0 = (u64)slice * a.k_per_slice, k1 = k0 + a.k_per_slice;
         if (k1 > a.K) k1 = a.K;
-        for (u64 k = k0 + wave; k < k1; k += BLOCK / WAVE) {
-            E2 v = ax_load(a, base + k * a.stride_k);
-            E2 b = gl::e2(a.b0[k], a.b1[k]);
-            acc = gl::add(acc, (a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0)));
+        // four rows in flight per wavefront: the loop is a chain of loads otherwise (a row is 512 B per wavefront)
+        constexpr u64 STEP = BLOCK / WAVE;
+        auto term = [&](E2 v, E2 b) { return a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0); };
+        u64 k = k0 + wave;
+        for (; k + 3 * STEP < k1; k += 4 * STEP) {
+            const E2 v0 = ax_load(a, base + k * a.stride_k), v1 = ax_load(a, base + (k + STEP) * a.stride_k);
+            const E2 v2 = ax_load(a, base + (k + 2 * STEP) * a.stride_k), v3 = ax_load(a, base + (k + 3 * STEP) * a.stride_k);
+            const E2 b0 = gl::e2(a.b0[k], a.b1[k]), b1 = gl::e2(a.b0[k + STEP], a.b1[k + STEP]);
+            const E2 b2 = gl::e2(a.b0[k + 2 * STEP], a.b1[k + 2 * STEP]), b3 = gl::e2(a.b0[k + 3 * STEP], a.b1[k + 3 * STEP]);
+            acc = gl::add(acc, gl::add(gl::add(term(v0, b0), term(v1, b1)), gl::add(term(v2, b2), term(v3, b3))));
         }
+        for (; k < k1; k += STEP) acc = gl::add(acc, term(ax_load(a, base + k * a.stride_k), gl::e2(a.b0[k], a.b1[k])));
     }
     lds[threadIdx.x * 2] = acc.c0;
     lds[threadIdx.x * 2 + 1] = acc.c1;
@@ -2087,11 +2094,17 @@ __global__ void __launch_bounds__(BLOCK) axis_dot_row_kernel(AxisArgs a)
     u64 k0 = (u64)slice * a.k_per_slice, k1 = k0 + a.k_per_slice;
     if (k1 > a.K) k1 = a.K;
     E2 acc[1] = {gl::e2_zero()};
-    for (u64 k = k0 + threadIdx.x; k < k1; k += BLOCK) {
-        E2 v = ax_load(a, base + k * a.stride_k);
-        E2 b = gl::e2(a.b0[k], a.b1[k]);
-        acc[0] = gl::add(acc[0], (a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0)));
+    // four elements in flight per lane
+    auto term = [&](E2 v, E2 b) { return a.in1 ? gl::mul(v, b) : gl::mul_base(b, v.c0); };
+    u64 k = k0 + threadIdx.x;
+    for (; k + 3 * BLOCK < k1; k += 4 * BLOCK) {
+        const E2 v0 = ax_load(a, base + k * a.stride_k), v1 = ax_load(a, base + (k + BLOCK) * a.stride_k);
+        const E2 v2 = ax_load(a, base + (k + 2 * BLOCK) * a.stride_k), v3 = ax_load(a, base + (k + 3 * BLOCK) * a.stride_k);
+        const E2 b0 = gl::e2(a.b0[k], a.b1[k]), b1 = gl::e2(a.b0[k + BLOCK], a.b1[k + BLOCK]);
+        const E2 b2 = gl::e2(a.b0[k + 2 * BLOCK], a.b1[k + 2 * BLOCK]), b3 = gl::e2(a.b0[k + 3 * BLOCK], a.b1[k + 3 * BLOCK]);
+        acc[0] = gl::add(acc[0], gl::add(gl::add(term(v0, b0), term(v1, b1)), gl::add(term(v2, b2), term(v3, b3))));
     }
+    for (; k < k1; k += BLOCK) acc[0] = gl::add(acc[0], term(ax_load(a, base + k * a.stride_k), gl::e2(a.b0[k], a.b1[k])));
     block_reduce<1>(acc, lds);
     if (threadIdx.x == 0) {
         u64 o = ((u64)slice * a.P + pre) * a.C + i;
