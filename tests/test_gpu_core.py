@@ -64,6 +64,31 @@ def test_eq_table(ctx, orc, m):
     assert (got == orc.eq_evals(point)).all()
 
 
+@pytest.mark.parametrize("m", [19, 21])
+def test_eq_table_read_as_entries_after_a_session(dp, ctx, orc, m):
+    """An eq table of more than 17 variables is built piecewise: the small suffix levels with the table, the rest when
+    something reads them.  A product session (which reads levels, not entries), then the table's own entries through a
+    view, an evaluation and a download: each finds what it needs, whatever was built before."""
+    point = rand_e2(m, 70 + m)
+    f = rand_base(1 << m, 71 + m)
+    eq, mf = ctx.eq_build(point), ctx.mle_from_base(f)
+    terms = [(np.array([1, 0], dtype=np.uint64), [0, 1])]
+    want_eq = orc.eq_evals(point)
+    ref = orc.sc_prove(m, [want_eq, orc.embed_base(f)], terms, orc.OracleTranscript(b"lazy"))
+    got = ctx.sumcheck_prover(m, [eq, mf], terms)(dp.Transcript(b"lazy"))
+    assert all((a == b).all() for a, b in zip(got, ref))
+    half = eq.view(1 << (m - 1), m - 1).download()
+    assert (half == want_eq[1 << (m - 1):]).all()
+    z = rand_e2(m, 72 + m)
+    assert (eq.evaluate(z) == orc.mle_evaluate(want_eq, z)).all()
+    assert (eq.download() == want_eq).all()
+    # and in the other order: entries first, a session afterwards
+    eq2 = ctx.eq_build(point)
+    assert (eq2.download() == want_eq).all()
+    got2 = ctx.sumcheck_prover(m, [eq2, mf], terms)(dp.Transcript(b"lazy"))
+    assert all((a == b).all() for a, b in zip(got2, ref))
+
+
 def test_i64_embedding_and_padding(ctx, orc):
     v = rand_i64(300, 31, lo=-2**40, hi=2**40)
     v[:4] = [0, -1, 2**62, -(2**62)]
