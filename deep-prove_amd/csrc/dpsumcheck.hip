@@ -2598,6 +2598,654 @@ int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u64 *out)
 
 }  // namespace
 
+namespace {
+
+// One round of a session on the fused kernels -- a product of full-size tables, or sums of several terms over shared
+// tables: what the ways a round can run have in common (the launch arguments, the mail, the message formed on the host
+// from the sums a kernel hands over), and one function per way: a trip of a resident launch, a multi-term launch, a
+// product launch.
+struct FusedRound {
+    dps_sc *sc;
+    dps_ctx *ctx;
+    u32 j;
+    const uint64_t *challenge;
+    uint64_t *evals_out;
+    u64 n_pairs;
+    u32 blocks;
+    E2 cst;            // the constant terms' share of every evaluation
+    dpk::FinArgs fa;   // (its sequence number and result area)
+    dpk::ProdArgs a;
+    dpk::FastFin ff;
+    bool has_eq;
+    u32 nf;
+    E2 base_scale, s1;
+    bool skip1;
+    // the kernels hand over the sums q(t); the message is formed from them here (take_sums)
+    struct {
+        u64 scale[2 * dpk::MAX_PTS];  // p(t) = scale(t) q(t) + const, t = 0..nf
+        u64 cext[2 * dpk::MAX_PTS];   // eq factor: p(nf + 1) = sum_i cext_i q(i) + k + const
+        u64 k0, k1;
+    } hf;
+    // sums of several terms: groups of tables, and whether the single group's descriptors travel in the kernel arguments
+    u32 n_groups;
+    bool inline_descs;
+    // What a launch for round jj looks like: the kernel, its grid, whether it stays for the later rounds.
+    // Nothing here depends on a challenge, so a launch can be planned (and made) before its round begins.
+    struct Plan {
+        bool split, reside;
+        u32 split_log, blocks;
+        u64 n_pairs;
+    };
+
+    int32_t begin();
+    void set_eq_weights(dpk::ProdArgs &pa, u32 jj, u32 blocks_jj) const;
+    void prepare_message();
+    void post_mail();
+    void form_message(const E2 *q);
+    int32_t take_sums(u32 n_slots);
+    int32_t end_waiting_launch();
+    int32_t launch_stages_at(u64 seq0);
+    int32_t resident_round();
+    Plan plan_round(u32 jj, bool skip1_jj) const;
+    int32_t launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj);
+    u32 slots_of(const Plan &p) const { return p.reside ? (n_groups > 1 ? n_groups : 0) : slots_for(p.blocks * n_groups); }
+    int32_t multi_term_round();
+    int32_t product_launch_ahead();
+    int32_t product_round();
+};
+
+
+// The arguments every way of running the round shares; ends a launch that waits on the GPU but cannot take this round.
+int32_t FusedRound::begin()
+{
+    a = sc->fast_args[j];
+    has_eq = sc->fast_eq >= 0;
+    nf = sc->fast_nf;
+    n_groups = sc->poly ? (u32)sc->poly_tabs.size() : 0;
+    inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
+    memset(&ff, 0, sizeof ff);
+    memset(&hf, 0, sizeof hf);
+    if (j >= 2) {
+        const E2 r = gl::e2(challenge[0], challenge[1]);
+        a.r0 = r.c0;
+        a.r1 = r.c1;
+        CHK(launch_folds(sc, j, true, challenge));
+        if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
+    }
+    // scale(t) = coeff * S * eq1(rho_{j-1}, t).  Only whether scale(1) vanishes matters to the kernel (it then has to
+    // evaluate t = 1); everything else about the message is worked out while the kernel runs (prepare_message).
+    base_scale = sc->fast_coeff;
+    if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
+    s1 = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2_one())) : base_scale;
+    skip1 = (j >= 2 || sc->have_claim) && !(s1.c0 == 0 && s1.c1 == 0);
+    a.skip1 = skip1 ? 1 : 0;
+    if (has_eq) set_eq_weights(a, j, blocks);
+    ff.partial = sc->d_partial;
+    ff.n_blocks = blocks;
+    ff.out_host = fa.out_host;
+    ff.seq = fa.seq;
+    ff.counter = sc->d_counter;
+    if (sc->tail_running && !sc->wait_any_skip1 && ((a.skip1 != 0) != sc->wait_skip1)) CHK(end_waiting_launch());
+    if (sc->tail_running && sc->wait_fresh &&
+        std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS))
+        CHK(end_waiting_launch());
+    return DPS_OK;
+}
+
+// where round jj finds its eq weights: level jj, or for the large rounds of a product (a grid whose stride is a
+// multiple of the low table's size) the low table of level jj and level jj + 16
+void FusedRound::set_eq_weights(dpk::ProdArgs &pa, u32 jj, u32 blocks_jj) const
+{
+        const u64 off = eq_level_off(sc->n_vars, jj);
+        pa.q0 = sc->eq_c0 + off;
+        pa.q1 = sc->eq_c1 + off;
+        if (sc->fast && sc->eq_info->fact_built && jj <= sc->eq_info->fact_levels && ((u64)blocks_jj * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
+            const u64 lo = eq_low_off(sc->n_vars, jj), hi = eq_level_off(sc->n_vars, jj + dpk::EQ_LO_BITS);
+            pa.lq0 = sc->eq_c0 + lo;
+            pa.lq1 = sc->eq_c1 + lo;
+            pa.hq0 = sc->eq_c0 + hi;
+            pa.hq1 = sc->eq_c1 + hi;
+        }
+}
+
+// scale(t), the claim and the extrapolation coefficients of this round's message: worked out while the kernel runs
+void FusedRound::prepare_message()
+{
+        if (j >= 2) {
+            // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
+            const E2 r = gl::e2(challenge[0], challenge[1]);
+            const u32 d = sc->degree;
+            E2 acc = gl::e2_zero();
+            for (u32 k = 0; k <= d; k++) {
+                E2 num = gl::e2_one();
+                for (u32 m = 0; m <= d; m++)
+                    if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+                acc = gl::add(acc, gl::mul(gl::mul_base(num, ctx->h_inv_den[d][k]), sc->last_msg[k]));
+            }
+            sc->claim = acc;
+        }
+        for (u32 t = 0; t <= sc->degree; t++) {
+            E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
+            hf.scale[2 * t] = sc_t.c0;
+            hf.scale[2 * t + 1] = sc_t.c1;
+        }
+        if (has_eq) {
+            // p(nf + 1) = sum_i cext_i q(i) + k + const
+            const E2 s_top = gl::e2(hf.scale[2 * (nf + 1)], hf.scale[2 * (nf + 1) + 1]);
+            E2 cext[dpk::MAX_PTS];
+            for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
+            if (skip1) {
+                // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
+                const E2 A = gl::mul(cext[1], h_e2_inv(s1));
+                cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(hf.scale[0], hf.scale[1])));
+                const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
+                hf.k0 = kk.c0;
+                hf.k1 = kk.c1;
+                cext[1] = gl::e2_zero();
+            }
+            for (u32 i = 0; i <= nf; i++) {
+                hf.cext[2 * i] = cext[i].c0;
+                hf.cext[2 * i + 1] = cext[i].c1;
+            }
+        }
+}
+
+// mail for a kernel that waits on the GPU: challenge, whether t = 1 is skipped; then the sequence number it waits for
+void FusedRound::post_mail()
+{
+        u64 *mb = mailbox(ctx);
+        mb[dpk::MAIL_R] = a.r0;
+        mb[dpk::MAIL_R + 1] = a.r1;
+        mb[dpk::MAIL_RA] = sc->prev_chal.c0;
+        mb[dpk::MAIL_RA + 1] = sc->prev_chal.c1;
+        mb[dpk::MAIL_SKIP1] = a.skip1;
+        send_mail(ctx, fa.seq);
+}
+
+// the message from the sums q(0..nf) (prepare_message has run): p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was
+// skipped; with an eq factor p(nf + 1) by extrapolation of q
+void FusedRound::form_message(const E2 *q)
+{
+        const u32 np = nf + 1;
+        E2 msg[dpk::MAX_PTS + 1];
+        for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(hf.scale[2 * t], hf.scale[2 * t + 1]), q[t]), cst);
+        if (a.skip1) msg[1] = gl::sub(sc->claim, msg[0]);
+        if (has_eq) {
+            E2 e = gl::add(gl::e2(hf.k0, hf.k1), cst);
+            for (u32 i = 0; i < np; i++)
+                if (!(a.skip1 && i == 1)) e = gl::add(e, gl::mul(gl::e2(hf.cext[2 * i], hf.cext[2 * i + 1]), q[i]));
+            msg[np] = e;
+        }
+        sc->last_msg.resize(sc->degree + 1);
+        for (u32 t = 0; t <= sc->degree; t++) {
+            evals_out[2 * t] = msg[t].c0;
+            evals_out[2 * t + 1] = msg[t].c1;
+            sc->last_msg[t] = msg[t];
+        }
+}
+
+// Waits for the sums q(t), t = 0..nf, of this round (one set in the main result area, or n_slots sets in areas of their own --
+// resident groups, or the workgroups of a small launch -- which are added) and forms the message.
+int32_t FusedRound::take_sums(u32 n_slots)
+{
+        prepare_message();
+        const u32 np = nf + 1;
+        E2 q[dpk::MAX_PTS];
+        u64 w[2 * dpk::MAX_PTS];
+        if (n_slots) {
+            for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+            for (u32 g = 0; g < n_slots; g++) {
+                CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
+                for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
+            }
+        } else {
+            CHK(wait_result(ctx, fa.seq, 0, 2 * np, w));
+            for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
+        }
+        form_message(q);
+        return DPS_OK;
+}
+
+// A launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an earlier
+// round, or one made ahead during the previous round.  It cannot be used when it was compiled for the other way
+// of getting p(1) (wait_any_skip1: the tail kernel, which takes either), or when it has had no mail yet and the
+// caller took its time: it may have given up waiting (it polls for much longer than the limit here, so up to
+// that limit it certainly has not).  Then it is ended and the round is launched normally.
+int32_t FusedRound::end_waiting_launch()
+{
+        __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
+        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+        __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
+        reset_device_words(ctx);
+        sc->tail_running = false;
+        sc->wait_fresh = false;
+        ctx->tail_owner = nullptr;
+        return DPS_OK;
+}
+
+// The launches of the resident rounds, queued one behind the other: the trip that starts at the first resident
+// round has the sequence number seq0 (a round's call takes one number whether or not it makes a trip).
+int32_t FusedRound::launch_stages_at(u64 seq0)
+{
+        const u32 first = sc->tail_j0;
+        for (size_t si = 0; si < sc->stages.size(); si++) {
+            const dps_sc::Stage &st = sc->stages[si];
+            // a stage of several workgroups and the single-workgroup stage that runs to the last round are one launch:
+            // the first workgroup takes the others' entries up and goes on alone
+            const bool merged = st.W > 1 && si + 2 == sc->stages.size() && sc->stages[si + 1].W == 1 && sc->stages[si + 1].cap <= st.cap;
+            const size_t last_si = merged ? si + 1 : si;
+            dpk::SliceArgs sa;
+            memset(&sa, 0, sizeof sa);
+            const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : nf;
+            for (u32 f = 0; f < n_tabs; f++) {
+                // the first stage reads what the launch of the round before it wrote (or the session's own tables)
+                if (si > 0) {
+                    sa.s0[f] = sc->stages[si - 1].h0[f];
+                    sa.s1[f] = sc->stages[si - 1].h1[f];
+                } else if (sc->poly) {
+                    const dpk::PolyTab &tb = sc->h_poly_groups[first - 1].tab[f];
+                    sa.s0[f] = tb.s0;
+                    sa.s1[f] = tb.s1;
+                } else {
+                    sa.s0[f] = sc->fast_args[first].s0[f];
+                    sa.s1[f] = sc->fast_args[first].s1[f];
+                }
+                sa.h0[f] = st.h0[f];
+                sa.h1[f] = st.h1[f];
+            }
+            sa.n_tabs = n_tabs;
+            if (sc->poly) {
+                sa.n_terms = (u32)sc->h_poly_terms.size();
+                for (u32 m = 0; m < sa.n_terms; m++) {
+                    const dpk::PolyTerm &pt = sc->h_poly_terms[m];
+                    dpk::SliceTerm &tm = sa.terms[m];
+                    tm.c0 = pt.c0, tm.c1 = pt.c1, tm.w = pt.w;
+                    tm.n_factors = pt.n_factors;
+                    memcpy(tm.slot, pt.slot, sizeof tm.slot);
+                }
+            }
+            sa.src_len = st.src_len;
+            sa.pend0 = st.pend0;
+            sa.n_vars = sc->n_vars;
+            sa.j0 = st.j0;
+            sa.n_trips = st.n_trips;
+            sa.dbl_mask = st.dbl_mask;
+            if (merged) {
+                sa.n_trips2 = sc->stages[si + 1].n_trips;
+                sa.dbl_mask2 = sc->stages[si + 1].dbl_mask;
+            }
+            sa.eq0 = sc->eq_c0;
+            sa.eq1 = sc->eq_c1;
+            sa.mail = ctx->d_pinned + (ctx->res_off - 64);
+            // (several workgroups: the first polls the host's mailbox and passes each mail on through device memory; with
+            // all 256 of them polling host memory a trip took 90 us instead of 18)
+            sa.relay = mail_relay(ctx);
+            sa.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
+            sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
+            sa.out_host = ctx->d_pinned + slice_area_off(ctx);
+            sa.seq0 = seq0 + (st.j0 - first);
+            sa.ctr = ctx->d_slice_ctr;
+            sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
+            ProfScope ps(ctx, DPS_K_TAIL, 0.0);
+            CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
+            HIPCHK(ctx, hipGetLastError());
+            // a launch of several workgroups that nobody takes over from inside leaves its counters as they are
+            if (st.W > 1 && !merged) reset_device_words(ctx);
+            si = last_si;
+        }
+        memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
+        // no resident launch of this context is running now: whatever an abandoned one left in the result area goes
+        for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
+        sc->tail_seq0 = seq0;
+        sc->tail_running = true;
+        sc->wait_any_skip1 = true;
+        sc->wait_slots = 0;
+        ctx->tail_owner = sc;
+        return DPS_OK;
+}
+
+// A round among the resident ones (slice_kernel): a trip to the launch, or the second round of a trip, answered here.
+int32_t FusedRound::resident_round()
+{
+    const u32 kind = sc->round_kind[j];
+    const u32 np = nf + 1;
+    E2 q[dpk::MAX_PTS];
+    int32_t rc = DPS_OK;
+    if (kind == 3) {
+        // Second round of a trip: the kernel handed over this round's sums as a polynomial in the challenge that has
+        // now been drawn (values at 0..nf-1 and the leading coefficient, per point t = 0, 2, .., nf); p(1) comes
+        // from the claim.  Nothing goes to the GPU.
+        const E2 r = gl::e2(challenge[0], challenge[1]);
+        E2 vanish = gl::e2_one(), basis[dpk::MAX_PTS];
+        for (u32 k = 0; k < nf; k++) {
+            E2 num = gl::e2_one();
+            for (u32 m = 0; m < nf; m++)
+                if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
+            basis[k] = gl::mul_base(num, ctx->h_inv_den[nf - 1][k]);
+            vanish = gl::mul(vanish, gl::sub(r, gl::e2(k, 0)));
+        }
+        for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
+        for (u32 ti = 0; ti < nf; ti++) {
+            E2 v = gl::mul(vanish, sc->stash[nf * nf + ti]);
+            for (u32 k = 0; k < nf; k++) v = gl::add(v, gl::mul(basis[k], sc->stash[k * nf + ti]));
+            q[ti == 0 ? 0 : ti + 1] = v;
+        }
+        prepare_message();
+        form_message(q);
+    } else {
+        if (!sc->tail_running) {
+            if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
+            CHK(launch_stages_at(fa.seq));
+        }
+        post_mail();
+        sc->wait_fresh = false;
+        prepare_message();
+        // sums of this round, and with a trip of two rounds those of the next
+        const u32 ns = kind == 2 ? np + np * nf : np;
+        u64 cnt[4 * dpk::SL_MAX_SUMS];
+        rc = wait_slice_sums(ctx, fa.seq, ns, a.skip1 != 0, cnt);
+        if (rc == DPS_OK) {
+            // several workgroups: the counters run on from trip to trip of the launch
+            if (sc->round_wide[j])
+                for (u32 c = 0; c < 4 * ns; c++) {
+                    if (a.skip1 && c >= 4 && c < 8) continue;
+                    const u64 now = cnt[c];
+                    cnt[c] = now - sc->ctr_seen[c];
+                    sc->ctr_seen[c] = now;
+                }
+            // limb w & 1 of sum w >> 1: counters 2w (low halves) and 2w + 1 (high halves)
+            u64 w[2 * dpk::SL_MAX_SUMS];
+            for (u32 i = 0; i < 2 * ns; i++) {
+                const unsigned __int128 t = (unsigned __int128)cnt[2 * i] + ((unsigned __int128)cnt[2 * i + 1] << 32);
+                w[i] = gl::reduce128((u64)t, (u64)(t >> 64));
+            }
+            for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
+            for (u32 i = np; i < ns; i++) sc->stash[i - np] = gl::e2(w[2 * i], w[2 * i + 1]);
+            form_message(q);
+            sc->last_trip_seq = fa.seq;
+        }
+    }
+    if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
+    if (j == sc->n_vars || rc != DPS_OK) {
+        // with its last trip the kernel publishes what is left of the tables and exits
+        sc->tail_running = false;
+        ctx->tail_owner = nullptr;
+        if (rc == DPS_OK) sc->pairs_seq = sc->last_trip_seq;
+    }
+    if (rc != DPS_OK) {
+        // the launch left without publishing (it gave up waiting, or the stream failed): nothing of it can be used again
+        sc->broken = true;
+        reset_device_words(ctx);
+    }
+    CHK(rc);
+    sc->round = j;
+    return DPS_OK;
+}
+
+FusedRound::Plan FusedRound::plan_round(u32 jj, bool skip1_jj) const
+{
+        Plan p;
+        p.n_pairs = 1ull << (sc->n_vars - jj);
+        p.split = p.n_pairs <= POLY_SPLIT_MAX_PAIRS;
+        p.split_log = 0;
+        p.blocks = blocks_for_pairs(p.n_pairs);
+        if (p.split) poly_split_plan(p.n_pairs, sc->poly_split_cap, n_groups <= POLY_RAW_MAX_GROUPS, &p.split_log, &p.blocks);
+        // a single workgroup (per group) from here on: it stays for the remaining rounds
+        // (several groups stay only with their tables in LDS: they must not read each other's stores)
+        p.reside = p.split && n_groups <= POLY_RAW_MAX_GROUPS && p.blocks == 1 && skip1_jj && jj < sc->n_vars &&
+                   sc->n_vars - jj + 1 <= (u32)dpk::POLY_RES_ROUNDS && (n_groups == 1 || poly_split_state_ok(ctx, nf, has_eq, true));
+        return p;
+}
+
+// Launches the kernel of round jj.  `ahead`: round jj has not begun (its challenge is not known); the kernel
+// waits for the mail of sequence number `seq_jj` and takes the challenge and the message's scalars from it.
+int32_t FusedRound::launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj)
+{
+        dpk::PolyArgs pa;
+        pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
+        pa.terms = sc->d_poly_terms;
+        pa.ops = sc->d_poly_ops;
+        if (inline_descs) {
+            pa.groups = nullptr;
+            pa.terms = nullptr;
+            pa.ops = nullptr;
+            pa.g0 = sc->h_poly_groups[jj - 1];
+            if (!p.split && !sc->h_poly_ops.empty())
+                memcpy(pa.o0, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
+            else
+                std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
+        } else {
+            CHK(ensure_descs(sc));
+        }
+        pa.q0 = pa.q1 = nullptr;
+        if (has_eq) {
+            const u64 off = eq_level_off(sc->n_vars, jj);
+            pa.q0 = sc->eq_c0 + off;
+            pa.q1 = sc->eq_c1 + off;
+        }
+        pa.n_pairs = p.n_pairs;
+        pa.r0 = ahead ? 0 : a.r0;
+        pa.r1 = ahead ? 0 : a.r1;
+        pa.j = jj;
+        pa.last_round = 0;
+        pa.n_vars = sc->n_vars;
+        pa.spin_limit = 4000000;
+        pa.eq0 = sc->eq_c0;
+        pa.eq1 = sc->eq_c1;
+        pa.mail = ctx->d_pinned + (ctx->res_off - 64);
+        pa.seq = seq_jj;
+        pa.split_log = p.split_log;
+        pa.split_cap = sc->poly_split_cap;
+        pa.lds_state = pa.state_off = pa.pad = 0;
+        pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
+        pa.group_stride = 1;
+        pa.raw_out = nullptr;
+        pa.wait_first = ahead ? 1 : 0;
+        if (ahead && !p.reside) pa.spin_limit = AHEAD_SPIN_LIMIT;
+        // (more workgroups than should poll the host's memory: the first one polls and passes the mail on)
+        pa.relay = ahead && p.blocks * n_groups > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
+        if (p.reside) {
+            pa.last_round = sc->n_vars;
+            if (n_groups > 1) {
+                // one resident workgroup per group, each publishing its own sums
+                CHK(ensure_descs(sc));
+                pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
+                pa.group_stride = n_groups;
+                pa.raw_out = ctx->d_pinned + poly_raw_off(ctx);
+            } else if (inline_descs) {
+                // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
+                // before anything else (and before it looks for mail); the area is not written again before a
+                // message of this launch has arrived
+                const size_t words = (size_t)(sc->n_vars - jj + 1) * sizeof(dpk::PolyGroup) / 8;
+                memcpy(ctx->h_pinned, &sc->h_poly_groups[jj - 1], words * 8);
+                pa.groups = reinterpret_cast<const dpk::PolyGroup *>(ctx->d_pinned);
+            } else {
+                pa.groups = sc->d_poly_groups + (size_t)(jj - 1);
+            }
+        }
+        dpk::FastFin fl = ff;
+        fl.seq = seq_jj;
+        fl.n_blocks = p.blocks * n_groups;
+        fl.slots = !p.reside && slots_for(fl.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
+        double pbytes = has_eq ? (double)p.n_pairs * 16.0 : 0.0;
+        for (u32 k = 0; k < sc->n_mles; k++)
+            if (sc->poly_owner[k] >= 0) pbytes += (double)p.n_pairs * (jj >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
+        ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
+        if (p.split)
+            CHK(launch_poly_split_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, p.reside, sc->d_partial, fl));
+        else
+            CHK(launch_poly_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, sc->d_partial, fl));
+        HIPCHK(ctx, hipGetLastError());
+        return DPS_OK;
+}
+
+// A round of sums of several terms over shared tables (poly_kernel / poly_split_kernel): this round's launch, or the mail for
+// one that waits on the GPU; then the next round's launch behind it.
+int32_t FusedRound::multi_term_round()
+{
+    // a launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an
+    // earlier round, or one made ahead during the previous round
+    const bool on_gpu = sc->tail_running;
+    bool stays;
+    u32 slots_now;
+    if (on_gpu) {
+        post_mail();
+        sc->wait_fresh = false;
+        stays = sc->wait_stays;
+        slots_now = sc->wait_slots;
+    } else {
+        const Plan p = plan_round(j, a.skip1 != 0);
+        CHK(launch_round(j, p, a.skip1 != 0, false, fa.seq));
+        stays = p.reside;
+        slots_now = slots_of(p);
+        if (p.reside) {
+            sc->tail_running = true;
+            sc->tail_seq0 = fa.seq;
+            ctx->tail_owner = sc;
+            sc->poly_raw = n_groups > 1;
+            sc->wait_slots = slots_now;
+            sc->wait_stays = true;
+            sc->wait_skip1 = true;
+            sc->wait_fresh = false;
+        }
+    }
+    if (!stays) {
+        // the launch of this round ends with it
+        sc->tail_running = false;
+        ctx->tail_owner = nullptr;
+        // The next round's launch is made now, behind this one: by the time this round's message has crossed to
+        // the host and the challenge is drawn, it is already on the GPU looking for its mail.  Only for rounds
+        // of few workgroups (every workgroup polls the mailbox), and not while launches are being timed.
+        if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
+            // p(1) comes from the claim unless the scale vanishes at 1, i.e. unless the eq point is 0 there
+            bool skip1_next = true;
+            if (has_eq) {
+                const E2 rho = sc->eq_info->point[j];
+                skip1_next = !(rho.c0 == 0 && rho.c1 == 0);
+            }
+            const Plan pn = plan_round(j + 1, skip1_next);
+            if (sc->tail_j0 && j + 1 == sc->tail_j0) {
+                // the rounds from here on are resident: their launches are queued now and wait for their first mail
+                CHK(launch_stages_at(ctx->seq + 1));
+                sc->wait_fresh = true;
+                sc->ahead_at = std::chrono::steady_clock::now();
+            } else {
+                CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
+                sc->tail_running = true;
+                sc->tail_seq0 = ctx->seq + 1;
+                ctx->tail_owner = sc;
+                sc->wait_stays = pn.reside;
+                sc->wait_skip1 = skip1_next;
+                sc->wait_fresh = true;
+                sc->ahead_at = std::chrono::steady_clock::now();
+                sc->poly_raw = pn.reside && n_groups > 1;
+                sc->wait_slots = slots_of(pn);
+            }
+        }
+    }
+    int32_t rc = take_sums(slots_now);
+    if (rc != DPS_OK) {
+        // a launch that left without publishing may have taken some of its tickets and written some of its tables
+        sc->broken = true;
+        reset_device_words(ctx);
+    }
+    if (stays && (rc != DPS_OK || j == sc->n_vars)) {
+        // a resident launch exits after the last round; one that can finish has published the tables' last pairs with it
+        sc->tail_running = false;
+        ctx->tail_owner = nullptr;
+        if (rc == DPS_OK && sc->poly_finish_in_kernel) sc->pairs_seq = fa.seq;
+    }
+    CHK(rc);
+    sc->round = j;
+    return DPS_OK;
+}
+
+// The next round's launch, made behind this round's (for the same reasons as in multi_term_round): the resident launches, or a
+// product kernel, which then waits for its challenge by mail.
+int32_t FusedRound::product_launch_ahead()
+{
+    if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
+        const u64 next_seq = ctx->seq + 1;
+        bool made = false;
+        if (sc->tail_j0 && j + 1 == sc->tail_j0) {
+            CHK(launch_stages_at(next_seq));
+            made = true;
+        } else {
+            // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
+            // p(1) comes from the claim unless the scale vanishes at 1
+            bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
+            if (has_eq) {
+                const E2 rho = sc->eq_info->point[j];
+                skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
+            }
+            dpk::ProdArgs an = sc->fast_args[j + 1];
+            if (has_eq) set_eq_weights(an, j + 1, blocks_for_pairs(n_pairs >> 1));
+            an.r0 = an.r1 = 0;
+            an.skip1 = skip1_next ? 1 : 0;
+            an.wait_first = 1;
+            an.spin_limit = AHEAD_SPIN_LIMIT;
+            an.mail = ctx->d_pinned + (ctx->res_off - 64);
+            an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
+            dpk::FastFin fn = ff;
+            fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
+            fn.seq = next_seq;
+            fn.slots = slots_for(fn.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
+            sc->wait_slots = slots_for(fn.n_blocks);
+            CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j + 1], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
+            HIPCHK(ctx, hipGetLastError());
+            sc->wait_any_skip1 = false;
+            sc->wait_skip1 = skip1_next;
+            made = true;
+        }
+        if (made) {
+            sc->tail_running = true;
+            sc->wait_fresh = true;
+            sc->ahead_at = std::chrono::steady_clock::now();
+            ctx->tail_owner = sc;
+        }
+    }
+
+    return DPS_OK;
+}
+
+// A round of a product of full-size tables (prod_kernel).
+int32_t FusedRound::product_round()
+{
+    u32 slots_now = sc->wait_slots;
+    if (sc->tail_running) {
+        // launched during the previous round
+        post_mail();
+        sc->wait_fresh = false;
+    } else {
+        slots_now = slots_for(blocks);
+        ff.slots = slots_now ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
+        // (in the factored form the eq weights are one entry per thread and one per workgroup and step: not counted)
+        double bytes = has_eq && !a.lq0 ? (double)n_pairs * 16.0 : 0.0;
+        for (u32 f = 0; f < nf; f++) {
+            double eb = a.s1[f] ? 16.0 : 8.0;
+            bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
+        }
+        ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
+        a.wait_first = 0;
+        CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j], has_eq, j >= 2, a, blocks, sc->d_partial, ff));
+        HIPCHK(ctx, hipGetLastError());
+    }
+    // this round's launch ends with the round
+    sc->tail_running = false;
+    ctx->tail_owner = nullptr;
+    CHK(product_launch_ahead());
+    if (const int32_t rc = take_sums(slots_now); rc != DPS_OK) {
+        sc->broken = true;
+        reset_device_words(ctx);
+        return rc;
+    }
+    if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
+    sc->round = j;
+    return DPS_OK;
+}
+
+}  // namespace
+
 extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
 {
     if (!sc || !evals_out) return DPS_ERR_INVALID;
@@ -2636,568 +3284,13 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         dpk::finalize_kernel<<<1, dpk::BLOCK, 0, ctx->stream>>>(fa);
         HIPCHK(ctx, hipGetLastError());
     } else if (sc->fast || sc->poly) {
-        dpk::ProdArgs a = sc->fast_args[j];
-        const bool has_eq = sc->fast_eq >= 0;
-        const u32 nf = sc->fast_nf;
-        dpk::FastFin ff;
-        memset(&ff, 0, sizeof ff);
-        // the kernels hand over the sums q(t); the message is formed from them here (take_sums)
-        struct {
-            u64 scale[2 * dpk::MAX_PTS];  // p(t) = scale(t) q(t) + const, t = 0..nf
-            u64 cext[2 * dpk::MAX_PTS];   // eq factor: p(nf + 1) = sum_i cext_i q(i) + k + const
-            u64 k0, k1;
-        } hf;
-        memset(&hf, 0, sizeof hf);
-        if (j >= 2) {
-            const E2 r = gl::e2(challenge[0], challenge[1]);
-            a.r0 = r.c0;
-            a.r1 = r.c1;
-            CHK(launch_folds(sc, j, true, challenge));
-            if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
-        }
-        // scale(t) = coeff * S * eq1(rho_{j-1}, t).  Only whether scale(1) vanishes matters to the kernel (it then has to
-        // evaluate t = 1); everything else about the message is worked out while the kernel runs (prepare_message).
-        E2 base_scale = sc->fast_coeff;
-        if (has_eq) base_scale = gl::mul(base_scale, sc->eq_scalar);
-        const E2 s1 = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2_one())) : base_scale;
-        const bool skip1 = (j >= 2 || sc->have_claim) && !(s1.c0 == 0 && s1.c1 == 0);
-        a.skip1 = skip1 ? 1 : 0;
-        // where round jj finds its eq weights: level jj, or for the large rounds of a product (a grid whose stride is a
-        // multiple of the low table's size) the low table of level jj and level jj + 16
-        auto set_eq_weights = [&](dpk::ProdArgs &pa, u32 jj, u32 blocks_jj) {
-            const u64 off = eq_level_off(sc->n_vars, jj);
-            pa.q0 = sc->eq_c0 + off;
-            pa.q1 = sc->eq_c1 + off;
-            if (sc->fast && sc->eq_info->fact_built && jj <= sc->eq_info->fact_levels && ((u64)blocks_jj * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0) {
-                const u64 lo = eq_low_off(sc->n_vars, jj), hi = eq_level_off(sc->n_vars, jj + dpk::EQ_LO_BITS);
-                pa.lq0 = sc->eq_c0 + lo;
-                pa.lq1 = sc->eq_c1 + lo;
-                pa.hq0 = sc->eq_c0 + hi;
-                pa.hq1 = sc->eq_c1 + hi;
-            }
-        };
-        if (has_eq) set_eq_weights(a, j, blocks);
-        auto prepare_message = [&]() {
-            if (j >= 2) {
-                // claim of this round: the previous message at the challenge (Lagrange over 0..degree)
-                const E2 r = gl::e2(challenge[0], challenge[1]);
-                const u32 d = sc->degree;
-                E2 acc = gl::e2_zero();
-                for (u32 k = 0; k <= d; k++) {
-                    E2 num = gl::e2_one();
-                    for (u32 m = 0; m <= d; m++)
-                        if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
-                    acc = gl::add(acc, gl::mul(gl::mul_base(num, ctx->h_inv_den[d][k]), sc->last_msg[k]));
-                }
-                sc->claim = acc;
-            }
-            for (u32 t = 0; t <= sc->degree; t++) {
-                E2 sc_t = has_eq ? gl::mul(base_scale, h_eq1(sc->eq_info->point[j - 1], gl::e2(t, 0))) : base_scale;
-                hf.scale[2 * t] = sc_t.c0;
-                hf.scale[2 * t + 1] = sc_t.c1;
-            }
-            if (has_eq) {
-                // p(nf + 1) = sum_i cext_i q(i) + k + const
-                const E2 s_top = gl::e2(hf.scale[2 * (nf + 1)], hf.scale[2 * (nf + 1) + 1]);
-                E2 cext[dpk::MAX_PTS];
-                for (u32 i = 0; i <= nf; i++) cext[i] = gl::mul_base(s_top, ctx->h_lagrange[(nf * 9 + (nf + 1)) * 9 + i]);
-                if (skip1) {
-                    // q(1) = (claim - 2 const - scale(0) q(0)) / scale(1)
-                    const E2 A = gl::mul(cext[1], h_e2_inv(s1));
-                    cext[0] = gl::sub(cext[0], gl::mul(A, gl::e2(hf.scale[0], hf.scale[1])));
-                    const E2 kk = gl::mul(A, gl::sub(sc->claim, gl::add(cst, cst)));
-                    hf.k0 = kk.c0;
-                    hf.k1 = kk.c1;
-                    cext[1] = gl::e2_zero();
-                }
-                for (u32 i = 0; i <= nf; i++) {
-                    hf.cext[2 * i] = cext[i].c0;
-                    hf.cext[2 * i + 1] = cext[i].c1;
-                }
-            }
-        };
-        ff.partial = sc->d_partial;
-        ff.n_blocks = blocks;
-        ff.out_host = fa.out_host;
-        ff.seq = fa.seq;
-        ff.counter = sc->d_counter;
-        // mail for a kernel that waits on the GPU: challenge, whether t = 1 is skipped; then the sequence number it waits for
-        auto post_mail = [&]() {
-            u64 *mb = mailbox(ctx);
-            mb[dpk::MAIL_R] = a.r0;
-            mb[dpk::MAIL_R + 1] = a.r1;
-            mb[dpk::MAIL_RA] = sc->prev_chal.c0;
-            mb[dpk::MAIL_RA + 1] = sc->prev_chal.c1;
-            mb[dpk::MAIL_SKIP1] = a.skip1;
-            send_mail(ctx, fa.seq);
-        };
-        // Waits for the sums q(t), t = 0..nf, of this round (one set in the main result area, or n_slots sets in areas
-        // of their own -- resident groups, or the workgroups of a small launch -- which are added) and
-        // forms the message: p(t) = scale(t) q(t) + const; p(1) from the claim when t = 1 was skipped; with an eq factor
-        // p(nf + 1) by extrapolation of q (coefficients above).
-        // the message from the sums q(0..nf) (prepare_message has run)
-        auto form_message = [&](const E2 *q) {
-            const u32 np = nf + 1;
-            E2 msg[dpk::MAX_PTS + 1];
-            for (u32 t = 0; t < np; t++) msg[t] = gl::add(gl::mul(gl::e2(hf.scale[2 * t], hf.scale[2 * t + 1]), q[t]), cst);
-            if (a.skip1) msg[1] = gl::sub(sc->claim, msg[0]);
-            if (has_eq) {
-                E2 e = gl::add(gl::e2(hf.k0, hf.k1), cst);
-                for (u32 i = 0; i < np; i++)
-                    if (!(a.skip1 && i == 1)) e = gl::add(e, gl::mul(gl::e2(hf.cext[2 * i], hf.cext[2 * i + 1]), q[i]));
-                msg[np] = e;
-            }
-            sc->last_msg.resize(sc->degree + 1);
-            for (u32 t = 0; t <= sc->degree; t++) {
-                evals_out[2 * t] = msg[t].c0;
-                evals_out[2 * t + 1] = msg[t].c1;
-                sc->last_msg[t] = msg[t];
-            }
-        };
-        auto take_sums = [&](u32 n_slots) -> int32_t {
-            prepare_message();
-            const u32 np = nf + 1;
-            E2 q[dpk::MAX_PTS];
-            u64 w[2 * dpk::MAX_PTS];
-            if (n_slots) {
-                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
-                for (u32 g = 0; g < n_slots; g++) {
-                    CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
-                    for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
-                }
-            } else {
-                CHK(wait_result(ctx, fa.seq, 0, 2 * np, w));
-                for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
-            }
-            form_message(q);
-            return DPS_OK;
-        };
-        // A launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an earlier
-        // round, or one made ahead during the previous round.  It cannot be used when it was compiled for the other way
-        // of getting p(1) (wait_any_skip1: the tail kernel, which takes either), or when it has had no mail yet and the
-        // caller took its time: it may have given up waiting (it polls for much longer than the limit here, so up to
-        // that limit it certainly has not).  Then it is ended and the round is launched normally.
-        auto end_waiting_launch = [&]() -> int32_t {
-            __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, dpk::MAIL_ABORT_SEQ, __ATOMIC_RELEASE);
-            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-            __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
-            reset_device_words(ctx);
-            sc->tail_running = false;
-            sc->wait_fresh = false;
-            ctx->tail_owner = nullptr;
-            return DPS_OK;
-        };
-        if (sc->tail_running && !sc->wait_any_skip1 && ((a.skip1 != 0) != sc->wait_skip1)) CHK(end_waiting_launch());
-        if (sc->tail_running && sc->wait_fresh &&
-            std::chrono::steady_clock::now() - sc->ahead_at > std::chrono::milliseconds(POLY_AHEAD_PATIENCE_MS))
-            CHK(end_waiting_launch());
-        // The launches of the resident rounds, queued one behind the other: the trip that starts at the first resident
-        // round has the sequence number seq0 (a round's call takes one number whether or not it makes a trip).
-        auto launch_stages_at = [&](u64 seq0) -> int32_t {
-            const u32 first = sc->tail_j0;
-            for (size_t si = 0; si < sc->stages.size(); si++) {
-                const dps_sc::Stage &st = sc->stages[si];
-                // a stage of several workgroups and the single-workgroup stage that runs to the last round are one launch:
-                // the first workgroup takes the others' entries up and goes on alone
-                const bool merged = st.W > 1 && si + 2 == sc->stages.size() && sc->stages[si + 1].W == 1 && sc->stages[si + 1].cap <= st.cap;
-                const size_t last_si = merged ? si + 1 : si;
-                dpk::SliceArgs sa;
-                memset(&sa, 0, sizeof sa);
-                const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : nf;
-                for (u32 f = 0; f < n_tabs; f++) {
-                    // the first stage reads what the launch of the round before it wrote (or the session's own tables)
-                    if (si > 0) {
-                        sa.s0[f] = sc->stages[si - 1].h0[f];
-                        sa.s1[f] = sc->stages[si - 1].h1[f];
-                    } else if (sc->poly) {
-                        const dpk::PolyTab &tb = sc->h_poly_groups[first - 1].tab[f];
-                        sa.s0[f] = tb.s0;
-                        sa.s1[f] = tb.s1;
-                    } else {
-                        sa.s0[f] = sc->fast_args[first].s0[f];
-                        sa.s1[f] = sc->fast_args[first].s1[f];
-                    }
-                    sa.h0[f] = st.h0[f];
-                    sa.h1[f] = st.h1[f];
-                }
-                sa.n_tabs = n_tabs;
-                if (sc->poly) {
-                    sa.n_terms = (u32)sc->h_poly_terms.size();
-                    for (u32 m = 0; m < sa.n_terms; m++) {
-                        const dpk::PolyTerm &pt = sc->h_poly_terms[m];
-                        dpk::SliceTerm &tm = sa.terms[m];
-                        tm.c0 = pt.c0, tm.c1 = pt.c1, tm.w = pt.w;
-                        tm.n_factors = pt.n_factors;
-                        memcpy(tm.slot, pt.slot, sizeof tm.slot);
-                    }
-                }
-                sa.src_len = st.src_len;
-                sa.pend0 = st.pend0;
-                sa.n_vars = sc->n_vars;
-                sa.j0 = st.j0;
-                sa.n_trips = st.n_trips;
-                sa.dbl_mask = st.dbl_mask;
-                if (merged) {
-                    sa.n_trips2 = sc->stages[si + 1].n_trips;
-                    sa.dbl_mask2 = sc->stages[si + 1].dbl_mask;
-                }
-                sa.eq0 = sc->eq_c0;
-                sa.eq1 = sc->eq_c1;
-                sa.mail = ctx->d_pinned + (ctx->res_off - 64);
-                // (several workgroups: the first polls the host's mailbox and passes each mail on through device memory; with
-                // all 256 of them polling host memory a trip took 90 us instead of 18)
-                sa.relay = mail_relay(ctx);
-                sa.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
-                sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
-                sa.out_host = ctx->d_pinned + slice_area_off(ctx);
-                sa.seq0 = seq0 + (st.j0 - first);
-                sa.ctr = ctx->d_slice_ctr;
-                sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
-                ProfScope ps(ctx, DPS_K_TAIL, 0.0);
-                CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
-                HIPCHK(ctx, hipGetLastError());
-                // a launch of several workgroups that nobody takes over from inside leaves its counters as they are
-                if (st.W > 1 && !merged) reset_device_words(ctx);
-                si = last_si;
-            }
-            memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
-            // no resident launch of this context is running now: whatever an abandoned one left in the result area goes
-            for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
-            sc->tail_seq0 = seq0;
-            sc->tail_running = true;
-            sc->wait_any_skip1 = true;
-            sc->wait_slots = 0;
-            ctx->tail_owner = sc;
-            return DPS_OK;
-        };
-        if (sc->tail_j0 && j >= sc->tail_j0) {
-            const u32 kind = sc->round_kind[j];
-            const u32 np = nf + 1;
-            E2 q[dpk::MAX_PTS];
-            int32_t rc = DPS_OK;
-            if (kind == 3) {
-                // Second round of a trip: the kernel handed over this round's sums as a polynomial in the challenge that has
-                // now been drawn (values at 0..nf-1 and the leading coefficient, per point t = 0, 2, .., nf); p(1) comes
-                // from the claim.  Nothing goes to the GPU.
-                const E2 r = gl::e2(challenge[0], challenge[1]);
-                E2 vanish = gl::e2_one(), basis[dpk::MAX_PTS];
-                for (u32 k = 0; k < nf; k++) {
-                    E2 num = gl::e2_one();
-                    for (u32 m = 0; m < nf; m++)
-                        if (m != k) num = gl::mul(num, gl::sub(r, gl::e2(m, 0)));
-                    basis[k] = gl::mul_base(num, ctx->h_inv_den[nf - 1][k]);
-                    vanish = gl::mul(vanish, gl::sub(r, gl::e2(k, 0)));
-                }
-                for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
-                for (u32 ti = 0; ti < nf; ti++) {
-                    E2 v = gl::mul(vanish, sc->stash[nf * nf + ti]);
-                    for (u32 k = 0; k < nf; k++) v = gl::add(v, gl::mul(basis[k], sc->stash[k * nf + ti]));
-                    q[ti == 0 ? 0 : ti + 1] = v;
-                }
-                prepare_message();
-                form_message(q);
-            } else {
-                if (!sc->tail_running) {
-                    if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
-                    CHK(launch_stages_at(fa.seq));
-                }
-                post_mail();
-                sc->wait_fresh = false;
-                prepare_message();
-                // sums of this round, and with a trip of two rounds those of the next
-                const u32 ns = kind == 2 ? np + np * nf : np;
-                u64 cnt[4 * dpk::SL_MAX_SUMS];
-                rc = wait_slice_sums(ctx, fa.seq, ns, a.skip1 != 0, cnt);
-                if (rc == DPS_OK) {
-                    // several workgroups: the counters run on from trip to trip of the launch
-                    if (sc->round_wide[j])
-                        for (u32 c = 0; c < 4 * ns; c++) {
-                            if (a.skip1 && c >= 4 && c < 8) continue;
-                            const u64 now = cnt[c];
-                            cnt[c] = now - sc->ctr_seen[c];
-                            sc->ctr_seen[c] = now;
-                        }
-                    // limb w & 1 of sum w >> 1: counters 2w (low halves) and 2w + 1 (high halves)
-                    u64 w[2 * dpk::SL_MAX_SUMS];
-                    for (u32 i = 0; i < 2 * ns; i++) {
-                        const unsigned __int128 t = (unsigned __int128)cnt[2 * i] + ((unsigned __int128)cnt[2 * i + 1] << 32);
-                        w[i] = gl::reduce128((u64)t, (u64)(t >> 64));
-                    }
-                    for (u32 t = 0; t < np; t++) q[t] = gl::e2(w[2 * t], w[2 * t + 1]);
-                    for (u32 i = np; i < ns; i++) sc->stash[i - np] = gl::e2(w[2 * i], w[2 * i + 1]);
-                    form_message(q);
-                    sc->last_trip_seq = fa.seq;
-                }
-            }
-            if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
-            if (j == sc->n_vars || rc != DPS_OK) {
-                // with its last trip the kernel publishes what is left of the tables and exits
-                sc->tail_running = false;
-                ctx->tail_owner = nullptr;
-                if (rc == DPS_OK) sc->pairs_seq = sc->last_trip_seq;
-            }
-            if (rc != DPS_OK) {
-                // the launch left without publishing (it gave up waiting, or the stream failed): nothing of it can be used again
-                sc->broken = true;
-                reset_device_words(ctx);
-            }
-            CHK(rc);
-            sc->round = j;
-            return DPS_OK;
-        }
-        if (sc->poly) {
-            const u32 n_groups = (u32)sc->poly_tabs.size();
-            const bool inline_descs = n_groups == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS;
-            // What a launch for round jj looks like: the kernel, its grid, whether it stays for the later rounds.
-            // Nothing here depends on a challenge, so a launch can be planned (and made) before its round begins.
-            struct Plan {
-                bool split, reside;
-                u32 split_log, blocks;
-                u64 n_pairs;
-            };
-            auto plan_round = [&](u32 jj, bool skip1_jj) {
-                Plan p;
-                p.n_pairs = 1ull << (sc->n_vars - jj);
-                p.split = p.n_pairs <= POLY_SPLIT_MAX_PAIRS;
-                p.split_log = 0;
-                p.blocks = blocks_for_pairs(p.n_pairs);
-                if (p.split) poly_split_plan(p.n_pairs, sc->poly_split_cap, n_groups <= POLY_RAW_MAX_GROUPS, &p.split_log, &p.blocks);
-                // a single workgroup (per group) from here on: it stays for the remaining rounds
-                // (several groups stay only with their tables in LDS: they must not read each other's stores)
-                p.reside = p.split && n_groups <= POLY_RAW_MAX_GROUPS && p.blocks == 1 && skip1_jj && jj < sc->n_vars &&
-                           sc->n_vars - jj + 1 <= (u32)dpk::POLY_RES_ROUNDS && (n_groups == 1 || poly_split_state_ok(ctx, nf, has_eq, true));
-                return p;
-            };
-            // Launches the kernel of round jj.  `ahead`: round jj has not begun (its challenge is not known); the kernel
-            // waits for the mail of sequence number `seq_jj` and takes the challenge and the message's scalars from it.
-            auto launch_round = [&](u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj) -> int32_t {
-                dpk::PolyArgs pa;
-                pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
-                pa.terms = sc->d_poly_terms;
-                pa.ops = sc->d_poly_ops;
-                if (inline_descs) {
-                    pa.groups = nullptr;
-                    pa.terms = nullptr;
-                    pa.ops = nullptr;
-                    pa.g0 = sc->h_poly_groups[jj - 1];
-                    if (!p.split && !sc->h_poly_ops.empty())
-                        memcpy(pa.o0, sc->h_poly_ops.data(), sc->h_poly_ops.size() * sizeof(dpk::PolyOp));
-                    else
-                        std::copy(sc->h_poly_terms.begin(), sc->h_poly_terms.end(), pa.t0);
-                } else {
-                    CHK(ensure_descs(sc));
-                }
-                pa.q0 = pa.q1 = nullptr;
-                if (has_eq) {
-                    const u64 off = eq_level_off(sc->n_vars, jj);
-                    pa.q0 = sc->eq_c0 + off;
-                    pa.q1 = sc->eq_c1 + off;
-                }
-                pa.n_pairs = p.n_pairs;
-                pa.r0 = ahead ? 0 : a.r0;
-                pa.r1 = ahead ? 0 : a.r1;
-                pa.j = jj;
-                pa.last_round = 0;
-                pa.n_vars = sc->n_vars;
-                pa.spin_limit = 4000000;
-                pa.eq0 = sc->eq_c0;
-                pa.eq1 = sc->eq_c1;
-                pa.mail = ctx->d_pinned + (ctx->res_off - 64);
-                pa.seq = seq_jj;
-                pa.split_log = p.split_log;
-                pa.split_cap = sc->poly_split_cap;
-                pa.lds_state = pa.state_off = pa.pad = 0;
-                pa.finish = sc->poly_finish_in_kernel ? 1 : 0;
-                pa.group_stride = 1;
-                pa.raw_out = nullptr;
-                pa.wait_first = ahead ? 1 : 0;
-                if (ahead && !p.reside) pa.spin_limit = AHEAD_SPIN_LIMIT;
-                // (more workgroups than should poll the host's memory: the first one polls and passes the mail on)
-                pa.relay = ahead && p.blocks * n_groups > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
-                if (p.reside) {
-                    pa.last_round = sc->n_vars;
-                    if (n_groups > 1) {
-                        // one resident workgroup per group, each publishing its own sums
-                        CHK(ensure_descs(sc));
-                        pa.groups = sc->d_poly_groups + (size_t)(jj - 1) * n_groups;
-                        pa.group_stride = n_groups;
-                        pa.raw_out = ctx->d_pinned + poly_raw_off(ctx);
-                    } else if (inline_descs) {
-                        // the descriptors of the remaining rounds go through pinned memory: the kernel copies them to LDS
-                        // before anything else (and before it looks for mail); the area is not written again before a
-                        // message of this launch has arrived
-                        const size_t words = (size_t)(sc->n_vars - jj + 1) * sizeof(dpk::PolyGroup) / 8;
-                        memcpy(ctx->h_pinned, &sc->h_poly_groups[jj - 1], words * 8);
-                        pa.groups = reinterpret_cast<const dpk::PolyGroup *>(ctx->d_pinned);
-                    } else {
-                        pa.groups = sc->d_poly_groups + (size_t)(jj - 1);
-                    }
-                }
-                dpk::FastFin fl = ff;
-                fl.seq = seq_jj;
-                fl.n_blocks = p.blocks * n_groups;
-                fl.slots = !p.reside && slots_for(fl.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
-                double pbytes = has_eq ? (double)p.n_pairs * 16.0 : 0.0;
-                for (u32 k = 0; k < sc->n_mles; k++)
-                    if (sc->poly_owner[k] >= 0) pbytes += (double)p.n_pairs * (jj >= 2 ? 4 * 16.0 + 2 * 16.0 : 2 * 16.0);
-                ProfScope ps(ctx, DPS_K_EVAL_TERMS, pbytes);
-                if (p.split)
-                    CHK(launch_poly_split_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, p.reside, sc->d_partial, fl));
-                else
-                    CHK(launch_poly_dispatch(ctx, nf, has_eq, skip1_jj, pa, dim3(p.blocks, n_groups), sc->poly_max_tabs, sc->d_partial, fl));
-                HIPCHK(ctx, hipGetLastError());
-                return DPS_OK;
-            };
-            // a launch that takes this round may already be on the GPU, waiting for the mail: a resident one from an
-            // earlier round, or one made ahead during the previous round
-            const bool on_gpu = sc->tail_running;
-            // result areas the launch of this round publishes to, 0 = the main one
-            auto slots_of = [&](const Plan &p) { return p.reside ? (n_groups > 1 ? n_groups : 0) : slots_for(p.blocks * n_groups); };
-            bool stays;
-            u32 slots_now;
-            if (on_gpu) {
-                post_mail();
-                sc->wait_fresh = false;
-                stays = sc->wait_stays;
-                slots_now = sc->wait_slots;
-            } else {
-                const Plan p = plan_round(j, a.skip1 != 0);
-                CHK(launch_round(j, p, a.skip1 != 0, false, fa.seq));
-                stays = p.reside;
-                slots_now = slots_of(p);
-                if (p.reside) {
-                    sc->tail_running = true;
-                    sc->tail_seq0 = fa.seq;
-                    ctx->tail_owner = sc;
-                    sc->poly_raw = n_groups > 1;
-                    sc->wait_slots = slots_now;
-                    sc->wait_stays = true;
-                    sc->wait_skip1 = true;
-                    sc->wait_fresh = false;
-                }
-            }
-            if (!stays) {
-                // the launch of this round ends with it
-                sc->tail_running = false;
-                ctx->tail_owner = nullptr;
-                // The next round's launch is made now, behind this one: by the time this round's message has crossed to
-                // the host and the challenge is drawn, it is already on the GPU looking for its mail.  Only for rounds
-                // of few workgroups (every workgroup polls the mailbox), and not while launches are being timed.
-                if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
-                    // p(1) comes from the claim unless the scale vanishes at 1, i.e. unless the eq point is 0 there
-                    bool skip1_next = true;
-                    if (has_eq) {
-                        const E2 rho = sc->eq_info->point[j];
-                        skip1_next = !(rho.c0 == 0 && rho.c1 == 0);
-                    }
-                    const Plan pn = plan_round(j + 1, skip1_next);
-                    if (sc->tail_j0 && j + 1 == sc->tail_j0) {
-                        // the rounds from here on are resident: their launches are queued now and wait for their first mail
-                        CHK(launch_stages_at(ctx->seq + 1));
-                        sc->wait_fresh = true;
-                        sc->ahead_at = std::chrono::steady_clock::now();
-                    } else {
-                        CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
-                        sc->tail_running = true;
-                        sc->tail_seq0 = ctx->seq + 1;
-                        ctx->tail_owner = sc;
-                        sc->wait_stays = pn.reside;
-                        sc->wait_skip1 = skip1_next;
-                        sc->wait_fresh = true;
-                        sc->ahead_at = std::chrono::steady_clock::now();
-                        sc->poly_raw = pn.reside && n_groups > 1;
-                        sc->wait_slots = slots_of(pn);
-                    }
-                }
-            }
-            int32_t rc = take_sums(slots_now);
-            if (rc != DPS_OK) {
-                // a launch that left without publishing may have taken some of its tickets and written some of its tables
-                sc->broken = true;
-                reset_device_words(ctx);
-            }
-            if (stays && (rc != DPS_OK || j == sc->n_vars)) {
-                // a resident launch exits after the last round; one that can finish has published the tables' last pairs with it
-                sc->tail_running = false;
-                ctx->tail_owner = nullptr;
-                if (rc == DPS_OK && sc->poly_finish_in_kernel) sc->pairs_seq = fa.seq;
-            }
-            CHK(rc);
-            sc->round = j;
-            return DPS_OK;
-        }
-        u32 slots_now = sc->wait_slots;
-        if (sc->tail_running) {
-            // launched during the previous round
-            post_mail();
-            sc->wait_fresh = false;
-        } else {
-            slots_now = slots_for(blocks);
-            ff.slots = slots_now ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
-            // (in the factored form the eq weights are one entry per thread and one per workgroup and step: not counted)
-            double bytes = has_eq && !a.lq0 ? (double)n_pairs * 16.0 : 0.0;
-            for (u32 f = 0; f < nf; f++) {
-                double eb = a.s1[f] ? 16.0 : 8.0;
-                bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
-            }
-            ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
-            a.wait_first = 0;
-            CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j], has_eq, j >= 2, a, blocks, sc->d_partial, ff));
-            HIPCHK(ctx, hipGetLastError());
-        }
-        // this round's launch ends with the round
-        sc->tail_running = false;
-        ctx->tail_owner = nullptr;
-        // The next round's launch is made now, behind this one (see the fused multi-term path below... the same reasons):
-        // the tail kernel, or a product kernel of few workgroups, which then waits for its challenge by mail.
-        if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
-            const u64 next_seq = ctx->seq + 1;
-            bool made = false;
-            if (sc->tail_j0 && j + 1 == sc->tail_j0) {
-                CHK(launch_stages_at(next_seq));
-                made = true;
-            } else {
-                // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
-                // p(1) comes from the claim unless the scale vanishes at 1
-                bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
-                if (has_eq) {
-                    const E2 rho = sc->eq_info->point[j];
-                    skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
-                }
-                dpk::ProdArgs an = sc->fast_args[j + 1];
-                if (has_eq) set_eq_weights(an, j + 1, blocks_for_pairs(n_pairs >> 1));
-                an.r0 = an.r1 = 0;
-                an.skip1 = skip1_next ? 1 : 0;
-                an.wait_first = 1;
-                an.spin_limit = AHEAD_SPIN_LIMIT;
-                an.mail = ctx->d_pinned + (ctx->res_off - 64);
-                an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
-                dpk::FastFin fn = ff;
-                fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
-                fn.seq = next_seq;
-                fn.slots = slots_for(fn.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
-                sc->wait_slots = slots_for(fn.n_blocks);
-                CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j + 1], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
-                HIPCHK(ctx, hipGetLastError());
-                sc->wait_any_skip1 = false;
-                sc->wait_skip1 = skip1_next;
-                made = true;
-            }
-            if (made) {
-                sc->tail_running = true;
-                sc->wait_fresh = true;
-                sc->ahead_at = std::chrono::steady_clock::now();
-                ctx->tail_owner = sc;
-            }
-        }
-        if (const int32_t rc = take_sums(slots_now); rc != DPS_OK) {
-            sc->broken = true;
-            reset_device_words(ctx);
-            return rc;
-        }
-        if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
-        sc->round = j;
-        return DPS_OK;
+        FusedRound fr;
+        memset(static_cast<void *>(&fr), 0, sizeof fr);
+        fr.sc = sc, fr.ctx = ctx, fr.j = j, fr.challenge = challenge, fr.evals_out = evals_out;
+        fr.n_pairs = n_pairs, fr.blocks = blocks, fr.cst = cst, fr.fa = fa;
+        CHK(fr.begin());
+        if (sc->tail_j0 && j >= sc->tail_j0) return fr.resident_round();
+        return sc->poly ? fr.multi_term_round() : fr.product_round();
     } else {
         if (j >= 2) CHK(launch_folds(sc, j, false, challenge));
         for (u32 base = 0; base < sc->n_terms; base += 65535) {
