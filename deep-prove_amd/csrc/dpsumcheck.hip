@@ -1916,51 +1916,73 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
 
 }  // namespace
 
-extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
-                                const dps_term *terms, uint32_t n_terms, dps_sc **out)
-{
-    if (!ctx || !out || (n_mles && !mles) || (n_terms && !terms) || n_vars > 40)
-        return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: bad argument");
-    DeviceGuard g(ctx->device);
-    tail_abort(ctx);
-    std::unique_ptr<dps_sc> sc(new (std::nothrow) dps_sc());
-    if (!sc) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
-    sc->ctx = ctx;
-    sc->n_vars = n_vars;
-    sc->n_mles = n_mles;
-    sc->round = 0;
-    sc->finished = false;
-    sc->scratch = sc->dev_block = nullptr;
-    sc->const_sum = gl::e2_zero();
-    sc->degree = 0;
-    std::vector<u32> nv0(n_mles);
-    for (u32 k = 0; k < n_mles; k++) {
-        const dps_mle *t = mles[k];
-        if (!t || t->ctx != ctx) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u belongs to another context", k);
-        if (is_raw(t->kind) || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
-        nv0[k] = log2u(t->len);
-        if (nv0[k] > n_vars) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u has %u variables, the sum has %u", k, nv0[k], n_vars);
-        if (t->pad_vars && t->pad_vars != n_vars)
-            return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is zero-padded to %u variables, the sum has %u", k, t->pad_vars, n_vars);
-        sc->keep.push_back(t->st);
-    }
-    for (u32 i = 0; i < n_terms; i++) {
-        const dps_term &t = terms[i];
-        if (!canonical(t.coeff, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: coefficient of term %u not canonical", i);
-        if (t.n_factors > DPS_MAX_FACTORS) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u has %u factors", i, t.n_factors);
-        if (t.n_factors > DPS_MAX_DEGREE) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_sc_begin: degree %u above %d", t.n_factors, DPS_MAX_DEGREE);
-        for (u32 f = 0; f < t.n_factors; f++)
-            if (t.factors[f] >= n_mles) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u names table %u", i, t.factors[f]);
-        if (t.n_factors == 0) {
-            sc->const_sum = gl::add(sc->const_sum, gl::e2(t.coeff[0], t.coeff[1]));
-        } else {
-            sc->terms.push_back(t);
-            sc->degree = std::max(sc->degree, t.n_factors);
-        }
-    }
-    sc->n_terms = (u32)sc->terms.size();
+namespace {
 
-    // fast path test
+// What dps_sc_begin works out for a new session, step by step: which kernels can take it, which rounds are resident, where
+// every table lies in every round (the launches' descriptors), and the device block that holds descriptors, partials and
+// hand-over buffers.
+struct SessionSetup {
+    dps_ctx *ctx;
+    dps_sc *sc;
+    u32 n_vars;
+    const dps_mle *const *mles;
+    u32 n_mles;
+    std::vector<u32> nv0;  // variables of every table as registered
+    // sums of several terms: the closed-form eq factor (-1: none), the degree without it, the groups of tables and the terms of each
+    int eq = -1;
+    u32 nf = 0;
+    std::vector<std::vector<u32>> groups;
+    std::vector<u32> tb, te;
+    std::vector<dpk::PolyTerm> poly_terms;
+    // descriptors of every round, from a dry run of the folds
+    std::vector<dpk::FoldDesc> folds, folds_extra;
+    std::vector<dpk::TermDesc> tdescs;
+    std::vector<dpk::PolyGroup> poly_groups;  // [round][group]
+    std::vector<dpk::FinTerm> fins;
+    std::vector<dpk::GatherDesc> gath;
+    std::vector<SessMle> sim;  // the tables as the round being described finds them
+    std::vector<const u64 *> pre0, pre1;  // where a table folded in this step lay before
+    std::vector<char> folded;
+    size_t bytes_fold = 0, bytes_fold_x = 0, bytes_terms = 0, bytes_fin = 0, bytes_gath = 0, bytes_pg = 0, bytes_pt = 0, bytes_po = 0;
+
+    // a zero-padded table keeps folding after it is down to one entry: both of its buffers hold at least that entry
+    bool zpad_of(u32 k) const { return mles[k]->pad_vars != 0 && nv0[k] < n_vars; }
+    u64 len_a(u32 k) const { return nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : (zpad_of(k) ? 1ull : 0ull); }
+    u64 len_b(u32 k) const { return nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : (zpad_of(k) ? 1ull : 0ull); }
+    bool in_fast(u32 k) const;
+
+    void detect_product();
+    bool closed_form_eq_factor();
+    bool group_terms();
+    void adopt_groups();
+    void nested_programs();
+    void detect_multi_term();
+    int32_t plan_and_ready_tables();
+    int32_t layout_scratch();
+    void fold_step(u32 j);
+    void poly_groups_of_round(u32 j);
+    void term_descs_of_round(u32 j);
+    void describe_rounds();
+    void launch_limits();
+    int32_t allocate_device_block();
+    int32_t stage_descriptors();
+    int32_t run();
+};
+
+
+// tables the fused kernels fold themselves (the others fold in launches of their own)
+bool SessionSetup::in_fast(u32 k) const
+{
+        if (sc->poly) return sc->poly_owner[k] >= 0;
+        if (!sc->fast) return false;
+        for (u32 f = 0; f < sc->fast_nf; f++)
+            if (sc->fast_order[f] == k) return true;
+        return false;
+}
+
+// One product of 2 or 3 distinct full-size tables (one of them possibly an eq table, taken in closed form): prod_kernel.
+void SessionSetup::detect_product()
+{
     sc->fast = false;
     sc->broken = false;
     sc->tail_j0 = 0;
@@ -2004,150 +2026,173 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         }
     }
 
-    // fused multi-term path: every table of every term is either full-size or constant in the low variables
+}
+
+// Sums of several terms (every table full-size or constant in the low variables).  True: no table stands in the way.
+// An eq table that is a factor of every term exactly once comes out in closed form (`eq`).
+bool SessionSetup::closed_form_eq_factor()
+{
+    bool ok = true;
+    for (const dps_term &t : sc->terms)
+        for (u32 f = 0; f < t.n_factors; f++)
+            if (mles[t.factors[f]]->pad_vars && nv0[t.factors[f]] < n_vars) ok = false;
+    if (ok) {
+        const dps_term &t0 = sc->terms[0];
+        for (u32 f = 0; f < t0.n_factors && eq < 0; f++) {
+            const u32 k = t0.factors[f];
+            const dps_mle *h = mles[k];
+            if (!(h->eq && h->eq->m == n_vars && h->kind == DPS_EXT2 && nv0[k] == n_vars)) continue;
+            bool all = true;
+            u32 inner = 0;
+            for (const dps_term &t : sc->terms) {
+                u32 cnt = 0;
+                for (u32 q = 0; q < t.n_factors; q++) cnt += t.factors[q] == k;
+                if (cnt != 1) all = false;
+                inner = std::max(inner, t.n_factors - 1);
+            }
+            if (all && inner >= 1) eq = (int)k;
+        }
+    }
+    return ok;
+}
+
+// The terms in order, a new group whenever the tables no longer fit one (POLY_MAXT).  False: a term has too many tables.
+bool SessionSetup::group_terms()
+{
+    nf = 0;
+    for (const dps_term &t : sc->terms) nf = std::max(nf, eq >= 0 ? t.n_factors - 1 : t.n_factors);
+    bool ok = nf >= 1 && nf <= 6;
+    // terms in order, a new group whenever the tables no longer fit
+    if (ok) {
+        std::vector<u32> cur;
+        u32 begin = 0;
+        for (u32 ti = 0; ti < sc->n_terms && ok; ti++) {
+            const dps_term &t = sc->terms[ti];
+            std::vector<u32> need;
+            for (u32 f = 0; f < t.n_factors; f++) {
+                const u32 k = t.factors[f];
+                if ((int)k == eq) continue;
+                if (std::find(need.begin(), need.end(), k) == need.end()) need.push_back(k);
+            }
+            if (need.size() > (size_t)dpk::POLY_MAXT) {
+                ok = false;
+                break;
+            }
+            std::vector<u32> merged = cur;
+            for (u32 k : need)
+                if (std::find(merged.begin(), merged.end(), k) == merged.end()) merged.push_back(k);
+            if (merged.size() > (size_t)dpk::POLY_MAXT) {
+                groups.push_back(cur);
+                tb.push_back(begin);
+                te.push_back(ti);
+                begin = ti;
+                merged = need;
+            }
+            cur = merged;
+        }
+        if (ok) {
+            groups.push_back(cur);
+            tb.push_back(begin);
+            te.push_back(sc->n_terms);
+        }
+    }
+    return ok && groups.size() <= 65535;
+}
+
+// the session takes the groups: owners of the tables, the terms with their tables as slots of their group
+void SessionSetup::adopt_groups()
+{
+    sc->poly = true;
+    sc->poly_tabs = groups;
+    sc->poly_term_begin = tb;
+    sc->poly_term_end = te;
+    sc->poly_owner.assign(n_mles, -1);
+    for (size_t g = 0; g < groups.size(); g++) {
+        sc->poly_max_tabs = std::max<u32>(sc->poly_max_tabs, (u32)groups[g].size());
+        for (u32 k : groups[g])
+            if (sc->poly_owner[k] < 0) sc->poly_owner[k] = (int)g;
+    }
+    sc->fast_nf = nf;
+    sc->fast_coeff = gl::e2_one();
+    if (eq >= 0) {
+        sc->fast_eq = eq;
+        sc->eq_info = mles[eq]->eq;
+        sc->eq_c0 = mles[eq]->p0();
+        sc->eq_c1 = mles[eq]->p1();
+    }
+    for (size_t g = 0; g < groups.size(); g++)
+        for (u32 ti = tb[g]; ti < te[g]; ti++) {
+            const dps_term &t = sc->terms[ti];
+            dpk::PolyTerm pt;
+            memset(&pt, 0, sizeof pt);
+            pt.c0 = t.coeff[0];
+            pt.c1 = t.coeff[1];
+            pt.w = gl::mul_small(t.coeff[1], (u32)gl::W);
+            for (u32 f = 0; f < t.n_factors; f++) {
+                if ((int)t.factors[f] == eq) continue;
+                const auto &gt = groups[g];
+                pt.slot[pt.n_factors++] = (uint8_t)(std::find(gt.begin(), gt.end(), t.factors[f]) - gt.begin());
+            }
+            poly_terms.push_back(pt);
+        }
+}
+
+void SessionSetup::nested_programs()
+{
+    // the nested form, where it saves products and fits the kernel's staging area
+    sc->poly_op_begin.assign(groups.size(), 0);
+    sc->poly_op_end.assign(groups.size(), 0);
+    // (only the kernel of the rounds of more than 2^16 pairs runs it: a smaller sum has no use for it)
+    bool use_ops = n_vars >= 1 && (1ull << (n_vars - 1)) > POLY_SPLIT_MAX_PAIRS;
+    std::vector<dpk::PolyOp> all_ops;
+    u32 plain = 0, nested = 0;
+    for (size_t g = 0; g < groups.size() && use_ops; g++) {
+        std::vector<HornerTerm> ts;
+        E2 root = gl::e2_zero();
+        for (u32 ti = tb[g]; ti < te[g]; ti++) {
+            const dpk::PolyTerm &pt = poly_terms[ti];
+            HornerTerm ht;
+            ht.coeff = gl::e2(pt.c0, pt.c1);
+            ht.slots.assign(pt.slot, pt.slot + pt.n_factors);
+            if (ht.slots.empty()) root = gl::add(root, ht.coeff);
+            plain += pt.n_factors;  // n_factors - 1 products and one for the coefficient
+            ts.push_back(std::move(ht));
+        }
+        std::vector<dpk::PolyOp> ops;
+        dpk::PolyOp enter;
+        memset(&enter, 0, sizeof enter);
+        enter.c0 = root.c0;
+        enter.c1 = root.c1;
+        enter.code = dpk::POLY_OP_ENTER;
+        ops.push_back(enter);
+        nested += horner_build(std::move(ts), 0, ops);
+        if (ops.size() > (size_t)dpk::POLY_LDS_OPS) use_ops = false;
+        sc->poly_op_begin[g] = (u32)all_ops.size();
+        all_ops.insert(all_ops.end(), ops.begin(), ops.end());
+        sc->poly_op_end[g] = (u32)all_ops.size();
+    }
+    if (use_ops && nested < plain) {
+        sc->h_poly_ops = all_ops;
+    } else {
+        sc->poly_op_begin.assign(groups.size(), 0);
+        sc->poly_op_end.assign(groups.size(), 0);
+    }
+}
+
+void SessionSetup::detect_multi_term()
+{
     sc->poly = false;
     sc->poly_max_tabs = 0;
     sc->d_poly_groups = nullptr;
     sc->d_poly_terms = nullptr;
-    std::vector<dpk::PolyTerm> poly_terms;
-    if (!sc->fast && sc->n_terms >= 1 && n_vars >= 1) {
-        bool ok = true;
-        for (const dps_term &t : sc->terms)
-            for (u32 f = 0; f < t.n_factors; f++)
-                if (mles[t.factors[f]]->pad_vars && nv0[t.factors[f]] < n_vars) ok = false;
-        // an eq table that is a factor of every term exactly once comes out in closed form
-        int eq = -1;
-        if (ok) {
-            const dps_term &t0 = sc->terms[0];
-            for (u32 f = 0; f < t0.n_factors && eq < 0; f++) {
-                const u32 k = t0.factors[f];
-                const dps_mle *h = mles[k];
-                if (!(h->eq && h->eq->m == n_vars && h->kind == DPS_EXT2 && nv0[k] == n_vars)) continue;
-                bool all = true;
-                u32 inner = 0;
-                for (const dps_term &t : sc->terms) {
-                    u32 cnt = 0;
-                    for (u32 q = 0; q < t.n_factors; q++) cnt += t.factors[q] == k;
-                    if (cnt != 1) all = false;
-                    inner = std::max(inner, t.n_factors - 1);
-                }
-                if (all && inner >= 1) eq = (int)k;
-            }
-        }
-        u32 nf = 0;
-        for (const dps_term &t : sc->terms) nf = std::max(nf, eq >= 0 ? t.n_factors - 1 : t.n_factors);
-        if (nf < 1 || nf > 6) ok = false;
-        // terms in order, a new group whenever the tables no longer fit
-        std::vector<std::vector<u32>> groups;
-        std::vector<u32> tb, te;
-        if (ok) {
-            std::vector<u32> cur;
-            u32 begin = 0;
-            for (u32 ti = 0; ti < sc->n_terms && ok; ti++) {
-                const dps_term &t = sc->terms[ti];
-                std::vector<u32> need;
-                for (u32 f = 0; f < t.n_factors; f++) {
-                    const u32 k = t.factors[f];
-                    if ((int)k == eq) continue;
-                    if (std::find(need.begin(), need.end(), k) == need.end()) need.push_back(k);
-                }
-                if (need.size() > (size_t)dpk::POLY_MAXT) {
-                    ok = false;
-                    break;
-                }
-                std::vector<u32> merged = cur;
-                for (u32 k : need)
-                    if (std::find(merged.begin(), merged.end(), k) == merged.end()) merged.push_back(k);
-                if (merged.size() > (size_t)dpk::POLY_MAXT) {
-                    groups.push_back(cur);
-                    tb.push_back(begin);
-                    te.push_back(ti);
-                    begin = ti;
-                    merged = need;
-                }
-                cur = merged;
-            }
-            if (ok) {
-                groups.push_back(cur);
-                tb.push_back(begin);
-                te.push_back(sc->n_terms);
-            }
-        }
-        if (ok && groups.size() <= 65535) {
-            sc->poly = true;
-            sc->poly_tabs = groups;
-            sc->poly_term_begin = tb;
-            sc->poly_term_end = te;
-            sc->poly_owner.assign(n_mles, -1);
-            for (size_t g = 0; g < groups.size(); g++) {
-                sc->poly_max_tabs = std::max<u32>(sc->poly_max_tabs, (u32)groups[g].size());
-                for (u32 k : groups[g])
-                    if (sc->poly_owner[k] < 0) sc->poly_owner[k] = (int)g;
-            }
-            sc->fast_nf = nf;
-            sc->fast_coeff = gl::e2_one();
-            if (eq >= 0) {
-                sc->fast_eq = eq;
-                sc->eq_info = mles[eq]->eq;
-                sc->eq_c0 = mles[eq]->p0();
-                sc->eq_c1 = mles[eq]->p1();
-            }
-            for (size_t g = 0; g < groups.size(); g++)
-                for (u32 ti = tb[g]; ti < te[g]; ti++) {
-                    const dps_term &t = sc->terms[ti];
-                    dpk::PolyTerm pt;
-                    memset(&pt, 0, sizeof pt);
-                    pt.c0 = t.coeff[0];
-                    pt.c1 = t.coeff[1];
-                    pt.w = gl::mul_small(t.coeff[1], (u32)gl::W);
-                    for (u32 f = 0; f < t.n_factors; f++) {
-                        if ((int)t.factors[f] == eq) continue;
-                        const auto &gt = groups[g];
-                        pt.slot[pt.n_factors++] = (uint8_t)(std::find(gt.begin(), gt.end(), t.factors[f]) - gt.begin());
-                    }
-                    poly_terms.push_back(pt);
-                }
-            // the nested form, where it saves products and fits the kernel's staging area
-            sc->poly_op_begin.assign(groups.size(), 0);
-            sc->poly_op_end.assign(groups.size(), 0);
-            // (only the kernel of the rounds of more than 2^16 pairs runs it: a smaller sum has no use for it)
-            bool use_ops = n_vars >= 1 && (1ull << (n_vars - 1)) > POLY_SPLIT_MAX_PAIRS;
-            std::vector<dpk::PolyOp> all_ops;
-            u32 plain = 0, nested = 0;
-            for (size_t g = 0; g < groups.size() && use_ops; g++) {
-                std::vector<HornerTerm> ts;
-                E2 root = gl::e2_zero();
-                for (u32 ti = tb[g]; ti < te[g]; ti++) {
-                    const dpk::PolyTerm &pt = poly_terms[ti];
-                    HornerTerm ht;
-                    ht.coeff = gl::e2(pt.c0, pt.c1);
-                    ht.slots.assign(pt.slot, pt.slot + pt.n_factors);
-                    if (ht.slots.empty()) root = gl::add(root, ht.coeff);
-                    plain += pt.n_factors;  // n_factors - 1 products and one for the coefficient
-                    ts.push_back(std::move(ht));
-                }
-                std::vector<dpk::PolyOp> ops;
-                dpk::PolyOp enter;
-                memset(&enter, 0, sizeof enter);
-                enter.c0 = root.c0;
-                enter.c1 = root.c1;
-                enter.code = dpk::POLY_OP_ENTER;
-                ops.push_back(enter);
-                nested += horner_build(std::move(ts), 0, ops);
-                if (ops.size() > (size_t)dpk::POLY_LDS_OPS) use_ops = false;
-                sc->poly_op_begin[g] = (u32)all_ops.size();
-                all_ops.insert(all_ops.end(), ops.begin(), ops.end());
-                sc->poly_op_end[g] = (u32)all_ops.size();
-            }
-            if (use_ops && nested < plain) {
-                sc->h_poly_ops = all_ops;
-            } else {
-                sc->poly_op_begin.assign(groups.size(), 0);
-                sc->poly_op_end.assign(groups.size(), 0);
-            }
-        }
-    }
+    if (sc->fast || sc->n_terms < 1 || n_vars < 1) return;
+    if (!closed_form_eq_factor() || !group_terms()) return;
+    adopt_groups();
+    nested_programs();
+}
 
+int32_t SessionSetup::plan_and_ready_tables()
+{
     // the last rounds run in one resident workgroup when every registered table belongs to the term
     // (from the round of 2^8 = TAIL_PAIRS pairs on, or from round 2 in a smaller sum; the tail kernel reads extension
     // tables, which every table is once folded, so a start in round 2 needs extension tables to begin with)
@@ -2159,12 +2204,12 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
     sc->prev_chal = gl::e2_zero();
-    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) plan_resident_rounds(sc.get(), sc->fast_nf);
+    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) plan_resident_rounds(sc, sc->fast_nf);
     // a sum of several terms over one group of full-size tables (a fraction-sum layer, a claim merge): the same launches
     if (sc->poly && sc->poly_tabs.size() == 1 && sc->fast_nf <= 4 && sc->n_terms <= (u32)dpk::SL_MAX_TERMS) {
         bool ok = n_mles == sc->poly_tabs[0].size() + (sc->fast_eq >= 0 ? 1 : 0);
         for (u32 k : sc->poly_tabs[0]) ok = ok && nv0[k] == n_vars && !mles[k]->pad_vars;
-        if (ok) plan_resident_rounds(sc.get(), (u32)sc->poly_tabs[0].size());
+        if (ok) plan_resident_rounds(sc, (u32)sc->poly_tabs[0].size());
     }
     // What this session reads of its tables: an eq table taken in closed form is read level by level -- level j in round j,
     // except in the large rounds of a product, which take the low table of level j and level j + 16 instead -- and
@@ -2183,13 +2228,15 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         }
     }
 
+    return DPS_OK;
+}
+
+int32_t SessionSetup::layout_scratch()
+{
     // scratch: two ping-pong buffers per table, extension limbs
     size_t scratch_words = 0;
     std::vector<size_t> off_a(n_mles), off_b(n_mles);
     // a zero-padded table keeps folding after it is down to one entry: both buffers hold at least that entry
-    auto zpad_of = [&](u32 k) { return mles[k]->pad_vars != 0 && nv0[k] < n_vars; };
-    auto len_a = [&](u32 k) { return nv0[k] >= 1 ? (1ull << (nv0[k] - 1)) : (zpad_of(k) ? 1ull : 0ull); };
-    auto len_b = [&](u32 k) { return nv0[k] >= 2 ? (1ull << (nv0[k] - 2)) : (zpad_of(k) ? 1ull : 0ull); };
     for (u32 k = 0; k < n_mles; k++) {
         u64 la = len_a(k), lb = len_b(k);
         off_a[k] = scratch_words;
@@ -2198,11 +2245,6 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         scratch_words += round_up(2 * lb, 32);
     }
     if (scratch_words) CHK(pool_alloc(ctx, scratch_words * 8, &sc->scratch));
-    auto cleanup = [&](int32_t rc) {
-        pool_free(ctx, sc->scratch);
-        pool_free(ctx, sc->dev_block);
-        return rc;
-    };
     u64 *sbase = (u64 *)sc->scratch;
     sc->m.resize(n_mles);
     for (u32 k = 0; k < n_mles; k++) {
@@ -2219,80 +2261,19 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         s.next = 0;
     }
 
-    // simulate the rounds to precompute every descriptor
-    std::vector<dpk::FoldDesc> folds, folds_extra;
-    std::vector<dpk::TermDesc> tdescs;
-    std::vector<SessMle> sim = sc->m;
-    auto in_fast = [&](u32 k) {
-        if (sc->poly) return sc->poly_owner[k] >= 0;
-        if (!sc->fast) return false;
-        for (u32 f = 0; f < sc->fast_nf; f++)
-            if (sc->fast_order[f] == k) return true;
-        return false;
-    };
-    sc->fold_off.assign(n_vars + 2, 0);
-    sc->fold_cnt.assign(n_vars + 2, 0);
-    sc->fold_extra_off.assign(n_vars + 2, 0);
-    sc->fold_extra_cnt.assign(n_vars + 2, 0);
-    sc->term_off.assign(n_vars + 2, 0);
-    sc->fast_args.resize(n_vars + 2);
-    sc->fast_nb.assign(n_vars + 2, 0);
-    std::vector<dpk::PolyGroup> poly_groups;  // [round][group]
-    std::vector<const u64 *> pre0(n_mles), pre1(n_mles);
-    std::vector<char> folded(n_mles);
-    for (u32 j = 1; j <= n_vars + 1; j++) {
-        std::fill(folded.begin(), folded.end(), 0);
-        // step j starts by folding, with the challenge of round j-1, the tables that were live-sized then
-        if (j >= 2) {
-            u32 prev_live = n_vars - (j - 1) + 1;
-            sc->fold_off[j] = (u32)folds.size();
-            sc->fold_extra_off[j] = (u32)folds_extra.size();
-            if (sc->fast && j <= n_vars) {
-                dpk::ProdArgs &pa = sc->fast_args[j];
-                memset(&pa, 0, sizeof pa);
-                u32 nb = 0;
-                for (u32 f = 0; f < sc->fast_nf; f++) {
-                    const SessMle &s = sim[sc->fast_order[f]];
-                    pa.s0[f] = s.c0;
-                    pa.s1[f] = s.c1;
-                    if (!s.c1) nb++;
-                    pa.d0[f] = s.buf0[s.next];
-                    pa.d1[f] = s.buf1[s.next];
-                }
-                pa.n_pairs = 1ull << (n_vars - j);
-                sc->fast_nb[j] = nb;
-            }
-            for (u32 k = 0; k < n_mles; k++) {
-                SessMle &s = sim[k];
-                if ((int)k == sc->fast_eq) continue;
-                if (s.zpad) {
-                    // depends on the low variables: folds in every step, and keeps folding against 0 once it is one entry
-                    const bool single = s.nv == 0;
-                    dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], single ? 1ull : 1ull << (s.nv - 1), single ? 1ull : 0ull};
-                    folds.push_back(d);
-                    folds_extra.push_back(d);
-                    s.c0 = d.d0;
-                    s.c1 = d.d1;
-                    if (!single) s.nv -= 1;
-                    s.next ^= 1;
-                    continue;
-                }
-                if (s.nv != prev_live) continue;
-                dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1), 0};
-                folds.push_back(d);
-                if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
-                pre0[k] = s.c0;
-                pre1[k] = s.c1;
-                folded[k] = 1;
-                s.c0 = d.d0;
-                s.c1 = d.d1;
-                s.nv -= 1;
-                s.next ^= 1;
-            }
-            sc->fold_cnt[j] = (u32)folds.size() - sc->fold_off[j];
-            sc->fold_extra_cnt[j] = (u32)folds_extra.size() - sc->fold_extra_off[j];
-        } else if (sc->fast) {
-            dpk::ProdArgs &pa = sc->fast_args[1];
+    return DPS_OK;
+}
+
+// Step j starts by folding, with the challenge of round j - 1, the tables that were live-sized then; the product
+// kernel's arguments of round j.
+void SessionSetup::fold_step(u32 j)
+{
+    if (j >= 2) {
+        u32 prev_live = n_vars - (j - 1) + 1;
+        sc->fold_off[j] = (u32)folds.size();
+        sc->fold_extra_off[j] = (u32)folds_extra.size();
+        if (sc->fast && j <= n_vars) {
+            dpk::ProdArgs &pa = sc->fast_args[j];
             memset(&pa, 0, sizeof pa);
             u32 nb = 0;
             for (u32 f = 0; f < sc->fast_nf; f++) {
@@ -2300,81 +2281,153 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
                 pa.s0[f] = s.c0;
                 pa.s1[f] = s.c1;
                 if (!s.c1) nb++;
+                pa.d0[f] = s.buf0[s.next];
+                pa.d1[f] = s.buf1[s.next];
             }
-            pa.n_pairs = 1ull << (n_vars - 1);
-            sc->fast_nb[1] = nb;
+            pa.n_pairs = 1ull << (n_vars - j);
+            sc->fast_nb[j] = nb;
         }
-        if (j <= n_vars && sc->poly) {
-            const u32 live = n_vars - j + 1;
-            for (size_t g = 0; g < sc->poly_tabs.size(); g++) {
-                dpk::PolyGroup pg;
-                memset(&pg, 0, sizeof pg);
-                pg.n_tabs = (u32)sc->poly_tabs[g].size();
-                pg.term_begin = sc->poly_term_begin[g];
-                pg.term_end = sc->poly_term_end[g];
-                pg.op_begin = sc->poly_op_begin[g];
-                pg.op_end = sc->poly_op_end[g];
-                for (u32 sl = 0; sl < pg.n_tabs; sl++) {
-                    const u32 k = sc->poly_tabs[g][sl];
-                    const SessMle &s = sim[k];
-                    dpk::PolyTab &tb = pg.tab[sl];
-                    if (folded[k]) {
-                        // folds with the previous challenge on the way in; the owning group writes the result
-                        tb.mode = dpk::POLY_PAIR_FOLD;
-                        tb.s0 = pre0[k];
-                        tb.s1 = pre1[k];
-                        if (sc->poly_owner[k] == (int)g) {
-                            tb.d0 = const_cast<u64 *>(s.c0);
-                            tb.d1 = const_cast<u64 *>(s.c1);
-                        }
-                    } else if (s.nv >= live) {
-                        tb.mode = dpk::POLY_PAIR;
-                        tb.s0 = s.c0;
-                        tb.s1 = s.c1;
-                    } else {
-                        tb.mode = dpk::POLY_BCAST;
-                        tb.s0 = s.c0;
-                        tb.s1 = s.c1;
-                        tb.shift = live - 1 - s.nv;
-                    }
-                }
-                poly_groups.push_back(pg);
+        for (u32 k = 0; k < n_mles; k++) {
+            SessMle &s = sim[k];
+            if ((int)k == sc->fast_eq) continue;
+            if (s.zpad) {
+                // depends on the low variables: folds in every step, and keeps folding against 0 once it is one entry
+                const bool single = s.nv == 0;
+                dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], single ? 1ull : 1ull << (s.nv - 1), single ? 1ull : 0ull};
+                folds.push_back(d);
+                folds_extra.push_back(d);
+                s.c0 = d.d0;
+                s.c1 = d.d1;
+                if (!single) s.nv -= 1;
+                s.next ^= 1;
+                continue;
             }
+            if (s.nv != prev_live) continue;
+            dpk::FoldDesc d{s.c0, s.c1, s.buf0[s.next], s.buf1[s.next], 1ull << (s.nv - 1), 0};
+            folds.push_back(d);
+            if (!in_fast(k) || j == n_vars + 1) folds_extra.push_back(d);
+            pre0[k] = s.c0;
+            pre1[k] = s.c1;
+            folded[k] = 1;
+            s.c0 = d.d0;
+            s.c1 = d.d1;
+            s.nv -= 1;
+            s.next ^= 1;
         }
-        if (j <= n_vars && !sc->fast && !sc->poly) {
-            u32 live = n_vars - j + 1;
-            sc->term_off[j] = (u32)tdescs.size();
-            for (const dps_term &t : sc->terms) {
-                dpk::TermDesc td;
-                memset(&td, 0, sizeof td);
-                td.n_factors = t.n_factors;
-                td.n_pairs = 1ull << (live - 1);
-                for (u32 f = 0; f < t.n_factors; f++) {
-                    const SessMle &s = sim[t.factors[f]];
-                    td.f[f].c0 = s.c0;
-                    td.f[f].c1 = s.c1;
-                    if (s.zpad) {
-                        // non-zero only where the higher variables are 0: the first 2^(nv-1) pairs, or entry 0 against 0
-                        td.f[f].pair = s.nv >= 1 ? 1 : 2;
-                        td.f[f].shift = 0;
-                        td.n_pairs = std::min<u64>(td.n_pairs, s.nv >= 1 ? 1ull << (s.nv - 1) : 1ull);
-                    } else if (s.nv >= live) {
-                        td.f[f].pair = 1;
-                        td.f[f].shift = 0;
-                    } else {
-                        td.f[f].pair = 0;
-                        td.f[f].shift = live - 1 - s.nv;
-                    }
-                }
-                tdescs.push_back(td);
-            }
+        sc->fold_cnt[j] = (u32)folds.size() - sc->fold_off[j];
+        sc->fold_extra_cnt[j] = (u32)folds_extra.size() - sc->fold_extra_off[j];
+    } else if (sc->fast) {
+        dpk::ProdArgs &pa = sc->fast_args[1];
+        memset(&pa, 0, sizeof pa);
+        u32 nb = 0;
+        for (u32 f = 0; f < sc->fast_nf; f++) {
+            const SessMle &s = sim[sc->fast_order[f]];
+            pa.s0[f] = s.c0;
+            pa.s1[f] = s.c1;
+            if (!s.c1) nb++;
         }
+        pa.n_pairs = 1ull << (n_vars - 1);
+        sc->fast_nb[1] = nb;
     }
-    std::vector<dpk::FinTerm> fins;
-    for (const dps_term &t : sc->terms) fins.push_back(dpk::FinTerm{t.coeff[0], t.coeff[1], t.n_factors, 0});
-    std::vector<dpk::GatherDesc> gath;
-    for (u32 k = 0; k < n_mles; k++) gath.push_back(dpk::GatherDesc{sim[k].c0, sim[k].c1});
+}
 
+void SessionSetup::poly_groups_of_round(u32 j)
+{
+    const u32 live = n_vars - j + 1;
+    for (size_t g = 0; g < sc->poly_tabs.size(); g++) {
+        dpk::PolyGroup pg;
+        memset(&pg, 0, sizeof pg);
+        pg.n_tabs = (u32)sc->poly_tabs[g].size();
+        pg.term_begin = sc->poly_term_begin[g];
+        pg.term_end = sc->poly_term_end[g];
+        pg.op_begin = sc->poly_op_begin[g];
+        pg.op_end = sc->poly_op_end[g];
+        for (u32 sl = 0; sl < pg.n_tabs; sl++) {
+            const u32 k = sc->poly_tabs[g][sl];
+            const SessMle &s = sim[k];
+            dpk::PolyTab &tb = pg.tab[sl];
+            if (folded[k]) {
+                // folds with the previous challenge on the way in; the owning group writes the result
+                tb.mode = dpk::POLY_PAIR_FOLD;
+                tb.s0 = pre0[k];
+                tb.s1 = pre1[k];
+                if (sc->poly_owner[k] == (int)g) {
+                    tb.d0 = const_cast<u64 *>(s.c0);
+                    tb.d1 = const_cast<u64 *>(s.c1);
+                }
+            } else if (s.nv >= live) {
+                tb.mode = dpk::POLY_PAIR;
+                tb.s0 = s.c0;
+                tb.s1 = s.c1;
+            } else {
+                tb.mode = dpk::POLY_BCAST;
+                tb.s0 = s.c0;
+                tb.s1 = s.c1;
+                tb.shift = live - 1 - s.nv;
+            }
+        }
+        poly_groups.push_back(pg);
+    }
+}
+
+void SessionSetup::term_descs_of_round(u32 j)
+{
+    u32 live = n_vars - j + 1;
+    sc->term_off[j] = (u32)tdescs.size();
+    for (const dps_term &t : sc->terms) {
+        dpk::TermDesc td;
+        memset(&td, 0, sizeof td);
+        td.n_factors = t.n_factors;
+        td.n_pairs = 1ull << (live - 1);
+        for (u32 f = 0; f < t.n_factors; f++) {
+            const SessMle &s = sim[t.factors[f]];
+            td.f[f].c0 = s.c0;
+            td.f[f].c1 = s.c1;
+            if (s.zpad) {
+                // non-zero only where the higher variables are 0: the first 2^(nv-1) pairs, or entry 0 against 0
+                td.f[f].pair = s.nv >= 1 ? 1 : 2;
+                td.f[f].shift = 0;
+                td.n_pairs = std::min<u64>(td.n_pairs, s.nv >= 1 ? 1ull << (s.nv - 1) : 1ull);
+            } else if (s.nv >= live) {
+                td.f[f].pair = 1;
+                td.f[f].shift = 0;
+            } else {
+                td.f[f].pair = 0;
+                td.f[f].shift = live - 1 - s.nv;
+            }
+        }
+        tdescs.push_back(td);
+    }
+}
+
+// a dry run of the rounds: every descriptor the launches will need
+void SessionSetup::describe_rounds()
+{
+    sim = sc->m;
+    sc->fold_off.assign(n_vars + 2, 0);
+    sc->fold_cnt.assign(n_vars + 2, 0);
+    sc->fold_extra_off.assign(n_vars + 2, 0);
+    sc->fold_extra_cnt.assign(n_vars + 2, 0);
+    sc->term_off.assign(n_vars + 2, 0);
+    sc->fast_args.resize(n_vars + 2);
+    sc->fast_nb.assign(n_vars + 2, 0);
+    pre0.assign(n_mles, nullptr), pre1.assign(n_mles, nullptr);
+    folded.assign(n_mles, 0);
+    for (u32 j = 1; j <= n_vars + 1; j++) {
+        std::fill(folded.begin(), folded.end(), 0);
+        fold_step(j);
+        if (j <= n_vars && sc->poly) poly_groups_of_round(j);
+        if (j <= n_vars && !sc->fast && !sc->poly) term_descs_of_round(j);
+    }
+
+    for (const dps_term &t : sc->terms) fins.push_back(dpk::FinTerm{t.coeff[0], t.coeff[1], t.n_factors, 0});
+
+    for (u32 k = 0; k < n_mles; k++) gath.push_back(dpk::GatherDesc{sim[k].c0, sim[k].c1});
+}
+
+// grid sizes the session can ask for (its partials are sized for the largest), and how a pair's work is spread in small rounds
+void SessionSetup::launch_limits()
+{
     sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
     sc->poly_split_cap = 0;
     sc->poly_finish_in_kernel = false;
@@ -2397,23 +2450,26 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
             sc->max_blocks = std::max(sc->max_blocks, bl);
         }
     }
-    size_t bytes_fold = round_up(folds.size() * sizeof(dpk::FoldDesc), 256);
-    size_t bytes_fold_x = round_up(folds_extra.size() * sizeof(dpk::FoldDesc), 256);
-    size_t bytes_terms = round_up(tdescs.size() * sizeof(dpk::TermDesc), 256);
-    size_t bytes_fin = round_up(fins.size() * sizeof(dpk::FinTerm), 256);
-    size_t bytes_gath = round_up(gath.size() * sizeof(dpk::GatherDesc), 256);
+}
+
+int32_t SessionSetup::allocate_device_block()
+{
+    bytes_fold = round_up(folds.size() * sizeof(dpk::FoldDesc), 256);
+    bytes_fold_x = round_up(folds_extra.size() * sizeof(dpk::FoldDesc), 256);
+    bytes_terms = round_up(tdescs.size() * sizeof(dpk::TermDesc), 256);
+    bytes_fin = round_up(fins.size() * sizeof(dpk::FinTerm), 256);
+    bytes_gath = round_up(gath.size() * sizeof(dpk::GatherDesc), 256);
     size_t bytes_partial = round_up((size_t)std::max<u32>(sc->n_terms, 1) * sc->max_blocks * 2 * dpk::MAX_PTS * 8, 256);
     size_t bytes_result = round_up((2 * dpk::MAX_PTS + 2 * (size_t)n_mles) * 8, 256) + 256;
-    size_t bytes_pg = round_up(poly_groups.size() * sizeof(dpk::PolyGroup), 256);
-    size_t bytes_pt = round_up(poly_terms.size() * sizeof(dpk::PolyTerm), 256);
-    size_t bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
+    bytes_pg = round_up(poly_groups.size() * sizeof(dpk::PolyGroup), 256);
+    bytes_pt = round_up(poly_terms.size() * sizeof(dpk::PolyTerm), 256);
+    bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
     // what a resident stage that does not run to the last round leaves for the next: two limb arrays per table
     size_t bytes_hand = 0;
     const u32 slice_tabs = sc->poly ? (sc->poly_tabs.empty() ? 0u : (u32)sc->poly_tabs[0].size()) : sc->fast_nf;
     for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * slice_tabs;
     size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result + bytes_hand;
-    int32_t rc = pool_alloc(ctx, total, &sc->dev_block);
-    if (rc != DPS_OK) return cleanup(rc);
+    CHK(pool_alloc(ctx, total, &sc->dev_block));
     char *p = (char *)sc->dev_block;
     sc->d_fold = (dpk::FoldDesc *)p;
     p += bytes_fold;
@@ -2445,6 +2501,11 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
         }
     }
     sc->d_counter = ctx->d_counter;
+    return DPS_OK;
+}
+
+int32_t SessionSetup::stage_descriptors()
+{
     // one staged upload of all descriptors
     std::vector<char> &stage = sc->stage;  // lives as long as the session: the upload is not waited for
     stage.assign(bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po, 0);
@@ -2473,8 +2534,76 @@ extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *co
     const bool self_contained = (sc->fast && sc->tail_j0) ||
                                 (sc->poly && sc->poly_tabs.size() == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS);
     if (!self_contained) {
-        rc = ensure_descs(sc.get());
-        if (rc != DPS_OK) return cleanup(rc);
+        CHK(ensure_descs(sc));
+    }
+    return DPS_OK;
+}
+
+int32_t SessionSetup::run()
+{
+    detect_product();
+    detect_multi_term();
+    CHK(plan_and_ready_tables());
+    CHK(layout_scratch());
+    describe_rounds();
+    launch_limits();
+    CHK(allocate_device_block());
+    return stage_descriptors();
+}
+
+}  // namespace
+
+extern "C" int32_t dps_sc_begin(dps_ctx *ctx, uint32_t n_vars, const dps_mle *const *mles, uint32_t n_mles,
+                                const dps_term *terms, uint32_t n_terms, dps_sc **out)
+{
+    if (!ctx || !out || (n_mles && !mles) || (n_terms && !terms) || n_vars > 40)
+        return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: bad argument");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    std::unique_ptr<dps_sc> sc(new (std::nothrow) dps_sc());
+    if (!sc) return fail(ctx, DPS_ERR_OOM, "host allocation failed");
+    sc->ctx = ctx;
+    sc->n_vars = n_vars;
+    sc->n_mles = n_mles;
+    sc->round = 0;
+    sc->finished = false;
+    sc->scratch = sc->dev_block = nullptr;
+    sc->const_sum = gl::e2_zero();
+    sc->degree = 0;
+    SessionSetup su;
+    su.ctx = ctx, su.sc = sc.get(), su.n_vars = n_vars, su.mles = mles, su.n_mles = n_mles;
+    std::vector<u32> &nv0 = su.nv0;
+    nv0.assign(n_mles, 0);
+    for (u32 k = 0; k < n_mles; k++) {
+        const dps_mle *t = mles[k];
+        if (!t || t->ctx != ctx) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u belongs to another context", k);
+        if (is_raw(t->kind) || !is_pow2(t->len)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is not a power-of-two field table", k);
+        nv0[k] = log2u(t->len);
+        if (nv0[k] > n_vars) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u has %u variables, the sum has %u", k, nv0[k], n_vars);
+        if (t->pad_vars && t->pad_vars != n_vars)
+            return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: table %u is zero-padded to %u variables, the sum has %u", k, t->pad_vars, n_vars);
+        sc->keep.push_back(t->st);
+    }
+    for (u32 i = 0; i < n_terms; i++) {
+        const dps_term &t = terms[i];
+        if (!canonical(t.coeff, 2)) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: coefficient of term %u not canonical", i);
+        if (t.n_factors > DPS_MAX_FACTORS) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u has %u factors", i, t.n_factors);
+        if (t.n_factors > DPS_MAX_DEGREE) return fail(ctx, DPS_ERR_UNSUPPORTED, "dps_sc_begin: degree %u above %d", t.n_factors, DPS_MAX_DEGREE);
+        for (u32 f = 0; f < t.n_factors; f++)
+            if (t.factors[f] >= n_mles) return fail(ctx, DPS_ERR_INVALID, "dps_sc_begin: term %u names table %u", i, t.factors[f]);
+        if (t.n_factors == 0) {
+            sc->const_sum = gl::add(sc->const_sum, gl::e2(t.coeff[0], t.coeff[1]));
+        } else {
+            sc->terms.push_back(t);
+            sc->degree = std::max(sc->degree, t.n_factors);
+        }
+    }
+    sc->n_terms = (u32)sc->terms.size();
+
+    if (const int32_t rc = su.run(); rc != DPS_OK) {
+        pool_free(ctx, sc->scratch);
+        pool_free(ctx, sc->dev_block);
+        return rc;
     }
     *out = sc.release();
     return DPS_OK;
