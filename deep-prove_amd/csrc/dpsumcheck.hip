@@ -70,6 +70,7 @@ struct dps_ctx {
     u64 *h_pinned = nullptr;    // host-visible result buffer
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
+    double wall_clock_scale = 1.0;  // rate of the device's real-time counter / 100 MHz
     hipEvent_t stage_event = nullptr;  // recorded after a launch that reads the staging region of the pinned buffer
     bool stage_pending = false;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
@@ -196,6 +197,10 @@ void pool_free(dps_ctx *ctx, void *p)
     ctx->free_blocks.emplace(it->second, p);
     ctx->live_blocks.erase(it);
 }
+
+// A kernel's patience, as the kernels count it: units of 256 ticks of the device's real-time counter.  `units`: the figure at
+// 100 MHz (2.56 us a unit); scaled by the counter's actual rate.
+u32 wait_units(const dps_ctx *ctx, u32 units) { return (u32)std::min<double>(4.0e9, (double)units * ctx->wall_clock_scale); }
 
 // profiling -----------------------------------------------------------------
 hipEvent_t prof_event(dps_ctx *ctx)
@@ -441,6 +446,13 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
     ctx->d_counter = (u32 *)((char *)ctx->d_lagrange + lag_bytes);
     ctx->d_slice_ctr = (u64 *)((char *)ctx->d_counter + 256);
     if (hipMemset(ctx->d_counter, 0, COUNTER_BYTES) != hipSuccess) return bail(DPS_ERR_HIP);
+    {
+        int khz = 0;
+        if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0)
+            ctx->wall_clock_scale = (double)khz / 100000.0;
+        else
+            (void)hipGetLastError();
+    }
     ctx->pinned_words = 16384;
     if (hipEventCreateWithFlags(&ctx->stage_event, hipEventDisableTiming) != hipSuccess) return bail(DPS_ERR_HIP);
     // fine-grained host memory: a kernel's system-scope stores become visible to the polling host while the kernel runs
@@ -1654,11 +1666,10 @@ u32 slots_for(u32 workgroups) { return workgroups > 1 && workgroups <= SLOT_MAX_
 // In a launch made ahead of its round every workgroup polls the host's mailbox up to this many workgroups; in a larger
 // one only the first does and passes the mail on through device memory
 constexpr u32 POLY_AHEAD_MAX_WORKGROUPS = 64;
-// ... and is trusted to be still waiting for its mail for this long (its own patience: spin_limit polls of pinned
-// memory, at least a few hundred milliseconds)
+// ... and is trusted to be still waiting for its mail for this long (its own patience is several times that)
 constexpr int POLY_AHEAD_PATIENCE_MS = 20;
-// Polls of the host's mailbox (2.5 us each) after which a launch made ahead gives up: about 150 ms, so that a caller who
-// went away does not leave up to 768 waiting workgroups on the GPU for long (a resident kernel, one workgroup, waits seconds)
+// How long a launch made ahead waits for its mail, in units of 2.56 us (wait_units): about 150 ms, so that a caller who
+// went away does not leave up to 768 waiting workgroups on the GPU for long (a resident launch waits ten seconds)
 constexpr u32 AHEAD_SPIN_LIMIT = 60000;
 
 // Rounds of at most this many pairs run on poly_split_kernel
@@ -3009,7 +3020,7 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
             // (several workgroups: the first polls the host's mailbox and passes each mail on through device memory; with
             // all 256 of them polling host memory a trip took 90 us instead of 18)
             sa.relay = mail_relay(ctx);
-            sa.spin_limit = 4000000;  // a few seconds of polling, then the kernel gives up
+            sa.spin_limit = wait_units(ctx, 4000000);  // ten seconds, then the kernel gives up
             sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
             sa.out_host = ctx->d_pinned + slice_area_off(ctx);
             sa.seq0 = seq0 + (st.j0 - first);
@@ -3158,7 +3169,7 @@ int32_t FusedRound::launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahea
         pa.j = jj;
         pa.last_round = 0;
         pa.n_vars = sc->n_vars;
-        pa.spin_limit = 4000000;
+        pa.spin_limit = wait_units(ctx, 4000000);
         pa.eq0 = sc->eq_c0;
         pa.eq1 = sc->eq_c1;
         pa.mail = ctx->d_pinned + (ctx->res_off - 64);
@@ -3170,7 +3181,7 @@ int32_t FusedRound::launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahea
         pa.group_stride = 1;
         pa.raw_out = nullptr;
         pa.wait_first = ahead ? 1 : 0;
-        if (ahead && !p.reside) pa.spin_limit = AHEAD_SPIN_LIMIT;
+        if (ahead && !p.reside) pa.spin_limit = wait_units(ctx, AHEAD_SPIN_LIMIT);
         // (more workgroups than should poll the host's memory: the first one polls and passes the mail on)
         pa.relay = ahead && p.blocks * n_groups > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
         if (p.reside) {
@@ -3312,7 +3323,7 @@ int32_t FusedRound::product_launch_ahead()
             an.r0 = an.r1 = 0;
             an.skip1 = skip1_next ? 1 : 0;
             an.wait_first = 1;
-            an.spin_limit = AHEAD_SPIN_LIMIT;
+            an.spin_limit = wait_units(ctx, AHEAD_SPIN_LIMIT);
             an.mail = ctx->d_pinned + (ctx->res_off - 64);
             an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
             dpk::FastFin fn = ff;

@@ -591,6 +591,11 @@ constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
 // check word of a mailbox: seq ^ xor over the payload words of rotl(word_i, i)
 __host__ __device__ __forceinline__ u64 mail_mix(u64 w, u32 i) { return (i >= (u32)MAIL_R && i < (u32)MAIL_WORDS) ? rotl64(w, i) : 0; }
 
+// How long a kernel waits is time, not a number of polls (a poll of host memory takes 2.5 us, one of device memory a
+// fraction of that): `spin_limit` counts units of 256 ticks of the device's real-time counter (100 MHz: 2.56 us a unit;
+// the host scales its figures by the counter's rate).
+__device__ __forceinline__ bool wait_time_left(u64 t0, u32 spin_limit) { return wall_clock64() - t0 <= ((u64)spin_limit << 8); }
+
 // Waits for mail number `want` and copies it to `box` (LDS).  The first wavefront
 // polls: every lane loads one mailbox word, so one load instruction (one trip over
 // the host link) fetches the whole mail; it is accepted when the sequence number
@@ -601,7 +606,8 @@ __device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, 
     if (threadIdx.x < WAVE) {
         const u32 l = threadIdx.x;
         int ok = 0;
-        for (u32 spins = 0; spins < spin_limit; spins++) {
+        const u64 t0 = wall_clock64();
+        do {
             const u64 w = l < (u32)MAIL_WORDS ? ld_sys(mail + l) : 0;
             u64 x = mail_mix(w, l);
 #pragma unroll
@@ -614,7 +620,8 @@ __device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, 
                 break;
             }
             __builtin_amdgcn_s_sleep(2);
-        }
+            // (one lane's clock decides for the wavefront: the lanes must leave the loop together)
+        } while (__shfl((int)wait_time_left(t0, spin_limit), 0, WAVE));
         if (l == 0) *ok_lds = ok;
     }
     __syncthreads();
@@ -630,7 +637,7 @@ __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, boo
 {
     if (relay == nullptr) return tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
     // (the others outlast the first workgroup, which always passes something on: their polls of device memory are quicker)
-    if (!first_wg) return tail_wait_mail(relay, spin_limit > (1u << 25) ? ~0u : spin_limit << 6, seq, box, ok_lds);
+    if (!first_wg) return tail_wait_mail(relay, spin_limit + spin_limit / 4 + 4000, seq, box, ok_lds);
     const bool ok = tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
     if (threadIdx.x == 0) {
         u64 w[MAIL_WORDS];
@@ -1121,13 +1128,14 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             if (wg != 0) return;
             if (tid == 0) {
                 int ok = 0;
-                for (u32 spins = 0; spins < a.spin_limit; spins++) {
+                const u64 t0 = wall_clock64();
+                do {
                     if (__hip_atomic_load(a.gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Wc) {
                         ok = 1;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(1);
-                }
+                } while (wait_time_left(t0, a.spin_limit));
                 *ok_flag = ok;
             }
             __syncthreads();

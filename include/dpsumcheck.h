@@ -71,7 +71,9 @@ int32_t dps_ctx_sync(dps_ctx *ctx);
 
 /* ---- table storage: DensePolynomial::{new, new_from_smart_slice, as_view, evals}
  *      (zkml/src/tensor/mod.rs:364,390,401; zkml/src/lookup/logup_gkr/circuit.rs:262-269) ---- */
-/* upload 2^n_vars canonical base elements */
+/* upload 2^n_vars canonical base elements.  Table entries (here, in dps_mle_from_ext2 and in wrapped device memory) are
+ * taken as they are, not checked: an entry >= p gives undefined results (challenges, points and coefficients, which are
+ * few, are checked and rejected with DPS_ERR_INVALID). */
 int32_t dps_mle_from_base(dps_ctx *ctx, const uint64_t *host, uint32_t n_vars, dps_mle **out);
 /* upload 2^n_vars extension elements given as two limb arrays */
 int32_t dps_mle_from_ext2(dps_ctx *ctx, const uint64_t *c0, const uint64_t *c1, uint32_t n_vars, dps_mle **out);

@@ -5,6 +5,7 @@
 //   wavefront: every lane must arrive, as the hardware operations need every lane enabled.
 #pragma once
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <cstdint>
 #include <cstdio>
@@ -119,6 +120,11 @@ inline int update_dpp(int old, int src, int ctrl, int row_mask, int /*bank_mask*
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, rm, bm, bc) emu::update_dpp(old, src, ctrl, rm, bm, bc)
 // (uniform by construction where the kernels use it; a lane alone cannot check that here)
 #define __builtin_amdgcn_readfirstlane(x) (x)
+// the device's real-time counter: 100 MHz
+inline uint64_t wall_clock64()
+{
+    return (uint64_t)(std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count() / 10);
+}
 #define __builtin_amdgcn_fence(order, scope) std::atomic_thread_fence(std::memory_order_seq_cst)
 #define __builtin_amdgcn_s_waitcnt(x) ((void)0)
 // (a polling lane gives the other host threads a turn: a workgroup here is hundreds of threads on a few cores)
