@@ -71,6 +71,7 @@ struct dps_ctx {
     u64 *d_pinned = nullptr;    // device address of the same buffer
     size_t pinned_words = 0;
     double wall_clock_scale = 1.0;  // rate of the device's real-time counter / 100 MHz
+    u64 logup_builds = 0;           // fraction trees built so far (their outputs rotate through a few areas of the pinned buffer)
     hipEvent_t stage_event = nullptr;  // recorded after a launch that reads the staging region of the pinned buffer
     bool stage_pending = false;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
@@ -3639,7 +3640,14 @@ struct dps_logup {
     u32 n_layers;  // including the input layer
     std::shared_ptr<Storage> arena;
     std::vector<u64> layer_off;  // per layer k >= 1: offset of the numerator array; the denominator follows
+    u64 out_seq = 0;             // the last launch of the build also hands the last layer's four entries to the host: under this
+    u32 out_slot = 0;            // sequence number, in this one of the context's areas for them (0: it does not)
+    u64 out_build = 0;           // the context's count of such builds after this one
 };
+
+// areas of the pinned buffer for the outputs of the trees built last (16 words each, behind the resident launches' result area)
+constexpr u32 LOGUP_OUT_AREAS = 8;
+size_t logup_out_off(const dps_ctx *ctx, u32 slot) { return slice_area_off(ctx) + dpk::SL_AREA_WORDS + 64 + 16 * (size_t)slot; }
 
 extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uint32_t n_cols, const dps_mle *numer,
                                    const uint64_t c[2], const uint64_t beta[2], dps_logup **out)
@@ -3700,12 +3708,31 @@ extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uin
             dpk::logup_first_kernel<<<grid_for(half), dpk::BLOCK, 0, ctx->stream>>>(a);
             HIPCHK(ctx, hipGetLastError());
         }
-        for (u32 k = 2; k < top; k++) {
+        // levels of more than 2^LOGUP_TAIL_BITS entries: a launch each; the others in one launch of one workgroup
+        u32 k = 2;
+        for (; k < top && (len >> k) > (1ull << dpk::LOGUP_TAIL_BITS); k++) {
             u64 prev = len >> (k - 1), cur = len >> k;
             const u64 *pn0 = st->c0 + lg->layer_off[k - 1], *pn1 = st->c1 + lg->layer_off[k - 1];
             u64 *n0 = st->c0 + lg->layer_off[k], *n1 = st->c1 + lg->layer_off[k];
             ProfScope ps(ctx, DPS_K_LOGUP, (double)prev * 32.0 + (double)cur * 32.0);
             dpk::logup_next_kernel<<<grid_for(cur), dpk::BLOCK, 0, ctx->stream>>>(pn0, pn1, pn0 + prev, pn1 + prev, cur, n0, n1, n0 + cur, n1 + cur);
+            HIPCHK(ctx, hipGetLastError());
+        }
+        if (k < top) {
+            dpk::LogupTailArgs ta;
+            memset(&ta, 0, sizeof ta);
+            ta.c0 = st->c0;
+            ta.c1 = st->c1;
+            ta.n_levels = top - k;
+            ta.first_cur = len >> k;
+            for (u32 l = 0; l <= ta.n_levels; l++) ta.off[l] = lg->layer_off[k - 1 + l];
+            lg->out_slot = (u32)(ctx->logup_builds++ % LOGUP_OUT_AREAS);
+            lg->out_build = ctx->logup_builds;
+            lg->out_seq = ++ctx->seq;
+            ta.out_host = ctx->d_pinned + logup_out_off(ctx, lg->out_slot);
+            ta.seq = lg->out_seq;
+            ProfScope ps(ctx, DPS_K_LOGUP, (double)ta.first_cur * 4 * 32.0);
+            dpk::logup_tail_kernel<<<1, dpk::LOGUP_TAIL_BLOCK, 0, ctx->stream>>>(ta);
             HIPCHK(ctx, hipGetLastError());
         }
     }
@@ -3738,6 +3765,11 @@ extern "C" int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8])
     if (lg->n_layers < 2) return fail(ctx, DPS_ERR_STATE, "dps_logup_outputs: the instance has no layer above its input");
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
+    if (lg->out_seq) {
+        // the build's last launch hands them over itself, unless a later build has taken the area since
+        if (ctx->logup_builds - lg->out_build < LOGUP_OUT_AREAS && wait_result_at(ctx, logup_out_off(ctx, lg->out_slot), lg->out_seq, 0, 8, out, 9, 8) == DPS_OK)
+            return DPS_OK;
+    }
     u64 off = lg->layer_off[lg->n_layers - 1];
     u64 a[4], b[4];
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));

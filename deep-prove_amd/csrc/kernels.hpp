@@ -2339,6 +2339,51 @@ logup_next_kernel(const u64 *__restrict__ pn0, const u64 *__restrict__ pn1, cons
     }
 }
 
+// The levels of at most 2^LOGUP_TAIL_BITS entries of a tree, all in one launch of one workgroup: below that a level is a
+// dispatch of 3 us whatever its size, and a tree has a dozen of them.  The four entries of the last level (n_lo, n_hi,
+// d_lo, d_hi, what the prover puts on the transcript first) also go to the host, as a round's result does.
+constexpr u32 LOGUP_TAIL_BITS = 11;
+constexpr int LOGUP_TAIL_BLOCK = 1024;
+struct LogupTailArgs {
+    u64 *c0, *c1;                       // the tree's arena
+    u64 off[LOGUP_TAIL_BITS + 2];       // off[0]: the level read first; off[l + 1]: level l of this launch
+    u32 n_levels;
+    u64 first_cur;                      // entries per array of the first level written
+    u64 *out_host;                      // 8 words + check word + sequence number (slots 8 and 9)
+    u64 seq;
+};
+__global__ void __launch_bounds__(LOGUP_TAIL_BLOCK) logup_tail_kernel(LogupTailArgs a)
+{
+    u64 cur = a.first_cur;
+    for (u32 l = 0; l < a.n_levels; l++, cur >>= 1) {
+        const u64 prev = 2 * cur;
+        const u64 *pn0 = a.c0 + a.off[l], *pn1 = a.c1 + a.off[l], *pd0 = pn0 + prev, *pd1 = pn1 + prev;
+        u64 *n0 = a.c0 + a.off[l + 1], *n1 = a.c1 + a.off[l + 1], *d0 = n0 + cur, *d1 = n1 + cur;
+        for (u64 i = threadIdx.x; i < cur; i += LOGUP_TAIL_BLOCK) {
+            const E2 nl = gl::e2(pn0[i], pn1[i]), nh = gl::e2(pn0[i + cur], pn1[i + cur]);
+            const E2 dl = gl::e2(pd0[i], pd1[i]), dh = gl::e2(pd0[i + cur], pd1[i + cur]);
+            const E2 num = gl::add(gl::mul(nl, dh), gl::mul(nh, dl));
+            const E2 den = gl::mul(dl, dh);
+            n0[i] = num.c0;
+            n1[i] = num.c1;
+            d0[i] = den.c0;
+            d1[i] = den.c1;
+        }
+        // the next level reads what other threads of this workgroup have just written
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const u64 *l0 = a.c0 + a.off[a.n_levels], *l1 = a.c1 + a.off[a.n_levels];
+        u64 w[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            w[2 * i] = l0[i];
+            w[2 * i + 1] = l1[i];
+        }
+        publish_words(a.out_host, 0, w, 8, a.seq, 9, 8);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // element-wise field operations on device vectors (arithmetic self-check)
 // ---------------------------------------------------------------------------
