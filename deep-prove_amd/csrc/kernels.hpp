@@ -2302,8 +2302,9 @@ struct LogupFirstArgs {
 __global__ void __launch_bounds__(BLOCK) logup_first_kernel(LogupFirstArgs a)
 {
     for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < a.half; i += (u64)gridDim.x * BLOCK) {
-        E2 dlo = gl::e2(a.c0, a.c1), dhi = dlo;
-        for (u32 k = 0; k < a.n_cols; k++) {
+        // (the first column's power of the column challenge is 1: no product)
+        E2 dlo = gl::e2(gl::add(a.c0, a.cols[0][i]), a.c1), dhi = gl::e2(gl::add(a.c0, a.cols[0][i + a.half]), a.c1);
+        for (u32 k = 1; k < a.n_cols; k++) {
             E2 pw = gl::e2(a.pw[2 * k], a.pw[2 * k + 1]);
             dlo = gl::add(dlo, gl::mul_base(pw, a.cols[k][i]));
             dhi = gl::add(dhi, gl::mul_base(pw, a.cols[k][i + a.half]));
@@ -2340,9 +2341,10 @@ logup_next_kernel(const u64 *__restrict__ pn0, const u64 *__restrict__ pn1, cons
 }
 
 // The levels of at most 2^LOGUP_TAIL_BITS entries of a tree, all in one launch of one workgroup: below that a level is a
-// dispatch of 3 us whatever its size, and a tree has a dozen of them.  The four entries of the last level (n_lo, n_hi,
-// d_lo, d_hi, what the prover puts on the transcript first) also go to the host, as a round's result does.
-constexpr u32 LOGUP_TAIL_BITS = 11;
+// dispatch of 3 us whatever its size, and a tree has ten of them.  A level is read from LDS, where the level before left
+// it (the first from device memory), and written to LDS and to the arena.  The four entries of the last level (n_lo,
+// n_hi, d_lo, d_hi, what the prover puts on the transcript first) also go to the host, as a round's result does.
+constexpr u32 LOGUP_TAIL_BITS = 10;
 constexpr int LOGUP_TAIL_BLOCK = 1024;
 struct LogupTailArgs {
     u64 *c0, *c1;                       // the tree's arena
@@ -2354,32 +2356,46 @@ struct LogupTailArgs {
 };
 __global__ void __launch_bounds__(LOGUP_TAIL_BLOCK) logup_tail_kernel(LogupTailArgs a)
 {
-    u64 cur = a.first_cur;
+    constexpr u32 CAP = 1u << LOGUP_TAIL_BITS;
+    // numerators (two limb arrays) and denominators (two) of a level: CAP entries each in `big`, half of that in `small`
+    __shared__ u64 big[4 * CAP], small_[2 * CAP];
+    u32 cur = (u32)a.first_cur;
     for (u32 l = 0; l < a.n_levels; l++, cur >>= 1) {
-        const u64 prev = 2 * cur;
-        const u64 *pn0 = a.c0 + a.off[l], *pn1 = a.c1 + a.off[l], *pd0 = pn0 + prev, *pd1 = pn1 + prev;
+        const u32 prev = 2 * cur;
+        const bool to_big = (l & 1) == 0;
+        const u32 cap_s = to_big ? CAP / 2 : CAP, cap_d = to_big ? CAP : CAP / 2;
+        const u64 *src = to_big ? small_ : big;
+        u64 *dst = to_big ? big : small_;
+        const u64 *g0 = a.c0 + a.off[l], *g1 = a.c1 + a.off[l];
         u64 *n0 = a.c0 + a.off[l + 1], *n1 = a.c1 + a.off[l + 1], *d0 = n0 + cur, *d1 = n1 + cur;
-        for (u64 i = threadIdx.x; i < cur; i += LOGUP_TAIL_BLOCK) {
-            const E2 nl = gl::e2(pn0[i], pn1[i]), nh = gl::e2(pn0[i + cur], pn1[i + cur]);
-            const E2 dl = gl::e2(pd0[i], pd1[i]), dh = gl::e2(pd0[i + cur], pd1[i + cur]);
+        for (u32 i = threadIdx.x; i < cur; i += LOGUP_TAIL_BLOCK) {
+            E2 nl, nh, dl, dh;
+            if (l == 0) {
+                nl = gl::e2(g0[i], g1[i]), nh = gl::e2(g0[i + cur], g1[i + cur]);
+                dl = gl::e2(g0[prev + i], g1[prev + i]), dh = gl::e2(g0[prev + i + cur], g1[prev + i + cur]);
+            } else {
+                nl = gl::e2(src[i], src[cap_s + i]), nh = gl::e2(src[i + cur], src[cap_s + i + cur]);
+                dl = gl::e2(src[2 * cap_s + i], src[3 * cap_s + i]), dh = gl::e2(src[2 * cap_s + i + cur], src[3 * cap_s + i + cur]);
+            }
             const E2 num = gl::add(gl::mul(nl, dh), gl::mul(nh, dl));
             const E2 den = gl::mul(dl, dh);
             n0[i] = num.c0;
             n1[i] = num.c1;
             d0[i] = den.c0;
             d1[i] = den.c1;
+            dst[i] = num.c0;
+            dst[cap_d + i] = num.c1;
+            dst[2 * cap_d + i] = den.c0;
+            dst[3 * cap_d + i] = den.c1;
         }
-        // the next level reads what other threads of this workgroup have just written
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        const u64 *l0 = a.c0 + a.off[a.n_levels], *l1 = a.c1 + a.off[a.n_levels];
-        u64 w[8];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            w[2 * i] = l0[i];
-            w[2 * i + 1] = l1[i];
-        }
+        // the last level: two numerators and two denominators, in the buffer written last
+        const bool in_big = ((a.n_levels - 1) & 1) == 0;
+        const u64 *dst = in_big ? big : small_;
+        const u32 cap_d = in_big ? CAP : CAP / 2;
+        const u64 w[8] = {dst[0], dst[cap_d], dst[1], dst[cap_d + 1], dst[2 * cap_d], dst[3 * cap_d], dst[2 * cap_d + 1], dst[3 * cap_d + 1]};
         publish_words(a.out_host, 0, w, 8, a.seq, 9, 8);
     }
 }
