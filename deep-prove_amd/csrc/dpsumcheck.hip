@@ -279,7 +279,25 @@ u64 h_pow(u64 a, u64 e)
     }
     return r;
 }
-u64 h_inv(u64 a) { return h_pow(a, gl::P - 2); }
+// a^(p - 2), p - 2 = 2^64 - 2^32 - 1: 63 squarings and 9 products along the runs of ones of the exponent (the round loop
+// of a sum with an eq factor inverts one element per round)
+u64 h_inv(u64 a)
+{
+    // base^(2^n) * tail
+    auto sq_mul = [](u64 base, int n, u64 tail) {
+        for (int i = 0; i < n; i++) base = gl::mul(base, base);
+        return gl::mul(base, tail);
+    };
+    const u64 t2 = sq_mul(a, 1, a);        // 2^2 - 1
+    const u64 t3 = sq_mul(t2, 1, a);       // 2^3 - 1
+    const u64 t6 = sq_mul(t3, 3, t3);      // 2^6 - 1
+    const u64 t12 = sq_mul(t6, 6, t6);     // 2^12 - 1
+    const u64 t24 = sq_mul(t12, 12, t12);  // 2^24 - 1
+    const u64 t30 = sq_mul(t24, 6, t6);    // 2^30 - 1
+    const u64 t31 = sq_mul(t30, 1, a);     // 2^31 - 1
+    const u64 t63 = sq_mul(t31, 32, t31);  // (2^31 - 1) 2^32 + 2^31 - 1
+    return sq_mul(t63, 1, a);              // 2^64 - 2^32 - 1
+}
 E2 h_e2_inv(E2 a)
 {
     u64 n = h_inv(gl::sub(gl::mul(a.c0, a.c0), gl::mul_small(gl::mul(a.c1, a.c1), (u32)gl::W)));
@@ -1223,6 +1241,86 @@ extern "C" int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint6
     return DPS_OK;
 }
 
+namespace {
+
+// The last step of a partial evaluation: what is left of the tensor is indexed by the stacked and contracted axes in
+// their original order; like the reference (axis.rs:1222-1233) the flat result is cut into chunks of `contraction`
+// entries, one table per chunk, each padded to a power of two.  `cur`: the result of the contractions so far (owned
+// here), or nullptr when no outer axis was fixed (the source is then read through `dims` / `strides`).
+int32_t rows_as_tables(dps_ctx *ctx, dps_mle *cur, const u64 *in0, const u64 *in1, int in_int, const std::vector<u64> &dims,
+                       const std::vector<u64> &strides, u64 stacked, u64 contraction, dps_mle **out)
+{
+    int32_t rc = DPS_OK;
+    u32 nv = log2u(contraction);
+    u64 tl = 1ull << nv;
+    dps_mle *all = nullptr;
+    // rows that are a power of two long already: the result is the table as it stands
+    const bool as_it_stands = cur && contraction == tl && cur->kind == DPS_EXT2 && cur->offset == 0 && cur->len == stacked * tl;
+    if (as_it_stands) {
+        all = cur;
+        cur = nullptr;
+    } else {
+        rc = new_table(ctx, DPS_EXT2, stacked * tl, &all);
+    }
+    if (rc == DPS_OK && !as_it_stands) {
+        if (cur) {
+            dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(cur->st->c0, cur->st->c1, stacked, contraction, tl,
+                                                                                    all->st->c0, all->st->c1);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
+        } else {
+            // no outer axis: contract a unit axis with the table {1} to copy the unpadded region
+            u64 one[2] = {0, 0};
+            dps_mle *unit = nullptr;
+            rc = dps_eq_build(ctx, one, 0, &unit);
+            dps_mle *flat = nullptr;
+            if (rc == DPS_OK) rc = new_table(ctx, DPS_EXT2, stacked * contraction, &flat);
+            if (rc == DPS_OK) {
+                AxisJob j;
+                j.in0 = in0;
+                j.in1 = in1;
+                j.in_int = in_int;
+                j.b0 = unit->p0();
+                j.b1 = unit->p1();
+                j.K = 1;
+                j.stride_k = 0;
+                j.post_dims = dims;
+                j.post_strides = strides;
+                j.o0 = flat->st->c0;
+                j.o1 = flat->st->c1;
+                rc = axis_dot(ctx, j);
+            }
+            if (rc == DPS_OK) {
+                dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(flat->st->c0, flat->st->c1, stacked, contraction,
+                                                                                        tl, all->st->c0, all->st->c1);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
+            }
+            (void)hipStreamSynchronize(ctx->stream);
+            delete unit;
+            delete flat;
+        }
+    }
+    // (no wait for the stream: the blocks given back are reused in stream order, and whoever consumes the result waits)
+    delete cur;
+    if (rc != DPS_OK) {
+        delete all;
+        return rc;
+    }
+    for (u64 s = 0; s < stacked; s++) {
+        rc = dps_mle_view(all, s * tl, nv, &out[s]);
+        if (rc != DPS_OK) {
+            for (u64 q = 0; q < s; q++) delete out[q];
+            delete all;
+            return rc;
+        }
+    }
+    delete all;  // the views keep the storage alive
+    return DPS_OK;
+}
+
+}  // namespace
+
 extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const uint64_t *padded_dims,
                                     const uint64_t *unpadded_dims, uint32_t n_dims, const int32_t *kinds,
                                     const uint64_t *const *points, dps_mle **out, uint32_t out_cap, uint32_t *n_out)
@@ -1318,75 +1416,7 @@ extern "C" int32_t dps_partial_eval(dps_ctx *ctx, const dps_mle *tensor, const u
         delete cur;
         return rc;
     }
-    // What is left is indexed by the stacked and contracted axes in their original
-    // order; like the reference (axis.rs:1222-1233) the flat result is cut into
-    // chunks of `contraction` entries, one table per chunk.
-    // gather (strided source when no outer axis was fixed) into padded rows
-    u32 nv = log2u(contraction);
-    u64 tl = 1ull << nv;
-    dps_mle *all = nullptr;
-    // rows that are a power of two long already: the result is the table as it stands
-    const bool as_it_stands = cur && contraction == tl && cur->kind == DPS_EXT2 && cur->offset == 0 && cur->len == stacked * tl;
-    if (as_it_stands) {
-        all = cur;
-        cur = nullptr;
-    } else {
-        rc = new_table(ctx, DPS_EXT2, stacked * tl, &all);
-    }
-    if (rc == DPS_OK && !as_it_stands) {
-        if (cur) {
-            dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(cur->st->c0, cur->st->c1, stacked, contraction, tl,
-                                                                                    all->st->c0, all->st->c1);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
-        } else {
-            // no outer axis: contract a unit axis with the table {1} to copy the unpadded region
-            u64 one[2] = {0, 0};
-            dps_mle *unit = nullptr;
-            rc = dps_eq_build(ctx, one, 0, &unit);
-            dps_mle *flat = nullptr;
-            if (rc == DPS_OK) rc = new_table(ctx, DPS_EXT2, stacked * contraction, &flat);
-            if (rc == DPS_OK) {
-                AxisJob j;
-                j.in0 = in0;
-                j.in1 = in1;
-                j.in_int = in_int;
-                j.b0 = unit->p0();
-                j.b1 = unit->p1();
-                j.K = 1;
-                j.stride_k = 0;
-                j.post_dims = dims;
-                j.post_strides = strides;
-                j.o0 = flat->st->c0;
-                j.o1 = flat->st->c1;
-                rc = axis_dot(ctx, j);
-            }
-            if (rc == DPS_OK) {
-                dpk::pad_rows_kernel<<<grid_for(stacked * tl), dpk::BLOCK, 0, ctx->stream>>>(flat->st->c0, flat->st->c1, stacked, contraction,
-                                                                                        tl, all->st->c0, all->st->c1);
-                hipError_t e = hipGetLastError();
-                if (e != hipSuccess) rc = fail(ctx, DPS_ERR_HIP, "pad launch: %s", hipGetErrorString(e));
-            }
-            (void)hipStreamSynchronize(ctx->stream);
-            delete unit;
-            delete flat;
-        }
-    }
-    // (no wait for the stream: the blocks given back are reused in stream order, and whoever consumes the result waits)
-    delete cur;
-    if (rc != DPS_OK) {
-        delete all;
-        return rc;
-    }
-    for (u64 s = 0; s < stacked; s++) {
-        rc = dps_mle_view(all, s * tl, nv, &out[s]);
-        if (rc != DPS_OK) {
-            for (u64 q = 0; q < s; q++) delete out[q];
-            delete all;
-            return rc;
-        }
-    }
-    delete all;  // the views keep the storage alive
+    CHK(rows_as_tables(ctx, cur, in0, in1, in_int, dims, strides, stacked, contraction, out));
     *n_out = (u32)stacked;
     return DPS_OK;
 }
