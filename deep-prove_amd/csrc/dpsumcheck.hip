@@ -1466,6 +1466,8 @@ struct dps_sc {
         u64 *h0[dpk::SL_MAX_TABS], *h1[dpk::SL_MAX_TABS];  // where a stage that is not the last leaves its entries (the next stage's source)
     };
     std::vector<Stage> stages;
+    std::vector<u32> slice_ids;                // the tables of the resident launches (session indices), in slot order
+    std::vector<dpk::SliceTerm> slice_terms;   // sums of several terms: the terms, their tables as slots of slice_ids
     std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip
     std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip)
     u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
@@ -1936,7 +1938,8 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
         u64 len = (entries / W) >> pend;  // entries per table and workgroup in the trip's first round
         st.cap = (u32)len;
         for (;;) {
-            const bool dbl = len >= 4 && j + 1 <= n && claim_gives_p1(j + 1);
+            // (as the last trip only when the 4 entries left of every table fit the hand-over)
+            const bool dbl = len >= 4 && j + 1 <= n && claim_gives_p1(j + 1) && !(j + 1 == n && n_tabs > (u32)dpk::SL_DBL_LAST_MAX_TABS);
             if (dbl) st.dbl_mask |= 1u << st.n_trips;
             st.n_trips++;
             sc->round_kind[j] = dbl ? 2 : 1;
@@ -2246,12 +2249,42 @@ int32_t SessionSetup::plan_and_ready_tables()
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
     sc->prev_chal = gl::e2_zero();
-    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) plan_resident_rounds(sc, sc->fast_nf);
-    // a sum of several terms over one group of full-size tables (a fraction-sum layer, a claim merge): the same launches
-    if (sc->poly && sc->poly_tabs.size() == 1 && sc->fast_nf <= 4 && sc->n_terms <= (u32)dpk::SL_MAX_TERMS) {
-        bool ok = n_mles == sc->poly_tabs[0].size() + (sc->fast_eq >= 0 ? 1 : 0);
-        for (u32 k : sc->poly_tabs[0]) ok = ok && nv0[k] == n_vars && !mles[k]->pad_vars;
-        if (ok) plan_resident_rounds(sc, (u32)sc->poly_tabs[0].size());
+    sc->slice_ids.clear();
+    sc->slice_terms.clear();
+    if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
+        sc->slice_ids.assign(sc->fast_order, sc->fast_order + sc->fast_nf);
+        plan_resident_rounds(sc, sc->fast_nf);
+    }
+    // A sum of several terms over full-size tables (a fraction-sum layer, a claim merge, the stacked products of an
+    // einsum): the same launches.  One group of tables from the first round that fits; more tables than a group holds
+    // (up to SL_MAX_TABS) when every round is resident, so that the groups' own launches are never needed.
+    if (sc->poly && sc->fast_nf <= 4 && sc->n_terms <= (u32)dpk::SL_MAX_TERMS) {
+        std::vector<u32> ids;
+        for (const auto &g : sc->poly_tabs)
+            for (u32 k : g)
+                if (std::find(ids.begin(), ids.end(), k) == ids.end()) ids.push_back(k);
+        bool ok = n_mles == ids.size() + (sc->fast_eq >= 0 ? 1 : 0) && ids.size() <= (size_t)dpk::SL_MAX_TABS;
+        for (u32 k : ids) ok = ok && nv0[k] == n_vars && !mles[k]->pad_vars;
+        if (ok) {
+            sc->slice_ids = ids;
+            for (const dps_term &t : sc->terms) {
+                dpk::SliceTerm tm;
+                memset(&tm, 0, sizeof tm);
+                tm.c0 = t.coeff[0], tm.c1 = t.coeff[1], tm.w = gl::mul_small(t.coeff[1], (u32)gl::W);
+                for (u32 f = 0; f < t.n_factors; f++)
+                    if ((int)t.factors[f] != sc->fast_eq) tm.slot[tm.n_factors++] = (uint8_t)(std::find(ids.begin(), ids.end(), t.factors[f]) - ids.begin());
+                sc->slice_terms.push_back(tm);
+            }
+            plan_resident_rounds(sc, (u32)ids.size());
+            if (sc->poly_tabs.size() > 1 && sc->tail_j0 != 1) {
+                // several groups and not every round resident: the groups' launches take the session
+                sc->stages.clear();
+                sc->tail_j0 = 0;
+                sc->fin_len = 0;
+                sc->round_kind.assign(n_vars + 2, 0);
+                sc->round_wide.assign(n_vars + 2, 0);
+            }
+        }
     }
     // What this session reads of its tables: an eq table taken in closed form is read level by level -- level j in round j,
     // except in the large rounds of a product, which take the low table of level j and level j + 16 instead -- and
@@ -2508,7 +2541,7 @@ int32_t SessionSetup::allocate_device_block()
     bytes_po = round_up(sc->h_poly_ops.size() * sizeof(dpk::PolyOp), 256);
     // what a resident stage that does not run to the last round leaves for the next: two limb arrays per table
     size_t bytes_hand = 0;
-    const u32 slice_tabs = sc->poly ? (sc->poly_tabs.empty() ? 0u : (u32)sc->poly_tabs[0].size()) : sc->fast_nf;
+    const u32 slice_tabs = (u32)sc->slice_ids.size();
     for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * slice_tabs;
     size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result + bytes_hand;
     CHK(pool_alloc(ctx, total, &sc->dev_block));
@@ -2573,7 +2606,7 @@ int32_t SessionSetup::stage_descriptors()
     // single group of terms, inline in the kernel arguments or staged in pinned memory for the resident launch) upload
     // nothing unless a step outside that flow needs the block (ensure_descs).
     sc->descs_uploaded = false;
-    const bool self_contained = (sc->fast && sc->tail_j0) ||
+    const bool self_contained = (sc->fast && sc->tail_j0) || sc->tail_j0 == 1 ||
                                 (sc->poly && sc->poly_tabs.size() == 1 && sc->h_poly_terms.size() <= (size_t)dpk::POLY_LDS_TERMS);
     if (!self_contained) {
         CHK(ensure_descs(sc));
@@ -3007,12 +3040,15 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
             const size_t last_si = merged ? si + 1 : si;
             dpk::SliceArgs sa;
             memset(&sa, 0, sizeof sa);
-            const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : nf;
+            const u32 n_tabs = (u32)sc->slice_ids.size();
             for (u32 f = 0; f < n_tabs; f++) {
                 // the first stage reads what the launch of the round before it wrote (or the session's own tables)
                 if (si > 0) {
                     sa.s0[f] = sc->stages[si - 1].h0[f];
                     sa.s1[f] = sc->stages[si - 1].h1[f];
+                } else if (sc->poly && first == 1) {
+                    sa.s0[f] = sc->m[sc->slice_ids[f]].c0;
+                    sa.s1[f] = sc->m[sc->slice_ids[f]].c1;
                 } else if (sc->poly) {
                     const dpk::PolyTab &tb = sc->h_poly_groups[first - 1].tab[f];
                     sa.s0[f] = tb.s0;
@@ -3026,14 +3062,8 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
             }
             sa.n_tabs = n_tabs;
             if (sc->poly) {
-                sa.n_terms = (u32)sc->h_poly_terms.size();
-                for (u32 m = 0; m < sa.n_terms; m++) {
-                    const dpk::PolyTerm &pt = sc->h_poly_terms[m];
-                    dpk::SliceTerm &tm = sa.terms[m];
-                    tm.c0 = pt.c0, tm.c1 = pt.c1, tm.w = pt.w;
-                    tm.n_factors = pt.n_factors;
-                    memcpy(tm.slot, pt.slot, sizeof tm.slot);
-                }
+                sa.n_terms = (u32)sc->slice_terms.size();
+                std::copy(sc->slice_terms.begin(), sc->slice_terms.end(), sa.terms);
             }
             sa.src_len = st.src_len;
             sa.pend0 = st.pend0;
@@ -3498,13 +3528,13 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
             // the resident launch left 2 entries per table, or 4 when its last trip covered two rounds (the challenge
             // between them is the one the last round's call brought)
             const u32 L = sc->fin_len;
-            const u32 n_tabs = sc->poly ? (u32)sc->poly_tabs[0].size() : sc->fast_nf;
+            const u32 n_tabs = (u32)sc->slice_ids.size();
             CHK(wait_result_at(ctx, slice_area_off(ctx), sc->pairs_seq, dpk::SL_FIN_SLOT, 2 * L * n_tabs, w, dpk::SL_FIN_SEQ_SLOT, dpk::SL_FIN_CHK_SLOT));
             for (u32 f = 0; f < n_tabs; f++) {
                 auto at = [&](u32 e) { return gl::e2(w[2 * (f * L + e)], w[2 * (f * L + e) + 1]); };
                 auto fold = [](E2 lo, E2 hi, E2 c) { return gl::add(lo, gl::mul(c, gl::sub(hi, lo))); };
                 const E2 v = L == 4 ? fold(fold(at(0), at(1), sc->prev_chal), fold(at(2), at(3), sc->prev_chal), r) : fold(at(0), at(1), r);
-                const u32 k = sc->poly ? sc->poly_tabs[0][f] : sc->fast_order[f];
+                const u32 k = sc->slice_ids[f];
                 final_evals_out[2 * k] = v.c0;
                 final_evals_out[2 * k + 1] = v.c1;
             }

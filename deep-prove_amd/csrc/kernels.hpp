@@ -1010,12 +1010,14 @@ constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
 constexpr u64 SL_CTR_MASK = (1ull << 56) - 1, SL_CTR_ONE = 1ull << 56;
 __host__ __device__ __forceinline__ u64 sl_tag(u64 trip_seq) { return 0x80 | (trip_seq & 0x7F); }
 // with the last trip of a run to the last round: the entries every table still has (2, or 4 after a trip of two rounds)
-constexpr int SL_FIN_SLOT = 104, SL_FIN_SEQ_SLOT = 160, SL_FIN_CHK_SLOT = 161, SL_AREA_WORDS = 192;
+constexpr int SL_FIN_SLOT = 104, SL_FIN_SEQ_SLOT = 168, SL_FIN_CHK_SLOT = 169, SL_AREA_WORDS = 192;
 static_assert(4 * SL_MAX_SUMS <= SL_FIN_SLOT, "the counters lie before the last entries");
 constexpr int SL_MAX_TRIPS = 32;
-constexpr int SL_MAX_TABS = 7;    // tables of a sum of several terms (a product has at most 3)
+constexpr int SL_MAX_TABS = 16;   // tables of a sum of several terms (a product has at most 3)
+constexpr int SL_DBL_LAST_MAX_TABS = 8;  // a trip of two rounds can be the last one only with so few tables (4 entries of each go to the host)
 constexpr int SL_MAX_TERMS = 24;
-static_assert(SL_FIN_SLOT + 2 * 4 * SL_MAX_TABS <= SL_FIN_SEQ_SLOT && 2 * 4 * SL_MAX_TABS <= WAVE, "the last entries of every table fit the result area and one wavefront");
+static_assert(SL_FIN_SLOT + WAVE <= SL_FIN_SEQ_SLOT && 2 * 4 * SL_DBL_LAST_MAX_TABS <= WAVE && 2 * 2 * SL_MAX_TABS <= WAVE,
+              "the last entries of every table fit the result area and one wavefront");
 // a term of a sum of several terms: coefficient (prepared: w = 7 c1) times the tables in `slot`
 struct SliceTerm {
     u64 c0, c1, w;

@@ -158,7 +158,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         Stage st{1, j, pend, entries, {}};
         u64 len = entries >> pend;
         while (j <= n_vars) {
-            const bool dbl = len >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1);
+            const bool dbl = len >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1) && !(j + 1 == n_vars && NT > (u32)dpk::SL_DBL_LAST_MAX_TABS);
             st.trips.push_back({j, dbl});
             const u32 p = dbl ? 2 : 1;
             j += p;
@@ -455,6 +455,11 @@ int main()
                              {Term{felt2(), {0, 1, 2}}, Term{felt2(), {3, 3, 4}}, Term{felt2(), {4}}, Term{felt2(), {}}});
     run_case<4, false, true>("degree 4, base-field tables, from round 1", 6, 1, 1, 3, {}, {Term{felt2(), {0, 0, 1, 2}}, Term{felt2(), {1, 2}}}, 2);
     run_case<2, true, true>("base-field tables folded once on the way in (from round 2)", 9, 2, 2, 3, {}, {Term{felt2(), {0, 1}}, Term{felt2(), {1, 2}}}, 2);
+    // the stacked products of an einsum: 16 tables, 8 terms of two factors each, every round resident
+    std::vector<Term> stacked;
+    for (u32 i = 0; i < 8; i++) stacked.push_back(Term{felt2(), {2 * i, 2 * i + 1}});
+    run_case<2, false, true>("16 tables, 8 products, from round 1 (the last two rounds go alone)", 8, 1, 1, 16, {}, stacked);
+    run_case<2, false, true>("the same with an odd number of rounds", 7, 1, 1, 16, {}, stacked);
     printf("%s\n", failures ? "FAILED" : "all cases ok");
     return failures ? 1 : 0;
 }

@@ -127,10 +127,25 @@ def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
            [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(pt)], [(one, [2, 0, 1])])
 
 
-@pytest.mark.parametrize("n_tabs", [4, 11])
+@pytest.mark.parametrize("n,n_tabs,n_terms,with_eq", [(7, 16, 8, False), (8, 16, 8, False), (8, 16, 24, True), (9, 16, 8, False),
+                                                      (12, 13, 10, True), (16, 16, 8, False), (16, 9, 12, True), (17, 16, 8, False)])
+def test_more_tables_than_a_group_all_rounds_resident(dp, ctx, orc, n, n_tabs, n_terms, with_eq):
+    """Up to 16 full-size tables whose first round fits the resident launches (2^15 pairs) run there from round 1,
+    as the stacked products of an einsum do; with 9 or more tables the last two rounds go one per trip.  n = 17 is
+    the first size that does not fit and runs the groups' launches."""
+    gpu, host, terms = _instance(ctx, orc, 1300 + n + n_tabs, n, [n] * n_tabs, [], n_terms, 2, with_eq)
+    # every table in some term: the stacked products first
+    one = np.array([1, 0], dtype=np.uint64)
+    e = [len(gpu) - 1] if with_eq else []
+    terms = [(one, [2 * i, min(2 * i + 1, n_tabs - 1)] + e) for i in range((n_tabs + 1) // 2)] + terms[(n_tabs + 1) // 2:]
+    _check(dp, ctx, orc, n, gpu, host, terms)
+    _check(dp, ctx, orc, n, gpu, host, terms)
+
+
+@pytest.mark.parametrize("n_tabs", [4, 11, 18])
 def test_resident_groups_give_way(dp, ctx, orc, n_tabs):
     """A multi-term session stays on the GPU from the round of 256 pairs on (one workgroup, or one per group of
-    tables).  Another call on the context makes the resident launch exit through its mailbox, the interrupted
+    tables), or from round 1 (up to 16 tables).  Another call on the context makes the resident launch exit through its mailbox, the interrupted
     session reports it, an unfinished session can simply be dropped, and the context keeps working."""
     n = 11
     gpu, host, terms = _instance(ctx, orc, 700 + n_tabs, n, [n] * n_tabs, [], 2 * n_tabs, 2, True)
@@ -156,13 +171,13 @@ def test_resident_groups_give_way(dp, ctx, orc, n_tabs):
         _check(dp, ctx, orc, n, gpu, host, terms)
 
 
-@pytest.mark.parametrize("n_tabs", [4, 11])
+@pytest.mark.parametrize("n_tabs", [4, 18])
 def test_launch_made_ahead_steps_aside(dp, ctx, orc, n_tabs):
     """Rounds of few workgroups are launched during the round before and wait for their challenge.  Such a launch
     has changed nothing yet: when another call needs the context, or the caller is slow, it ends, and the session
     carries on with ordinary launches and the same messages."""
     import time
-    # 11 tables are several groups: launches of their own up to round 5 (a launch stays for the later rounds from
+    # 18 tables are several groups: launches of their own up to round 5 (a launch stays for the later rounds from
     # n - j + 1 <= 9 on).  4 tables are one group, whose rounds are resident from the first that fits 256 workgroups of 512
     # pairs (round 3 of 20): rounds 1 and 2 are launches, and the resident launches are queued during round 2.
     n, afters = (14, (1, 3, 4, 5)) if n_tabs > 7 else (20, (1, 2))
