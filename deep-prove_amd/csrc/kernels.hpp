@@ -276,9 +276,8 @@ __device__ __forceinline__ E2 fold1(E2 lo, E2 hi, E2 r) { return gl::add(lo, gl:
 __device__ __forceinline__ E2 fold1p(E2 lo, E2 hi, gl::E2P r) { return gl::fma(gl::sub(hi, lo), r, lo); }
 __device__ __forceinline__ E2 fold1_base(u64 lo, u64 hi, E2 r)
 {
-    E2 d = gl::mul_base(r, gl::sub(hi, lo));
-    d.c0 = gl::add(d.c0, lo);
-    return d;
+    const u64 d = gl::sub(hi, lo);
+    return gl::e2(gl::muladd(r.c0, d, lo), gl::mul(r.c1, d));
 }
 
 __device__ __forceinline__ void fold_body(const FoldDesc &d, E2 r)
@@ -822,11 +821,12 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             }
         }
     };
-    // one loop step on loaded operands
-    auto step = [&](u64 i, const Raw &w) {
-        E2 lo[NF], hi[NF];
-        // base-field arithmetic applies only while the sources are read unfolded
-        constexpr int NBE = FOLD ? 0 : NB;
+    // One loop step on loaded operands, in two parts: the first uses up the operands (and folds them), the second
+    // evaluates.  Between the two the fold kernels ask for the next step's operands, so that a wavefront's loads are
+    // in flight while it evaluates.
+    // base-field arithmetic applies only while the sources are read unfolded
+    constexpr int NBE = FOLD ? 0 : NB;
+    auto take = [&](u64 i, const Raw &w, E2 (&lo)[NF], E2 (&hi)[NF], E2 &rest) {
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             if (FOLD) {
@@ -849,12 +849,10 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 }
             }
         }
-        E2 rest = gl::e2_one();
-        gl::E2P restp = gl::prep(rest);
-        if (EQ) {
-            rest = gl::e2(w.q0, w.q1);
-            restp = gl::prep(rest);
-        }
+        rest = EQ ? gl::e2(w.q0, w.q1) : gl::e2_one();
+    };
+    auto evaluate = [&](const E2 (&lo)[NF], const E2 (&hi)[NF], E2 rest) {
+        const gl::E2P restp = gl::prep(rest);
         E2 dl[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) dl[f] = gl::sub(hi[f], lo[f]);
@@ -922,10 +920,17 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             rp = gl::prep(r);
         }
         for (; i < a.n_pairs; i += stride) {
-            step(i, w);
+            E2 lo[NF], hi[NF], rest;
+            take(i, w, lo, hi, rest);
             if (i + stride < a.n_pairs) load_raw(i + stride, w);
+            evaluate(lo, hi, rest);
         }
     } else {
+        auto step = [&](u64 i, const Raw &w) {
+            E2 lo[NF], hi[NF], rest;
+            take(i, w, lo, hi, rest);
+            evaluate(lo, hi, rest);
+        };
         // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
         Raw wa, wb;
         if (i < a.n_pairs) load_raw(i, wa);
@@ -2419,6 +2424,21 @@ field_op_kernel(int op, const u64 *__restrict__ a0, const u64 *__restrict__ a1, 
     case 3: r = gl::e2(gl::mul(a.c0, b.c0), gl::mul(a.c1, b.c1)); break;  // two independent base products
     case 4: r = gl::mul_base(a, b.c0); break;
     case 5: r = gl::e2(gl::from_i64((int64_t)a.c0), gl::mul_small(a.c1, (u32)b.c1)); break;
+    case 6: r = gl::fma(a, gl::prep(b), a); break;
+    case 7: r = gl::e2(gl::muladd(a.c0, b.c0, a.c1), gl::dot2(a.c0, b.c0, a.c1, b.c1, b.c0)); break;
+    case 8: {
+        // a long unreduced sum: 40 (a b + b a.c1 + a) + (0, 40 b.c0)
+        gl::E2Acc acc = gl::e2acc_zero();
+        const gl::E2P bp = gl::prep(b);
+        for (int k = 0; k < 40; k++) {
+            gl::acc_mul(acc, a, bp);
+            gl::acc_mul_base(acc, b, a.c1);
+            gl::acc_e2(acc, a);
+            gl::acc_add64(acc.c1, b.c0);
+        }
+        r = gl::acc_reduce(acc);
+        break;
+    }
     default: r = gl::e2_zero();
     }
     o0[i] = r.c0;

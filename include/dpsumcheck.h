@@ -226,7 +226,9 @@ const char *dps_kernel_name(int32_t kernel);
 /* ---- arithmetic self-check: element-wise field operations on device vectors ----
  * a, b, out: n c0 limbs followed by n c1 limbs.  op: 0 add, 1 sub, 2 extension
  * product, 3 two independent base products (c0*c0, c1*c1), 4 extension times
- * base (b.c0), 5 (embed int64 a.c0, a.c1 times the 32-bit constant b.c1). */
+ * base (b.c0), 5 (embed int64 a.c0, a.c1 times the 32-bit constant b.c1),
+ * 6 a b + a with one reduction per limb, 7 (a.c0 b.c0 + a.c1, a.c0 b.c0 + a.c1 b.c1 + b.c0)
+ * in the base field, 8 the unreduced sum 40 (a b + b a.c1 + a) + (0, 40 b.c0). */
 int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *a, const uint64_t *b, uint64_t n, uint64_t *out);
 
 /* ---- bandwidth yardstick: `reps` launches of a plain device-to-device copy of

@@ -39,7 +39,7 @@ def test_device_field_arithmetic(ctx):
     b1 = [b0[(i * 7 + 3) % len(b0)] for i in range(len(b0))]
     A = np.array(list(zip(a0, a1)), dtype=np.uint64)
     B = np.array(list(zip(b0, b1)), dtype=np.uint64)
-    got = {op: ctx.field_op(op, A, B) for op in range(5)}
+    got = {op: ctx.field_op(op, A, B) for op in (0, 1, 2, 3, 4, 6, 7, 8)}
     for i in range(len(a0)):
         x, y = E2(a0[i], a1[i]), E2(b0[i], b1[i])
         assert tuple(int(v) for v in got[0][i]) == (x + y).pair()
@@ -47,6 +47,11 @@ def test_device_field_arithmetic(ctx):
         assert tuple(int(v) for v in got[2][i]) == (x * y).pair()
         assert tuple(int(v) for v in got[3][i]) == (a0[i] * b0[i] % P, a1[i] * b1[i] % P)
         assert tuple(int(v) for v in got[4][i]) == (x * E2(b0[i])).pair()
+        # products gathered without a reduction per product: one product pair plus a term, and a long sum
+        assert tuple(int(v) for v in got[6][i]) == (x * y + x).pair()
+        assert tuple(int(v) for v in got[7][i]) == ((a0[i] * b0[i] + a1[i]) % P, (a0[i] * b0[i] + a1[i] * b1[i] + b0[i]) % P)
+        long_sum = E2(40) * (x * y + y * E2(a1[i]) + x) + E2(0, 40 * b0[i] % P)
+        assert tuple(int(v) for v in got[8][i]) == long_sum.pair()
     # int64 embedding and multiplication by a 32-bit constant
     ints = [0, 1, -1, 2047, -2048, 2**40, -(2**40), 2**62, -(2**62), -(2**63), 2**63 - 1]
     A = np.array([[x % 2**64, vals[i]] for i, x in enumerate(ints)], dtype=np.uint64)
