@@ -36,6 +36,7 @@ namespace {
 // 3 workgroups per CU on 256 CUs: measured best for the streaming kernels (each workgroup pays a fixed
 // reduction + ticket epilogue, so more, thinner workgroups lose more than they gain in latency hiding)
 constexpr u32 MAX_BLOCKS = 768;
+constexpr u32 PAIR12_BLOCKS = 1024;  // workgroups of the launch of the first two rounds (64 quads each: a stride of 2^16 quads)
 
 // ---------------------------------------------------------------------------
 // context
@@ -1472,6 +1473,7 @@ struct dps_sc {
     std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip)
     u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
     E2 prev_chal;                     // the challenge of the call before this one
+    bool pair12;                      // rounds 1 and 2 are one launch that writes nothing (pair12_kernel); round 3 folds twice on its way in
     E2 stash[dpk::SL_MAX_SUMS];       // a trip of two rounds: the second round's sums as a polynomial in the first round's challenge
     u64 last_trip_seq;
     u32 fin_len;                      // entries per table the last trip leaves to the host (2, or 4 after a trip of two rounds)
@@ -1620,6 +1622,16 @@ template <int NF, int NB, bool EQ>
 void launch_prod(dps_ctx *ctx, bool fold, const dpk::ProdArgs &a, u32 blocks, u64 *partial, const dpk::FastFin &ff)
 {
     if constexpr (EQ) {
+        if constexpr (NF == 2 && NB == 2) {
+            if (a.two) {
+                // (planned only where the weights come factored: plan_first_two_rounds)
+                if (a.skip1)
+                    dpk::prod_kernel<2, 2, true, true, true, true, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+                else
+                    dpk::prod_kernel<2, 2, true, true, false, true, true><<<blocks, dpk::BLOCK, 0, ctx->stream>>>(a, partial, ff);
+                return;
+            }
+        }
         if (a.lq0) {
             // large round: eq weights as a product of a small low table and a later level
             if (fold && a.skip1)
@@ -2008,6 +2020,7 @@ struct SessionSetup {
     void poly_groups_of_round(u32 j);
     void term_descs_of_round(u32 j);
     void describe_rounds();
+    void plan_first_two_rounds();
     void launch_limits();
     int32_t allocate_device_block();
     int32_t stage_descriptors();
@@ -2504,6 +2517,8 @@ void SessionSetup::describe_rounds()
 void SessionSetup::launch_limits()
 {
     sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
+    // (the launch of the first two rounds: 18 words a workgroup where the others have at most 16)
+    if (sc->pair12) sc->max_blocks = std::max<u32>(sc->max_blocks, (PAIR12_BLOCKS * 2 * dpk::PAIR12_SUMS + 2 * dpk::MAX_PTS - 1) / (2 * dpk::MAX_PTS));
     sc->poly_split_cap = 0;
     sc->poly_finish_in_kernel = false;
     if (sc->poly) {
@@ -2614,6 +2629,28 @@ int32_t SessionSetup::stage_descriptors()
     return DPS_OK;
 }
 
+// eq * f * g over two base-field tables, large enough for the factored eq weights: rounds 1 and 2 are one launch that
+// reads the tables once and writes nothing (pair12_kernel), and round 3 reads them again and folds twice on its way in.
+void SessionSetup::plan_first_two_rounds()
+{
+    sc->pair12 = false;
+    if (!sc->fast || sc->fast_eq < 0 || sc->fast_nf != 2 || n_mles != 3 || sc->fast_nb[1] != 2) return;
+    if (n_vars < dpk::EQ_LO_BITS + 3 || (sc->tail_j0 && sc->tail_j0 <= 3)) return;
+    if (!sc->eq_info->fact_built || sc->eq_info->fact_levels < 3) return;
+    if (((u64)blocks_for_pairs(1ull << (n_vars - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return;
+    // (round 2's p(1) comes from the claim: its scale must not vanish at 1)
+    const E2 rho2 = sc->eq_info->point[1];
+    if ((rho2.c0 == 0 && rho2.c1 == 0) || (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0)) return;
+    sc->pair12 = true;
+    dpk::ProdArgs &p3 = sc->fast_args[3];
+    for (u32 f = 0; f < 2; f++) {
+        p3.s0[f] = sc->fast_args[1].s0[f];
+        p3.s1[f] = nullptr;
+    }
+    p3.two = 1;
+    sc->fast_nb[3] = 2;
+}
+
 int32_t SessionSetup::run()
 {
     detect_product();
@@ -2621,6 +2658,7 @@ int32_t SessionSetup::run()
     CHK(plan_and_ready_tables());
     CHK(layout_scratch());
     describe_rounds();
+    plan_first_two_rounds();
     launch_limits();
     CHK(allocate_device_block());
     return stage_descriptors();
@@ -2856,6 +2894,8 @@ struct FusedRound {
     int32_t multi_term_round();
     int32_t product_launch_ahead();
     int32_t product_round();
+    int32_t first_two_rounds_launch();
+    int32_t second_round_from_stash();
 };
 
 
@@ -2873,6 +2913,8 @@ int32_t FusedRound::begin()
         const E2 r = gl::e2(challenge[0], challenge[1]);
         a.r0 = r.c0;
         a.r1 = r.c1;
+        a.ra0 = sc->prev_chal.c0;
+        a.ra1 = sc->prev_chal.c1;
         CHK(launch_folds(sc, j, true, challenge));
         if (has_eq) sc->eq_scalar = gl::mul(sc->eq_scalar, h_eq1(sc->eq_info->point[j - 2], r));
     }
@@ -3424,7 +3466,7 @@ int32_t FusedRound::product_round()
         double bytes = has_eq && !a.lq0 ? (double)n_pairs * 16.0 : 0.0;
         for (u32 f = 0; f < nf; f++) {
             double eb = a.s1[f] ? 16.0 : 8.0;
-            bytes += (j >= 2) ? (double)n_pairs * (4 * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
+            bytes += (j >= 2) ? (double)n_pairs * ((a.two ? 8 : 4) * eb + 2 * 16.0) : (double)n_pairs * 2 * eb;
         }
         ProfScope ps(ctx, j >= 2 ? DPS_K_FOLD_EVAL : DPS_K_EVAL_FIRST, bytes);
         a.wait_first = 0;
@@ -3441,6 +3483,71 @@ int32_t FusedRound::product_round()
         return rc;
     }
     if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
+    sc->round = j;
+    return DPS_OK;
+}
+
+// Round 1 of a session whose first two rounds are one launch: the launch, round 1's message, and round 2's sums kept as
+// a polynomial in the challenge to come.
+int32_t FusedRound::first_two_rounds_launch()
+{
+    dpk::Pair12Args pa;
+    pa.f = a.s0[0];
+    pa.g = a.s0[1];
+    pa.n_quads = n_pairs >> 1;
+    // the weights of round 2's pairs: low table of level 2, level 2 + 16
+    const u64 lo = eq_low_off(sc->n_vars, 2), hi = eq_level_off(sc->n_vars, 2 + dpk::EQ_LO_BITS);
+    pa.lq0 = sc->eq_c0 + lo;
+    pa.lq1 = sc->eq_c1 + lo;
+    pa.hq0 = sc->eq_c0 + hi;
+    pa.hq1 = sc->eq_c1 + hi;
+    ff.n_blocks = PAIR12_BLOCKS;
+    ff.slots = nullptr;
+    {
+        ProfScope ps(ctx, DPS_K_EVAL_FIRST, (double)n_pairs * 2 * 2 * 8.0);
+        dpk::pair12_kernel<<<PAIR12_BLOCKS, dpk::PAIR12_BLOCK, 0, ctx->stream>>>(pa, sc->d_partial, ff);
+        HIPCHK(ctx, hipGetLastError());
+    }
+    a.skip1 = 0;  // (every point of round 1 is computed: round 2 needs them as well)
+    skip1 = false;
+    prepare_message();
+    u64 w[2 * dpk::PAIR12_SUMS];
+    if (const int32_t rc = wait_result_at(ctx, ctx->res_off, fa.seq, 0, 2 * dpk::PAIR12_SUMS, w, dpk::PAIR12_SEQ_SLOT, dpk::PAIR12_CHK_SLOT);
+        rc != DPS_OK) {
+        sc->broken = true;
+        reset_device_words(ctx);
+        return rc;
+    }
+    // pair 0's three (value at 0, at 1, leading coefficient of the product along x0), pair 1's, those of round 2 at t = 2
+    for (u32 k = 0; k < (u32)dpk::PAIR12_SUMS; k++) sc->stash[k] = gl::e2(w[2 * k], w[2 * k + 1]);
+    // round 1 sums over the pairs of either kind, weighted by eq1(rho_2, x1); its q(2) = 2 q(1) - q(0) + 2 c
+    const E2 rho2 = sc->eq_info->point[1], n2 = gl::sub(gl::e2_one(), rho2);
+    E2 q[3];
+    for (u32 k = 0; k < 3; k++) q[k] = gl::add(gl::mul(n2, sc->stash[k]), gl::mul(rho2, sc->stash[3 + k]));
+    const E2 c = q[2];
+    q[2] = gl::add(gl::sub(gl::add(q[1], q[1]), q[0]), gl::add(c, c));
+    form_message(q);
+    sc->round = j;
+    return DPS_OK;
+}
+
+// Round 2 of such a session: nothing goes to the GPU.  Each of round 2's sums q(0), q(1), q(2) is a polynomial of degree 2
+// in round 1's challenge, known by its values at 0 and 1 and its leading coefficient; then round 3 is launched ahead.
+int32_t FusedRound::second_round_from_stash()
+{
+    const E2 r = gl::e2(challenge[0], challenge[1]);
+    const E2 rr = gl::mul(r, gl::sub(r, gl::e2_one()));
+    E2 q[3];
+    for (u32 t = 0; t < 3; t++) {
+        const E2 v0 = sc->stash[3 * t], v1 = sc->stash[3 * t + 1], lead = sc->stash[3 * t + 2];
+        q[t] = gl::add(gl::add(v0, gl::mul(r, gl::sub(v1, v0))), gl::mul(rr, lead));
+    }
+    prepare_message();
+    form_message(q);
+    sc->tail_running = false;
+    ctx->tail_owner = nullptr;
+    CHK(product_launch_ahead());
+    sc->prev_chal = r;
     sc->round = j;
     return DPS_OK;
 }
@@ -3491,6 +3598,8 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         fr.n_pairs = n_pairs, fr.blocks = blocks, fr.cst = cst, fr.fa = fa;
         CHK(fr.begin());
         if (sc->tail_j0 && j >= sc->tail_j0) return fr.resident_round();
+        if (sc->pair12 && j == 1) return fr.first_two_rounds_launch();
+        if (sc->pair12 && j == 2) return fr.second_round_from_stash();
         return sc->poly ? fr.multi_term_round() : fr.product_round();
     } else {
         if (j >= 2) CHK(launch_folds(sc, j, false, challenge));

@@ -6,6 +6,8 @@
 // once per round, reductions finished in registers/LDS with one partial per
 // workgroup, and grids sized to a few workgroups per CU.
 #pragma once
+#include <type_traits>
+
 #include "gl.hpp"
 
 namespace dpk {
@@ -662,6 +664,10 @@ __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, boo
 // FOLD = false: first round, the source pairs are evaluated as they are.
 // FOLD = true : source quads are folded with r, the folded pair is written and
 //               evaluated: every table is read once and written once per round.
+// TWO         : the sources are two rounds old (base-field tables nobody has folded yet: the first two rounds were
+//               one launch, pair12_kernel).  Eight source entries make a folded pair; an entry of it is the
+//               combination sum_ab e_a(ra) e_b(r) x[a + 2 b] of four of them, e_0(c) = 1 - c, e_1(c) = c: four
+//               products gathered unreduced and reduced once, which costs no more than one fold of a folded table.
 //
 // The eq factor is never folded or streamed as a table of this round's size.
 // After the variables below v are bound, eq(rho, .) restricted to the remaining
@@ -684,7 +690,9 @@ struct ProdArgs {
     const u64 *q1;
     u64 n_pairs;  // pairs evaluated this round
     u64 r0, r1;   // fold challenge
+    u64 ra0, ra1;  // TWO variants: the challenge of the round before that (a mail brings it as MAIL_RA)
     u32 skip1;    // 1: t = 1 is not evaluated (the launch picks the kernel variant accordingly)
+    u32 two;      // 1: the sources are two rounds old (the launch picks the TWO variant)
     // A launch made before its round began (wait_first): the challenge is not in r0, r1; the kernel waits for the mail
     // with the launch's sequence number and takes it from there.
     u32 wait_first;
@@ -767,10 +775,11 @@ __device__ __forceinline__ void publish_sums(u64 *out_host, u64 seq, u32 *counte
     }
 }
 
-template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT = false>
+template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT = false, bool TWO = false>
 __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict__ partial, FastFin ff)
 {
     static_assert(!FACT || EQ, "factored weights belong to the eq factor");
+    static_assert(!TWO || (FOLD && NB == NF), "two folds at once: from base-field sources only");
     constexpr int NP = NF + 1;
     __shared__ u32 lds[(BLOCK / WAVE) * 6 * NP];
     __shared__ int last_flag;
@@ -778,6 +787,13 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     __shared__ int ok_flag;
     E2 r = gl::e2(a.r0, a.r1);
     gl::E2P rp = gl::prep(r);
+    // TWO: the weights of a folded entry's four sources
+    E2 k2[4];
+    auto set_two = [&](E2 ra, E2 rb) {
+        const E2 na = gl::sub(gl::e2_one(), ra), nb = gl::sub(gl::e2_one(), rb);
+        k2[0] = gl::mul(na, nb), k2[1] = gl::mul(ra, nb), k2[2] = gl::mul(na, rb), k2[3] = gl::mul(ra, rb);
+    };
+    if (TWO) set_two(gl::e2(a.ra0, a.ra1), r);
     // a compile-time switch: as a run-time flag the compiler evaluates t = 1 anyway and discards it
     constexpr bool skip1 = SKIP1;
     // running sums, reduced once after the loop
@@ -792,12 +808,18 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     // their zeros and are never read.)
     struct Raw {
         U64x2 a0[NF] = {}, b0[NF] = {}, a1[NF] = {}, b1[NF] = {};
+        U64x2 c0[TWO ? NF : 1] = {}, e0[TWO ? NF : 1] = {};  // TWO: entries 4..7 of the eight
         u64 q0 = 0, q1 = 0;
     };
     auto load_raw = [&](u64 i, Raw &w) {
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            if (FOLD) {
+            if (TWO) {
+                w.a0[f] = ld2(a.s0[f] + 8 * i);
+                w.b0[f] = ld2(a.s0[f] + 8 * i + 2);
+                w.c0[f] = ld2(a.s0[f] + 8 * i + 4);
+                w.e0[f] = ld2(a.s0[f] + 8 * i + 6);
+            } else if (FOLD) {
                 w.a0[f] = ld2(a.s0[f] + 4 * i);
                 w.b0[f] = ld2(a.s0[f] + 4 * i + 2);
                 if (f >= NB) {
@@ -830,7 +852,18 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             if (FOLD) {
-                if (f < NB) {
+                if (TWO) {
+                    auto comb = [&](U64x2 u, U64x2 v) {
+                        gl::E2Acc t = gl::e2acc_zero();
+                        gl::acc_mul_base(t, k2[0], u.x);
+                        gl::acc_mul_base(t, k2[1], u.y);
+                        gl::acc_mul_base(t, k2[2], v.x);
+                        gl::acc_mul_base(t, k2[3], v.y);
+                        return gl::acc_reduce(t);
+                    };
+                    lo[f] = comb(w.a0[f], w.b0[f]);
+                    hi[f] = comb(w.c0[f], w.e0[f]);
+                } else if (f < NB) {
                     lo[f] = fold1_base(w.a0[f].x, w.a0[f].y, r);
                     hi[f] = fold1_base(w.b0[f].x, w.b0[f].y, r);
                 } else {
@@ -918,6 +951,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             // (kept in scalar registers, as the kernel argument would be)
             r = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
             rp = gl::prep(r);
+            if (TWO) set_two(gl::e2(uniform64(box[MAIL_RA]), uniform64(box[MAIL_RA + 1])), r);
         }
         for (; i < a.n_pairs; i += stride) {
             E2 lo[NF], hi[NF], rest;
@@ -978,6 +1012,162 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
         E2 q[NP];
         gather_partials<NP>(ff, lds, q);
         publish_sums<NP>(ff.out_host, ff.seq, ff.counter, q);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The first two rounds of eq(rho, x) f(x) g(x), f and g in the base field, from one pass over the tables.
+//
+// With the lowest variable x0 bound to a challenge c, a table's value at (c, x1, x') is linear in c, so round 2's sums
+// are a polynomial of degree 2 in the challenge round 1 has not drawn yet: the kernel hands over its values at c = 0, 1 and
+// its leading coefficient, and the host evaluates it when the challenge is there.  All of it is base-field arithmetic on
+// the entries as stored: a quad (f00, f10, f01, f11) = f[4 x' + x0 + 2 x1] and the same of g give, all weighted by
+// R(x') = eq(rho_3.., x'),
+//   pair x1 = 0:  f00 g00,  f10 g10,  (f10 - f00)(g10 - g00)       (round 1's q(0), q(1) and leading coefficient over the
+//   pair x1 = 1:  f01 g01,  f11 g11,  (f11 - f01)(g11 - g01)        pairs of either kind: the host weights them with
+//                                                                  1 - rho_2 and rho_2; and round 2 at t = 0, pair 0 alone)
+//   round 2 at t = 2, with F_a = 2 f_a1 - f_a0, G_a likewise:  F0 G0,  F1 G1,  (F1 - F0)(G1 - G0)
+// nine products where round 1 alone takes six, each row the same three products of a pair of values.  A workgroup is
+// three wavefronts that walk the same quads, one row each (three unreduced sums a lane, as in round 1's kernel; the
+// quad comes from HBM once and twice more from the caches).  R is taken as in the FACT variants of prod_kernel:
+// hi[x' >> 16], the same for a workgroup's step, weights the products; lo[x' & 0xFFFF], the same for all steps of a
+// lane (the grid's stride, 64 quads a workgroup, is a multiple of 2^16), weights the sums.  Round 3 then reads the same
+// tables again and folds them twice on the way in (prod_kernel's TWO variant): nothing is written for the first two rounds.
+// ---------------------------------------------------------------------------
+struct Pair12Args {
+    const u64 *f, *g;
+    u64 n_quads;
+    const u64 *lq0, *lq1, *hq0, *hq1;
+};
+constexpr int PAIR12_BLOCK = 3 * WAVE;
+constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's three, pair 1's three, the three of t = 2
+constexpr int PAIR12_SEQ_SLOT = 62, PAIR12_CHK_SLOT = 63;
+static_assert(2 * PAIR12_SUMS <= PAIR12_SEQ_SLOT, "the sums fit the result area");
+
+// sums over the wavefront of canonical values (as block_sum does it: 22-bit pieces added as integers), valid in lane 63
+template <int NV>
+__device__ __forceinline__ void wave_sum_field(u64 (&v)[NV])
+{
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const u32 lo = (u32)v[i], hi = (u32)(v[i] >> 32);
+        const u64 c0 = wave_sum_u32(lo & 0x3FFFFFu);
+        const u64 c1 = wave_sum_u32((lo >> 22) | ((hi & 0xFFFu) << 10));
+        const u64 c2 = wave_sum_u32(hi >> 12);
+        const unsigned __int128 t = (unsigned __int128)c0 + ((unsigned __int128)c1 << 22) + ((unsigned __int128)c2 << 44);
+        v[i] = gl::reduce128((u64)t, (u64)(t >> 64));
+    }
+}
+
+__global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 *__restrict__ partial, FastFin ff)
+{
+    __shared__ int last_flag;
+    gl::E2Acc lz[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) lz[k] = gl::e2acc_zero();
+    const u32 lane = threadIdx.x & (WAVE - 1);
+    const u32 row = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const u64 stride = (u64)gridDim.x * WAVE;
+    const u64 q0 = (u64)blockIdx.x * WAVE + lane;
+    // The loop, compiled once for rows 0 and 1 (their own pair: two loads) and once for row 2 (the whole quad, and the
+    // values at t = 2 made of it): a wavefront takes one or the other, no lane pays for both.
+    auto run = [&](auto last_row) {
+        constexpr bool ROW2 = decltype(last_row)::value;
+        struct Raw {
+            U64x2 f0 = {}, f1 = {}, g0 = {}, g1 = {};
+            u64 h0 = 0, h1 = 0;
+        };
+        auto load_raw = [&](u64 q, Raw &w) {
+            if (ROW2) {
+                w.f0 = ld2(a.f + 4 * q);
+                w.f1 = ld2(a.f + 4 * q + 2);
+                w.g0 = ld2(a.g + 4 * q);
+                w.g1 = ld2(a.g + 4 * q + 2);
+            } else {
+                w.f0 = ld2(a.f + 4 * q + 2 * row);
+                w.g0 = ld2(a.g + 4 * q + 2 * row);
+            }
+            // the same entry for the whole workgroup (its 64 quads lie within one run of 2^16)
+            const u32 hi = __builtin_amdgcn_readfirstlane((u32)(q >> EQ_LO_BITS));
+            w.h0 = a.hq0[hi];
+            w.h1 = a.hq1[hi];
+        };
+        auto step = [&](const Raw &w) {
+            const E2 H = gl::e2(w.h0, w.h1);
+            u64 fl = w.f0.x, fh = w.f0.y, gl_ = w.g0.x, gh = w.g0.y;
+            if (ROW2) {
+                // t = 2 of round 2: 2 (x1 = 1) - (x1 = 0), at x0 = 0 and at x0 = 1
+                fl = gl::add(w.f1.x, gl::sub(w.f1.x, w.f0.x));
+                fh = gl::add(w.f1.y, gl::sub(w.f1.y, w.f0.y));
+                gl_ = gl::add(w.g1.x, gl::sub(w.g1.x, w.g0.x));
+                gh = gl::add(w.g1.y, gl::sub(w.g1.y, w.g0.y));
+            }
+            gl::acc_mul_base(lz[0], H, gl::mul(fl, gl_));
+            gl::acc_mul_base(lz[1], H, gl::mul(fh, gh));
+            gl::acc_mul_base(lz[2], H, gl::mul(gl::sub(fh, fl), gl::sub(gh, gl_)));
+        };
+        // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
+        u64 q = q0;
+        Raw wa, wb;
+        if (q < a.n_quads) load_raw(q, wa);
+        while (q < a.n_quads) {
+            if (q + stride < a.n_quads) load_raw(q + stride, wb);
+            step(wa);
+            q += stride;
+            if (q >= a.n_quads) break;
+            if (q + stride < a.n_quads) load_raw(q + stride, wa);
+            step(wb);
+            q += stride;
+        }
+    };
+    if (row == 2)
+        run(std::true_type{});
+    else
+        run(std::false_type{});
+    // the low part of the weight, then the wavefront's three sums: words 6 row .. 6 row + 5 of the workgroup's 18
+    const u32 lo = (u32)q0 & ((1u << EQ_LO_BITS) - 1);
+    const gl::E2P lp = gl::prep(gl::e2(a.lq0[lo], a.lq1[lo]));
+    u64 v[6];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        const E2 x = q0 < a.n_quads ? gl::mulp(gl::acc_reduce(lz[k]), lp) : gl::e2_zero();
+        v[2 * k] = x.c0, v[2 * k + 1] = x.c1;
+    }
+    wave_sum_field<6>(v);
+    auto publish = [&](const u64 *w) {
+        if (ff.counter) *ff.counter = 0;
+        publish_words(ff.out_host, 0, w, 2 * PAIR12_SUMS, ff.seq, PAIR12_SEQ_SLOT, PAIR12_CHK_SLOT);
+    };
+    __shared__ u64 own[2 * PAIR12_SUMS];
+    if (gridDim.x == 1) {
+        if (lane == WAVE - 1)
+#pragma unroll
+            for (int k = 0; k < 6; k++) own[6 * row + k] = v[k];
+        __syncthreads();
+        if (threadIdx.x == 0) publish(own);
+        return;
+    }
+    if (lane == WAVE - 1) {
+        u64 *o = partial + blockIdx.x;
+        const u64 total = gridDim.x;
+#pragma unroll
+        for (int k = 0; k < 6; k++) st_agent(o + (u64)(6 * row + k) * total, v[k]);
+    }
+    // (every wavefront's stores acknowledged before the workgroup's ticket is taken)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (take_ticket(ff.counter, gridDim.x, &last_flag) && row == 0) {
+        // the last workgroup's first wavefront adds up the workgroups' words
+        u64 s[2 * PAIR12_SUMS];
+#pragma unroll
+        for (int k = 0; k < 2 * PAIR12_SUMS; k++) s[k] = 0;
+        for (u32 b = lane; b < gridDim.x; b += WAVE) {
+#pragma unroll
+            for (int k = 0; k < 2 * PAIR12_SUMS; k++) s[k] = gl::add(s[k], ld_agent(partial + (u64)k * gridDim.x + b));
+        }
+        wave_sum_field<2 * PAIR12_SUMS>(s);
+        if (lane == WAVE - 1) publish(s);
     }
 }
 
