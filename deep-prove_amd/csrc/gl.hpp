@@ -46,7 +46,9 @@ GL_FN u64 add(u64 a, u64 b)
 #if GL_LIMBS
 GL_FN u64 pack(u32 lo, u32 hi) { return ((u64)hi << 32) | lo; }
 
-// l0 + 2^32 l1 + 2^64 l2 + 2^96 l3 + 2^128 l4 mod p (l4 < 2^31), canonical: (l0, l1) - (l3, l4) + l2 (2^32 - 1)
+// l0 + 2^32 l1 + 2^64 l2 + 2^96 l3 + 2^128 l4 mod p (l4 < 2^31): (l0, l1) - (l3, l4) + l2 (2^32 - 1); canonical, or
+// (CANON = false) any representative below 2^64, for values that only go into further products
+template <bool CANON = true>
 GL_FN u64 reduce160(u32 l0, u32 l1, u32 l2, u32 l3, u32 l4)
 {
     u32 b, c;
@@ -65,6 +67,7 @@ GL_FN u64 reduce160(u32 l0, u32 l1, u32 l2, u32 l3, u32 l4)
     m = 0u - c;
     r0 = __builtin_addc(r0, m, 0u, &c);
     r1 = __builtin_addc(r1, 0u, c, &c);
+    if (!CANON) return pack(r0, r1);
     // r >= p exactly when r + EPS wraps, and r - p is that wrapped sum
     u32 s0 = __builtin_addc(r0, 0xFFFFFFFFu, 0u, &c);
     u32 s1 = __builtin_addc(r1, 0u, c, &c);
@@ -116,6 +119,17 @@ GL_FN u64 mul(u64 a, u64 b)
 {
     u128 p = (u128)a * b;
     return reduce128((u64)p, (u64)(p >> 64));
+}
+
+// a b mod p as any representative below 2^64 (not canonical): for a product that only goes into further products
+GL_FN u64 mul_any(u64 a, u64 b)
+{
+#if GL_LIMBS
+    const u128 p = (u128)a * b;
+    return reduce160<false>((u32)p, (u32)(p >> 32), (u32)(p >> 64), (u32)(p >> 96), 0u);
+#else
+    return mul(a, b);
+#endif
 }
 
 // a * small constant (c < 2^32)

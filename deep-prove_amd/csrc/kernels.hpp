@@ -899,7 +899,7 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
                 if (NBE > 0) {
                     u64 b = cur[0].c0;
 #pragma unroll
-                    for (int f = 1; f < NBE; f++) b = gl::mul(b, cur[f].c0);
+                    for (int f = 1; f < NBE; f++) b = (NBE == NF && EQ) ? gl::mul_any(b, cur[f].c0) : gl::mul(b, cur[f].c0);
                     if (NBE == NF) {
                         if (EQ)
                             gl::acc_mul_base(lz[t], rest, b);
@@ -1102,9 +1102,9 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
                 gl_ = gl::add(w.g1.x, gl::sub(w.g1.x, w.g0.x));
                 gh = gl::add(w.g1.y, gl::sub(w.g1.y, w.g0.y));
             }
-            gl::acc_mul_base(lz[0], H, gl::mul(fl, gl_));
-            gl::acc_mul_base(lz[1], H, gl::mul(fh, gh));
-            gl::acc_mul_base(lz[2], H, gl::mul(gl::sub(fh, fl), gl::sub(gh, gl_)));
+            gl::acc_mul_base(lz[0], H, gl::mul_any(fl, gl_));
+            gl::acc_mul_base(lz[1], H, gl::mul_any(fh, gh));
+            gl::acc_mul_base(lz[2], H, gl::mul_any(gl::sub(fh, fl), gl::sub(gh, gl_)));
         };
         // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
         u64 q = q0;

@@ -5,8 +5,9 @@
 // from the sums worked out here with plain loops.  tests/test_kernel_emulation.py builds and runs the quick set; the
 // full set (no argument) takes a few minutes, most of it thread hand-offs.  Covers every way the kernel hands over
 // its result (single workgroup, per-workgroup result areas, partials + ticket + gather), both evaluation modes, the
-// eq weights streamed and taken from two small tables, and a launch that waits for its challenge by mail (directly
-// and through the relay).
+// eq weights streamed and taken from two small tables, a launch that waits for its challenge by mail (directly
+// and through the relay), the variant that folds its sources twice on the way in, and the kernel of the first two
+// rounds (pair12_kernel).
 #include <chrono>
 #include <thread>
 #include <vector>
@@ -36,14 +37,14 @@ static u64 felt()
 }
 
 template <class K, class... A>
-static void launch(u32 blocks, K kernel, A... args)
+static void launch_threads(u32 blocks, u32 threads, K kernel, A... args)
 {
     gridDim = dim3(blocks);
-    blockDim = dim3(dpk::BLOCK);
+    blockDim = dim3(threads);
     for (u32 b = 0; b < blocks; b++) {
-        emu::default_group.reset(dpk::BLOCK);
+        emu::default_group.reset(threads);
         std::vector<std::thread> th;
-        for (u32 t = 0; t < (u32)dpk::BLOCK; t++)
+        for (u32 t = 0; t < threads; t++)
             th.emplace_back([=] {
                 threadIdx = dim3(t);
                 blockIdx = dim3(b);
@@ -51,6 +52,11 @@ static void launch(u32 blocks, K kernel, A... args)
             });
         for (auto &x : th) x.join();
     }
+}
+template <class K, class... A>
+static void launch(u32 blocks, K kernel, A... args)
+{
+    launch_threads(blocks, dpk::BLOCK, kernel, args...);
 }
 
 static int failures = 0;
@@ -63,12 +69,13 @@ struct Case {
     int wait;         // 0: challenge in the arguments, 1: by mail, every workgroup polling, 2: by mail through the relay
 };
 
-template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT>
+// TWO: the sources are two rounds old and are folded with `ra`, then with `r`, on the way in
+template <int NF, int NB, bool FOLD, bool EQ, bool SKIP1, bool FACT, bool TWO = false>
 static void run_case(const Case &c)
 {
     constexpr int NP = NF + 1;
     const u64 np = c.n_pairs;
-    const u64 src_len = FOLD ? 4 * np : 2 * np;
+    const u64 src_len = TWO ? 8 * np : FOLD ? 4 * np : 2 * np;
     std::vector<std::vector<u64>> s0(NF), s1(NF), d0(NF), d1(NF);
     for (int f = 0; f < NF; f++) {
         s0[f].resize(src_len);
@@ -100,7 +107,7 @@ static void run_case(const Case &c)
         for (auto &x : q0) x = felt();
         for (auto &x : q1) x = felt();
     }
-    const E2 r = gl::e2(felt(), felt());
+    const E2 r = gl::e2(felt(), felt()), ra = gl::e2(felt(), felt());
 
     // what the launch has to produce, by plain loops
     E2 want[NP];
@@ -110,7 +117,14 @@ static void run_case(const Case &c)
         E2 lo[NF], hi[NF];
         for (int f = 0; f < NF; f++) {
             auto at = [&](u64 k) { return gl::e2(s0[f][k], f >= NB ? s1[f][k] : 0); };
-            if (FOLD) {
+            if (TWO) {
+                auto once = [&](u64 k) { return gl::add(at(k), gl::mul(ra, gl::sub(at(k + 1), at(k)))); };
+                auto twice = [&](u64 k) { return gl::add(once(k), gl::mul(r, gl::sub(once(k + 2), once(k)))); };
+                lo[f] = twice(8 * i);
+                hi[f] = twice(8 * i + 4);
+                folded[f][2 * i] = lo[f];
+                folded[f][2 * i + 1] = hi[f];
+            } else if (FOLD) {
                 lo[f] = gl::add(at(4 * i), gl::mul(r, gl::sub(at(4 * i + 1), at(4 * i))));
                 hi[f] = gl::add(at(4 * i + 2), gl::mul(r, gl::sub(at(4 * i + 3), at(4 * i + 2))));
                 folded[f][2 * i] = lo[f];
@@ -162,6 +176,8 @@ static void run_case(const Case &c)
             std::this_thread::sleep_for(std::chrono::milliseconds(30));
             mail[dpk::MAIL_R] = r.c0;
             mail[dpk::MAIL_R + 1] = r.c1;
+            mail[dpk::MAIL_RA] = ra.c0;
+            mail[dpk::MAIL_RA + 1] = ra.c1;
             mail[dpk::MAIL_SKIP1] = SKIP1;
             u64 chk = seq;
             for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
@@ -170,8 +186,10 @@ static void run_case(const Case &c)
         });
     } else {
         a.r0 = r.c0, a.r1 = r.c1;
+        a.ra0 = ra.c0, a.ra1 = ra.c1;
     }
-    launch(c.blocks, dpk::prod_kernel<NF, NB, FOLD, EQ, SKIP1, FACT>, a, partial.data(), ff);
+    a.two = TWO;
+    launch(c.blocks, dpk::prod_kernel<NF, NB, FOLD, EQ, SKIP1, FACT, TWO>, a, partial.data(), ff);
     if (host.joinable()) host.join();
 
     E2 got[NP];
@@ -192,10 +210,50 @@ static void run_case(const Case &c)
     if (FOLD)
         for (int f = 0; f < NF && ok; f++)
             for (u64 k = 0; k < 2 * np && ok; k++) ok = d0[f][k] == folded[f][k].c0 && d1[f][k] == folded[f][k].c1;
-    printf("%-58s NF=%d NB=%d fold=%d eq=%d skip1=%d fact=%d pairs=%llu workgroups=%u : %s\n", c.name, NF, NB, (int)FOLD, (int)EQ, (int)SKIP1, (int)FACT,
-           (unsigned long long)np, c.blocks, ok ? "ok" : "MISMATCH");
+    printf("%-58s NF=%d NB=%d fold=%d eq=%d skip1=%d fact=%d two=%d pairs=%llu workgroups=%u : %s\n", c.name, NF, NB, (int)FOLD, (int)EQ, (int)SKIP1,
+           (int)FACT, (int)TWO, (unsigned long long)np, c.blocks, ok ? "ok" : "MISMATCH");
     // the sums are printed so that builds with different fills for uninitialised locals can be compared
     for (int t = 0; t < NP; t++) printf("    q(%d) = %016llx %016llx\n", t, (unsigned long long)got[t].c0, (unsigned long long)got[t].c1);
+    if (!ok) failures++;
+}
+
+// pair12_kernel: the nine sums of the first two rounds of eq * f * g against plain loops over the quads.  With more than one
+// step a lane the grid's stride has to be a multiple of 2^16 quads (1024 workgroups), as in the library's launches.
+static void run_first_two_rounds(const char *name, u64 n_quads, u32 blocks)
+{
+    std::vector<u64> f(4 * n_quads), g(4 * n_quads), lq0(65536), lq1(65536), hq0((n_quads + 65535) >> 16), hq1(hq0.size());
+    for (auto *v : {&f, &g, &lq0, &lq1, &hq0, &hq1})
+        for (auto &x : *v) x = felt();
+    E2 want[dpk::PAIR12_SUMS];
+    for (auto &w : want) w = gl::e2_zero();
+    for (u64 q = 0; q < n_quads; q++) {
+        const E2 w = gl::mul(gl::e2(hq0[q >> 16], hq1[q >> 16]), gl::e2(lq0[q & 65535], lq1[q & 65535]));
+        const u64 *a = &f[4 * q], *b = &g[4 * q];
+        auto three = [&](int row, u64 fl, u64 fh, u64 gl_, u64 gh) {
+            const u64 v[3] = {gl::mul(fl, gl_), gl::mul(fh, gh), gl::mul(gl::sub(fh, fl), gl::sub(gh, gl_))};
+            for (int k = 0; k < 3; k++) want[3 * row + k] = gl::add(want[3 * row + k], gl::mul_base(w, v[k]));
+        };
+        three(0, a[0], a[1], b[0], b[1]);
+        three(1, a[2], a[3], b[2], b[3]);
+        auto at2 = [](u64 lo, u64 hi) { return gl::sub(gl::add(hi, hi), lo); };
+        three(2, at2(a[0], a[2]), at2(a[1], a[3]), at2(b[0], b[2]), at2(b[1], b[3]));
+    }
+    dpk::Pair12Args pa;
+    pa.f = f.data(), pa.g = g.data(), pa.n_quads = n_quads;
+    pa.lq0 = lq0.data(), pa.lq1 = lq1.data(), pa.hq0 = hq0.data(), pa.hq1 = hq1.data();
+    std::vector<u64> out_host(64, 0), partial(2 * dpk::PAIR12_SUMS * (size_t)blocks + 64, 0);
+    u32 counter = 0;
+    const u64 seq = 91;
+    dpk::FastFin ff;
+    memset(&ff, 0, sizeof ff);
+    ff.partial = partial.data(), ff.n_blocks = blocks, ff.out_host = out_host.data(), ff.seq = seq, ff.counter = &counter;
+    launch_threads(blocks, dpk::PAIR12_BLOCK, dpk::pair12_kernel, pa, partial.data(), ff);
+    u64 chk = seq;
+    for (int k = 0; k < 2 * dpk::PAIR12_SUMS; k++) chk ^= dpk::rotl64(out_host[k], k + 1);
+    bool ok = out_host[dpk::PAIR12_SEQ_SLOT] == seq && out_host[dpk::PAIR12_CHK_SLOT] == chk && counter == 0;
+    for (int k = 0; k < dpk::PAIR12_SUMS; k++) ok = ok && gl::eq(gl::e2(out_host[2 * k], out_host[2 * k + 1]), want[k]);
+    printf("%-58s quads=%llu workgroups=%u : %s\n", name, (unsigned long long)n_quads, blocks, ok ? "ok" : "MISMATCH");
+    for (int k = 0; k < dpk::PAIR12_SUMS; k++) printf("    sum %d = %016llx %016llx\n", k, (unsigned long long)out_host[2 * k], (unsigned long long)out_host[2 * k + 1]);
     if (!ok) failures++;
 }
 
@@ -218,8 +276,16 @@ int main(int argc, char **argv)
     // the challenge arrives by mail: every workgroup polls / the first one relays it
     run_case<2, 0, true, false, true, false>({"launch made ahead, every workgroup polls the mailbox", 1200, 3, true, 1});
     run_case<2, 2, true, false, true, false>({"launch made ahead, mail relayed by the first workgroup", 4500, 18, false, 2});
+    // sources folded twice on the way in (round 3 behind the launch of the first two rounds): challenges in the arguments, by mail
+    run_case<2, 2, true, false, true, false, true>({"two folds on the way in", 700, 3, false, 0});
+    run_case<2, 2, true, false, false, false, true>({"two folds on the way in, t = 1 evaluated, by mail", 300, 2, true, 1});
+    // the first two rounds from one pass: one workgroup, several (ticket and gather by the first wavefront)
+    run_first_two_rounds("first two rounds, one workgroup", 50, 1);
+    run_first_two_rounds("first two rounds, ragged quads, five workgroups", 300, 5);
     // eq weights as a product of two small tables (the grid's stride is a multiple of 2^16 pairs)
     if (!quick) {
+        run_first_two_rounds("first two rounds, two steps a lane", (1ull << 16) + 1000, 1024);
+        run_case<2, 2, true, true, true, true, true>({"two folds on the way in, eq weights from two small tables", 1ull << 16, 256, false, 0});
         run_case<2, 2, false, true, false, true>({"first round, eq weights from two small tables", 3ull << 16, 256, false, 0});
         run_case<2, 2, true, true, true, true>({"fold, eq weights from two small tables", 1ull << 17, 256, false, 0});
     }

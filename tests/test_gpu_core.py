@@ -343,6 +343,39 @@ def test_large_rounds_take_eq_weights_from_two_small_tables(dp, ctx, orc, n, kin
     _check_prove(dp, ctx, orc, n, tabs_gpu, tabs_ref, [(np.array([7, 3], dtype=np.uint64), [e] + list(range(e)))])
 
 
+@pytest.mark.parametrize("n,zero_at", [(21, None), (21, 0), (21, 1), (21, 2), (22, 3), (20, None)])
+def test_first_two_rounds_in_one_launch(dp, ctx, orc, n, zero_at):
+    """eq * f * g over base-field tables of 21 variables and more (with fewer, round 3 is already one of the resident
+    rounds): one launch reads the tables once for rounds 1 and 2 (round 2's sums as a polynomial in round 1's challenge)
+    and writes nothing, round 3 folds the tables twice on its way in.  An eq point with a zero coordinate in round 1, in
+    round 2 (then the ordinary launches take the session: round 2's value at 1 cannot come from the claim), in round 3
+    (which then evaluates at 1 itself) and in a later round; the same proof when the caller states the sum, and when the
+    session is driven round by round with another call on the context after round 2."""
+    f, g = rand_base(1 << n, 8300 + n), rand_base(1 << n, 8301 + n)
+    r = rand_e2(n, 8302 + n)
+    if zero_at is not None:
+        r[zero_at] = 0
+    gpu = [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(r)]
+    ref = [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(r)]
+    terms = [(np.array([5, 11], dtype=np.uint64), [0, 2, 1])]
+    want = orc.sc_prove(n, ref, terms, orc.OracleTranscript(b"two"))
+    got = ctx.sumcheck_prove(n, gpu, terms, dp.Transcript(b"two"))
+    assert all((a == b).all() for a, b in zip(got, want))
+    # the sum stated by the caller
+    p1 = to_E2(want[0][0])
+    again = ctx.sumcheck_prover(n, gpu, terms, claim=from_E2([p1[0] + p1[1]])[0])(dp.Transcript(b"two"))
+    assert all((a == b).all() for a, b in zip(again, want))
+    # round by round; after round 2 another call ends the launch made ahead for round 3, which is then launched again
+    s = ctx.session(n, gpu, terms)
+    chal = None
+    for j in range(n):
+        assert (s.round(chal) == want[0][j]).all(), j
+        chal = want[1][j]
+        if j == 1 and n >= 21:
+            assert (ctx.eq_build(want[1][:3]).download() == orc.eq_evals(want[1][:3])).all()
+    assert (s.finish(chal) == want[2]).all()
+
+
 def test_prepared_prover_gives_the_same_proofs(dp, ctx, orc):
     """sumcheck_prover marshals handles and terms once; each call is the proof sumcheck_prove gives."""
     n = 11
