@@ -81,6 +81,8 @@ dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
 dev.dps_debug_read.restype = _i32
 dev.dps_debug_read.argtypes = [_vp, _u64, _u32, _vp]
+dev.dps_debug_issue_cost.restype = _i32
+dev.dps_debug_issue_cost.argtypes = [_vp, _i32, _u32, _u32, _vp, _vp, _vp, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
            "dps_partial_eval", "dps_sc_begin", "dps_sc_set_claim", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
@@ -566,6 +568,19 @@ def _read_ms(self, n_bytes, reps=10):
 
 
 Context.read_ms = _read_ms
+
+
+def _issue_cost(self, kind, iters=4000, waves_per_simd=8):
+    """(name, ms, clock in MHz, compute units) of a launch of `iters` x 32 vector instructions of one kind per wavefront
+    (dps_debug_issue_cost)"""
+    ms, name, khz, cus = C.c_double(0), C.c_char_p(), C.c_int32(0), C.c_int32(0)
+    self._chk(dev.dps_debug_issue_cost(self._c, kind, iters, waves_per_simd, C.byref(ms), C.byref(name), C.byref(khz), C.byref(cus)),
+              "dps_debug_issue_cost")
+    return name.value.decode(), ms.value, khz.value / 1e3, cus.value
+
+
+Context.issue_cost = _issue_cost
+ISSUE_COST_KINDS = 10
 
 
 # ---- einsum and LogUp drivers of the host mirror ----

@@ -4059,3 +4059,52 @@ extern "C" int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps,
     if (avg_ms_out) *avg_ms_out = (double)ms / reps;
     return DPS_OK;
 }
+
+// ---------------------------------------------------------------------------
+// what a vector instruction costs to issue (see issue_cost_kernel): the duration of a launch of `iters` iterations of
+// 32 instructions of one kind, at `waves_per_simd` wavefronts on every SIMD of the device
+// ---------------------------------------------------------------------------
+extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t iters, uint32_t waves_per_simd, double *ms_out, const char **name_out,
+                                        int32_t *clock_khz_out, int32_t *compute_units_out)
+{
+    static const char *const names[dpk::ISSUE_COST_KINDS] = {"v_mov_b32", "v_add_u32", "v_add_co_u32", "v_add_co_u32 + v_addc_co_u32 (a pair, 2 wait states between)",
+                                                            "v_cmp_lt_u64", "v_lshl_add_u64", "v_mad_u64_u32 (running sum, carry out)", "v_mul_hi_u32", "v_add3_u32",
+                                                            "v_sub_co_u32 + v_cndmask_b32 (a pair, 2 wait states between)"};
+    if (!ctx || kind < 0 || kind >= dpk::ISSUE_COST_KINDS || iters == 0 || waves_per_simd == 0 || waves_per_simd > 8)
+        return fail(ctx, DPS_ERR_INVALID, "dps_debug_issue_cost: bad argument");
+    DeviceGuard g(ctx->device);
+    tail_abort(ctx);
+    hipDeviceProp_t prop;
+    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    // a workgroup is one wavefront on each of a compute unit's four SIMDs
+    const u32 blocks = (u32)prop.multiProcessorCount * waves_per_simd;
+    void *p = nullptr;
+    CHK(pool_alloc(ctx, (size_t)blocks * dpk::BLOCK * 8, &p));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    float best = 0.f;
+    for (int rep = 0; rep < 3 && e == hipSuccess; rep++) {
+        e = hipEventRecord(e0, ctx->stream);
+        switch (kind) {
+#define IC(K) case K: dpk::issue_cost_kernel<K><<<blocks, dpk::BLOCK, 0, ctx->stream>>>((u64 *)p, iters); break;
+            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9)
+#undef IC
+        }
+        if (e == hipSuccess) e = hipGetLastError();
+        if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (rep == 0 || ms < best) best = ms;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    pool_free(ctx, p);
+    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "issue cost: %s", hipGetErrorString(e));
+    if (ms_out) *ms_out = (double)best;
+    if (name_out) *name_out = names[kind];
+    if (clock_khz_out) *clock_khz_out = prop.clockRate;
+    if (compute_units_out) *compute_units_out = prop.multiProcessorCount;
+    return DPS_OK;
+}
