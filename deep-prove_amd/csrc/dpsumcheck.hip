@@ -4069,7 +4069,9 @@ extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t ite
 {
     static const char *const names[dpk::ISSUE_COST_KINDS] = {"v_mov_b32", "v_add_u32", "v_add_co_u32", "v_add_co_u32 + v_addc_co_u32 (a pair, 2 wait states between)",
                                                             "v_cmp_lt_u64", "v_lshl_add_u64", "v_mad_u64_u32 (running sum, carry out)", "v_mul_hi_u32", "v_add3_u32",
-                                                            "v_sub_co_u32 + v_cndmask_b32 (a pair, 2 wait states between)"};
+                                                            "v_sub_co_u32 + v_cndmask_b32 of constants (a pair, 2 wait states between)",
+                                                            "v_cmp_lt_u32 + v_cndmask_b32 of registers (a pair, 2 wait states between)",
+                                                            "v_cndmask_b32 of registers (the mask not written in the loop)", "v_and_b32 / v_xor_b32 / v_or_b32 / v_sub_u32"};
     if (!ctx || kind < 0 || kind >= dpk::ISSUE_COST_KINDS || iters == 0 || waves_per_simd == 0 || waves_per_simd > 8)
         return fail(ctx, DPS_ERR_INVALID, "dps_debug_issue_cost: bad argument");
     DeviceGuard g(ctx->device);
@@ -4088,7 +4090,7 @@ extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t ite
         e = hipEventRecord(e0, ctx->stream);
         switch (kind) {
 #define IC(K) case K: dpk::issue_cost_kernel<K><<<blocks, dpk::BLOCK, 0, ctx->stream>>>((u64 *)p, iters); break;
-            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9)
+            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9) IC(10) IC(11) IC(12)
 #undef IC
         }
         if (e == hipSuccess) e = hipGetLastError();
