@@ -580,7 +580,7 @@ def _issue_cost(self, kind, iters=4000, waves_per_simd=8):
 
 
 Context.issue_cost = _issue_cost
-ISSUE_COST_KINDS = 13
+ISSUE_COST_KINDS = 18
 
 
 # ---- einsum and LogUp drivers of the host mirror ----

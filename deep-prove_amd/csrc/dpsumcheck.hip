@@ -4071,7 +4071,11 @@ extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t ite
                                                             "v_cmp_lt_u64", "v_lshl_add_u64", "v_mad_u64_u32 (running sum, carry out)", "v_mul_hi_u32", "v_add3_u32",
                                                             "v_sub_co_u32 + v_cndmask_b32 of constants (a pair, 2 wait states between)",
                                                             "v_cmp_lt_u32 + v_cndmask_b32 of registers (a pair, 2 wait states between)",
-                                                            "v_cndmask_b32 of registers (the mask not written in the loop)", "v_and_b32 / v_xor_b32 / v_or_b32 / v_sub_u32"};
+                                                            "v_cndmask_b32 of registers (the mask not written in the loop)", "v_and_b32 / v_xor_b32 / v_or_b32 / v_sub_u32",
+                                                            "v_cmp_lt_u32 + three v_cndmask_b32 of registers", "v_cndmask_b32 of registers, mask set by s_mov_b64 every four",
+                                                            "v_cndmask_b32 of registers, mask in s[2:3], never written",
+                                                            "v_cmp_lt_u32 into s[2:3] + three v_cndmask_b32 of registers by s[2:3]",
+                                                            "v_cmp_lt_u32 + two v_cndmask_b32 of registers by vcc (a 64-bit select)"};
     if (!ctx || kind < 0 || kind >= dpk::ISSUE_COST_KINDS || iters == 0 || waves_per_simd == 0 || waves_per_simd > 8)
         return fail(ctx, DPS_ERR_INVALID, "dps_debug_issue_cost: bad argument");
     DeviceGuard g(ctx->device);
@@ -4090,7 +4094,7 @@ extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t ite
         e = hipEventRecord(e0, ctx->stream);
         switch (kind) {
 #define IC(K) case K: dpk::issue_cost_kernel<K><<<blocks, dpk::BLOCK, 0, ctx->stream>>>((u64 *)p, iters); break;
-            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9) IC(10) IC(11) IC(12)
+            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9) IC(10) IC(11) IC(12) IC(13) IC(14) IC(15) IC(16) IC(17)
 #undef IC
         }
         if (e == hipSuccess) e = hipGetLastError();

@@ -2658,7 +2658,7 @@ __global__ __launch_bounds__(BLOCK) void read_kernel(const uint4 *__restrict__ s
 // feeding each other round), run at a chosen number of wavefronts per SIMD.  The arithmetic of gl.hpp is written for
 // what this measures; no counterpart in the reference.
 // ---------------------------------------------------------------------------
-constexpr int ISSUE_COST_KINDS = 13;
+constexpr int ISSUE_COST_KINDS = 18;
 constexpr int ISSUE_COST_COPIES = 32;
 #define DPK_R8(x) x x x x x x x x
 template <int KIND>
@@ -2693,6 +2693,21 @@ __global__ void __launch_bounds__(BLOCK) issue_cost_kernel(u64 *out, u32 iters)
                          : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
         if (KIND == 11)
             asm volatile(DPK_R8("v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
+                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
+        if (KIND == 13)
+            asm volatile(DPK_R8("v_cmp_lt_u32 vcc, %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n")
+                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
+        if (KIND == 14)
+            asm volatile(DPK_R8("s_mov_b64 vcc, s[2:3]\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
+                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
+        if (KIND == 15)
+            asm volatile(DPK_R8("v_cndmask_b32 %0, %1, %2, s[2:3]\n v_cndmask_b32 %1, %2, %3, s[2:3]\n v_cndmask_b32 %2, %3, %0, s[2:3]\n v_cndmask_b32 %3, %0, %1, s[2:3]\n")
+                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+        if (KIND == 16)
+            asm volatile(DPK_R8("v_cmp_lt_u32 s[2:3], %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, s[2:3]\n v_cndmask_b32 %1, %2, %3, s[2:3]\n v_cndmask_b32 %2, %3, %0, s[2:3]\n")
+                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"s2", "s3");
+        if (KIND == 17)
+            asm volatile(DPK_R8("v_cmp_lt_u32 vcc, %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cmp_lt_u32 vcc, %2, %3\n s_nop 1\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
                          : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
         if (KIND == 12)
             asm volatile(DPK_R8("v_and_b32 %0, %1, %2\n v_xor_b32 %1, %2, %3\n v_or_b32 %2, %3, %0\n v_sub_u32 %3, %0, %1\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));

@@ -240,7 +240,7 @@ int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *av
 int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
 
 /* ---- what a vector instruction costs to issue: a launch of `iters` iterations of 32 instructions of one kind
- * (kind 0 .. 12, named in *name_out) at waves_per_simd (1 .. 8) wavefronts on every SIMD; returns the best of three
+ * (kind 0 .. 17, named in *name_out) at waves_per_simd (1 .. 8) wavefronts on every SIMD; returns the best of three
  *  launches in milliseconds, and the device's clock (kHz) and number of compute units.  No counterpart in the reference; the
  * device arithmetic is written for what this shows. */
 int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t iters, uint32_t waves_per_simd, double *ms_out, const char **name_out,
