@@ -2660,6 +2660,7 @@ __global__ __launch_bounds__(BLOCK) void read_kernel(const uint4 *__restrict__ s
 // ---------------------------------------------------------------------------
 constexpr int ISSUE_COST_KINDS = 18;
 constexpr int ISSUE_COST_COPIES = 32;
+#if defined(__HIPCC__)  // machine instructions by name: for the device compiler only
 #define DPK_R8(x) x x x x x x x x
 template <int KIND>
 __global__ void __launch_bounds__(BLOCK) issue_cost_kernel(u64 *out, u32 iters)
@@ -2715,5 +2716,6 @@ __global__ void __launch_bounds__(BLOCK) issue_cost_kernel(u64 *out, u32 iters)
     out[(u64)blockIdx.x * BLOCK + threadIdx.x] = x ^ y ^ z ^ w ^ a ^ b ^ c ^ d;
 }
 #undef DPK_R8
+#endif
 
 }  // namespace dpk
