@@ -51,27 +51,30 @@ GL_FN u64 pack(u32 lo, u32 hi) { return ((u64)hi << 32) | lo; }
 template <bool CANON = true>
 GL_FN u64 reduce160(u32 l0, u32 l1, u32 l2, u32 l3, u32 l4)
 {
+    // t = (l0, l1) - (l3, l4) as a wrapped word, b its borrow
     u32 b, c;
-    u32 t0 = __builtin_subc(l0, l3, 0u, &b);
-    u32 t1 = __builtin_subc(l1, l4, b, &b);
-    // below zero: p = 2^64 - EPS is owed, which on the wrapped word is - EPS (the word is above 2^63: no second borrow)
-    u32 m = 0u - b;
-    t0 = __builtin_subc(t0, m, 0u, &b);
-    t1 = __builtin_subc(t1, 0u, b, &b);
-    // u = l2 (2^32 - 1) = (l2 << 32) - l2, at most 2^64 - 2^33 + 1
-    u32 u0 = __builtin_subc(0u, l2, 0u, &b);
-    u32 u1 = __builtin_subc(l2, 0u, b, &b);
-    u32 r0 = __builtin_addc(t0, u0, 0u, &c);
-    u32 r1 = __builtin_addc(t1, u1, c, &c);
-    // past 2^64: add EPS (the wrapped sum is at most 2^64 - 2^33: no second carry)
-    m = 0u - c;
-    r0 = __builtin_addc(r0, m, 0u, &c);
-    r1 = __builtin_addc(r1, 0u, c, &c);
-    if (!CANON) return pack(r0, r1);
+    const u32 t0 = __builtin_subc(l0, l3, 0u, &b);
+    const u32 t1 = __builtin_subc(l1, l4, b, &b);
+    // r = t + l2 (2^32 - 1) by one multiply-add (the product is at most 2^64 - 2^33 + 1), x = all ones when it carries
+    u64 r, s;
+    u32 x;
+    asm("v_mad_u64_u32 %[r], %[s], %[l2], -1, %[t]\n\t"
+        "s_nop 1\n\t"
+        "v_cndmask_b32_e64 %[x], 0, -1, %[s]"
+        : [r] "=v"(r), [s] "=s"(s), [x] "=v"(x)
+        : [l2] "v"(l2), [t] "v"(pack(t0, t1)));
+    // The value is r + (carry - borrow) 2^64 = r + (carry - borrow) EPS (mod p).  Carry alone: the wrapped word is
+    // below 2^64 - 2^33, adding EPS does not wrap.  Borrow alone: t is above 2^63 as a word and nothing wrapped after
+    // it, subtracting EPS stays above zero.  Both or neither: r as it is.
+    u32 w;
+    const u32 d0 = __builtin_subc(x, 0u - b, 0u, &w);  // (all ones or 0) - (all ones or 0) as a 64-bit word (d0, -w)
+    r += pack(d0, 0u - w);
+    if (!CANON) return r;
     // r >= p exactly when r + EPS wraps, and r - p is that wrapped sum
+    const u32 r0 = (u32)r, r1 = (u32)(r >> 32);
     u32 s0 = __builtin_addc(r0, 0xFFFFFFFFu, 0u, &c);
     u32 s1 = __builtin_addc(r1, 0u, c, &c);
-    return c ? pack(s0, s1) : pack(r0, r1);
+    return c ? pack(s0, s1) : r;
 }
 
 // (hi * 2^64 + lo) mod p, canonical

@@ -26,7 +26,10 @@ def ctx(dp):
 
 ONE = np.array([1, 0], dtype=np.uint64)
 EDGE = [0, 1, 2, 7, P - 1, P - 2, 2**32, 2**32 - 1, 2**32 + 1, 2**63, 2**63 - 1, (P - 1) // 2, (P + 1) // 2, 0xFFFFFFFF,
-        0xFFFFFFFF00000000, 0xFFFFFFFE00000001, 0xFFFFFFFEFFFFFFFF]
+        0xFFFFFFFF00000000, 0xFFFFFFFE00000001, 0xFFFFFFFEFFFFFFFF,
+        # products whose top limb exceeds the low word while the third limb is zero, one, or large (borrow alone, borrow
+        # and carry together in the reduction)
+        2**48, 2**48 + 2**16, 2**48 + 2**47 + 1]
 
 
 def test_device_field_arithmetic(ctx):
