@@ -1469,14 +1469,20 @@ struct dps_sc {
     std::vector<Stage> stages;
     std::vector<u32> slice_ids;                // the tables of the resident launches (session indices), in slot order
     std::vector<dpk::SliceTerm> slice_terms;   // sums of several terms: the terms, their tables as slots of slice_ids
-    std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip
+    std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip,
+                                      // 4 worked out on the host
     std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip)
     u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
     E2 prev_chal;                     // the challenge of the call before this one
     bool pair12;                      // rounds 1 and 2 are one launch that writes nothing (pair12_kernel); round 3 folds twice on its way in
     E2 stash[dpk::SL_MAX_SUMS];       // a trip of two rounds: the second round's sums as a polynomial in the first round's challenge
     u64 last_trip_seq;
-    u32 fin_len;                      // entries per table the last trip leaves to the host (2, or 4 after a trip of two rounds)
+    u32 fin_len;                      // entries per table the last trip leaves to the host: the state of its first round
+    u32 fin_pend;                     // ... and the folds that state is still owed (the rounds of that trip)
+    u32 host_rounds;                  // the last rounds are worked out on the host from those entries (round_kind 4)
+    std::vector<E2> host_state;       // the tables of the round in hand there, table by table
+    u32 host_len;                     // entries per table in host_state (0: not taken over yet)
+    bool host_fresh;                  // ... as the launch left them: the folds of its last trip are still owed
     u32 tail_j0;        // first resident round, 0 = none
     bool tail_running;
     u64 tail_seq0;
@@ -1913,6 +1919,10 @@ u32 slice_pairs_per_workgroup(u32 n_tabs, u32 lds_bytes)
 // ... and the fewest it is given when the sum is small enough for that: shorter chains of work per lane, more workgroups
 constexpr u32 SLICE_MIN_PAIRS = 128;
 constexpr u32 SLICE_MAX_WORKGROUPS = 256;
+// the rounds a resident launch leaves to the host: at most so many, and so many extension multiplications in all
+// (measured: 2 to 6 rounds and 400 to 3000 multiplications differ by a few percent; these were the best over the benchmark configurations)
+constexpr u32 HOST_TAIL_MAX_ROUNDS = 5;
+constexpr u64 HOST_TAIL_MULTS = 800;
 
 // Which rounds of a session are resident, in which launches, and how they pair up into trips.  `n_tabs`: tables in LDS.
 // A trip covers two rounds when the second one's p(1) can come from the claim (its eq coordinate is not zero) and the
@@ -1938,6 +1948,29 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
     while (pairs_of(j) > (u64)per_wg_max * SLICE_MAX_WORKGROUPS) j++;
     const u32 per_wg = (u32)std::min<u64>(per_wg_max, std::max<u64>(SLICE_MIN_PAIRS, pairs_of(j) / SLICE_MAX_WORKGROUPS));
     sc->tail_j0 = j;
+    // The last rounds are the host's: a trip costs the way to the GPU and back and a workgroup's barriers whatever it
+    // carries, a round of a few pairs costs the host a microsecond.  As many rounds as stay below HOST_TAIL_MULTS
+    // extension multiplications in all and whose tables fit the hand-over (the trip before them can cover two rounds:
+    // four times the entries of the first host round), and never the first resident round.
+    u32 host_rounds = 0;
+    {
+        u32 factors = 0;  // multiplications per pair and point
+        if (sc->poly)
+            for (const dpk::SliceTerm &t : sc->slice_terms) factors += t.n_factors + 1;
+        else
+            factors = sc->fast_nf;
+        factors += has_eq ? 1 : 0;
+        const u64 per_pair = (u64)factors * (sc->fast_nf + 1) + 2 * n_tabs;
+        // (the launch keeps a trip for its single workgroup, which hands the tables over, and two rounds before it when
+        // several workgroups start)
+        const u32 gpu_rounds_min = pairs_of(j) > per_wg ? 3 : 1;
+        while (host_rounds < HOST_TAIL_MAX_ROUNDS && host_rounds + gpu_rounds_min <= n - j && (((u64)2 << host_rounds) - 1) * per_pair <= HOST_TAIL_MULTS &&
+               (u64)n_tabs * ((u64)8 << (host_rounds + 1)) <= (u64)dpk::SL_FIN_MAX_WORDS)
+            host_rounds++;
+    }
+    const u32 n_gpu = n - host_rounds;  // the last round of a trip
+    sc->host_rounds = host_rounds;
+    for (u32 r = n_gpu + 1; r <= n; r++) sc->round_kind[r] = 4;
     u32 pend = j == 1 ? 0 : 1;                   // a launch that starts with round 1 has nothing to fold first
     u64 entries = (u64)1 << (n - j + 1 + pend);  // of the tables the stage to come starts from (before its pending folds)
     auto add_stage = [&](u32 W) {
@@ -1950,8 +1983,8 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
         u64 len = (entries / W) >> pend;  // entries per table and workgroup in the trip's first round
         st.cap = (u32)len;
         for (;;) {
-            // (as the last trip only when the 4 entries left of every table fit the hand-over)
-            const bool dbl = len >= 4 && j + 1 <= n && claim_gives_p1(j + 1) && !(j + 1 == n && n_tabs > (u32)dpk::SL_DBL_LAST_MAX_TABS);
+            bool dbl = len >= 4 && j + 1 <= n_gpu && claim_gives_p1(j + 1);
+            if (W > 1 && j + 1 == n_gpu) dbl = false;  // the last trip is the single workgroup's
             if (dbl) st.dbl_mask |= 1u << st.n_trips;
             st.n_trips++;
             sc->round_kind[j] = dbl ? 2 : 1;
@@ -1959,16 +1992,17 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
             if (dbl) sc->round_kind[j + 1] = 3;
             pend = dbl ? 2 : 1;
             j += pend;
-            // several workgroups go on while each still has a pair after the pending folds; one goes on to the last round
-            if (j > n || (W > 1 && (len >> pend) < 2) || st.n_trips == (u32)dpk::SL_MAX_TRIPS) break;
+            // several workgroups go on while each still has a pair after the pending folds; one goes on to the last trip
+            if (j > n_gpu || (W > 1 && (j == n_gpu || (len >> pend) < 2)) || st.n_trips == (u32)dpk::SL_MAX_TRIPS) break;
             len >>= pend;
         }
         entries = len * W;
         sc->fin_len = (u32)len;
+        sc->fin_pend = pend;
         sc->stages.push_back(st);
     };
     if (pairs_of(j) > per_wg) add_stage((u32)(pairs_of(j) / per_wg));
-    while (j <= n) add_stage(1);
+    while (j <= n_gpu) add_stage(1);
 }
 
 }  // namespace
@@ -2261,6 +2295,11 @@ int32_t SessionSetup::plan_and_ready_tables()
     memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
     sc->last_trip_seq = 0;
     sc->fin_len = 0;
+    sc->fin_pend = 0;
+    sc->host_rounds = 0;
+    sc->host_len = 0;
+    sc->host_fresh = false;
+    sc->host_state.clear();
     sc->prev_chal = gl::e2_zero();
     sc->slice_ids.clear();
     sc->slice_terms.clear();
@@ -2294,6 +2333,7 @@ int32_t SessionSetup::plan_and_ready_tables()
                 sc->stages.clear();
                 sc->tail_j0 = 0;
                 sc->fin_len = 0;
+                sc->host_rounds = 0;
                 sc->round_kind.assign(n_vars + 2, 0);
                 sc->round_wide.assign(n_vars + 2, 0);
             }
@@ -2838,6 +2878,122 @@ int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u64 *out)
     }
 }
 
+// the area of dpk::SL_FIN_AREA_WORDS words where a resident launch leaves the tables' entries with its last trip
+size_t slice_fin_off(const dps_ctx *ctx) { return ctx->pinned_words / 2 + 4096; }
+
+// ... and those entries, `n` words published under the sequence number of that trip
+int32_t wait_slice_entries(dps_ctx *ctx, u64 seq, u32 n, u64 *out)
+{
+    volatile u64 *base = ctx->h_pinned + slice_fin_off(ctx);
+    auto take = [&]() {
+        if (__atomic_load_n(base + dpk::SL_FIN_SEQ_SLOT, __ATOMIC_ACQUIRE) != seq) return false;
+        u64 chk = seq;
+        for (u32 i = 0; i < n; i++) {
+            out[i] = base[i];
+            chk ^= dpk::sl_fin_mix(out[i], i);
+        }
+        return chk == base[dpk::SL_FIN_CHK_SLOT];
+    };
+    for (u64 spins = 0;; spins++) {
+        if (take()) return DPS_OK;
+        if ((spins & 0xFFFFF) == 0xFFFFF) {
+            hipError_t q = hipStreamQuery(ctx->stream);
+            if (q == hipSuccess) {
+                if (take()) return DPS_OK;
+                return fail(ctx, DPS_ERR_HIP, "the tables' last entries were not published");
+            }
+            if (q != hipErrorNotReady) return fail(ctx, DPS_ERR_HIP, "stream error while waiting for a round: %s", hipGetErrorString(q));
+        }
+    }
+}
+
+// The end of a session whose resident launch has left (slice_kernel, with its last trip): the state of that trip's
+// first round comes over with the trip (host_tail_load, in the same call: no other session's launch can overwrite the
+// area in between), is folded with the challenges drawn since, and from then on the host holds the tables.
+int32_t host_tail_load(dps_sc *sc, u64 seq)
+{
+    const u32 n_tabs = (u32)sc->slice_ids.size(), L = sc->fin_len;
+    std::vector<u64> w(2 * (size_t)L * n_tabs);
+    CHK(wait_slice_entries(sc->ctx, seq, (u32)w.size(), w.data()));
+    sc->host_state.resize((size_t)L * n_tabs);
+    for (size_t i = 0; i < sc->host_state.size(); i++) sc->host_state[i] = gl::e2(w[2 * i], w[2 * i + 1]);
+    sc->host_len = L;
+    sc->host_fresh = true;
+    return DPS_OK;
+}
+
+// `r`: the challenge the call in hand brought (sc->prev_chal: the one before it)
+void host_tail_advance(dps_sc *sc, E2 r)
+{
+    const u32 n_tabs = (u32)sc->slice_ids.size();
+    auto fold_all = [&](E2 c) {
+        const u32 half = sc->host_len / 2;
+        for (u32 f = 0; f < n_tabs; f++) {
+            const E2 *src = sc->host_state.data() + (size_t)f * sc->host_len;
+            E2 *dst = sc->host_state.data() + (size_t)f * half;  // (in place: a new entry lies before the old ones still to be read)
+            for (u32 i = 0; i < half; i++) {
+                const E2 lo = src[2 * i], hi = src[2 * i + 1];
+                dst[i] = gl::add(lo, gl::mul(c, gl::sub(hi, lo)));
+            }
+        }
+        sc->host_len = half;
+    };
+    // the last trip covered two rounds: the challenge between them first
+    if (sc->host_fresh && sc->fin_pend == 2) fold_all(sc->prev_chal);
+    sc->host_fresh = false;
+    fold_all(r);
+}
+
+// The sums q(t), t = 0 .. nf, of a round on the tables the host holds (q(1) left out when it comes from the claim):
+// what slice_kernel adds up, by the definition.
+void host_tail_sums(dps_sc *sc, u32 j, u32 nf, bool skip1, E2 *q)
+{
+    const u32 n_tabs = (u32)sc->slice_ids.size();
+    const u32 len = sc->host_len, n_pairs = len / 2;
+    const bool has_eq = sc->fast_eq >= 0;
+    // eq(rho_{j+1..n}, x) over the pairs: variable j + 1 is the lowest bit of the pair's index
+    std::vector<E2> weight(n_pairs, gl::e2_one());
+    if (has_eq) {
+        u32 have = 1;
+        for (u32 i = j + 1; i <= sc->n_vars; i++) {
+            const E2 rho = sc->eq_info->point[i - 1], one_minus = gl::sub(gl::e2_one(), rho);
+            for (u32 x = 0; x < have; x++) {
+                weight[x + have] = gl::mul(weight[x], rho);
+                weight[x] = gl::mul(weight[x], one_minus);
+            }
+            have *= 2;
+        }
+    }
+    for (u32 t = 0; t <= nf; t++) q[t] = gl::e2_zero();
+    E2 val[dpk::SL_MAX_TABS];
+    for (u32 p = 0; p < n_pairs; p++) {
+        E2 lo[dpk::SL_MAX_TABS], d[dpk::SL_MAX_TABS];
+        for (u32 f = 0; f < n_tabs; f++) {
+            lo[f] = sc->host_state[(size_t)f * len + 2 * p];
+            d[f] = gl::sub(sc->host_state[(size_t)f * len + 2 * p + 1], lo[f]);
+            val[f] = lo[f];
+        }
+        for (u32 t = 0; t <= nf; t++) {
+            if (t > 0)
+                for (u32 f = 0; f < n_tabs; f++) val[f] = gl::add(val[f], d[f]);
+            if (t == 1 && skip1) continue;
+            E2 g;
+            if (sc->poly) {
+                g = gl::e2_zero();
+                for (const dpk::SliceTerm &tm : sc->slice_terms) {
+                    E2 prod = gl::e2(tm.c0, tm.c1);
+                    for (u32 k = 0; k < tm.n_factors; k++) prod = gl::mul(prod, val[tm.slot[k]]);
+                    g = gl::add(g, prod);
+                }
+            } else {
+                g = val[0];
+                for (u32 f = 1; f < n_tabs; f++) g = gl::mul(g, val[f]);
+            }
+            q[t] = gl::add(q[t], has_eq ? gl::mul(g, weight[p]) : g);
+        }
+    }
+}
+
 }  // namespace
 
 namespace {
@@ -3126,6 +3282,7 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
             sa.spin_limit = wait_units(ctx, 4000000);  // ten seconds, then the kernel gives up
             sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
             sa.out_host = ctx->d_pinned + slice_area_off(ctx);
+            sa.fin_out = ctx->d_pinned + slice_fin_off(ctx);
             sa.seq0 = seq0 + (st.j0 - first);
             sa.ctr = ctx->d_slice_ctr;
             sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
@@ -3154,7 +3311,14 @@ int32_t FusedRound::resident_round()
     const u32 np = nf + 1;
     E2 q[dpk::MAX_PTS];
     int32_t rc = DPS_OK;
-    if (kind == 3) {
+    if (kind == 4) {
+        // A round of the few pairs that are left once the launch has gone: worked out here.
+        if (sc->host_len < 4) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the tables of the last rounds are not here");
+        host_tail_advance(sc, gl::e2(challenge[0], challenge[1]));
+        host_tail_sums(sc, j, nf, a.skip1 != 0, q);
+        prepare_message();
+        form_message(q);
+    } else if (kind == 3) {
         // Second round of a trip: the kernel handed over this round's sums as a polynomial in the challenge that has
         // now been drawn (values at 0..nf-1 and the leading coefficient, per point t = 0, 2, .., nf); p(1) comes
         // from the claim.  Nothing goes to the GPU.
@@ -3206,10 +3370,12 @@ int32_t FusedRound::resident_round()
             for (u32 i = np; i < ns; i++) sc->stash[i - np] = gl::e2(w[2 * i], w[2 * i + 1]);
             form_message(q);
             sc->last_trip_seq = fa.seq;
+            // the last trip: what is left of the tables has come with it
+            if (j + (kind == 2 ? 1 : 0) == sc->n_vars - sc->host_rounds) rc = host_tail_load(sc, fa.seq);
         }
     }
     if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
-    if (j == sc->n_vars || rc != DPS_OK) {
+    if ((kind != 4 && j == sc->n_vars - sc->host_rounds) || rc != DPS_OK) {
         // with its last trip the kernel publishes what is left of the tables and exits
         sc->tail_running = false;
         ctx->tail_owner = nullptr;
@@ -3634,18 +3800,15 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
         // groups are resident), the single-product one its factors
         if (!sc->stages.empty()) {
-            // the resident launch left 2 entries per table, or 4 when its last trip covered two rounds (the challenge
-            // between them is the one the last round's call brought)
-            const u32 L = sc->fin_len;
+            // the host holds the tables: the last fold leaves one entry each
+            if (sc->host_len < 2) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: the tables' last entries are not here");
+            host_tail_advance(sc, r);
             const u32 n_tabs = (u32)sc->slice_ids.size();
-            CHK(wait_result_at(ctx, slice_area_off(ctx), sc->pairs_seq, dpk::SL_FIN_SLOT, 2 * L * n_tabs, w, dpk::SL_FIN_SEQ_SLOT, dpk::SL_FIN_CHK_SLOT));
+            if (sc->host_len != 1) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: %u entries left of every table", sc->host_len);
             for (u32 f = 0; f < n_tabs; f++) {
-                auto at = [&](u32 e) { return gl::e2(w[2 * (f * L + e)], w[2 * (f * L + e) + 1]); };
-                auto fold = [](E2 lo, E2 hi, E2 c) { return gl::add(lo, gl::mul(c, gl::sub(hi, lo))); };
-                const E2 v = L == 4 ? fold(fold(at(0), at(1), sc->prev_chal), fold(at(2), at(3), sc->prev_chal), r) : fold(at(0), at(1), r);
                 const u32 k = sc->slice_ids[f];
-                final_evals_out[2 * k] = v.c0;
-                final_evals_out[2 * k + 1] = v.c1;
+                final_evals_out[2 * k] = sc->host_state[f].c0;
+                final_evals_out[2 * k + 1] = sc->host_state[f].c1;
             }
         }
         const u32 n_areas = sc->poly && sc->stages.empty() ? (u32)sc->poly_tabs.size() : 0;

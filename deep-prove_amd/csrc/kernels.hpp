@@ -1178,8 +1178,9 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
 // the hand-off to the host and back).  From there on the tables live in LDS: every workgroup of this launch owns a
 // contiguous slice of every table -- binding the lowest variable turns entries 2i, 2i+1 into entry i, so what a
 // workgroup needs in the next round is what it has just made -- and stays on the GPU, waiting for each challenge in
-// the host's mailbox.  With one workgroup it runs to the last round; with several it runs until a workgroup is down to
-// an entry or two per table, leaves them in device memory (`h0/h1`) and a single-workgroup launch queued behind it goes on.
+// the host's mailbox.  With one workgroup it runs to its last trip (the session's last round, or a few rounds before it:
+// the host does those from the entries the trip leaves it); with several it runs until a workgroup is down to an entry or
+// two per table, leaves them in device memory (`h0/h1`) and the first workgroup, or a launch queued behind, goes on.
 //
 // A trip to the host can cover two rounds.  With S the state of round j (pairs (S[2i], S[2i+1])), the tables of round
 // j+1 are S[2i] + r_j (S[2i+1] - S[2i]): linear in the challenge r_j that is not known yet, so the sums of round j+1
@@ -1204,15 +1205,19 @@ constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
 // is one store, so it is whole when its tag is there; the host clears the tags it has taken.
 constexpr u64 SL_CTR_MASK = (1ull << 56) - 1, SL_CTR_ONE = 1ull << 56;
 __host__ __device__ __forceinline__ u64 sl_tag(u64 trip_seq) { return 0x80 | (trip_seq & 0x7F); }
-// with the last trip of a run to the last round: the entries every table still has (2, or 4 after a trip of two rounds)
-constexpr int SL_FIN_SLOT = 104, SL_FIN_SEQ_SLOT = 168, SL_FIN_CHK_SLOT = 169, SL_AREA_WORDS = 192;
-static_assert(4 * SL_MAX_SUMS <= SL_FIN_SLOT, "the counters lie before the last entries");
+// With its last trip a launch that hands the session's end to the host leaves the state of that trip's first round: every
+// table's entries, in an area of their own (`fin_out`: SL_FIN_MAX_WORDS words, then the trip's sequence number and a
+// check word).  The host folds them with the challenges it has drawn since and does what is left: the last fold, or a
+// few rounds of a handful of pairs, which cost it less than a trip costs.
+constexpr int SL_AREA_WORDS = 192;
+constexpr int SL_FIN_MAX_WORDS = 1024, SL_FIN_SEQ_SLOT = SL_FIN_MAX_WORDS, SL_FIN_CHK_SLOT = SL_FIN_MAX_WORDS + 1, SL_FIN_AREA_WORDS = SL_FIN_MAX_WORDS + 2;
+static_assert(4 * SL_MAX_SUMS <= SL_AREA_WORDS, "the counters fit the result area");
 constexpr int SL_MAX_TRIPS = 32;
 constexpr int SL_MAX_TABS = 16;   // tables of a sum of several terms (a product has at most 3)
-constexpr int SL_DBL_LAST_MAX_TABS = 8;  // a trip of two rounds can be the last one only with so few tables (4 entries of each go to the host)
 constexpr int SL_MAX_TERMS = 24;
-static_assert(SL_FIN_SLOT + WAVE <= SL_FIN_SEQ_SLOT && 2 * 4 * SL_DBL_LAST_MAX_TABS <= WAVE && 2 * 2 * SL_MAX_TABS <= WAVE,
-              "the last entries of every table fit the result area and one wavefront");
+static_assert(2 * 4 * SL_MAX_TABS <= SL_FIN_MAX_WORDS, "the last entries of every table fit their area");
+// the check word's share of word i of that area
+__host__ __device__ __forceinline__ u64 sl_fin_mix(u64 word, u32 i) { return rotl64(word, (i & 31) + 1); }
 // a term of a sum of several terms: coefficient (prepared: w = 7 c1) times the tables in `slot`
 struct SliceTerm {
     u64 c0, c1, w;
@@ -1238,9 +1243,10 @@ struct SliceArgs {
     const u64 *mail;   // host mailbox
     u64 *relay;        // several workgroups: the first passes each mail on through these words of device memory
     u32 spin_limit;
-    u32 finish;        // a single workgroup that runs to the last round: the remaining entries go to the host with the last
-                       // trip; else they go to h0 / h1
+    u32 finish;        // the launch's last trip is the last of the session's launches: the state of that trip's first round goes to
+                       // the host (fin_out) with it; else what is left goes to h0 / h1
     u64 *out_host;     // result area of SL_AREA_WORDS words
+    u64 *fin_out;      // ... and the area of SL_FIN_AREA_WORDS words for the entries left with the last trip (finish)
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
     u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero when the launch starts
     u32 *gate;         // ... and the count of workgroups that have left their tables in h0 / h1 (zero when the launch starts)
@@ -1524,21 +1530,20 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             }
         }
     } else if (wave == 0) {
-        // to the host, which does the last fold or two: entry e of table f at words 2 (f len + e), + 1
+        // to the host: entry e of table f at words 2 (f len + e), + 1 (len is a power of two)
         const u32 n_words = nt * len * 2;
-        const bool mine = lane < n_words;
-        u64 word = 0;
-        if (mine) {
-            const u32 f = lane / (2 * len), e = (lane >> 1) % len;
-            word = tab(big, f, lane & 1)[e];
+        u64 x = 0;
+        for (u32 w = lane; w < n_words; w += WAVE) {
+            const u32 f = w >> (len_log + 1), e = (w >> 1) & (len - 1);
+            const u64 word = tab(big, f, w & 1)[e];
+            x ^= sl_fin_mix(word, w);
+            st_sys(a.fin_out + w, word);
         }
-        u64 x = mine ? rotl64(word, lane + 1) : 0;
 #pragma unroll
         for (int off = WAVE / 2; off >= 1; off >>= 1) x ^= __shfl_xor(x, off, WAVE);
-        if (mine) st_sys(a.out_host + SL_FIN_SLOT + lane, word);
         if (lane == 0) {
-            st_sys(a.out_host + SL_FIN_CHK_SLOT, x ^ trip_seq);
-            st_sys(a.out_host + SL_FIN_SEQ_SLOT, trip_seq);
+            st_sys(a.fin_out + SL_FIN_CHK_SLOT, x ^ trip_seq);
+            st_sys(a.fin_out + SL_FIN_SEQ_SLOT, trip_seq);
         }
     }
 }

@@ -98,11 +98,13 @@ struct Term {
 // eq point with a zero coordinate there).  TERMS = false: the product of NF tables.  TERMS = true: sum_k coeff_k prod tables
 // over `n_tabs` tables, NF the largest number of factors; `base_tabs` of the tables are base-field ones (j0 <= 2 only).
 // `separate`: the stage of several workgroups and the single workgroup after it are two launches (as when the rounds left
-// are more than one launch can run); otherwise they are one.
+// are more than one launch can run); otherwise they are one.  `host_rounds`: the last rounds are not the launch's (the
+// library works them out on the host): its last trip ends before them and hands over that many more entries.
 template <int NF, bool EQ, bool TERMS = false>
 static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_in, std::vector<u32> single_rounds = {}, std::vector<Term> terms = {},
-                     u32 base_tabs = 0, bool separate = false)
+                     u32 base_tabs = 0, bool separate = false, u32 host_rounds = 0)
 {
+    const u32 n_gpu = n_vars - host_rounds;  // the last round of a trip
     constexpr int NP = NF + 1, NPT = NF, NSMP = NF + 1, NS = NP + NSMP * NPT;
     const u32 NT = TERMS ? n_tabs_in : (u32)NF;
     if (!TERMS) {
@@ -145,11 +147,12 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
             Stage st{wide, j, pend, entries, {}};
             u64 len_wg = (entries / wide) >> pend;
             for (;;) {
-                const bool dbl = len_wg >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1);
+                // (the last trip is the single workgroup's, which hands the tables over)
+                const bool dbl = len_wg >= 4 && j + 1 < n_gpu && !is_single(j) && !is_single(j + 1);
                 st.trips.push_back({j, dbl});
                 pend = dbl ? 2 : 1;
                 j += pend;
-                if ((len_wg >> pend) < 2 || j > n_vars) break;
+                if ((len_wg >> pend) < 2 || j >= n_gpu) break;
                 len_wg >>= pend;
             }
             entries = len_wg * wide;
@@ -157,8 +160,8 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         }
         Stage st{1, j, pend, entries, {}};
         u64 len = entries >> pend;
-        while (j <= n_vars) {
-            const bool dbl = len >= 4 && j + 1 <= n_vars && !is_single(j) && !is_single(j + 1) && !(j + 1 == n_vars && NT > (u32)dpk::SL_DBL_LAST_MAX_TABS);
+        while (j <= n_gpu) {
+            const bool dbl = len >= 4 && j + 1 <= n_gpu && !is_single(j) && !is_single(j + 1);
             st.trips.push_back({j, dbl});
             const u32 p = dbl ? 2 : 1;
             j += p;
@@ -167,7 +170,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         stages.push_back(st);
     }
 
-    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
+    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
     u32 gate = 0;
     const u64 seq_first = 1000;
     bool ok = true;
@@ -234,6 +237,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         a.spin_limit = 1u << 24;
         a.finish = last_si + 1 == stages.size();
         a.out_host = area.data();
+        a.fin_out = fin.data();
         a.seq0 = seq_first + (st.j0 - j0);
         a.ctr = gctr.data();
         a.gate = &gate;
@@ -250,7 +254,6 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         std::vector<std::vector<u64>> lds;
         auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap, dpk::BLOCK), dpk::slice_kernel<NF, EQ, TERMS, dpk::BLOCK>, a, groups, lds);
         // ---- the host's side ----
-        u32 len_after = 0;
         std::vector<u64> seen(4 * dpk::SL_MAX_SUMS, 0);  // the counters of several workgroups run on from trip to trip
         for (size_t sj = si; sj <= last_si && ok; sj++) {
             const Stage &sx = stages[sj];
@@ -369,7 +372,6 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
                         }
                     }
                 }
-                len_after = dbl ? 4 : 2;
             }
         }
         if (!ok) {
@@ -413,18 +415,19 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
             if (stages[si + 1].pend0 != (st.trips.back().second ? 2u : 1u)) ok = false, printf("%s: pending folds disagree\n", name);
         }
         if (last_si + 1 == stages.size()) {
-            // the last entries of every table, published with the last trip
+            // what is left of every table, published with the last trip: the state of that trip's first round
             const auto &last = stages[last_si].trips.back();
             fold_to(last.first);
             const u64 seq = seq_first + (last.first - j0);
+            const u32 len_left = (u32)state[0].size();
+            if (len_left != ((last.second ? 4u : 2u) << host_rounds)) ok = false, printf("%s: %u entries left\n", name, len_left);
             u64 c = seq;
-            const u32 n_words = NT * len_after * 2;
-            for (u32 i = 0; i < n_words; i++) c ^= dpk::rotl64(area[dpk::SL_FIN_SLOT + i], i + 1);
-            if (area[dpk::SL_FIN_SEQ_SLOT] != seq || area[dpk::SL_FIN_CHK_SLOT] != c) ok = false, printf("%s: last entries not handed over\n", name);
-            if (state[0].size() != len_after) ok = false, printf("%s: %zu entries left, %u expected\n", name, state[0].size(), len_after);
+            const u32 n_words = NT * len_left * 2;
+            for (u32 i = 0; i < n_words; i++) c ^= dpk::sl_fin_mix(fin[i], i);
+            if (fin[dpk::SL_FIN_SEQ_SLOT] != seq || fin[dpk::SL_FIN_CHK_SLOT] != c) ok = false, printf("%s: last entries not handed over\n", name);
             for (u32 f = 0; f < NT && ok; f++)
-                for (u32 e = 0; e < len_after; e++)
-                    if (area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e)] != state[f][e].c0 || area[dpk::SL_FIN_SLOT + 2 * (f * len_after + e) + 1] != state[f][e].c1)
+                for (u32 e = 0; e < len_left; e++)
+                    if (fin[2 * (f * len_left + e)] != state[f][e].c0 || fin[2 * (f * len_left + e) + 1] != state[f][e].c1)
                         ok = false, printf("%s: last entry %u of table %u differs\n", name, e, f);
         }
         si = last_si + 1;
@@ -432,7 +435,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
     size_t n_trips = 0;
     for (auto &s : stages) n_trips += s.trips.size();
     printf("%-60s degree %d eq=%d n=%u from round %u, %zu stage(s), %zu trips for %u rounds : %s\n", name, NF, (int)EQ, n_vars, j0, stages.size(), n_trips,
-           n_vars - j0 + 1, ok ? "ok" : "MISMATCH");
+           n_gpu - j0 + 1, ok ? "ok" : "MISMATCH");
     if (!ok) failures++;
 }
 
@@ -458,8 +461,14 @@ int main()
     // the stacked products of an einsum: 16 tables, 8 terms of two factors each, every round resident
     std::vector<Term> stacked;
     for (u32 i = 0; i < 8; i++) stacked.push_back(Term{felt2(), {2 * i, 2 * i + 1}});
-    run_case<2, false, true>("16 tables, 8 products, from round 1 (the last two rounds go alone)", 8, 1, 1, 16, {}, stacked);
+    run_case<2, false, true>("16 tables, 8 products, from round 1", 8, 1, 1, 16, {}, stacked);
     run_case<2, false, true>("the same with an odd number of rounds", 7, 1, 1, 16, {}, stacked);
+    // launches that leave the last rounds to the host: more entries handed over than a wavefront has lanes
+    run_case<2, true>("two tables and eq, the last four rounds left out", 10, 2, 1, 0, {}, {}, 0, false, 4);
+    run_case<2, true>("the same with a single round as the last trip", 9, 2, 1, 0, {}, {}, 0, false, 4);
+    run_case<2, true>("four workgroups, then one, the last three rounds left out", 12, 3, 4, 0, {}, {}, 0, false, 3);
+    run_case<2, false, true>("16 tables, 8 products, the last two rounds left out", 8, 1, 1, 16, {}, stacked, 0, false, 2);
+    run_case<2, true, true>("fraction-sum layer over 4 workgroups, the last three rounds left out", 11, 2, 4, 4, {}, {la, lb, lc}, 0, false, 3);
     printf("%s\n", failures ? "FAILED" : "all cases ok");
     return failures ? 1 : 0;
 }

@@ -297,6 +297,33 @@ def test_resident_kernel_gives_way(dp, ctx, orc):
         assert (proof == ref_proof).all() and (point == ref_point).all()
 
 
+@pytest.mark.parametrize("n,with_eq", [(12, False), (13, True), (9, True)])
+def test_last_rounds_are_the_hosts(dp, ctx, orc, n, with_eq):
+    """The resident launch leaves before the last rounds: the tables' entries come to the host with its last trip, and
+    the rounds that are left (and the final evaluations) are worked out there.  From then on the session needs nothing
+    of the GPU: other calls on the context, whole proofs included, between its last rounds do not disturb it."""
+    f, g = rand_base(1 << n, 8200 + n), rand_e2(1 << n, 8201 + n)
+    gpu, host, fs = [ctx.mle_from_base(f), ctx.mle_from_ext2(g)], [orc.embed_base(f), g], [0, 1]
+    if with_eq:
+        pt = rand_e2(n, 8202 + n)
+        gpu.append(ctx.eq_build(pt))
+        host.append(orc.eq_evals(pt))
+        fs = [2, 0, 1]
+    terms = [(np.array([3, 5], dtype=np.uint64), fs)]
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"host tail"))
+    for first_other in (n - 2, n - 1, n):  # rounds completed before the first other call
+        s = ctx.session(n, gpu, terms)
+        chal = None
+        for j in range(n):
+            assert (s.round(chal) == ref_proof[j]).all(), (first_other, j)
+            chal = ref_point[j]
+            if j + 1 >= first_other:
+                proof, point, finals = ctx.sumcheck_prove(n, gpu, terms, dp.Transcript(b"host tail"))
+                assert (proof == ref_proof).all() and (point == ref_point).all() and (finals == ref_finals).all()
+        assert (s.finish(chal) == ref_finals).all()
+        del s
+
+
 def test_views_are_borrowed_halves(dp, ctx, orc):
     # SmartSlice::Borrowed halves as used by the LogUp layers (circuit.rs:260-271)
     n = 8
