@@ -3684,8 +3684,14 @@ int32_t FusedRound::first_two_rounds_launch()
         reset_device_words(ctx);
         return rc;
     }
-    // pair 0's three (value at 0, at 1, leading coefficient of the product along x0), pair 1's, those of round 2 at t = 2
+    // pair 0's three (value at 0, at 1, leading coefficient of the product along x0), pair 1's, and the same three products
+    // of the slopes along x1: each product is a quadratic in x1 with these as its values at 0 and 1 and its leading
+    // coefficient, so at x1 = 2 (round 2 at t = 2) it is 2 v(1) - v(0) + 2 lead
     for (u32 k = 0; k < (u32)dpk::PAIR12_SUMS; k++) sc->stash[k] = gl::e2(w[2 * k], w[2 * k + 1]);
+    for (u32 k = 0; k < 3; k++) {
+        const E2 v0 = sc->stash[k], v1 = sc->stash[3 + k], lead = sc->stash[6 + k];
+        sc->stash[6 + k] = gl::add(gl::sub(gl::add(v1, v1), v0), gl::add(lead, lead));
+    }
     // round 1 sums over the pairs of either kind, weighted by eq1(rho_2, x1); its q(2) = 2 q(1) - q(0) + 2 c
     const E2 rho2 = sc->eq_info->point[1], n2 = gl::sub(gl::e2_one(), rho2);
     E2 q[3];

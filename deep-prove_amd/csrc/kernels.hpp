@@ -1026,8 +1026,10 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
 //   pair x1 = 0:  f00 g00,  f10 g10,  (f10 - f00)(g10 - g00)       (round 1's q(0), q(1) and leading coefficient over the
 //   pair x1 = 1:  f01 g01,  f11 g11,  (f11 - f01)(g11 - g01)        pairs of either kind: the host weights them with
 //                                                                  1 - rho_2 and rho_2; and round 2 at t = 0, pair 0 alone)
-//   round 2 at t = 2, with F_a = 2 f_a1 - f_a0, G_a likewise:  F0 G0,  F1 G1,  (F1 - F0)(G1 - G0)
-// nine products where round 1 alone takes six, each row the same three products of a pair of values.  A workgroup is
+//   the slopes along x1, D_a = f_a1 - f_a0, E_a likewise:  D0 E0,  D1 E1,  (D1 - D0)(E1 - E0)
+// (each of the three products is a quadratic in x1 known at 0 and at 1: with its leading coefficient the host has it at
+// x1 = 2, which is round 2 at t = 2: 2 (row 1) - (row 0) + 2 (row 2)).
+// Nine products where round 1 alone takes six, each row the same three products of a pair of values.  A workgroup is
 // three wavefronts that walk the same quads, one row each (three unreduced sums a lane, as in round 1's kernel; the
 // quad comes from HBM once and twice more from the caches).  R is taken as in the FACT variants of prod_kernel:
 // hi[x' >> 16], the same for a workgroup's step, weights the products; lo[x' & 0xFFFF], the same for all steps of a
@@ -1040,7 +1042,7 @@ struct Pair12Args {
     const u64 *lq0, *lq1, *hq0, *hq1;
 };
 constexpr int PAIR12_BLOCK = 3 * WAVE;
-constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's three, pair 1's three, the three of t = 2
+constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's three, pair 1's three, the three of the slopes along x1
 constexpr int PAIR12_SEQ_SLOT = 62, PAIR12_CHK_SLOT = 63;
 static_assert(2 * PAIR12_SUMS <= PAIR12_SEQ_SLOT, "the sums fit the result area");
 
@@ -1070,7 +1072,7 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
     const u64 stride = (u64)gridDim.x * WAVE;
     const u64 q0 = (u64)blockIdx.x * WAVE + lane;
     // The loop, compiled once for rows 0 and 1 (their own pair: two loads) and once for row 2 (the whole quad, and the
-    // values at t = 2 made of it): a wavefront takes one or the other, no lane pays for both.
+    // slopes along x1 made of it): a wavefront takes one or the other, no lane pays for both.
     auto run = [&](auto last_row) {
         constexpr bool ROW2 = decltype(last_row)::value;
         struct Raw {
@@ -1096,11 +1098,11 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
             const E2 H = gl::e2(w.h0, w.h1);
             u64 fl = w.f0.x, fh = w.f0.y, gl_ = w.g0.x, gh = w.g0.y;
             if (ROW2) {
-                // t = 2 of round 2: 2 (x1 = 1) - (x1 = 0), at x0 = 0 and at x0 = 1
-                fl = gl::add(w.f1.x, gl::sub(w.f1.x, w.f0.x));
-                fh = gl::add(w.f1.y, gl::sub(w.f1.y, w.f0.y));
-                gl_ = gl::add(w.g1.x, gl::sub(w.g1.x, w.g0.x));
-                gh = gl::add(w.g1.y, gl::sub(w.g1.y, w.g0.y));
+                // the slopes along x1, at x0 = 0 and at x0 = 1
+                fl = gl::sub(w.f1.x, w.f0.x);
+                fh = gl::sub(w.f1.y, w.f0.y);
+                gl_ = gl::sub(w.g1.x, w.g0.x);
+                gh = gl::sub(w.g1.y, w.g0.y);
             }
             gl::acc_mul_base(lz[0], H, gl::mul_any(fl, gl_));
             gl::acc_mul_base(lz[1], H, gl::mul_any(fh, gh));

@@ -224,8 +224,9 @@ static void run_first_two_rounds(const char *name, u64 n_quads, u32 blocks)
     std::vector<u64> f(4 * n_quads), g(4 * n_quads), lq0(65536), lq1(65536), hq0((n_quads + 65535) >> 16), hq1(hq0.size());
     for (auto *v : {&f, &g, &lq0, &lq1, &hq0, &hq1})
         for (auto &x : *v) x = felt();
-    E2 want[dpk::PAIR12_SUMS];
+    E2 want[dpk::PAIR12_SUMS], want_at2[3];
     for (auto &w : want) w = gl::e2_zero();
+    for (auto &w : want_at2) w = gl::e2_zero();
     for (u64 q = 0; q < n_quads; q++) {
         const E2 w = gl::mul(gl::e2(hq0[q >> 16], hq1[q >> 16]), gl::e2(lq0[q & 65535], lq1[q & 65535]));
         const u64 *a = &f[4 * q], *b = &g[4 * q];
@@ -235,8 +236,13 @@ static void run_first_two_rounds(const char *name, u64 n_quads, u32 blocks)
         };
         three(0, a[0], a[1], b[0], b[1]);
         three(1, a[2], a[3], b[2], b[3]);
+        // the third row: the slopes along x1 ...
+        three(2, gl::sub(a[2], a[0]), gl::sub(a[3], a[1]), gl::sub(b[2], b[0]), gl::sub(b[3], b[1]));
+        // ... from which the host makes round 2 at t = 2; that, by the definition, for the check below
         auto at2 = [](u64 lo, u64 hi) { return gl::sub(gl::add(hi, hi), lo); };
-        three(2, at2(a[0], a[2]), at2(a[1], a[3]), at2(b[0], b[2]), at2(b[1], b[3]));
+        const u64 fl = at2(a[0], a[2]), fh = at2(a[1], a[3]), gl_ = at2(b[0], b[2]), gh = at2(b[1], b[3]);
+        const u64 v[3] = {gl::mul(fl, gl_), gl::mul(fh, gh), gl::mul(gl::sub(fh, fl), gl::sub(gh, gl_))};
+        for (int k = 0; k < 3; k++) want_at2[k] = gl::add(want_at2[k], gl::mul_base(w, v[k]));
     }
     dpk::Pair12Args pa;
     pa.f = f.data(), pa.g = g.data(), pa.n_quads = n_quads;
@@ -252,6 +258,12 @@ static void run_first_two_rounds(const char *name, u64 n_quads, u32 blocks)
     for (int k = 0; k < 2 * dpk::PAIR12_SUMS; k++) chk ^= dpk::rotl64(out_host[k], k + 1);
     bool ok = out_host[dpk::PAIR12_SEQ_SLOT] == seq && out_host[dpk::PAIR12_CHK_SLOT] == chk && counter == 0;
     for (int k = 0; k < dpk::PAIR12_SUMS; k++) ok = ok && gl::eq(gl::e2(out_host[2 * k], out_host[2 * k + 1]), want[k]);
+    // what the host does with the third row: 2 v(1) - v(0) + 2 lead is the product at x1 = 2
+    for (int k = 0; k < 3; k++) {
+        const E2 v0 = gl::e2(out_host[2 * k], out_host[2 * k + 1]), v1 = gl::e2(out_host[2 * (3 + k)], out_host[2 * (3 + k) + 1]);
+        const E2 lead = gl::e2(out_host[2 * (6 + k)], out_host[2 * (6 + k) + 1]);
+        ok = ok && gl::eq(gl::add(gl::sub(gl::add(v1, v1), v0), gl::add(lead, lead)), want_at2[k]);
+    }
     printf("%-58s quads=%llu workgroups=%u : %s\n", name, (unsigned long long)n_quads, blocks, ok ? "ok" : "MISMATCH");
     for (int k = 0; k < dpk::PAIR12_SUMS; k++) printf("    sum %d = %016llx %016llx\n", k, (unsigned long long)out_host[2 * k], (unsigned long long)out_host[2 * k + 1]);
     if (!ok) failures++;
