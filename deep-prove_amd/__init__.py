@@ -764,10 +764,9 @@ def _flat_claims(claims):
     return points, evals
 
 
-def claims_batching_prove(ctx, polys, claims, transcript):
-    """Claims-batching sumcheck of the opening proof.  polys: per committed polynomial
-    the list of its chunk tables (Mle); claims: per polynomial a list of (point, eval).
-    Returns (proof[n, 3, 2], point[n, 2], chunk_evals[total_chunks, 2])."""
+def claims_batching_prover(ctx, polys, claims):
+    """The same statement as claims_batching_prove with the call's arguments marshalled once: returns run(transcript) ->
+    (proof[n, 3, 2], point[n, 2], chunk_evals[total_chunks, 2]), for callers that prove over the same tables repeatedly."""
     n = len(polys)
     cpp = (_u32 * n)(*[len(c) for c in polys])
     flat = [m.handle for c in polys for m in c]
@@ -775,14 +774,26 @@ def claims_batching_prove(ctx, polys, claims, transcript):
     npc = (_u32 * n)(*[len(c) for c in claims])
     points, evals = _flat_claims(claims)
     n_vars = max((len(c[0]).bit_length() - 1) for c in polys)
-    proof = np.zeros((n_vars, 3, 2), dtype=np.uint64)
-    point = np.zeros((n_vars, 2), dtype=np.uint64)
-    out = np.zeros((len(flat), 2), dtype=np.uint64)
-    nv = _u32(0)
-    ctx._chk_host(host.dph_claims_batching_prove(ctx._c, n, cpp, chunks, npc, _ptr(points), _ptr(evals), transcript._t, _ptr(proof), _ptr(point),
-                                                 _ptr(out), C.byref(nv)), "dph_claims_batching_prove")
-    assert nv.value == n_vars
-    return proof, point, out
+    keep = (polys, cpp, chunks, npc, points, evals)  # what the pointers below point into
+
+    def run(transcript):
+        proof = np.zeros((n_vars, 3, 2), dtype=np.uint64)
+        point = np.zeros((n_vars, 2), dtype=np.uint64)
+        out = np.zeros((len(flat), 2), dtype=np.uint64)
+        nv = _u32(0)
+        ctx._chk_host(host.dph_claims_batching_prove(ctx._c, n, keep[1], keep[2], keep[3], _ptr(keep[4]), _ptr(keep[5]), transcript._t, _ptr(proof),
+                                                     _ptr(point), _ptr(out), C.byref(nv)), "dph_claims_batching_prove")
+        assert nv.value == n_vars
+        return proof, point, out
+
+    return run
+
+
+def claims_batching_prove(ctx, polys, claims, transcript):
+    """Claims-batching sumcheck of the opening proof.  polys: per committed polynomial
+    the list of its chunk tables (Mle); claims: per polynomial a list of (point, eval).
+    Returns (proof[n, 3, 2], point[n, 2], chunk_evals[total_chunks, 2])."""
+    return claims_batching_prover(ctx, polys, claims)(transcript)
 
 
 def claims_batching_verify(shapes, claims, proof, chunk_evals, transcript):
