@@ -1823,6 +1823,16 @@ int32_t launch_poly_split_dispatch(dps_ctx *ctx, u32 nf, bool eq, bool skip1, dp
 }
 
 u32 blocks_for_pairs(u64 n_pairs) { return grid_for(n_pairs); }
+// Workgroups of a product launch (prod_kernel): one thread per pair up to MAX_BLOCKS workgroups -- and in the rounds where that
+// gives a thread fewer than four pairs (2^19 pairs and fewer), four pairs a thread down to 256 workgroups: fewer partial sums
+// to gather, fewer workgroups to hand the mail to, and these launches are latency by then (cfg3: 0.427 -> 0.422 ms with 512 and
+// 256 workgroups in rounds 5 and 6).  The launches of sums of several terms are arithmetic and keep a thread per pair
+// (with this rule cfg5 3.65 -> 3.79 ms, linking 1.01 -> 1.09).
+u32 product_blocks(u64 n_pairs)
+{
+    const u32 full = grid_for(n_pairs), few = grid_for(n_pairs, dpk::BLOCK * 4);
+    return std::min<u32>(full, std::max<u32>(few, 256));
+}
 
 }  // namespace
 
@@ -2679,7 +2689,7 @@ void SessionSetup::plan_first_two_rounds()
     // (a lane of that launch adds up its quads without carries)
     if (((u64)1 << (n_vars - 2)) > dpk::PAIR12_MAX_STEPS * PAIR12_BLOCKS * dpk::WAVE) return;
     if (!sc->eq_info->fact_built || sc->eq_info->fact_levels < 3) return;
-    if (((u64)blocks_for_pairs(1ull << (n_vars - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return;
+    if (((u64)product_blocks(1ull << (n_vars - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return;
     // (round 2's p(1) comes from the claim: its scale must not vanish at 1)
     const E2 rho2 = sc->eq_info->point[1];
     if ((rho2.c0 == 0 && rho2.c1 == 0) || (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0)) return;
@@ -3590,15 +3600,15 @@ int32_t FusedRound::product_launch_ahead()
                 skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
             }
             dpk::ProdArgs an = sc->fast_args[j + 1];
-            if (has_eq) set_eq_weights(an, j + 1, blocks_for_pairs(n_pairs >> 1));
+            if (has_eq) set_eq_weights(an, j + 1, product_blocks(n_pairs >> 1));
             an.r0 = an.r1 = 0;
             an.skip1 = skip1_next ? 1 : 0;
             an.wait_first = 1;
             an.spin_limit = wait_units(ctx, AHEAD_SPIN_LIMIT);
             an.mail = ctx->d_pinned + (ctx->res_off - 64);
-            an.relay = blocks_for_pairs(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
+            an.relay = product_blocks(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
             dpk::FastFin fn = ff;
-            fn.n_blocks = blocks_for_pairs(n_pairs >> 1);
+            fn.n_blocks = product_blocks(n_pairs >> 1);
             fn.seq = next_seq;
             fn.slots = slots_for(fn.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
             sc->wait_slots = slots_for(fn.n_blocks);
@@ -3741,7 +3751,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
     if (ctx->tail_owner != sc) tail_abort(ctx);
     const u32 live = sc->n_vars - j + 1;
     const u64 n_pairs = 1ull << (live - 1);
-    u32 blocks = blocks_for_pairs(n_pairs);
+    u32 blocks = sc->fast ? product_blocks(n_pairs) : blocks_for_pairs(n_pairs);
     // constant terms: c summed over 2^(live-1) suffixes at every evaluation point
     E2 cst = gl::mul_base(sc->const_sum, h_pow(2, live - 1));
     dpk::FinArgs fa;
