@@ -1044,6 +1044,7 @@ struct Pair12Args {
 constexpr int PAIR12_BLOCK = 3 * WAVE;
 constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's three, pair 1's three, the three of the slopes along x1
 constexpr int PAIR12_SEQ_SLOT = 62, PAIR12_CHK_SLOT = 63;
+constexpr u32 PAIR12_LEAD = 4, PAIR12_LEAD_SPINS = 1u << 16;  // steps the other rows may be ahead of row 2; polls before they go on anyway
 constexpr u64 PAIR12_MAX_STEPS = 1024;  // quads a lane can add up without a carry (see the kernel)
 static_assert(2 * PAIR12_SUMS <= PAIR12_SEQ_SLOT, "the sums fit the result area");
 
@@ -1065,6 +1066,7 @@ __device__ __forceinline__ void wave_sum_field(u64 (&v)[NV])
 __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 *__restrict__ partial, FastFin ff)
 {
     __shared__ int last_flag;
+    __shared__ u32 row2_done;  // steps the wavefront of row 2 has behind it
     // A lane's three sums of (product) x (high weight), unreduced and without carries: the weight's limbs are cut into
     // pieces of 22, 22 and 20 bits (it is the same for the whole workgroup: scalar work), so a 32-bit half of the product
     // times a piece stays below 2^54 and PAIR12_MAX_STEPS of them below 2^64.  Six multiply-adds per product and limb,
@@ -1129,19 +1131,35 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
             }
         };
         // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
+        // Row 2's steps are the dearer ones: left alone the other two wavefronts run ahead of it until the lines they
+        // have read are gone from the L2 when it asks for them (1.5 x the tables fetched).  So it says how far it is (a
+        // word in LDS, every second step), and the others do not go more than PAIR12_LEAD steps beyond that: they sleep,
+        // which leaves their SIMDs to the wavefronts that are behind.  The wait is bounded: only the traffic depends on it.
         u64 q = q0;
+        u32 done = 0;  // steps of this wavefront
         Raw wa, wb;
         if (q < a.n_quads) load_raw(q, wa);
         while (q < a.n_quads) {
+            if (!ROW2) {
+                for (u32 spin = 0; spin < PAIR12_LEAD_SPINS && __hip_atomic_load(&row2_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) + PAIR12_LEAD < done; spin++)
+                    __builtin_amdgcn_s_sleep(2);
+            }
             if (q + stride < a.n_quads) load_raw(q + stride, wb);
             step(wa);
             q += stride;
-            if (q >= a.n_quads) break;
-            if (q + stride < a.n_quads) load_raw(q + stride, wa);
-            step(wb);
-            q += stride;
+            done += 2;
+            if (q < a.n_quads) {
+                if (q + stride < a.n_quads) load_raw(q + stride, wa);
+                step(wb);
+                q += stride;
+            }
+            if (ROW2 && lane == 0) __hip_atomic_store(&row2_done, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
+        // (a wavefront of row 2 that is through lets the others run to their end)
+        if (ROW2 && lane == 0) __hip_atomic_store(&row2_done, 0x7FFFFFFFu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
+    if (threadIdx.x == 0) row2_done = 0;
+    __syncthreads();
     if (row == 2)
         run(std::true_type{});
     else
