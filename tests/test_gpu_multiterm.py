@@ -131,8 +131,9 @@ def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
                                                       (12, 13, 10, True), (16, 16, 8, False), (16, 9, 12, True), (17, 16, 8, False)])
 def test_more_tables_than_a_group_all_rounds_resident(dp, ctx, orc, n, n_tabs, n_terms, with_eq):
     """Up to 16 full-size tables whose first round fits the resident launches (2^15 pairs) run there from round 1,
-    as the stacked products of an einsum do; with 9 or more tables the last two rounds go one per trip.  n = 17 is
-    the first size that does not fit and runs the groups' launches."""
+    as the stacked products of an einsum do; the last rounds (one or two with so many tables and terms) are worked out
+    on the host from the entries the launch hands over.  n = 17 is the first size that does not fit and runs the
+    groups' launches."""
     gpu, host, terms = _instance(ctx, orc, 1300 + n + n_tabs, n, [n] * n_tabs, [], n_terms, 2, with_eq)
     # every table in some term: the stacked products first
     one = np.array([1, 0], dtype=np.uint64)
