@@ -10,6 +10,8 @@ import pytest
 
 from util import py_rng, rand_base, rand_e2
 
+P = 0xFFFFFFFF00000001
+
 pytestmark = pytest.mark.gpu
 
 
@@ -125,6 +127,35 @@ def test_eq_point_with_a_zero_coordinate(dp, ctx, orc, n, zero_at):
     one = np.array([1, 0], dtype=np.uint64)
     _check(dp, ctx, orc, n, [ctx.mle_from_base(f), ctx.mle_from_base(g), ctx.eq_build(pt)],
            [orc.embed_base(f), orc.embed_base(g), orc.eq_evals(pt)], [(one, [2, 0, 1])])
+
+
+@pytest.mark.parametrize("n,zeros", [(6, (5,)), (9, (8, 6)), (11, (10, 9, 7, 6)), (12, (11, 3))])
+@pytest.mark.parametrize("kind", ["product", "terms"])
+def test_last_rounds_on_the_host_with_zero_coordinates(dp, ctx, orc, n, zeros, kind):
+    """The rounds the host works out after the resident launch has left (and the last trips before them): with an eq
+    point that has zero coordinates there, p(1) cannot come from the claim in those rounds and is evaluated; with the
+    sum stated by the caller; round by round and through the callback entry."""
+    pt = rand_e2(n, 4100 + n)
+    for z in zeros:
+        pt[z] = 0
+    if kind == "product":
+        f, g = rand_base(1 << n, 4200 + n), rand_e2(1 << n, 4201 + n)
+        gpu, host = [ctx.mle_from_base(f), ctx.mle_from_ext2(g), ctx.eq_build(pt)], [orc.embed_base(f), g, orc.eq_evals(pt)]
+        terms = [(np.array([7, 9], dtype=np.uint64), [2, 0, 1])]
+    else:
+        gpu, host, terms = _instance(ctx, orc, 4300 + n, n, [n] * 5, [1], 6, 3, True, eq_point=pt)
+        terms.append((np.array([11, 0], dtype=np.uint64), []))  # and a constant term
+    _check(dp, ctx, orc, n, gpu, host, terms)
+    ref_proof, ref_point, ref_finals = orc.sc_prove(n, host, terms, orc.OracleTranscript(b"multi"))
+    # the same with the sum stated, round by round
+    claim = np.array([(int(ref_proof[0][0][k]) + int(ref_proof[0][1][k])) % P for k in range(2)], dtype=np.uint64)
+    s = ctx.session(n, gpu, terms)
+    s.set_claim(claim)
+    chal = None
+    for j in range(n):
+        assert (s.round(chal) == ref_proof[j]).all(), j
+        chal = ref_point[j]
+    assert (s.finish(chal) == ref_finals).all()
 
 
 @pytest.mark.parametrize("n,n_tabs,n_terms,with_eq", [(7, 16, 8, False), (8, 16, 8, False), (8, 16, 24, True), (9, 16, 8, False),
