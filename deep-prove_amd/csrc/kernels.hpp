@@ -941,6 +941,13 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x;
     if (FOLD) {
         Raw w;
+        // TWO: from the far end back.  The launch of the first two rounds has just walked the same tables upwards: what it
+        // read last is what the memory-side cache still holds.
+        u64 steps = 0;
+        if (TWO) {
+            steps = i < a.n_pairs ? (a.n_pairs - i + stride - 1) / stride : 0;
+            if (steps) i += (steps - 1) * stride;
+        }
         if (i < a.n_pairs) load_raw(i, w);
         if (a.wait_first) {
             // A launch made ahead of its round waits here for its challenge, with the operands of its first step already
@@ -953,11 +960,20 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
             rp = gl::prep(r);
             if (TWO) set_two(gl::e2(uniform64(box[MAIL_RA]), uniform64(box[MAIL_RA + 1])), r);
         }
-        for (; i < a.n_pairs; i += stride) {
-            E2 lo[NF], hi[NF], rest;
-            take(i, w, lo, hi, rest);
-            if (i + stride < a.n_pairs) load_raw(i + stride, w);
-            evaluate(lo, hi, rest);
+        if (TWO) {
+            for (; steps > 0; steps--, i -= stride) {
+                E2 lo[NF], hi[NF], rest;
+                take(i, w, lo, hi, rest);
+                if (steps > 1) load_raw(i - stride, w);
+                evaluate(lo, hi, rest);
+            }
+        } else {
+            for (; i < a.n_pairs; i += stride) {
+                E2 lo[NF], hi[NF], rest;
+                take(i, w, lo, hi, rest);
+                if (i + stride < a.n_pairs) load_raw(i + stride, w);
+                evaluate(lo, hi, rest);
+            }
         }
     } else {
         auto step = [&](u64 i, const Raw &w) {
