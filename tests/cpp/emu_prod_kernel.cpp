@@ -290,6 +290,7 @@ int main(int argc, char **argv)
     run_case<2, 2, true, false, true, false>({"launch made ahead, mail relayed by the first workgroup", 4500, 18, false, 2});
     // sources folded twice on the way in (round 3 behind the launch of the first two rounds): challenges in the arguments, by mail
     run_case<2, 2, true, false, true, false, true>({"two folds on the way in", 700, 3, false, 0});
+    run_case<2, 2, true, false, true, false, true>({"two folds on the way in, ten steps a thread (walked from the far end back), ragged", 4900, 2, false, 0});
     run_case<2, 2, true, false, false, false, true>({"two folds on the way in, t = 1 evaluated, by mail", 300, 2, true, 1});
     // the first two rounds from one pass: one workgroup, several (ticket and gather by the first wavefront)
     run_first_two_rounds("first two rounds, one workgroup", 50, 1);
