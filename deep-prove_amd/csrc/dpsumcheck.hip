@@ -2686,8 +2686,6 @@ void SessionSetup::plan_first_two_rounds()
     sc->pair12 = false;
     if (!sc->fast || sc->fast_eq < 0 || sc->fast_nf != 2 || n_mles != 3 || sc->fast_nb[1] != 2) return;
     if (n_vars < dpk::EQ_LO_BITS + 3 || (sc->tail_j0 && sc->tail_j0 <= 3)) return;
-    // (a lane of that launch adds up its quads without carries)
-    if (((u64)1 << (n_vars - 2)) > dpk::PAIR12_MAX_STEPS * PAIR12_BLOCKS * dpk::WAVE) return;
     if (!sc->eq_info->fact_built || sc->eq_info->fact_levels < 3) return;
     if (((u64)product_blocks(1ull << (n_vars - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return;
     // (round 2's p(1) comes from the claim: its scale must not vanish at 1)

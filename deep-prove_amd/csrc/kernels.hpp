@@ -1061,7 +1061,6 @@ constexpr int PAIR12_BLOCK = 3 * WAVE;
 constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's three, pair 1's three, the three of the slopes along x1
 constexpr int PAIR12_SEQ_SLOT = 62, PAIR12_CHK_SLOT = 63;
 constexpr u32 PAIR12_LEAD = 4, PAIR12_LEAD_SPINS = 1u << 16;  // steps the other rows may be ahead of row 2; polls before they go on anyway
-constexpr u64 PAIR12_MAX_STEPS = 1024;  // quads a lane can add up without a carry (see the kernel)
 static_assert(2 * PAIR12_SUMS <= PAIR12_SEQ_SLOT, "the sums fit the result area");
 
 // sums over the wavefront of canonical values (as block_sum does it: 22-bit pieces added as integers), valid in lane 63
@@ -1083,19 +1082,16 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
 {
     __shared__ int last_flag;
     __shared__ u32 row2_done;  // steps the wavefront of row 2 has behind it
-    // A lane's three sums of (product) x (high weight), unreduced and without carries: the weight's limbs are cut into
-    // pieces of 22, 22 and 20 bits (it is the same for the whole workgroup: scalar work), so a 32-bit half of the product
-    // times a piece stays below 2^54 and PAIR12_MAX_STEPS of them below 2^64.  Six multiply-adds per product and limb,
-    // nothing else.  lz[k][c][i][j]: sum k, weight limb c, product half i, piece j.
-    u64 lz[3][2][2][3];
+    // A lane's three sums of (product) x (high weight), unreduced, their carries counted (gl::E2Acc).  Sums without carries
+    // (the weight's limbs cut into 22-bit pieces, six multiply-adds per product and limb and nothing else) make the loop
+    // 7 % shorter and cost 22 more registers -- 136, a few more than four wavefronts per SIMD allow.  Three per SIMD is
+    // exactly what this launch's 1024 workgroups of three wavefronts fill the GPU with, with no room to spare: behind
+    // a launch of a few workgroups (which every launch is that a caller makes before a proof, the eq build among them) the
+    // dispatcher places some workgroups where they have to wait for others to finish, and the launch takes 105 us instead
+    // of 80.  With room for a fourth wavefront it takes 86 to 90 us wherever its workgroups land.
+    gl::E2Acc lz[3];
 #pragma unroll
-    for (int k = 0; k < 3; k++)
-#pragma unroll
-        for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 3; j++) lz[k][c][i][j] = 0;
+    for (int k = 0; k < 3; k++) lz[k] = gl::e2acc_zero();
     const u32 lane = threadIdx.x & (WAVE - 1);
     const u32 row = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const u64 stride = (u64)gridDim.x * WAVE;
@@ -1132,19 +1128,10 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
                 gl_ = gl::sub(w.g1.x, w.g0.x);
                 gh = gl::sub(w.g1.y, w.g0.y);
             }
-            const u64 pr[3] = {gl::mul_any(fl, gl_), gl::mul_any(fh, gh), gl::mul_any(gl::sub(fh, fl), gl::sub(gh, gl_))};
-            const u64 hw[2] = {w.h0, w.h1};
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const u32 piece[3] = {(u32)hw[c] & 0x3FFFFFu, (u32)(hw[c] >> 22) & 0x3FFFFFu, (u32)(hw[c] >> 44)};
-#pragma unroll
-                for (int k = 0; k < 3; k++)
-#pragma unroll
-                    for (int j = 0; j < 3; j++) {
-                        lz[k][c][0][j] += (u64)(u32)pr[k] * piece[j];
-                        lz[k][c][1][j] += (u64)(u32)(pr[k] >> 32) * piece[j];
-                    }
-            }
+            const E2 H = gl::e2(w.h0, w.h1);
+            gl::acc_mul_base(lz[0], H, gl::mul_any(fl, gl_));
+            gl::acc_mul_base(lz[1], H, gl::mul_any(fh, gh));
+            gl::acc_mul_base(lz[2], H, gl::mul_any(gl::sub(fh, fl), gl::sub(gh, gl_)));
         };
         // two operand sets used in turn, so that a step's loads are in flight during the whole previous step
         // Row 2's steps are the dearer ones: left alone the other two wavefronts run ahead of it until the lines they
@@ -1186,20 +1173,7 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
     u64 v[6];
 #pragma unroll
     for (int k = 0; k < 3; k++) {
-        // sum k: the pieces back in place, word (i, j) times 2^(32 i + 22 j) (2^76 = 2^12 (2^32 - 1) mod p)
-        u64 limb[2];
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
-            gl::Acc t = gl::acc_zero();
-            gl::acc_prod(t, lz[k][c][0][0], 1ull);
-            gl::acc_prod(t, lz[k][c][0][1], 1ull << 22);
-            gl::acc_prod(t, lz[k][c][0][2], 1ull << 44);
-            gl::acc_prod(t, lz[k][c][1][0], 1ull << 32);
-            gl::acc_prod(t, lz[k][c][1][1], 1ull << 54);
-            gl::acc_prod(t, lz[k][c][1][2], (1ull << 44) - (1ull << 12));
-            limb[c] = gl::acc_reduce(t);
-        }
-        const E2 x = q0 < a.n_quads ? gl::mulp(gl::e2(limb[0], limb[1]), lp) : gl::e2_zero();
+        const E2 x = q0 < a.n_quads ? gl::mulp(gl::acc_reduce(lz[k]), lp) : gl::e2_zero();
         v[2 * k] = x.c0, v[2 * k + 1] = x.c1;
     }
     wave_sum_field<6>(v);
