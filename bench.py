@@ -25,9 +25,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 P = 0xFFFFFFFF00000001
-# Counters cannot be read from inside this script: the HBM bytes of one round-2 launch at n = 24 (rocprofv3 FETCH_SIZE and
+# Counters cannot be read from inside this script: the HBM bytes of the dominant launch (round 3) at n = 24 (rocprofv3 FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads for the library's plain copy kernel) and the vector-ALU issue
-# shares of rounds 1 and 2 are taken from the committed summaries of those runs, as "key: value" lines.
+# shares of the first launch and of the dominant one are taken from the committed summaries of those runs, as "key: value" lines.
 TRAFFIC_PROFILE = "profiles/prod_kernel_cfg3_n24_hbm_traffic.txt"
 VALU_PROFILE = "profiles/prod_kernel_cfg3_n24_valu.txt"
 
@@ -200,27 +200,6 @@ def other_config(args):
     return out
 
 
-def issue_costs():
-    """Loops of one vector instruction kind (dps_debug_issue_cost): nanoseconds per instruction and wavefront at 8 and at 2
-    wavefronts per SIMD, and cycles at the device's reported clock.  The device arithmetic (csrc/gl.hpp) is written for these."""
-    dp = importlib.import_module("deep-prove_amd")
-    ctx = dp.Context(0)
-    iters, rows, mhz, cus = 4000, [], 0.0, 0
-    for kind in range(dp.ISSUE_COST_KINDS):
-        row = {}
-        for waves in (8, 2):
-            name, ms, mhz, cus = ctx.issue_cost(kind, iters, waves)
-            ns = ms * 1e6 / (iters * 32 * waves)  # a SIMD issues for its `waves` wavefronts in turn
-            row["name"] = name
-            row[f"ns_per_instruction_at_{waves}_waves"] = round(ns, 3)
-            row[f"cycles_at_{waves}_waves"] = round(ns * mhz / 1e3, 2)
-        rows.append(row)
-    ctx.close()
-    return {"metric": "vector instruction issue cost", "unit": "ns per instruction and wavefront", "n_gpus": 1, "clock_mhz": mhz,
-            "compute_units": cus, "iterations": iters, "instructions_per_iteration": 32,
-            "note": "pairs are counted as two instructions; a SIMD's time is divided among its wavefronts", "kinds": rows}
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -228,16 +207,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--nvars", type=int, default=24, help="variables of the sum (24 is the benchmark configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", default="3", choices=["1", "2", "3", "4", "5", "opening", "linking", "issue-cost"],
-                    help="3 (default) is the benchmark configuration; the others time the remaining configurations the same way; "
-                         "issue-cost: what a vector instruction of each kind costs to issue on this GPU (not a proof)")
+    ap.add_argument("--config", default="3", choices=["1", "2", "3", "4", "5", "opening", "linking"],
+                    help="3 (default) is the benchmark configuration; the others time the remaining configurations the same way")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
-    if args.config == "issue-cost":
-        print(json.dumps(issue_costs()))
-        return
     if args.config != "3":
         print(json.dumps(other_config(args)))
         return

@@ -81,8 +81,6 @@ dev.dps_debug_copy.restype = _i32
 dev.dps_debug_copy.argtypes = [_vp, _u64, _u32, _vp]
 dev.dps_debug_read.restype = _i32
 dev.dps_debug_read.argtypes = [_vp, _u64, _u32, _vp]
-dev.dps_debug_issue_cost.restype = _i32
-dev.dps_debug_issue_cost.argtypes = [_vp, _i32, _u32, _u32, _vp, _vp, _vp, _vp]
 for _f in ["dps_ctx_create", "dps_ctx_destroy", "dps_ctx_sync", "dps_mle_from_base", "dps_mle_from_ext2", "dps_mle_info",
            "dps_mle_download", "dps_mle_free", "dps_eq_build", "dps_mle_evaluate", "dps_mle_fix_low", "dps_mle_fix_high",
            "dps_partial_eval", "dps_sc_begin", "dps_sc_set_claim", "dps_sc_degree", "dps_sc_round", "dps_sc_finish", "dps_sc_abort", "dps_sc_free",
@@ -119,12 +117,36 @@ dev.dps_logup_free.argtypes = [_vp]
 dev.dps_profile_enable.argtypes = [_vp, _i32]
 dev.dps_profile_reset.argtypes = [_vp]
 dev.dps_profile_read.argtypes = [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]
+dev.dps_ctx_pool_info.restype = _i32
+dev.dps_ctx_pool_info.argtypes = [_vp, _vp, _vp, _vp]
+dev.dps_device_set_resident_budget.restype = _i32
+dev.dps_device_set_resident_budget.argtypes = [_i32, _i32]
+dev.dps_device_resident_budget.restype = _i32
+dev.dps_device_resident_budget.argtypes = [_i32, _vp, _vp]
 host.dph_sumcheck_prove.restype = _i32
 host.dph_sumcheck_prove.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _vp]
 host.dph_sumcheck_prove_claimed.restype = _i32
 host.dph_sumcheck_prove_claimed.argtypes = [_vp, _u32, _vp, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp]
 host.dph_sumcheck_verify.restype = _i32
 host.dph_sumcheck_verify.argtypes = [_vp, _vp, _u32, _u32, _vp, _vp, _vp]
+
+
+def set_resident_budget(device, compute_units):
+    """Cap, in compute units, on what the launches that wait on the GPU (resident launches, launches made ahead) of all
+    contexts of this process may hold on `device` together; -1: the whole device (the default), 0: none ever waits
+    (dps_device_set_resident_budget)."""
+    rc = dev.dps_device_set_resident_budget(device, compute_units)
+    if rc != 0:
+        raise DpsError(rc, "dps_device_set_resident_budget")
+
+
+def resident_budget(device):
+    """(compute units held now by waiting launches, cap in force) on `device` (dps_device_resident_budget)"""
+    used, cap = C.c_int32(0), C.c_int32(0)
+    rc = dev.dps_device_resident_budget(device, C.byref(used), C.byref(cap))
+    if rc != 0:
+        raise DpsError(rc, "dps_device_resident_budget")
+    return used.value, cap.value
 
 
 def _ptr(a):
@@ -373,6 +395,12 @@ class Context:
         if rc != 0:
             raise DpsError(rc, f"{what}: {host.dph_last_error().decode()}")
 
+    def pool_info(self):
+        """(device blocks handed out, blocks cached for reuse, bytes of both) (dps_ctx_pool_info)"""
+        a, b, c = C.c_uint64(0), C.c_uint64(0), C.c_uint64(0)
+        self._chk(dev.dps_ctx_pool_info(self._c, C.byref(a), C.byref(b), C.byref(c)), "dps_ctx_pool_info")
+        return a.value, b.value, c.value
+
     def sync(self):
         self._chk(dev.dps_ctx_sync(self._c), "dps_ctx_sync")
 
@@ -568,19 +596,6 @@ def _read_ms(self, n_bytes, reps=10):
 
 
 Context.read_ms = _read_ms
-
-
-def _issue_cost(self, kind, iters=4000, waves_per_simd=8):
-    """(name, ms, clock in MHz, compute units) of a launch of `iters` x 32 vector instructions of one kind per wavefront
-    (dps_debug_issue_cost)"""
-    ms, name, khz, cus = C.c_double(0), C.c_char_p(), C.c_int32(0), C.c_int32(0)
-    self._chk(dev.dps_debug_issue_cost(self._c, kind, iters, waves_per_simd, C.byref(ms), C.byref(name), C.byref(khz), C.byref(cus)),
-              "dps_debug_issue_cost")
-    return name.value.decode(), ms.value, khz.value / 1e3, cus.value
-
-
-Context.issue_cost = _issue_cost
-ISSUE_COST_KINDS = 18
 
 
 # ---- einsum and LogUp drivers of the host mirror ----

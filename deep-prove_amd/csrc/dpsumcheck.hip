@@ -78,6 +78,7 @@ struct dps_ctx {
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
     u64 seq = 0;                // last sequence number handed to a launch
     struct dps_sc *tail_owner = nullptr;  // session whose tail kernel is resident on the stream
+    u32 units_held = 0;         // compute units of the device's ledger that launch holds (admit_waiting_launch)
     u64 *ws = nullptr;          // this device's copy of the allocation-free entry point's work area
     bool profiling = false;
     std::vector<ProfRec> recs;
@@ -156,6 +157,66 @@ int32_t work_area_of_device(int device, u64 **out)
     }
     *out = ptr_of[device];
     return DPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Admission of launches that wait on the GPU.
+//
+// Some launches stay on the GPU while the host takes its turn: the resident launches of the late rounds (their
+// workgroups hold a compute unit each from the first trip to the last, and a trip completes only when every one of them
+// has added its share) and the launches made ahead of their round (they wait for the challenge by mail, the large
+// ones behind their first workgroup, which passes it on).  Contexts are used from different threads, so several such
+// launches can meet on one GPU; if two of them were each placed in part, neither could ever complete -- each would
+// wait for workgroups that find no room while the other waits.  So every launch that waits takes its place in a
+// ledger of the device first: one compute unit per workgroup (a workgroup touches one compute unit, and any workgroup
+// fits an untouched one, so launches admitted together are placed together, in whatever order their workgroups
+// arrive), up to the device's number of compute units.  A launch that does not get its place is not made: a round
+// that would have been launched ahead is launched when its challenge is there, and a session whose resident launch
+// is refused runs the same rounds as launches of their own.  The results are the same bits either way.
+// Launches that wait for nothing (all others) come and go by themselves and are not counted.
+// ---------------------------------------------------------------------------
+struct DeviceLedger {
+    std::mutex mu;
+    int total = -1;  // compute units of the device (-1: not asked yet)
+    int limit = -1;  // the caller's limit (dps_device_set_resident_budget; -1: none)
+    int used = 0;
+};
+DeviceLedger &ledger_of(int device)
+{
+    static DeviceLedger ledgers[WS_MAX_DEVICES];
+    return ledgers[device];
+}
+
+// `together`: the launch makes progress only with all of its workgroups on the GPU (refused when the device is too
+// small for that); a launch whose workgroups each run to the end once the mail is there takes at most the whole budget.
+bool admit_waiting_launch(dps_ctx *ctx, u32 workgroups, bool together)
+{
+    DeviceLedger &l = ledger_of(ctx->device);
+    std::lock_guard<std::mutex> lock(l.mu);
+    // (a context has one waiting launch at a time: whatever it still holds is of a launch that has ended)
+    l.used -= (int)ctx->units_held;
+    ctx->units_held = 0;
+    const int budget = l.limit >= 0 ? std::min(l.limit, l.total) : l.total;
+    int want = (int)std::min<u32>(workgroups, 1u << 20);
+    if (want > budget) {
+        if (together) return false;
+        want = budget;
+    }
+    if (want <= 0 || l.used + want > budget) return false;
+    l.used += want;
+    ctx->units_held = (u32)want;
+    return true;
+}
+
+// the context's waiting launch has had its last mail (or was told to leave and has left): its place is free again
+void waiting_launch_over(dps_ctx *ctx)
+{
+    ctx->tail_owner = nullptr;
+    if (!ctx->units_held) return;
+    DeviceLedger &l = ledger_of(ctx->device);
+    std::lock_guard<std::mutex> lock(l.mu);
+    l.used -= (int)ctx->units_held;
+    ctx->units_held = 0;
 }
 
 // A resident tail kernel blocks the stream until its session finishes.  Any other
@@ -439,6 +500,13 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
     if (hipStreamCreate(&ctx->stream) != hipSuccess) return bail(DPS_ERR_HIP);
     // (the context's device is current here)
     if (int32_t rc = work_area_of_device(device, &ctx->ws); rc != DPS_OK) return bail(rc);
+    {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) return bail(DPS_ERR_HIP);
+        DeviceLedger &l = ledger_of(device);
+        std::lock_guard<std::mutex> lock(l.mu);
+        l.total = cus;
+    }
     // Lagrange weights: a polynomial of degree k known at 0..k, evaluated at t <= 8
     std::vector<u64> lag(9 * 9 * 9, 0);
     for (u32 k = 0; k <= 8; k++)
@@ -493,6 +561,7 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
     (void)hipStreamSynchronize(ctx->stream);
+    waiting_launch_over(ctx);
     prof_collect(ctx);
     for (auto e : ctx->ev_pool) (void)hipEventDestroy(e);
     if (ctx->stage_event) (void)hipEventDestroy(ctx->stage_event);
@@ -505,12 +574,44 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
     return DPS_OK;
 }
 
+extern "C" int32_t dps_device_set_resident_budget(int32_t device, int32_t compute_units)
+{
+    if (device < 0 || device >= WS_MAX_DEVICES || compute_units < -1) return DPS_ERR_INVALID;
+    DeviceLedger &l = ledger_of(device);
+    std::lock_guard<std::mutex> lock(l.mu);
+    l.limit = compute_units;
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_device_resident_budget(int32_t device, int32_t *in_use, int32_t *budget)
+{
+    if (device < 0 || device >= WS_MAX_DEVICES) return DPS_ERR_INVALID;
+    DeviceLedger &l = ledger_of(device);
+    std::lock_guard<std::mutex> lock(l.mu);
+    if (in_use) *in_use = l.used;
+    // (before the first context on the device its size is not known: -1)
+    if (budget) *budget = l.total < 0 ? -1 : (l.limit >= 0 ? std::min(l.limit, l.total) : l.total);
+    return DPS_OK;
+}
+
 extern "C" int32_t dps_ctx_sync(dps_ctx *ctx)
 {
     if (!ctx) return DPS_ERR_INVALID;
     DeviceGuard g(ctx->device);
     tail_abort(ctx);
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return DPS_OK;
+}
+
+extern "C" int32_t dps_ctx_pool_info(const dps_ctx *ctx, uint64_t *blocks_in_use, uint64_t *blocks_cached, uint64_t *bytes)
+{
+    if (!ctx) return DPS_ERR_INVALID;
+    u64 total = 0;
+    for (const auto &kv : ctx->live_blocks) total += kv.second;
+    for (const auto &kv : ctx->free_blocks) total += kv.first;
+    if (blocks_in_use) *blocks_in_use = ctx->live_blocks.size();
+    if (blocks_cached) *blocks_cached = ctx->free_blocks.size();
+    if (bytes) *bytes = total;
     return DPS_OK;
 }
 
@@ -1552,6 +1653,16 @@ void send_mail(dps_ctx *ctx, u64 seq)
 // gone -- it says "leave" under a sequence number that the launch made in its place will wait for again.
 void reset_device_words(dps_ctx *ctx) { (void)hipMemsetAsync(ctx->d_counter, 0, COUNTER_BYTES, ctx->stream); }
 
+// ... and, once the stream has drained, what such a launch published part-way: the counter words of a trip are accepted
+// by a 7-bit tag, so a word nobody took must not stay for the trip that carries the same tag 128 sequence numbers later
+size_t slice_area_off(const dps_ctx *ctx);
+size_t slice_fin_off(const dps_ctx *ctx);
+void clear_resident_results(dps_ctx *ctx)
+{
+    for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
+    ctx->h_pinned[slice_fin_off(ctx) + dpk::SL_FIN_SEQ_SLOT] = 0;
+}
+
 void tail_abort(dps_ctx *ctx)
 {
     dps_sc *owner = ctx->tail_owner;
@@ -1560,6 +1671,7 @@ void tail_abort(dps_ctx *ctx)
     (void)hipStreamSynchronize(ctx->stream);
     __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
     reset_device_words(ctx);
+    clear_resident_results(ctx);
     owner->tail_running = false;
     // a launch that has had no mail yet has changed nothing: its session goes on with ordinary launches
     if (owner->wait_fresh)
@@ -1567,7 +1679,7 @@ void tail_abort(dps_ctx *ctx)
     else
         owner->broken = true;
     owner->wait_fresh = false;
-    ctx->tail_owner = nullptr;
+    waiting_launch_over(ctx);
 }
 
 // result area of the resident product launches (dpk::SL_AREA_WORDS words of the pinned buffer, behind the areas of resident groups)
@@ -1613,6 +1725,35 @@ int32_t launch_slice_dispatch(dps_ctx *ctx, bool terms, u32 nf, bool eq, u32 wor
     SLICE_VARIANTS(SK)
 #undef SK
     return fail(ctx, DPS_ERR_UNSUPPORTED, "no resident kernel for degree %u, eq %d, several terms %d", nf, (int)eq, (int)terms);
+}
+// Workgroups of a resident launch of the variant that one compute unit holds at once, with the LDS it is launched with
+// (the runtime's occupancy calculation; 0: such a workgroup does not fit, or no such variant).  Asked once per
+// variant, device and LDS size.
+template <int NF, bool EQ, bool TERMS>
+int slice_occupancy(dps_ctx *ctx, u32 n_tabs, u32 cap)
+{
+    static std::mutex mu;
+    static std::map<std::pair<int, size_t>, int> known;
+    const size_t lds = dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = known.find({ctx->device, lds});
+    if (it != known.end()) return it->second;
+    int n = 0;
+    if (lds > slice_lds_granted<NF, EQ, TERMS>(ctx) ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(&dpk::slice_kernel<NF, EQ, TERMS>), (int)dpk::SL_BLOCK, lds) != hipSuccess) {
+        (void)hipGetLastError();
+        n = 0;
+    }
+    known[{ctx->device, lds}] = n;
+    return n;
+}
+int slice_workgroups_per_cu(dps_ctx *ctx, bool terms, u32 nf, bool eq, u32 n_tabs, u32 cap)
+{
+#define SK(NF_, EQ_, T_) \
+    if (terms == T_ && nf == NF_ && eq == EQ_) return slice_occupancy<NF_, EQ_, T_>(ctx, n_tabs, cap);
+    SLICE_VARIANTS(SK)
+#undef SK
+    return 0;
 }
 // LDS a launch of the variant can have; 0: no such variant
 u32 slice_lds_limit(dps_ctx *ctx, bool terms, u32 nf, bool eq)
@@ -2013,6 +2154,20 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
     };
     if (pairs_of(j) > per_wg) add_stage((u32)(pairs_of(j) / per_wg));
     while (j <= n_gpu) add_stage(1);
+}
+
+// The session's resident launch found no place on the device (admit_waiting_launch): the rounds it would have run, and
+// those the host would have worked out behind it, are launches of their own like the rounds before them.  Every
+// round's launch was described at set-up whatever the plan, and the eq levels those rounds read are built.
+void drop_resident_plan(dps_sc *sc)
+{
+    sc->stages.clear();
+    sc->tail_j0 = 0;
+    sc->fin_len = 0;
+    sc->fin_pend = 0;
+    sc->host_rounds = 0;
+    std::fill(sc->round_kind.begin(), sc->round_kind.end(), 0);
+    std::fill(sc->round_wide.begin(), sc->round_wide.end(), 0);
 }
 
 }  // namespace
@@ -3052,6 +3207,7 @@ struct FusedRound {
     void form_message(const E2 *q);
     int32_t take_sums(u32 n_slots);
     int32_t end_waiting_launch();
+    bool admit_stages();
     int32_t launch_stages_at(u64 seq0);
     int32_t resident_round();
     Plan plan_round(u32 jj, bool skip1_jj) const;
@@ -3229,10 +3385,23 @@ int32_t FusedRound::end_waiting_launch()
         HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
         __atomic_store_n(mailbox(ctx) + dpk::MAIL_SEQ, (u64)0, __ATOMIC_RELEASE);
         reset_device_words(ctx);
+        clear_resident_results(ctx);
         sc->tail_running = false;
         sc->wait_fresh = false;
-        ctx->tail_owner = nullptr;
+        waiting_launch_over(ctx);
         return DPS_OK;
+}
+
+// The session's resident launches ask for their place on the device: the widest stage's workgroups, which hold a
+// compute unit each and all have to be there at once.
+bool FusedRound::admit_stages()
+{
+        u32 widest = 1;
+        for (const dps_sc::Stage &st : sc->stages) {
+            widest = std::max(widest, st.W);
+            if (slice_workgroups_per_cu(ctx, sc->poly, sc->fast_nf, sc->fast_eq >= 0, (u32)sc->slice_ids.size(), st.cap) < 1) return false;
+        }
+        return admit_waiting_launch(ctx, widest, true);
 }
 
 // The launches of the resident rounds, queued one behind the other: the trip that starts at the first resident
@@ -3388,13 +3557,15 @@ int32_t FusedRound::resident_round()
     if ((kind != 4 && j == sc->n_vars - sc->host_rounds) || rc != DPS_OK) {
         // with its last trip the kernel publishes what is left of the tables and exits
         sc->tail_running = false;
-        ctx->tail_owner = nullptr;
+        waiting_launch_over(ctx);
         if (rc == DPS_OK) sc->pairs_seq = sc->last_trip_seq;
     }
     if (rc != DPS_OK) {
         // the launch left without publishing (it gave up waiting, or the stream failed): nothing of it can be used again
+        // (the wait only fails once the stream has drained, so nothing of it is still to land)
         sc->broken = true;
         reset_device_words(ctx);
+        clear_resident_results(ctx);
     }
     CHK(rc);
     sc->round = j;
@@ -3513,7 +3684,10 @@ int32_t FusedRound::multi_term_round()
         stays = sc->wait_stays;
         slots_now = sc->wait_slots;
     } else {
-        const Plan p = plan_round(j, a.skip1 != 0);
+        Plan p = plan_round(j, a.skip1 != 0);
+        // a launch that stays needs its place on the device (one workgroup per group, all there at once); without it
+        // the round is a launch of its own
+        if (p.reside && !admit_waiting_launch(ctx, std::max<u32>(n_groups, 1), true)) p.reside = false;
         CHK(launch_round(j, p, a.skip1 != 0, false, fa.seq));
         stays = p.reside;
         slots_now = slots_of(p);
@@ -3531,7 +3705,7 @@ int32_t FusedRound::multi_term_round()
     if (!stays) {
         // the launch of this round ends with it
         sc->tail_running = false;
-        ctx->tail_owner = nullptr;
+        waiting_launch_over(ctx);
         // The next round's launch is made now, behind this one: by the time this round's message has crossed to
         // the host and the challenge is drawn, it is already on the GPU looking for its mail.  Only for rounds
         // of few workgroups (every workgroup polls the mailbox), and not while launches are being timed.
@@ -3545,10 +3719,13 @@ int32_t FusedRound::multi_term_round()
             const Plan pn = plan_round(j + 1, skip1_next);
             if (sc->tail_j0 && j + 1 == sc->tail_j0) {
                 // the rounds from here on are resident: their launches are queued now and wait for their first mail
-                CHK(launch_stages_at(ctx->seq + 1));
-                sc->wait_fresh = true;
-                sc->ahead_at = std::chrono::steady_clock::now();
-            } else {
+                // (when the device has room for them now; else the next round asks again)
+                if (admit_stages()) {
+                    CHK(launch_stages_at(ctx->seq + 1));
+                    sc->wait_fresh = true;
+                    sc->ahead_at = std::chrono::steady_clock::now();
+                }
+            } else if (admit_waiting_launch(ctx, pn.blocks * std::max<u32>(n_groups, 1), pn.reside)) {
                 CHK(launch_round(j + 1, pn, skip1_next, true, ctx->seq + 1));
                 sc->tail_running = true;
                 sc->tail_seq0 = ctx->seq + 1;
@@ -3571,7 +3748,7 @@ int32_t FusedRound::multi_term_round()
     if (stays && (rc != DPS_OK || j == sc->n_vars)) {
         // a resident launch exits after the last round; one that can finish has published the tables' last pairs with it
         sc->tail_running = false;
-        ctx->tail_owner = nullptr;
+        waiting_launch_over(ctx);
         if (rc == DPS_OK && sc->poly_finish_in_kernel) sc->pairs_seq = fa.seq;
     }
     CHK(rc);
@@ -3587,9 +3764,12 @@ int32_t FusedRound::product_launch_ahead()
         const u64 next_seq = ctx->seq + 1;
         bool made = false;
         if (sc->tail_j0 && j + 1 == sc->tail_j0) {
-            CHK(launch_stages_at(next_seq));
-            made = true;
-        } else {
+            // (when the device has room for the resident launches now; else the next round asks again)
+            if (admit_stages()) {
+                CHK(launch_stages_at(next_seq));
+                made = true;
+            }
+        } else if (admit_waiting_launch(ctx, product_blocks(n_pairs >> 1), false)) {
             // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
             // p(1) comes from the claim unless the scale vanishes at 1
             bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
@@ -3651,7 +3831,7 @@ int32_t FusedRound::product_round()
     }
     // this round's launch ends with the round
     sc->tail_running = false;
-    ctx->tail_owner = nullptr;
+    waiting_launch_over(ctx);
     CHK(product_launch_ahead());
     if (const int32_t rc = take_sums(slots_now); rc != DPS_OK) {
         sc->broken = true;
@@ -3727,7 +3907,7 @@ int32_t FusedRound::second_round_from_stash()
     prepare_message();
     form_message(q);
     sc->tail_running = false;
-    ctx->tail_owner = nullptr;
+    waiting_launch_over(ctx);
     CHK(product_launch_ahead());
     sc->prev_chal = r;
     sc->round = j;
@@ -3779,6 +3959,9 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         fr.sc = sc, fr.ctx = ctx, fr.j = j, fr.challenge = challenge, fr.evals_out = evals_out;
         fr.n_pairs = n_pairs, fr.blocks = blocks, fr.cst = cst, fr.fa = fa;
         CHK(fr.begin());
+        // the resident rounds begin here and their launch is not on the GPU yet: with no place for it on the device
+        // these rounds are launches of their own
+        if (sc->tail_j0 && j == sc->tail_j0 && !sc->tail_running && !fr.admit_stages()) drop_resident_plan(sc);
         if (sc->tail_j0 && j >= sc->tail_j0) return fr.resident_round();
         if (sc->pair12 && j == 1) return fr.first_two_rounds_launch();
         if (sc->pair12 && j == 2) return fr.second_round_from_stash();
@@ -3914,10 +4097,11 @@ extern "C" int32_t dps_sc_prove(dps_sc *sc, dps_round_fn fn, void *user, uint64_
 }
 
 // ---------------------------------------------------------------------------
-// DensePolynomial::evaluate for callers that must not allocate (code under HIP graph capture, tight serving loops):
+// DensePolynomial::evaluate for callers that must not allocate (tight serving loops, harnesses that forbid hipMalloc):
 // the same value as dps_mle_evaluate, with everything beyond the table and the result kept in `scratch`.
 // No hipMalloc, hipFree, stream wait or host allocation on the way; the result crosses through the context's
-// pinned result area like a round message.
+// pinned result area like a round message, and the call returns when it is there (the host polls for it, so this is
+// not a call to make under stream capture).
 // ---------------------------------------------------------------------------
 namespace {
 
@@ -3944,9 +4128,22 @@ extern "C" int32_t dps_mle_evaluate_noalloc(dps_ctx *ctx, const dps_mle *mle, co
                     dpk::WS_MAX_VARS);
     if (!canonical(point, 2 * (size_t)n)) return fail(ctx, DPS_ERR_INVALID, "dps_mle_evaluate_noalloc: point not canonical");
     if (!ctx->ws) return fail(ctx, DPS_ERR_STATE, "dps_mle_evaluate_noalloc: the context has no work area");
+    // (ending a launch that waits on the GPU for a session of this context would mean a stream wait and a memset)
+    if (ctx->tail_owner) return fail(ctx, DPS_ERR_STATE, "dps_mle_evaluate_noalloc: a session of this context has a launch waiting on the GPU");
+    if (mle->eq && !(mle->eq->built & 1)) {
+        // An eq table whose entries nobody has read yet is not in memory (building it takes a scratch block and host
+        // vectors), and need not be: the multilinear extension of eq(rho, .) at z is prod_i eq1(rho_i, z_i).
+        E2 v = gl::e2_one();
+        for (u32 i = 0; i < n; i++) v = gl::mul(v, h_eq1(mle->eq->point[i], gl::e2(point[2 * i], point[2 * i + 1])));
+        out[0] = v.c0;
+        out[1] = v.c1;
+        return DPS_OK;
+    }
     DeviceGuard g(ctx->device);
-    tail_abort(ctx);
-    CHK(plain_ready(mle));  // (an eq table that nobody has read yet: launches into its own storage, no allocation)
+    // every context on a GPU shares that GPU's work area: one call at a time per device, from the first launch until the
+    // result is here
+    static std::mutex area_in_use[WS_MAX_DEVICES];
+    std::lock_guard<std::mutex> lock(area_in_use[ctx->device]);
     dpk::WsPoint pt;
     memset(&pt, 0, sizeof pt);
     if (n) memcpy(pt.p, point, 16 * (size_t)n);
@@ -4236,60 +4433,5 @@ extern "C" int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps,
     pool_free(ctx, p);
     if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "read: %s", hipGetErrorString(e));
     if (avg_ms_out) *avg_ms_out = (double)ms / reps;
-    return DPS_OK;
-}
-
-// ---------------------------------------------------------------------------
-// what a vector instruction costs to issue (see issue_cost_kernel): the duration of a launch of `iters` iterations of
-// 32 instructions of one kind, at `waves_per_simd` wavefronts on every SIMD of the device
-// ---------------------------------------------------------------------------
-extern "C" int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t iters, uint32_t waves_per_simd, double *ms_out, const char **name_out,
-                                        int32_t *clock_khz_out, int32_t *compute_units_out)
-{
-    static const char *const names[dpk::ISSUE_COST_KINDS] = {"v_mov_b32", "v_add_u32", "v_add_co_u32", "v_add_co_u32 + v_addc_co_u32 (a pair, 2 wait states between)",
-                                                            "v_cmp_lt_u64", "v_lshl_add_u64", "v_mad_u64_u32 (running sum, carry out)", "v_mul_hi_u32", "v_add3_u32",
-                                                            "v_sub_co_u32 + v_cndmask_b32 of constants (a pair, 2 wait states between)",
-                                                            "v_cmp_lt_u32 + v_cndmask_b32 of registers (a pair, 2 wait states between)",
-                                                            "v_cndmask_b32 of registers (the mask not written in the loop)", "v_and_b32 / v_xor_b32 / v_or_b32 / v_sub_u32",
-                                                            "v_cmp_lt_u32 + three v_cndmask_b32 of registers", "v_cndmask_b32 of registers, mask set by s_mov_b64 every four",
-                                                            "v_cndmask_b32 of registers, mask in s[2:3], never written",
-                                                            "v_cmp_lt_u32 into s[2:3] + three v_cndmask_b32 of registers by s[2:3]",
-                                                            "v_cmp_lt_u32 + two v_cndmask_b32 of registers by vcc (a 64-bit select)"};
-    if (!ctx || kind < 0 || kind >= dpk::ISSUE_COST_KINDS || iters == 0 || waves_per_simd == 0 || waves_per_simd > 8)
-        return fail(ctx, DPS_ERR_INVALID, "dps_debug_issue_cost: bad argument");
-    DeviceGuard g(ctx->device);
-    tail_abort(ctx);
-    hipDeviceProp_t prop;
-    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
-    // a workgroup is one wavefront on each of a compute unit's four SIMDs
-    const u32 blocks = (u32)prop.multiProcessorCount * waves_per_simd;
-    void *p = nullptr;
-    CHK(pool_alloc(ctx, (size_t)blocks * dpk::BLOCK * 8, &p));
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    hipError_t e = hipEventCreate(&e0);
-    if (e == hipSuccess) e = hipEventCreate(&e1);
-    float best = 0.f;
-    for (int rep = 0; rep < 3 && e == hipSuccess; rep++) {
-        e = hipEventRecord(e0, ctx->stream);
-        switch (kind) {
-#define IC(K) case K: dpk::issue_cost_kernel<K><<<blocks, dpk::BLOCK, 0, ctx->stream>>>((u64 *)p, iters); break;
-            IC(0) IC(1) IC(2) IC(3) IC(4) IC(5) IC(6) IC(7) IC(8) IC(9) IC(10) IC(11) IC(12) IC(13) IC(14) IC(15) IC(16) IC(17)
-#undef IC
-        }
-        if (e == hipSuccess) e = hipGetLastError();
-        if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        float ms = 0.f;
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-        if (rep == 0 || ms < best) best = ms;
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    pool_free(ctx, p);
-    if (e != hipSuccess) return fail(ctx, DPS_ERR_HIP, "issue cost: %s", hipGetErrorString(e));
-    if (ms_out) *ms_out = (double)best;
-    if (name_out) *name_out = names[kind];
-    if (clock_khz_out) *clock_khz_out = prop.clockRate;
-    if (compute_units_out) *compute_units_out = prop.multiProcessorCount;
     return DPS_OK;
 }

@@ -2701,69 +2701,4 @@ __global__ __launch_bounds__(BLOCK) void read_kernel(const uint4 *__restrict__ s
     if (acc == 0x9e3779b9u) out[blockIdx.x] = acc;  // (practically never: the loads cannot be dropped, nothing is written)
 }
 
-// ---------------------------------------------------------------------------
-// What a vector instruction costs to issue: loops of one instruction kind (32 copies an iteration, four registers
-// feeding each other round), run at a chosen number of wavefronts per SIMD.  The arithmetic of gl.hpp is written for
-// what this measures; no counterpart in the reference.
-// ---------------------------------------------------------------------------
-constexpr int ISSUE_COST_KINDS = 18;
-constexpr int ISSUE_COST_COPIES = 32;
-#if defined(__HIPCC__)  // machine instructions by name: for the device compiler only
-#define DPK_R8(x) x x x x x x x x
-template <int KIND>
-__global__ void __launch_bounds__(BLOCK) issue_cost_kernel(u64 *out, u32 iters)
-{
-    u32 a = threadIdx.x * 2654435761u + 1, b = a ^ 0x9e3779b9u, c = a + 77, d = b + 13;
-    u64 x = a, y = b, z = c, w = d;
-    for (u32 i = 0; i < iters; i++) {
-        if (KIND == 0) asm volatile(DPK_R8("v_mov_b32 %0, %1\n v_mov_b32 %1, %2\n v_mov_b32 %2, %3\n v_mov_b32 %3, %0\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        if (KIND == 1) asm volatile(DPK_R8("v_add_u32 %0, %1, %2\n v_add_u32 %1, %2, %3\n v_add_u32 %2, %3, %0\n v_add_u32 %3, %0, %1\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        if (KIND == 2)
-            asm volatile(DPK_R8("v_add_co_u32 %0, vcc, %1, %2\n v_add_co_u32 %1, vcc, %2, %3\n v_add_co_u32 %2, vcc, %3, %0\n v_add_co_u32 %3, vcc, %0, %1\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 3)
-            asm volatile(DPK_R8("v_add_co_u32 %0, vcc, %1, %2\n s_nop 1\n v_addc_co_u32 %1, vcc, %2, %3, vcc\n v_add_co_u32 %2, vcc, %3, %0\n s_nop 1\n v_addc_co_u32 %3, vcc, %0, %1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 4) asm volatile(DPK_R8("v_cmp_lt_u64 vcc, %0, %1\n v_cmp_lt_u64 vcc, %1, %2\n v_cmp_lt_u64 vcc, %2, %3\n v_cmp_lt_u64 vcc, %3, %0\n") : "+v"(x), "+v"(y), "+v"(z), "+v"(w)::"vcc");
-        if (KIND == 5)
-            asm volatile(DPK_R8("v_lshl_add_u64 %0, %1, 0, %2\n v_lshl_add_u64 %1, %2, 0, %3\n v_lshl_add_u64 %2, %3, 0, %0\n v_lshl_add_u64 %3, %0, 0, %1\n") : "+v"(x), "+v"(y), "+v"(z), "+v"(w));
-        if (KIND == 6)
-            asm volatile(DPK_R8("v_mad_u64_u32 %0, s[4:5], %4, %5, %0\n v_mad_u64_u32 %1, s[6:7], %5, %6, %1\n v_mad_u64_u32 %2, s[8:9], %6, %7, %2\n v_mad_u64_u32 %3, s[10:11], %7, %4, %3\n")
-                         : "+v"(x), "+v"(y), "+v"(z), "+v"(w)
-                         : "v"(a), "v"(b), "v"(c), "v"(d)
-                         : "s4", "s5", "s6", "s7", "s8", "s9", "s10", "s11");
-        if (KIND == 7) asm volatile(DPK_R8("v_mul_hi_u32 %0, %1, %2\n v_mul_hi_u32 %1, %2, %3\n v_mul_hi_u32 %2, %3, %0\n v_mul_hi_u32 %3, %0, %1\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        if (KIND == 8) asm volatile(DPK_R8("v_add3_u32 %0, %1, %2, %3\n v_add3_u32 %1, %2, %3, %0\n v_add3_u32 %2, %3, %0, %1\n v_add3_u32 %3, %0, %1, %2\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        if (KIND == 9)
-            asm volatile(DPK_R8("v_sub_co_u32 %0, vcc, %1, %2\n s_nop 1\n v_cndmask_b32 %1, 0, -1, vcc\n v_sub_co_u32 %2, vcc, %3, %0\n s_nop 1\n v_cndmask_b32 %3, 0, -1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 10)
-            asm volatile(DPK_R8("v_cmp_lt_u32 vcc, %0, %1\n s_nop 1\n v_cndmask_b32 %0, %2, %3, vcc\n v_cmp_lt_u32 vcc, %2, %3\n s_nop 1\n v_cndmask_b32 %2, %0, %1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 11)
-            asm volatile(DPK_R8("v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 13)
-            asm volatile(DPK_R8("v_cmp_lt_u32 vcc, %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 14)
-            asm volatile(DPK_R8("s_mov_b64 vcc, s[2:3]\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 15)
-            asm volatile(DPK_R8("v_cndmask_b32 %0, %1, %2, s[2:3]\n v_cndmask_b32 %1, %2, %3, s[2:3]\n v_cndmask_b32 %2, %3, %0, s[2:3]\n v_cndmask_b32 %3, %0, %1, s[2:3]\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        if (KIND == 16)
-            asm volatile(DPK_R8("v_cmp_lt_u32 s[2:3], %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, s[2:3]\n v_cndmask_b32 %1, %2, %3, s[2:3]\n v_cndmask_b32 %2, %3, %0, s[2:3]\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"s2", "s3");
-        if (KIND == 17)
-            asm volatile(DPK_R8("v_cmp_lt_u32 vcc, %0, %1\n s_nop 1\n v_cndmask_b32 %0, %1, %2, vcc\n v_cndmask_b32 %1, %2, %3, vcc\n v_cmp_lt_u32 vcc, %2, %3\n s_nop 1\n v_cndmask_b32 %2, %3, %0, vcc\n v_cndmask_b32 %3, %0, %1, vcc\n")
-                         : "+v"(a), "+v"(b), "+v"(c), "+v"(d)::"vcc");
-        if (KIND == 12)
-            asm volatile(DPK_R8("v_and_b32 %0, %1, %2\n v_xor_b32 %1, %2, %3\n v_or_b32 %2, %3, %0\n v_sub_u32 %3, %0, %1\n") : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-    }
-    out[(u64)blockIdx.x * BLOCK + threadIdx.x] = x ^ y ^ z ^ w ^ a ^ b ^ c ^ d;
-}
-#undef DPK_R8
-#endif
-
 }  // namespace dpk

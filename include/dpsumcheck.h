@@ -23,7 +23,8 @@
  *   - Every function returns a dps_status; nothing throws or aborts.  Host
  *     buffers are borrowed for the duration of the call only.  A context owns one
  *     HIP stream; calls on one context must not overlap, different contexts may be
- *     used from different threads.
+ *     used from different threads at the same time (see dps_device_set_resident_budget
+ *     for how their launches share one GPU).
  */
 #ifndef DPSUMCHECK_H
 #define DPSUMCHECK_H
@@ -68,6 +69,17 @@ const char *dps_last_error(const dps_ctx *ctx);
 const char *dps_status_str(int32_t status);
 /* wait for everything queued on the context's stream */
 int32_t dps_ctx_sync(dps_ctx *ctx);
+/* Contexts on one GPU, several threads (the reference proves the chunks of a model concurrently from a thread pool,
+ * zkml/src/graph/executor.rs:148, zkml/src/iop/mod.rs:268-279).  Some launches of a session stay on the GPU while the
+ * host takes its turn (the resident launches of the late rounds, the launches made ahead of their round); launches of
+ * that kind from different contexts share the device through a process-wide ledger, one compute unit per workgroup,
+ * so that those admitted are always placed together and none waits for room another holds.  A launch that finds no
+ * place is not made and its rounds run as ordinary launches: same results, bit for bit, more launches.
+ * dps_device_set_resident_budget caps what all contexts of this process together may hold on `device` (compute units;
+ * -1: the whole device, the default; 0: no launch ever waits on the GPU) -- for a GPU shared with other work.
+ * dps_device_resident_budget reads the ledger: units held now, and the cap in force (-1 before the first context). */
+int32_t dps_device_set_resident_budget(int32_t device, int32_t compute_units);
+int32_t dps_device_resident_budget(int32_t device, int32_t *in_use, int32_t *budget);
 
 /* ---- table storage: DensePolynomial::{new, new_from_smart_slice, as_view, evals}
  *      (zkml/src/tensor/mod.rs:364,390,401; zkml/src/lookup/logup_gkr/circuit.rs:262-269) ---- */
@@ -118,12 +130,15 @@ int32_t dps_eq_build_many(dps_ctx *ctx, const uint64_t *const *points, const uin
 /* ---- DensePolynomial::{evaluate, fix_low_variables, fix_high_variables}
  *      (zkml/src/layers/einsum/prove.rs:208, zkml/src/tensor/mod.rs:1892, zkml/src/iop/prover.rs:448,509) ---- */
 int32_t dps_mle_evaluate(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*n */, uint32_t n, uint64_t out[2]);
-/* The same evaluation for callers that cannot allocate.  No counterpart in the reference: it is for code under HIP
- * graph capture, tight serving loops and harnesses that forbid hipMalloc.  The call makes no hipMalloc, hipFree or
- * host allocation and waits for no stream; its eq tables, partial sums and ticket counter live in a file-scope
- * device array of the library (144 KiB per GPU, held until the process ends).  At most 24 variables
- * (DPS_ERR_UNSUPPORTED beyond).  Every call on one GPU shares that GPU's array: calls that overlap on one GPU,
- * from this or another context, race. */
+/* The same evaluation for callers that cannot allocate.  No counterpart in the reference: it is for tight serving
+ * loops and harnesses that forbid hipMalloc.  The call makes no hipMalloc, hipFree or host allocation and waits for
+ * no stream (it returns when the value has crossed to the host, which it polls for: not a call to record under stream
+ * capture); its eq tables, partial sums and ticket counter live in a file-scope device array of the library (144 KiB
+ * per GPU, held until the process ends).  At most 24 variables (DPS_ERR_UNSUPPORTED beyond).  Every context on one
+ * GPU shares that GPU's array: the library lets one such call at a time use it, others wait their turn.  An eq table
+ * whose entries have not been read yet (dps_eq_build keeps a large one unmaterialised) is evaluated in closed form on
+ * the host.  DPS_ERR_STATE while a session of the context has a launch waiting on the GPU (between its rounds):
+ * ending that launch would take a stream wait. */
 int32_t dps_mle_evaluate_noalloc(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*n */, uint32_t n, uint64_t out[2]);
 /* point[j] binds variable j */
 int32_t dps_mle_fix_low(dps_ctx *ctx, const dps_mle *mle, const uint64_t *point /* 2*k */, uint32_t k, dps_mle **out);
@@ -200,7 +215,10 @@ int32_t dps_logup_layer(const dps_logup *lg, uint32_t k, dps_mle **num, dps_mle 
 int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8]);
 int32_t dps_logup_free(dps_logup *lg);
 
-/* ---- measurement: HIP-event timing of the library's own launches ---- */
+/* ---- measurement: the context's device memory, and HIP-event timing of the library's own launches ---- */
+/* Device blocks the context has taken from the driver (hipMalloc): those handed out, those cached for reuse, and the
+ * bytes of both.  Unchanged across a call means the call took nothing from the driver and gave nothing back. */
+int32_t dps_ctx_pool_info(const dps_ctx *ctx, uint64_t *blocks_in_use, uint64_t *blocks_cached, uint64_t *bytes);
 enum {
     DPS_K_EVAL_FIRST = 0, /* first-round evaluation of a product of full-size tables */
     DPS_K_FOLD_EVAL = 1,  /* fused fold + evaluation of a product */
@@ -238,13 +256,6 @@ int32_t dps_debug_field_op(dps_ctx *ctx, int32_t op, const uint64_t *a, const ui
 int32_t dps_debug_copy(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
 /* the same for a launch that only reads n_bytes (what a round's first evaluation is read against) */
 int32_t dps_debug_read(dps_ctx *ctx, uint64_t n_bytes, uint32_t reps, double *avg_ms_out);
-
-/* ---- what a vector instruction costs to issue: a launch of `iters` iterations of 32 instructions of one kind
- * (kind 0 .. 17, named in *name_out) at waves_per_simd (1 .. 8) wavefronts on every SIMD; returns the best of three
- *  launches in milliseconds, and the device's clock (kHz) and number of compute units.  No counterpart in the reference; the
- * device arithmetic is written for what this shows. */
-int32_t dps_debug_issue_cost(dps_ctx *ctx, int32_t kind, uint32_t iters, uint32_t waves_per_simd, double *ms_out, const char **name_out,
-                             int32_t *clock_khz_out, int32_t *compute_units_out);
 
 #ifdef __cplusplus
 }

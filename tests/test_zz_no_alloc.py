@@ -80,3 +80,98 @@ def test_evaluate_noalloc_full_size_and_limits(dp, ctx):
         small.zero_pad(5).evaluate_noalloc(rand_e2(5, 3))
     # the context is still usable
     assert (small.evaluate_noalloc(ps) == small.evaluate(ps)).all()
+
+
+def _device_free_bytes():
+    import torch
+
+    return torch.cuda.mem_get_info(0)[0]
+
+
+def test_evaluate_noalloc_takes_nothing_from_the_driver(dp, ctx, orc):
+    # neither the context's pool nor the device's free memory moves across the calls, whatever the table is --
+    # including an eq table of 20 variables whose entries have never been read (dps_eq_build keeps them
+    # unmaterialised: that one is evaluated in closed form, prod eq1(rho_i, z_i))
+    n = 20
+    rho, z = rand_e2(n, 34001), rand_e2(n, 34002)
+    eq = ctx.eq_build(rho)
+    base = ctx.mle_from_base(rand_base(1 << 18, 34003))
+    zb = rand_e2(18, 34004)
+    small_eq = ctx.eq_build(rand_e2(11, 34005))
+    zs = rand_e2(11, 34006)
+    ctx.sync()
+    pool0, free0 = ctx.pool_info(), _device_free_bytes()
+    got_eq = eq.evaluate_noalloc(z)
+    got_base = base.evaluate_noalloc(zb)
+    got_small = small_eq.evaluate_noalloc(zs)
+    assert ctx.pool_info() == pool0 and _device_free_bytes() == free0
+    assert (got_eq == orc.identity_eval(rho, z)).all()
+    # the allocating call builds the table's entries and evaluates them: the same element
+    assert (eq.evaluate(z) == got_eq).all()
+    # ... and once they are there the entry point reads them like any table's
+    pool1 = ctx.pool_info()
+    assert (eq.evaluate_noalloc(z) == got_eq).all() and ctx.pool_info() == pool1
+    assert (got_base == base.evaluate(zb)).all() and (got_small == small_eq.evaluate(zs)).all()
+
+
+def test_evaluate_noalloc_refuses_while_a_launch_waits(dp, ctx, orc):
+    # between the rounds of a small product session its resident launch waits on the GPU for the next challenge: ending
+    # it would take a stream wait, so the entry point says so instead, and the session goes on undisturbed
+    n = 12
+    f, g = rand_base(1 << n, 35001), rand_base(1 << n, 35002)
+    terms = [(np.array([1, 0], np.uint64), [0, 1])]
+    mf, mg = ctx.mle_from_base(f), ctx.mle_from_base(g)
+    other = ctx.mle_from_base(rand_base(1 << 6, 35003))
+    zo = rand_e2(6, 35004)
+    want_other = other.evaluate(zo)
+    tr = dp.Transcript(b"busy")
+    tr.append_u64(n)
+    tr.append_u64(2)
+    s = ctx.session(n, [mf, mg], terms)
+    msgs, point = [], []
+    ch = None
+    for j in range(1, n + 1):
+        msgs.append(s.round(ch))
+        if j == 2:
+            with pytest.raises(dp.DpsError) as e:
+                other.evaluate_noalloc(zo)
+            assert e.value.status == 4
+        tr.append_scalars(msgs[-1])
+        ch = tr.challenge_scalar()
+        point.append(ch)
+    finals = s.finish(ch)
+    otr = orc.OracleTranscript(b"busy")
+    oproof, opoint, ofinals = orc.sc_prove(n, [orc.embed_base(f), orc.embed_base(g)], terms, otr)
+    assert (np.array(msgs) == oproof).all() and (np.array(point) == opoint).all() and (finals == ofinals).all()
+    assert (other.evaluate_noalloc(zo) == want_other).all()
+
+
+def test_evaluate_noalloc_from_two_threads(dp, orc):
+    # two contexts on two threads share the GPU's one work area: the library lets one call at a time use it
+    import threading
+
+    errors = []
+
+    def worker(seed):
+        try:
+            c = dp.Context(0)
+            tabs = [(c.mle_from_ext2(rand_e2(1 << k, seed + k)), rand_e2(k, seed + 100 + k)) for k in (7, 13, 16)]
+            want = [t.evaluate(z) for t, z in tabs]
+            for it in range(50):
+                t, z = tabs[it % 3]
+                got = t.evaluate_noalloc(z)
+                if not (got == want[it % 3]).all():
+                    errors.append("thread %d call %d: %r != %r" % (seed, it, got, want[it % 3]))
+                    return
+            del tabs
+            c.close()
+        except Exception as ex:  # noqa: BLE001 -- reported by the main thread
+            errors.append("thread %d: %r" % (seed, ex))
+
+    ts = [threading.Thread(target=worker, args=(36000 + 1000 * i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join(120)
+    assert not any(t.is_alive() for t in ts), "a thread did not finish"
+    assert not errors, errors
