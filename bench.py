@@ -114,6 +114,11 @@ def other_config(args):
         extra["with_upload_of_int64_host_tensors_ms"] = round(_timed(lambda: dp.einsum_prove(ctx, ops, lhs, rhs, claims, dp.Transcript(b"bench")), args.steps, args.warmup)[0], 4)
         extra["same_bits_as_host_tensor_path"] = exact_vs_host_path
         extra["note"] = "value: int64 tensors resident on the device (weights and activations uploaded once, outside the step)"
+        if orc:
+            # the checker's restatement of the whole driver: partial evaluations, batched sumcheck, input claims
+            cpu_ms, _, (ref, _otr) = _timed(lambda: orc.einsum_prove(ops, lhs, rhs, claims, b"bench"), 1, 0)
+            exact = bool((got["proof"] == ref["proof"]).all() and (got["evaluations"] == ref["evaluations"]).all()
+                         and all((a[0] == b[0]).all() and (a[1] == b[1]).all() for a, b in zip(got["claims"], ref["claims"])))
     elif cfg == "5":
         log_l, log_t = 22, 16
         rng = np.random.Generator(np.random.PCG64(600))
@@ -424,6 +429,20 @@ def main():
         }
         out["speedup_vs_cpu"] = round(cpu_ms / ms_per_step, 1)
         out["bit_exact"] = bit_exact
+        del tabs
+    if n == 24:
+        # The remaining configurations in the same record: a few steps each of the same measurement `--config X` makes
+        # (a step = one complete proof, inputs resident in HBM), the CPU checker run once each to compare the bits.
+        del prover, claimed, mf, mg, me
+        others = {}
+        for name, key in (("1", "cfg1"), ("2", "cfg2"), ("4", "cfg4"), ("5", "cfg5"), ("opening", "opening"), ("linking", "linking")):
+            sub = argparse.Namespace(config=name, steps=5, warmup=2, no_cpu=args.no_cpu)
+            res = other_config(sub)
+            others[key] = {"ms": res["value"], "min_step_ms": res["min_step_ms"], "steps": sub.steps, "warmup": sub.warmup,
+                           "bit_exact": res.get("bit_exact"), "workload": res["config"]["workload"]}
+            if "cpu_baseline" in res:
+                others[key]["cpu_port_ms"] = res["cpu_baseline"]["value"]
+        out["other_configs"] = others
     print(json.dumps(out))
 
 

@@ -7,6 +7,7 @@
 // workgroup, and grids sized to a few workgroups per CU.
 #pragma once
 #include <type_traits>
+#include <utility>
 
 #include "gl.hpp"
 
@@ -1694,6 +1695,52 @@ struct PolyArgs {
     u64 *raw_out;    // nullptr: a single workgroup, which publishes to the main result area
 };
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_each(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_each(f, std::make_integer_sequence<int, N>{});
+}
+
+// A node of the nested program at depth D: starts from its constant, adds table * c for every LEAF, table * (child's
+// value) for every child (ENTER D + 1 ... LEAVE D + 1, walked by the next depth's function), and ends at the LEAVE of its
+// own depth, which it leaves for its parent to read the table from (or at the end of the program: the root).
+// `op(o)`: operation o; `table(slot)`: the slot's table at the evaluation point in hand.
+template <int D, int MAXD, typename OpAt, typename TableAt>
+__device__ __forceinline__ E2 poly_walk(u32 &pc, u32 n_ops, E2 acc, OpAt &&op, TableAt &&table)
+{
+    while (pc < n_ops) {
+        const PolyOp &o = op(pc);
+        const u32 code = __builtin_amdgcn_readfirstlane(o.code);
+        const u32 kind = code & 3, sl = code >> 8;
+        if (kind == POLY_OP_LEAF) {
+            gl::E2P cp;
+            cp.c0 = o.c0;
+            cp.c1 = o.c1;
+            cp.w = o.w;
+            acc = gl::fma(table(sl), cp, acc);
+            pc++;
+        } else if (kind == POLY_OP_ENTER) {
+            pc++;
+            if constexpr (D < MAXD) {
+                const E2 child = poly_walk<D + 1, MAXD>(pc, n_ops, gl::e2(o.c0, o.c1), op, table);
+                // (the child stopped at its LEAVE, which names the table on the edge to it)
+                const u32 edge = __builtin_amdgcn_readfirstlane(op(pc).code) >> 8;
+                acc = gl::fma(child, gl::prep(table(edge)), acc);
+                pc++;
+            }
+        } else {
+            break;
+        }
+    }
+    return acc;
+}
+
 template <int NF, bool EQ, bool SKIP1>
 __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict__ partial, FastFin ff)
 {
@@ -1797,49 +1844,26 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
             for (u32 k = 0; k < n_tabs; k++) take(g.tab[k], k);
         gl::E2P restp = gl::prep(gl::e2_one());
         if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
-#pragma unroll
-        for (int t = 0; t < NP; t++) {
+        // (one copy of the body per evaluation point, t a compile-time constant in each)
+        static_for<NP>([&](auto point) {
+            constexpr int t = decltype(point)::value;
             if (!(t == 1 && SKIP1)) {
                 E2 gsum;
                 if (n_ops) {
                     // the nested program: every index below is a compile-time constant inside its case.  Read from
                     // the kernel arguments an operation arrives in scalar registers and its branches are uniform.
-                    E2 hv[NF + 2];
-#pragma unroll
-                    for (int d = 0; d < NF + 2; d++) hv[d] = gl::e2_zero();
-                    auto step = [&](const PolyOp &op) {
-                        const u32 kind = op.code & 3, dep = (op.code >> 2) & 7, sl = op.code >> 8;
-                        if (kind == POLY_OP_ENTER) {
-                            const E2 c = gl::e2(op.c0, op.c1);
-#pragma unroll
-                            for (int d = 0; d < NF + 1; d++)
-                                if (dep == (u32)d) hv[d] = c;
-                        } else if (kind == POLY_OP_LEAF) {
-                            gl::E2P cp;
-                            cp.c0 = op.c0;
-                            cp.c1 = op.c1;
-                            cp.w = op.w;
-                            const E2 p = gl::mulp(gl::e2(cur0(sl), cur1(sl)), cp);
-#pragma unroll
-                            for (int d = 0; d < NF + 1; d++)
-                                if (dep == (u32)d) hv[d] = gl::add(hv[d], p);
-                        } else {
-                            const gl::E2P vp = gl::prep(gl::e2(cur0(sl), cur1(sl)));
-                            E2 child = hv[1];
-#pragma unroll
-                            for (int d = 2; d < NF + 1; d++)
-                                if (dep == (u32)d) child = hv[d];
-                            const E2 p = gl::mulp(child, vp);
-#pragma unroll
-                            for (int d = 1; d < NF + 1; d++)
-                                if (dep == (u32)d) hv[d - 1] = gl::add(hv[d - 1], p);
-                        }
-                    };
+                    // The nested program, walked with one function per depth (poly_walk): a node's running value is a
+                    // local of its depth's function, so no value is ever picked by a run-time index -- as an array
+                    // indexed by the operation's depth the values lived in scratch memory (a store per depth and two
+                    // dependent loads per operation, and a fifth of a gigabyte of write-backs per round), and picked
+                    // by select chains they cost forty more registers.  The operations are the same for the whole
+                    // wavefront: read from the kernel arguments they arrive in scalar registers, the branches are uniform.
+                    auto table = [&](u32 sl) { return gl::e2(cur0(sl), cur1(sl)); };
+                    u32 pc = 1;  // (operation 0 enters the root with its constant)
                     if (inl)
-                        for (u32 o = 0; o < n_ops; o++) step(a.o0[o]);
+                        gsum = poly_walk<0, NF - 1>(pc, n_ops, gl::e2(a.o0[0].c0, a.o0[0].c1), [&](u32 o) -> const PolyOp & { return a.o0[o]; }, table);
                     else
-                        for (u32 o = 0; o < n_ops; o++) step(lops[o]);
-                    gsum = hv[0];
+                        gsum = poly_walk<0, NF - 1>(pc, n_ops, gl::e2(lops[0].c0, lops[0].c1), [&](u32 o) -> const PolyOp & { return lops[o]; }, table);
                 } else {
                     gl::E2Acc G = gl::e2acc_zero();
                     for (u32 j = 0; j < n_terms; j++) {
@@ -1870,7 +1894,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
                     cur1(k) = gl::add(cur1(k), dl1(k));
                 }
             }
-        }
+        });
     }
     E2 acc[NP];
 #pragma unroll

@@ -781,6 +781,108 @@ def linking_verify(cfg, initial_claim, proof, evaluations, weight_eval, transcri
         total = e2_add(total, v)
     return bool((total == expected).all()), point, ch
 
+# ---------------------------------------------------------------------------
+# EinSum::prove_internal (zkml/src/layers/einsum/prove.rs:138-316) restated with the pieces above: axis
+# classification, partial evaluation of both sides, the batched sumcheck over the contracted axes, the
+# input claims, the aggregation sumcheck when several operations share the left-hand side, and the bias
+# claims (prove.rs:191-214, axis.rs:582-637).  ops: (lhs axes, rhs axes, output axes[, bias axes]) as strings.
+# ---------------------------------------------------------------------------
+AXIS_CONTRACTED, AXIS_OUTER, AXIS_STACKED = 0, 1, 2
+
+
+def _pad_shape(shape):
+    return [1 << max(0, (int(d) - 1).bit_length()) for d in shape]
+
+
+def _pad_tensor(t):
+    out = np.zeros(_pad_shape(t.shape), dtype=np.int64)
+    out[tuple(slice(0, d) for d in t.shape)] = t
+    return out
+
+
+def einsum_prove(ops, lhs, rhs, claims, label=b"m2vec", biases=None):
+    """prove_internal restated with the checker's pieces (einsum/prove.rs:138-316), one or more RHS; a bias gives a
+    claim of its own, its padded tensor's MLE at the slices of the output claim's point that its axes name
+    (prove.rs:191-214, axis.rs:582-637)."""
+    R = len(ops)
+    tr = OracleTranscript(label)
+    lp, lpad = _pad_tensor(lhs), _pad_shape(lhs.shape)
+
+    def classify(op, ch):
+        l, r, o = ch in op[0], ch in op[1], ch in op[2]
+        return AXIS_STACKED if (l and r and o) else AXIS_CONTRACTED if (l and r) else AXIS_OUTER
+
+    def split(shape, point):
+        out, start = [None] * len(shape), 0
+        for a in reversed(range(len(shape))):
+            ln = max(0, (shape[a] - 1).bit_length())
+            out[a] = point[start:start + ln]
+            start += ln
+        return out
+
+    def reconstruct(fixes, pts, sc_point, shape):
+        out, skip = [], 0
+        for a in reversed(range(len(fixes))):
+            if fixes[a] == AXIS_CONTRACTED:
+                ln = max(0, (shape[a] - 1).bit_length())
+                out.append(sc_point[skip:skip + ln])
+                skip += ln
+            else:
+                out.append(pts[a])
+        return np.concatenate(out) if out else np.zeros((0, 2), np.uint64)
+
+    lfix, rfix, lpts, rpts, ltabs, rtabs, coeffs, bias_claims = [], [], [], [], [], [], [], []
+    for r, op in enumerate(ops):
+        rpad = _pad_shape(rhs[r].shape)
+        out_shape = [lpad[op[0].index(c)] if c in op[0] else rpad[op[1].index(c)] for c in op[2]]
+        sl = split(out_shape, claims[r][0])
+        if biases is not None and biases[r] is not None:
+            bpt = [sl[op[2].index(c)] for c in reversed(op[3])]
+            bpt = np.concatenate(bpt) if bpt else np.zeros((0, 2), np.uint64)
+            bias_claims.append((r, bpt, mle_evaluate(embed_i64(_pad_tensor(biases[r]).reshape(-1)), bpt)))
+        lk = [classify(op, c) for c in op[0]]
+        rk = [classify(op, c) for c in op[1]]
+        lpt = [None if k == AXIS_CONTRACTED else sl[op[2].index(c)] for c, k in zip(op[0], lk)]
+        rpt = [None if k == AXIS_CONTRACTED else sl[op[2].index(c)] for c, k in zip(op[1], rk)]
+        lfix.append(lk); rfix.append(rk); lpts.append(lpt); rpts.append(rpt)
+        ltabs.append(partial_eval(lp, lpad, list(lhs.shape), lk, lpt))
+        rtabs.append(partial_eval(_pad_tensor(rhs[r]), rpad, list(rhs[r].shape), rk, rpt))
+        coeffs.append(stacking_coeffs(lpad, list(lhs.shape), lk, lpt))
+    S = ltabs[0].shape[0]
+    gamma = tr.append_and_sample(b"batching_challenge")
+    tabs = [t for v in ltabs for t in v] + [t for v in rtabs for t in v]
+    nv = int(tabs[0].shape[0]).bit_length() - 1
+    terms, gpow = [], np.array([1, 0], np.uint64)
+    for r in range(R):
+        for j in range(S):
+            terms.append((e2_mul(gpow, coeffs[r][j]), [r * S + j, R * S + r * S + j]))
+        gpow = e2_mul(gpow, gamma)
+    proof, point, finals = sc_prove(nv, tabs, terms, tr)
+    half = len(finals) // 2
+    out_claims = []
+    for r in range(R):
+        ev = np.zeros(2, np.uint64)
+        for j in range(S):
+            ev = e2_add(ev, e2_mul(coeffs[r][j], finals[half + r * S + j]))
+        out_claims.append((reconstruct(rfix[r], rpts[r], point, _pad_shape(rhs[r].shape)), ev))
+    agg = None
+    if R > 1:
+        eqs = [eq_evals(reconstruct(lfix[r], lpts[r], point, lpad)) for r in range(R)]
+        g2 = tr.append_and_sample(b"input_batching_challenge")
+        aterms, gp = [], np.array([1, 0], np.uint64)
+        for r in range(R):
+            aterms.append((gp, [0, 1 + r]))
+            gp = e2_mul(gp, g2)
+        full = embed_i64(lp.reshape(-1))
+        agg, apoint, afinals = sc_prove(int(full.shape[0]).bit_length() - 1, [full] + eqs, aterms, tr)
+        lhs_claim = (apoint, afinals[0])
+    else:
+        ev = np.zeros(2, np.uint64)
+        for j in range(S):
+            ev = e2_add(ev, e2_mul(coeffs[0][j], finals[j]))
+        lhs_claim = (reconstruct(lfix[0], lpts[0], point, lpad), ev)
+    return dict(proof=proof, evaluations=finals, aggregation_proof=agg, claims=[lhs_claim] + out_claims, bias_claims=bias_claims), tr
+
 
 def num_threads():
     return lib().orc_num_threads()

@@ -126,87 +126,7 @@ def test_partial_eval_matches_checker(ctx, orc, case):
 
 
 def _oracle_einsum(orc, ops, lhs, rhs, claims, label=b"m2vec", biases=None):
-    """prove_internal restated with the checker's pieces (einsum/prove.rs:138-316), one or more RHS; a bias gives a
-    claim of its own, its padded tensor's MLE at the slices of the output claim's point that its axes name
-    (prove.rs:191-214, axis.rs:582-637)."""
-    R = len(ops)
-    tr = orc.OracleTranscript(label)
-    lp, lpad = _padded(lhs), _pad(lhs.shape)
-
-    def classify(op, ch):
-        l, r, o = ch in op[0], ch in op[1], ch in op[2]
-        return S_ if (l and r and o) else C_ if (l and r) else O_
-
-    def split(shape, point):
-        out, start = [None] * len(shape), 0
-        for a in reversed(range(len(shape))):
-            ln = max(0, (shape[a] - 1).bit_length())
-            out[a] = point[start:start + ln]
-            start += ln
-        return out
-
-    def reconstruct(fixes, pts, sc_point, shape):
-        out, skip = [], 0
-        for a in reversed(range(len(fixes))):
-            if fixes[a] == C_:
-                ln = max(0, (shape[a] - 1).bit_length())
-                out.append(sc_point[skip:skip + ln])
-                skip += ln
-            else:
-                out.append(pts[a])
-        return np.concatenate(out) if out else np.zeros((0, 2), np.uint64)
-
-    lfix, rfix, lpts, rpts, ltabs, rtabs, coeffs, bias_claims = [], [], [], [], [], [], [], []
-    for r, op in enumerate(ops):
-        rpad = _pad(rhs[r].shape)
-        out_shape = [lpad[op[0].index(c)] if c in op[0] else rpad[op[1].index(c)] for c in op[2]]
-        sl = split(out_shape, claims[r][0])
-        if biases is not None and biases[r] is not None:
-            bpt = [sl[op[2].index(c)] for c in reversed(op[3])]
-            bpt = np.concatenate(bpt) if bpt else np.zeros((0, 2), np.uint64)
-            bias_claims.append((r, bpt, orc.mle_evaluate(orc.embed_i64(_padded(biases[r]).reshape(-1)), bpt)))
-        lk = [classify(op, c) for c in op[0]]
-        rk = [classify(op, c) for c in op[1]]
-        lpt = [None if k == C_ else sl[op[2].index(c)] for c, k in zip(op[0], lk)]
-        rpt = [None if k == C_ else sl[op[2].index(c)] for c, k in zip(op[1], rk)]
-        lfix.append(lk); rfix.append(rk); lpts.append(lpt); rpts.append(rpt)
-        ltabs.append(orc.partial_eval(lp, lpad, list(lhs.shape), lk, lpt))
-        rtabs.append(orc.partial_eval(_padded(rhs[r]), rpad, list(rhs[r].shape), rk, rpt))
-        coeffs.append(orc.stacking_coeffs(lpad, list(lhs.shape), lk, lpt))
-    S = ltabs[0].shape[0]
-    gamma = tr.append_and_sample(b"batching_challenge")
-    tabs = [t for v in ltabs for t in v] + [t for v in rtabs for t in v]
-    nv = int(tabs[0].shape[0]).bit_length() - 1
-    terms, gpow = [], np.array([1, 0], np.uint64)
-    for r in range(R):
-        for j in range(S):
-            terms.append((orc.e2_mul(gpow, coeffs[r][j]), [r * S + j, R * S + r * S + j]))
-        gpow = orc.e2_mul(gpow, gamma)
-    proof, point, finals = orc.sc_prove(nv, tabs, terms, tr)
-    half = len(finals) // 2
-    out_claims = []
-    for r in range(R):
-        ev = np.zeros(2, np.uint64)
-        for j in range(S):
-            ev = orc.e2_add(ev, orc.e2_mul(coeffs[r][j], finals[half + r * S + j]))
-        out_claims.append((reconstruct(rfix[r], rpts[r], point, _pad(rhs[r].shape)), ev))
-    agg = None
-    if R > 1:
-        eqs = [orc.eq_evals(reconstruct(lfix[r], lpts[r], point, lpad)) for r in range(R)]
-        g2 = tr.append_and_sample(b"input_batching_challenge")
-        aterms, gp = [], np.array([1, 0], np.uint64)
-        for r in range(R):
-            aterms.append((gp, [0, 1 + r]))
-            gp = orc.e2_mul(gp, g2)
-        full = orc.embed_i64(lp.reshape(-1))
-        agg, apoint, afinals = orc.sc_prove(int(full.shape[0]).bit_length() - 1, [full] + eqs, aterms, tr)
-        lhs_claim = (apoint, afinals[0])
-    else:
-        ev = np.zeros(2, np.uint64)
-        for j in range(S):
-            ev = orc.e2_add(ev, orc.e2_mul(coeffs[0][j], finals[j]))
-        lhs_claim = (reconstruct(lfix[0], lpts[0], point, lpad), ev)
-    return dict(proof=proof, evaluations=finals, aggregation_proof=agg, claims=[lhs_claim] + out_claims, bias_claims=bias_claims), tr
+    return orc.einsum_prove(ops, lhs, rhs, claims, label, biases)
 
 
 def _check_einsum(dp, ctx, orc, ops, lhs, rhs, seed, biases=None):
