@@ -1576,6 +1576,15 @@ struct dps_sc {
     u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
     E2 prev_chal;                     // the challenge of the call before this one
     bool pair12;                      // rounds 1 and 2 are one launch that writes nothing (pair12_kernel); round 3 folds twice on its way in
+    // Launches that cover two rounds each behind that one (quad_kernel): launch k takes rounds quad_j0 + 2 k and + 1, reading
+    // the state of two rounds before its first (the unfolded tables for the first launch, then what the launch before wrote)
+    struct QuadStep {
+        u32 j, blocks;
+        const u64 *s0[2], *s1[2];
+        u64 *d0[2], *d1[2];
+    };
+    std::vector<QuadStep> quads;      // in round order; round_kind 5 at a launch's first round, 6 at its second
+    bool fast_all_base;               // every streamed table of the product is a base-field table as registered
     E2 stash[dpk::SL_MAX_SUMS];       // a trip of two rounds: the second round's sums as a polynomial in the first round's challenge
     u64 last_trip_seq;
     u32 fin_len;                      // entries per table the last trip leaves to the host: the state of its first round
@@ -2075,10 +2084,47 @@ constexpr u32 SLICE_MAX_WORKGROUPS = 256;
 constexpr u32 HOST_TAIL_MAX_ROUNDS = 5;
 constexpr u64 HOST_TAIL_MULTS = 800;
 
+// eq * f * g over two base-field tables, large enough for the factored eq weights: rounds 1 and 2 can be one launch
+// that reads the tables once and writes nothing (pair12_kernel).  `first_resident`: the first round of the resident
+// launches (0: none).  Only what is known when the session is set up enters here.
+bool first_two_rounds_fit(const dps_sc *sc, u32 n_mles, u32 first_resident)
+{
+    const u32 n = sc->n_vars;
+    if (!sc->fast || sc->fast_eq < 0 || sc->fast_nf != 2 || n_mles != 3 || !sc->fast_all_base) return false;
+    if (n < dpk::EQ_LO_BITS + 3 || (first_resident && first_resident <= 3)) return false;
+    if (sc->eq_info->fact_levels < 3) return false;
+    if (((u64)product_blocks(1ull << (n - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return false;
+    // (round 2's p(1) comes from the claim: its scale must not vanish at 1)
+    const E2 rho2 = sc->eq_info->point[1];
+    return !((rho2.c0 == 0 && rho2.c1 == 0) || (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0));
+}
+
+// Workgroups of a launch that covers two rounds (quad_kernel) over `n_quads` quads, QUAD_STEP of them a workgroup's step:
+// a stride of exactly the low eq table's size (1024 workgroups: four wavefronts on every SIMD)
+u32 quad_blocks(u64 n_quads) { return (u32)std::min<u64>(n_quads / dpk::QUAD_STEP, ((u64)1 << dpk::EQ_LO_BITS) / dpk::QUAD_STEP); }
+
+// How many such launches follow the launch of the first two rounds: all of rounds 3 .. first_resident - 1 in pairs, when
+// they are an even number of rounds, every one takes p(1) from its claim (no zero among those coordinates of the eq
+// point) and every launch's quads still make a full stride of the factored weights.
+u32 quad_launches_fit(const dps_sc *sc, u32 n_mles, u32 first_resident)
+{
+    const u32 n = sc->n_vars;
+    if (!first_two_rounds_fit(sc, n_mles, first_resident) || first_resident < 5 || ((first_resident - 3) & 1)) return 0;
+    for (u32 j = 3; j < first_resident; j++) {
+        const E2 rho = sc->eq_info->point[j - 1];
+        if (rho.c0 == 0 && rho.c1 == 0) return 0;
+    }
+    for (u32 j = 3; j < first_resident; j += 2) {
+        // the launch's weights are those of round j + 1's pairs: low table of level j + 1, level j + 1 + 16
+        if (j + 1 > sc->eq_info->fact_levels || n < j + 1 + dpk::EQ_LO_BITS) return 0;
+    }
+    return (first_resident - 3) / 2;
+}
+
 // Which rounds of a session are resident, in which launches, and how they pair up into trips.  `n_tabs`: tables in LDS.
 // A trip covers two rounds when the second one's p(1) can come from the claim (its eq coordinate is not zero) and the
 // workgroups still hold a quad each.  The first resident round is the first whose pairs fit 256 workgroups.
-void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
+void plan_resident_rounds(dps_sc *sc, u32 n_tabs, u32 n_mles)
 {
     const u32 n = sc->n_vars;
     const bool has_eq = sc->fast_eq >= 0;
@@ -2122,7 +2168,9 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs)
     const u32 n_gpu = n - host_rounds;  // the last round of a trip
     sc->host_rounds = host_rounds;
     for (u32 r = n_gpu + 1; r <= n; r++) sc->round_kind[r] = 4;
-    u32 pend = j == 1 ? 0 : 1;                   // a launch that starts with round 1 has nothing to fold first
+    // a launch that starts with round 1 has nothing to fold first; one behind a launch that covered two rounds
+    // (quad_kernel) finds the state of two rounds ago
+    u32 pend = j == 1 ? 0 : (!sc->poly && quad_launches_fit(sc, n_mles, j) ? 2 : 1);
     u64 entries = (u64)1 << (n - j + 1 + pend);  // of the tables the stage to come starts from (before its pending folds)
     auto add_stage = [&](u32 W) {
         dps_sc::Stage st;
@@ -2166,7 +2214,9 @@ void drop_resident_plan(dps_sc *sc)
     sc->fin_len = 0;
     sc->fin_pend = 0;
     sc->host_rounds = 0;
-    std::fill(sc->round_kind.begin(), sc->round_kind.end(), 0);
+    // (the rounds of launches that cover two rounds, kinds 5 and 6, stay what they are)
+    for (uint8_t &k : sc->round_kind)
+        if (k <= 4) k = 0;
     std::fill(sc->round_wide.begin(), sc->round_wide.end(), 0);
 }
 
@@ -2219,7 +2269,7 @@ struct SessionSetup {
     void poly_groups_of_round(u32 j);
     void term_descs_of_round(u32 j);
     void describe_rounds();
-    void plan_first_two_rounds();
+    int32_t plan_first_two_rounds();
     void launch_limits();
     int32_t allocate_device_block();
     int32_t stage_descriptors();
@@ -2241,6 +2291,8 @@ bool SessionSetup::in_fast(u32 k) const
 void SessionSetup::detect_product()
 {
     sc->fast = false;
+    sc->fast_all_base = false;
+    sc->quads.clear();
     sc->broken = false;
     sc->tail_j0 = 0;
     sc->tail_running = false;
@@ -2276,6 +2328,8 @@ void SessionSetup::detect_product()
             for (u32 f = 0; f < t.n_factors; f++)
                 if ((int)t.factors[f] != sc->fast_eq && mles[t.factors[f]]->kind != DPS_BASE) sc->fast_order[w++] = t.factors[f];
             sc->fast_nf = w;
+            sc->fast_all_base = true;
+            for (u32 f = 0; f < w; f++) sc->fast_all_base = sc->fast_all_base && mles[sc->fast_order[f]]->kind == DPS_BASE;
             // compiled variants: 2 or 3 streamed tables without an eq factor, 1 or 2 with one
             sc->fast = sc->fast_eq >= 0 ? (w >= 1 && w <= 2) : (w >= 2 && w <= 3);
             if (!sc->fast) sc->fast_eq = -1;
@@ -2470,7 +2524,7 @@ int32_t SessionSetup::plan_and_ready_tables()
     sc->slice_terms.clear();
     if (sc->fast && n_vars >= 3 && n_mles == sc->terms[0].n_factors) {
         sc->slice_ids.assign(sc->fast_order, sc->fast_order + sc->fast_nf);
-        plan_resident_rounds(sc, sc->fast_nf);
+        plan_resident_rounds(sc, sc->fast_nf, n_mles);
     }
     // A sum of several terms over full-size tables (a fraction-sum layer, a claim merge, the stacked products of an
     // einsum): the same launches.  One group of tables from the first round that fits; more tables than a group holds
@@ -2492,7 +2546,7 @@ int32_t SessionSetup::plan_and_ready_tables()
                     if ((int)t.factors[f] != sc->fast_eq) tm.slot[tm.n_factors++] = (uint8_t)(std::find(ids.begin(), ids.end(), t.factors[f]) - ids.begin());
                 sc->slice_terms.push_back(tm);
             }
-            plan_resident_rounds(sc, (u32)ids.size());
+            plan_resident_rounds(sc, (u32)ids.size(), n_mles);
             if (sc->poly_tabs.size() > 1 && sc->tail_j0 != 1) {
                 // several groups and not every round resident: the groups' launches take the session
                 sc->stages.clear();
@@ -2724,6 +2778,7 @@ void SessionSetup::launch_limits()
     sc->max_blocks = n_vars >= 1 ? blocks_for_pairs(1ull << (n_vars - 1)) : 1;
     // (the launch of the first two rounds: 18 words a workgroup where the others have at most 16)
     if (sc->pair12) sc->max_blocks = std::max<u32>(sc->max_blocks, (PAIR12_BLOCKS * 2 * dpk::PAIR12_SUMS + 2 * dpk::MAX_PTS - 1) / (2 * dpk::MAX_PTS));
+    for (const dps_sc::QuadStep &q : sc->quads) sc->max_blocks = std::max<u32>(sc->max_blocks, q.blocks);
     sc->poly_split_cap = 0;
     sc->poly_finish_in_kernel = false;
     if (sc->poly) {
@@ -2836,16 +2891,13 @@ int32_t SessionSetup::stage_descriptors()
 
 // eq * f * g over two base-field tables, large enough for the factored eq weights: rounds 1 and 2 are one launch that
 // reads the tables once and writes nothing (pair12_kernel), and round 3 reads them again and folds twice on its way in.
-void SessionSetup::plan_first_two_rounds()
+int32_t SessionSetup::plan_first_two_rounds()
 {
     sc->pair12 = false;
-    if (!sc->fast || sc->fast_eq < 0 || sc->fast_nf != 2 || n_mles != 3 || sc->fast_nb[1] != 2) return;
-    if (n_vars < dpk::EQ_LO_BITS + 3 || (sc->tail_j0 && sc->tail_j0 <= 3)) return;
-    if (!sc->eq_info->fact_built || sc->eq_info->fact_levels < 3) return;
-    if (((u64)product_blocks(1ull << (n_vars - 3)) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) != 0) return;
-    // (round 2's p(1) comes from the claim: its scale must not vanish at 1)
-    const E2 rho2 = sc->eq_info->point[1];
-    if ((rho2.c0 == 0 && rho2.c1 == 0) || (sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0)) return;
+    sc->quads.clear();
+    if (!first_two_rounds_fit(sc, n_mles, sc->tail_j0)) return DPS_OK;
+    // (what the static test stands for; the resident launch's plan has counted on it)
+    if (sc->fast_nb[1] != 2 || !sc->eq_info->fact_built) return fail(ctx, DPS_ERR_STATE, "dps_sc_begin: the eq table's low tables are missing");
     sc->pair12 = true;
     dpk::ProdArgs &p3 = sc->fast_args[3];
     for (u32 f = 0; f < 2; f++) {
@@ -2854,6 +2906,28 @@ void SessionSetup::plan_first_two_rounds()
     }
     p3.two = 1;
     sc->fast_nb[3] = 2;
+    // Rounds 3 .. tail_j0 - 1 in launches of two rounds each (what the resident launch's plan counted on when it took
+    // two pending folds): the first reads the unfolded tables and writes the state of round 3 where round 3 would
+    // have; each later one reads what the one before wrote and writes into the table's other scratch buffer.
+    const u32 n_quad = quad_launches_fit(sc, n_mles, sc->tail_j0);
+    for (u32 q = 0; q < n_quad; q++) {
+        dps_sc::QuadStep st;
+        memset(&st, 0, sizeof st);
+        st.j = 3 + 2 * q;
+        st.blocks = quad_blocks(1ull << (n_vars - st.j - 1));
+        for (u32 f = 0; f < 2; f++) {
+            const SessMle &m = sc->m[sc->fast_order[f]];
+            const int into = q & 1 ? 0 : 1;  // round 3's state lies in the smaller buffer, as it always does
+            st.d0[f] = m.buf0[into];
+            st.d1[f] = m.buf1[into];
+            st.s0[f] = q == 0 ? sc->fast_args[1].s0[f] : sc->quads[q - 1].d0[f];
+            st.s1[f] = q == 0 ? nullptr : sc->quads[q - 1].d1[f];
+        }
+        sc->quads.push_back(st);
+        sc->round_kind[st.j] = 5;
+        sc->round_kind[st.j + 1] = 6;
+    }
+    return DPS_OK;
 }
 
 int32_t SessionSetup::run()
@@ -2863,7 +2937,7 @@ int32_t SessionSetup::run()
     CHK(plan_and_ready_tables());
     CHK(layout_scratch());
     describe_rounds();
-    plan_first_two_rounds();
+    CHK(plan_first_two_rounds());
     launch_limits();
     CHK(allocate_device_block());
     return stage_descriptors();
@@ -3218,6 +3292,11 @@ struct FusedRound {
     int32_t product_round();
     int32_t first_two_rounds_launch();
     int32_t second_round_from_stash();
+    const dps_sc::QuadStep *quad_at(u32 jj) const;
+    int32_t launch_quad(const dps_sc::QuadStep &q, bool ahead, u64 seq_q);
+    int32_t quad_first_round();
+    int32_t quad_second_round();
+    int32_t catch_up_after_quads();
 };
 
 
@@ -3430,6 +3509,10 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
                     const dpk::PolyTab &tb = sc->h_poly_groups[first - 1].tab[f];
                     sa.s0[f] = tb.s0;
                     sa.s1[f] = tb.s1;
+                } else if (!sc->quads.empty()) {
+                    // the state of two rounds ago, as the last launch of two rounds left it
+                    sa.s0[f] = sc->quads.back().d0[f];
+                    sa.s1[f] = sc->quads.back().d1[f];
                 } else {
                     sa.s0[f] = sc->fast_args[first].s0[f];
                     sa.s1[f] = sc->fast_args[first].s1[f];
@@ -3769,6 +3852,15 @@ int32_t FusedRound::product_launch_ahead()
                 CHK(launch_stages_at(next_seq));
                 made = true;
             }
+        } else if (const dps_sc::QuadStep *q = quad_at(j + 1)) {
+            // the next two rounds are one launch
+            if (admit_waiting_launch(ctx, q->blocks, false)) {
+                CHK(launch_quad(*q, true, next_seq));
+                sc->wait_any_skip1 = false;
+                sc->wait_skip1 = true;
+                sc->wait_slots = 0;
+                made = true;
+            }
         } else if (admit_waiting_launch(ctx, product_blocks(n_pairs >> 1), false)) {
             // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
             // p(1) comes from the claim unless the scale vanishes at 1
@@ -3914,6 +4006,146 @@ int32_t FusedRound::second_round_from_stash()
     return DPS_OK;
 }
 
+const dps_sc::QuadStep *FusedRound::quad_at(u32 jj) const
+{
+    for (const dps_sc::QuadStep &q : sc->quads)
+        if (q.j == jj) return &q;
+    return nullptr;
+}
+
+// The launch of rounds q.j and q.j + 1 (quad_kernel).  `ahead`: made before round q.j begins; it waits for the mail of
+// sequence number seq_q, which brings the challenges of the two rounds before.
+int32_t FusedRound::launch_quad(const dps_sc::QuadStep &q, bool ahead, u64 seq_q)
+{
+    dpk::ProdArgs qa;
+    memset(&qa, 0, sizeof qa);
+    for (u32 f = 0; f < 2; f++) {
+        qa.s0[f] = q.s0[f];
+        qa.s1[f] = q.s1[f];
+        qa.d0[f] = q.d0[f];
+        qa.d1[f] = q.d1[f];
+    }
+    const u64 n_quads = 1ull << (sc->n_vars - q.j - 1);
+    qa.n_pairs = n_quads;
+    qa.skip1 = 1;
+    if (!ahead) {
+        qa.r0 = a.r0, qa.r1 = a.r1;
+        qa.ra0 = sc->prev_chal.c0, qa.ra1 = sc->prev_chal.c1;
+    }
+    qa.wait_first = ahead ? 1 : 0;
+    qa.spin_limit = wait_units(ctx, AHEAD_SPIN_LIMIT);
+    qa.mail = ctx->d_pinned + (ctx->res_off - 64);
+    qa.relay = ahead && q.blocks > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
+    // the weights of round q.j + 1's pairs: low table of that level, and the level 16 rounds later
+    const u64 lo = eq_low_off(sc->n_vars, q.j + 1), hi = eq_level_off(sc->n_vars, q.j + 1 + dpk::EQ_LO_BITS);
+    qa.lq0 = sc->eq_c0 + lo;
+    qa.lq1 = sc->eq_c1 + lo;
+    qa.hq0 = sc->eq_c0 + hi;
+    qa.hq1 = sc->eq_c1 + hi;
+    dpk::FastFin fq = ff;
+    fq.n_blocks = q.blocks;
+    fq.seq = seq_q;
+    fq.slots = nullptr;
+    // sixteen source entries read and four written per table and quad
+    const double src_bytes = q.s1[0] ? 16.0 : 8.0;
+    ProfScope ps(ctx, DPS_K_FOLD_EVAL, (double)n_quads * 2 * (16 * src_bytes + 4 * 16.0));
+    if (q.s1[0])
+        dpk::quad_kernel<false><<<q.blocks, dpk::BLOCK, 0, ctx->stream>>>(qa, sc->d_partial, fq);
+    else
+        dpk::quad_kernel<true><<<q.blocks, dpk::BLOCK, 0, ctx->stream>>>(qa, sc->d_partial, fq);
+    HIPCHK(ctx, hipGetLastError());
+    return DPS_OK;
+}
+
+// The first round of a launch that covers two: the launch (or the mail for it), this round's message from the sums over
+// the pairs of either kind, and the next round's sums kept as polynomials in the challenge to come.
+int32_t FusedRound::quad_first_round()
+{
+    const dps_sc::QuadStep &q = *quad_at(j);
+    if (sc->tail_running) {
+        // (the launch's sums serve either way of getting p(1); its mail always says the one it was compiled for)
+        const u32 keep = a.skip1;
+        a.skip1 = 1;
+        post_mail();
+        a.skip1 = keep;
+        sc->wait_fresh = false;
+    } else {
+        CHK(launch_quad(q, false, fa.seq));
+    }
+    // the launch ends with the round; the round after it needs no launch
+    sc->tail_running = false;
+    waiting_launch_over(ctx);
+    prepare_message();
+    u64 w[2 * dpk::QUAD_SUMS];
+    if (const int32_t rc = wait_result(ctx, fa.seq, 0, 2 * dpk::QUAD_SUMS, w); rc != DPS_OK) {
+        sc->broken = true;
+        reset_device_words(ctx);
+        return rc;
+    }
+    E2 v[dpk::QUAD_SUMS];
+    for (u32 k = 0; k < (u32)dpk::QUAD_SUMS; k++) v[k] = gl::e2(w[2 * k], w[2 * k + 1]);
+    const E2 A0 = v[0], A1 = v[1], Al = v[2], B0 = v[3], B2 = v[4];
+    // the even pairs' product at t = 2 from its values at 0, 1 and its leading coefficient
+    const E2 A2 = gl::add(gl::sub(gl::add(A1, A1), A0), gl::add(Al, Al));
+    // pairs of either kind weighted by eq1(rho, .), rho the eq point's coordinate of the variable the next round binds
+    const E2 rho = sc->eq_info->point[j], nrho = gl::sub(gl::e2_one(), rho);
+    E2 qs[3];
+    qs[0] = gl::add(gl::mul(nrho, A0), gl::mul(rho, B0));
+    qs[1] = gl::e2_zero();
+    qs[2] = gl::add(gl::mul(nrho, A2), gl::mul(rho, B2));
+    // the next round at t = 0 and t = 2: value at c = 0, at c = 1, leading coefficient in c
+    sc->stash[0] = A0, sc->stash[1] = A1, sc->stash[2] = Al;
+    sc->stash[3] = v[5], sc->stash[4] = v[6], sc->stash[5] = v[7];
+    // (a.skip1 is off only when the scale has vanished, and then no q matters: the message is the constant terms')
+    form_message(qs);
+    if (challenge) sc->prev_chal = gl::e2(challenge[0], challenge[1]);
+    sc->round = j;
+    return DPS_OK;
+}
+
+// Its second round: nothing goes to the GPU but the launch after it, made ahead.
+int32_t FusedRound::quad_second_round()
+{
+    const E2 r = gl::e2(challenge[0], challenge[1]);
+    sc->tail_running = false;
+    waiting_launch_over(ctx);
+    CHK(product_launch_ahead());
+    const E2 rr = gl::mul(r, gl::sub(r, gl::e2_one()));
+    E2 qs[3];
+    for (u32 t = 0; t < 2; t++) {
+        const E2 v0 = sc->stash[3 * t], v1 = sc->stash[3 * t + 1], lead = sc->stash[3 * t + 2];
+        qs[t == 0 ? 0 : 2] = gl::add(gl::add(v0, gl::mul(r, gl::sub(v1, v0))), gl::mul(rr, lead));
+    }
+    qs[1] = gl::e2_zero();
+    prepare_message();
+    form_message(qs);
+    sc->prev_chal = r;
+    sc->round = j;
+    return DPS_OK;
+}
+
+// The resident launch found no place on the device and the launches of two rounds each have run: the state in memory
+// is two rounds old, where the ordinary launch of this round expects one fold pending.  The older of the two folds is
+// made here (into the table's other buffer, and from there to where this round's launch reads).
+int32_t FusedRound::catch_up_after_quads()
+{
+    const dps_sc::QuadStep &q = sc->quads.back();
+    const u64 n_out = 1ull << (sc->n_vars - q.j);  // entries of the state of round q.j + 1
+    for (u32 f = 0; f < 2; f++) {
+        const SessMle &m = sc->m[sc->fast_order[f]];
+        const int other = q.d0[f] == m.buf0[0] ? 1 : 0;
+        u64 *t0 = m.buf0[other], *t1 = m.buf1[other];
+        dpk::refold_kernel<<<grid_for(n_out), dpk::BLOCK, 0, ctx->stream>>>(q.d0[f], q.d1[f], t0, t1, n_out, sc->prev_chal.c0, sc->prev_chal.c1);
+        HIPCHK(ctx, hipGetLastError());
+        u64 *want0 = const_cast<u64 *>(sc->fast_args[j].s0[f]), *want1 = const_cast<u64 *>(sc->fast_args[j].s1[f]);
+        if (want0 != t0) {
+            HIPCHK(ctx, hipMemcpyAsync(want0, t0, n_out * 8, hipMemcpyDeviceToDevice, ctx->stream));
+            HIPCHK(ctx, hipMemcpyAsync(want1, t1, n_out * 8, hipMemcpyDeviceToDevice, ctx->stream));
+        }
+    }
+    return DPS_OK;
+}
+
 }  // namespace
 
 extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t *evals_out)
@@ -3961,10 +4193,15 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
         CHK(fr.begin());
         // the resident rounds begin here and their launch is not on the GPU yet: with no place for it on the device
         // these rounds are launches of their own
-        if (sc->tail_j0 && j == sc->tail_j0 && !sc->tail_running && !fr.admit_stages()) drop_resident_plan(sc);
+        if (sc->tail_j0 && j == sc->tail_j0 && !sc->tail_running && !fr.admit_stages()) {
+            if (!sc->quads.empty()) CHK(fr.catch_up_after_quads());
+            drop_resident_plan(sc);
+        }
         if (sc->tail_j0 && j >= sc->tail_j0) return fr.resident_round();
         if (sc->pair12 && j == 1) return fr.first_two_rounds_launch();
         if (sc->pair12 && j == 2) return fr.second_round_from_stash();
+        if (sc->round_kind[j] == 5) return fr.quad_first_round();
+        if (sc->round_kind[j] == 6) return fr.quad_second_round();
         return sc->poly ? fr.multi_term_round() : fr.product_round();
     } else {
         if (j >= 2) CHK(launch_folds(sc, j, false, challenge));

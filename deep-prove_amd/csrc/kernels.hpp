@@ -1032,6 +1032,231 @@ __global__ void __launch_bounds__(BLOCK) prod_kernel(ProdArgs a, u64 *__restrict
     }
 }
 
+// sums over the wavefront of canonical values (as block_sum does it: 22-bit pieces added as integers), valid in lane 63
+template <int NV>
+__device__ __forceinline__ void wave_sum_field(u64 (&v)[NV])
+{
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const u32 lo = (u32)v[i], hi = (u32)(v[i] >> 32);
+        const u64 c0 = wave_sum_u32(lo & 0x3FFFFFu);
+        const u64 c1 = wave_sum_u32((lo >> 22) | ((hi & 0xFFFu) << 10));
+        const u64 c2 = wave_sum_u32(hi >> 12);
+        const unsigned __int128 t = (unsigned __int128)c0 + ((unsigned __int128)c1 << 22) + ((unsigned __int128)c2 << 44);
+        v[i] = gl::reduce128((u64)t, (u64)(t >> 64));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Two rounds of eq(rho, x) f(x) g(x) from one pass over tables that are two folds behind: quad_kernel.
+//
+// The launch reads the state of two rounds ago (the unfolded base-field tables behind pair12_kernel, SRC_BASE, or the
+// extension tables the launch of this kind before it wrote), folds it twice on the way in with the two challenges
+// drawn since, writes the state S of its first round, round j, and hands over what rounds j and j + 1 need: S is not read
+// again until the launch after this one folds it twice in turn.
+//
+// Round j + 1's tables are S[2i] + c (S[2i+1] - S[2i]) with c the challenge of round j, not drawn yet: its sums are
+// polynomials of degree 2 in c, known by their values at c = 0, 1 and their leading coefficient.  Per quad (S0..S3 of f,
+// T0..T3 of g), everything weighted by R(m) = eq(rho_{j+2..}, m), m the quad's index:
+//   A0 = S0 T0, A1 = S1 T1, Al = (S1 - S0)(T1 - T0)       round j + 1 at t = 0 as a polynomial in c; and the even pairs of
+//                                                         round j: their q(0), q(1), leading coefficient
+//   B0 = S2 T2, B2 = (2 S3 - S2)(2 T3 - T2)               the odd pairs of round j at t = 0 and t = 2
+//   C0 = (2 S2 - S0)(2 T2 - T0), C1 = (2 S3 - S1)(2 T3 - T1), Cl = their differences' product
+//                                                         round j + 1 at t = 2 as a polynomial in c
+// Round j sums over the pairs of either kind, weighted by eq1(rho_{j+1}, .): the host has q_j(0) = (1 - rho) A0 + rho B0
+// and q_j(2) = (1 - rho)(2 A1 - A0 + 2 Al) + rho B2; both rounds take p(1) from their claims (the host only plans this
+// launch where the eq point allows that).  Eight products and eight sums a quad where two launches of prod_kernel make
+// eight as well -- and one pass over memory less: the state of round j + 1 is never written or read.
+// R(m) = hi[m >> 16] lo[m & 65535] as in the FACT variants of prod_kernel; the hi weight goes onto f's four entries
+// (S~ = hi S, four products a quad, the weight in scalar registers) so that the eight products need none.
+// ---------------------------------------------------------------------------
+// One fold of an extension table into another buffer: dst[i] = src[2i] + r (src[2i+1] - src[2i]).  The catch-up step of a
+// session whose launches of two rounds each are followed by ordinary launches after all (the state in memory is then a
+// fold behind what those expect).
+__global__ void __launch_bounds__(BLOCK) refold_kernel(const u64 *s0, const u64 *s1, u64 *d0, u64 *d1, u64 n_out, u64 r0, u64 r1)
+{
+    const gl::E2P rp = gl::prep(gl::e2(r0, r1));
+    for (u64 i = (u64)blockIdx.x * BLOCK + threadIdx.x; i < n_out; i += (u64)gridDim.x * BLOCK) {
+        const U64x2 x = ld2(s0 + 2 * i), y = ld2(s1 + 2 * i);
+        const E2 v = fold1p(gl::e2(x.x, y.x), gl::e2(x.y, y.y), rp);
+        d0[i] = v.c0;
+        d1[i] = v.c1;
+    }
+}
+
+constexpr int QUAD_SUMS = 8;  // handed over in this order: A0, A1, Al, B0, B2, C0, C1, Cl
+static_assert(QUAD_SUMS <= MAX_PTS, "the sums fit a workgroup's partials and the result area");
+
+// How the work of a workgroup's step -- QUAD_STEP quads, 4 QUAD_STEP entries of S per table -- is spread over its 256
+// lanes: first every lane makes two adjacent entries of S of one table (wavefronts 0 and 1 the first table's, 2 and 3 the
+// second's: 8 source entries, coalesced 16-byte loads, two 16-byte stores) and leaves them in LDS; after a barrier
+// wavefront w takes two of the eight products of every quad (lane = quad), reading the entries it needs from LDS, where
+// entry c of quad q of a table lies at [c][q] so that a wavefront's reads are conflict-free.  Short chains of dependent
+// arithmetic in many wavefronts (about 100 registers, four or five wavefronts per SIMD) instead of a lane per quad with
+// 250 registers and two: the launch is bound by the latency of those chains, not by their number.  The loads of the
+// next step are in flight while the products of this one are made; LDS holds two steps' entries, one barrier a step.
+constexpr int QUAD_STEP = 64;
+static_assert(BLOCK == 4 * QUAD_STEP && BLOCK == 4 * WAVE, "a lane per quad in each of four wavefronts");
+
+template <bool SRC_BASE>
+__global__ void __launch_bounds__(BLOCK) quad_kernel(ProdArgs a, u64 *__restrict__ partial, FastFin ff)
+{
+    constexpr int NS = QUAD_SUMS;
+    __shared__ u64 ent[2][2][4][QUAD_STEP][2];  // [step parity][table][entry of the quad][quad][limb]
+    __shared__ u64 own[2 * NS];
+    __shared__ int last_flag;
+    __shared__ u64 box[MAIL_WORDS];
+    __shared__ int ok_flag;
+    const u32 tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const u32 wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    // making the entries: this lane's table, and which two adjacent entries of the step's 4 QUAD_STEP
+    const u32 tab = wave >> 1, pi = tid & (2 * WAVE - 1);
+    const u64 *src0 = a.s0[tab], *src1 = a.s1[tab];
+    u64 *dst0 = a.d0[tab], *dst1 = a.d1[tab];
+    const u64 n_quads = a.n_pairs;
+    const u64 stride = (u64)gridDim.x * QUAD_STEP;
+    u64 m0 = (u64)blockIdx.x * QUAD_STEP;  // first quad of the step in hand
+    struct Raw {
+        U64x2 x[4] = {}, y[4] = {};
+    };
+    auto load_raw = [&](u64 first_quad, Raw &w) {
+        // entries 2 pi, 2 pi + 1 of the step are made of 8 source entries
+        const u64 e = 16 * first_quad + 8 * (u64)pi;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            w.x[c] = ld2(src0 + e + 2 * c);
+            if (!SRC_BASE) w.y[c] = ld2(src1 + e + 2 * c);
+        }
+    };
+    Raw raw;
+    if (m0 < n_quads) load_raw(m0, raw);
+    E2 ra = gl::e2(a.ra0, a.ra1), rb = gl::e2(a.r0, a.r1);
+    if (a.wait_first) {
+        // made ahead of its round: both challenges come by mail (the one of the round before this launch's first, and
+        // the one before that); the first step's loads are on their way meanwhile
+        if (!wait_first_mail(a.mail, a.relay, blockIdx.x == 0, a.spin_limit, ff.seq, 0, box, &ok_flag)) return;
+        if (box[MAIL_SKIP1] != 1) return;
+        rb = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
+        ra = gl::e2(uniform64(box[MAIL_RA]), uniform64(box[MAIL_RA + 1]));
+    }
+    // SRC_BASE: an entry of S is sum_ab e_a(ra) e_b(rb) x[a + 2 b] over four source entries, e_0(c) = 1 - c, e_1(c) = c
+    E2 k2[4];
+    if (SRC_BASE) {
+        const E2 na = gl::sub(gl::e2_one(), ra), nb = gl::sub(gl::e2_one(), rb);
+        k2[0] = gl::mul(na, nb), k2[1] = gl::mul(ra, nb), k2[2] = gl::mul(na, rb), k2[3] = gl::mul(ra, rb);
+    }
+    const gl::E2P rap = gl::prep(ra), rbp = gl::prep(rb);
+    // sums 2 wave and 2 wave + 1, unreduced (two a lane: their registers are affordable, a reduction per product is not)
+    gl::E2Acc acc0 = gl::e2acc_zero(), acc1 = gl::e2acc_zero();
+    u32 parity = 0;
+    for (; m0 < n_quads; m0 += stride, parity ^= 1) {
+        // ---- two entries of S of this lane's table ----
+        E2 v[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if (SRC_BASE) {
+                gl::E2Acc t = gl::e2acc_zero();
+                gl::acc_mul_base(t, k2[0], raw.x[2 * h].x);
+                gl::acc_mul_base(t, k2[1], raw.x[2 * h].y);
+                gl::acc_mul_base(t, k2[2], raw.x[2 * h + 1].x);
+                gl::acc_mul_base(t, k2[3], raw.x[2 * h + 1].y);
+                v[h] = gl::acc_reduce(t);
+            } else {
+                const E2 lo = fold1p(gl::e2(raw.x[2 * h].x, raw.y[2 * h].x), gl::e2(raw.x[2 * h].y, raw.y[2 * h].y), rap);
+                const E2 hi = fold1p(gl::e2(raw.x[2 * h + 1].x, raw.y[2 * h + 1].x), gl::e2(raw.x[2 * h + 1].y, raw.y[2 * h + 1].y), rap);
+                v[h] = fold1p(lo, hi, rbp);
+            }
+        }
+        {
+            const u64 e = 4 * m0 + 2 * (u64)pi;
+            st2_stream(dst0 + e, v[0].c0, v[1].c0);
+            st2_stream(dst1 + e, v[0].c1, v[1].c1);
+        }
+        // the next step's source entries, on their way while this step's products are made
+        if (m0 + stride < n_quads) load_raw(m0 + stride, raw);
+        if (tab == 0) {
+            // the high part of the weight goes onto the first table's entries: the same for the whole workgroup's step
+            const u32 hi = __builtin_amdgcn_readfirstlane((u32)(m0 >> EQ_LO_BITS));
+            const gl::E2P hp = gl::prep(gl::e2(a.hq0[hi], a.hq1[hi]));
+            v[0] = gl::mulp(v[0], hp);
+            v[1] = gl::mulp(v[1], hp);
+        }
+        {
+            const u32 q = pi >> 1, c = 2 * (pi & 1);
+            ent[parity][tab][c][q][0] = v[0].c0;
+            ent[parity][tab][c][q][1] = v[0].c1;
+            ent[parity][tab][c + 1][q][0] = v[1].c0;
+            ent[parity][tab][c + 1][q][1] = v[1].c1;
+        }
+        __syncthreads();
+        // ---- two of the eight products of quad `lane` ----
+        auto S = [&](int c) { return gl::e2(ent[parity][0][c][lane][0], ent[parity][0][c][lane][1]); };
+        auto T = [&](int c) { return gl::e2(ent[parity][1][c][lane][0], ent[parity][1][c][lane][1]); };
+        auto twice_less = [](E2 x, E2 y) { return gl::sub(gl::add(x, x), y); };  // 2 x - y
+        if (m0 + lane < n_quads) {
+            if (wave == 0) {
+                gl::acc_mul(acc0, S(0), gl::prep(T(0)));  // A0
+                gl::acc_mul(acc1, S(1), gl::prep(T(1)));  // A1
+            } else if (wave == 1) {
+                gl::acc_mul(acc0, gl::sub(S(1), S(0)), gl::prep(gl::sub(T(1), T(0))));  // Al
+                gl::acc_mul(acc1, S(2), gl::prep(T(2)));                                // B0
+            } else if (wave == 2) {
+                gl::acc_mul(acc0, twice_less(S(3), S(2)), gl::prep(twice_less(T(3), T(2))));  // B2
+                gl::acc_mul(acc1, twice_less(S(2), S(0)), gl::prep(twice_less(T(2), T(0))));  // C0
+            } else {
+                const E2 cs0 = twice_less(S(2), S(0)), cs1 = twice_less(S(3), S(1));
+                const E2 ct0 = twice_less(T(2), T(0)), ct1 = twice_less(T(3), T(1));
+                gl::acc_mul(acc0, cs1, gl::prep(ct1));                              // C1
+                gl::acc_mul(acc1, gl::sub(cs1, cs0), gl::prep(gl::sub(ct1, ct0)));  // Cl
+            }
+        }
+    }
+    // the low part of the weight, the same for all quads of this lane (the grid's stride is a multiple of 2^EQ_LO_BITS)
+    u64 w4[4];
+    {
+        const u64 lo = ((u64)blockIdx.x * QUAD_STEP + lane) & ((1u << EQ_LO_BITS) - 1);
+        const gl::E2P lp = gl::prep(gl::e2(a.lq0[lo], a.lq1[lo]));
+        const E2 s0 = gl::mulp(gl::acc_reduce(acc0), lp), s1 = gl::mulp(gl::acc_reduce(acc1), lp);
+        w4[0] = s0.c0, w4[1] = s0.c1, w4[2] = s1.c0, w4[3] = s1.c1;
+    }
+    // the wavefront's two sums: words 4 wave .. 4 wave + 3 of the workgroup's 16
+    wave_sum_field<4>(w4);
+    auto publish = [&](const u64 *w) {
+        if (ff.counter) *ff.counter = 0;
+        publish_words(ff.out_host, 0, w, 2 * NS, ff.seq);
+    };
+    if (gridDim.x == 1) {
+        if (lane == WAVE - 1)
+#pragma unroll
+            for (int k = 0; k < 4; k++) own[4 * wave + k] = w4[k];
+        __syncthreads();
+        if (tid == 0) publish(own);
+        return;
+    }
+    if (lane == WAVE - 1) {
+        u64 *o = partial + blockIdx.x;
+        const u64 total = gridDim.x;
+#pragma unroll
+        for (int k = 0; k < 4; k++) st_agent(o + (u64)(4 * wave + k) * total, w4[k]);
+    }
+    // (every wavefront's stores acknowledged before the workgroup's ticket is taken)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (take_ticket(ff.counter, gridDim.x, &last_flag) && wave == 0) {
+        // the last workgroup's first wavefront adds up the workgroups' words
+        u64 sum[2 * NS];
+#pragma unroll
+        for (int k = 0; k < 2 * NS; k++) sum[k] = 0;
+        for (u32 b = lane; b < gridDim.x; b += WAVE) {
+#pragma unroll
+            for (int k = 0; k < 2 * NS; k++) sum[k] = gl::add(sum[k], ld_agent(partial + (u64)k * gridDim.x + b));
+        }
+        wave_sum_field<2 * NS>(sum);
+        if (lane == WAVE - 1) publish(sum);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // The first two rounds of eq(rho, x) f(x) g(x), f and g in the base field, from one pass over the tables.
 //
@@ -1063,21 +1288,6 @@ constexpr int PAIR12_SUMS = 9;  // handed to the host in this order: pair 0's th
 constexpr int PAIR12_SEQ_SLOT = 62, PAIR12_CHK_SLOT = 63;
 constexpr u32 PAIR12_LEAD = 4, PAIR12_LEAD_SPINS = 1u << 16;  // steps the other rows may be ahead of row 2; polls before they go on anyway
 static_assert(2 * PAIR12_SUMS <= PAIR12_SEQ_SLOT, "the sums fit the result area");
-
-// sums over the wavefront of canonical values (as block_sum does it: 22-bit pieces added as integers), valid in lane 63
-template <int NV>
-__device__ __forceinline__ void wave_sum_field(u64 (&v)[NV])
-{
-#pragma unroll
-    for (int i = 0; i < NV; i++) {
-        const u32 lo = (u32)v[i], hi = (u32)(v[i] >> 32);
-        const u64 c0 = wave_sum_u32(lo & 0x3FFFFFu);
-        const u64 c1 = wave_sum_u32((lo >> 22) | ((hi & 0xFFFu) << 10));
-        const u64 c2 = wave_sum_u32(hi >> 12);
-        const unsigned __int128 t = (unsigned __int128)c0 + ((unsigned __int128)c1 << 22) + ((unsigned __int128)c2 << 44);
-        v[i] = gl::reduce128((u64)t, (u64)(t >> 64));
-    }
-}
 
 __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 *__restrict__ partial, FastFin ff)
 {

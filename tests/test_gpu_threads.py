@@ -63,6 +63,7 @@ def test_rounds_without_a_place_on_the_device(dp, orc, budget):
         ("product", 18, _product(orc, 18, 41000)),   # resident from round 1 in 256 workgroups
         ("product", 21, _product(orc, 21, 41100)),   # first two rounds in one launch, rounds 3.. ahead, resident from round 4
         ("product", 13, _product(orc, 13, 41200)),   # a narrow resident launch (fits the larger budgets)
+        ("product", 22, _product(orc, 22, 41700)),   # rounds 3 and 4 one launch; without the resident launch behind it, a catch-up fold
         ("layer", 17, _layer(orc, 17, 41300)),       # several terms: a launch of its own, then resident
         ("layer", 11, _layer(orc, 11, 41400)),
         ("stacked", 8, _stacked(orc, 8, 41500)),     # three groups of tables, every round resident when admitted
