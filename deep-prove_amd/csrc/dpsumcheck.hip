@@ -3288,7 +3288,7 @@ struct FusedRound {
     int32_t launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj);
     u32 slots_of(const Plan &p) const { return p.reside ? (n_groups > 1 ? n_groups : 0) : slots_for(p.blocks * n_groups); }
     int32_t multi_term_round();
-    int32_t product_launch_ahead();
+    int32_t product_launch_ahead(u32 ahead = 1);
     int32_t product_round();
     int32_t first_two_rounds_launch();
     int32_t second_round_from_stash();
@@ -3841,18 +3841,22 @@ int32_t FusedRound::multi_term_round()
 
 // The next round's launch, made behind this round's (for the same reasons as in multi_term_round): the resident launches, or a
 // product kernel, which then waits for its challenge by mail.
-int32_t FusedRound::product_launch_ahead()
+int32_t FusedRound::product_launch_ahead(u32 ahead)
 {
-    if (j < sc->n_vars && !ctx->profiling && !sc->no_ahead) {
-        const u64 next_seq = ctx->seq + 1;
+    // `ahead`: 1, the round after this one; or 2 when that one is answered on the host (the second round of a launch that
+    // covers two): the launch is then queued behind this round's and waits for its mail from the moment that one ends
+    const u32 jn = j + ahead;
+    if (jn <= sc->n_vars && !ctx->profiling && !sc->no_ahead) {
+        const u64 next_seq = ctx->seq + ahead;
+        const u64 pairs_n = 1ull << (sc->n_vars - jn);
         bool made = false;
-        if (sc->tail_j0 && j + 1 == sc->tail_j0) {
+        if (sc->tail_j0 && jn == sc->tail_j0) {
             // (when the device has room for the resident launches now; else the next round asks again)
             if (admit_stages()) {
                 CHK(launch_stages_at(next_seq));
                 made = true;
             }
-        } else if (const dps_sc::QuadStep *q = quad_at(j + 1)) {
+        } else if (const dps_sc::QuadStep *q = quad_at(jn)) {
             // the next two rounds are one launch
             if (admit_waiting_launch(ctx, q->blocks, false)) {
                 CHK(launch_quad(*q, true, next_seq));
@@ -3861,28 +3865,28 @@ int32_t FusedRound::product_launch_ahead()
                 sc->wait_slots = 0;
                 made = true;
             }
-        } else if (admit_waiting_launch(ctx, product_blocks(n_pairs >> 1), false)) {
+        } else if (sc->round_kind[jn] == 0 && admit_waiting_launch(ctx, product_blocks(pairs_n), false)) {
             // (more workgroups than should poll the host's memory: workgroup 0 polls and passes the mail on)
             // p(1) comes from the claim unless the scale vanishes at 1
             bool skip1_next = !(sc->fast_coeff.c0 == 0 && sc->fast_coeff.c1 == 0);
             if (has_eq) {
-                const E2 rho = sc->eq_info->point[j];
+                const E2 rho = sc->eq_info->point[jn - 1];
                 skip1_next = skip1_next && !(rho.c0 == 0 && rho.c1 == 0) && !(sc->eq_scalar.c0 == 0 && sc->eq_scalar.c1 == 0);
             }
-            dpk::ProdArgs an = sc->fast_args[j + 1];
-            if (has_eq) set_eq_weights(an, j + 1, product_blocks(n_pairs >> 1));
+            dpk::ProdArgs an = sc->fast_args[jn];
+            if (has_eq) set_eq_weights(an, jn, product_blocks(pairs_n));
             an.r0 = an.r1 = 0;
             an.skip1 = skip1_next ? 1 : 0;
             an.wait_first = 1;
             an.spin_limit = wait_units(ctx, AHEAD_SPIN_LIMIT);
             an.mail = ctx->d_pinned + (ctx->res_off - 64);
-            an.relay = product_blocks(n_pairs >> 1) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
+            an.relay = product_blocks(pairs_n) > POLY_AHEAD_MAX_WORKGROUPS ? mail_relay(ctx) : nullptr;
             dpk::FastFin fn = ff;
-            fn.n_blocks = product_blocks(n_pairs >> 1);
+            fn.n_blocks = product_blocks(pairs_n);
             fn.seq = next_seq;
             fn.slots = slots_for(fn.n_blocks) ? ctx->d_pinned + poly_raw_off(ctx) : nullptr;
             sc->wait_slots = slots_for(fn.n_blocks);
-            CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[j + 1], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
+            CHK(launch_prod_dispatch(ctx, nf, sc->fast_nb[jn], has_eq, true, an, fn.n_blocks, sc->d_partial, fn));
             HIPCHK(ctx, hipGetLastError());
             sc->wait_any_skip1 = false;
             sc->wait_skip1 = skip1_next;
@@ -3956,6 +3960,10 @@ int32_t FusedRound::first_two_rounds_launch()
         dpk::pair12_kernel<<<PAIR12_BLOCKS, dpk::PAIR12_BLOCK, 0, ctx->stream>>>(pa, sc->d_partial, ff);
         HIPCHK(ctx, hipGetLastError());
     }
+    // round 2 needs no launch: round 3's is queued behind this one now and waits for its mail from the moment this ends
+    sc->tail_running = false;
+    waiting_launch_over(ctx);
+    CHK(product_launch_ahead(2));
     a.skip1 = 0;  // (every point of round 1 is computed: round 2 needs them as well)
     skip1 = false;
     prepare_message();
@@ -3998,9 +4006,8 @@ int32_t FusedRound::second_round_from_stash()
     }
     prepare_message();
     form_message(q);
-    sc->tail_running = false;
-    waiting_launch_over(ctx);
-    CHK(product_launch_ahead());
+    // (round 3's launch is usually waiting already, made behind the launch of the first two rounds)
+    if (!sc->tail_running) CHK(product_launch_ahead());
     sc->prev_chal = r;
     sc->round = j;
     return DPS_OK;
@@ -4072,9 +4079,11 @@ int32_t FusedRound::quad_first_round()
     } else {
         CHK(launch_quad(q, false, fa.seq));
     }
-    // the launch ends with the round; the round after it needs no launch
+    // the launch ends with the round; the round after it needs no launch, so the launch after that is queued behind
+    // this one now
     sc->tail_running = false;
     waiting_launch_over(ctx);
+    CHK(product_launch_ahead(2));
     prepare_message();
     u64 w[2 * dpk::QUAD_SUMS];
     if (const int32_t rc = wait_result(ctx, fa.seq, 0, 2 * dpk::QUAD_SUMS, w); rc != DPS_OK) {
@@ -4107,9 +4116,8 @@ int32_t FusedRound::quad_first_round()
 int32_t FusedRound::quad_second_round()
 {
     const E2 r = gl::e2(challenge[0], challenge[1]);
-    sc->tail_running = false;
-    waiting_launch_over(ctx);
-    CHK(product_launch_ahead());
+    // (the launch of the rounds after this one is usually waiting already, made behind this pair's)
+    if (!sc->tail_running) CHK(product_launch_ahead());
     const E2 rr = gl::mul(r, gl::sub(r, gl::e2_one()));
     E2 qs[3];
     for (u32 t = 0; t < 2; t++) {

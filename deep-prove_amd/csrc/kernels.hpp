@@ -1139,13 +1139,15 @@ __global__ void __launch_bounds__(BLOCK) quad_kernel(ProdArgs a, u64 *__restrict
         rb = gl::e2(uniform64(box[MAIL_R]), uniform64(box[MAIL_R + 1]));
         ra = gl::e2(uniform64(box[MAIL_RA]), uniform64(box[MAIL_RA + 1]));
     }
-    // SRC_BASE: an entry of S is sum_ab e_a(ra) e_b(rb) x[a + 2 b] over four source entries, e_0(c) = 1 - c, e_1(c) = c
+    // an entry of S is sum_ab e_a(ra) e_b(rb) x[a + 2 b] over four source entries, e_0(c) = 1 - c, e_1(c) = c
     E2 k2[4];
-    if (SRC_BASE) {
+    gl::E2P k2p[4];
+    {
         const E2 na = gl::sub(gl::e2_one(), ra), nb = gl::sub(gl::e2_one(), rb);
         k2[0] = gl::mul(na, nb), k2[1] = gl::mul(ra, nb), k2[2] = gl::mul(na, rb), k2[3] = gl::mul(ra, rb);
+#pragma unroll
+        for (int k = 0; k < 4; k++) k2p[k] = gl::prep(k2[k]);
     }
-    const gl::E2P rap = gl::prep(ra), rbp = gl::prep(rb);
     // sums 2 wave and 2 wave + 1, unreduced (two a lane: their registers are affordable, a reduction per product is not)
     gl::E2Acc acc0 = gl::e2acc_zero(), acc1 = gl::e2acc_zero();
     u32 parity = 0;
@@ -1162,9 +1164,14 @@ __global__ void __launch_bounds__(BLOCK) quad_kernel(ProdArgs a, u64 *__restrict
                 gl::acc_mul_base(t, k2[3], raw.x[2 * h + 1].y);
                 v[h] = gl::acc_reduce(t);
             } else {
-                const E2 lo = fold1p(gl::e2(raw.x[2 * h].x, raw.y[2 * h].x), gl::e2(raw.x[2 * h].y, raw.y[2 * h].y), rap);
-                const E2 hi = fold1p(gl::e2(raw.x[2 * h + 1].x, raw.y[2 * h + 1].x), gl::e2(raw.x[2 * h + 1].y, raw.y[2 * h + 1].y), rap);
-                v[h] = fold1p(lo, hi, rbp);
+                // the same combination of extension entries: sixteen products gathered unreduced and two reductions,
+                // where three folds one after the other are twelve products and six reductions
+                gl::E2Acc t = gl::e2acc_zero();
+                gl::acc_mul(t, gl::e2(raw.x[2 * h].x, raw.y[2 * h].x), k2p[0]);
+                gl::acc_mul(t, gl::e2(raw.x[2 * h].y, raw.y[2 * h].y), k2p[1]);
+                gl::acc_mul(t, gl::e2(raw.x[2 * h + 1].x, raw.y[2 * h + 1].x), k2p[2]);
+                gl::acc_mul(t, gl::e2(raw.x[2 * h + 1].y, raw.y[2 * h + 1].y), k2p[3]);
+                v[h] = gl::acc_reduce(t);
             }
         }
         {
