@@ -6,8 +6,8 @@
 // full set (no argument) takes a few minutes, most of it thread hand-offs.  Covers every way the kernel hands over
 // its result (single workgroup, per-workgroup result areas, partials + ticket + gather), both evaluation modes, the
 // eq weights streamed and taken from two small tables, a launch that waits for its challenge by mail (directly
-// and through the relay), the variant that folds its sources twice on the way in, and the kernel of the first two
-// rounds (pair12_kernel).
+// and through the relay), the variant that folds its sources twice on the way in, the kernel of the first two
+// rounds (pair12_kernel) and the kernel that covers two rounds from sources two folds behind (quad_kernel).
 #include <chrono>
 #include <thread>
 #include <vector>
@@ -269,6 +269,117 @@ static void run_first_two_rounds(const char *name, u64 n_quads, u32 blocks)
     if (!ok) failures++;
 }
 
+// quad_kernel: two rounds from sources that are two folds behind.  The state S it must write is worked out by folding
+// the sources twice with plain loops; its eight sums are not compared with their formulas but used as the host uses
+// them -- round j's q(0) and q(2) over the pairs of either kind, round j + 1's q(0) and q(2) at a random challenge -- and
+// those are compared with direct sums over the pairs of S and over the pairs of S folded with that challenge.
+// `wait`: as in Case.  More than one step a workgroup needs the library's stride of 2^16 quads (1024 workgroups).
+template <bool SRC_BASE>
+static void run_two_rounds(const char *name, u64 n_quads, u32 blocks, int wait)
+{
+    const u64 n_src = 16 * n_quads, n_state = 4 * n_quads;
+    std::vector<u64> s0[2], s1[2], d0[2], d1[2];
+    for (int f = 0; f < 2; f++) {
+        s0[f].resize(n_src);
+        for (auto &x : s0[f]) x = felt();
+        if (!SRC_BASE) {
+            s1[f].resize(n_src);
+            for (auto &x : s1[f]) x = felt();
+        }
+        d0[f].assign(n_state, 0);
+        d1[f].assign(n_state, 0);
+    }
+    std::vector<u64> lq0(65536), lq1(65536), hq0((n_quads + 65535) >> 16), hq1(hq0.size());
+    for (auto *v : {&lq0, &lq1, &hq0, &hq1})
+        for (auto &x : *v) x = felt();
+    const E2 ra = gl::e2(felt(), felt()), rb = gl::e2(felt(), felt());
+    // the state, by two plain folds
+    std::vector<E2> S[2];
+    for (int f = 0; f < 2; f++) {
+        S[f].resize(n_state);
+        auto at = [&](u64 k) { return gl::e2(s0[f][k], SRC_BASE ? 0 : s1[f][k]); };
+        auto once = [&](u64 k) { return gl::add(at(k), gl::mul(ra, gl::sub(at(k + 1), at(k)))); };
+        for (u64 e = 0; e < n_state; e++) S[f][e] = gl::add(once(4 * e), gl::mul(rb, gl::sub(once(4 * e + 2), once(4 * e))));
+    }
+    auto weight = [&](u64 m) { return gl::mul(gl::e2(hq0[m >> 16], hq1[m >> 16]), gl::e2(lq0[m & 65535], lq1[m & 65535])); };
+
+    dpk::ProdArgs a;
+    memset(&a, 0, sizeof a);
+    for (int f = 0; f < 2; f++) {
+        a.s0[f] = s0[f].data();
+        a.s1[f] = SRC_BASE ? nullptr : s1[f].data();
+        a.d0[f] = d0[f].data();
+        a.d1[f] = d1[f].data();
+    }
+    a.lq0 = lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
+    a.n_pairs = n_quads;
+    a.skip1 = 1;
+    std::vector<u64> mail(64, 0), relay(64, 0), out_host(64, 0), partial(2 * dpk::QUAD_SUMS * (size_t)blocks + 64, 0);
+    u32 counter = 0;
+    const u64 seq = 55;
+    dpk::FastFin ff;
+    memset(&ff, 0, sizeof ff);
+    ff.partial = partial.data(), ff.n_blocks = blocks, ff.out_host = out_host.data(), ff.seq = seq, ff.counter = &counter;
+    std::thread host;
+    if (wait) {
+        a.wait_first = 1;
+        a.spin_limit = 1u << 30;
+        a.mail = mail.data();
+        a.relay = wait == 2 ? relay.data() : nullptr;
+        host = std::thread([&] {
+            std::this_thread::sleep_for(std::chrono::milliseconds(30));
+            mail[dpk::MAIL_R] = rb.c0, mail[dpk::MAIL_R + 1] = rb.c1;
+            mail[dpk::MAIL_RA] = ra.c0, mail[dpk::MAIL_RA + 1] = ra.c1;
+            mail[dpk::MAIL_SKIP1] = 1;
+            u64 chk = seq;
+            for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
+            mail[dpk::MAIL_CHK] = chk;
+            __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
+        });
+    } else {
+        a.r0 = rb.c0, a.r1 = rb.c1;
+        a.ra0 = ra.c0, a.ra1 = ra.c1;
+    }
+    launch(blocks, dpk::quad_kernel<SRC_BASE>, a, partial.data(), ff);
+    if (host.joinable()) host.join();
+
+    u64 chk = seq;
+    for (int k = 0; k < 2 * dpk::QUAD_SUMS; k++) chk ^= dpk::rotl64(out_host[k], k + 1);
+    bool ok = out_host[dpk::HOST_SEQ_SLOT] == seq && out_host[dpk::HOST_CHK_SLOT] == chk && counter == 0;
+    for (int f = 0; f < 2 && ok; f++)
+        for (u64 e = 0; e < n_state && ok; e++) ok = d0[f][e] == S[f][e].c0 && d1[f][e] == S[f][e].c1;
+    E2 v[dpk::QUAD_SUMS];
+    for (int k = 0; k < dpk::QUAD_SUMS; k++) v[k] = gl::e2(out_host[2 * k], out_host[2 * k + 1]);
+    const E2 A0 = v[0], A1 = v[1], Al = v[2], B0 = v[3], B2 = v[4], C0 = v[5], C1 = v[6], Cl = v[7];
+    // round j: pair p of S has the weight eq1(rho, p & 1) R(p >> 1), rho any element
+    const E2 rho = gl::e2(felt(), felt()), nrho = gl::sub(gl::e2_one(), rho);
+    auto line = [](E2 lo, E2 hi, u64 t) { return gl::add(lo, gl::mul_base(gl::sub(hi, lo), t)); };
+    E2 qj[3] = {gl::e2_zero(), gl::e2_zero(), gl::e2_zero()};
+    for (u64 p = 0; p < 2 * n_quads; p++) {
+        const E2 w = gl::mul(p & 1 ? rho : nrho, weight(p >> 1));
+        for (u64 t = 0; t <= 2; t += 2) qj[t] = gl::add(qj[t], gl::mul(w, gl::mul(line(S[0][2 * p], S[0][2 * p + 1], t), line(S[1][2 * p], S[1][2 * p + 1], t))));
+    }
+    const E2 A2 = gl::add(gl::sub(gl::add(A1, A1), A0), gl::add(Al, Al));
+    ok = ok && gl::eq(qj[0], gl::add(gl::mul(nrho, A0), gl::mul(rho, B0)));
+    ok = ok && gl::eq(qj[2], gl::add(gl::mul(nrho, A2), gl::mul(rho, B2)));
+    // round j + 1 at a challenge c: fold S with c and sum over its pairs
+    const E2 c = gl::e2(felt(), felt()), cc = gl::mul(c, gl::sub(c, gl::e2_one()));
+    E2 qn[3] = {gl::e2_zero(), gl::e2_zero(), gl::e2_zero()};
+    for (u64 m = 0; m < n_quads; m++) {
+        E2 lo[2], hi[2];
+        for (int f = 0; f < 2; f++) {
+            lo[f] = gl::add(S[f][4 * m], gl::mul(c, gl::sub(S[f][4 * m + 1], S[f][4 * m])));
+            hi[f] = gl::add(S[f][4 * m + 2], gl::mul(c, gl::sub(S[f][4 * m + 3], S[f][4 * m + 2])));
+        }
+        for (u64 t = 0; t <= 2; t += 2) qn[t] = gl::add(qn[t], gl::mul(weight(m), gl::mul(line(lo[0], hi[0], t), line(lo[1], hi[1], t))));
+    }
+    ok = ok && gl::eq(qn[0], gl::add(gl::add(A0, gl::mul(c, gl::sub(A1, A0))), gl::mul(cc, Al)));
+    ok = ok && gl::eq(qn[2], gl::add(gl::add(C0, gl::mul(c, gl::sub(C1, C0))), gl::mul(cc, Cl)));
+    printf("%-58s base=%d quads=%llu workgroups=%u : %s\n", name, (int)SRC_BASE, (unsigned long long)n_quads, blocks, ok ? "ok" : "MISMATCH");
+    for (int k = 0; k < dpk::QUAD_SUMS; k++) printf("    sum %d = %016llx %016llx\n", k, (unsigned long long)v[k].c0, (unsigned long long)v[k].c1);
+    if (!ok) failures++;
+}
+
 int main(int argc, char **argv)
 {
     // "quick": without the three-table variants and the two 256-workgroup cases (the suite's CPU run)
@@ -295,8 +406,15 @@ int main(int argc, char **argv)
     // the first two rounds from one pass: one workgroup, several (ticket and gather by the first wavefront)
     run_first_two_rounds("first two rounds, one workgroup", 50, 1);
     run_first_two_rounds("first two rounds, ragged quads, five workgroups", 300, 5);
+    // two rounds from sources two folds behind (a workgroup's step is 64 quads): one workgroup; several (ticket, gather by the
+    // first wavefront); the challenges by mail, directly and through the relay
+    run_two_rounds<true>("two rounds a launch, base-field sources, one workgroup", 64, 1, 0);
+    run_two_rounds<true>("two rounds a launch, base-field sources, by mail", 64 * 5, 5, 1);
+    run_two_rounds<false>("two rounds a launch, extension sources", 64 * 3, 3, 0);
+    run_two_rounds<false>("two rounds a launch, extension sources, mail relayed", 64 * 4, 4, 2);
     // eq weights as a product of two small tables (the grid's stride is a multiple of 2^16 pairs)
     if (!quick) {
+        run_two_rounds<true>("two rounds a launch, two steps in some workgroups", (1ull << 16) + 64 * 3, 1024, 0);
         run_first_two_rounds("first two rounds, two steps a lane", (1ull << 16) + 1000, 1024);
         run_case<2, 2, true, true, true, true, true>({"two folds on the way in, eq weights from two small tables", 1ull << 16, 256, false, 0});
         run_case<2, 2, false, true, false, true>({"first round, eq weights from two small tables", 3ull << 16, 256, false, 0});
