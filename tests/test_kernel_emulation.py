@@ -1,4 +1,5 @@
-"""The hot kernels' bodies on the CPU under the host sanitizers (tests/cpp/emu_prod_kernel.cpp, tests/cpp/emu_slice_kernel.cpp):
+"""The hot kernels' bodies on the CPU under the host sanitizers (tests/cpp/emu_prod_kernel.cpp, tests/cpp/emu_slice_kernel.cpp,
+tests/cpp/emu_poly_kernel.cpp):
 no GPU involved."""
 import os
 import shutil
@@ -37,3 +38,10 @@ def test_prod_kernel_body_under_host_sanitizers(tmp_path):
 def test_slice_kernel_body_under_host_sanitizers(tmp_path):
     # the resident rounds: trips of one and two rounds, one and several workgroups, hand-over between launches
     _build_and_run(tmp_path, "emu_slice_kernel.cpp", [])
+
+
+@needs_clang
+def test_poly_kernel_body_under_host_sanitizers(tmp_path):
+    # sums of several terms over shared tables: term by term and as a nested program, a pair's work over 1, 4 and 16 lanes,
+    # many groups, launches made ahead, a launch that stays for every remaining round
+    _build_and_run(tmp_path, "emu_poly_kernel.cpp", [])
