@@ -36,6 +36,11 @@ namespace {
 // 3 workgroups per CU on 256 CUs: measured best for the streaming kernels (each workgroup pays a fixed
 // reduction + ticket epilogue, so more, thinner workgroups lose more than they gain in latency hiding)
 constexpr u32 MAX_BLOCKS = 768;
+// areas of pinned memory for the outputs (and the small levels) of the fraction trees built last
+constexpr u32 LOGUP_OUT_AREAS = 8;
+constexpr size_t LOGUP_SHADOW_STRIDE = 2048;  // words per tree: dpk::LOGUP_SHADOW_WORDS rounded up
+// A sum of at most this many variables over tables the host holds copies of is worked out on the host, every round of it
+constexpr u32 HOST_ONLY_MAX_VARS = 7;
 constexpr u32 PAIR12_BLOCKS = 1024;  // workgroups of the launch of the first two rounds (64 quads each: a stride of 2^16 quads)
 
 // ---------------------------------------------------------------------------
@@ -73,6 +78,8 @@ struct dps_ctx {
     size_t pinned_words = 0;
     double wall_clock_scale = 1.0;  // rate of the device's real-time counter / 100 MHz
     u64 logup_builds = 0;           // fraction trees built so far (their outputs rotate through a few areas of the pinned buffer)
+    u64 *h_shadow = nullptr;        // host copies of those trees' small levels, one area per output area (written by the build's last launch)
+    u64 *d_shadow = nullptr;        // device address of the same memory
     hipEvent_t stage_event = nullptr;  // recorded after a launch that reads the staging region of the pinned buffer
     bool stage_pending = false;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
@@ -415,6 +422,11 @@ struct dps_mle {
     u64 len;
     std::shared_ptr<EqInfo> eq;  // set on eq tables (and on views covering the whole table)
     u32 pad_vars = 0;            // > 0: read by a sumcheck as zero-padded to this many variables
+    // A small level of a fraction tree: the host's copy of these entries (limb arrays), valid once the build's last launch has
+    // published under sh_seq in output area sh_slot, and until the context has built LOGUP_OUT_AREAS more trees (sh_build)
+    const u64 *sh0 = nullptr, *sh1 = nullptr;
+    u64 sh_seq = 0, sh_build = 0;
+    u32 sh_slot = 0;
     const u64 *p0() const { return st->c0 + offset; }
     const u64 *p1() const { return st->c1 ? st->c1 + offset : nullptr; }
 };
@@ -551,6 +563,13 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
     if (hipHostGetDevicePointer((void **)&ctx->d_pinned, ctx->h_pinned, 0) != hipSuccess) return bail(DPS_ERR_HIP);
     memset(ctx->h_pinned, 0, ctx->pinned_words * 8);
     ctx->res_off = ctx->pinned_words - 64;
+    // (without this memory the trees' small levels are simply not copied to the host)
+    if (hipHostMalloc((void **)&ctx->h_shadow, (size_t)LOGUP_OUT_AREAS * LOGUP_SHADOW_STRIDE * 8, hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess ||
+        hipHostGetDevicePointer((void **)&ctx->d_shadow, ctx->h_shadow, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        if (ctx->h_shadow) (void)hipHostFree(ctx->h_shadow);
+        ctx->h_shadow = ctx->d_shadow = nullptr;
+    }
     *out = ctx;
     return DPS_OK;
 }
@@ -569,6 +588,7 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
     for (auto &kv : ctx->live_blocks) (void)hipFree(kv.first);
     if (ctx->d_lagrange) (void)hipFree(ctx->d_lagrange);
     if (ctx->h_pinned) (void)hipHostFree(ctx->h_pinned);
+    if (ctx->h_shadow) (void)hipHostFree(ctx->h_shadow);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return DPS_OK;
@@ -836,6 +856,11 @@ extern "C" int32_t dps_mle_view(const dps_mle *src, uint64_t offset, uint32_t n_
     }
     *out = new (std::nothrow) dps_mle{ctx, src->st, src->kind, src->offset + offset, len, nullptr};
     if (*out && offset == 0 && len == src->len) (*out)->eq = src->eq;
+    if (*out && src->sh0) {
+        (*out)->sh0 = src->sh0 + offset;
+        (*out)->sh1 = src->sh1 + offset;
+        (*out)->sh_seq = src->sh_seq, (*out)->sh_build = src->sh_build, (*out)->sh_slot = src->sh_slot;
+    }
     return *out ? DPS_OK : fail(ctx, DPS_ERR_OOM, "host allocation failed");
 }
 
@@ -1039,7 +1064,9 @@ extern "C" int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point, uint32_t m,
     // Up to 17 variables everything comes out of one launch.  Of a larger table only the levels of at most 2^17 entries
     // and the low tables are built now, in that one launch (what a product session reads, 13 MB at 24 variables); the
     // large levels wait for whoever reads them.
-    const u64 small = ((2ull << m) - 1) & ~((1ull << eq_first_direct(m)) - 1);
+    // (nothing at all of a table so small that the sums over it may be the host's, which reads the point: then whoever
+    // reads entries builds them)
+    const u64 small = m <= HOST_ONLY_MAX_VARS ? 0 : ((2ull << m) - 1) & ~((1ull << eq_first_direct(m)) - 1);
     int32_t rc = eq_ensure(ctx, *t->eq, t->st->c0, t->st->c1, small, true);
     if (rc != DPS_OK) {
         delete t;
@@ -1375,6 +1402,7 @@ int32_t rows_as_tables(dps_ctx *ctx, dps_mle *cur, const u64 *in0, const u64 *in
             u64 one[2] = {0, 0};
             dps_mle *unit = nullptr;
             rc = dps_eq_build(ctx, one, 0, &unit);
+            if (rc == DPS_OK) rc = plain_ready(unit);
             dps_mle *flat = nullptr;
             if (rc == DPS_OK) rc = new_table(ctx, DPS_EXT2, stacked * contraction, &flat);
             if (rc == DPS_OK) {
@@ -1590,6 +1618,7 @@ struct dps_sc {
     u32 fin_len;                      // entries per table the last trip leaves to the host: the state of its first round
     u32 fin_pend;                     // ... and the folds that state is still owed (the rounds of that trip)
     u32 host_rounds;                  // the last rounds are worked out on the host from those entries (round_kind 4)
+    bool host_only = false;           // every round is: the tables were small levels of fraction trees, which the host has copies of
     std::vector<E2> host_state;       // the tables of the round in hand there, table by table
     u32 host_len;                     // entries per table in host_state (0: not taken over yet)
     bool host_fresh;                  // ... as the launch left them: the folds of its last trip are still owed
@@ -1666,6 +1695,10 @@ void reset_device_words(dps_ctx *ctx) { (void)hipMemsetAsync(ctx->d_counter, 0, 
 // by a 7-bit tag, so a word nobody took must not stay for the trip that carries the same tag 128 sequence numbers later
 size_t slice_area_off(const dps_ctx *ctx);
 size_t slice_fin_off(const dps_ctx *ctx);
+// the area of the pinned buffer for the outputs of a fraction tree (16 words each, behind the resident launches' result area)
+size_t logup_out_off(const dps_ctx *ctx, u32 slot) { return slice_area_off(ctx) + dpk::SL_AREA_WORDS + 64 + 16 * (size_t)slot; }
+int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out, int seq_slot = dpk::HOST_SEQ_SLOT,
+                       int chk_slot = dpk::HOST_CHK_SLOT);
 void clear_resident_results(dps_ctx *ctx)
 {
     for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
@@ -2558,6 +2591,47 @@ int32_t SessionSetup::plan_and_ready_tables()
             }
         }
     }
+    // A small sum over tables the host has copies of (the small levels of fraction trees): every round is the host's.
+    // A launch would take longer to start than the few hundred field products take here.
+    sc->host_only = false;
+    if (!sc->slice_ids.empty() && n_vars >= 1 && n_vars <= HOST_ONLY_MAX_VARS) {
+        bool ok = true;
+        for (u32 k : sc->slice_ids) {
+            const dps_mle *t = mles[k];
+            ok = ok && t->sh0 && ctx->logup_builds - t->sh_build < LOGUP_OUT_AREAS && t->len == (1ull << n_vars);
+        }
+        if (ok) {
+            // the copies are there once the builds' last launches have published (the same wait as for a tree's outputs)
+            u64 seen_seq[LOGUP_OUT_AREAS] = {};
+            for (u32 k : sc->slice_ids) {
+                const dps_mle *t = mles[k];
+                if (seen_seq[t->sh_slot] == t->sh_seq) continue;
+                u64 w[8];
+                if (wait_result_at(ctx, logup_out_off(ctx, t->sh_slot), t->sh_seq, 0, 8, w, 9, 8) != DPS_OK) ok = false;
+                seen_seq[t->sh_slot] = t->sh_seq;
+            }
+        }
+        if (ok) {
+            const u32 len = 1u << n_vars, n_tabs = (u32)sc->slice_ids.size();
+            sc->host_state.resize((size_t)len * n_tabs);
+            for (u32 f = 0; f < n_tabs; f++) {
+                const dps_mle *t = mles[sc->slice_ids[f]];
+                for (u32 i = 0; i < len; i++) sc->host_state[(size_t)f * len + i] = gl::e2(t->sh0[i], t->sh1[i]);
+            }
+            sc->host_len = len;
+            sc->host_fresh = false;
+            sc->host_only = true;
+            sc->stages.clear();
+            sc->tail_j0 = 0;
+            sc->fin_len = 0;
+            sc->fin_pend = 0;
+            sc->host_rounds = n_vars;
+            sc->round_kind.assign(n_vars + 2, 4);
+            std::fill(sc->round_wide.begin(), sc->round_wide.end(), 0);
+            sc->pairs_seq = 1;  // (dps_sc_finish: the last entries are with the host)
+            return DPS_OK;      // nothing of any table is read on the device
+        }
+    }
     // What this session reads of its tables: an eq table taken in closed form is read level by level -- level j in round j,
     // except in the large rounds of a product, which take the low table of level j and level j + 16 instead -- and
     // anything else as ordinary entries.  Whatever of that an eq table has not built yet is built now, on the stream.
@@ -3049,8 +3123,6 @@ namespace {
 // word; the words are accepted once the check word agrees with them, since the
 // kernel's stores may land in any order.  If the result does not arrive the
 // stream is queried to surface the error.
-int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n, u64 *out, int seq_slot = dpk::HOST_SEQ_SLOT,
-                       int chk_slot = dpk::HOST_CHK_SLOT);
 int32_t wait_result(dps_ctx *ctx, u64 seq, u32 slot0, u32 n, u64 *out) { return wait_result_at(ctx, ctx->res_off, seq, slot0, n, out); }
 
 // the same hand-off in another 64-word area of the pinned buffer
@@ -3575,8 +3647,9 @@ int32_t FusedRound::resident_round()
     int32_t rc = DPS_OK;
     if (kind == 4) {
         // A round of the few pairs that are left once the launch has gone: worked out here.
-        if (sc->host_len < 4) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the tables of the last rounds are not here");
-        host_tail_advance(sc, gl::e2(challenge[0], challenge[1]));
+        if (sc->host_len < (j == 1 ? 2u : 4u)) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the tables of the last rounds are not here");
+        // (round 1 of a sum that is the host's from the start has nothing to fold)
+        if (j >= 2) host_tail_advance(sc, gl::e2(challenge[0], challenge[1]));
         host_tail_sums(sc, j, nf, a.skip1 != 0, q);
         prepare_message();
         form_message(q);
@@ -4205,7 +4278,7 @@ extern "C" int32_t dps_sc_round(dps_sc *sc, const uint64_t *challenge, uint64_t 
             if (!sc->quads.empty()) CHK(fr.catch_up_after_quads());
             drop_resident_plan(sc);
         }
-        if (sc->tail_j0 && j >= sc->tail_j0) return fr.resident_round();
+        if ((sc->tail_j0 && j >= sc->tail_j0) || sc->host_only) return fr.resident_round();
         if (sc->pair12 && j == 1) return fr.first_two_rounds_launch();
         if (sc->pair12 && j == 2) return fr.second_round_from_stash();
         if (sc->round_kind[j] == 5) return fr.quad_first_round();
@@ -4243,7 +4316,7 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
         u64 w[8 * dpk::SL_MAX_TABS];
         // the fused multi-term kernel publishes its group's tables in slot order (one area per group when several
         // groups are resident), the single-product one its factors
-        if (!sc->stages.empty()) {
+        if (!sc->stages.empty() || sc->host_only) {
             // the host holds the tables: the last fold leaves one entry each
             if (sc->host_len < 2) return fail(ctx, DPS_ERR_STATE, "dps_sc_finish: the tables' last entries are not here");
             host_tail_advance(sc, r);
@@ -4255,7 +4328,7 @@ extern "C" int32_t dps_sc_finish(dps_sc *sc, const uint64_t *challenge, uint64_t
                 final_evals_out[2 * k + 1] = sc->host_state[f].c1;
             }
         }
-        const u32 n_areas = sc->poly && sc->stages.empty() ? (u32)sc->poly_tabs.size() : 0;
+        const u32 n_areas = sc->poly && sc->stages.empty() && !sc->host_only ? (u32)sc->poly_tabs.size() : 0;
         for (u32 g = 0; g < n_areas; g++) {
             const u32 n_fin = sc->poly ? (u32)sc->poly_tabs[g].size() : sc->fast_nf;
             const size_t base = sc->poly_raw ? poly_raw_off(ctx) + 64 * (size_t)g : ctx->res_off;
@@ -4433,11 +4506,10 @@ struct dps_logup {
     u64 out_seq = 0;             // the last launch of the build also hands the last layer's four entries to the host: under this
     u32 out_slot = 0;            // sequence number, in this one of the context's areas for them (0: it does not)
     u64 out_build = 0;           // the context's count of such builds after this one
+    u32 shadow_first = 0;        // layers shadow_first.. of at most LOGUP_SHADOW_MAX entries per array also lie in host memory (0: none do)
 };
 
-// areas of the pinned buffer for the outputs of the trees built last (16 words each, behind the resident launches' result area)
-constexpr u32 LOGUP_OUT_AREAS = 8;
-size_t logup_out_off(const dps_ctx *ctx, u32 slot) { return slice_area_off(ctx) + dpk::SL_AREA_WORDS + 64 + 16 * (size_t)slot; }
+static_assert(LOGUP_SHADOW_STRIDE >= dpk::LOGUP_SHADOW_WORDS, "a tree's small levels fit their area");
 
 extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uint32_t n_cols, const dps_mle *numer,
                                    const uint64_t c[2], const uint64_t beta[2], dps_logup **out)
@@ -4521,6 +4593,10 @@ extern "C" int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uin
             lg->out_seq = ++ctx->seq;
             ta.out_host = ctx->d_pinned + logup_out_off(ctx, lg->out_slot);
             ta.seq = lg->out_seq;
+            if (ctx->d_shadow) {
+                ta.shadow = ctx->d_shadow + (size_t)lg->out_slot * LOGUP_SHADOW_STRIDE;
+                lg->shadow_first = k;
+            }
             ProfScope ps(ctx, DPS_K_LOGUP, (double)ta.first_cur * 4 * 32.0);
             dpk::logup_tail_kernel<<<1, dpk::LOGUP_TAIL_BLOCK, 0, ctx->stream>>>(ta);
             HIPCHK(ctx, hipGetLastError());
@@ -4545,6 +4621,13 @@ extern "C" int32_t dps_logup_layer(const dps_logup *lg, uint32_t k, dps_mle **nu
     *num = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k], sz, nullptr};
     *den = new (std::nothrow) dps_mle{lg->ctx, lg->arena, DPS_EXT2, lg->layer_off[k] + sz, sz, nullptr};
     if (!*num || !*den) return fail(lg->ctx, DPS_ERR_OOM, "host allocation failed");
+    if (lg->shadow_first && k >= lg->shadow_first && sz <= dpk::LOGUP_SHADOW_MAX) {
+        // the build's last launch also left this layer in host memory
+        const u64 *sh = lg->ctx->h_shadow + (size_t)lg->out_slot * LOGUP_SHADOW_STRIDE + dpk::logup_shadow_off((u32)sz);
+        (*num)->sh0 = sh, (*num)->sh1 = sh + sz;
+        (*den)->sh0 = sh + 2 * sz, (*den)->sh1 = sh + 3 * sz;
+        for (dps_mle *t : {*num, *den}) t->sh_seq = lg->out_seq, t->sh_build = lg->out_build, t->sh_slot = lg->out_slot;
+    }
     return DPS_OK;
 }
 

@@ -2832,6 +2832,13 @@ logup_next_kernel(const u64 *__restrict__ pn0, const u64 *__restrict__ pn1, cons
 // n_hi, d_lo, d_hi, what the prover puts on the transcript first) also go to the host, as a round's result does.
 constexpr u32 LOGUP_TAIL_BITS = 10;
 constexpr int LOGUP_TAIL_BLOCK = 1024;
+// The levels of at most LOGUP_SHADOW_MAX entries per array also go to host memory (`shadow`): a sumcheck over such a
+// layer is a few hundred field products, which the host does in less time than a launch takes to start, and for that
+// it needs the entries.  A level of `cur` entries per array lies at word 4 (cur - 2) of the area (the levels below it
+// take 4 * 2, 4 * 4, ... words): numerators' limb arrays c0 and c1, then the denominators', `cur` words each.
+constexpr u32 LOGUP_SHADOW_MAX = 256;
+constexpr u32 LOGUP_SHADOW_WORDS = 4 * (2 * LOGUP_SHADOW_MAX - 2);
+__host__ __device__ __forceinline__ u32 logup_shadow_off(u32 cur) { return 4 * (cur - 2); }
 struct LogupTailArgs {
     u64 *c0, *c1;                       // the tree's arena
     u64 off[LOGUP_TAIL_BITS + 2];       // off[0]: the level read first; off[l + 1]: level l of this launch
@@ -2839,6 +2846,7 @@ struct LogupTailArgs {
     u64 first_cur;                      // entries per array of the first level written
     u64 *out_host;                      // 8 words + check word + sequence number (slots 8 and 9)
     u64 seq;
+    u64 *shadow;                        // host memory for the small levels (LOGUP_SHADOW_WORDS words), or nullptr
 };
 __global__ void __launch_bounds__(LOGUP_TAIL_BLOCK) logup_tail_kernel(LogupTailArgs a)
 {
@@ -2873,7 +2881,20 @@ __global__ void __launch_bounds__(LOGUP_TAIL_BLOCK) logup_tail_kernel(LogupTailA
             dst[cap_d + i] = num.c1;
             dst[2 * cap_d + i] = den.c0;
             dst[3 * cap_d + i] = den.c1;
+            if (a.shadow && cur <= LOGUP_SHADOW_MAX) {
+                u64 *sh = a.shadow + logup_shadow_off(cur);
+                st_sys(sh + i, num.c0);
+                st_sys(sh + cur + i, num.c1);
+                st_sys(sh + 2 * cur + i, den.c0);
+                st_sys(sh + 3 * cur + i, den.c1);
+            }
         }
+        __syncthreads();
+    }
+    // (the host reads the small levels once it has seen the sequence number below: every lane's stores to host memory
+    // are out before the workgroup meets, and the number is written after that)
+    if (a.shadow) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
         __syncthreads();
     }
     if (threadIdx.x == 0) {
