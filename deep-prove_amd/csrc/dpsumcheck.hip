@@ -3354,7 +3354,7 @@ struct FusedRound {
     int32_t take_sums(u32 n_slots);
     int32_t end_waiting_launch();
     bool admit_stages();
-    int32_t launch_stages_at(u64 seq0);
+    int32_t launch_stages_at(u64 seq0, u32 first_go = 0);
     int32_t resident_round();
     Plan plan_round(u32 jj, bool skip1_jj) const;
     int32_t launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahead, u64 seq_jj);
@@ -3557,7 +3557,7 @@ bool FusedRound::admit_stages()
 
 // The launches of the resident rounds, queued one behind the other: the trip that starts at the first resident
 // round has the sequence number seq0 (a round's call takes one number whether or not it makes a trip).
-int32_t FusedRound::launch_stages_at(u64 seq0)
+int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
 {
         const u32 first = sc->tail_j0;
         for (size_t si = 0; si < sc->stages.size(); si++) {
@@ -3615,6 +3615,7 @@ int32_t FusedRound::launch_stages_at(u64 seq0)
             sa.relay = mail_relay(ctx);
             sa.spin_limit = wait_units(ctx, 4000000);  // ten seconds, then the kernel gives up
             sa.finish = last_si + 1 == sc->stages.size() ? 1 : 0;
+            sa.first_go = si == 0 && st.pend0 == 0 && st.j0 == 1 ? first_go : 0;
             sa.out_host = ctx->d_pinned + slice_area_off(ctx);
             sa.fin_out = ctx->d_pinned + slice_fin_off(ctx);
             sa.seq0 = seq0 + (st.j0 - first);
@@ -3677,7 +3678,8 @@ int32_t FusedRound::resident_round()
     } else {
         if (!sc->tail_running) {
             if (j != sc->tail_j0) return fail(ctx, DPS_ERR_STATE, "dps_sc_round: the resident launch of the last rounds is gone");
-            CHK(launch_stages_at(fa.seq));
+            // (a launch for round 1 needs nothing of its first mail but whether t = 1 is evaluated: it is told at once)
+            CHK(launch_stages_at(fa.seq, sc->tail_j0 == 1 && j == 1 ? (a.skip1 ? 2u : 1u) : 0u));
         }
         post_mail();
         sc->wait_fresh = false;

@@ -1506,6 +1506,9 @@ struct SliceArgs {
     u32 spin_limit;
     u32 finish;        // the launch's last trip is the last of the session's launches: the state of that trip's first round goes to
                        // the host (fin_out) with it; else what is left goes to h0 / h1
+    u32 first_go;      // a launch that starts with round 1 (nothing pending), made when that round is due: its first trip starts
+                       // without a look into the mailbox; 1: t = 1 is evaluated, 2: it comes from the claim.  0: every trip waits for its mail
+    u32 pad_go;
     u64 *out_host;     // result area of SL_AREA_WORDS words
     u64 *fin_out;      // ... and the area of SL_FIN_AREA_WORDS words for the entries left with the last trip (finish)
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
@@ -1615,11 +1618,21 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             in_big = true;
         }
         trip_seq = a.seq0 + (j - a.j0);
-        if (!wait_first_mail(a.mail, Wc > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
-        if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
-        const bool skip1 = box[MAIL_SKIP1] != 0;
-        const E2 rb_ = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
-        const gl::E2P rb = gl::prep(rb_), ra = gl::prep(gl::e2(box[MAIL_RA], box[MAIL_RA + 1]));
+        bool skip1;
+        E2 rb_ = gl::e2_zero(), ra_ = gl::e2_zero();
+        if (k == 0 && a.first_go) {
+            // a launch made for round 1, when it is that round's turn: nothing is pending, whether t = 1 is evaluated came
+            // with the launch, and the trip over the host link that a look into the mailbox costs is saved
+            skip1 = a.first_go == 2;
+            __syncthreads();
+        } else {
+            if (!wait_first_mail(a.mail, Wc > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
+            if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
+            skip1 = box[MAIL_SKIP1] != 0;
+            rb_ = gl::e2(box[MAIL_R], box[MAIL_R + 1]);
+            ra_ = gl::e2(box[MAIL_RA], box[MAIL_RA + 1]);
+        }
+        const gl::E2P rb = gl::prep(rb_), ra = gl::prep(ra_);
         // ---- the pending folds ----
         if (k == 0 || regroup) {
             // from device memory: entry i of the state is the source's entry i (nothing pending), or is made of its entries

@@ -100,6 +100,7 @@ struct Term {
 // `separate`: the stage of several workgroups and the single workgroup after it are two launches (as when the rounds left
 // are more than one launch can run); otherwise they are one.  `host_rounds`: the last rounds are not the launch's (the
 // library works them out on the host): its last trip ends before them and hands over that many more entries.
+static bool g_first_go = false;  // launches that start with round 1 are told at once whether t = 1 is evaluated, and get no first mail
 template <int NF, bool EQ, bool TERMS = false>
 static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_in, std::vector<u32> single_rounds = {}, std::vector<Term> terms = {},
                      u32 base_tabs = 0, bool separate = false, u32 host_rounds = 0)
@@ -236,6 +237,9 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         a.relay = relay.data();
         a.spin_limit = 1u << 24;
         a.finish = last_si + 1 == stages.size();
+        // a launch for round 1 told at once whether t = 1 is evaluated: its first trip gets no mail here at all
+        const bool go = g_first_go && si == 0 && st.pend0 == 0 && st.j0 == 1;
+        a.first_go = go ? (is_single(st.j0) ? 1 : 2) : 0;
         a.out_host = area.data();
         a.fin_out = fin.data();
         a.seq0 = seq_first + (st.j0 - j0);
@@ -268,7 +272,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
                 u64 chk = seq;
                 for (u32 i = dpk::MAIL_R; i < (u32)dpk::MAIL_WORDS; i++) chk ^= dpk::mail_mix(mail[i], i);
                 mail[dpk::MAIL_CHK] = chk;
-                __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
+                if (!(go && sj == si && k == 0)) __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
                 // the result: every counter of the trip's sums, tagged with the trip
                 const int ns = dbl ? NS : NP;
                 u64 cnt[4 * dpk::SL_MAX_SUMS];
@@ -469,6 +473,13 @@ int main()
     run_case<2, true>("four workgroups, then one, the last three rounds left out", 12, 3, 4, 0, {}, {}, 0, false, 3);
     run_case<2, false, true>("16 tables, 8 products, the last two rounds left out", 8, 1, 1, 16, {}, stacked, 0, false, 2);
     run_case<2, true, true>("fraction-sum layer over 4 workgroups, the last three rounds left out", 11, 2, 4, 4, {}, {la, lb, lc}, 0, false, 3);
+    // launches for round 1 whose first trip starts without mail
+    g_first_go = true;
+    run_case<2, true>("from round 1, first trip without mail", 8, 1, 1, 0);
+    run_case<2, true, true>("fraction-sum layer from round 1 over 4 workgroups, first trip without mail", 10, 1, 4, 4, {}, {la, lb, lc}, 0, false, 3);
+    run_case<2, false>("two tables from round 1, t = 1 evaluated in round 1, first trip without mail", 8, 1, 1, 0, {1, 4});
+    run_case<2, false, true>("16 tables, 8 products, from round 1, first trip without mail", 8, 1, 1, 16, {}, stacked, 0, false, 2);
+    g_first_go = false;
     printf("%s\n", failures ? "FAILED" : "all cases ok");
     return failures ? 1 : 0;
 }
