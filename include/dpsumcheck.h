@@ -122,6 +122,8 @@ int32_t dps_mle_free(dps_mle *mle);
 
 /* ---- poly::eq::evals (zkml/src/layers/hadamard.rs:103, zkml/src/layers/einsum/axis.rs:1032,
  *      zkml/src/lookup/logup_gkr/prover.rs:247-249): out[i] = prod_j (bit_j(i) ? r_j : 1 - r_j) ---- */
+/* (Entries are materialised when something reads them: a table of more than 17 variables has only its small suffix
+ * tables built here, one of at most 7 variables nothing -- a sum the host works out reads the point.) */
 int32_t dps_eq_build(dps_ctx *ctx, const uint64_t *point /* 2*m */, uint32_t m, dps_mle **out);
 /* `count` eq tables, table i at points[i] of m[i] coordinates (zkml/src/poly_commit/prover.rs:176-181 and
  * zkml/src/iop/same_poly.rs:88-91 build one per claim): every table of at most 2^16 entries comes out of one launch. */
@@ -209,7 +211,10 @@ int32_t dps_logup_build(dps_ctx *ctx, const dps_mle *const *cols, uint32_t n_col
                         const uint64_t c[2], const uint64_t beta[2], dps_logup **out);
 /* number of layers including the input layer 0 */
 int32_t dps_logup_num_layers(const dps_logup *lg, uint32_t *n_layers);
-/* numerator and denominator tables of layer k >= 1 (views; free them with dps_mle_free) */
+/* numerator and denominator tables of layer k >= 1 (views; free them with dps_mle_free).  The layers of at most 256
+ * entries per array also lie in host memory (the build's last launch leaves them there; the copies of the last 8
+ * trees of a context are kept): a sumcheck of at most 7 variables over such tables, or windows into them, and an
+ * eq factor runs on the host from its first round, without a launch -- same messages, bit for bit. */
 int32_t dps_logup_layer(const dps_logup *lg, uint32_t k, dps_mle **num, dps_mle **den);
 /* LogUpCircuit::outputs (circuit.rs:558-560): n_lo, n_hi, d_lo, d_hi of the last layer */
 int32_t dps_logup_outputs(const dps_logup *lg, uint64_t out[8]);
