@@ -525,13 +525,19 @@ class Context:
         cl = None if claim is None else np.ascontiguousarray(_e2(claim))
         clp = None if cl is None else cl.ctypes.data
 
+        # (the three results share one buffer: taking an array's address costs more than making the array)
+        n_proof, n_point = n_vars * (degree + 1) * 2, n_vars * 2
+        n_words = n_proof + n_point + max(1, n_mles) * 2
+        call, ctx_c = host.dph_sumcheck_prove_claimed, self._c
+
         def prove(transcript):
-            proof = np.zeros((n_vars, degree + 1, 2), dtype=np.uint64)
-            point = np.zeros((n_vars, 2), dtype=np.uint64)
-            finals = np.zeros((max(1, n_mles), 2), dtype=np.uint64)
-            self._chk_host(host.dph_sumcheck_prove_claimed(self._c, n_vars, hs, n_mles, tarr, nt, clp, transcript._t, proof.ctypes.data,
-                                                           point.ctypes.data, finals.ctypes.data, dref), "dph_sumcheck_prove")
-            return proof, point, finals[:n_mles]
+            buf = np.zeros(n_words, dtype=np.uint64)
+            base = buf.ctypes.data
+            rc = call(ctx_c, n_vars, hs, n_mles, tarr, nt, clp, transcript._t, base, base + 8 * n_proof, base + 8 * (n_proof + n_point), dref)
+            if rc != 0:
+                self._chk_host(rc, "dph_sumcheck_prove")
+            return (buf[:n_proof].reshape(n_vars, degree + 1, 2), buf[n_proof:n_proof + n_point].reshape(n_vars, 2),
+                    buf[n_proof + n_point:n_proof + n_point + 2 * n_mles].reshape(n_mles, 2))
 
         prove.keep = (keep, cl)
         return prove

@@ -2154,6 +2154,17 @@ u32 quad_launches_fit(const dps_sc *sc, u32 n_mles, u32 first_resident)
     return (first_resident - 3) / 2;
 }
 
+// A round of a sum of several terms with a common eq factor whose launch (poly_kernel, a thread per pair) takes the eq
+// weights from the low table of its level and from the level 16 rounds later instead of streaming its own level: the
+// rounds of more than 2^16 pairs, whose grid stride is a multiple of 2^16, of a table that has its low tables.
+bool poly_round_weights_factored(const dps_sc *sc, u32 jj)
+{
+    if (!sc->poly || sc->fast_eq < 0 || !sc->eq_info || !sc->eq_info->fact_built || jj > sc->eq_info->fact_levels) return false;
+    const u64 n_pairs = 1ull << (sc->n_vars - jj);
+    if (n_pairs <= POLY_SPLIT_MAX_PAIRS) return false;  // (those rounds spread a pair over lanes: poly_split_kernel)
+    return ((u64)blocks_for_pairs(n_pairs) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0;
+}
+
 // Passes the lanes of a workgroup make over `n_quads` quads for the second round of a trip: a lane keeps one sample at one
 // point for some of the terms (slice_kernel's q_split), the lanes of a pass cover BLOCK / (q_split NF (NF + 1)) quads
 u32 slice_second_round_passes(const dps_sc *sc, u32 n_quads)
@@ -2658,6 +2669,9 @@ int32_t SessionSetup::plan_and_ready_tables()
             if (sc->fast) {
                 first_level = sc->eq_info->fact_levels + 1;
                 if (sc->tail_j0) first_level = std::min(first_level, sc->tail_j0);
+            } else if (sc->poly) {
+                // the large rounds of a sum of several terms read level j + 16 and the low table of level j
+                while (first_level <= n_vars && poly_round_weights_factored(sc, first_level)) first_level++;
             }
             const u64 need = ((2ull << n_vars) - 1) & ~((1ull << first_level) - 1);
             CHK(eq_ensure(ctx, *sc->eq_info, const_cast<u64 *>(sc->eq_c0), const_cast<u64 *>(sc->eq_c1), need, sc->fast));
@@ -3577,6 +3591,10 @@ bool FusedRound::admit_stages()
 int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
 {
         const u32 first = sc->tail_j0;
+        // No resident launch of this context is running now: whatever an abandoned one left in the result area goes -- before
+        // the launch is made, which may start its first trip at once (first_go) and publish while this thread is still here.
+        memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
+        for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
         for (size_t si = 0; si < sc->stages.size(); si++) {
             const dps_sc::Stage &st = sc->stages[si];
             // a stage of several workgroups and the single-workgroup stage that runs to the last round are one launch:
@@ -3645,9 +3663,6 @@ int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
             if (st.W > 1 && !merged) reset_device_words(ctx);
             si = last_si;
         }
-        memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
-        // no resident launch of this context is running now: whatever an abandoned one left in the result area goes
-        for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
         sc->tail_seq0 = seq0;
         sc->tail_running = true;
         sc->wait_any_skip1 = true;
@@ -3783,10 +3798,19 @@ int32_t FusedRound::launch_round(u32 jj, const Plan &p, bool skip1_jj, bool ahea
             CHK(ensure_descs(sc));
         }
         pa.q0 = pa.q1 = nullptr;
+        pa.lq0 = pa.lq1 = pa.hq0 = pa.hq1 = nullptr;
         if (has_eq) {
             const u64 off = eq_level_off(sc->n_vars, jj);
             pa.q0 = sc->eq_c0 + off;
             pa.q1 = sc->eq_c1 + off;
+            if (!p.split && poly_round_weights_factored(sc, jj)) {
+                // not streamed: the low table of level jj and level jj + 16 (as the large rounds of a product take them)
+                const u64 lo = eq_low_off(sc->n_vars, jj), hi = eq_level_off(sc->n_vars, jj + dpk::EQ_LO_BITS);
+                pa.lq0 = sc->eq_c0 + lo;
+                pa.lq1 = sc->eq_c1 + lo;
+                pa.hq0 = sc->eq_c0 + hi;
+                pa.hq1 = sc->eq_c1 + hi;
+            }
         }
         pa.n_pairs = p.n_pairs;
         pa.r0 = ahead ? 0 : a.r0;
@@ -4424,7 +4448,15 @@ extern "C" int32_t dps_sc_prove(dps_sc *sc, dps_round_fn fn, void *user, uint64_
     uint64_t chal[2] = {0, 0};
     for (u32 j = 1; j <= sc->n_vars; j++) {
         uint64_t *msg = proof_out + (size_t)(j - 1) * npts * 2;
-        CHK(dps_sc_round(sc, j == 1 ? nullptr : chal, msg));
+        if (const int32_t rc = dps_sc_round(sc, j == 1 ? nullptr : chal, msg); rc != DPS_OK) {
+            // which round of which kind of session it was
+            char where[160];
+            snprintf(where, sizeof where, " [round %u of %u: %s, round kind %u, resident from %u%s%s]", j, sc->n_vars,
+                     sc->fast ? "one product" : sc->poly ? "several terms" : "general", j < sc->round_kind.size() ? (u32)sc->round_kind[j] : 0u, sc->tail_j0,
+                     sc->host_only ? ", on the host" : "", poly_round_weights_factored(sc, j) ? ", factored weights" : "");
+            ctx->err += where;
+            return rc;
+        }
         if (fn(user, j, msg, npts, chal) != 0) return fail(ctx, DPS_ERR_CALLBACK, "transcript callback failed in round %u", j);
         if (!canonical(chal, 2)) return fail(ctx, DPS_ERR_CALLBACK, "transcript callback returned a non-canonical challenge in round %u", j);
         point_out[2 * (j - 1)] = chal[0];

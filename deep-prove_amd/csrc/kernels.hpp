@@ -1923,6 +1923,10 @@ struct PolyArgs {
     // message, which is the sum over the groups, so each publishes its own sums q(t) (and later its tables' final
     // evaluations) to its 64-word slot raw_out + 64 * blockIdx.y, laid out like the main result area, and the host adds.
     u64 *raw_out;    // nullptr: a single workgroup, which publishes to the main result area
+    // poly_kernel, rounds of at least 2^EQ_LO_BITS pairs whose grid stride is a multiple of that: the weights of the common eq
+    // factor are not streamed (q0, q1) but taken as in the FACT variants of prod_kernel, R(i) = hi[i >> EQ_LO_BITS] * lo[i & mask]
+    // -- hi per workgroup and step (scalar loads) on the running sums, lo once per thread at the end.  nullptr: streamed.
+    const u64 *lq0, *lq1, *hq0, *hq1;
 };
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
@@ -1990,6 +1994,7 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     const u64 n_pairs = a.n_pairs;
     E2 r = gl::e2(a.r0, a.r1);
     const u64 *q0 = a.q0, *q1 = a.q1;
+    const bool fact = EQ && a.lq0 != nullptr;
     {
         const bool inl = a.groups == nullptr;  // a single group handed over in the kernel arguments
         const u64 *src = inl ? reinterpret_cast<const u64 *>(&a.g0) : reinterpret_cast<const u64 *>(a.groups + blockIdx.y);
@@ -2073,7 +2078,15 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
         else
             for (u32 k = 0; k < n_tabs; k++) take(g.tab[k], k);
         gl::E2P restp = gl::prep(gl::e2_one());
-        if (EQ) restp = gl::prep(gl::e2(q0[i], q1[i]));
+        if (EQ) {
+            if (fact) {
+                // (the same entry for the whole workgroup: its pairs lie within one run of 2^EQ_LO_BITS)
+                const u32 hi = __builtin_amdgcn_readfirstlane((u32)(i >> EQ_LO_BITS));
+                restp = gl::prep(gl::e2(a.hq0[hi], a.hq1[hi]));
+            } else {
+                restp = gl::prep(gl::e2(q0[i], q1[i]));
+            }
+        }
         // (one copy of the body per evaluation point, t a compile-time constant in each)
         static_for<NP>([&](auto point) {
             constexpr int t = decltype(point)::value;
@@ -2129,6 +2142,13 @@ __global__ void __launch_bounds__(BLOCK) poly_kernel(PolyArgs a, u64 *__restrict
     E2 acc[NP];
 #pragma unroll
     for (int t = 0; t < NP; t++) acc[t] = lz[t];
+    if (EQ && fact) {
+        // the low part of the weights: the same for all of a thread's pairs (the grid's stride is a multiple of 2^EQ_LO_BITS)
+        const u32 lo = (blockIdx.x * BLOCK + tid) & ((1u << EQ_LO_BITS) - 1);
+        const gl::E2P lp = gl::prep(gl::e2(a.lq0[lo], a.lq1[lo]));
+#pragma unroll
+        for (int t = 0; t < NP; t++) acc[t] = gl::mulp(acc[t], lp);
+    }
     block_reduce<NP>(acc, lds);
     if (gridDim.x * gridDim.y == 1) {
         publish_sums<NP>(ff.out_host, ff.seq, ff.counter, acc);

@@ -232,12 +232,23 @@ static bool folds_written(const std::vector<GroupCase> &groups, u64 n_pairs)
 // terms travel in the kernel arguments.  `slots`: per-workgroup result areas instead of partials + ticket.
 template <int NF, bool EQ, bool SKIP1>
 static void run_round(const char *name, std::vector<GroupCase> groups, u64 n_pairs, E2 r, u32 gx, int split_log, bool nested, bool inline_descs, bool slots,
-                      int wait = 0 /* 1: the challenge comes by mail, 2: by mail through the relay */)
+                      int wait = 0 /* 1: the challenge comes by mail, 2: by mail through the relay */,
+                      bool fact = false /* the eq weights as products of a low and a high table (poly_kernel, stride a multiple of 2^16) */)
 {
     constexpr int NP = NF + 1;
     std::vector<E2> w(n_pairs);
     std::vector<u64> q0(n_pairs), q1(n_pairs);
     for (u64 i = 0; i < n_pairs; i++) w[i] = felt2(), q0[i] = w[i].c0, q1[i] = w[i].c1;
+    std::vector<u64> lq0, lq1, hq0, hq1;
+    if (fact) {
+        const u64 lo_n = (u64)1 << dpk::EQ_LO_BITS, hi_n = (n_pairs + lo_n - 1) / lo_n;
+        lq0.resize(lo_n), lq1.resize(lo_n), hq0.resize(hi_n), hq1.resize(hi_n);
+        for (u64 i = 0; i < lo_n; i++) lq0[i] = felt(), lq1[i] = felt();
+        for (u64 i = 0; i < hi_n; i++) hq0[i] = felt(), hq1[i] = felt();
+        for (u64 i = 0; i < n_pairs; i++) w[i] = gl::mul(gl::e2(hq0[i >> dpk::EQ_LO_BITS], hq1[i >> dpk::EQ_LO_BITS]), gl::e2(lq0[i & (lo_n - 1)], lq1[i & (lo_n - 1)]));
+        // (the streamed table is not to be read)
+        q0.assign(1, 0), q1.assign(1, 0);
+    }
     E2 want[NP];
     want_sums<NP>(groups, n_pairs, EQ ? &w : nullptr, SKIP1, want);
 
@@ -275,6 +286,7 @@ static void run_round(const char *name, std::vector<GroupCase> groups, u64 n_pai
         a.ops = po.data();
     }
     a.q0 = q0.data(), a.q1 = q1.data();
+    if (fact) a.lq0 = lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
     a.n_pairs = n_pairs;
     a.r0 = r.c0, a.r1 = r.c1;
     a.j = 2, a.n_vars = 30;
@@ -500,6 +512,14 @@ int main()
         for (int k = 0; k < 60; k++) g.terms.push_back({coeff(), {(u32)(k % 7), (u32)((k * 3 + 1) % 7), (u32)((k * 5 + 2) % 7)}});
         run_round<3, true, true>("sixty terms over seven tables, lanes sharing a pair", {g}, np, r, 1, 3, false, false, false);
         run_round<3, true, true>("the same, poly_kernel", {g}, np, r, 2, -1, false, false, false);
+    }
+    // ---- eq weights from a low and a high table: 256 workgroups (a stride of 2^16 pairs), the second step a few pairs only ----
+    {
+        const u64 np = ((u64)1 << 16) + 300;
+        GroupCase g;
+        for (int k = 0; k < 2; k++) g.tabs.push_back(make_tab(dpk::POLY_PAIR, true, false, 0, np, r));
+        g.terms = {{coeff(), {0, 1}}, {coeff(), {1}}};
+        run_round<2, true, true>("eq weights as low x high table, 256 workgroups", {g}, np, r, 256, -1, false, true, false, 0, true);
     }
     // ---- a launch that stays for every remaining round, folded tables in LDS, last pairs handed over ----
     run_resident<2>("resident from 64 pairs down, four lanes a pair growing to sixteen", 4, {{gl::e2_one(), {0, 3}}, {gl::e2_one(), {1, 2}}, {coeff(), {2, 3}}}, 6, 2, 4);
