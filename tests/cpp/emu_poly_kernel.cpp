@@ -41,6 +41,7 @@ static int failures = 0;
 static std::vector<u64> dyn_lds;
 
 // a grid of gx x gy workgroups, one after the other (the kernels' static LDS is shared by whatever runs at once)
+static std::vector<u32> only_blocks;  // not empty: only these workgroups (x indices) of the grid are run
 template <class K, class... A>
 static void launch(u32 gx, u32 gy, size_t lds_words, K kernel, A... args)
 {
@@ -48,6 +49,7 @@ static void launch(u32 gx, u32 gy, size_t lds_words, K kernel, A... args)
     blockDim = dim3(dpk::BLOCK);
     for (u32 by = 0; by < gy; by++)
         for (u32 bx = 0; bx < gx; bx++) {
+            if (!only_blocks.empty() && std::find(only_blocks.begin(), only_blocks.end(), bx) == only_blocks.end()) continue;
             dyn_lds.assign(lds_words + 16, 0xAAAAAAAAAAAAAAAAull);
             emu::default_group.reset(dpk::BLOCK);
             emu::default_group.dyn = dyn_lds.data();
@@ -338,6 +340,67 @@ static void run_round(const char *name, std::vector<GroupCase> groups, u64 n_pai
     if (!ok) failures++;
 }
 
+// The eq weights as products of a low and a high table (poly_kernel with a grid stride of 2^16 pairs): three of the 256
+// workgroups are run, each publishing to a result area of its own, and each one's sums are compared with plain loops over its
+// own pairs (a workgroup's pairs: b * BLOCK + t + k * 2^16).
+static void run_factored_weights(E2 r)
+{
+    constexpr int NF = 2, NP = 3;
+    const u64 n_pairs = ((u64)1 << 16) + 300, lo_n = (u64)1 << dpk::EQ_LO_BITS;
+    const u32 gx = 256;
+    GroupCase g;
+    for (int k = 0; k < 2; k++) g.tabs.push_back(make_tab(dpk::POLY_PAIR, true, false, 0, n_pairs, r));
+    g.terms = {{felt2(), {0, 1}}, {felt2(), {1}}};
+    std::vector<u64> lq0(lo_n), lq1(lo_n), hq0(2), hq1(2), q0(1, 0), q1(1, 0);
+    for (u64 i = 0; i < lo_n; i++) lq0[i] = felt(), lq1[i] = felt();
+    for (u64 i = 0; i < 2; i++) hq0[i] = felt(), hq1[i] = felt();
+    dpk::PolyArgs a;
+    memset(&a, 0, sizeof a);
+    a.g0.n_tabs = 2;
+    for (u32 k = 0; k < 2; k++) a.g0.tab[k] = desc_of(g.tabs[k]);
+    a.g0.term_begin = 0, a.g0.term_end = 2;
+    for (u32 k = 0; k < 2; k++) a.t0[k] = poly_term(g.terms[k]);
+    a.q0 = q0.data(), a.q1 = q1.data();  // (the streamed table is not to be read)
+    a.lq0 = lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
+    a.n_pairs = n_pairs;
+    a.r0 = r.c0, a.r1 = r.c1;
+    a.j = 2, a.n_vars = 30, a.split_cap = 4, a.group_stride = 1;
+    std::vector<u64> out_host(64, 0), areas(64 * (size_t)gx, 0), partial(2 * dpk::MAX_PTS * (size_t)gx + 64, 0);
+    u32 counter = 0;
+    dpk::FastFin ff;
+    memset(&ff, 0, sizeof ff);
+    ff.partial = partial.data(), ff.n_blocks = gx, ff.out_host = out_host.data(), ff.seq = 77, ff.counter = &counter, ff.slots = areas.data();
+    only_blocks = {0, 1, 255};
+    launch(gx, 1, (size_t)2 * 4 * dpk::BLOCK, dpk::poly_kernel<NF, true, true>, a, partial.data(), ff);
+    bool ok = true;
+    for (u32 b : only_blocks) {
+        E2 want[NP] = {gl::e2_zero(), gl::e2_zero(), gl::e2_zero()};
+        for (u64 i = (u64)b * dpk::BLOCK; i < n_pairs; i += (u64)gx * dpk::BLOCK)
+            for (u64 t = 0; t < (u64)dpk::BLOCK && i + t < n_pairs; t++) {
+                const u64 p = i + t;
+                const E2 w = gl::mul(gl::e2(hq0[p >> dpk::EQ_LO_BITS], hq1[p >> dpk::EQ_LO_BITS]), gl::e2(lq0[p & (lo_n - 1)], lq1[p & (lo_n - 1)]));
+                for (int pt = 0; pt < NP; pt++) {
+                    if (pt == 1) continue;
+                    E2 G = gl::e2_zero();
+                    for (const Term &tm : g.terms) {
+                        E2 prod = tm.coeff;
+                        for (u32 sl : tm.slots) prod = gl::mul(prod, gl::add(g.tabs[sl].lo[p], gl::mul_base(gl::sub(g.tabs[sl].hi[p], g.tabs[sl].lo[p]), (u64)pt)));
+                        G = gl::add(G, prod);
+                    }
+                    want[pt] = gl::add(want[pt], gl::mul(G, w));
+                }
+            }
+        const u64 *area = areas.data() + 64 * (size_t)b;
+        u64 chk = ff.seq;
+        for (int k = 0; k < 2 * NP; k++) chk ^= dpk::rotl64(area[k], k + 1);
+        if (area[dpk::HOST_SEQ_SLOT] != ff.seq || area[dpk::HOST_CHK_SLOT] != chk) ok = false;
+        for (int pt = 0; pt < NP; pt++) ok = ok && gl::eq(gl::e2(area[2 * pt], area[2 * pt + 1]), want[pt]);
+    }
+    only_blocks.clear();
+    printf("%-70s pairs=%llu, workgroups 0, 1 and 255 of %u : %s\n", "eq weights as a low and a high table", (unsigned long long)n_pairs, gx, ok ? "ok" : "MISMATCH");
+    if (!ok) failures++;
+}
+
 // A launch of poly_split_kernel that stays for every round down to one pair (one group, folded tables kept in LDS, the
 // challenges by mail), and hands over the last pairs with its last round.  Every round's sums and the last pairs are
 // compared with plain folds of reference tables.
@@ -513,14 +576,8 @@ int main()
         run_round<3, true, true>("sixty terms over seven tables, lanes sharing a pair", {g}, np, r, 1, 3, false, false, false);
         run_round<3, true, true>("the same, poly_kernel", {g}, np, r, 2, -1, false, false, false);
     }
-    // ---- eq weights from a low and a high table: 256 workgroups (a stride of 2^16 pairs), the second step a few pairs only ----
-    {
-        const u64 np = ((u64)1 << 16) + 300;
-        GroupCase g;
-        for (int k = 0; k < 2; k++) g.tabs.push_back(make_tab(dpk::POLY_PAIR, true, false, 0, np, r));
-        g.terms = {{coeff(), {0, 1}}, {coeff(), {1}}};
-        run_round<2, true, true>("eq weights as low x high table, 256 workgroups", {g}, np, r, 256, -1, false, true, false, 0, true);
-    }
+    // ---- eq weights from a low and a high table: a grid of 256 workgroups (a stride of 2^16 pairs), the second step a few pairs only ----
+    run_factored_weights(r);
     // ---- a launch that stays for every remaining round, folded tables in LDS, last pairs handed over ----
     run_resident<2>("resident from 64 pairs down, four lanes a pair growing to sixteen", 4, {{gl::e2_one(), {0, 3}}, {gl::e2_one(), {1, 2}}, {coeff(), {2, 3}}}, 6, 2, 4);
     run_resident<3>("resident from 16 pairs down, degree 3", 5, {{coeff(), {0, 1, 2}}, {coeff(), {3, 4}}, {coeff(), {4}}}, 4, 4, 4);
