@@ -1533,6 +1533,7 @@ __host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap, u32 blk) 
 // A workgroup of these launches is 1024 threads: what a round costs here is the longest chain of dependent field
 // multiplications in any one lane, and with more lanes each has fewer units of work behind one another.
 constexpr int SL_BLOCK = 1024;
+constexpr int SL_PRE = 2;  // items (table, entry) a thread of a launch made ahead asks for before it waits for its first mail
 
 // NF: tables of the product, or with TERMS the largest number of factors of a term (the degree of the polynomial summed)
 // BLK: threads of a workgroup (SL_BLOCK in the library; the kernel's CPU test runs smaller ones)
@@ -1620,6 +1621,29 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
         trip_seq = a.seq0 + (j - a.j0);
         bool skip1;
         E2 rb_ = gl::e2_zero(), ra_ = gl::e2_zero();
+        // A launch made ahead of its first round finds its sources complete (the launch before it on the stream has ended)
+        // but not yet its challenges: the entries this thread will fold are asked for before it waits for the mail, so
+        // that they cross from device memory during the wait (up to SL_PRE items a thread; more are loaded after the mail).
+        U64x2 pre[SL_PRE][4];
+        const bool have_pre = k == 0 && !a.first_go && pend >= 1 && (nt << len_log) <= (u32)(SL_PRE * BLOCK);
+        if (have_pre) {
+            const u64 base = (u64)wg * src_each;
+#pragma unroll
+            for (int sidx = 0; sidx < SL_PRE; sidx++) {
+                const u32 u = tid + (u32)sidx * BLOCK;
+                if (u < (nt << len_log)) {
+                    const u32 f = u >> len_log, i = u & (len - 1);
+                    const u64 *p0 = a.s0[f], *p1 = a.s1[f];
+                    const u64 e = base + ((u64)i << pend);
+                    pre[sidx][0] = ld2(p0 + e);
+                    pre[sidx][2] = p1 ? ld2(p1 + e) : U64x2{0, 0};
+                    if (pend == 2) {
+                        pre[sidx][1] = ld2(p0 + e + 2);
+                        pre[sidx][3] = ld2(p1 + e + 2);
+                    }
+                }
+            }
+        }
         if (k == 0 && a.first_go) {
             // a launch made for round 1, when it is that round's turn: nothing is pending, whether t = 1 is evaluated came
             // with the launch, and the trip over the host link that a look into the mailbox costs is saved
@@ -1634,7 +1658,26 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
         }
         const gl::E2P rb = gl::prep(rb_), ra = gl::prep(ra_);
         // ---- the pending folds ----
-        if (k == 0 || regroup) {
+        if (have_pre) {
+            // (the entries asked for before the wait)
+#pragma unroll
+            for (int sidx = 0; sidx < SL_PRE; sidx++) {
+                const u32 u = tid + (u32)sidx * BLOCK;
+                if (u < (nt << len_log)) {
+                    const u32 f = u >> len_log, i = u & (len - 1);
+                    const U64x2 x0 = pre[sidx][0], x1 = pre[sidx][2];
+                    E2 v;
+                    if (pend == 1) {
+                        v = a.s1[f] ? fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), rb) : fold1_base(x0.x, x0.y, rb_);
+                    } else {
+                        const U64x2 y0 = pre[sidx][1], y1 = pre[sidx][3];
+                        v = fold1p(fold1p(gl::e2(x0.x, x1.x), gl::e2(x0.y, x1.y), ra), fold1p(gl::e2(y0.x, y1.x), gl::e2(y0.y, y1.y), ra), rb);
+                    }
+                    tab(true, f, 0)[i] = v.c0;
+                    tab(true, f, 1)[i] = v.c1;
+                }
+            }
+        } else if (k == 0 || regroup) {
             // from device memory: entry i of the state is the source's entry i (nothing pending), or is made of its entries
             // 2i, 2i+1 (one fold) or 4i..4i+3 (two)
             const u64 base = (u64)wg * src_each;

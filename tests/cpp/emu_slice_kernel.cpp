@@ -100,6 +100,7 @@ struct Term {
 // `separate`: the stage of several workgroups and the single workgroup after it are two launches (as when the rounds left
 // are more than one launch can run); otherwise they are one.  `host_rounds`: the last rounds are not the launch's (the
 // library works them out on the host): its last trip ends before them and hands over that many more entries.
+static bool g_two_behind = false;  // the first launch's sources are two folds behind its first round (as behind a launch that covered two rounds)
 static bool g_first_go = false;  // launches that start with round 1 are told at once whether t = 1 is evaluated, and get no first mail
 template <int NF, bool EQ, bool TERMS = false>
 static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_in, std::vector<u32> single_rounds = {}, std::vector<Term> terms = {},
@@ -113,7 +114,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         for (u32 f = 0; f < NT; f++) t.tabs.push_back(f);
         terms = {t};
     }
-    const u32 first_pend = j0 == 1 ? 0 : 1;
+    const u32 first_pend = j0 == 1 ? 0 : (g_two_behind && j0 >= 3 ? 2 : 1);
     auto is_single = [&](u32 j) {
         for (u32 x : single_rounds)
             if (x == j) return true;
@@ -473,6 +474,13 @@ int main()
     run_case<2, true>("four workgroups, then one, the last three rounds left out", 12, 3, 4, 0, {}, {}, 0, false, 3);
     run_case<2, false, true>("16 tables, 8 products, the last two rounds left out", 8, 1, 1, 16, {}, stacked, 0, false, 2);
     run_case<2, true, true>("fraction-sum layer over 4 workgroups, the last three rounds left out", 11, 2, 4, 4, {}, {la, lb, lc}, 0, false, 3);
+    // sources two folds behind the first round: entries asked for before the first mail (few items a thread) and after it (many)
+    g_two_behind = true;
+    run_case<2, true>("two tables and eq from round 3, sources two folds behind", 9, 3, 1, 0);
+    run_case<2, true>("the same with more entries than are asked for ahead", 11, 3, 1, 0);
+    run_case<2, true>("four workgroups from round 3, sources two folds behind", 12, 3, 4, 0);
+    run_case<2, false, true>("16 tables, 8 products from round 3, sources two folds behind", 8, 3, 1, 16, {}, stacked, 0, false, 2);
+    g_two_behind = false;
     // launches for round 1 whose first trip starts without mail
     g_first_go = true;
     run_case<2, true>("from round 1, first trip without mail", 8, 1, 1, 0);
