@@ -41,6 +41,7 @@ constexpr u32 LOGUP_OUT_AREAS = 8;
 constexpr size_t LOGUP_SHADOW_STRIDE = 2048;  // words per tree: dpk::LOGUP_SHADOW_WORDS rounded up
 // A sum of at most this many variables over tables the host holds copies of is worked out on the host, every round of it
 constexpr u32 HOST_ONLY_MAX_VARS = 7;
+constexpr size_t DESC_STAGE_BYTES = 256 << 10;  // pinned staging buffer of a context for descriptor uploads
 constexpr u32 PAIR12_BLOCKS = 1024;  // workgroups of the launch of the first two rounds (64 quads each: a stride of 2^16 quads)
 
 // ---------------------------------------------------------------------------
@@ -82,6 +83,11 @@ struct dps_ctx {
     u64 *d_shadow = nullptr;        // device address of the same memory
     hipEvent_t stage_event = nullptr;  // recorded after a launch that reads the staging region of the pinned buffer
     bool stage_pending = false;
+    // A session's descriptor block goes to the device through this pinned buffer (a copy from pageable memory is staged by
+    // the runtime inside the call: 70 us for the 70 KB of a 17-group session); the event says when the copy has read it
+    char *h_desc_stage = nullptr;
+    hipEvent_t desc_event = nullptr;
+    bool desc_pending = false;
     size_t res_off = 0;         // round results: h_pinned[res_off ..], sequence number at res_off + HOST_SEQ_SLOT
     u64 seq = 0;                // last sequence number handed to a launch
     struct dps_sc *tail_owner = nullptr;  // session whose tail kernel is resident on the stream
@@ -563,6 +569,13 @@ extern "C" int32_t dps_ctx_create(int32_t device, dps_ctx **out)
     if (hipHostGetDevicePointer((void **)&ctx->d_pinned, ctx->h_pinned, 0) != hipSuccess) return bail(DPS_ERR_HIP);
     memset(ctx->h_pinned, 0, ctx->pinned_words * 8);
     ctx->res_off = ctx->pinned_words - 64;
+    // (without this buffer descriptor blocks are uploaded from where they are)
+    if (hipHostMalloc((void **)&ctx->h_desc_stage, DESC_STAGE_BYTES, hipHostMallocDefault) != hipSuccess ||
+        hipEventCreateWithFlags(&ctx->desc_event, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        if (ctx->h_desc_stage) (void)hipHostFree(ctx->h_desc_stage);
+        ctx->h_desc_stage = nullptr;
+    }
     // (without this memory the trees' small levels are simply not copied to the host)
     if (hipHostMalloc((void **)&ctx->h_shadow, (size_t)LOGUP_OUT_AREAS * LOGUP_SHADOW_STRIDE * 8, hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess ||
         hipHostGetDevicePointer((void **)&ctx->d_shadow, ctx->h_shadow, 0) != hipSuccess) {
@@ -589,6 +602,8 @@ extern "C" int32_t dps_ctx_destroy(dps_ctx *ctx)
     if (ctx->d_lagrange) (void)hipFree(ctx->d_lagrange);
     if (ctx->h_pinned) (void)hipHostFree(ctx->h_pinned);
     if (ctx->h_shadow) (void)hipHostFree(ctx->h_shadow);
+    if (ctx->h_desc_stage) (void)hipHostFree(ctx->h_desc_stage);
+    if (ctx->desc_event) (void)hipEventDestroy(ctx->desc_event);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return DPS_OK;
@@ -2091,7 +2106,24 @@ u32 horner_build(std::vector<HornerTerm> ts, u32 depth, std::vector<dpk::PolyOp>
 int32_t ensure_descs(dps_sc *sc)
 {
     if (sc->descs_uploaded || sc->stage.empty()) return DPS_OK;
-    hipError_t e = hipMemcpyAsync(sc->dev_block, sc->stage.data(), sc->stage.size(), hipMemcpyHostToDevice, sc->ctx->stream);
+    dps_ctx *ctx = sc->ctx;
+    const void *from = sc->stage.data();
+    const bool staged = ctx->h_desc_stage && sc->stage.size() <= DESC_STAGE_BYTES;
+    if (staged) {
+        // through the context's pinned buffer: the copy is then queued, not made inside the call (the buffer's previous
+        // copy, of another session, has long been made; waited for all the same)
+        if (ctx->desc_pending) {
+            HIPCHK(ctx, hipEventSynchronize(ctx->desc_event));
+            ctx->desc_pending = false;
+        }
+        memcpy(ctx->h_desc_stage, sc->stage.data(), sc->stage.size());
+        from = ctx->h_desc_stage;
+    }
+    hipError_t e = hipMemcpyAsync(sc->dev_block, from, sc->stage.size(), hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess && staged) {
+        e = hipEventRecord(ctx->desc_event, ctx->stream);
+        ctx->desc_pending = e == hipSuccess;
+    }
     if (e != hipSuccess) return fail(sc->ctx, DPS_ERR_HIP, "descriptor upload: %s", hipGetErrorString(e));
     sc->descs_uploaded = true;
     return DPS_OK;
