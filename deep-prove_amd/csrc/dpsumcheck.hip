@@ -150,7 +150,8 @@ size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Behind the Lagrange weights: the ticket counter (and at +128 the words through which a launch's first workgroup
 // passes the mail on), then the sum counters of a resident launch of several workgroups and their ticket.
-constexpr size_t COUNTER_BYTES = 256 + 4 * dpk::SL_MAX_SUMS * 8 + 256;
+constexpr size_t SLICE_CTR_WORDS = (size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE;  // counters of a resident launch, each apart
+constexpr size_t COUNTER_BYTES = 256 + SLICE_CTR_WORDS * 8 + 256;
 
 // Address of `scratch` on a device, asked for once per device with that device current (every GPU has its own copy).
 constexpr int WS_MAX_DEVICES = 64;
@@ -1615,8 +1616,8 @@ struct dps_sc {
     std::vector<dpk::SliceTerm> slice_terms;   // sums of several terms: the terms, their tables as slots of slice_ids
     std::vector<uint8_t> round_kind;  // per round (1-based): 0 a launch of its own, 1 starts a trip, 2 starts a trip of two rounds, 3 second round of a trip,
                                       // 4 worked out on the host
-    std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip)
-    u64 ctr_seen[4 * dpk::SL_MAX_SUMS];  // ... what those counters held after the trip before
+    std::vector<uint8_t> round_wide;  // per round: its trip is made by several workgroups (whose counters run on from trip to trip): the sets of counters they add into
+    u64 ctr_seen[dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS];  // ... what those counters held after the trip before
     E2 prev_chal;                     // the challenge of the call before this one
     bool pair12;                      // rounds 1 and 2 are one launch that writes nothing (pair12_kernel); round 3 folds twice on its way in
     // Launches that cover two rounds each behind that one (quad_kernel): launch k takes rounds quad_j0 + 2 k and + 1, reading
@@ -1716,7 +1717,7 @@ int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n,
                        int chk_slot = dpk::HOST_CHK_SLOT);
 void clear_resident_results(dps_ctx *ctx)
 {
-    for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
+    for (u32 c = 0; c < dpk::SL_MAX_GROUPS * (u32)dpk::SL_GROUP_WORDS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
     ctx->h_pinned[slice_fin_off(ctx) + dpk::SL_FIN_SEQ_SLOT] = 0;
 }
 
@@ -2197,6 +2198,15 @@ bool poly_round_weights_factored(const dps_sc *sc, u32 jj)
     return ((u64)blocks_for_pairs(n_pairs) * dpk::BLOCK) % (1ull << dpk::EQ_LO_BITS) == 0;
 }
 
+// Sets of counters the workgroups of a resident launch add their sums into (log2): adds to one counter are served one
+// after the other, so a set is shared by no more than 32 of them and by at least 8 (the host waits for every set)
+u32 slice_counter_sets_log(u32 W)
+{
+    u32 l = 0;
+    while (l < 3 && (W >> l) > 8 && (1u << (l + 1)) <= dpk::SL_MAX_GROUPS) l++;
+    return l;
+}
+
 // Passes the lanes of a workgroup make over `n_quads` quads for the second round of a trip: a lane keeps one sample at one
 // point for some of the terms (slice_kernel's q_split), the lanes of a pass cover BLOCK / (q_split NF (NF + 1)) quads
 u32 slice_second_round_passes(const dps_sc *sc, u32 n_quads)
@@ -2280,7 +2290,7 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs, u32 n_mles)
             if (dbl) st.dbl_mask |= 1u << st.n_trips;
             st.n_trips++;
             sc->round_kind[j] = dbl ? 2 : 1;
-            sc->round_wide[j] = W > 1;
+            sc->round_wide[j] = W > 1 ? (uint8_t)(1u << slice_counter_sets_log(W)) : 0;
             if (dbl) sc->round_kind[j + 1] = 3;
             pend = dbl ? 2 : 1;
             j += pend;
@@ -3220,22 +3230,27 @@ int32_t wait_result_at(dps_ctx *ctx, size_t base_off, u64 seq, u32 slot0, u32 n,
 // launch's result area, whole once it carries the trip's tag (dpk::sl_tag) in its top byte.  `skip1`: the counters of
 // q(1) do not come (zeros are returned for them).  The tags are cleared as the words are taken, so that a word of 128
 // trips ago cannot pass for this trip's.
-int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u64 *out)
+int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u32 n_sets, u64 *out)
 {
-    volatile u64 *base = ctx->h_pinned + slice_area_off(ctx);
+    volatile u64 *area = ctx->h_pinned + slice_area_off(ctx);
     const u64 tag = dpk::sl_tag(seq);
-    u32 c = 0;
+    u32 c = 0, set = 0;
     const u32 n = 4 * n_sums;
+    // (set by set: `out` holds SL_GROUP_WORDS words per set)
     auto take = [&]() {
-        for (; c < n; c++) {
-            if (skip1 && c >= 4 && c < 8) {
-                out[c] = 0;
-                continue;
+        for (; set < n_sets; set++, c = 0) {
+            volatile u64 *base = area + (size_t)set * dpk::SL_GROUP_WORDS;
+            u64 *o = out + (size_t)set * dpk::SL_GROUP_WORDS;
+            for (; c < n; c++) {
+                if (skip1 && c >= 4 && c < 8) {
+                    o[c] = 0;
+                    continue;
+                }
+                const u64 v = __atomic_load_n(base + c, __ATOMIC_ACQUIRE);
+                if ((v >> 56) != tag) return false;
+                o[c] = v & dpk::SL_CTR_MASK;
+                base[c] = 0;
             }
-            const u64 v = __atomic_load_n(base + c, __ATOMIC_ACQUIRE);
-            if ((v >> 56) != tag) return false;
-            out[c] = v & dpk::SL_CTR_MASK;
-            base[c] = 0;
         }
         return true;
     };
@@ -3626,7 +3641,7 @@ int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
         // No resident launch of this context is running now: whatever an abandoned one left in the result area goes -- before
         // the launch is made, which may start its first trip at once (first_go) and publish while this thread is still here.
         memset(sc->ctr_seen, 0, sizeof sc->ctr_seen);
-        for (u32 c = 0; c < 4 * (u32)dpk::SL_MAX_SUMS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
+        for (u32 c = 0; c < dpk::SL_MAX_GROUPS * (u32)dpk::SL_GROUP_WORDS; c++) ctx->h_pinned[slice_area_off(ctx) + c] = 0;
         for (size_t si = 0; si < sc->stages.size(); si++) {
             const dps_sc::Stage &st = sc->stages[si];
             // a stage of several workgroups and the single-workgroup stage that runs to the last round are one launch:
@@ -3687,7 +3702,8 @@ int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
             sa.fin_out = ctx->d_pinned + slice_fin_off(ctx);
             sa.seq0 = seq0 + (st.j0 - first);
             sa.ctr = ctx->d_slice_ctr;
-            sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + 4 * dpk::SL_MAX_SUMS);
+            sa.gate = reinterpret_cast<u32 *>(ctx->d_slice_ctr + SLICE_CTR_WORDS);
+            sa.groups_log = slice_counter_sets_log(st.W);
             ProfScope ps(ctx, DPS_K_TAIL, 0.0);
             CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
             HIPCHK(ctx, hipGetLastError());
@@ -3750,16 +3766,21 @@ int32_t FusedRound::resident_round()
         prepare_message();
         // sums of this round, and with a trip of two rounds those of the next
         const u32 ns = kind == 2 ? np + np * nf : np;
-        u64 cnt[4 * dpk::SL_MAX_SUMS];
-        rc = wait_slice_sums(ctx, fa.seq, ns, a.skip1 != 0, cnt);
+        u64 cnt[dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS];
+        const u32 n_sets = sc->round_wide[j] ? sc->round_wide[j] : 1;
+        rc = wait_slice_sums(ctx, fa.seq, ns, a.skip1 != 0, n_sets, cnt);
         if (rc == DPS_OK) {
-            // several workgroups: the counters run on from trip to trip of the launch
+            // several workgroups: the counters run on from trip to trip of the launch, and the sets of counters add up
             if (sc->round_wide[j])
                 for (u32 c = 0; c < 4 * ns; c++) {
                     if (a.skip1 && c >= 4 && c < 8) continue;
-                    const u64 now = cnt[c];
-                    cnt[c] = now - sc->ctr_seen[c];
-                    sc->ctr_seen[c] = now;
+                    u64 sum = 0;
+                    for (u32 set = 0; set < n_sets; set++) {
+                        const u64 now = cnt[set * dpk::SL_GROUP_WORDS + c];
+                        sum += now - sc->ctr_seen[set * dpk::SL_GROUP_WORDS + c];
+                        sc->ctr_seen[set * dpk::SL_GROUP_WORDS + c] = now;
+                    }
+                    cnt[c] = sum;
                 }
             // limb w & 1 of sum w >> 1: counters 2w (low halves) and 2w + 1 (high halves)
             u64 w[2 * dpk::SL_MAX_SUMS];

@@ -1459,8 +1459,15 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
 // below 2^56), so the top byte counts the adds: the workgroup whose add makes it a multiple of the number of workgroups has
 // been handed, by that same atomic, the sum of everyone else's shares, and passes the total straight on to the host.  No
 // ticket, no fence, no second trip through device memory.  The host recombines the halves and reduces.
+// The adds to one counter are served one after the other (11 ns each, measured), and so are adds to neighbouring words:
+// every counter has 256 bytes of its own, and the workgroups of a large launch add into up to SL_MAX_GROUPS sets of
+// counters (workgroup w into set w mod G), each set complete with its own last add and handed to the host in an area of
+// its own; the host adds the sets up.  (256 workgroups, 36 counters: the last add returned 6 us after the workgroups'
+// sums were ready with one set of adjacent words, 3 us with the words apart, 1.5 us with eight sets.)
 // ---------------------------------------------------------------------------
 constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
+constexpr u32 SL_CTR_STRIDE = 32;  // 64-bit words from one counter in device memory to the next
+constexpr u32 SL_MAX_GROUPS = 8;   // sets of counters (and result areas) of one launch
 // A trip's result: the 4 counters of every sum (32-bit halves of both limbs, added up as integers), one word each in the
 // first 4 * SL_MAX_SUMS words of the result area: the count in the low 56 bits, the trip's tag in the top byte.  A word
 // is one store, so it is whole when its tag is there; the host clears the tags it has taken.
@@ -1470,9 +1477,9 @@ __host__ __device__ __forceinline__ u64 sl_tag(u64 trip_seq) { return 0x80 | (tr
 // table's entries, in an area of their own (`fin_out`: SL_FIN_MAX_WORDS words, then the trip's sequence number and a
 // check word).  The host folds them with the challenges it has drawn since and does what is left: the last fold, or a
 // few rounds of a handful of pairs, which cost it less than a trip costs.
-constexpr int SL_AREA_WORDS = 192;
+constexpr int SL_GROUP_WORDS = 4 * SL_MAX_SUMS;  // a set's part of the result area
+constexpr int SL_AREA_WORDS = SL_GROUP_WORDS * (int)SL_MAX_GROUPS + 32;
 constexpr int SL_FIN_MAX_WORDS = 1024, SL_FIN_SEQ_SLOT = SL_FIN_MAX_WORDS, SL_FIN_CHK_SLOT = SL_FIN_MAX_WORDS + 1, SL_FIN_AREA_WORDS = SL_FIN_MAX_WORDS + 2;
-static_assert(4 * SL_MAX_SUMS <= SL_AREA_WORDS, "the counters fit the result area");
 constexpr int SL_MAX_TRIPS = 32;
 constexpr int SL_MAX_TABS = 16;   // tables of a sum of several terms (a product has at most 3)
 constexpr int SL_MAX_TERMS = 24;
@@ -1508,11 +1515,11 @@ struct SliceArgs {
                        // the host (fin_out) with it; else what is left goes to h0 / h1
     u32 first_go;      // a launch that starts with round 1 (nothing pending), made when that round is due: its first trip starts
                        // without a look into the mailbox; 1: t = 1 is evaluated, 2: it comes from the claim.  0: every trip waits for its mail
-    u32 pad_go;
-    u64 *out_host;     // result area of SL_AREA_WORDS words
+    u32 groups_log;    // several workgroups: they add into 2^groups_log sets of counters (workgroup w into set w mod 2^groups_log)
+    u64 *out_host;     // result area of SL_AREA_WORDS words: SL_GROUP_WORDS per set of counters
     u64 *fin_out;      // ... and the area of SL_FIN_AREA_WORDS words for the entries left with the last trip (finish)
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
-    u64 *ctr;          // several workgroups: 4 * SL_MAX_SUMS counters in device memory, zero when the launch starts
+    u64 *ctr;          // several workgroups: SL_MAX_GROUPS * 4 * SL_MAX_SUMS counters in device memory, SL_CTR_STRIDE words apart, zero when the launch starts
     u32 *gate;         // ... and the count of workgroups that have left their tables in h0 / h1 (zero when the launch starts)
     u64 *h0[SL_MAX_TABS];  // where each workgroup leaves its last state (workgroup-major): for the first workgroup to go on with,
     u64 *h1[SL_MAX_TABS];  // or (a launch that ends before the last round) for the launch queued behind this one
@@ -1610,7 +1617,7 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             if (*ok_flag == 0) return;
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             // every workgroup has made its last add: counters and gate go back to zero for the launch after this one
-            for (u32 c = tid; c < 4 * (u32)SL_MAX_SUMS; c += BLOCK) st_agent(a.ctr + c, 0);
+            for (u32 c = tid; c < SL_MAX_GROUPS * 4 * (u32)SL_MAX_SUMS; c += BLOCK) st_agent(a.ctr + (size_t)c * SL_CTR_STRIDE, 0);
             if (tid == 0) __hip_atomic_store(a.gate, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             src_each = (u64)Wc * len;
             len = (u32)(src_each >> pend);
@@ -1825,12 +1832,16 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
 #pragma unroll
             for (int w = 0; w < BLOCK / WAVE; w++) v += ctr[w * 4 * SL_MAX_SUMS + c];
             bool mine = true;
+            u32 set = 0;
             if (Wc > 1) {
-                const u64 before = __hip_atomic_fetch_add(a.ctr + c, v + SL_CTR_ONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                mine = ((((before >> 56) + 1) & (u64)(Wc - 1)) == 0);
+                // (the workgroups of a set: every 2^groups_log-th one)
+                set = wg & ((1u << a.groups_log) - 1);
+                const u64 before = __hip_atomic_fetch_add(a.ctr + (size_t)(set * (u32)SL_GROUP_WORDS + c) * SL_CTR_STRIDE, v + SL_CTR_ONE, __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT);
+                mine = ((((before >> 56) + 1) & (u64)((Wc >> a.groups_log) - 1)) == 0);
                 v = (before + v) & SL_CTR_MASK;
             }
-            if (mine) st_sys(a.out_host + c, v | (sl_tag(trip_seq) << 56));
+            if (mine) st_sys(a.out_host + set * (u32)SL_GROUP_WORDS + c, v | (sl_tag(trip_seq) << 56));
         }
         pend = dbl ? 2 : 1;
         j += pend;

@@ -172,7 +172,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         stages.push_back(st);
     }
 
-    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr(4 * dpk::SL_MAX_SUMS, 0);
+    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE, 0);
     u32 gate = 0;
     const u64 seq_first = 1000;
     bool ok = true;
@@ -245,6 +245,9 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         a.fin_out = fin.data();
         a.seq0 = seq_first + (st.j0 - j0);
         a.ctr = gctr.data();
+        // (sets of counters: more of them per workgroup than the library would take, so that small launches have several)
+        a.groups_log = st.W >= 8 ? 2 : st.W >= 4 ? 1 : 0;
+        const u32 n_sets_wide = 1u << a.groups_log;
         a.gate = &gate;
         a.n_tabs = NT;
         a.n_terms = TERMS ? (u32)terms.size() : 0;
@@ -259,7 +262,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         std::vector<std::vector<u64>> lds;
         auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap, dpk::BLOCK), dpk::slice_kernel<NF, EQ, TERMS, dpk::BLOCK>, a, groups, lds);
         // ---- the host's side ----
-        std::vector<u64> seen(4 * dpk::SL_MAX_SUMS, 0);  // the counters of several workgroups run on from trip to trip
+        std::vector<u64> seen((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS, 0);  // the counters of several workgroups run on from trip to trip
         for (size_t sj = si; sj <= last_si && ok; sj++) {
             const Stage &sx = stages[sj];
             for (size_t k = 0; k < sx.trips.size() && ok; k++) {
@@ -276,23 +279,28 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
                 if (!(go && sj == si && k == 0)) __atomic_store_n(&mail[dpk::MAIL_SEQ], seq, __ATOMIC_SEQ_CST);
                 // the result: every counter of the trip's sums, tagged with the trip
                 const int ns = dbl ? NS : NP;
-                u64 cnt[4 * dpk::SL_MAX_SUMS];
+                u64 cnt[4 * dpk::SL_MAX_SUMS] = {0};
                 const auto t0 = std::chrono::steady_clock::now();
+                // (several workgroups: every set of counters comes in its own part of the area, and the sets add up)
+                const u32 n_sets = sx.W > 1 ? n_sets_wide : 1;
+                u32 set = 0;
                 for (int c = 0; c < 4 * ns && ok;) {
                     if (skip1 && c >= 4 && c < 8) {
                         cnt[c++] = 0;
                         continue;
                     }
-                    const u64 v = __atomic_load_n(&area[c], __ATOMIC_SEQ_CST);
+                    const size_t at = (size_t)set * dpk::SL_GROUP_WORDS + c;
+                    const u64 v = __atomic_load_n(&area[at], __ATOMIC_SEQ_CST);
                     if ((v >> 56) == dpk::sl_tag(seq)) {
-                        cnt[c] = v & dpk::SL_CTR_MASK;
+                        const u64 now = v & dpk::SL_CTR_MASK;
                         if (sx.W > 1) {
-                            const u64 now = cnt[c];
-                            cnt[c] = now - seen[c];
-                            seen[c] = now;
+                            cnt[c] += now - seen[at];
+                            seen[at] = now;
+                        } else {
+                            cnt[c] = now;
                         }
-                        area[c] = 0;
-                        c++;
+                        area[at] = 0;
+                        if (++set == n_sets) set = 0, c++;
                         continue;
                     }
                     if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(60)) {
