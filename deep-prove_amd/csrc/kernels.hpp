@@ -589,6 +589,10 @@ constexpr int MAIL_SEQ = 0, MAIL_CHK = 1, MAIL_R = 2, MAIL_SKIP1 = 4, MAIL_RA = 
 constexpr u64 MAIL_SKIP1_LEAVE = 2;
 static_assert(MAIL_WORDS <= WAVE, "one wavefront reads the mailbox with one load");
 constexpr u64 MAIL_ABORT_SEQ = ~(u64)0;
+// A mail passed on through device memory (wait_first_mail) is written MAIL_RELAY_COPIES times, 256 bytes apart, and a
+// workgroup polls the copy of its number: polls of one place are served one after the other, and with 255 workgroups on
+// one copy the last of them saw the mail 2 us after the first.
+constexpr u32 MAIL_RELAY_COPIES = 16, MAIL_RELAY_STRIDE = 32, MAIL_RELAY_WORDS = MAIL_RELAY_COPIES * MAIL_RELAY_STRIDE;
 
 // check word of a mailbox: seq ^ xor over the payload words of rotl(word_i, i)
 __host__ __device__ __forceinline__ u64 mail_mix(u64 w, u32 i) { return (i >= (u32)MAIL_R && i < (u32)MAIL_WORDS) ? rotl64(w, i) : 0; }
@@ -631,29 +635,27 @@ __device__ __forceinline__ bool tail_wait_mail(const u64 *mail, u32 spin_limit, 
 }
 
 // The first mail of a launch made ahead of its round.  With few workgroups each polls the host's mailbox (relay ==
-// nullptr).  With many, only the first one does (first_wg) and copies the mail to MAIL_WORDS words of device memory, where
-// the others look for it; when no mail comes it passes on a mail of this number with `reject_skip1` in the skip word, a
-// value the calling variant does not accept, so that every workgroup leaves.  True: the mail is in `box`.
+// nullptr).  With many, only the first one does (first_wg) and copies the mail to device memory (MAIL_RELAY_WORDS words:
+// several copies), where the others look for it; when no mail comes it passes on a mail of this number with `reject_skip1`
+// in the skip word, a value the calling variant does not accept, so that every workgroup leaves.  True: the mail is in `box`.
 __device__ __forceinline__ bool wait_first_mail(const u64 *mail, u64 *relay, bool first_wg, u32 spin_limit, u64 seq, u64 reject_skip1, u64 *box,
                                                 int *ok_lds)
 {
     if (relay == nullptr) return tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
     // (the others outlast the first workgroup, which always passes something on: their polls of device memory are quicker)
-    if (!first_wg) return tail_wait_mail(relay, spin_limit + spin_limit / 4 + 4000, seq, box, ok_lds);
+    if (!first_wg) {
+        const u32 copy = (blockIdx.x + blockIdx.y * gridDim.x) & (MAIL_RELAY_COPIES - 1);
+        return tail_wait_mail(relay + copy * MAIL_RELAY_STRIDE, spin_limit + spin_limit / 4 + 4000, seq, box, ok_lds);
+    }
     const bool ok = tail_wait_mail(mail, spin_limit, seq, box, ok_lds);
-    if (threadIdx.x == 0) {
-        u64 w[MAIL_WORDS];
-#pragma unroll
-        for (int k = 0; k < MAIL_WORDS; k++) w[k] = box[k];
-        if (!ok) {
-#pragma unroll
-            for (int k = 0; k < MAIL_WORDS; k++) w[k] = 0;
-            w[MAIL_SEQ] = seq;
-            w[MAIL_SKIP1] = reject_skip1;
-            w[MAIL_CHK] = seq ^ mail_mix(reject_skip1, MAIL_SKIP1);
+    if (threadIdx.x < WAVE) {
+        // (a copy is accepted by its check word, so the order in which the words land does not matter)
+        for (u32 u = threadIdx.x; u < MAIL_RELAY_COPIES * (u32)MAIL_WORDS; u += WAVE) {
+            const u32 k = u % (u32)MAIL_WORDS, copy = u / (u32)MAIL_WORDS;
+            const u64 none = k == (u32)MAIL_SEQ ? seq : k == (u32)MAIL_SKIP1 ? reject_skip1 : k == (u32)MAIL_CHK ? (seq ^ mail_mix(reject_skip1, MAIL_SKIP1)) : 0;
+            const u64 w = ok ? box[k] : none;
+            st_sys(relay + copy * MAIL_RELAY_STRIDE + k, w);
         }
-#pragma unroll
-        for (int k = 0; k < MAIL_WORDS; k++) st_sys(relay + k, w[k]);
     }
     return ok;
 }

@@ -293,7 +293,7 @@ static void run_round(const char *name, std::vector<GroupCase> groups, u64 n_pai
     a.r0 = r.c0, a.r1 = r.c1;
     a.j = 2, a.n_vars = 30;
     const u64 seq = 31;
-    std::vector<u64> mail(64, 0), relay(64, 0);
+    std::vector<u64> mail(64, 0), relay(dpk::MAIL_RELAY_WORDS, 0);
     if (wait) {
         // the mail is there before the launch (workgroups run one after the other here); the arguments hold no challenge
         a.r0 = a.r1 = 0x1234;

@@ -154,7 +154,7 @@ static void run_case(const Case &c)
     a.lq0 = lq0.empty() ? nullptr : lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
     a.n_pairs = np;
     a.skip1 = SKIP1;
-    std::vector<u64> mail(64, 0), relay(64, 0), out_host(64, 0), slots(64 * 64, 0), partial(2 * NP * (size_t)c.blocks + 64, 0);
+    std::vector<u64> mail(64, 0), relay(dpk::MAIL_RELAY_WORDS, 0), out_host(64, 0), slots(64 * 64, 0), partial(2 * NP * (size_t)c.blocks + 64, 0);
     u32 counter = 0;
     const u64 seq = 77;
     dpk::FastFin ff;
@@ -314,7 +314,7 @@ static void run_two_rounds(const char *name, u64 n_quads, u32 blocks, int wait)
     a.lq0 = lq0.data(), a.lq1 = lq1.data(), a.hq0 = hq0.data(), a.hq1 = hq1.data();
     a.n_pairs = n_quads;
     a.skip1 = 1;
-    std::vector<u64> mail(64, 0), relay(64, 0), out_host(64, 0), partial(2 * dpk::QUAD_SUMS * (size_t)blocks + 64, 0);
+    std::vector<u64> mail(64, 0), relay(dpk::MAIL_RELAY_WORDS, 0), out_host(64, 0), partial(2 * dpk::QUAD_SUMS * (size_t)blocks + 64, 0);
     u32 counter = 0;
     const u64 seq = 55;
     dpk::FastFin ff;

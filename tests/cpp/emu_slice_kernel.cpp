@@ -172,7 +172,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         stages.push_back(st);
     }
 
-    std::vector<u64> mail(64, 0), relay(64, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE, 0);
+    std::vector<u64> mail(64, 0), relay(dpk::MAIL_RELAY_WORDS, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE, 0);
     u32 gate = 0;
     const u64 seq_first = 1000;
     bool ok = true;
