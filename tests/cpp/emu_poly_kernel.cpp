@@ -57,7 +57,7 @@ static void launch(u32 gx, u32 gy, size_t lds_words, K kernel, A... args)
             for (u32 t = 0; t < (u32)dpk::BLOCK; t++)
                 th.emplace_back([=] {
                     threadIdx = dim3(t);
-                    blockIdx = dim3(bx, by);
+                    blockIdx = dim3(bx, by, 0);
                     kernel(args...);
                 });
             for (auto &x : th) x.join();

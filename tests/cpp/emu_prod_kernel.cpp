@@ -47,7 +47,7 @@ static void launch_threads(u32 blocks, u32 threads, K kernel, A... args)
         for (u32 t = 0; t < threads; t++)
             th.emplace_back([=] {
                 threadIdx = dim3(t);
-                blockIdx = dim3(b);
+                blockIdx = dim3(b, 0, 0);  // (indices start at zero in every dimension)
                 kernel(args...);
             });
         for (auto &x : th) x.join();

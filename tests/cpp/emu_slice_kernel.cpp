@@ -73,7 +73,7 @@ static std::vector<std::thread> launch_all(u32 blocks, size_t lds_words, K kerne
             th.emplace_back([=] {
                 emu::group = g;
                 threadIdx = dim3(t);
-                blockIdx = dim3(b);
+                blockIdx = dim3(b, 0, 0);  // (indices start at zero in every dimension)
                 kernel(args);
             });
     }
