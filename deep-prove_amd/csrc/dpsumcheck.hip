@@ -1609,7 +1609,7 @@ struct dps_sc {
     struct Stage {
         u32 W, j0, pend0, n_trips, dbl_mask, cap;
         u64 src_len;
-        u64 *h0[dpk::SL_MAX_TABS], *h1[dpk::SL_MAX_TABS];  // where a stage that is not the last leaves its entries (the next stage's source)
+        u64 *h0[dpk::SL_MAX_TABS + 1], *h1[dpk::SL_MAX_TABS + 1];  // where a stage that is not the last leaves its entries (the next stage's source)
     };
     std::vector<Stage> stages;
     std::vector<u32> slice_ids;                // the tables of the resident launches (session indices), in slot order
@@ -1766,7 +1766,7 @@ u32 slice_lds_granted(dps_ctx *ctx)
 template <int NF, bool EQ, bool TERMS>
 void launch_slice(dps_ctx *ctx, u32 workgroups, u32 n_tabs, u32 cap, const dpk::SliceArgs &a)
 {
-    dpk::slice_kernel<NF, EQ, TERMS><<<workgroups, dpk::SL_BLOCK, dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8, ctx->stream>>>(a);
+    dpk::slice_kernel<NF, EQ, TERMS><<<workgroups, dpk::SL_BLOCK, dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK, EQ) * 8, ctx->stream>>>(a);
 }
 
 // the compiled variants: a product of 1 or 2 tables times eq, of 2 or 3 without; sums of several terms up to degree 4
@@ -1793,7 +1793,7 @@ int slice_occupancy(dps_ctx *ctx, u32 n_tabs, u32 cap)
 {
     static std::mutex mu;
     static std::map<std::pair<int, size_t>, int> known;
-    const size_t lds = dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8;
+    const size_t lds = dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK, EQ) * 8;
     std::lock_guard<std::mutex> lock(mu);
     auto it = known.find({ctx->device, lds});
     if (it != known.end()) return it->second;
@@ -2137,10 +2137,10 @@ namespace {
 
 // Most pairs a workgroup of a resident launch can take in its first round: its LDS holds twice as many entries per table
 // and half of that again.
-u32 slice_pairs_per_workgroup(u32 n_tabs, u32 lds_bytes)
+u32 slice_pairs_per_workgroup(u32 n_tabs, bool eq, u32 lds_bytes)
 {
     u32 cap = 4096;
-    while (cap > 2 && dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK) * 8 > lds_bytes) cap >>= 1;
+    while (cap > 2 && dpk::slice_lds_words(n_tabs, cap, dpk::SL_BLOCK, eq) * 8 > lds_bytes) cap >>= 1;
     return cap / 2;
 }
 // ... and the fewest it is given when the sum is small enough for that: shorter chains of work per lane, more workgroups
@@ -2238,7 +2238,7 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs, u32 n_mles)
     if (lds_bytes == 0) return;
     // (more pairs per workgroup would make more rounds resident, but a trip's arithmetic is a workgroup's alone: with 512
     // pairs of a 3-term sum the first trip took 75 us where a launch for the round and a trip of 128 pairs take 66)
-    const u32 per_wg_max = std::min<u32>(slice_pairs_per_workgroup(n_tabs, lds_bytes), sc->poly ? 128 : 512);
+    const u32 per_wg_max = std::min<u32>(slice_pairs_per_workgroup(n_tabs, has_eq, lds_bytes), sc->poly ? 128 : 512);
     auto pairs_of = [&](u32 round) { return (u64)1 << (n - round); };
     u32 j = first_ok;
     while (pairs_of(j) > (u64)per_wg_max * SLICE_MAX_WORKGROUPS) j++;
@@ -2965,7 +2965,7 @@ int32_t SessionSetup::allocate_device_block()
     // what a resident stage that does not run to the last round leaves for the next: two limb arrays per table
     size_t bytes_hand = 0;
     const u32 slice_tabs = (u32)sc->slice_ids.size();
-    for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * slice_tabs;
+    for (size_t i = 0; i + 1 < sc->stages.size(); i++) bytes_hand += round_up((size_t)sc->stages[i + 1].src_len * 8, 256) * 2 * (slice_tabs + 1);
     size_t total = bytes_fold + bytes_fold_x + bytes_terms + bytes_fin + bytes_gath + bytes_pg + bytes_pt + bytes_po + bytes_partial + bytes_result + bytes_hand;
     CHK(pool_alloc(ctx, total, &sc->dev_block));
     char *p = (char *)sc->dev_block;
@@ -2991,7 +2991,7 @@ int32_t SessionSetup::allocate_device_block()
     p += bytes_result;
     for (size_t i = 0; i + 1 < sc->stages.size(); i++) {
         const size_t limb = round_up((size_t)sc->stages[i + 1].src_len * 8, 256);
-        for (u32 f = 0; f < slice_tabs; f++) {
+        for (u32 f = 0; f <= slice_tabs; f++) {
             sc->stages[i].h0[f] = (u64 *)p;
             p += limb;
             sc->stages[i].h1[f] = (u64 *)p;
@@ -3675,6 +3675,9 @@ int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
                 sa.h0[f] = st.h0[f];
                 sa.h1[f] = st.h1[f];
             }
+            // (the eq weights of the workgroups go where one more table would)
+            sa.hw0 = st.h0[n_tabs];
+            sa.hw1 = st.h1[n_tabs];
             sa.n_tabs = n_tabs;
             if (sc->poly) {
                 sa.n_terms = (u32)sc->slice_terms.size();

@@ -1525,6 +1525,7 @@ struct SliceArgs {
     u32 *gate;         // ... and the count of workgroups that have left their tables in h0 / h1 (zero when the launch starts)
     u64 *h0[SL_MAX_TABS];  // where each workgroup leaves its last state (workgroup-major): for the first workgroup to go on with,
     u64 *h1[SL_MAX_TABS];  // or (a launch that ends before the last round) for the launch queued behind this one
+    u64 *hw0, *hw1;        // ... and its eq weights (eq factor only; half as many entries), for the first workgroup to go on with
     // a sum of several terms (TERMS): the tables are those of all terms, the polynomial summed is sum_k coeff_k prod table
     u32 n_tabs, n_terms;
     SliceTerm terms[SL_MAX_TERMS];
@@ -1538,7 +1539,12 @@ __host__ __device__ constexpr u32 sl_lds_flags(u32 blk) { return sl_lds_box(blk)
 __host__ __device__ constexpr u32 sl_lds_terms(u32 blk) { return sl_lds_flags(blk) + 2; }
 __host__ __device__ constexpr u32 sl_lds_tables(u32 blk) { return sl_lds_terms(blk) + SL_MAX_TERMS * (sizeof(SliceTerm) / 8); }
 static_assert(sizeof(SliceTerm) % 8 == 0, "terms are copied as 64-bit words");
-__host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap, u32 blk) { return sl_lds_tables(blk) + n_tabs * 2 * (cap + cap / 2); }
+// (`eq`: the weights of the eq factor, one per pair of a table's entries, are kept like a table of half the size)
+__host__ __device__ constexpr u32 sl_weights_cap(u32 cap) { return cap / 2 > 0 ? cap / 2 : 1; }
+__host__ __device__ constexpr u32 slice_lds_words(u32 n_tabs, u32 cap, u32 blk, bool eq)
+{
+    return sl_lds_tables(blk) + n_tabs * 2 * (cap + cap / 2) + (eq ? 2 * (sl_weights_cap(cap) + sl_weights_cap(cap / 2)) : 0);
+}
 // A workgroup of these launches is 1024 threads: what a round costs here is the longest chain of dependent field
 // multiplications in any one lane, and with more lanes each has fewer units of work behind one another.
 constexpr int SL_BLOCK = 1024;
@@ -1572,6 +1578,12 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
     u64 *const buf_big = dyn + SL_LDS_TABLES, *const buf_small = buf_big + (size_t)nt * 2 * cap;
     bool in_big = true;  // where the current state is
     auto tab = [&](bool big, u32 f, int limb) -> u64 * { return big ? buf_big + (size_t)(f * 2 + limb) * cap : buf_small + (size_t)(f * 2 + limb) * (cap / 2); };
+    // The weights of the eq factor, R_j(p) = eq(rho_{j+1..}, p) for the pairs p of round j, live beside the tables in the
+    // same two buffers: read once when the launch starts, and from round to round the weight of a pair is the sum of the
+    // weights of the two pairs it is made of (R_{j+1}(p) = R_j(2p) + R_j(2p + 1)), so a fold of the tables is an add here.
+    u64 *const wts_big = buf_small + (size_t)nt * 2 * (cap / 2), *const wts_small = wts_big + 2 * sl_weights_cap(cap);
+    auto wts = [&](bool big, int limb) -> u64 * { return big ? wts_big + (size_t)limb * sl_weights_cap(cap) : wts_small + (size_t)limb * sl_weights_cap(cap / 2); };
+    auto weight = [&](bool big, u32 p) { return gl::e2(wts(big, 0)[p], wts(big, 1)[p]); };
     if (TERMS) {
         // the terms are read per pair and point: staged in LDS once (visible after the first wait's barrier)
         const u64 *src = reinterpret_cast<const u64 *>(a.terms);
@@ -1598,6 +1610,11 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
                 st_agent(a.h0[f] + (u64)wg * len + i, tab(in_big, f, 0)[i]);
                 st_agent(a.h1[f] + (u64)wg * len + i, tab(in_big, f, 1)[i]);
             }
+            if (EQ)
+                for (u32 i = tid; i < (len >> 1); i += BLOCK) {
+                    st_agent(a.hw0 + (u64)wg * (len >> 1) + i, wts(in_big, 0)[i]);
+                    st_agent(a.hw1 + (u64)wg * (len >> 1) + i, wts(in_big, 1)[i]);
+                }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
@@ -1727,7 +1744,31 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
                 tab(!in_big, f, 0)[i] = v.c0;
                 tab(!in_big, f, 1)[i] = v.c1;
             }
+            if (EQ)
+                for (u32 i = tid; i < (len >> 1); i += BLOCK) {
+                    E2 v = weight(in_big, i << pend);
+                    for (u32 q = 1; q < (1u << pend); q++) v = gl::add(v, weight(in_big, (i << pend) + q));
+                    wts(!in_big, 0)[i] = v.c0;
+                    wts(!in_big, 1)[i] = v.c1;
+                }
             in_big = !in_big;
+        }
+        if (EQ && k == 0) {
+            // the weights of round j's pairs, from the eq table's level of that round
+            const u64 e0 = ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) + (u64)wg * (len >> 1);
+            for (u32 i = tid; i < (len >> 1); i += BLOCK) {
+                wts(true, 0)[i] = a.eq0[e0 + i];
+                wts(true, 1)[i] = a.eq1[e0 + i];
+            }
+        } else if (EQ && regroup) {
+            // ... or from what the workgroups left, added up in runs of 2^pend
+            for (u32 i = tid; i < (len >> 1); i += BLOCK) {
+                const u64 e = (u64)i << pend;
+                E2 v = gl::e2(a.hw0[e], a.hw1[e]);
+                for (u32 q = 1; q < (1u << pend); q++) v = gl::add(v, gl::e2(a.hw0[e + q], a.hw1[e + q]));
+                wts(true, 0)[i] = v.c0;
+                wts(true, 1)[i] = v.c1;
+            }
         }
         // this wavefront's counters start the trip at zero
         for (u32 c = lane; c < 4 * (u32)NS; c += WAVE) ctr[wave * 4 * SL_MAX_SUMS + c] = 0;
@@ -1786,7 +1827,6 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
         // ---- round j: pairs of the state; units taken from the last thread down, those of the quads from the first up ----
         {
             const u32 n_pairs = len >> 1;
-            const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - j))) + (u64)wg * n_pairs : 0;
             const u32 rt = BLOCK - 1 - tid;
             const u32 m0 = rt % p_split, t = (rt / p_split) % (u32)NP, slot = rt / (p_split * (u32)NP), n_slots = BLOCK / (p_split * (u32)NP);
             E2 acc = gl::e2_zero();
@@ -1795,7 +1835,7 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
                 for (u32 p = slot; p < n_pairs; p += n_slots) {
                     any = true;
                     const E2 g = poly_of([&](u32 f) { return line_at(ent(f, 2 * p), ent(f, 2 * p + 1), t); }, false, m0, p_split);
-                    acc = EQ ? gl::fma(g, gl::prep(gl::e2(a.eq0[eq_off + p], a.eq1[eq_off + p])), acc) : gl::add(acc, g);
+                    acc = EQ ? gl::fma(g, gl::prep(weight(big, p)), acc) : gl::add(acc, g);
                 }
             }
             if (any) flush(t, acc);
@@ -1803,7 +1843,6 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
         // ---- round j + 1 as a polynomial in the challenge of round j: quads of the state ----
         if (dbl) {
             const u32 n_quads = len >> 2;
-            const u64 eq_off = EQ ? ((2ull << a.n_vars) - (2ull << (a.n_vars - (j + 1)))) + (u64)wg * n_quads : 0;
             // a lane keeps one sample at one point (of some of the terms)
             const u32 m0 = tid % q_split, ti = (tid / q_split) % (u32)NPT, smp = (tid / (q_split * (u32)NPT)) % (u32)NSMP;
             const u32 slot = tid / (q_split * (u32)(NPT * NSMP)), n_slots = BLOCK / (q_split * (u32)(NPT * NSMP));
@@ -1821,7 +1860,8 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
                         return line_at(line_at(e0, e1, smp), line_at(e2_, e3, smp), t);
                     };
                     const E2 g = poly_of(sampled, smp == (u32)NF, m0, q_split);
-                    acc = EQ ? gl::fma(g, gl::prep(gl::e2(a.eq0[eq_off + u], a.eq1[eq_off + u])), acc) : gl::add(acc, g);
+                    // (the weight of a quad of round j + 1: those of its two pairs of round j)
+                    acc = EQ ? gl::fma(g, gl::prep(gl::add(weight(big, 2 * u), weight(big, 2 * u + 1))), acc) : gl::add(acc, g);
                 }
             }
             if (any) flush(NP + smp * NPT + ti, acc);

@@ -221,6 +221,9 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
             a.h0[f] = h0[f].data();
             a.h1[f] = h1[f].data();
         }
+        // (where the workgroups leave their eq weights for the first of them)
+        std::vector<u64> hw0(st.src_len, 0), hw1(st.src_len, 0);
+        a.hw0 = hw0.data(), a.hw1 = hw1.data();
         a.src_len = st.src_len;
         a.pend0 = st.pend0;
         a.n_vars = n_vars;
@@ -260,7 +263,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         const u32 cap = (u32)((st.src_len / st.W) >> st.pend0);
         std::vector<std::unique_ptr<emu::Group>> groups;
         std::vector<std::vector<u64>> lds;
-        auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap, dpk::BLOCK), dpk::slice_kernel<NF, EQ, TERMS, dpk::BLOCK>, a, groups, lds);
+        auto threads = launch_all(st.W, dpk::slice_lds_words(NT, cap, dpk::BLOCK, EQ), dpk::slice_kernel<NF, EQ, TERMS, dpk::BLOCK>, a, groups, lds);
         // ---- the host's side ----
         std::vector<u64> seen((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS, 0);  // the counters of several workgroups run on from trip to trip
         for (size_t sj = si; sj <= last_si && ok; sj++) {
