@@ -2144,7 +2144,9 @@ u32 slice_pairs_per_workgroup(u32 n_tabs, bool eq, u32 lds_bytes)
     return cap / 2;
 }
 // ... and the fewest it is given when the sum is small enough for that: shorter chains of work per lane, more workgroups
-constexpr u32 SLICE_MIN_PAIRS = 128;
+// (measured with 128, 64, 32, 16: 8 products over 16 tables 0.130, 0.119, 0.114, 0.111 ms; the fraction-tree proof 3.37, 3.30,
+// 3.28, 3.38 ms -- more workgroups cost little since their sums go into several sets of counters)
+constexpr u32 SLICE_MIN_PAIRS = 32;
 constexpr u32 SLICE_MAX_WORKGROUPS = 256;
 // the rounds a resident launch leaves to the host: at most so many, and so many extension multiplications in all
 // (measured: 2 to 6 rounds and 400 to 3000 multiplications differ by a few percent; these were the best over the benchmark configurations)
