@@ -151,7 +151,8 @@ size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Behind the Lagrange weights: the ticket counter (and at +128 the words through which a launch's first workgroup
 // passes the mail on), then the sum counters of a resident launch of several workgroups and their ticket.
 constexpr size_t SLICE_CTR_WORDS = (size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE;  // counters of a resident launch, each apart
-constexpr size_t COUNTER_BYTES = 256 + SLICE_CTR_WORDS * 8 + 256 + (size_t)dpk::MAIL_RELAY_WORDS * 8;
+constexpr size_t SLICE_GATE_BYTES = (size_t)dpk::SL_MAX_GROUPS * dpk::SL_GATE_STRIDE * 4;  // the gate counts of a resident launch behind its counters
+constexpr size_t COUNTER_BYTES = 256 + SLICE_CTR_WORDS * 8 + SLICE_GATE_BYTES + (size_t)dpk::MAIL_RELAY_WORDS * 8;
 
 // Address of `scratch` on a device, asked for once per device with that device current (every GPU has its own copy).
 constexpr int WS_MAX_DEVICES = 64;
@@ -1691,7 +1692,7 @@ namespace {
 u64 *mailbox(dps_ctx *ctx) { return ctx->h_pinned + ctx->res_off - 64; }
 // device memory through which the first workgroup of a large launch made ahead passes the mail on (dpk::MAIL_RELAY_WORDS
 // words behind the counters of the resident launches and their gate)
-u64 *mail_relay(dps_ctx *ctx) { return reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 256 + SLICE_CTR_WORDS * 8 + 256); }
+u64 *mail_relay(dps_ctx *ctx) { return reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 256 + SLICE_CTR_WORDS * 8 + SLICE_GATE_BYTES); }
 
 // completes a mail: check word over the payload as it stands, then the sequence number the kernel waits for
 void send_mail(dps_ctx *ctx, u64 seq)
