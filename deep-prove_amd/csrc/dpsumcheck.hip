@@ -151,8 +151,7 @@ size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Behind the Lagrange weights: the ticket counter (and at +128 the words through which a launch's first workgroup
 // passes the mail on), then the sum counters of a resident launch of several workgroups and their ticket.
 constexpr size_t SLICE_CTR_WORDS = (size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE;  // counters of a resident launch, each apart
-constexpr size_t SLICE_GATE_BYTES = (size_t)dpk::SL_MAX_GROUPS * dpk::SL_GATE_STRIDE * 4;  // the gate counts of a resident launch behind its counters
-constexpr size_t COUNTER_BYTES = 256 + SLICE_CTR_WORDS * 8 + SLICE_GATE_BYTES + (size_t)dpk::MAIL_RELAY_WORDS * 8;
+constexpr size_t COUNTER_BYTES = 256 + SLICE_CTR_WORDS * 8 + 256 + (size_t)dpk::MAIL_RELAY_WORDS * 8;
 
 // Address of `scratch` on a device, asked for once per device with that device current (every GPU has its own copy).
 constexpr int WS_MAX_DEVICES = 64;
@@ -1692,7 +1691,7 @@ namespace {
 u64 *mailbox(dps_ctx *ctx) { return ctx->h_pinned + ctx->res_off - 64; }
 // device memory through which the first workgroup of a large launch made ahead passes the mail on (dpk::MAIL_RELAY_WORDS
 // words behind the counters of the resident launches and their gate)
-u64 *mail_relay(dps_ctx *ctx) { return reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 256 + SLICE_CTR_WORDS * 8 + SLICE_GATE_BYTES); }
+u64 *mail_relay(dps_ctx *ctx) { return reinterpret_cast<u64 *>(reinterpret_cast<char *>(ctx->d_counter) + 256 + SLICE_CTR_WORDS * 8 + 256); }
 
 // completes a mail: check word over the payload as it stands, then the sequence number the kernel waits for
 void send_mail(dps_ctx *ctx, u64 seq)
@@ -2148,6 +2147,10 @@ u32 slice_pairs_per_workgroup(u32 n_tabs, bool eq, u32 lds_bytes)
 // (measured with 128, 64, 32, 16: 8 products over 16 tables 0.130, 0.119, 0.114, 0.111 ms; the fraction-tree proof 3.37, 3.30,
 // 3.28, 3.38 ms -- more workgroups cost little since their sums go into several sets of counters)
 constexpr u32 SLICE_MIN_PAIRS = 32;
+// ... and a sum that could be cut finer takes half the device at most, so that two such sums of two contexts find room
+// side by side (a launch that fills the device alone sends every other context's resident rounds back to launches of their own)
+constexpr u32 SLICE_SMALL_SUM_WORKGROUPS = 128;
+constexpr u32 SLICE_ONE_WORKGROUP_TERM_PAIRS = 512;  // pairs x terms up to which one workgroup takes the whole sum
 constexpr u32 SLICE_MAX_WORKGROUPS = 256;
 // the rounds a resident launch leaves to the host: at most so many, and so many extension multiplications in all
 // (measured: 2 to 6 rounds and 400 to 3000 multiplications differ by a few percent; these were the best over the benchmark configurations)
@@ -2245,7 +2248,12 @@ void plan_resident_rounds(dps_sc *sc, u32 n_tabs, u32 n_mles)
     auto pairs_of = [&](u32 round) { return (u64)1 << (n - round); };
     u32 j = first_ok;
     while (pairs_of(j) > (u64)per_wg_max * SLICE_MAX_WORKGROUPS) j++;
-    const u32 per_wg = (u32)std::min<u64>(per_wg_max, std::max<u64>(SLICE_MIN_PAIRS, pairs_of(j) / SLICE_MAX_WORKGROUPS));
+    // (a small sum stays with one workgroup -- 128 pairs of three terms: four workgroups were 7 us slower over the eight
+    // rounds; 128 pairs of eight terms over 16 tables: four workgroups were 13 us faster)
+    const u64 term_pairs = pairs_of(j) * (sc->poly ? std::max<size_t>(sc->slice_terms.size(), 1) : 1);
+    const u32 per_wg = term_pairs <= SLICE_ONE_WORKGROUP_TERM_PAIRS && pairs_of(j) <= per_wg_max
+                           ? (u32)pairs_of(j)
+                           : (u32)std::min<u64>(per_wg_max, std::max<u64>(SLICE_MIN_PAIRS, pairs_of(j) / SLICE_SMALL_SUM_WORKGROUPS));
     sc->tail_j0 = j;
     // The last rounds are the host's: a trip costs the way to the GPU and back and a workgroup's barriers whatever it
     // carries, a round of a few pairs costs the host a microsecond.  As many rounds as stay below HOST_TAIL_MULTS
@@ -3264,7 +3272,27 @@ int32_t wait_slice_sums(dps_ctx *ctx, u64 seq, u32 n_sums, bool skip1, u32 n_set
             hipError_t q = hipStreamQuery(ctx->stream);
             if (q == hipSuccess) {
                 if (take()) return DPS_OK;
-                return fail(ctx, DPS_ERR_HIP, "round result was not published");
+                // what the launch left behind, for whoever reads the message: how many workgroups had added to the first
+                // counter of every set, and the number of the last mail in every copy the first workgroup passes on
+                std::string left;
+                {
+                    std::vector<u64> words(SLICE_CTR_WORDS), relay(dpk::MAIL_RELAY_WORDS);
+                    if (hipMemcpy(words.data(), ctx->d_slice_ctr, words.size() * 8, hipMemcpyDeviceToHost) == hipSuccess &&
+                        hipMemcpy(relay.data(), mail_relay(ctx), relay.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+                        left = "; adds per set:";
+                        for (u32 g = 0; g < n_sets; g++) left += " " + std::to_string(words[(size_t)g * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE] >> 56);
+                        left += "; mail numbers passed on:";
+                        for (u32 k = 0; k < dpk::MAIL_RELAY_COPIES; k++) left += " " + std::to_string(relay[(size_t)k * dpk::MAIL_RELAY_STRIDE + dpk::MAIL_SEQ]);
+                        left += "; waited for " + std::to_string(seq) + ", set " + std::to_string(set) + " word " + std::to_string(c);
+                        left += "; mailbox " + std::to_string(mailbox(ctx)[dpk::MAIL_SEQ]);
+                        left += "; the first workgroup waited for " + std::to_string(area[dpk::SL_WAITING_SLOT]) + " and had " + std::to_string(area[dpk::SL_HAD_SLOT]);
+                        left += "; tags in the area:";
+                        for (u32 g = 0; g < n_sets; g++) left += " " + std::to_string(area[(size_t)g * dpk::SL_GROUP_WORDS] >> 56);
+                    } else {
+                        (void)hipGetLastError();
+                    }
+                }
+                return fail(ctx, DPS_ERR_HIP, "round result was not published%s", left.c_str());
             }
             if (q != hipErrorNotReady) return fail(ctx, DPS_ERR_HIP, "stream error while waiting for a round: %s", hipGetErrorString(q));
         }

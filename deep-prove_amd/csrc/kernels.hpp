@@ -1470,7 +1470,6 @@ __global__ void __launch_bounds__(PAIR12_BLOCK) pair12_kernel(Pair12Args a, u64 
 constexpr int SL_MAX_SUMS = 25;  // (NF + 1)^2 extension sums per trip at NF = 4
 constexpr u32 SL_CTR_STRIDE = 32;  // 64-bit words from one counter in device memory to the next
 constexpr u32 SL_MAX_GROUPS = 8;   // sets of counters (and result areas) of one launch
-constexpr u32 SL_GATE_STRIDE = 64; // 32-bit words from the gate count of one set to the next
 // A trip's result: the 4 counters of every sum (32-bit halves of both limbs, added up as integers), one word each in the
 // first 4 * SL_MAX_SUMS words of the result area: the count in the low 56 bits, the trip's tag in the top byte.  A word
 // is one store, so it is whole when its tag is there; the host clears the tags it has taken.
@@ -1482,6 +1481,9 @@ __host__ __device__ __forceinline__ u64 sl_tag(u64 trip_seq) { return 0x80 | (tr
 // few rounds of a handful of pairs, which cost it less than a trip costs.
 constexpr int SL_GROUP_WORDS = 4 * SL_MAX_SUMS;  // a set's part of the result area
 constexpr int SL_AREA_WORDS = SL_GROUP_WORDS * (int)SL_MAX_GROUPS + 32;
+// (behind the sets: where the first workgroup says which mail it is waiting for and which it has had last -- read by the
+// host only to say more when a result does not come)
+constexpr int SL_WAITING_SLOT = SL_GROUP_WORDS * (int)SL_MAX_GROUPS, SL_HAD_SLOT = SL_WAITING_SLOT + 1;
 constexpr int SL_FIN_MAX_WORDS = 1024, SL_FIN_SEQ_SLOT = SL_FIN_MAX_WORDS, SL_FIN_CHK_SLOT = SL_FIN_MAX_WORDS + 1, SL_FIN_AREA_WORDS = SL_FIN_MAX_WORDS + 2;
 constexpr int SL_MAX_TRIPS = 32;
 constexpr int SL_MAX_TABS = 16;   // tables of a sum of several terms (a product has at most 3)
@@ -1523,8 +1525,7 @@ struct SliceArgs {
     u64 *fin_out;      // ... and the area of SL_FIN_AREA_WORDS words for the entries left with the last trip (finish)
     u64 seq0;          // sequence number of the trip that starts at round j0; the one that starts at round j has seq0 + (j - j0)
     u64 *ctr;          // several workgroups: SL_MAX_GROUPS * 4 * SL_MAX_SUMS counters in device memory, SL_CTR_STRIDE words apart, zero when the launch starts
-    u32 *gate;         // ... and the counts of workgroups that have left their tables in h0 / h1, one per set of counters, SL_GATE_STRIDE
-                       // 32-bit words apart (zero when the launch starts)
+    u32 *gate;         // ... and the count of workgroups that have left their tables in h0 / h1 (zero when the launch starts)
     u64 *h0[SL_MAX_TABS];  // where each workgroup leaves its last state (workgroup-major): for the first workgroup to go on with,
     u64 *h1[SL_MAX_TABS];  // or (a launch that ends before the last round) for the launch queued behind this one
     u64 *hw0, *hw1;        // ... and its eq weights (eq factor only; half as many entries), for the first workgroup to go on with
@@ -1620,17 +1621,13 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
-            // (counted with its set: a few dozen adds to one word instead of hundreds)
-            if (tid == 0) __hip_atomic_fetch_add(a.gate + (wg & ((1u << a.groups_log) - 1)) * SL_GATE_STRIDE, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) __hip_atomic_fetch_add(a.gate, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (wg != 0) return;
             if (tid == 0) {
                 int ok = 0;
                 const u64 t0 = wall_clock64();
                 do {
-                    bool all = true;
-                    for (u32 set = 0; set < (1u << a.groups_log); set++)
-                        all = all && __hip_atomic_load(a.gate + set * SL_GATE_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (Wc >> a.groups_log);
-                    if (all) {
+                    if (__hip_atomic_load(a.gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Wc) {
                         ok = 1;
                         break;
                     }
@@ -1643,7 +1640,7 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             // every workgroup has made its last add: counters and gate go back to zero for the launch after this one
             for (u32 c = tid; c < SL_MAX_GROUPS * 4 * (u32)SL_MAX_SUMS; c += BLOCK) st_agent(a.ctr + (size_t)c * SL_CTR_STRIDE, 0);
-            if (tid < SL_MAX_GROUPS) __hip_atomic_store(a.gate + tid * SL_GATE_STRIDE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) __hip_atomic_store(a.gate, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             src_each = (u64)Wc * len;
             len = (u32)(src_each >> pend);
             len_log = (u32)__builtin_ctz(len);
@@ -1682,7 +1679,9 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
             skip1 = a.first_go == 2;
             __syncthreads();
         } else {
+            if (wg == 0 && tid == 0) st_sys(a.out_host + SL_WAITING_SLOT, trip_seq);
             if (!wait_first_mail(a.mail, Wc > 1 ? a.relay : nullptr, wg == 0, a.spin_limit, trip_seq, MAIL_SKIP1_LEAVE, box, ok_flag)) return;
+            if (wg == 0 && tid == 0) st_sys(a.out_host + SL_HAD_SLOT, trip_seq);
             if (box[MAIL_SKIP1] >= MAIL_SKIP1_LEAVE) return;
             skip1 = box[MAIL_SKIP1] != 0;
             rb_ = gl::e2(box[MAIL_R], box[MAIL_R + 1]);

@@ -173,7 +173,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
     }
 
     std::vector<u64> mail(64, 0), relay(dpk::MAIL_RELAY_WORDS, 0), area(dpk::SL_AREA_WORDS, 0), fin(dpk::SL_FIN_AREA_WORDS, 0), gctr((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GROUP_WORDS * dpk::SL_CTR_STRIDE, 0);
-    std::vector<u32> gate((size_t)dpk::SL_MAX_GROUPS * dpk::SL_GATE_STRIDE, 0);
+    u32 gate = 0;
     const u64 seq_first = 1000;
     bool ok = true;
     // device-side tables of the stage to come
@@ -251,7 +251,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
         // (sets of counters: more of them per workgroup than the library would take, so that small launches have several)
         a.groups_log = st.W >= 8 ? 2 : st.W >= 4 ? 1 : 0;
         const u32 n_sets_wide = 1u << a.groups_log;
-        a.gate = gate.data();
+        a.gate = &gate;
         a.n_tabs = NT;
         a.n_terms = TERMS ? (u32)terms.size() : 0;
         for (size_t m = 0; TERMS && m < terms.size(); m++) {
@@ -400,8 +400,7 @@ static void run_case(const char *name, u32 n_vars, u32 j0, u32 wide, u32 n_tabs_
             // nobody took over inside the launch: its counters stay as they are, the library clears them behind it
             for (auto &c : gctr) c = 0;
         }
-        for (u32 g : gate)
-            if (g != 0) ok = false, printf("%s: gate left at %u\n", name, g);
+        if (gate != 0) ok = false, printf("%s: gate left at %u\n", name, gate);
         for (u64 c : gctr)
             if (c) ok = false, printf("%s: a counter was left at %llx\n", name, (unsigned long long)c);
         if (st.W > 1) {
