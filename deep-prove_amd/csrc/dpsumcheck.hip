@@ -3742,8 +3742,6 @@ int32_t FusedRound::launch_stages_at(u64 seq0, u32 first_go)
             ProfScope ps(ctx, DPS_K_TAIL, 0.0);
             CHK(launch_slice_dispatch(ctx, sc->poly, nf, has_eq, st.W, n_tabs, st.cap, sa));
             HIPCHK(ctx, hipGetLastError());
-            // a launch of several workgroups that nobody takes over from inside leaves its counters as they are
-            if (st.W > 1 && !merged) reset_device_words(ctx);
             si = last_si;
         }
         sc->tail_seq0 = seq0;

@@ -1904,6 +1904,31 @@ __global__ void __launch_bounds__(BLK) slice_kernel(SliceArgs a)
                 a.h1[f][(u64)wg * len + i] = tab(big, f, 1)[i];
             }
         }
+        if (Wc > 1) {
+            // Several workgroups to the end, nobody took over inside the launch: the first one waits at the gate until every
+            // workgroup has made its last add, and leaves counters and gate at zero for the launch after this one.  (Clearing
+            // them from the host, with a fill queued behind the launch, is a second launch and one more thing on the stream
+            // between this launch and the one that goes on from its tables.)
+            __syncthreads();
+            if (tid == 0) __hip_atomic_fetch_add(a.gate, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (wg != 0) return;
+            if (tid == 0) {
+                int ok = 0;
+                const u64 t0 = wall_clock64();
+                do {
+                    if (__hip_atomic_load(a.gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Wc) {
+                        ok = 1;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                } while (wait_time_left(t0, a.spin_limit));
+                *ok_flag = ok;
+            }
+            __syncthreads();
+            if (*ok_flag == 0) return;  // (a workgroup gave up on the way: the host clears everything behind a failed session)
+            for (u32 c = tid; c < SL_MAX_GROUPS * 4 * (u32)SL_MAX_SUMS; c += BLOCK) st_agent(a.ctr + (size_t)c * SL_CTR_STRIDE, 0);
+            if (tid == 0) __hip_atomic_store(a.gate, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     } else if (wave == 0) {
         // to the host: entry e of table f at words 2 (f len + e), + 1 (len is a power of two)
         const u32 n_words = nt * len * 2;
