@@ -3625,6 +3625,14 @@ int32_t FusedRound::take_sums(u32 n_slots)
             for (u32 t = 0; t < np; t++) q[t] = gl::e2_zero();
             for (u32 g = 0; g < n_slots; g++) {
                 CHK(wait_result_at(ctx, poly_raw_off(ctx) + 64 * (size_t)g, fa.seq, 0, 2 * np, w));
+                // (the groups publish within a microsecond or two of each other, and every area read is a miss in the host's
+                // caches -- the device has just written it: once the first is there the others are asked for together)
+                if (g == 0)
+                    for (u32 h = 1; h < n_slots; h++) {
+                        const u64 *area = ctx->h_pinned + poly_raw_off(ctx) + 64 * (size_t)h;
+                        __builtin_prefetch(area);
+                        __builtin_prefetch(area + 8);
+                    }
                 for (u32 t = 0; t < np; t++) q[t] = gl::add(q[t], gl::e2(w[2 * t], w[2 * t + 1]));
             }
         } else {
